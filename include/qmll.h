@@ -1,0 +1,214 @@
+/*
+ * libqmll -- C ABI of the MI355X (gfx950) kernels behind the QML-Lightning hot path:
+ * FCHL19 representation (+ Jacobian / VJP), SORF (sign diagonal . fast Walsh-Hadamard
+ * stacks), cos features and their derivatives, RFF features, and the Z^T Z / Z^T y
+ * accumulation.
+ *
+ * Conventions for every entry point
+ *   - all pointers are DEVICE pointers of the current HIP device unless marked "host";
+ *     tensors are dense row-major with the shapes written next to them;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); work is only
+ *     enqueued: nothing here allocates, frees, synchronises or throws;
+ *   - the return value is QMLL_OK or a negative QMLL_ERR_* code; qmll_last_error() gives
+ *     the message of the calling thread's last failure;
+ *   - shapes are validated on the host before any launch; a bad argument never reaches
+ *     a kernel.
+ *
+ * Each declaration cites the reference interface it replaces (paths relative to the
+ * reference tree, nickjbrowning/qml-lightning).
+ */
+#ifndef QMLL_H
+#define QMLL_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QMLL_OK 0
+#define QMLL_ERR_INVALID (-1)   /* bad shape / null pointer / unsupported size */
+#define QMLL_ERR_LAUNCH (-2)    /* HIP refused the launch */
+#define QMLL_ERR_NOT_POW2 (-3)  /* "input size must be power of 2." (hadamard_kernel.cu:730) */
+
+typedef void* qmll_stream_t;
+
+/* FCHL19 hyper-parameters as FCHLCuda hands them to its kernels
+ * (qml_lightning/representations/FCHL.py:25-40): three_body_weight already includes
+ * sqrt(eta3/pi). */
+typedef struct qmll_fchl_params {
+    int nspecies;
+    int nRs2;
+    int nRs3;
+    float eta2;
+    float eta3;
+    float two_body_decay;
+    float three_body_weight;
+    float three_body_decay;
+    float rcut;
+} qmll_fchl_params;
+
+int qmll_version(void);
+const char* qmll_last_error(void);
+
+/* ---- neighbours and element types ------------------------------------------------ */
+
+/* Replaces pairlist_gpu.get_num_neighbours_gpu (qml_lightning/cuda/pairlist_cuda.cpp:21-40,
+ * kernel pairlist_kernel.cu:145-224).  X f32 [B,n,3], natoms i32 [B], cell/inv_cell f32
+ * [B,3,3] or NULL (no periodic images) -> nneigh i32 [B,n] (every slot written; padded
+ * atoms get 0).  j counts for i when 0 < |d_ij|^2 < rcut^2. */
+int qmll_num_neighbours(const float* X, const int* natoms, const float* cell, const float* inv_cell,
+                        int B, int n, float rcut, int* nneigh, qmll_stream_t stream);
+
+/* Replaces pairlist_gpu.get_neighbour_list_gpu (pairlist_cuda.cpp:42-65, kernel
+ * pairlist_kernel.cu:326-391).  -> nlist i32 [B,n,max_neighbours], ascending j, unused
+ * slots -1 (every slot written).  An atom with more than max_neighbours neighbours keeps
+ * the first max_neighbours of them. */
+int qmll_neighbour_list(const float* X, const int* natoms, const float* cell, const float* inv_cell,
+                        int B, int n, int max_neighbours, float rcut, int* nlist, qmll_stream_t stream);
+
+/* Replaces fchl_gpu.get_element_types_gpu (qml_lightning/cuda/fchl_cuda.cpp:36-62, kernel
+ * fchl_cuda_kernel.cu:1716-1742).  Z f32 [B,n] charges, species f32 [nspecies] ->
+ * types i32 [B,n]: index of int(charge) in species, -1 if absent, 0 for padded slots. */
+int qmll_element_types(const float* Z, const int* natoms, const float* species, int B, int n, int nspecies,
+                       int* types, qmll_stream_t stream);
+
+/* ---- FCHL19 ---------------------------------------------------------------------- */
+
+/* Replaces fchl_gpu.get_fchl_representation / FCHLCuda (fchl_cuda.cpp:64-95, launcher
+ * fchl_cuda_kernel.cu:1804-1846, kernel :476-674).  One wavefront per entry of
+ * atomIDs/molIDs (i32 [A], one per real atom).  nlist i32 [B,n,nn_stride] + nneigh i32
+ * [B,n] may both be NULL: the kernel then builds each atom's neighbour list itself in LDS
+ * (same rule as qmll_neighbour_list), which removes the host sync on max(nneigh).
+ * rep f32 [B,n,R], R = ns*nRs2 + ns*(ns+1)*nRs3: rows of the listed atoms are
+ * overwritten; rows of padded slots are left untouched (the caller zero-fills, as the
+ * reference wrapper does at fchl_cuda.cpp:83). */
+int qmll_fchl19_forward(const float* X, const int* types, const float* cell, const float* inv_cell,
+                        const int* atomIDs, const int* molIDs, const int* natoms,
+                        const int* nlist, const int* nneigh, int nn_stride,
+                        int A, int B, int n, const float* Rs2, const float* Rs3,
+                        const qmll_fchl_params* prm, float* rep, qmll_stream_t stream);
+
+/* Replaces fchl_gpu.fchl_backwards / FCHLBackwardsCuda (fchl_cuda.cpp:169-202, launcher
+ * fchl_cuda_kernel.cu:1885-1926, kernel :1325-1714): grad_X[m,j,:] += sum_{i,f}
+ * grad_rep[m,i,f] d rep[m,i,f]/d X[m,j,:].  grad_X f32 [B,n,3] is accumulated with
+ * atomics and must be zero-filled by the caller (reference: fchl_cuda.cpp:196). */
+int qmll_fchl19_vjp(const float* X, const int* types, const float* cell, const float* inv_cell,
+                    const int* atomIDs, const int* molIDs, const int* natoms,
+                    const int* nlist, const int* nneigh, int nn_stride,
+                    int A, int B, int n, const float* Rs2, const float* Rs3,
+                    const qmll_fchl_params* prm, const float* grad_rep, float* grad_X,
+                    qmll_stream_t stream);
+
+/* Replaces fchl_gpu.get_fchl_and_derivative / FCHLRepresentationAndDerivativeCuda and
+ * FCHLDerivativeCuda (fchl_cuda.cpp:97-167, launchers fchl_cuda_kernel.cu:1848-1883,
+ * 1928-1964, kernels :676-1005, :1007-1323).  jac f32 [B,n,n,3,R] with
+ * jac[m,i,j,x,f] = d rep[m,i,f]/d X[m,j,x]: for every listed atom i the rows of i itself
+ * and of its neighbours are overwritten in full; all other rows are left untouched (the
+ * caller zero-fills, reference: fchl_cuda.cpp:187).  rep may be NULL (Jacobian only). */
+int qmll_fchl19_jacobian(const float* X, const int* types, const float* cell, const float* inv_cell,
+                         const int* atomIDs, const int* molIDs, const int* natoms,
+                         const int* nlist, const int* nneigh, int nn_stride,
+                         int A, int B, int n, const float* Rs2, const float* Rs3,
+                         const qmll_fchl_params* prm, float* rep, float* jac, qmll_stream_t stream);
+
+/* ---- SORF ------------------------------------------------------------------------ */
+
+/* Replaces sorf_gpu.hadamard_transform_gpu / hadamard_gpu and sorf_matrix_gpu /
+ * compute_sorf_matrix (qml_lightning/cuda/hadamard_cuda.cpp:47-56, 72-87; kernels
+ * hadamard_kernel.cu:5-102, 424-539).  x f32 [A,d], D f32 [T,S,d] (+-1) ->
+ * out f32 [A,S,d] (== [A,S*d]) = normalisation * prod_m (H/sqrt(d) diag(D[m,s])) x.
+ * d must be a power of two in [2, 2048] (QMLL_ERR_NOT_POW2 otherwise). */
+int qmll_sorf_forward(const float* x, const float* D, int A, int d, int S, int T, float normalisation,
+                      float* out, qmll_stream_t stream);
+
+/* Replaces sorf_gpu.hadamard_transform_backwards_gpu / hadamard_backwards_gpu
+ * (hadamard_cuda.cpp:58-70; kernel hadamard_kernel.cu:204-312).  g f32 [A,S,d] ->
+ * gx f32 [A,d], the adjoint of qmll_sorf_forward summed over stacks (overwritten). */
+int qmll_sorf_adjoint(const float* g, const float* D, int A, int d, int S, int T, float normalisation,
+                      float* gx, qmll_stream_t stream);
+
+/* Replaces sorf_gpu.CosFeaturesCUDA / cos_features_gpu (hadamard_cuda.cpp:23-32; kernel
+ * hadamard_kernel.cu:778-800).  coeffs f32 [A,F], bias f32 [F], mol_index i32 [A]
+ * (row of Zf each atom adds to, values in [0,nmol)) -> Zf f32 [nmol,F] +=
+ * sqrt(2/F) cos(coeffs+bias), accumulated with atomics into caller-zeroed memory. */
+int qmll_cos_features_f32(const float* coeffs, const float* bias, const int* mol_index, int A, int F, int nmol,
+                          float* Zf, qmll_stream_t stream);
+
+/* Replaces sorf_gpu.compute_hadamard_features / compute_molecular_featurization
+ * (hadamard_cuda.cpp:89-93; kernel hadamard_kernel.cu:541-563): same as above but every
+ * fp32 feature value is widened and accumulated into Zf f64 [nmol,F] (in place). */
+int qmll_cos_features_f64(const float* coeffs, const float* bias, const int* mol_index, int A, int F, int nmol,
+                          double* Zf, qmll_stream_t stream);
+
+/* Replaces sorf_gpu.CosDerivativeFeaturesCUDA / cos_derivative_features_gpu
+ * (hadamard_cuda.cpp:34-45; kernel hadamard_kernel.cu:816-839).  gZ f32 [nmol,F] ->
+ * gc f32 [A,F] = gZ[mol(a),f] * -sin(coeffs+bias) * sqrt(2/F) (overwritten). */
+int qmll_cos_features_backward(const float* gZ, const float* coeffs, const float* bias, const int* mol_index,
+                               int A, int F, int nmol, float* gc, qmll_stream_t stream);
+
+/* Replaces sorf_gpu.compute_partial_feature_derivatives (hadamard_cuda.cpp:95-109, kernel
+ * hadamard_kernel.cu:565-585): out f64 [A,F] = +sin(coeffs+bias) * sqrt(2/F), each value
+ * computed in fp32 and widened. */
+int qmll_sin_coeffs_f64(const float* coeffs, const float* bias, int A, int F, double* out, qmll_stream_t stream);
+
+/* Replaces sorf_gpu.compute_molecular_featurization_derivative (hadamard_cuda.cpp:95-109,
+ * launcher hadamard_kernel.cu:905-932, kernel :587-717).  cos_derivs f64 [A,F] (from
+ * qmll_sin_coeffs_f64), input_derivative f32 [A,n,3,d] (projected Jacobian rows of the A
+ * atoms), D f32 [T,S,d], mol_index i32 [A] -> G f64 [nmol,n,3,F] +=
+ * normalisation * cos_derivs[a,s*d+p] * (prod_m (H/sqrt(d) diag(D[m,s])) u)[p],
+ * accumulated with fp64 atomics into caller-owned memory. */
+int qmll_derivative_features(const double* cos_derivs, double normalisation, const int* mol_index,
+                             const float* input_derivative, const float* D,
+                             int A, int n, int d, int S, int T, int nmol, double* G, qmll_stream_t stream);
+
+/* Fused predict path for one element: SORF (T = ntransforms) + cos features + energy
+ * contraction + the gradient with respect to the projected representation, without ever
+ * materialising the [A,F] coefficients.  The result equals the chain
+ * get_SORF_coefficients -> get_cos_features -> matmul(Z, alpha) and its autograd
+ * backward (qml_lightning/models/hadamard_features.py:113-121, torchscript/SORF.cpp:74-136)
+ * for d(sum E)/dE = 1.
+ *   x f32 [A,d], D f32 [T,S,d], bias f32 [S*d], alpha f32 [S*d],
+ *   out_index i32 [A] or NULL (slot of e_atom each atom writes; NULL = a)
+ *   -> e_atom[out_index[a]] = sum_f sqrt(2/F) cos(c[a,f]+b[f]) alpha[f]  (overwritten, no atomics;
+ *      the molecular energy is the sum of its atoms' slots)
+ *   -> gx f32 [A,d] = d e_atom[a] / d x[a,:]  (overwritten; NULL = energies only) */
+int qmll_sorf_energy_fused(const float* x, const float* D, const float* bias, const float* alpha,
+                           const int* out_index, int A, int d, int S, int T, float normalisation,
+                           float* e_atom, float* gx, qmll_stream_t stream);
+
+/* ---- RFF ------------------------------------------------------------------------- */
+
+/* Replaces rff_gpu.get_rff / compute_rff (qml_lightning/cuda/random_features.cpp:11-20,
+ * kernel random_features_kernel.cu:5-41).  x f32 [A,d], W f64 [d,F], b f64 [F],
+ * mol_index i32 [A] -> Zf f64 [nmol,F] += sqrt(2/F) cos(x.W + b) (fp64 arithmetic). */
+int qmll_rff_features(const float* x, const double* W, const double* b, const int* mol_index,
+                      int A, int d, int F, int nmol, double* Zf, qmll_stream_t stream);
+
+/* Replaces rff_gpu.get_rff_derivatives / compute_rff_derivatives (random_features.cpp:22-33,
+ * kernel random_features_kernel.cu:43-94).  grad f32 [A,n,3,d] -> G f64 [nmol,n,3,F] +=
+ * sqrt(2/F) sin(x.W+b)_f * (grad[a,j,c,:].W)_f. */
+int qmll_rff_derivative_features(const float* x, const float* grad, const double* W, const double* b,
+                                 const int* mol_index, int A, int n, int d, int F, int nmol, double* G,
+                                 qmll_stream_t stream);
+
+/* ---- Gram ------------------------------------------------------------------------ */
+
+/* Replaces the Gram accumulation of BaseKernel.build_Z_components
+ * (qml_lightning/models/kernel.py:190-192: ZTZ += Z^T Z, ZtrainY += Z^T y, both fp64).
+ * Z f64 [M,F] row-major (lda = F), y f64 [M] or NULL -> ZTZ f64 [F,F] += Z^T Z (both
+ * triangles written), ZTy f64 [F] += Z^T y.  fp64 MFMA. */
+int qmll_gram_f64(const double* Z, const double* y, int M, int F, double* ZTZ, double* ZTy, qmll_stream_t stream);
+
+/* Feature-tiled variant (kernel.py:172-181, ntiles > 1): ZTZ_tile f64 [f1-f0, F] +=
+ * Z[:, f0:f1]^T Z, ZTy f64 [F] (rows f0..f1 updated) += Z[:, f0:f1]^T y. */
+int qmll_gram_tile_f64(const double* Z, const double* y, int M, int F, int f0, int f1, double* ZTZ_tile, double* ZTy,
+                       qmll_stream_t stream);
+
+/* Replaces utils_gpu.matmul_and_reduce (qml_lightning/cuda/utils_cuda.cpp:26-33, kernel
+ * utils_kernel.cu:70-129): C f64 [Ar,Bc] += (double)(A f32 [Ar,K] . B f32 [K,Bc]) with the
+ * K-sum carried in fp32 with Kahan compensation. */
+int qmll_matmul_and_reduce(const float* A, const float* B, int Ar, int K, int Bc, double* C, qmll_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QMLL_H */

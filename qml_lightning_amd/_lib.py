@@ -1,0 +1,80 @@
+"""ctypes binding of libqmll.so, the C-ABI HIP library (declarations: include/qmll.h).
+
+The library is the only compute path: if it is missing or a call fails this module
+raises; there is no CPU or eager fallback.
+"""
+import ctypes
+import os
+from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_void_p
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.environ.get("QML_LIGHTNING_AMD_LIB", os.path.join(HERE, "libqmll.so"))
+
+QMLL_OK = 0
+QMLL_ERR_INVALID = -1
+QMLL_ERR_LAUNCH = -2
+QMLL_ERR_NOT_POW2 = -3
+
+
+class FchlParams(Structure):
+    """Mirror of struct qmll_fchl_params."""
+    _fields_ = [("nspecies", c_int), ("nRs2", c_int), ("nRs3", c_int), ("eta2", c_float), ("eta3", c_float),
+                ("two_body_decay", c_float), ("three_body_weight", c_float), ("three_body_decay", c_float),
+                ("rcut", c_float)]
+
+
+P = c_void_p  # every device pointer and the stream travel as void*
+_FCHL_COMMON = [P, P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, P, P, POINTER(FchlParams)]
+
+# name -> argtypes (restype is int unless listed in _RESTYPES)
+PROTOTYPES = {
+    "qmll_version": [],
+    "qmll_last_error": [],
+    "qmll_num_neighbours": [P, P, P, P, c_int, c_int, c_float, P, P],
+    "qmll_neighbour_list": [P, P, P, P, c_int, c_int, c_int, c_float, P, P],
+    "qmll_element_types": [P, P, P, c_int, c_int, c_int, P, P],
+    "qmll_fchl19_forward": _FCHL_COMMON + [P, P],
+    "qmll_fchl19_vjp": _FCHL_COMMON + [P, P, P],
+    "qmll_fchl19_jacobian": _FCHL_COMMON + [P, P, P],
+    "qmll_sorf_forward": [P, P, c_int, c_int, c_int, c_int, c_float, P, P],
+    "qmll_sorf_adjoint": [P, P, c_int, c_int, c_int, c_int, c_float, P, P],
+    "qmll_cos_features_f32": [P, P, P, c_int, c_int, c_int, P, P],
+    "qmll_cos_features_f64": [P, P, P, c_int, c_int, c_int, P, P],
+    "qmll_cos_features_backward": [P, P, P, P, c_int, c_int, c_int, P, P],
+    "qmll_sin_coeffs_f64": [P, P, c_int, c_int, P, P],
+    "qmll_derivative_features": [P, c_double, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, P],
+    "qmll_sorf_energy_fused": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_float, P, P, P],
+    "qmll_rff_features": [P, P, P, P, c_int, c_int, c_int, c_int, P, P],
+    "qmll_rff_derivative_features": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
+    "qmll_gram_f64": [P, P, c_int, c_int, P, P, P],
+    "qmll_gram_tile_f64": [P, P, c_int, c_int, c_int, c_int, P, P, P],
+    "qmll_matmul_and_reduce": [P, P, c_int, c_int, c_int, P, P],
+}
+_RESTYPES = {"qmll_last_error": c_char_p}
+
+_lib = None
+
+
+def lib():
+    """The loaded library (loaded once).  Raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "qml_lightning_amd: %s not found -- build it with `python -m qml_lightning_amd.build` "
+                "(there is no fallback path)" % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, argtypes in PROTOTYPES.items():
+            fn = getattr(handle, name)
+            fn.argtypes = argtypes
+            fn.restype = _RESTYPES.get(name, c_int)
+        _lib = handle
+    return _lib
+
+
+def check(rc, what=""):
+    """Turn a negative status into the exception the reference raises for the same fault:
+    RuntimeError carrying the library's message (TORCH_CHECK -> RuntimeError there)."""
+    if rc != QMLL_OK:
+        msg = lib().qmll_last_error().decode("utf-8", "replace")
+        raise RuntimeError(msg or ("%s failed with status %d" % (what, rc)))

@@ -1,0 +1,711 @@
+// FCHL19 representation, its VJP and its explicit Jacobian for gfx950.
+// Replaces qml_lightning/cuda/fchl_cuda_kernel.cu:476-674 (forward), :1325-1714 (VJP),
+// :676-1005 and :1007-1323 (Jacobian) of the reference.
+//
+// Layout: one wavefront (64 lanes, one workgroup) per central atom.  The atom's
+// neighbour list is staged in LDS as displacement vectors d_ij = R_i - R_j (minimum-imaged
+// once when a cell is given), distances, element types and atom indices; it is either
+// read from a caller-supplied list or built in the kernel from the molecule's coordinates
+// with a ballot/popcount compaction (ascending j, same rule as the neighbour-list kernel),
+// so the forward/backward pair needs no host round trip for max(nneigh).
+//
+// Arithmetic per atom (nn neighbours): nn*nRs2 + nn(nn-1)/2*nRs3 exponentials forward;
+// the kernels are VALU/transcendental bound, HBM traffic is 4R bytes out (forward) or in
+// (VJP) per atom.
+//
+// The derivatives are written in terms of the three distances a=r_ij, b=r_ik, c=r_jk of a
+// triple: every bin value T depends on positions only through (a,b,c) and
+// cos_i = (a^2+b^2-c^2)/(2ab) etc., so dT = T_a da + T_b db + T_c dc with
+// da/dR_i = u_ij, da/dR_j = -u_ij, db/dR_i = u_ik, db/dR_k = -u_ik, dc/dR_j = u_jk,
+// dc/dR_k = -u_jk.  This is algebraically the reference's 40-term expansion; the
+// degenerate-angle guard sqrt(max(1e-10, a^2 b^2 - (d_ij.d_ik)^2)) is kept.
+#include "qmll_common.h"
+
+namespace {
+
+struct FchlArgs {
+    const float* X;
+    const int* types;
+    const float* cell;
+    const float* inv_cell;
+    const int* atomIDs;
+    const int* molIDs;
+    const int* natoms;
+    const int* nlist;
+    const int* nneigh;
+    int nn_stride;
+    int n;
+    int B;
+    int cap;  // capacity of the LDS neighbour arrays
+    const float* Rs2;
+    const float* Rs3;
+    qmll_fchl_params p;
+};
+
+constexpr int TCH = 256;  // triples per LDS chunk
+constexpr float PI_F = 3.14159265358979323846f;
+
+struct Stage {
+    float* dx;
+    float* dy;
+    float* dz;
+    float* r;
+    int* el;
+    int* j;
+    float* next;  // first free float after the neighbour arrays
+};
+
+__device__ __forceinline__ Stage carve(float* smem, int cap) {
+    Stage s;
+    s.dx = smem;
+    s.dy = s.dx + cap;
+    s.dz = s.dy + cap;
+    s.r = s.dz + cap;
+    s.el = (int*)(s.r + cap);
+    s.j = s.el + cap;
+    s.next = (float*)(s.j + cap);
+    return s;
+}
+
+__device__ __forceinline__ void min_image(float& dx, float& dy, float& dz, const float* c, const float* ic) {
+    float s0 = ic[0] * dx + ic[1] * dy + ic[2] * dz;
+    float s1 = ic[3] * dx + ic[4] * dy + ic[5] * dz;
+    float s2 = ic[6] * dx + ic[7] * dy + ic[8] * dz;
+    s0 -= roundf(s0);
+    s1 -= roundf(s1);
+    s2 -= roundf(s2);
+    dx = c[0] * s0 + c[1] * s1 + c[2] * s2;
+    dy = c[3] * s0 + c[4] * s1 + c[5] * s2;
+    dz = c[6] * s0 + c[7] * s1 + c[8] * s2;
+}
+
+// Fill the LDS neighbour arrays of atom (m,i); returns the neighbour count.  Neighbours
+// whose element type is negative (charge not in `species`) are dropped.
+__device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i, int lane) {
+    const float* Xm = a.X + (size_t)m * a.n * 3;
+    const int* tm = a.types + (size_t)m * a.n;
+    const bool pbc = a.cell != nullptr;
+    float c[9], ic[9];
+    if (pbc) {
+        for (int t = 0; t < 9; ++t) {
+            c[t] = a.cell[(size_t)m * 9 + t];
+            ic[t] = a.inv_cell[(size_t)m * 9 + t];
+        }
+    }
+    const float xi = Xm[i * 3 + 0], yi = Xm[i * 3 + 1], zi = Xm[i * 3 + 2];
+    const float rc2 = a.p.rcut * a.p.rcut;
+    int count = 0;
+    const bool have_list = a.nlist != nullptr;
+    int total;
+    const int* li = nullptr;
+    if (have_list) {
+        total = a.nneigh[(size_t)m * a.n + i];
+        if (total > a.nn_stride) total = a.nn_stride;
+        li = a.nlist + ((size_t)m * a.n + i) * a.nn_stride;
+    } else {
+        total = a.natoms[m];
+        if (total > a.n) total = a.n;
+    }
+    for (int base = 0; base < total; base += QMLL_WAVE) {
+        const int t = base + lane;
+        bool ok = t < total;
+        int j = 0;
+        float dx = 0.f, dy = 0.f, dz = 0.f, r2 = 0.f;
+        int e = -1;
+        if (ok) {
+            j = have_list ? li[t] : t;
+            ok = j >= 0 && j < a.n;
+        }
+        if (ok) {
+            dx = xi - Xm[j * 3 + 0];
+            dy = yi - Xm[j * 3 + 1];
+            dz = zi - Xm[j * 3 + 2];
+            if (pbc) min_image(dx, dy, dz, c, ic);
+            r2 = dx * dx + dy * dy + dz * dz;
+            e = tm[j];
+            // a supplied list is authoritative (it may be stale on purpose, e.g. finite
+            // differences with a frozen list); only the built-in search applies the cutoff
+            ok = (have_list ? (r2 > 0.0f) : (r2 < rc2 && r2 > 0.0f)) && e >= 0;
+        }
+        const unsigned long long mask = __ballot(ok);
+        const int pos = count + __popcll(mask & ((1ull << lane) - 1ull));
+        if (ok && pos < a.cap) {
+            s.dx[pos] = dx;
+            s.dy[pos] = dy;
+            s.dz[pos] = dz;
+            s.r[pos] = sqrtf(r2);
+            s.el[pos] = e;
+            s.j[pos] = j;
+        }
+        count += __popcll(mask);
+    }
+    return count < a.cap ? count : a.cap;
+}
+
+__device__ __forceinline__ float cutoff(float r, float inv_rc) { return 0.5f * (cosf(r * PI_F * inv_rc) + 1.0f); }
+__device__ __forceinline__ float dcutoff(float r, float inv_rc) { return -0.5f * PI_F * inv_rc * sinf(r * PI_F * inv_rc); }
+
+// row index of pair t in the list of pairs (j<k) over nn items, rows enumerated j = 0..nn-2
+__device__ __forceinline__ void unrank_pair(int t, int nn, int& j, int& k) {
+    const float b = (float)(2 * nn - 1);
+    int jj = (int)((b - sqrtf(fmaxf(b * b - 8.0f * (float)t, 0.0f))) * 0.5f);
+    if (jj < 0) jj = 0;
+    if (jj > nn - 2) jj = nn - 2;
+    // offset(j) = j (2nn - j - 1) / 2
+    while (jj > 0 && (jj * (2 * nn - jj - 1)) / 2 > t) --jj;
+    while (((jj + 1) * (2 * nn - jj - 2)) / 2 <= t) ++jj;
+    j = jj;
+    k = jj + 1 + (t - (jj * (2 * nn - jj - 1)) / 2);
+}
+
+__device__ __forceinline__ int pair_offset(int ej, int ek, int ns, int nRs2, int nRs3) {
+    const int p = ej < ek ? ej : ek;
+    const int q = ej < ek ? ek : ej;
+    return ns * nRs2 + 2 * nRs3 * (-(p * (p + 1)) / 2 + q + ns * p);   // fchl_cuda_kernel.cu:658-661
+}
+
+// geometry of one triple (central atom i, neighbours j<k in list order)
+struct Triple {
+    float a, b, c;           // r_ij, r_ik, r_jk
+    float ci, cj, ck;        // cosines at i, j, k
+    float cosT, sinT;        // cos/sin of the clamped angle at i
+    float guard_inv;         // a b / sqrt(max(1e-10, a^2 b^2 - (d_ij.d_ik)^2))
+    float ujk[3];            // (R_j - R_k)/c
+};
+
+__device__ __forceinline__ Triple triple_geometry(const Stage& s, int j, int k) {
+    Triple t;
+    const float ax = s.dx[j], ay = s.dy[j], az = s.dz[j];   // d_ij = R_i - R_j
+    const float bx = s.dx[k], by = s.dy[k], bz = s.dz[k];   // d_ik
+    const float cx = bx - ax, cy = by - ay, cz = bz - az;   // d_jk = R_j - R_k
+    t.a = s.r[j];
+    t.b = s.r[k];
+    const float c2 = cx * cx + cy * cy + cz * cz;
+    t.c = sqrtf(c2);
+    const float ia = 1.0f / t.a, ib = 1.0f / t.b, ic = 1.0f / t.c;
+    const float vi = ax * bx + ay * by + az * bz;           // (R_j-R_i).(R_k-R_i)
+    t.ci = vi * ia * ib;
+    t.ck = (cx * bx + cy * by + cz * bz) * ic * ib;         // (R_j-R_k).(R_i-R_k)
+    t.cj = -(ax * cx + ay * cy + az * cz) * ia * ic;        // (R_i-R_j).(R_k-R_j)
+    const float cc = fminf(1.0f, fmaxf(-1.0f, t.ci));
+    t.cosT = cc;
+    t.sinT = sqrtf(fmaxf(0.0f, 1.0f - cc * cc));
+    const float a2b2 = (t.a * t.a) * (t.b * t.b);
+    t.guard_inv = t.a * t.b * rsqrtf(fmaxf(1e-10f, a2b2 - vi * vi));
+    t.ujk[0] = cx * ic;
+    t.ujk[1] = cy * ic;
+    t.ujk[2] = cz * ic;
+    return t;
+}
+
+// ---------------------------------------------------------------------------------
+// forward
+// ---------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* __restrict__ rep) {
+    extern __shared__ float smem[];
+    const int lane = threadIdx.x;
+    const int m = a.molIDs[blockIdx.x];
+    const int i = a.atomIDs[blockIdx.x];
+    if (m < 0 || m >= a.B || i < 0 || i >= a.n) return;   // malformed index: write nothing
+    const int ns = a.p.nspecies, nRs2 = a.p.nRs2, nRs3 = a.p.nRs3;
+    const int R = ns * nRs2 + ns * (ns + 1) * nRs3;
+
+    Stage s = carve(smem, a.cap);
+    float* smu = s.next;            // [cap]  mu_j
+    float* sis2 = smu + a.cap;      // [cap]  1/(2 sigma_j^2)
+    float* spre = sis2 + a.cap;     // [cap]  r^-d2 fc / (sigma sqrt(2pi))
+    float* slnRs2 = spre + a.cap;   // [nRs2]
+    float* sinvRs2 = slnRs2 + nRs2; // [nRs2]
+    float* sRs3 = sinvRs2 + nRs2;   // [nRs3]
+    float* acc = sRs3 + nRs3;       // [R]
+    float* trip = acc + R;          // [TCH][4]: rho, Kc, Ks, bin offset
+
+    for (int t = lane; t < R; t += QMLL_WAVE) acc[t] = 0.0f;
+    for (int t = lane; t < nRs2; t += QMLL_WAVE) {
+        const float v = a.Rs2[t];
+        slnRs2[t] = logf(v);
+        sinvRs2[t] = 1.0f / v;
+    }
+    for (int t = lane; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
+
+    const int nn = stage_neighbours(a, s, m, i, lane);
+    __syncthreads();
+
+    const float inv_rc = 1.0f / a.p.rcut;
+    // per-neighbour two-body factors
+    for (int j = lane; j < nn; j += QMLL_WAVE) {
+        const float r = s.r[j];
+        const float s2 = logf(1.0f + a.p.eta2 / (r * r));
+        smu[j] = logf(r) - 0.5f * s2;                    // ln(r / sqrt(1 + eta2/r^2))
+        sis2[j] = 0.5f / s2;
+        spre[j] = rsqrtf(s2) * 0.3989422804014327f * powf(r, -a.p.two_body_decay) * cutoff(r, inv_rc);
+    }
+    __syncthreads();
+    for (int it = lane; it < nn * nRs2; it += QMLL_WAVE) {
+        const int j = it / nRs2;
+        const int z = it - j * nRs2;
+        const float u = slnRs2[z] - smu[j];
+        const float v = spre[j] * sinvRs2[z] * expf(-u * u * sis2[j]);
+        atomicAdd(&acc[s.el[j] * nRs2 + z], v);
+    }
+
+    // three-body
+    const int ntrip = nn * (nn - 1) / 2;
+    const float zeta2 = 2.0f * expf(-0.5f * PI_F * PI_F);
+    for (int c0 = 0; c0 < ntrip; c0 += TCH) {
+        const int nchunk = min(TCH, ntrip - c0);
+        __syncthreads();
+        for (int tt = lane; tt < nchunk; tt += QMLL_WAVE) {
+            int j, k;
+            unrank_pair(c0 + tt, nn, j, k);
+            const Triple t = triple_geometry(s, j, k);
+            const float ksi = a.p.three_body_weight * (1.0f + 3.0f * t.ci * t.cj * t.ck) *
+                              powf(t.a * t.b * t.c, -a.p.three_body_decay);
+            const float f = zeta2 * ksi * cutoff(t.a, inv_rc) * cutoff(t.b, inv_rc);
+            trip[tt * 4 + 0] = 0.5f * (t.a + t.b);
+            trip[tt * 4 + 1] = f * t.cosT;
+            trip[tt * 4 + 2] = f * t.sinT;
+            trip[tt * 4 + 3] = __int_as_float(pair_offset(s.el[j], s.el[k], ns, nRs2, nRs3));
+        }
+        __syncthreads();
+        for (int it = lane; it < nchunk * nRs3; it += QMLL_WAVE) {
+            const int tt = it / nRs3;
+            const int l = it - tt * nRs3;
+            const float d = trip[tt * 4 + 0] - sRs3[l];
+            const float e = expf(-a.p.eta3 * d * d);
+            const int off = __float_as_int(trip[tt * 4 + 3]) + 2 * l;
+            atomicAdd(&acc[off], e * trip[tt * 4 + 1]);
+            atomicAdd(&acc[off + 1], e * trip[tt * 4 + 2]);
+        }
+    }
+    __syncthreads();
+    float* out = rep + ((size_t)m * a.n + i) * R;
+    for (int t = lane; t < R; t += QMLL_WAVE) out[t] = acc[t];
+}
+
+// ---------------------------------------------------------------------------------
+// d/dr of the two-body bin values of one neighbour, contracted or not
+// ---------------------------------------------------------------------------------
+struct TwoBody {
+    float mu, s2, s2p, mup, pre, fc, dfc, d2_over_r;
+};
+
+__device__ __forceinline__ TwoBody two_body_setup(float r, const qmll_fchl_params& p, float inv_rc) {
+    TwoBody t;
+    const float r2 = r * r;
+    t.s2 = logf(1.0f + p.eta2 / r2);
+    t.mu = logf(r) - 0.5f * t.s2;
+    t.s2p = -2.0f * p.eta2 / (r * (r2 + p.eta2));      // d sigma^2 / dr
+    t.mup = 1.0f / r - 0.5f * t.s2p;                   // d mu / dr
+    t.pre = rsqrtf(t.s2) * 0.3989422804014327f * powf(r, -p.two_body_decay);
+    t.fc = cutoff(r, inv_rc);
+    t.dfc = dcutoff(r, inv_rc);
+    t.d2_over_r = p.two_body_decay / r;
+    return t;
+}
+
+// value and r-derivative of bin z
+__device__ __forceinline__ void two_body_bin(const TwoBody& t, float lnRs, float invRs, float& val, float& dval) {
+    const float u = lnRs - t.mu;
+    const float inv_s2 = 1.0f / t.s2;
+    const float Bz = t.pre * invRs * expf(-0.5f * u * u * inv_s2);
+    const float Q = -0.5f * t.s2p * inv_s2 - t.d2_over_r + u * inv_s2 * (t.mup + 0.5f * u * t.s2p * inv_s2);
+    val = Bz * t.fc;
+    dval = Bz * (t.fc * Q + t.dfc);
+}
+
+// partial derivatives with respect to (a,b,c) of the triple's prefactor
+// K = w3 (1 + 3 ci cj ck) (abc)^-d3 fc(a) fc(b), and of cos_i
+struct TripleDeriv {
+    float K, Ka, Kb, Kc;     // K and its partials
+    float cia, cib, cic;     // partials of cos_i
+};
+
+__device__ __forceinline__ TripleDeriv triple_derivatives(const Triple& t, const qmll_fchl_params& p, float inv_rc) {
+    TripleDeriv d;
+    const float ia = 1.0f / t.a, ib = 1.0f / t.b, ic = 1.0f / t.c;
+    // d cos / d distance (law of cosines)
+    d.cia = ib - t.ci * ia;
+    d.cib = ia - t.ci * ib;
+    d.cic = -t.c * ia * ib;
+    const float cja = ic - t.cj * ia, cjb = -t.b * ia * ic, cjc = ia - t.cj * ic;
+    const float cka = -t.a * ib * ic, ckb = ic - t.ck * ib, ckc = ib - t.ck * ic;
+    const float P = 1.0f + 3.0f * t.ci * t.cj * t.ck;
+    const float Pa = 3.0f * (d.cia * t.cj * t.ck + t.ci * cja * t.ck + t.ci * t.cj * cka);
+    const float Pb = 3.0f * (d.cib * t.cj * t.ck + t.ci * cjb * t.ck + t.ci * t.cj * ckb);
+    const float Pc = 3.0f * (d.cic * t.cj * t.ck + t.ci * cjc * t.ck + t.ci * t.cj * ckc);
+    const float dec = p.three_body_weight * powf(t.a * t.b * t.c, -p.three_body_decay);
+    const float fa = cutoff(t.a, inv_rc), fb = cutoff(t.b, inv_rc);
+    const float dfa = dcutoff(t.a, inv_rc), dfb = dcutoff(t.b, inv_rc);
+    const float ksi = dec * P;
+    const float ksia = dec * (Pa - p.three_body_decay * P * ia);
+    const float ksib = dec * (Pb - p.three_body_decay * P * ib);
+    const float ksic = dec * (Pc - p.three_body_decay * P * ic);
+    d.K = ksi * fa * fb;
+    d.Ka = ksia * fa * fb + ksi * dfa * fb;
+    d.Kb = ksib * fa * fb + ksi * fa * dfb;
+    d.Kc = ksic * fa * fb;
+    return d;
+}
+
+// ---------------------------------------------------------------------------------
+// VJP
+// ---------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float* __restrict__ grad_rep,
+                                                         float* __restrict__ grad_X) {
+    extern __shared__ float smem[];
+    const int lane = threadIdx.x;
+    const int m = a.molIDs[blockIdx.x];
+    const int i = a.atomIDs[blockIdx.x];
+    if (m < 0 || m >= a.B || i < 0 || i >= a.n) return;   // malformed index: write nothing
+    const int ns = a.p.nspecies, nRs2 = a.p.nRs2, nRs3 = a.p.nRs3;
+    const int R = ns * nRs2 + ns * (ns + 1) * nRs3;
+
+    Stage s = carve(smem, a.cap);
+    float* sgx = s.next;             // [cap] gradient on neighbour j
+    float* sgy = sgx + a.cap;
+    float* sgz = sgy + a.cap;
+    float* slnRs2 = sgz + a.cap;     // [nRs2]
+    float* sinvRs2 = slnRs2 + nRs2;  // [nRs2]
+    float* sRs3 = sinvRs2 + nRs2;    // [nRs3]
+    float* gin = sRs3 + nRs3;        // [R]
+
+    const float* gsrc = grad_rep + ((size_t)m * a.n + i) * R;
+    for (int t = lane; t < R; t += QMLL_WAVE) gin[t] = gsrc[t];
+    for (int t = lane; t < nRs2; t += QMLL_WAVE) {
+        const float v = a.Rs2[t];
+        slnRs2[t] = logf(v);
+        sinvRs2[t] = 1.0f / v;
+    }
+    for (int t = lane; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
+    for (int t = lane; t < a.cap; t += QMLL_WAVE) {
+        sgx[t] = 0.0f;
+        sgy[t] = 0.0f;
+        sgz[t] = 0.0f;
+    }
+    const int nn = stage_neighbours(a, s, m, i, lane);
+    __syncthreads();
+
+    const float inv_rc = 1.0f / a.p.rcut;
+    float gix = 0.0f, giy = 0.0f, giz = 0.0f;
+
+    // two-body: lane per neighbour, serial over bins
+    for (int j = lane; j < nn; j += QMLL_WAVE) {
+        const float r = s.r[j];
+        const TwoBody tb = two_body_setup(r, a.p, inv_rc);
+        const float* g = gin + s.el[j] * nRs2;
+        float gr = 0.0f;
+        for (int z = 0; z < nRs2; ++z) {
+            float val, dval;
+            two_body_bin(tb, slnRs2[z], sinvRs2[z], val, dval);
+            gr = fmaf(g[z], dval, gr);
+        }
+        const float ir = 1.0f / r;
+        const float ux = s.dx[j] * ir, uy = s.dy[j] * ir, uz = s.dz[j] * ir;   // dr/dR_i
+        gix += gr * ux;
+        giy += gr * uy;
+        giz += gr * uz;
+        sgx[j] -= gr * ux;   // each lane owns its own j here
+        sgy[j] -= gr * uy;
+        sgz[j] -= gr * uz;
+    }
+    __syncthreads();
+
+    // three-body: lane per triple, serial over radial bins
+    const int ntrip = nn * (nn - 1) / 2;
+    const float zeta2 = 2.0f * expf(-0.5f * PI_F * PI_F);
+    for (int tt = lane; tt < ntrip; tt += QMLL_WAVE) {
+        int j, k;
+        unrank_pair(tt, nn, j, k);
+        const Triple t = triple_geometry(s, j, k);
+        const TripleDeriv d = triple_derivatives(t, a.p, inv_rc);
+        const float* g = gin + pair_offset(s.el[j], s.el[k], ns, nRs2, nRs3);
+        const float rho = 0.5f * (t.a + t.b);
+        float Gc = 0.f, Gs = 0.f, Hc = 0.f, Hs = 0.f;
+        for (int l = 0; l < nRs3; ++l) {
+            const float dl = rho - sRs3[l];
+            const float e = expf(-a.p.eta3 * dl * dl);
+            const float de = -2.0f * a.p.eta3 * dl * e;   // d e / d rho
+            const float gc = g[2 * l], gs = g[2 * l + 1];
+            Gc = fmaf(gc, e, Gc);
+            Gs = fmaf(gs, e, Gs);
+            Hc = fmaf(gc, de, Hc);
+            Hs = fmaf(gs, de, Hs);
+        }
+        const float S0 = Gc * t.cosT + Gs * t.sinT;
+        const float S1 = 0.5f * (Hc * t.cosT + Hs * t.sinT);                      // d rho/da = d rho/db = 1/2
+        const float Sth = (Gc * t.sinT - Gs * t.cosT) * t.guard_inv;               // multiplies d cos_i
+        const float Ea = zeta2 * (d.Ka * S0 + d.K * (S1 + Sth * d.cia));
+        const float Eb = zeta2 * (d.Kb * S0 + d.K * (S1 + Sth * d.cib));
+        const float Ec = zeta2 * (d.Kc * S0 + d.K * (Sth * d.cic));
+        const float ia = 1.0f / t.a, ib = 1.0f / t.b;
+        const float uax = s.dx[j] * ia, uay = s.dy[j] * ia, uaz = s.dz[j] * ia;   // u_ij
+        const float ubx = s.dx[k] * ib, uby = s.dy[k] * ib, ubz = s.dz[k] * ib;   // u_ik
+        gix += Ea * uax + Eb * ubx;
+        giy += Ea * uay + Eb * uby;
+        giz += Ea * uaz + Eb * ubz;
+        atomicAdd(&sgx[j], -Ea * uax + Ec * t.ujk[0]);
+        atomicAdd(&sgy[j], -Ea * uay + Ec * t.ujk[1]);
+        atomicAdd(&sgz[j], -Ea * uaz + Ec * t.ujk[2]);
+        atomicAdd(&sgx[k], -Eb * ubx - Ec * t.ujk[0]);
+        atomicAdd(&sgy[k], -Eb * uby - Ec * t.ujk[1]);
+        atomicAdd(&sgz[k], -Eb * ubz - Ec * t.ujk[2]);
+    }
+    __syncthreads();
+    gix = wave_sum(gix);
+    giy = wave_sum(giy);
+    giz = wave_sum(giz);
+    float* gm = grad_X + (size_t)m * a.n * 3;
+    if (lane == 0) {
+        atomicAdd(&gm[i * 3 + 0], gix);
+        atomicAdd(&gm[i * 3 + 1], giy);
+        atomicAdd(&gm[i * 3 + 2], giz);
+    }
+    for (int j = lane; j < nn; j += QMLL_WAVE) {
+        const int jj = s.j[j];
+        atomicAdd(&gm[jj * 3 + 0], sgx[j]);
+        atomicAdd(&gm[jj * 3 + 1], sgy[j]);
+        atomicAdd(&gm[jj * 3 + 2], sgz[j]);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// explicit Jacobian (and the representation itself when rep != NULL)
+//
+// Output-centric and atomic-free: the wavefront of central atom i produces, one target
+// atom at a time (i itself, then each neighbour), the three rows jac[m,i,target,0..2,:]
+// in an LDS row buffer and streams them out coalesced.  For a neighbour target only the
+// triples that contain it contribute; for the self row all triples do.
+// ---------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* __restrict__ rep,
+                                                              float* __restrict__ jac) {
+    extern __shared__ float smem[];
+    const int lane = threadIdx.x;
+    const int m = a.molIDs[blockIdx.x];
+    const int i = a.atomIDs[blockIdx.x];
+    if (m < 0 || m >= a.B || i < 0 || i >= a.n) return;   // malformed index: write nothing
+    const int ns = a.p.nspecies, nRs2 = a.p.nRs2, nRs3 = a.p.nRs3;
+    const int R = ns * nRs2 + ns * (ns + 1) * nRs3;
+
+    Stage s = carve(smem, a.cap);
+    float* slnRs2 = s.next;          // [nRs2]
+    float* sinvRs2 = slnRs2 + nRs2;  // [nRs2]
+    float* sRs3 = sinvRs2 + nRs2;    // [nRs3]
+    float* row = sRs3 + nRs3;        // [3][R] rows being assembled (+ [R] value row)
+    float* val = row + 3 * R;        // [R]   representation row (self pass only)
+
+    for (int t = lane; t < nRs2; t += QMLL_WAVE) {
+        const float v = a.Rs2[t];
+        slnRs2[t] = logf(v);
+        sinvRs2[t] = 1.0f / v;
+    }
+    for (int t = lane; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
+    const int nn = stage_neighbours(a, s, m, i, lane);
+    __syncthreads();
+
+    const float inv_rc = 1.0f / a.p.rcut;
+    const float zeta2 = 2.0f * expf(-0.5f * PI_F * PI_F);
+    float* jbase = jac + (((size_t)m * a.n + i) * a.n) * 3 * R;
+
+    // target = -1: central atom; target = 0..nn-1: neighbour at that list position
+    for (int target = -1; target < nn; ++target) {
+        for (int t = lane; t < 3 * R; t += QMLL_WAVE) row[t] = 0.0f;
+        if (target < 0)
+            for (int t = lane; t < R; t += QMLL_WAVE) val[t] = 0.0f;
+        __syncthreads();
+
+        // two-body: items (neighbour j, bin z); a neighbour target only sees its own pair
+        {
+            const int j0 = target < 0 ? 0 : target;
+            const int j1 = target < 0 ? nn : target + 1;
+            const float sign = target < 0 ? 1.0f : -1.0f;   // dr/dR_i = u_ij, dr/dR_j = -u_ij
+            for (int it = lane; it < (j1 - j0) * nRs2; it += QMLL_WAVE) {
+                const int j = j0 + it / nRs2;
+                const int z = it % nRs2;
+                const float r = s.r[j];
+                const TwoBody tb = two_body_setup(r, a.p, inv_rc);
+                float v, dv;
+                two_body_bin(tb, slnRs2[z], sinvRs2[z], v, dv);
+                const float ir = sign * dv / r;
+                const int bin = s.el[j] * nRs2 + z;
+                atomicAdd(&row[0 * R + bin], ir * s.dx[j]);
+                atomicAdd(&row[1 * R + bin], ir * s.dy[j]);
+                atomicAdd(&row[2 * R + bin], ir * s.dz[j]);
+                if (target < 0) atomicAdd(&val[bin], v);
+            }
+        }
+        // three-body: items (triple, radial bin l)
+        {
+            // self: all pairs (j<k); neighbour target: the nn-1 pairs {target, other}
+            const int ntr = target < 0 ? nn * (nn - 1) / 2 : nn - 1;
+            for (int it = lane; it < ntr * nRs3; it += QMLL_WAVE) {
+                const int tt = it / nRs3;
+                const int l = it - tt * nRs3;
+                int j, k;
+                if (target < 0) {
+                    unrank_pair(tt, nn, j, k);
+                } else {
+                    const int o = tt < target ? tt : tt + 1;
+                    j = o < target ? o : target;
+                    k = o < target ? target : o;
+                }
+                const Triple t = triple_geometry(s, j, k);
+                const TripleDeriv d = triple_derivatives(t, a.p, inv_rc);
+                const float rho = 0.5f * (t.a + t.b);
+                const float dl = rho - sRs3[l];
+                const float e = expf(-a.p.eta3 * dl * dl);
+                const float de = -a.p.eta3 * dl * e;          // (d e/d rho) * (d rho/d a)
+                // T_c = zeta2 K e cosT, T_s = zeta2 K e sinT; partials wrt a, b, c
+                const float dcos = t.sinT * t.guard_inv;       // d cosT = dcos * d cos_i
+                const float dsin = -t.cosT * t.guard_inv;      // d sinT = dsin * d cos_i
+                float Tca, Tcb, Tcc, Tsa, Tsb, Tsc;
+                {
+                    const float Ke = zeta2 * d.K * e;
+                    const float base_a = zeta2 * (d.Ka * e + d.K * de);
+                    const float base_b = zeta2 * (d.Kb * e + d.K * de);
+                    const float base_c = zeta2 * (d.Kc * e);
+                    Tca = base_a * t.cosT + Ke * dcos * d.cia;
+                    Tcb = base_b * t.cosT + Ke * dcos * d.cib;
+                    Tcc = base_c * t.cosT + Ke * dcos * d.cic;
+                    Tsa = base_a * t.sinT + Ke * dsin * d.cia;
+                    Tsb = base_b * t.sinT + Ke * dsin * d.cib;
+                    Tsc = base_c * t.sinT + Ke * dsin * d.cic;
+                    if (target < 0) {
+                        const int off = pair_offset(s.el[j], s.el[k], ns, nRs2, nRs3) + 2 * l;
+                        atomicAdd(&val[off], Ke * t.cosT);
+                        atomicAdd(&val[off + 1], Ke * t.sinT);
+                    }
+                }
+                const float ia = 1.0f / t.a, ib = 1.0f / t.b;
+                const float ua[3] = {s.dx[j] * ia, s.dy[j] * ia, s.dz[j] * ia};
+                const float ub[3] = {s.dx[k] * ib, s.dy[k] * ib, s.dz[k] * ib};
+                const int off = pair_offset(s.el[j], s.el[k], ns, nRs2, nRs3) + 2 * l;
+#pragma unroll
+                for (int x = 0; x < 3; ++x) {
+                    float gc, gs;
+                    if (target < 0) {            // d/dR_i
+                        gc = Tca * ua[x] + Tcb * ub[x];
+                        gs = Tsa * ua[x] + Tsb * ub[x];
+                    } else if (j == target) {    // d/dR_j
+                        gc = -Tca * ua[x] + Tcc * t.ujk[x];
+                        gs = -Tsa * ua[x] + Tsc * t.ujk[x];
+                    } else {                     // d/dR_k
+                        gc = -Tcb * ub[x] - Tcc * t.ujk[x];
+                        gs = -Tsb * ub[x] - Tsc * t.ujk[x];
+                    }
+                    atomicAdd(&row[x * R + off], gc);
+                    atomicAdd(&row[x * R + off + 1], gs);
+                }
+            }
+        }
+        __syncthreads();
+        const int tj = target < 0 ? i : s.j[target];
+        float* dst = jbase + (size_t)tj * 3 * R;
+        for (int t = lane; t < 3 * R; t += QMLL_WAVE) dst[t] = row[t];
+        if (target < 0 && rep != nullptr) {
+            float* out = rep + ((size_t)m * a.n + i) * R;
+            for (int t = lane; t < R; t += QMLL_WAVE) out[t] = val[t];
+        }
+        __syncthreads();
+    }
+}
+
+int fill_args(FchlArgs& a, const float* X, const int* types, const float* cell, const float* inv_cell,
+              const int* atomIDs, const int* molIDs, const int* natoms, const int* nlist, const int* nneigh,
+              int nn_stride, int A, int B, int n, const float* Rs2, const float* Rs3, const qmll_fchl_params* prm,
+              const char* who) {
+    QMLL_REQUIRE(prm != nullptr, QMLL_ERR_INVALID, "%s: null params", who);
+    QMLL_REQUIRE(A >= 0 && B >= 0 && n >= 0, QMLL_ERR_INVALID, "%s: negative size A=%d B=%d n=%d", who, A, B, n);
+    QMLL_REQUIRE(prm->nspecies > 0 && prm->nRs2 > 0 && prm->nRs3 > 0, QMLL_ERR_INVALID,
+                 "%s: nspecies=%d nRs2=%d nRs3=%d must be positive", who, prm->nspecies, prm->nRs2, prm->nRs3);
+    QMLL_REQUIRE(prm->rcut > 0.0f, QMLL_ERR_INVALID, "%s: rcut must be positive", who);
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(X && types && atomIDs && molIDs && natoms && Rs2 && Rs3, QMLL_ERR_INVALID, "%s: null pointer", who);
+    QMLL_REQUIRE((cell == nullptr) == (inv_cell == nullptr), QMLL_ERR_INVALID,
+                 "%s: cell and inv_cell must both be given or both be NULL", who);
+    QMLL_REQUIRE((nlist == nullptr) == (nneigh == nullptr), QMLL_ERR_INVALID,
+                 "%s: nlist and nneigh must both be given or both be NULL", who);
+    QMLL_REQUIRE(nlist == nullptr || nn_stride > 0, QMLL_ERR_INVALID, "%s: nn_stride=%d", who, nn_stride);
+    a.X = X;
+    a.types = types;
+    a.cell = cell;
+    a.inv_cell = inv_cell;
+    a.atomIDs = atomIDs;
+    a.molIDs = molIDs;
+    a.natoms = natoms;
+    a.nlist = nlist;
+    a.nneigh = nneigh;
+    a.nn_stride = nn_stride;
+    a.n = n;
+    a.B = B;
+    a.cap = nlist ? nn_stride : n;
+    if (a.cap < 1) a.cap = 1;
+    a.Rs2 = Rs2;
+    a.Rs3 = Rs3;
+    a.p = *prm;
+    return QMLL_OK;
+}
+
+constexpr size_t LDS_LIMIT = 64 * 1024;
+
+}  // namespace
+
+extern "C" int qmll_fchl19_forward(const float* X, const int* types, const float* cell, const float* inv_cell,
+                                   const int* atomIDs, const int* molIDs, const int* natoms, const int* nlist,
+                                   const int* nneigh, int nn_stride, int A, int B, int n, const float* Rs2,
+                                   const float* Rs3, const qmll_fchl_params* prm, float* rep, qmll_stream_t stream) {
+    FchlArgs a;
+    int rc = fill_args(a, X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, nn_stride, A, B, n, Rs2, Rs3,
+                       prm, "qmll_fchl19_forward");
+    if (rc) return rc;
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(rep != nullptr, QMLL_ERR_INVALID, "qmll_fchl19_forward: null output");
+    const int R = prm->nspecies * prm->nRs2 + prm->nspecies * (prm->nspecies + 1) * prm->nRs3;
+    const size_t lds = sizeof(float) * ((size_t)9 * a.cap + 2 * prm->nRs2 + prm->nRs3 + R + 4 * TCH);
+    QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
+                 "qmll_fchl19_forward: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R, LDS_LIMIT);
+    hipLaunchKernelGGL(fchl19_forward_kernel, dim3(A), dim3(64), lds, (hipStream_t)stream, a, rep);
+    QMLL_CHECK_LAUNCH("qmll_fchl19_forward");
+    return QMLL_OK;
+}
+
+extern "C" int qmll_fchl19_vjp(const float* X, const int* types, const float* cell, const float* inv_cell,
+                               const int* atomIDs, const int* molIDs, const int* natoms, const int* nlist,
+                               const int* nneigh, int nn_stride, int A, int B, int n, const float* Rs2, const float* Rs3,
+                               const qmll_fchl_params* prm, const float* grad_rep, float* grad_X,
+                               qmll_stream_t stream) {
+    FchlArgs a;
+    int rc = fill_args(a, X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, nn_stride, A, B, n, Rs2, Rs3,
+                       prm, "qmll_fchl19_vjp");
+    if (rc) return rc;
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(grad_rep && grad_X, QMLL_ERR_INVALID, "qmll_fchl19_vjp: null gradient pointer");
+    const int R = prm->nspecies * prm->nRs2 + prm->nspecies * (prm->nspecies + 1) * prm->nRs3;
+    const size_t lds = sizeof(float) * ((size_t)9 * a.cap + 2 * prm->nRs2 + prm->nRs3 + R);
+    QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
+                 "qmll_fchl19_vjp: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R, LDS_LIMIT);
+    hipLaunchKernelGGL(fchl19_vjp_kernel, dim3(A), dim3(64), lds, (hipStream_t)stream, a, grad_rep, grad_X);
+    QMLL_CHECK_LAUNCH("qmll_fchl19_vjp");
+    return QMLL_OK;
+}
+
+extern "C" int qmll_fchl19_jacobian(const float* X, const int* types, const float* cell, const float* inv_cell,
+                                    const int* atomIDs, const int* molIDs, const int* natoms, const int* nlist,
+                                    const int* nneigh, int nn_stride, int A, int B, int n, const float* Rs2,
+                                    const float* Rs3, const qmll_fchl_params* prm, float* rep, float* jac,
+                                    qmll_stream_t stream) {
+    FchlArgs a;
+    int rc = fill_args(a, X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, nn_stride, A, B, n, Rs2, Rs3,
+                       prm, "qmll_fchl19_jacobian");
+    if (rc) return rc;
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(jac != nullptr, QMLL_ERR_INVALID, "qmll_fchl19_jacobian: null output");
+    const int R = prm->nspecies * prm->nRs2 + prm->nspecies * (prm->nspecies + 1) * prm->nRs3;
+    const size_t lds = sizeof(float) * ((size_t)6 * a.cap + 2 * prm->nRs2 + prm->nRs3 + 4 * (size_t)R);
+    QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
+                 "qmll_fchl19_jacobian: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R,
+                 LDS_LIMIT);
+    hipLaunchKernelGGL(fchl19_jacobian_kernel, dim3(A), dim3(64), lds, (hipStream_t)stream, a, rep, jac);
+    QMLL_CHECK_LAUNCH("qmll_fchl19_jacobian");
+    return QMLL_OK;
+}

@@ -1,0 +1,241 @@
+// Normal-equation accumulation Z^T Z / Z^T y on the fp64 matrix cores of gfx950.
+// Replaces the torch.matmul calls of qml_lightning/models/kernel.py:172-192 and
+// qml_lightning/cuda/utils_kernel.cu:70-129 (matmul_and_reduce) of the reference.
+//
+// C[i,j] += sum_m Z[m,i] Z[m,j].  Z is row-major [M,F], so for a fixed m both operand
+// fragments are contiguous in memory: the A fragment of v_mfma_f64_16x16x4_f64 (16 rows i
+// x 4 steps k) is Z[m0+k, i0+i] and the B fragment is Z[m0+k, j0+j]; no transpose is
+// ever materialised.  A workgroup (256 threads, 4 wavefronts) owns a 128x128 tile of C;
+// each wavefront keeps a 64x64 sub-tile (4x4 MFMA tiles, 128 accumulator registers) and
+// the two 128-wide column panels of Z are staged through LDS KB rows at a time with the
+// next panel's global loads in flight during the MFMAs.  In the symmetric mode only tiles
+// on or above the diagonal are computed and the mirror image is written from the same
+// accumulators.  Algorithmic work: M*F*(F+1) flops, 8*M*F bytes read once (re-reads of a
+// panel by the tiles of one row/column are served from L2: consecutive workgroup ids walk
+// along a tile row).
+#include "qmll_common.h"
+
+namespace {
+
+typedef double double4_t __attribute__((ext_vector_type(4)));
+
+constexpr int TILE = 128;     // C tile edge per workgroup
+constexpr int KB = 16;        // rows of Z staged per step
+constexpr int GT = 256;       // threads
+constexpr int LDS_STRIDE = TILE + 2;   // doubles per staged row (pad: spreads the 4 k-rows over banks)
+
+// map a linear tile id to (ti, tj) with ti <= tj, walking row by row over the upper triangle
+__device__ __forceinline__ void upper_tile(int t, int nt, int& ti, int& tj) {
+    // row ti starts at offset ti*nt - ti(ti-1)/2
+    const float b = (float)(2 * nt + 1);
+    int r = (int)((b - sqrtf(fmaxf(b * b - 8.0f * (float)t, 0.0f))) * 0.5f);
+    if (r < 0) r = 0;
+    if (r > nt - 1) r = nt - 1;
+    while (r > 0 && r * nt - (r * (r - 1)) / 2 > t) --r;
+    while (r + 1 < nt && (r + 1) * nt - ((r + 1) * r) / 2 <= t) ++r;
+    ti = r;
+    tj = r + (t - (r * nt - (r * (r - 1)) / 2));
+}
+
+// SYM: C is [F,F], tiles ti<=tj, mirrored on store.  !SYM: rows f0..f1 of C, C_tile [f1-f0, F].
+template <bool SYM>
+__global__ __launch_bounds__(GT) void gram_kernel(const double* __restrict__ Z, int M, int F, int f0, int f1,
+                                                   int ntj, double* __restrict__ C) {
+    __shared__ double sA[KB][LDS_STRIDE];
+    __shared__ double sB[KB][LDS_STRIDE];
+
+    int ti, tj;
+    if (SYM) {
+        upper_tile(blockIdx.x, ntj, ti, tj);
+    } else {
+        ti = blockIdx.x / ntj;
+        tj = blockIdx.x % ntj;
+    }
+    const int i0 = f0 + ti * TILE;   // first feature of the A panel (rows of C)
+    const int j0 = tj * TILE;        // first feature of the B panel (columns of C)
+    const int ilim = SYM ? F : f1;
+    const bool same = SYM && ti == tj;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;   // wavefront's 64x64 sub-tile
+    const int l16 = lane & 15, lk = lane >> 4;
+
+    double4_t acc[4][4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[p][q] = (double4_t){0.0, 0.0, 0.0, 0.0};
+
+    // global -> register staging: KB x 128 doubles per panel = 2048; 256 threads x 8
+    // thread t loads row (t / 16) , columns (t % 16) * 8 .. +8   (KB = 16)
+    const int lr = tid >> 4;
+    const int lc = (tid & 15) * 8;
+    double ra[8], rb[8];
+
+    auto load_panels = [&](int m0) {
+        const int m = m0 + lr;
+        const bool rowok = m < M;
+        const double* zr = Z + (size_t)m * F;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const int ca = i0 + lc + q;
+            ra[q] = (rowok && ca < ilim) ? zr[ca] : 0.0;
+        }
+        if (!same) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int cb = j0 + lc + q;
+                rb[q] = (rowok && cb < F) ? zr[cb] : 0.0;
+            }
+        }
+    };
+    auto store_panels = [&]() {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) sA[lr][lc + q] = ra[q];
+        if (!same) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) sB[lr][lc + q] = rb[q];
+        }
+    };
+
+    const int nsteps = (M + KB - 1) / KB;
+    load_panels(0);
+    const double(*pa)[LDS_STRIDE] = sA;
+    const double(*pb)[LDS_STRIDE] = same ? sA : sB;
+    for (int step = 0; step < nsteps; ++step) {
+        __syncthreads();                 // everyone is done reading the previous panel
+        store_panels();
+        __syncthreads();
+        if (step + 1 < nsteps) load_panels((step + 1) * KB);   // in flight during the MFMAs
+#pragma unroll
+        for (int kk = 0; kk < KB; kk += 4) {
+            double fa[4], fb[4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) fa[p] = pa[kk + lk][wi + p * 16 + l16];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) fb[q] = pb[kk + lk][wj + q * 16 + l16];
+#pragma unroll
+            for (int p = 0; p < 4; ++p)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    acc[p][q] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[p], fb[q], acc[p][q], 0, 0, 0);
+        }
+    }
+
+    // accumulator layout of v_mfma_f64_16x16x4_f64: lane holds rows 4*(lane/16)+r, r=0..3,
+    // of column lane%16
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int gi = i0 + wi + p * 16 + lk * 4 + r;
+                const int gj = j0 + wj + q * 16 + l16;
+                if (gi < ilim && gj < F) {
+                    const double v = acc[p][q][r];
+                    if (SYM) {
+                        if (same) {
+                            C[(size_t)gi * F + gj] += v;      // the full diagonal tile was computed
+                        } else {
+                            C[(size_t)gi * F + gj] += v;
+                            C[(size_t)gj * F + gi] += v;
+                        }
+                    } else {
+                        C[(size_t)(gi - f0) * F + gj] += v;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ZTy[f] += sum_m Z[m,f] y[m] for f in [f0,f1): thread = feature, rows split over grid.y
+constexpr int GV_ROWS = 512;
+__global__ __launch_bounds__(256) void gemv_t_kernel(const double* __restrict__ Z, const double* __restrict__ y, int M,
+                                                      int F, int f0, int f1, double* __restrict__ out) {
+    const int f = f0 + blockIdx.x * 256 + threadIdx.x;
+    if (f >= f1) return;
+    const int m0 = blockIdx.y * GV_ROWS;
+    const int m1 = min(M, m0 + GV_ROWS);
+    double s = 0.0;
+    for (int m = m0; m < m1; ++m) s = fma(Z[(size_t)m * F + f], y[m], s);
+    unsafeAtomicAdd(&out[f], s);
+}
+
+// C += double(A.B) with the fp32 Kahan inner sum of the reference (utils_kernel.cu:104-117)
+constexpr int MR = 16;
+__global__ __launch_bounds__(MR* MR) void matmul_and_reduce_kernel(const float* __restrict__ A,
+                                                                   const float* __restrict__ B, int Ar, int K, int Bc,
+                                                                   double* __restrict__ C) {
+    __shared__ float As[MR][MR + 1];
+    __shared__ float Bs[MR][MR + 1];
+    const int tx = threadIdx.x % MR, ty = threadIdx.x / MR;
+    const int row = blockIdx.y * MR + ty, col = blockIdx.x * MR + tx;
+    float sum = 0.0f, c = 0.0f;
+    for (int k0 = 0; k0 < K; k0 += MR) {
+        As[ty][tx] = (row < Ar && k0 + tx < K) ? A[(size_t)row * K + k0 + tx] : 0.0f;
+        Bs[ty][tx] = (k0 + ty < K && col < Bc) ? B[(size_t)(k0 + ty) * Bc + col] : 0.0f;
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < MR; ++k) {
+            const float yv = __builtin_fmaf(As[ty][k], Bs[k][tx], -c);
+            const float t = sum + yv;
+            c = (t - sum) - yv;
+            sum = t;
+        }
+        __syncthreads();
+    }
+    if (row < Ar && col < Bc) C[(size_t)row * Bc + col] += (double)sum;
+}
+
+}  // namespace
+
+static int gram_launch(const double* Z, const double* y, int M, int F, int f0, int f1, bool sym, double* C,
+                       double* ZTy, hipStream_t stream, const char* who) {
+    QMLL_REQUIRE(M >= 0 && F > 0, QMLL_ERR_INVALID, "%s: bad size M=%d F=%d", who, M, F);
+    QMLL_REQUIRE(0 <= f0 && f0 < f1 && f1 <= F, QMLL_ERR_INVALID, "%s: bad feature range [%d,%d) of %d", who, f0, f1, F);
+    if (M == 0) return QMLL_OK;
+    QMLL_REQUIRE(Z && C, QMLL_ERR_INVALID, "%s: null pointer", who);
+    QMLL_REQUIRE((y == nullptr) == (ZTy == nullptr), QMLL_ERR_INVALID, "%s: y and ZTy must both be given or both be NULL",
+                 who);
+    const int ntj = (F + TILE - 1) / TILE;
+    if (sym) {
+        const long long ntiles = (long long)ntj * (ntj + 1) / 2;
+        QMLL_REQUIRE(ntiles < 2147483647LL, QMLL_ERR_INVALID, "%s: too many tiles", who);
+        hipLaunchKernelGGL(gram_kernel<true>, dim3((unsigned)ntiles), dim3(GT), 0, stream, Z, M, F, 0, F, ntj, C);
+    } else {
+        const int nti = (f1 - f0 + TILE - 1) / TILE;
+        hipLaunchKernelGGL(gram_kernel<false>, dim3((unsigned)(nti * ntj)), dim3(GT), 0, stream, Z, M, F, f0, f1, ntj, C);
+    }
+    QMLL_CHECK_LAUNCH(who);
+    if (y) {
+        dim3 grid((f1 - f0 + 255) / 256, (M + GV_ROWS - 1) / GV_ROWS);
+        hipLaunchKernelGGL(gemv_t_kernel, grid, dim3(256), 0, stream, Z, y, M, F, f0, f1, ZTy);
+        QMLL_CHECK_LAUNCH(who);
+    }
+    return QMLL_OK;
+}
+
+extern "C" int qmll_gram_f64(const double* Z, const double* y, int M, int F, double* ZTZ, double* ZTy,
+                             qmll_stream_t stream) {
+    return gram_launch(Z, y, M, F, 0, F > 0 ? F : 1, true, ZTZ, ZTy, (hipStream_t)stream, "qmll_gram_f64");
+}
+
+extern "C" int qmll_gram_tile_f64(const double* Z, const double* y, int M, int F, int f0, int f1, double* ZTZ_tile,
+                                  double* ZTy, qmll_stream_t stream) {
+    return gram_launch(Z, y, M, F, f0, f1, false, ZTZ_tile, ZTy, (hipStream_t)stream, "qmll_gram_tile_f64");
+}
+
+extern "C" int qmll_matmul_and_reduce(const float* A, const float* B, int Ar, int K, int Bc, double* C,
+                                      qmll_stream_t stream) {
+    QMLL_REQUIRE(Ar >= 0 && K >= 0 && Bc >= 0, QMLL_ERR_INVALID, "qmll_matmul_and_reduce: bad size %d %d %d", Ar, K, Bc);
+    if (Ar == 0 || Bc == 0) return QMLL_OK;
+    QMLL_REQUIRE(A && B && C, QMLL_ERR_INVALID, "qmll_matmul_and_reduce: null pointer");
+    dim3 grid((Bc + MR - 1) / MR, (Ar + MR - 1) / MR);
+    QMLL_REQUIRE(grid.y <= 65535, QMLL_ERR_INVALID, "qmll_matmul_and_reduce: too many rows (%d)", Ar);
+    hipLaunchKernelGGL(matmul_and_reduce_kernel, grid, dim3(MR * MR), 0, (hipStream_t)stream, A, B, Ar, K, Bc, C);
+    QMLL_CHECK_LAUNCH("qmll_matmul_and_reduce");
+    return QMLL_OK;
+}

@@ -1,0 +1,106 @@
+// Shared device/host helpers for the gfx950 kernels of libqmll.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/qmll.h"
+
+#define QMLL_WAVE 64
+
+// thread-local text of the last failure, returned by qmll_last_error()
+void qmll_set_error(const char* fmt, ...);
+
+#define QMLL_REQUIRE(cond, code, ...)          \
+    do {                                        \
+        if (!(cond)) {                          \
+            qmll_set_error(__VA_ARGS__);        \
+            return (code);                      \
+        }                                       \
+    } while (0)
+
+// call after every launch: a failed launch is reported, never swallowed
+#define QMLL_CHECK_LAUNCH(name)                                                         \
+    do {                                                                                \
+        hipError_t e__ = hipGetLastError();                                             \
+        if (e__ != hipSuccess) {                                                        \
+            qmll_set_error("%s: launch failed: %s", name, hipGetErrorString(e__));      \
+            return QMLL_ERR_LAUNCH;                                                     \
+        }                                                                               \
+    } while (0)
+
+static inline bool qmll_is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+static inline int qmll_log2(int v) {
+    int l = 0;
+    while ((1 << l) < v) ++l;
+    return l;
+}
+
+#ifdef __HIPCC__
+
+__device__ __forceinline__ int lane_id() { return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
+
+// value held by lane (lane ^ MASK); MASK is a power of two below 64
+template <int MASK>
+__device__ __forceinline__ float lane_xor(float v) {
+    int vi = __float_as_int(v);
+    int r;
+    if constexpr (MASK == 1) {
+        r = __builtin_amdgcn_update_dpp(0, vi, 0xB1, 0xf, 0xf, false);   // quad_perm [1,0,3,2]
+    } else if constexpr (MASK == 2) {
+        r = __builtin_amdgcn_update_dpp(0, vi, 0x4E, 0xf, 0xf, false);   // quad_perm [2,3,0,1]
+    } else if constexpr (MASK == 8) {
+        r = __builtin_amdgcn_update_dpp(0, vi, 0x128, 0xf, 0xf, false);  // row_ror:8
+    } else if constexpr (MASK == 4) {
+        r = __builtin_amdgcn_ds_swizzle(vi, 0x101F);                     // bit mode: and 0x1f, xor 4
+    } else if constexpr (MASK == 16) {
+        r = __builtin_amdgcn_ds_swizzle(vi, 0x401F);                     // bit mode: and 0x1f, xor 16
+    } else {
+        r = __shfl_xor(vi, MASK, 64);
+    }
+    return __int_as_float(r);
+}
+
+// sum over the 64 lanes, result in every lane
+__device__ __forceinline__ float wave_sum(float v) {
+    v += lane_xor<1>(v);
+    v += lane_xor<2>(v);
+    v += lane_xor<4>(v);
+    v += lane_xor<8>(v);
+    v += lane_xor<16>(v);
+    v += lane_xor<32>(v);
+    return v;
+}
+
+// sin and cos of an fp32 argument to ~1 ulp for |x| < 2^15 (3-term Cody-Waite reduction
+// by pi/2 with FMA, then minimax polynomials on [-pi/4, pi/4]); larger arguments take the
+// library routine.
+__device__ __forceinline__ void sincos_f32(float x, float* s, float* c) {
+    if (__builtin_expect(fabsf(x) > 32000.0f, 0)) {
+        sincosf(x, s, c);
+        return;
+    }
+    float kf = rintf(x * 0.63661977236758134308f);
+    int k = (int)kf;
+    float r = fmaf(kf, -1.57079601287841796875f, x);          // pi/2 split in three fp32 parts
+    r = fmaf(kf, -3.1391647326017846353352069854736328125e-07f, r);
+    r = fmaf(kf, -5.3903029534742383e-15f, r);
+    float r2 = r * r;
+    // sin(r) ~ r + r^3 * P(r^2), cos(r) ~ 1 - r^2/2 + r^4 * Q(r^2)
+    float ps = fmaf(r2, 2.86567956e-6f, -1.98559923e-4f);
+    ps = fmaf(ps, r2, 8.33338592e-3f);
+    ps = fmaf(ps, r2, -1.66666672e-1f);
+    float sr = fmaf(ps * r2, r, r);
+    float pc = fmaf(r2, 2.44677067e-5f, -1.38877297e-3f);
+    pc = fmaf(pc, r2, 4.16666567e-2f);
+    pc = fmaf(pc, r2, -0.5f);
+    float cr = fmaf(pc, r2, 1.0f);
+    float ss = (k & 1) ? cr : sr;
+    float cc = (k & 1) ? sr : cr;
+    if (k & 2) ss = -ss;
+    if ((k + 1) & 2) cc = -cc;
+    *s = ss;
+    *c = cc;
+}
+
+#endif  // __HIPCC__

@@ -1,0 +1,522 @@
+// SORF (sign diagonal . fast Walsh-Hadamard stacks), cos features and their derivatives
+// for gfx950.  Replaces qml_lightning/cuda/hadamard_kernel.cu of the reference
+// (kernels :5-102, :204-312, :424-539, :541-585, :587-717, :778-839).
+//
+// A length-d transform lives in the registers of one wavefront: lane L holds the EPL =
+// d/64 consecutive elements L*EPL .. L*EPL+EPL-1 (d < 64: 64/d transforms share a
+// wavefront, one element per lane).  Butterflies over the low log2(EPL) index bits are
+// register-to-register; the six lane-index bits go through DPP (xor 1, 2, 8), ds_swizzle
+// (xor 4, 16) and a cross-half exchange (xor 32).  The stages of a Walsh-Hadamard
+// transform commute, so this order gives the reference's natural-order result.  The
+// H/sqrt(d) scalings of the T chained transforms and the coefficient normalisation are
+// folded into one multiply.  No LDS is used for the transform itself.
+//
+// Two-op contract (coefficients materialised, [A,S,d] fp32): both ops are HBM bound,
+// 4d + 4Sd bytes per atom forward.  The fused kernel keeps coefficients in registers and is
+// VALU bound (one sincos per feature).
+#include "qmll_common.h"
+
+namespace {
+
+template <int EPL>
+__device__ __forceinline__ void load_vec(float (&v)[EPL], const float* __restrict__ p) {
+    if constexpr (EPL == 1) {
+        v[0] = p[0];
+    } else if constexpr (EPL == 2) {
+        const float2 t = *reinterpret_cast<const float2*>(p);
+        v[0] = t.x;
+        v[1] = t.y;
+    } else {
+#pragma unroll
+        for (int q = 0; q < EPL / 4; ++q) {
+            const float4 t = reinterpret_cast<const float4*>(p)[q];
+            v[4 * q + 0] = t.x;
+            v[4 * q + 1] = t.y;
+            v[4 * q + 2] = t.z;
+            v[4 * q + 3] = t.w;
+        }
+    }
+}
+
+template <int EPL>
+__device__ __forceinline__ void store_vec(const float (&v)[EPL], float* __restrict__ p) {
+    if constexpr (EPL == 1) {
+        p[0] = v[0];
+    } else if constexpr (EPL == 2) {
+        *reinterpret_cast<float2*>(p) = make_float2(v[0], v[1]);
+    } else {
+#pragma unroll
+        for (int q = 0; q < EPL / 4; ++q)
+            reinterpret_cast<float4*>(p)[q] = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+    }
+}
+
+template <int MASK>
+__device__ __forceinline__ float butterfly(float v, int lane) {
+    const float p = lane_xor<MASK>(v);
+    return (lane & MASK) ? p - v : v + p;
+}
+
+// unnormalised Walsh-Hadamard transform of the d = EPL*LANES values held by LANES lanes
+template <int EPL, int LANES>
+__device__ __forceinline__ void fwht_wave(float (&v)[EPL], int lane) {
+#pragma unroll
+    for (int h = 1; h < EPL; h <<= 1) {
+#pragma unroll
+        for (int q = 0; q < EPL; ++q) {
+            if ((q & h) == 0) {
+                const float a = v[q], b = v[q + h];
+                v[q] = a + b;
+                v[q + h] = a - b;
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < EPL; ++q) {
+        float t = v[q];
+        if constexpr (LANES > 1) t = butterfly<1>(t, lane);
+        if constexpr (LANES > 2) t = butterfly<2>(t, lane);
+        if constexpr (LANES > 4) t = butterfly<4>(t, lane);
+        if constexpr (LANES > 8) t = butterfly<8>(t, lane);
+        if constexpr (LANES > 16) t = butterfly<16>(t, lane);
+        if constexpr (LANES > 32) t = butterfly<32>(t, lane);
+        v[q] = t;
+    }
+}
+
+template <int LOG2D>
+struct Shape {
+    static constexpr int d = 1 << LOG2D;
+    static constexpr int EPL = d >= 64 ? d / 64 : 1;
+    static constexpr int LANES = d >= 64 ? 64 : d;
+    static constexpr int G = 64 / LANES;   // transforms per wavefront
+};
+
+// forward chain for stack s: v <- prod_m H diag(D[m,s]) v   (unnormalised)
+template <int LOG2D>
+__device__ __forceinline__ void chain_forward(float (&v)[Shape<LOG2D>::EPL], const float* __restrict__ D, int S, int T,
+                                              int s, int e0, int lane) {
+    using Sh = Shape<LOG2D>;
+    for (int m = 0; m < T; ++m) {
+        float dv[Sh::EPL];
+        load_vec<Sh::EPL>(dv, D + ((size_t)m * S + s) * Sh::d + e0);
+#pragma unroll
+        for (int q = 0; q < Sh::EPL; ++q) v[q] *= dv[q];
+        fwht_wave<Sh::EPL, Sh::LANES>(v, lane);
+    }
+}
+
+// adjoint chain: v <- prod_{m=T-1..0} diag(D[m,s]) H v   (unnormalised)
+template <int LOG2D>
+__device__ __forceinline__ void chain_adjoint(float (&v)[Shape<LOG2D>::EPL], const float* __restrict__ D, int S, int T,
+                                              int s, int e0, int lane) {
+    using Sh = Shape<LOG2D>;
+    for (int m = T - 1; m >= 0; --m) {
+        fwht_wave<Sh::EPL, Sh::LANES>(v, lane);
+        float dv[Sh::EPL];
+        load_vec<Sh::EPL>(dv, D + ((size_t)m * S + s) * Sh::d + e0);
+#pragma unroll
+        for (int q = 0; q < Sh::EPL; ++q) v[q] *= dv[q];
+    }
+}
+
+constexpr int SORF_THREADS = 256;
+constexpr int SORF_WAVES = SORF_THREADS / 64;
+
+// ---- two-op contract: coefficients ------------------------------------------------
+template <int LOG2D>
+__global__ __launch_bounds__(SORF_THREADS) void sorf_forward_kernel(const float* __restrict__ x,
+                                                                     const float* __restrict__ D, int S, int T,
+                                                                     float scale, float* __restrict__ out) {
+    using Sh = Shape<LOG2D>;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub = lane / Sh::LANES, l = lane % Sh::LANES;
+    const int e0 = l * Sh::EPL;
+    const size_t a = blockIdx.x;
+    float xv[Sh::EPL];
+    load_vec<Sh::EPL>(xv, x + a * Sh::d + e0);
+    const int step = SORF_WAVES * gridDim.y * Sh::G;
+    for (int s = (blockIdx.y * SORF_WAVES + wave) * Sh::G + sub; s < S; s += step) {
+        float v[Sh::EPL];
+#pragma unroll
+        for (int q = 0; q < Sh::EPL; ++q) v[q] = xv[q];
+        chain_forward<LOG2D>(v, D, S, T, s, e0, lane);
+#pragma unroll
+        for (int q = 0; q < Sh::EPL; ++q) v[q] *= scale;
+        store_vec<Sh::EPL>(v, out + (a * S + s) * Sh::d + e0);
+    }
+}
+
+// ---- two-op contract: adjoint summed over stacks ----------------------------------
+template <int LOG2D>
+__global__ __launch_bounds__(SORF_THREADS) void sorf_adjoint_kernel(const float* __restrict__ g,
+                                                                     const float* __restrict__ D, int S, int T,
+                                                                     float scale, float* __restrict__ gx) {
+    using Sh = Shape<LOG2D>;
+    __shared__ float red[SORF_WAVES][Sh::d];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub = lane / Sh::LANES, l = lane % Sh::LANES;
+    const int e0 = l * Sh::EPL;
+    const size_t a = blockIdx.x;
+    float acc[Sh::EPL];
+#pragma unroll
+    for (int q = 0; q < Sh::EPL; ++q) acc[q] = 0.0f;
+    for (int s = wave * Sh::G + sub; s < S; s += SORF_WAVES * Sh::G) {
+        float v[Sh::EPL];
+        load_vec<Sh::EPL>(v, g + (a * S + s) * Sh::d + e0);
+        chain_adjoint<LOG2D>(v, D, S, T, s, e0, lane);
+#pragma unroll
+        for (int q = 0; q < Sh::EPL; ++q) acc[q] += v[q];
+    }
+    // fold the 64/d transforms that share a wavefront (d < 64)
+    if constexpr (Sh::G > 1) {
+#pragma unroll
+        for (int mask = Sh::LANES; mask < 64; mask <<= 1) acc[0] += __shfl_xor(acc[0], mask, 64);
+    }
+    if (sub == 0) {
+#pragma unroll
+        for (int q = 0; q < Sh::EPL; ++q) red[wave][e0 + q] = acc[q];
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < Sh::d; e += SORF_THREADS) {
+        float t = 0.0f;
+#pragma unroll
+        for (int w = 0; w < SORF_WAVES; ++w) t += red[w][e];
+        gx[a * Sh::d + e] = scale * t;
+    }
+}
+
+// ---- fused predict path ------------------------------------------------------------
+template <int LOG2D, bool WITH_GRAD>
+__global__ __launch_bounds__(SORF_THREADS) void sorf_energy_fused_kernel(
+    const float* __restrict__ x, const float* __restrict__ D, const float* __restrict__ bias,
+    const float* __restrict__ alpha, const int* __restrict__ out_index, int S, int T, float scale, float normf,
+    float* __restrict__ e_atom, float* __restrict__ gx) {
+    using Sh = Shape<LOG2D>;
+    __shared__ float red[SORF_WAVES][Sh::d];
+    __shared__ float ered[SORF_WAVES];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub = lane / Sh::LANES, l = lane % Sh::LANES;
+    const int e0 = l * Sh::EPL;
+    const size_t a = blockIdx.x;
+    float xv[Sh::EPL], acc[Sh::EPL];
+    load_vec<Sh::EPL>(xv, x + a * Sh::d + e0);
+#pragma unroll
+    for (int q = 0; q < Sh::EPL; ++q) acc[q] = 0.0f;
+    float energy = 0.0f;
+    for (int s = wave * Sh::G + sub; s < S; s += SORF_WAVES * Sh::G) {
+        float v[Sh::EPL], bv[Sh::EPL], av[Sh::EPL];
+#pragma unroll
+        for (int q = 0; q < Sh::EPL; ++q) v[q] = xv[q];
+        chain_forward<LOG2D>(v, D, S, T, s, e0, lane);
+        load_vec<Sh::EPL>(bv, bias + (size_t)s * Sh::d + e0);
+        load_vec<Sh::EPL>(av, alpha + (size_t)s * Sh::d + e0);
+#pragma unroll
+        for (int q = 0; q < Sh::EPL; ++q) {
+            float sn, cs;
+            sincos_f32(fmaf(v[q], scale, bv[q]), &sn, &cs);
+            const float w = av[q] * normf;
+            energy = fmaf(w, cs, energy);
+            v[q] = -w * sn;                       // d E / d coefficient
+        }
+        if constexpr (WITH_GRAD) {
+            chain_adjoint<LOG2D>(v, D, S, T, s, e0, lane);
+#pragma unroll
+            for (int q = 0; q < Sh::EPL; ++q) acc[q] += v[q];
+        }
+    }
+    energy = wave_sum(energy);
+    if (lane == 0) ered[wave] = energy;
+    if constexpr (WITH_GRAD) {
+        if constexpr (Sh::G > 1) {
+#pragma unroll
+            for (int mask = Sh::LANES; mask < 64; mask <<= 1) acc[0] += __shfl_xor(acc[0], mask, 64);
+        }
+        if (sub == 0) {
+#pragma unroll
+            for (int q = 0; q < Sh::EPL; ++q) red[wave][e0 + q] = acc[q];
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = 0.0f;
+#pragma unroll
+        for (int w = 0; w < SORF_WAVES; ++w) t += ered[w];
+        e_atom[out_index ? out_index[a] : (int)a] = t;
+    }
+    if constexpr (WITH_GRAD) {
+        for (int e = threadIdx.x; e < Sh::d; e += SORF_THREADS) {
+            float t = 0.0f;
+#pragma unroll
+            for (int w = 0; w < SORF_WAVES; ++w) t += red[w][e];
+            gx[a * Sh::d + e] = scale * t;
+        }
+    }
+}
+
+// ---- derivative (force) features ----------------------------------------------------
+// One workgroup per (atom a, target atom j): for x in 0..2 and every stack, the chain of
+// u = input_derivative[a,j,x,:] times cos_derivs[a,:] is added into G[mol(a),j,x,:].
+// Several atoms of one molecule add into the same row, hence the fp64 atomics (the
+// reference does the same, hadamard_kernel.cu:712).  All-zero u rows (targets that are
+// not neighbours of a) are skipped.
+template <int LOG2D>
+__global__ __launch_bounds__(SORF_THREADS) void derivative_features_kernel(
+    const double* __restrict__ cos_derivs, double normalisation, const int* __restrict__ mol_index,
+    const float* __restrict__ input_derivative, const float* __restrict__ D, int n, int S, int T, float hscale,
+    double* __restrict__ G) {
+    using Sh = Shape<LOG2D>;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub = lane / Sh::LANES, l = lane % Sh::LANES;
+    const int e0 = l * Sh::EPL;
+    const size_t a = blockIdx.x / n;
+    const int j = blockIdx.x % n;
+    const int mol = mol_index[a];
+    const size_t F = (size_t)S * Sh::d;
+    for (int xc = 0; xc < 3; ++xc) {
+        float uv[Sh::EPL];
+        load_vec<Sh::EPL>(uv, input_derivative + ((a * n + j) * 3 + xc) * Sh::d + e0);
+        float nz = 0.0f;
+#pragma unroll
+        for (int q = 0; q < Sh::EPL; ++q) nz += fabsf(uv[q]);
+        if (__ballot(nz != 0.0f) == 0ull) continue;    // wave-uniform: nothing to add
+        double* Grow = G + (((size_t)mol * n + j) * 3 + xc) * F;
+        for (int s = wave * Sh::G + sub; s < S; s += SORF_WAVES * Sh::G) {
+            float v[Sh::EPL];
+#pragma unroll
+            for (int q = 0; q < Sh::EPL; ++q) v[q] = uv[q];
+            chain_forward<LOG2D>(v, D, S, T, s, e0, lane);
+#pragma unroll
+            for (int q = 0; q < Sh::EPL; ++q) {
+                const size_t f = (size_t)s * Sh::d + e0 + q;
+                const double val = normalisation * cos_derivs[a * F + f] * (double)(v[q] * hscale);
+                unsafeAtomicAdd(&Grow[f], val);
+            }
+        }
+    }
+}
+
+// ---- elementwise feature kernels ----------------------------------------------------
+// Thread = feature column f, workgroup = (feature tile, atom chunk).  Within its chunk a
+// thread keeps a running sum while consecutive atoms belong to the same molecule and
+// flushes it with one atomic when the molecule changes: atoms arrive molecule-major, so
+// this is about one atomic per (molecule, feature) instead of one per (atom, feature).
+constexpr int CF_THREADS = 256;
+constexpr int CF_ATOMS = 32;
+
+template <typename OutT>
+__global__ __launch_bounds__(CF_THREADS) void cos_features_kernel(const float* __restrict__ coeffs,
+                                                                   const float* __restrict__ bias,
+                                                                   const int* __restrict__ mol_index, int A, int F,
+                                                                   int nmol, float normf, OutT* __restrict__ Zf) {
+    const int f = blockIdx.y * CF_THREADS + threadIdx.x;
+    if (f >= F) return;
+    const int a0 = blockIdx.x * CF_ATOMS;
+    const int a1 = min(A, a0 + CF_ATOMS);
+    const float b = bias[f];
+    int cur = -1;
+    OutT run = 0;
+    for (int a = a0; a < a1; ++a) {
+        const int mol = mol_index[a];
+        if (mol != cur) {
+            if (cur >= 0 && cur < nmol) unsafeAtomicAdd(&Zf[(size_t)cur * F + f], run);
+            cur = mol;
+            run = 0;
+        }
+        float sn, cs;
+        sincos_f32(coeffs[(size_t)a * F + f] + b, &sn, &cs);
+        run += (OutT)(cs * normf);
+    }
+    if (cur >= 0 && cur < nmol) unsafeAtomicAdd(&Zf[(size_t)cur * F + f], run);
+}
+
+__global__ __launch_bounds__(CF_THREADS) void cos_features_backward_kernel(const float* __restrict__ gZ,
+                                                                            const float* __restrict__ coeffs,
+                                                                            const float* __restrict__ bias,
+                                                                            const int* __restrict__ mol_index, int F,
+                                                                            int nmol, float normf,
+                                                                            float* __restrict__ gc) {
+    const int f = blockIdx.y * CF_THREADS + threadIdx.x;
+    if (f >= F) return;
+    const size_t a = blockIdx.x;
+    const int mol = mol_index[a];
+    float sn, cs;
+    sincos_f32(coeffs[a * F + f] + bias[f], &sn, &cs);
+    const float gz = (mol >= 0 && mol < nmol) ? gZ[(size_t)mol * F + f] : 0.0f;
+    gc[a * F + f] = gz * -sn * normf;
+}
+
+__global__ __launch_bounds__(CF_THREADS) void sin_coeffs_kernel(const float* __restrict__ coeffs,
+                                                                 const float* __restrict__ bias, int F, float normf,
+                                                                 double* __restrict__ out) {
+    const int f = blockIdx.y * CF_THREADS + threadIdx.x;
+    if (f >= F) return;
+    const size_t a = blockIdx.x;
+    float sn, cs;
+    sincos_f32(coeffs[a * F + f] + bias[f], &sn, &cs);
+    out[a * F + f] = (double)(sn * normf);
+}
+
+int check_sorf(const char* who, int A, int d, int S, int T) {
+    QMLL_REQUIRE(A >= 0 && S > 0 && T > 0, QMLL_ERR_INVALID, "%s: bad size A=%d S=%d T=%d", who, A, S, T);
+    QMLL_REQUIRE(qmll_is_pow2(d), QMLL_ERR_NOT_POW2, "%s: input size must be power of 2. (got %d)", who, d);
+    QMLL_REQUIRE(d >= 2 && d <= 2048, QMLL_ERR_INVALID, "%s: transform length %d outside [2, 2048]", who, d);
+    return QMLL_OK;
+}
+
+// total scale of T chained H/sqrt(d) transforms
+float hnorm(int d, int T) { return powf(2.0f, -0.5f * (float)qmll_log2(d) * (float)T); }
+
+#define DISPATCH_LOG2D(log2d, CALL)   \
+    switch (log2d) {                  \
+        case 1: { CALL(1); } break;   \
+        case 2: { CALL(2); } break;   \
+        case 3: { CALL(3); } break;   \
+        case 4: { CALL(4); } break;   \
+        case 5: { CALL(5); } break;   \
+        case 6: { CALL(6); } break;   \
+        case 7: { CALL(7); } break;   \
+        case 8: { CALL(8); } break;   \
+        case 9: { CALL(9); } break;   \
+        case 10: { CALL(10); } break; \
+        case 11: { CALL(11); } break; \
+        default: break;               \
+    }
+
+}  // namespace
+
+extern "C" int qmll_sorf_forward(const float* x, const float* D, int A, int d, int S, int T, float normalisation,
+                                 float* out, qmll_stream_t stream) {
+    int rc = check_sorf("qmll_sorf_forward", A, d, S, T);
+    if (rc) return rc;
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(x && D && out, QMLL_ERR_INVALID, "qmll_sorf_forward: null pointer");
+    const float scale = normalisation * hnorm(d, T);
+    const int G = d >= 64 ? 1 : 64 / d;
+    int ny = (S + SORF_WAVES * G - 1) / (SORF_WAVES * G);
+    if (ny > 8) ny = 8;   // each wavefront streams >= S/32 stacks: keeps the x row and D hot
+    dim3 grid(A, ny);
+#define CALL(L) \
+    hipLaunchKernelGGL(sorf_forward_kernel<L>, grid, dim3(SORF_THREADS), 0, (hipStream_t)stream, x, D, S, T, scale, out)
+    DISPATCH_LOG2D(qmll_log2(d), CALL)
+#undef CALL
+    QMLL_CHECK_LAUNCH("qmll_sorf_forward");
+    return QMLL_OK;
+}
+
+extern "C" int qmll_sorf_adjoint(const float* g, const float* D, int A, int d, int S, int T, float normalisation,
+                                 float* gx, qmll_stream_t stream) {
+    int rc = check_sorf("qmll_sorf_adjoint", A, d, S, T);
+    if (rc) return rc;
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(g && D && gx, QMLL_ERR_INVALID, "qmll_sorf_adjoint: null pointer");
+    const float scale = normalisation * hnorm(d, T);
+#define CALL(L) \
+    hipLaunchKernelGGL(sorf_adjoint_kernel<L>, dim3(A), dim3(SORF_THREADS), 0, (hipStream_t)stream, g, D, S, T, scale, gx)
+    DISPATCH_LOG2D(qmll_log2(d), CALL)
+#undef CALL
+    QMLL_CHECK_LAUNCH("qmll_sorf_adjoint");
+    return QMLL_OK;
+}
+
+extern "C" int qmll_sorf_energy_fused(const float* x, const float* D, const float* bias, const float* alpha,
+                                      const int* out_index, int A, int d, int S, int T, float normalisation,
+                                      float* e_atom, float* gx, qmll_stream_t stream) {
+    int rc = check_sorf("qmll_sorf_energy_fused", A, d, S, T);
+    if (rc) return rc;
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(x && D && bias && alpha && e_atom, QMLL_ERR_INVALID, "qmll_sorf_energy_fused: null pointer");
+    const float scale = normalisation * hnorm(d, T);
+    const float normf = sqrtf(2.0f / ((float)S * (float)d));
+#define CALL(L)                                                                                                      \
+    if (gx)                                                                                                          \
+        hipLaunchKernelGGL((sorf_energy_fused_kernel<L, true>), dim3(A), dim3(SORF_THREADS), 0, (hipStream_t)stream, \
+                           x, D, bias, alpha, out_index, S, T, scale, normf, e_atom, gx);                            \
+    else                                                                                                             \
+        hipLaunchKernelGGL((sorf_energy_fused_kernel<L, false>), dim3(A), dim3(SORF_THREADS), 0, (hipStream_t)stream, \
+                           x, D, bias, alpha, out_index, S, T, scale, normf, e_atom, gx)
+    DISPATCH_LOG2D(qmll_log2(d), CALL)
+#undef CALL
+    QMLL_CHECK_LAUNCH("qmll_sorf_energy_fused");
+    return QMLL_OK;
+}
+
+extern "C" int qmll_derivative_features(const double* cos_derivs, double normalisation, const int* mol_index,
+                                        const float* input_derivative, const float* D, int A, int n, int d, int S,
+                                        int T, int nmol, double* G, qmll_stream_t stream) {
+    int rc = check_sorf("qmll_derivative_features", A, d, S, T);
+    if (rc) return rc;
+    QMLL_REQUIRE(n >= 0 && nmol >= 0, QMLL_ERR_INVALID, "qmll_derivative_features: bad size n=%d nmol=%d", n, nmol);
+    if (A == 0 || n == 0) return QMLL_OK;
+    QMLL_REQUIRE(cos_derivs && mol_index && input_derivative && D && G, QMLL_ERR_INVALID,
+                 "qmll_derivative_features: null pointer");
+    QMLL_REQUIRE((long long)A * n < 2147483647LL, QMLL_ERR_INVALID, "qmll_derivative_features: A*n too large");
+    const float hscale = hnorm(d, T);
+#define CALL(L)                                                                                                   \
+    hipLaunchKernelGGL(derivative_features_kernel<L>, dim3((unsigned)(A * n)), dim3(SORF_THREADS), 0,             \
+                       (hipStream_t)stream, cos_derivs, normalisation, mol_index, input_derivative, D, n, S, T, \
+                       hscale, G)
+    DISPATCH_LOG2D(qmll_log2(d), CALL)
+#undef CALL
+    QMLL_CHECK_LAUNCH("qmll_derivative_features");
+    return QMLL_OK;
+}
+
+static int check_feat(const char* who, int A, int F, int nmol) {
+    QMLL_REQUIRE(A >= 0 && F > 0 && nmol >= 0, QMLL_ERR_INVALID, "%s: bad size A=%d F=%d nmol=%d", who, A, F, nmol);
+    QMLL_REQUIRE(F <= 65535 * CF_THREADS, QMLL_ERR_INVALID, "%s: too many features (%d)", who, F);
+    return QMLL_OK;
+}
+
+extern "C" int qmll_cos_features_f32(const float* coeffs, const float* bias, const int* mol_index, int A, int F,
+                                     int nmol, float* Zf, qmll_stream_t stream) {
+    int rc = check_feat("qmll_cos_features_f32", A, F, nmol);
+    if (rc) return rc;
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(coeffs && bias && mol_index && Zf, QMLL_ERR_INVALID, "qmll_cos_features_f32: null pointer");
+    dim3 grid((A + CF_ATOMS - 1) / CF_ATOMS, (F + CF_THREADS - 1) / CF_THREADS);
+    hipLaunchKernelGGL(cos_features_kernel<float>, grid, dim3(CF_THREADS), 0, (hipStream_t)stream, coeffs, bias,
+                       mol_index, A, F, nmol, sqrtf(2.0f / (float)F), Zf);
+    QMLL_CHECK_LAUNCH("qmll_cos_features_f32");
+    return QMLL_OK;
+}
+
+extern "C" int qmll_cos_features_f64(const float* coeffs, const float* bias, const int* mol_index, int A, int F,
+                                     int nmol, double* Zf, qmll_stream_t stream) {
+    int rc = check_feat("qmll_cos_features_f64", A, F, nmol);
+    if (rc) return rc;
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(coeffs && bias && mol_index && Zf, QMLL_ERR_INVALID, "qmll_cos_features_f64: null pointer");
+    dim3 grid((A + CF_ATOMS - 1) / CF_ATOMS, (F + CF_THREADS - 1) / CF_THREADS);
+    hipLaunchKernelGGL(cos_features_kernel<double>, grid, dim3(CF_THREADS), 0, (hipStream_t)stream, coeffs, bias,
+                       mol_index, A, F, nmol, sqrtf(2.0f / (float)F), Zf);
+    QMLL_CHECK_LAUNCH("qmll_cos_features_f64");
+    return QMLL_OK;
+}
+
+extern "C" int qmll_cos_features_backward(const float* gZ, const float* coeffs, const float* bias,
+                                          const int* mol_index, int A, int F, int nmol, float* gc,
+                                          qmll_stream_t stream) {
+    int rc = check_feat("qmll_cos_features_backward", A, F, nmol);
+    if (rc) return rc;
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(gZ && coeffs && bias && mol_index && gc, QMLL_ERR_INVALID, "qmll_cos_features_backward: null pointer");
+    dim3 grid(A, (F + CF_THREADS - 1) / CF_THREADS);
+    hipLaunchKernelGGL(cos_features_backward_kernel, grid, dim3(CF_THREADS), 0, (hipStream_t)stream, gZ, coeffs, bias,
+                       mol_index, F, nmol, sqrtf(2.0f / (float)F), gc);
+    QMLL_CHECK_LAUNCH("qmll_cos_features_backward");
+    return QMLL_OK;
+}
+
+extern "C" int qmll_sin_coeffs_f64(const float* coeffs, const float* bias, int A, int F, double* out,
+                                   qmll_stream_t stream) {
+    int rc = check_feat("qmll_sin_coeffs_f64", A, F, 0);
+    if (rc) return rc;
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(coeffs && bias && out, QMLL_ERR_INVALID, "qmll_sin_coeffs_f64: null pointer");
+    dim3 grid(A, (F + CF_THREADS - 1) / CF_THREADS);
+    hipLaunchKernelGGL(sin_coeffs_kernel, grid, dim3(CF_THREADS), 0, (hipStream_t)stream, coeffs, bias, F,
+                       sqrtf(2.0f / (float)F), out);
+    QMLL_CHECK_LAUNCH("qmll_sin_coeffs_f64");
+    return QMLL_OK;
+}

@@ -1,0 +1,67 @@
+"""Drop-in for the reference's `fchl_gpu` extension (qml_lightning/cuda/fchl_cuda.cpp:204-212).
+Argument order is the reference's; the charges argument is accepted and unused by the
+kernels there too (element types carry the information)."""
+from .. import ops
+
+
+def _prm(species, Rs2, Rs3, eta2, eta3, two_body_decay, three_body_weight, three_body_decay, rcut):
+    return ops.make_params(species.shape[0], Rs2, Rs3, eta2, eta3, two_body_decay, three_body_weight,
+                           three_body_decay, rcut)
+
+
+def get_element_types_gpu(coordinates, charges, natom_counts, species):
+    return ops.element_types(coordinates, charges, natom_counts, species)
+
+
+def get_fchl_representation(coordinates, charges, species, element_types, cell, inv_cell, blockAtomIDs, blockMolIDs,
+                            neighbourlist, nneighbours, two_body_gridpoints, three_body_gridpoints, eta2, eta3,
+                            two_body_decay, three_body_weight, three_body_decay, rcut):
+    prm = _prm(species, two_body_gridpoints, three_body_gridpoints, eta2, eta3, two_body_decay, three_body_weight,
+               three_body_decay, rcut)
+    return ops.fchl_forward(coordinates, element_types, cell, inv_cell, blockAtomIDs, blockMolIDs,
+                            _counts(coordinates, nneighbours), two_body_gridpoints, three_body_gridpoints, prm,
+                            neighbourlist, nneighbours)
+
+
+def get_fchl_derivative(coordinates, charges, species, element_types, cell, inv_cell, blockAtomIDs, blockMolIDs,
+                        neighbourlist, nneighbours, two_body_gridpoints, three_body_gridpoints, eta2, eta3,
+                        two_body_decay, three_body_weight, three_body_decay, rcut):
+    prm = _prm(species, two_body_gridpoints, three_body_gridpoints, eta2, eta3, two_body_decay, three_body_weight,
+               three_body_decay, rcut)
+    _, jac = ops.fchl_jacobian(coordinates, element_types, cell, inv_cell, blockAtomIDs, blockMolIDs,
+                               _counts(coordinates, nneighbours), two_body_gridpoints, three_body_gridpoints, prm,
+                               neighbourlist, nneighbours, with_rep=False)
+    return jac
+
+
+def get_fchl_and_derivative(coordinates, charges, species, element_types, cell, inv_cell, blockAtomIDs, blockMolIDs,
+                            neighbourlist, nneighbours, two_body_gridpoints, three_body_gridpoints, eta2, eta3,
+                            two_body_decay, three_body_weight, three_body_decay, rcut, gradients):
+    prm = _prm(species, two_body_gridpoints, three_body_gridpoints, eta2, eta3, two_body_decay, three_body_weight,
+               three_body_decay, rcut)
+    counts = _counts(coordinates, nneighbours)
+    if gradients:
+        rep, jac = ops.fchl_jacobian(coordinates, element_types, cell, inv_cell, blockAtomIDs, blockMolIDs, counts,
+                                     two_body_gridpoints, three_body_gridpoints, prm, neighbourlist, nneighbours)
+        return [rep, jac]
+    return [ops.fchl_forward(coordinates, element_types, cell, inv_cell, blockAtomIDs, blockMolIDs, counts,
+                             two_body_gridpoints, three_body_gridpoints, prm, neighbourlist, nneighbours)]
+
+
+def fchl_backwards(coordinates, charges, species, element_types, cell, inv_cell, blockAtomIDs, blockMolIDs,
+                   neighbourlist, nneighbours, two_body_gridpoints, three_body_gridpoints, eta2, eta3, two_body_decay,
+                   three_body_weight, three_body_decay, rcut, grad_in):
+    prm = _prm(species, two_body_gridpoints, three_body_gridpoints, eta2, eta3, two_body_decay, three_body_weight,
+               three_body_decay, rcut)
+    return ops.fchl_vjp(grad_in, coordinates, element_types, cell, inv_cell, blockAtomIDs, blockMolIDs,
+                        _counts(coordinates, nneighbours), two_body_gridpoints, three_body_gridpoints, prm,
+                        neighbourlist, nneighbours)
+
+
+def _counts(coordinates, nneighbours):
+    """The reference's signatures carry no atom counts: with a neighbour list given they are
+    not needed (the list is authoritative), so any int32 [B] tensor does."""
+    import torch
+    B = coordinates.shape[0] if coordinates.dim() == 3 else 1
+    n = coordinates.shape[-2]
+    return torch.full((B,), n, dtype=torch.int32, device=coordinates.device)

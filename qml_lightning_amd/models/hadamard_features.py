@@ -1,0 +1,226 @@
+"""HadamardFeaturesModel: SORF feature model (qml_lightning/models/hadamard_features.py:13-256).
+
+`forward(X, Z, atomIDs, molIDs, atom_counts[, cell, inv_cell])` is TorchScript-compilable
+and differentiable in X.  With `fused=False` it is the reference's own operator sequence
+(get_SORF_coefficients -> get_cos_features -> matmul with alpha), so a file written by
+`save_jit_model` then only needs the operators the reference registers.  With
+`fused=True` (default) each element goes through one kernel that never materialises the
+[atoms, nfeatures] coefficients and already returns the gradient with respect to the
+projected representation; the numbers are the same.
+"""
+from typing import Final, Optional
+
+import numpy as np
+import torch
+
+from .. import ops
+from ..cuda.sorf_gpu import (compute_hadamard_features, compute_molecular_featurization_derivative,
+                             compute_partial_feature_derivatives, sorf_matrix_gpu)
+from ..representations.dimensionality_reduction import project_representation
+from .kernel import BaseKernel, _default_device
+
+_fused_registered = False
+
+
+def _register_fused_op():
+    """qml_lightning_sorf::sorf_energy(sub, D, bias, alpha, coeff_normalisation, ntransforms)
+    -> per-atom energies [A]; autograd on `sub`.  Not part of the reference's operator set."""
+    global _fused_registered
+    if _fused_registered:
+        return
+    _fused_registered = True
+    lib = torch.library.Library("qml_lightning_sorf", "FRAGMENT")
+    lib.define("sorf_energy(Tensor sub, Tensor D, Tensor bias, Tensor alpha, Tensor coeff_normalisation, "
+               "Tensor ntransforms) -> (Tensor, Tensor)")
+
+    def impl(sub, D, bias, alpha, cn, nt):
+        e_atom = torch.empty(sub.shape[0], dtype=torch.float32, device=sub.device)
+        gx = ops.sorf_energy_fused(sub, D, bias, alpha, None, ops._scalar(cn), int(nt.item()), e_atom, with_grad=True)
+        return e_atom, gx
+
+    lib.impl("sorf_energy", impl, "CompositeExplicitAutograd")
+
+    def setup(ctx, inputs, output):
+        ctx.save_for_backward(output[1])
+        ctx.set_materialize_grads(False)
+
+    def backward(ctx, g_e, g_gx):
+        (gx,) = ctx.saved_tensors
+        gsub = gx * g_e[:, None] if g_e is not None else None
+        return gsub, None, None, None, None, None
+
+    torch.library.register_autograd("qml_lightning_sorf::sorf_energy", backward, setup_context=setup, lib=lib)
+    ops._libs.append(lib)
+
+
+_register_fused_op()
+
+
+class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
+
+    fused: Final[bool]
+
+    def __init__(self, rep=None, elements=np.array([1, 6, 7, 8]), ntransforms=2, sigma=3.0, llambda=1e-11, npcas=128,
+                 nbatch_train=64, nbatch_test=64, nstacks=32, fused=True):
+        torch.nn.Module.__init__(self)
+        BaseKernel.__init__(self, rep, npcas, elements, sigma, llambda)
+        self.device = _default_device()
+        self.ntransforms = torch.tensor(ntransforms)
+        self.nstacks = nstacks
+        self.nbatch_train = nbatch_train
+        self.nbatch_test = nbatch_test
+        self.species = torch.from_numpy(np.asarray(elements)).float().to(self.device)
+        self.npcas = npcas
+        self.fused = fused
+        self.Dmat = torch.zeros((len(elements), ntransforms, nstacks, npcas), dtype=torch.float32, device=self.device)
+        self.get_SORF_diagonals(elements, ntransforms, nstacks, npcas)
+        self.bias = torch.zeros((len(elements), self.nfeatures()), dtype=torch.float32, device=self.device)
+        self.get_bias(elements, nstacks * npcas)
+        self.is_trained = False
+        self.alpha = torch.zeros(self.nfeatures(), device=self.device, dtype=torch.float)
+
+    @torch.jit.unused
+    def get_SORF_diagonals(self, elements, ntransforms, nstacks, npcas):
+        """Rademacher diagonals per element (hadamard_features.py:44-53)."""
+        for e in elements:
+            D = np.random.uniform(-1, 1, (ntransforms, nstacks, npcas))
+            D = np.where(D > 0.0, 1.0, -1.0)
+            self.Dmat[self.element2index[int(e)]] = torch.from_numpy(D).float().to(self.device)
+
+    @torch.jit.unused
+    def get_bias(self, elements, nfeatures):
+        """b ~ U(0, 2 pi) per element (hadamard_features.py:55-61)."""
+        for e in elements:
+            v = np.random.uniform(0.0, 1.0, [nfeatures]) * 2.0 * np.pi
+            self.bias[self.element2index[int(e)]] = torch.from_numpy(v).float().to(self.device)
+
+    def nfeatures(self):
+        return self.npcas * self.nstacks
+
+    @torch.jit.unused
+    def calculate_features(self, representation, element, indexes, feature_matrix, grad=None,
+                           derivative_features=None):
+        """Add one element's cos features (and force features) into the fp64 batch
+        matrices (hadamard_features.py:66-80)."""
+        coeff_normalisation = np.sqrt(representation.shape[1]) / self.sigma
+        element_idx = self.element2index[int(element)]
+        coeffs = ops.sorf_forward(representation, self.Dmat[element_idx], coeff_normalisation, int(self.ntransforms))
+        coeffs = coeffs.view(coeffs.shape[0], -1)
+        compute_hadamard_features(coeffs, self.bias[element_idx], indexes, feature_matrix)
+        if derivative_features is not None and grad is not None:
+            cos_derivs = torch.empty(coeffs.shape, device=coeffs.device, dtype=torch.float64)
+            compute_partial_feature_derivatives(coeffs, self.bias[element_idx], cos_derivs)
+            compute_molecular_featurization_derivative(cos_derivs, coeff_normalisation, self.Dmat[element_idx], grad,
+                                                       indexes, derivative_features)
+
+    def forward(self, X, Z, atomIDs, molIDs, atom_counts, cell: Optional[torch.Tensor] = None,
+                inv_cell: Optional[torch.Tensor] = None):
+        """Total energies [B] (fp32), differentiable in X (hadamard_features.py:82-123)."""
+        if cell is None:
+            cell = torch.empty(0, 3, 3, device=X.device)
+        if inv_cell is None:
+            inv_cell = torch.empty(0, 3, 3, device=X.device)
+        assert X.is_cuda, "X tensor must reside on GPU"
+        assert Z.is_cuda, "Z tensor must reside on GPU"
+        assert atomIDs.is_cuda, "atomIDs tensor must reside on GPU"
+        assert molIDs.is_cuda, "molIDs tensor must reside on GPU"
+        assert atom_counts.is_cuda, "atom_counts tensor must reside on GPU"
+        assert cell.is_cuda, "cell tensor must reside on GPU"
+        assert inv_cell.is_cuda, "inv_cell tensor must reside on GPU"
+
+        coeff_normalisation = torch.sqrt(torch.tensor(self.npcas)) / self.sigma
+        torch_rep = self.rep.forward(X, Z, atomIDs, molIDs, atom_counts, cell, inv_cell)
+        alpha = self.alpha.float()
+
+        if self.fused:
+            nslots = X.shape[0] * X.shape[1]
+            flat_rep = torch_rep.view(nslots, torch_rep.shape[2])
+            e_slots = torch.zeros(nslots, device=X.device, dtype=torch.float32)
+            for e in self.elements:
+                element_idx = self.element2index[e]
+                idx = torch.where(Z.reshape(-1).int() == e.item())[0]
+                if idx.shape[0] == 0:
+                    continue
+                sub = project_representation(flat_rep.index_select(0, idx), self.reductors[element_idx])
+                e_atom, _ = torch.ops.qml_lightning_sorf.sorf_energy(sub, self.Dmat[element_idx],
+                                                                     self.bias[element_idx], alpha,
+                                                                     coeff_normalisation, self.ntransforms)
+                e_slots = e_slots.index_put((idx,), e_atom)
+            return e_slots.view(X.shape[0], X.shape[1]).sum(dim=1)
+
+        Ztest = torch.zeros(X.shape[0], self.nfeatures(), device=X.device, dtype=torch.float32)
+        for e in self.elements:
+            indexes = Z.int() == e.item()
+            element_idx = self.element2index[e]
+            batch_indexes = torch.where(indexes)[0].type(torch.int)
+            sub = torch_rep[indexes]
+            if sub.shape[0] == 0:
+                continue
+            sub = project_representation(sub, self.reductors[element_idx])
+            coeffs = torch.ops.qml_lightning_sorf.get_SORF_coefficients(sub, self.Dmat[element_idx],
+                                                                        coeff_normalisation, self.ntransforms)
+            coeffs = coeffs.view(coeffs.shape[0], coeffs.shape[1] * coeffs.shape[2])
+            features = torch.ops.qml_lightning_sorf.get_cos_features(coeffs, self.bias[element_idx],
+                                                                     torch.tensor(X.shape[0]), batch_indexes)
+            Ztest = Ztest + features
+        return torch.matmul(Ztest, alpha)
+
+    @torch.jit.unused
+    def predict_opt(self, coordinates, charges, atomIDs, molIDs, natom_counts, cells=None, inv_cells=None,
+                    forces=True, print_info=False, profiler=False):
+        """Energies (and forces = -dE/dX by autograd) for tensors already on the device
+        (hadamard_features.py:125-179)."""
+        if self.is_trained is False:
+            raise RuntimeError("Error: must train the model first by calling train()!")
+        with torch.autograd.profiler.profile(enabled=profiler, use_device='cuda', with_stack=True) as prof:
+            start = torch.cuda.Event(enable_timing=True)
+            end = torch.cuda.Event(enable_timing=True)
+            start.record()
+            if forces:
+                coordinates.requires_grad = True
+            total_energies = self.forward(coordinates, charges, atomIDs, molIDs, natom_counts, cells, inv_cells)
+            if forces:
+                forces_torch, = torch.autograd.grad(-total_energies.sum(), coordinates)
+            end.record()
+            torch.cuda.synchronize()
+        if print_info:
+            print("prediction for", coordinates.shape[0], "molecules time: ", start.elapsed_time(end), "ms")
+        result = (total_energies, forces_torch) if forces else total_energies
+        if profiler:
+            result = (result,) + (prof,)
+        return result
+
+    @torch.jit.unused
+    def predict(self, X, Z, max_natoms, cells=None, inv_cells=None, forces=True, print_info=False, profiler=False):
+        """Batched predict from lists of numpy arrays (hadamard_features.py:181-251)."""
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        start.record()
+        predict_energies = torch.zeros(len(X), device=self.device, dtype=torch.float32)
+        predict_forces = torch.zeros(len(X), max_natoms, 3, device=self.device, dtype=torch.float32)
+        for i in self._progress(range(0, len(X), self.nbatch_test), print_info):
+            sl = slice(i, i + self.nbatch_test)
+            data = self.format_data(X[sl], Z[sl], cells=cells[sl] if cells is not None else None,
+                                    inv_cells=inv_cells[sl] if cells is not None else None)
+            result = self.predict_opt(data['coordinates'], data['charges'], data['atomIDs'], data['molIDs'],
+                                      data['natom_counts'], data['cells'], data['inv_cells'], forces=forces,
+                                      print_info=False, profiler=False)
+            if forces:
+                predict_energies[sl] = result[0].detach()
+                n = result[1].shape[1]
+                # padded slots carry exactly zero force, so the padded block can be copied whole
+                predict_forces[sl, :n] = result[1]
+            else:
+                predict_energies[sl] = result.detach()
+        end.record()
+        torch.cuda.synchronize()
+        if print_info:
+            print("prediction for", len(X), "molecules time: ", start.elapsed_time(end), "ms")
+        if forces:
+            return (predict_energies, predict_forces)
+        return predict_energies
+
+    @torch.jit.unused
+    def save_jit_model(self, file_name='model_sorf.pt'):
+        script = torch.jit.script(self)
+        script.save(file_name)

@@ -1,0 +1,397 @@
+"""BaseKernel: host orchestration shared by the SORF and RFF models
+(qml_lightning/models/kernel.py:15-722 of the reference): batch formatting, the training
+loop that assembles the rows Z = [Z_E ; G] and accumulates Z^T Z / Z^T y, the solve, the
+explicit-Jacobian predict route, reductor fitting and self energies.
+
+Same class / method names, argument meaning, row order and dtypes as the reference; what
+differs is underneath: one fp64 row buffer per batch (energy rows and force rows are
+views of it, no concatenation copy), per-element atom indices built once on the host by
+`format_data` (no boolean-mask device syncs), the hand-written fp64 MFMA Gram kernel, and
+no `empty_cache()` between batches.
+"""
+import numpy as np
+import torch
+
+from .. import ops
+from ..cuda.utils_gpu import matmul_and_reduce
+from ..representations.dimensionality_reduction import project_derivative, project_representation
+
+
+def _default_device():
+    return torch.device("cuda" if torch.cuda.is_available() else "cpu")
+
+
+class BaseKernel():
+
+    def __init__(self, rep, npcas, elements, sigma, llambda):
+        super(BaseKernel, self).__init__()
+        self.npcas = npcas
+        self.self_energy = None
+        self.elements = torch.tensor(np.asarray(elements))
+        self.rep = rep
+        dev = _default_device()
+        self.reductors = torch.zeros(len(elements), rep.get_repsize(), npcas, dtype=torch.float32, device=dev)
+        self.element2index = torch.zeros(int(max(elements)) + 1, dtype=torch.long)
+        for i, e in enumerate(self.elements):
+            self.element2index[int(e)] = i
+        self._convert_from_hartree_to_kcal = False
+        self.hartree2kcalmol = 627.5
+        self._subtract_self_energies = False
+        self.sigma = sigma
+        self.llambda = llambda
+
+    # -- to be provided by the feature model -------------------------------------------
+    def calculate_features(self, rep, element, indexes, feature_matrix, grad=None, derivative_matrix=None):
+        raise NotImplementedError("Abstract method only.")
+
+    def nfeatures(self):
+        raise NotImplementedError("Abstract method only.")
+
+    def predict(self, X, Q, max_natoms, cells=None, inv_cells=None, forces=False, print_info=True, use_backward=True):
+        raise NotImplementedError("Abstract method only.")
+
+    # -- rows of one batch ----------------------------------------------------------------
+    def _batch_rows(self, data, with_forces, zero_energy_rows=False):
+        """fp64 row matrix [B (+ B*n*3), F] of one formatted batch: B energy rows, then the
+        B*n*3 force rows in (molecule, atom, xyz) order (kernel.py:134-170)."""
+        coordinates, charges = data['coordinates'], data['charges']
+        atomIDs, molIDs, natom_counts = data['atomIDs'], data['molIDs'], data['natom_counts']
+        cells, inv_cells = data['cells'], data['inv_cells']
+        B, n = charges.shape
+        F = self.nfeatures()
+        if with_forces:
+            representation, rep_derivative = self.rep.get_representation_and_derivative(
+                coordinates, charges, atomIDs, molIDs, natom_counts, cells, inv_cells)
+        else:
+            representation = self.rep.get_representation(coordinates, charges, atomIDs, molIDs, natom_counts, cells,
+                                                         inv_cells)
+            rep_derivative = None
+        nrows = B + (B * n * 3 if with_forces else 0)
+        rows = torch.zeros(nrows, F, device=coordinates.device, dtype=torch.float64)
+        Zenergy = rows[:B]
+        G = rows[B:].view(B, n, 3, F) if with_forces else None
+        flat_rep = representation.view(B * n, -1)
+        flat_jac = rep_derivative.view(B * n, n, 3, -1) if with_forces else None
+        for e in self.elements:
+            idx = self._element_index(data, charges, int(e))
+            if idx.shape[0] == 0:
+                continue
+            element_idx = self.element2index[int(e)]
+            batch_indexes = torch.div(idx, n, rounding_mode='floor').to(torch.int32)
+            sub = project_representation(flat_rep.index_select(0, idx), self.reductors[element_idx])
+            sub_grad = None
+            if with_forces:
+                sub_grad = project_derivative(flat_jac.index_select(0, idx), self.reductors[element_idx])
+            self.calculate_features(sub, e, batch_indexes, Zenergy, sub_grad, G)
+        if zero_energy_rows:
+            Zenergy.fill_(0)        # energy rows stay, as zeros, so the row count is unchanged (kernel.py:164-165)
+        return rows
+
+    @staticmethod
+    def _element_index(data, charges, e):
+        """Flat (molecule-major) indices of the atoms of element e.  `format_data` prepares
+        them on the host; tensors that did not come from it fall back to a device search."""
+        table = data.get('element_index')
+        if table is not None:
+            idx = table.get(e)
+            if idx is None:
+                return torch.zeros(0, dtype=torch.long, device=charges.device)
+            return idx
+        return torch.nonzero(charges.reshape(-1).int() == e).reshape(-1)
+
+    # -- training -------------------------------------------------------------------------
+    def build_Z_components(self, X, Q, E=None, F=None, cells=None, inv_cells=None, print_info=True, cpu_solve=False,
+                           ntiles=1, use_specialized_matmul=False):
+        """Z^T Z [F,F] and Z^T y [F,1] in fp64 over the training set (kernel.py:46-217).
+
+        X, Q: lists of [natoms_i,3] coordinates / [natoms_i] charges; E, F: energies /
+        forces (either may be None).  cpu_solve keeps Z^T Z on the host; ntiles > 1 builds
+        it in row blocks of ceil(nfeatures/ntiles) features; use_specialized_matmul takes
+        the fp32-Kahan -> fp64 product instead of the fp64 one.
+        """
+        if self.reductors is None:
+            raise RuntimeError("ERROR: Must call model.get_reductors() first to initialize the projection matrices.")
+        if E is None and F is None:
+            raise RuntimeError("ERROR: must have either E, F or both as input to train().")
+        nf = self.nfeatures()
+        dev = self.device
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        ZTZ = torch.zeros(nf, nf, device=torch.device('cpu') if cpu_solve else dev, dtype=torch.float64)
+        ZtrainY = torch.zeros(nf, 1, device=dev, dtype=torch.float64)
+        start.record()
+        nsub = int(np.ceil(nf / ntiles))
+        for tile in range(ntiles):
+            lo, hi = tile * nsub, min(nsub * (tile + 1), nf)
+            if ntiles > 1:
+                if print_info:
+                    print("tile:", tile + 1, "of", ntiles, "tiles, tile size:", hi - lo)
+                ZTZ_tile = torch.zeros(hi - lo, nf, device=dev, dtype=torch.float64)
+            for i in self._progress(range(0, len(X), self.nbatch_train), print_info):
+                sl = slice(i, i + self.nbatch_train)
+                data = self.format_data(X[sl], Q[sl], E=E[sl] if E is not None else None,
+                                        F=F[sl] if F is not None else None,
+                                        cells=cells[sl] if cells is not None else None,
+                                        inv_cells=inv_cells[sl] if cells is not None else None)
+                zbatch = data['charges'].shape[0]
+                targets = self._targets(data, zbatch, E is not None, F is not None)
+                rows = self._batch_rows(data, F is not None, zero_energy_rows=E is None)
+                if ntiles > 1:
+                    if use_specialized_matmul:
+                        matmul_and_reduce(rows[:, lo:hi].float().T.contiguous(), rows.float(), ZTZ_tile)
+                        ZtrainY[lo:hi] += torch.matmul(rows[:, lo:hi].T, targets)
+                    else:
+                        ops.gram(rows, targets, ZTZ_tile, ZtrainY, f0=lo, f1=hi)
+                elif cpu_solve:
+                    part = torch.zeros(nf, nf, device=dev, dtype=torch.float64)
+                    ops.gram(rows, targets, part, ZtrainY)
+                    ZTZ += part.cpu()
+                elif use_specialized_matmul:
+                    r32 = rows.float()
+                    matmul_and_reduce(r32.T.contiguous(), r32, ZTZ)
+                    ZtrainY += torch.matmul(rows.T, targets)
+                else:
+                    ops.gram(rows, targets, ZTZ, ZtrainY)
+                del rows
+            if ntiles > 1:
+                ZTZ[lo:hi, :] += ZTZ_tile.cpu() if cpu_solve else ZTZ_tile
+        end.record()
+        torch.cuda.synchronize()
+        if print_info:
+            print("ZTZ time: ", start.elapsed_time(end), "ms")
+        return ZTZ, ZtrainY
+
+    @staticmethod
+    def _progress(it, show):
+        if show:
+            from tqdm import tqdm
+            return tqdm(it)
+        return it
+
+    def _targets(self, data, zbatch, has_E, has_F):
+        """Target column in the row order of `_batch_rows` (kernel.py:118-124)."""
+        energies, forces = data['energies'], data['forces']
+        if has_E and not has_F:
+            return energies[:, None]
+        if has_F and not has_E:
+            zero = torch.zeros((zbatch, 1), device=forces.device, dtype=torch.float64)
+            return torch.cat((zero, forces.flatten()[:, None]), dim=0)
+        return torch.cat((energies[:, None], forces.flatten()[:, None]), dim=0)
+
+    def train(self, X, Q, E=None, F=None, cells=None, inv_cells=None, print_info=True, cpu_solve=False, ntiles=1,
+              use_specialized_matmul=False):
+        """alpha = (Z^T Z + lambda I)^-1 Z^T y (kernel.py:219-247)."""
+        ZTZ, ZtrainY = self.build_Z_components(X, Q, E, F, cells, inv_cells, print_info, cpu_solve, ntiles,
+                                               use_specialized_matmul=use_specialized_matmul)
+        ZTZ.diagonal().add_(self.llambda)
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        start.record()
+        if cpu_solve:
+            self.alpha = torch.linalg.solve(ZTZ, ZtrainY.cpu())[:, 0].to(self.device)
+        else:
+            self.alpha = torch.linalg.solve(ZTZ, ZtrainY)[:, 0]
+        end.record()
+        torch.cuda.synchronize()
+        if print_info:
+            print("coefficients time: ", start.elapsed_time(end), "ms")
+        self.is_trained = True
+
+    def hyperparam_opt_nested_cv(self, X, Q, E, F=None, cells=None, inv_cells=None,
+                                 sigmas=np.linspace(1.5, 12.5, 10), lambdas=np.logspace(-11, -5, 9), kfolds=5,
+                                 print_info=True, use_rmse=False):
+        """K-fold grid search over (sigma, lambda) (kernel.py:249-347)."""
+        from sklearn.model_selection import KFold
+        kf = KFold(n_splits=kfolds, shuffle=False)
+        best = (None, None, np.inf)
+        for sigma in sigmas:
+            for llambda in lambdas:
+                fold_error = 0.0
+                for train_index, test_index in kf.split(X):
+                    pick = lambda seq, ids: [seq[z] for z in ids]
+                    self.sigma, self.llambda = sigma, llambda
+                    self.train(pick(X, train_index), pick(Q, train_index), pick(E, train_index),
+                               pick(F, train_index) if F is not None else None, cells, inv_cells, print_info=False)
+                    Xt, Qt = pick(X, test_index), pick(Q, test_index)
+                    data = self.format_data(Xt, Qt, pick(E, test_index), pick(F, test_index) if F is not None else None,
+                                            cells=cells, inv_cells=inv_cells)
+                    max_natoms = int(data['natom_counts'].max().item())
+                    err = torch.sqrt if use_rmse else (lambda v: v)
+                    red = (lambda d: torch.mean(d * d)) if use_rmse else (lambda d: torch.mean(torch.abs(d)))
+                    if F is not None:
+                        ep, fp = self.predict(Xt, Qt, max_natoms, cells=cells, inv_cells=inv_cells, forces=True,
+                                              print_info=False)
+                        e_err = err(red(ep - data['energies']))
+                        f_err = err(red(fp - data['forces']))
+                        fold_error += 0.5 * float(e_err + f_err)
+                    else:
+                        ep = self.predict(Xt, Qt, max_natoms, cells=cells, inv_cells=inv_cells, forces=False,
+                                          print_info=False)
+                        fold_error += float(err(red(ep - data['energies'])))
+                fold_error /= kfolds
+                if print_info:
+                    print("sigma", sigma, "lambda", llambda, "error", fold_error)
+                if fold_error < best[2]:
+                    best = (sigma, llambda, fold_error)
+        if print_info:
+            print("Best error: ", best[2], "sigma = ", best[0], "lambda = ", best[1])
+        return best[0], best[1]
+
+    # -- explicit-Jacobian predict route ----------------------------------------------------
+    def predict_cuda(self, X, Q, max_natoms, cells=None, inv_cells=None, forces=False, print_info=True):
+        """fp64 energies [N] (and forces [N,max_natoms,3]) as Z.alpha and G.alpha
+        (kernel.py:349-445)."""
+        if self.is_trained is False:
+            raise RuntimeError("Error: must train the model first by calling train()!")
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        predict_energies = torch.zeros(len(X), device=self.device, dtype=torch.float64)
+        predict_forces = torch.zeros(len(X), max_natoms, 3, device=self.device, dtype=torch.float64)
+        alpha = self.alpha.double()
+        start.record()
+        for i in self._progress(range(0, len(X), self.nbatch_test), print_info):
+            sl = slice(i, i + self.nbatch_test)
+            data = self.format_data(X[sl], Q[sl], cells=cells[sl] if cells is not None else None,
+                                    inv_cells=inv_cells[sl] if cells is not None else None)
+            B, n = data['charges'].shape
+            rows = self._batch_rows(data, forces is True)
+            out = torch.matmul(rows, alpha)
+            predict_energies[sl] = out[:B]
+            if forces is True:
+                predict_forces[sl, :n] = out[B:].reshape(B, n, 3)
+        end.record()
+        torch.cuda.synchronize()
+        if print_info:
+            print("prediction for", len(X), "molecules time: ", start.elapsed_time(end), "ms")
+        if forces is True:
+            return (predict_energies, predict_forces)
+        return predict_energies
+
+    # -- reductors ----------------------------------------------------------------------
+    def get_reductors(self, X, Q, cells=None, inv_cells=None, npcas=128, npca_choice=256, nsamples=4096,
+                      print_info=True):
+        """Per element: left singular vectors of a [repsize, nselected] sample of atomic
+        representations, first `npcas` columns, no mean-centring (kernel.py:447-540)."""
+        for e in self.elements:
+            element_idx = self.element2index[int(e)]
+            ids = np.array([i for i in range(len(Q)) if int(e) in Q[i]], dtype=np.int64)
+            if len(ids) == 0:
+                continue
+            pick = np.random.choice(ids, size=min(len(ids), 1024))
+            sub_X = [X[i] for i in pick]
+            sub_Q = [Q[i] for i in pick]
+            chunks, nselected = [], 0
+            for i in range(0, len(sub_X), self.nbatch_train):
+                if nselected > nsamples:
+                    break
+                data = self.format_data(sub_X[i:i + self.nbatch_train], sub_Q[i:i + self.nbatch_train], cells=cells,
+                                        inv_cells=inv_cells)
+                rep = self.rep.get_representation(data['coordinates'], data['charges'], data['atomIDs'],
+                                                  data['molIDs'], data['natom_counts'], data['cells'],
+                                                  data['inv_cells'])
+                idx = self._element_index(data, data['charges'], int(e))
+                if idx.shape[0] == 0:
+                    continue
+                rows = rep.view(-1, rep.shape[-1]).index_select(0, idx)
+                rows = rows[torch.randperm(rows.shape[0], device=rows.device)[:npca_choice]]
+                nselected += rows.shape[0]
+                chunks.append(rows)
+            if not chunks:
+                continue
+            mat = torch.cat(chunks)
+            U, S, _ = torch.linalg.svd(mat.T, full_matrices=False)
+            reductor = U[:, :npcas]
+            if print_info:
+                cev = 100 - (S.sum() - S[:npcas].sum()) / S.sum() * 100
+                print(f"element {int(e)}: {reductor.shape[0]} -> {reductor.shape[1]}  "
+                      f"Cumulative Explained Feature Variance = {float(cev):6.2f} %")
+            if reductor.shape[1] < npcas:
+                raise RuntimeError(f"ERROR - not enough atomic environments in input dataset for element {int(e)}. "
+                                   "Either increase npca_choice or provide more structures.")
+            self.reductors[element_idx] = reductor
+
+    # -- unit conversion / self energies ----------------------------------------------------
+    def set_subtract_self_energies(self, subtract):
+        self._subtract_self_energies = subtract
+
+    def subtract_self_energies(self):
+        return self._subtract_self_energies
+
+    def set_convert_hartree2kcal(self, convert):
+        self._convert_from_hartree_to_kcal = convert
+
+    def convert_hartree2kcal(self):
+        return self._convert_from_hartree_to_kcal
+
+    def calculate_self_energy(self, Q, E):
+        """Least-squares per-element contribution to E (kernel.py:554-599)."""
+        counts = torch.zeros(len(Q), len(self.elements), dtype=torch.float64)
+        for i, q in enumerate(Q):
+            q = np.asarray(q)
+            for j, e in enumerate(self.elements):
+                counts[i, j] = float((q == int(e)).sum())
+        energies = torch.tensor(np.asarray(E, dtype=np.float64))
+        if self.convert_hartree2kcal():
+            energies = energies * self.hartree2kcalmol
+        XTX = counts.T @ counts
+        beta = torch.linalg.lstsq(XTX, counts.T @ energies[:, None]).solution[:, 0]
+        species = self.elements.long()
+        self.self_energy = torch.zeros(int(torch.max(species)) + 1, dtype=torch.float64)
+        self.self_energy[species] = beta
+        print("Self Energies: ", self.self_energy)
+
+    # -- batch formatting -------------------------------------------------------------------
+    def format_data(self, X, Q, E=None, F=None, cells=None, inv_cells=None):
+        """Lists of per-molecule arrays -> zero-padded device tensors with the keys
+        coordinates / charges / natom_counts / atomIDs / molIDs / energies / forces /
+        cells / inv_cells (kernel.py:601-722), plus 'element_index': {element: int64 flat
+        indices of its atoms}, computed here on the host so later gathers need no device
+        search."""
+        if self.subtract_self_energies() and self.self_energy is None:
+            raise RuntimeError("ERROR: must call model.calculate_self_energy first - this computes atomic "
+                               "contributes to the potential energy.")
+        dev = self.device
+        zbatch = len(X)
+        counts = np.array([np.asarray(x).shape[0] for x in X], dtype=np.int32)
+        n = int(counts.max()) if zbatch else 0
+        coords = np.zeros((zbatch, n, 3), dtype=np.float32)
+        charges = np.zeros((zbatch, n), dtype=np.float32)
+        for j in range(zbatch):
+            coords[j, :counts[j]] = np.asarray(X[j], dtype=np.float32)
+            charges[j, :counts[j]] = np.asarray(Q[j], dtype=np.float32)
+        molIDs = np.repeat(np.arange(zbatch, dtype=np.int32), counts)
+        atomIDs = np.concatenate([np.arange(c, dtype=np.int32) for c in counts]) if zbatch else np.zeros(0, np.int32)
+        data = {
+            'coordinates': torch.from_numpy(coords).to(dev),
+            'charges': torch.from_numpy(charges).to(dev),
+            'natom_counts': torch.from_numpy(counts).to(dev),
+            'atomIDs': torch.from_numpy(atomIDs).to(dev),
+            'molIDs': torch.from_numpy(molIDs).to(dev),
+            'energies': None,
+            'forces': None,
+            'cells': torch.empty((0, 3, 3), device=dev),
+            'inv_cells': torch.empty((0, 3, 3), device=dev),
+        }
+        flat_q = charges.reshape(-1).astype(np.int64)
+        data['element_index'] = {int(e): torch.from_numpy(np.nonzero(flat_q == int(e))[0]).to(dev)
+                                 for e in self.elements}
+        if E is not None:
+            energies = np.array(E, dtype=np.float64).reshape(zbatch).copy()
+            if self.convert_hartree2kcal():
+                energies *= self.hartree2kcalmol
+            if self.subtract_self_energies():
+                se = self.self_energy.numpy()
+                for j in range(zbatch):
+                    energies[j] -= se[np.asarray(Q[j]).astype(np.int64)].sum()
+            data['energies'] = torch.from_numpy(energies).to(dev)
+        if F is not None:
+            forces = np.zeros((zbatch, n, 3), dtype=np.float64)
+            for j in range(zbatch):
+                forces[j, :counts[j]] = np.asarray(F[j], dtype=np.float64)
+            if self.convert_hartree2kcal():
+                forces *= self.hartree2kcalmol
+            data['forces'] = torch.from_numpy(forces).to(dev)
+        if cells is not None:
+            data['cells'] = torch.from_numpy(np.asarray(cells, dtype=np.float32).reshape(zbatch, 3, 3)).to(dev)
+            data['inv_cells'] = torch.from_numpy(np.asarray(inv_cells, dtype=np.float32).reshape(zbatch, 3, 3)).to(dev)
+        return data

@@ -1,0 +1,119 @@
+"""RandomFourrierFeaturesModel (qml_lightning/models/random_features.py:17-236): features
+sqrt(2/F) cos(x W + b) with W ~ N(0,1)/(2 sigma^2) per element."""
+from typing import Optional
+
+import numpy as np
+import torch
+
+from ..cuda.rff_gpu import get_rff, get_rff_derivatives
+from ..representations.dimensionality_reduction import project_representation
+from .kernel import BaseKernel, _default_device
+
+
+class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
+
+    def __init__(self, rep=None, elements=np.array([1, 6, 7, 8]), sigma=2.0, llambda=1e-10,
+                 nstacks=8192, npcas=128, nbatch_train=64, nbatch_test=64):
+        torch.nn.Module.__init__(self)
+        BaseKernel.__init__(self, rep, npcas, elements, sigma, llambda)
+        self.device = _default_device()
+        self.npcas = npcas
+        self.nbatch_train = nbatch_train
+        self.nbatch_test = nbatch_test
+        self._nfeatures = nstacks * self.npcas
+        self.species = torch.from_numpy(np.asarray(elements)).float().to(self.device)
+        self.sample_elemental_basis()
+        self.feature_normalisation = float(np.sqrt(2.0 / self._nfeatures))
+        self.is_trained = False
+        self.alpha = torch.zeros(self._nfeatures, device=self.device, dtype=torch.float)
+
+    @torch.jit.unused
+    def sample_elemental_basis(self):
+        """W [ne,d,F] = N(0,1)/(2 sigma^2), b [ne,F] = U(0,2pi) (random_features.py:42-55)."""
+        D, d = self.nfeatures(), self.npcas
+        self.W = torch.zeros((len(self.elements), d, D), dtype=torch.float32, device=self.device)
+        self.b = torch.zeros((len(self.elements), D), dtype=torch.float32, device=self.device)
+        for e in self.elements:
+            idx = self.element2index[int(e)]
+            self.W[idx] = torch.from_numpy(np.random.normal(0.0, 1.0, [d, D]) / (2 * self.sigma ** 2)).to(self.device)
+            self.b[idx] = torch.from_numpy(np.random.uniform(0.0, 1.0, [D]) * 2.0 * np.pi).to(self.device)
+
+    def nfeatures(self):
+        return self._nfeatures
+
+    @torch.jit.unused
+    def calculate_features(self, rep, element, indexes, feature_matrix, grad=None, derivative_matrix=None):
+        """fp64 features / force features of one element (random_features.py:60-67)."""
+        idx = self.element2index[int(element)]
+        W, b = self.W[idx].double(), self.b[idx].double()
+        get_rff(rep, W, b, indexes, feature_matrix)
+        if derivative_matrix is not None and grad is not None:
+            get_rff_derivatives(rep, grad, W, b, indexes, derivative_matrix)
+
+    def forward(self, X, Z, atomIDs, molIDs, atom_counts, cell: Optional[torch.Tensor] = None,
+                inv_cell: Optional[torch.Tensor] = None):
+        """Total energies [B], differentiable in X; the feature GEMM is the BLAS library's
+        (random_features.py:69-102)."""
+        if cell is None:
+            cell = torch.empty(0, 3, 3, device=X.device)
+        if inv_cell is None:
+            inv_cell = torch.empty(0, 3, 3, device=X.device)
+        assert X.is_cuda, "X tensor must reside on GPU"
+        assert Z.is_cuda, "Z tensor must reside on GPU"
+        torch_rep = self.rep.forward(X, Z, atomIDs, molIDs, atom_counts, cell, inv_cell)
+        Ztest = torch.zeros(X.shape[0], self.nfeatures(), device=X.device, dtype=torch.float32)
+        for e in self.elements:
+            indexes = Z.int() == e.item()
+            element_idx = self.element2index[e]
+            batch_indexes = torch.where(indexes)[0]
+            sub = torch_rep[indexes]
+            if sub.shape[0] == 0:
+                continue
+            sub = project_representation(sub, self.reductors[element_idx])
+            feats = self.feature_normalisation * torch.cos(torch.matmul(sub, self.W[element_idx])
+                                                           + self.b[element_idx][None, :])
+            Ztest = Ztest.index_add(0, batch_indexes, feats)
+        return torch.matmul(Ztest, self.alpha.float())
+
+    @torch.jit.unused
+    def predict_opt(self, coordinates, charges, atomIDs, molIDs, natom_counts, zcells=None, zinv_cells=None,
+                    forces=True, print_info=False, profiler=False):
+        if self.is_trained is False:
+            raise RuntimeError("Error: must train the model first by calling train()!")
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        start.record()
+        if forces:
+            coordinates.requires_grad = True
+        total_energies = self.forward(coordinates, charges, atomIDs, molIDs, natom_counts, zcells, zinv_cells)
+        if forces:
+            forces_torch, = torch.autograd.grad(-total_energies.sum(), coordinates)
+        end.record()
+        torch.cuda.synchronize()
+        if print_info:
+            print("prediction for", coordinates.shape[0], "molecules time: ", start.elapsed_time(end), "ms")
+        return (total_energies, forces_torch) if forces else total_energies
+
+    @torch.jit.unused
+    def predict(self, X, Z, max_natoms, cells=None, inv_cells=None, forces=True, print_info=False):
+        predict_energies = torch.zeros(len(X), device=self.device, dtype=torch.float32)
+        predict_forces = torch.zeros(len(X), max_natoms, 3, device=self.device, dtype=torch.float32)
+        for i in self._progress(range(0, len(X), self.nbatch_test), print_info):
+            sl = slice(i, i + self.nbatch_test)
+            data = self.format_data(X[sl], Z[sl], cells=cells[sl] if cells is not None else None,
+                                    inv_cells=inv_cells[sl] if cells is not None else None)
+            result = self.predict_opt(data['coordinates'], data['charges'], data['atomIDs'], data['molIDs'],
+                                      data['natom_counts'], data['cells'], data['inv_cells'], forces=forces)
+            if forces:
+                predict_energies[sl] = result[0].detach()
+                predict_forces[sl, :result[1].shape[1]] = result[1]
+            else:
+                predict_energies[sl] = result.detach()
+        if forces:
+            return (predict_energies, predict_forces)
+        return predict_energies
+
+    @torch.jit.unused
+    def save_jit_model(self, file_name='model_rff.pt'):
+        script = torch.jit.script(self)
+        script.save(file_name)

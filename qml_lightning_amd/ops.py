@@ -1,0 +1,438 @@
+"""Tensor-level entry points over libqmll and the `torch.ops` the reference registers.
+
+Two layers:
+  * plain functions (`fchl_forward`, `sorf_forward`, ...): allocate outputs with torch,
+    pass `data_ptr()`s and the current HIP stream to the C ABI, return tensors;
+  * `torch.library` definitions of the operators the reference's TorchScript libraries
+    export (qml_lightning/cuda/torchscript/FCHL19.cpp:318-333, SORF.cpp:138-150), with
+    autograd, so that `torch.ops.qml_lightning_fchl.fchl_forwards` etc. resolve from Python
+    and from TorchScript exactly as they do with the reference's `.so` files loaded.
+
+Everything here requires the tensors to live on a HIP device ("cuda" in PyTorch-ROCm);
+there is no CPU implementation.
+"""
+import ctypes
+import math
+
+import torch
+
+from . import _lib
+from ._lib import FchlParams, check
+
+_P = ctypes.c_void_p
+
+
+def _ptr(t):
+    return _P(t.data_ptr()) if t is not None else _P(0)
+
+
+def _stream():
+    return _P(torch.cuda.current_stream().cuda_stream)
+
+
+def _need_cuda(t, name):
+    # same fault, same exception type as the reference's TORCH_CHECK (fchl_cuda.cpp:30-34)
+    if not t.is_cuda:
+        raise RuntimeError("%s must be a CUDA tensor" % name)
+
+
+def _f32(t):
+    return t.contiguous() if t.dtype == torch.float32 else t.float().contiguous()
+
+
+def _i32(t):
+    return t.contiguous() if t.dtype == torch.int32 else t.to(torch.int32).contiguous()
+
+
+def _cells(cell, inv_cell):
+    """[B,3,3] pair or None; an empty [0,3,3] tensor means 'no periodic images'
+    (reference: fchl_cuda_kernel.cu:548)."""
+    if cell is None or cell.numel() == 0:
+        return None, None
+    return _f32(cell), _f32(inv_cell)
+
+
+def _batched(X, Z=None):
+    if X.dim() == 2:                       # fchl_cuda.cpp:72-76
+        X = X.unsqueeze(0)
+    if Z is not None and Z.dim() == 1:
+        Z = Z.unsqueeze(0)
+    return X, Z
+
+
+def _scalar(v):
+    return float(v.item()) if torch.is_tensor(v) else float(v)
+
+
+def make_params(nspecies, Rs2, Rs3, eta2, eta3, two_body_decay, three_body_weight, three_body_decay, rcut):
+    return FchlParams(int(nspecies), int(Rs2.shape[0]), int(Rs3.shape[0]), _scalar(eta2), _scalar(eta3),
+                      _scalar(two_body_decay), _scalar(three_body_weight), _scalar(three_body_decay), _scalar(rcut))
+
+
+# ---------------------------------------------------------------------------------------
+# neighbours / element types
+# ---------------------------------------------------------------------------------------
+def num_neighbours(X, natoms, rcut, cell=None, inv_cell=None):
+    _need_cuda(X, "coordinates")
+    X, _ = _batched(X)
+    X = _f32(X)
+    natoms = _i32(natoms)
+    cell, inv_cell = _cells(cell, inv_cell)
+    B, n, _ = X.shape
+    out = torch.empty((B, n), dtype=torch.int32, device=X.device)
+    check(_lib.lib().qmll_num_neighbours(_ptr(X), _ptr(natoms), _ptr(cell), _ptr(inv_cell), B, n, _scalar(rcut),
+                                         _ptr(out), _stream()), "qmll_num_neighbours")
+    return out
+
+
+def neighbour_list(X, natoms, max_neighbours, rcut, cell=None, inv_cell=None):
+    _need_cuda(X, "coordinates")
+    X, _ = _batched(X)
+    X = _f32(X)
+    natoms = _i32(natoms)
+    cell, inv_cell = _cells(cell, inv_cell)
+    B, n, _ = X.shape
+    nn = int(max_neighbours.item()) if torch.is_tensor(max_neighbours) else int(max_neighbours)
+    out = torch.empty((B, n, nn), dtype=torch.int32, device=X.device)
+    check(_lib.lib().qmll_neighbour_list(_ptr(X), _ptr(natoms), _ptr(cell), _ptr(inv_cell), B, n, nn, _scalar(rcut),
+                                         _ptr(out), _stream()), "qmll_neighbour_list")
+    return out
+
+
+def element_types(X, Z, natoms, species):
+    _need_cuda(X, "coordinates")
+    _need_cuda(Z, "charges")
+    _need_cuda(species, "species")
+    X, Z = _batched(X, Z)
+    Z = _f32(Z)
+    natoms = _i32(natoms)
+    species = _f32(species)
+    B, n = Z.shape
+    out = torch.empty((B, n), dtype=torch.int32, device=Z.device)
+    check(_lib.lib().qmll_element_types(_ptr(Z), _ptr(natoms), _ptr(species), B, n, species.shape[0], _ptr(out),
+                                        _stream()), "qmll_element_types")
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+# FCHL19
+# ---------------------------------------------------------------------------------------
+def _fchl_args(X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3, prm):
+    B, n, _ = X.shape
+    nn_stride = int(nlist.shape[2]) if nlist is not None else 0
+    return [_ptr(X), _ptr(types), _ptr(cell), _ptr(inv_cell), _ptr(atomIDs), _ptr(molIDs), _ptr(natoms),
+            _ptr(nlist), _ptr(nneigh), nn_stride, int(atomIDs.shape[0]), B, n, _ptr(Rs2), _ptr(Rs3),
+            ctypes.byref(prm)]
+
+
+def _fchl_prepare(X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3):
+    _need_cuda(X, "coordinates")
+    X, _ = _batched(X)
+    X = _f32(X)
+    if types.dim() == 1:
+        types = types.unsqueeze(0)
+    types = _i32(types)
+    cell, inv_cell = _cells(cell, inv_cell)
+    atomIDs, molIDs, natoms = _i32(atomIDs), _i32(molIDs), _i32(natoms)
+    if nlist is not None:
+        nlist, nneigh = _i32(nlist), _i32(nneigh)
+        if nlist.shape[2] == 0:
+            nlist, nneigh = None, None
+    return X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, _f32(Rs2), _f32(Rs3)
+
+
+def repsize(prm):
+    return prm.nspecies * prm.nRs2 + prm.nspecies * (prm.nspecies + 1) * prm.nRs3
+
+
+def fchl_forward(X, types, cell, inv_cell, atomIDs, molIDs, natoms, Rs2, Rs3, prm, nlist=None, nneigh=None):
+    """rep f32 [B,n,R]; zero rows for padded slots (fchl_cuda.cpp:83)."""
+    X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3 = _fchl_prepare(
+        X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3)
+    B, n, _ = X.shape
+    rep = torch.zeros((B, n, repsize(prm)), dtype=torch.float32, device=X.device)
+    args = _fchl_args(X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3, prm)
+    check(_lib.lib().qmll_fchl19_forward(*args, _ptr(rep), _stream()), "qmll_fchl19_forward")
+    return rep
+
+
+def fchl_vjp(grad_rep, X, types, cell, inv_cell, atomIDs, molIDs, natoms, Rs2, Rs3, prm, nlist=None, nneigh=None):
+    """grad_X f32 [B,n,3] (fchl_cuda.cpp:196)."""
+    X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3 = _fchl_prepare(
+        X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3)
+    B, n, _ = X.shape
+    grad_rep = _f32(grad_rep).reshape(B, n, repsize(prm))
+    gX = torch.zeros((B, n, 3), dtype=torch.float32, device=X.device)
+    args = _fchl_args(X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3, prm)
+    check(_lib.lib().qmll_fchl19_vjp(*args, _ptr(grad_rep), _ptr(gX), _stream()), "qmll_fchl19_vjp")
+    return gX
+
+
+def fchl_jacobian(X, types, cell, inv_cell, atomIDs, molIDs, natoms, Rs2, Rs3, prm, nlist=None, nneigh=None,
+                  with_rep=True):
+    """(rep f32 [B,n,R] or None, jac f32 [B,n,n,3,R]) (fchl_cuda.cpp:186-187)."""
+    X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3 = _fchl_prepare(
+        X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3)
+    B, n, _ = X.shape
+    R = repsize(prm)
+    rep = torch.zeros((B, n, R), dtype=torch.float32, device=X.device) if with_rep else None
+    jac = torch.zeros((B, n, n, 3, R), dtype=torch.float32, device=X.device)
+    args = _fchl_args(X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3, prm)
+    check(_lib.lib().qmll_fchl19_jacobian(*args, _ptr(rep), _ptr(jac), _stream()), "qmll_fchl19_jacobian")
+    return rep, jac
+
+
+# ---------------------------------------------------------------------------------------
+# SORF / features
+# ---------------------------------------------------------------------------------------
+def sorf_forward(u, D, normalisation, ntransforms):
+    """[A,d] x [T,S,d] -> [A,S,d] (hadamard_cuda.cpp:47-56)."""
+    _need_cuda(u, "input")
+    _need_cuda(D, "dmatrix")
+    u, D = _f32(u), _f32(D)
+    A, d = u.shape
+    T, S = int(ntransforms), int(D.shape[1])
+    if T > D.shape[0]:
+        raise RuntimeError("ntransforms (%d) exceeds the %d diagonals given" % (T, D.shape[0]))
+    out = torch.empty((A, S, d), dtype=torch.float32, device=u.device)
+    check(_lib.lib().qmll_sorf_forward(_ptr(u), _ptr(D), A, d, S, T, float(normalisation), _ptr(out), _stream()),
+          "qmll_sorf_forward")
+    return out
+
+
+def sorf_adjoint(g, D, normalisation, ntransforms):
+    """[A,S,d] -> [A,d] (hadamard_cuda.cpp:58-70)."""
+    _need_cuda(g, "input")
+    _need_cuda(D, "dmatrix")
+    g, D = _f32(g), _f32(D)
+    A, S, d = g.shape
+    T = int(ntransforms)
+    out = torch.empty((A, d), dtype=torch.float32, device=g.device)
+    check(_lib.lib().qmll_sorf_adjoint(_ptr(g), _ptr(D), A, d, S, T, float(normalisation), _ptr(out), _stream()),
+          "qmll_sorf_adjoint")
+    return out
+
+
+def cos_features(coeffs, bias, nmol, mol_index, out=None):
+    """f32 [nmol,F] (new, zero-initialised) or accumulate into a given f32/f64 tensor."""
+    _need_cuda(coeffs, "coeffs")
+    _need_cuda(bias, "b")
+    _need_cuda(mol_index, "batch_indexes")
+    coeffs, bias, mol_index = _f32(coeffs), _f32(bias), _i32(mol_index)
+    A, F = coeffs.shape
+    if out is None:
+        out = torch.zeros((int(nmol), F), dtype=torch.float32, device=coeffs.device)
+    if not out.is_contiguous():
+        raise RuntimeError("feature matrix must be contiguous")
+    fn = _lib.lib().qmll_cos_features_f64 if out.dtype == torch.float64 else _lib.lib().qmll_cos_features_f32
+    check(fn(_ptr(coeffs), _ptr(bias), _ptr(mol_index), A, F, int(out.shape[0]), _ptr(out), _stream()),
+          "qmll_cos_features")
+    return out
+
+
+def cos_features_backward(gZ, coeffs, bias, nmol, mol_index):
+    gZ, coeffs, bias, mol_index = _f32(gZ), _f32(coeffs), _f32(bias), _i32(mol_index)
+    A, F = coeffs.shape
+    out = torch.empty((A, F), dtype=torch.float32, device=coeffs.device)
+    check(_lib.lib().qmll_cos_features_backward(_ptr(gZ), _ptr(coeffs), _ptr(bias), _ptr(mol_index), A, F,
+                                                int(gZ.shape[0]), _ptr(out), _stream()), "qmll_cos_features_backward")
+    return out
+
+
+def sin_coeffs(coeffs, bias, out):
+    coeffs, bias = _f32(coeffs), _f32(bias)
+    A, F = coeffs.shape
+    if out.dtype != torch.float64 or not out.is_contiguous() or tuple(out.shape) != (A, F):
+        raise RuntimeError("sin_coeffs output must be a contiguous float64 [A,F] tensor")
+    check(_lib.lib().qmll_sin_coeffs_f64(_ptr(coeffs), _ptr(bias), A, F, _ptr(out), _stream()), "qmll_sin_coeffs_f64")
+    return out
+
+
+def derivative_features(cos_derivs, normalisation, D, input_derivatives, mol_index, G):
+    D, u, mol_index = _f32(D), _f32(input_derivatives), _i32(mol_index)
+    A, n, _, d = u.shape
+    T, S, _ = D.shape
+    if (cos_derivs.dtype != torch.float64 or not cos_derivs.is_contiguous() or G.dtype != torch.float64
+            or not G.is_contiguous()):
+        raise RuntimeError("derivative features need contiguous float64 cos_derivs and output")
+    if G.shape[1] != n or G.shape[3] != S * d:
+        raise RuntimeError("feature_derivatives has shape %s, expected [nmol,%d,3,%d]" % (tuple(G.shape), n, S * d))
+    check(_lib.lib().qmll_derivative_features(_ptr(cos_derivs), float(normalisation), _ptr(mol_index), _ptr(u), _ptr(D),
+                                              A, n, d, S, T, int(G.shape[0]), _ptr(G), _stream()),
+          "qmll_derivative_features")
+    return G
+
+
+def sorf_energy_fused(x, D, bias, alpha, out_index, normalisation, ntransforms, e_atom, with_grad=True):
+    """Per-atom energies written into e_atom[out_index]; returns d e_atom / d x or None."""
+    x, D, bias, alpha = _f32(x), _f32(D), _f32(bias), _f32(alpha)
+    A, d = x.shape
+    S, T = int(D.shape[1]), int(ntransforms)
+    gx = torch.empty((A, d), dtype=torch.float32, device=x.device) if with_grad else None
+    check(_lib.lib().qmll_sorf_energy_fused(_ptr(x), _ptr(D), _ptr(bias), _ptr(alpha), _ptr(out_index), A, d, S, T,
+                                            float(normalisation), _ptr(e_atom), _ptr(gx), _stream()),
+          "qmll_sorf_energy_fused")
+    return gx
+
+
+# ---------------------------------------------------------------------------------------
+# RFF / Gram
+# ---------------------------------------------------------------------------------------
+def rff_features(x, W, b, mol_index, Zf):
+    x, mol_index = _f32(x), _i32(mol_index)
+    W, b = W.double().contiguous(), b.double().contiguous()
+    A, d = x.shape
+    F = W.shape[1]
+    check(_lib.lib().qmll_rff_features(_ptr(x), _ptr(W), _ptr(b), _ptr(mol_index), A, d, F, int(Zf.shape[0]), _ptr(Zf),
+                                       _stream()), "qmll_rff_features")
+    return Zf
+
+
+def rff_derivative_features(x, grad, W, b, mol_index, G):
+    x, grad, mol_index = _f32(x), _f32(grad), _i32(mol_index)
+    W, b = W.double().contiguous(), b.double().contiguous()
+    A, n, _, d = grad.shape
+    F = W.shape[1]
+    check(_lib.lib().qmll_rff_derivative_features(_ptr(x), _ptr(grad), _ptr(W), _ptr(b), _ptr(mol_index), A, n, d, F,
+                                                  int(G.shape[0]), _ptr(G), _stream()), "qmll_rff_derivative_features")
+    return G
+
+
+def gram(Zrows, y, ZTZ, ZTy, f0=None, f1=None):
+    """ZTZ += Z^T Z (or the row block f0:f1 of it), ZTy += Z^T y, fp64, in place."""
+    if Zrows.dtype != torch.float64 or not Zrows.is_contiguous():
+        raise RuntimeError("gram needs a contiguous float64 row matrix")
+    M, F = Zrows.shape
+    yv = None
+    if y is not None:
+        yv = y.reshape(-1).double().contiguous()
+        if yv.shape[0] != M:
+            raise RuntimeError("targets have %d rows, features have %d" % (yv.shape[0], M))
+    zty = ZTy if ZTy is not None else None
+    if f0 is None:
+        check(_lib.lib().qmll_gram_f64(_ptr(Zrows), _ptr(yv), M, F, _ptr(ZTZ), _ptr(zty), _stream()), "qmll_gram_f64")
+    else:
+        check(_lib.lib().qmll_gram_tile_f64(_ptr(Zrows), _ptr(yv), M, F, int(f0), int(f1), _ptr(ZTZ), _ptr(zty),
+                                            _stream()), "qmll_gram_tile_f64")
+    return ZTZ, ZTy
+
+
+def matmul_and_reduce(A, B, C):
+    A, B = _f32(A), _f32(B)
+    if C.dtype != torch.float64 or not C.is_contiguous():
+        raise RuntimeError("matmul_and_reduce accumulates into a contiguous float64 tensor")
+    check(_lib.lib().qmll_matmul_and_reduce(_ptr(A), _ptr(B), A.shape[0], A.shape[1], B.shape[1], _ptr(C), _stream()),
+          "qmll_matmul_and_reduce")
+    return C
+
+
+# ---------------------------------------------------------------------------------------
+# torch.ops registration (names and argument order of the reference's TORCH_LIBRARY blocks)
+# ---------------------------------------------------------------------------------------
+_FCHL_SIG = ("Tensor X, Tensor Z, Tensor species, Tensor atomIDs, Tensor molIDs, Tensor atom_counts, Tensor cell, "
+             "Tensor inv_cell, Tensor Rs2, Tensor Rs3, Tensor eta2, Tensor eta3, Tensor two_body_decay, "
+             "Tensor three_body_weight, Tensor three_body_decay, Tensor rcut")
+
+_registered = False
+_libs = []
+
+
+def _fchl_fwd_impl(X, Z, species, atomIDs, molIDs, atom_counts, cell, inv_cell, Rs2, Rs3, eta2, eta3, two_body_decay,
+                   three_body_weight, three_body_decay, rcut):
+    for t, name in ((X, "coordinates"), (Z, "charges"), (species, "species"), (atomIDs, "atomIDs"),
+                    (molIDs, "molIDs"), (atom_counts, "atom_counts"), (cell, "cell"), (inv_cell, "inv_cell")):
+        _need_cuda(t, name)                                  # torchscript/FCHL19.cpp:251-258
+    prm = make_params(species.shape[0], Rs2, Rs3, eta2, eta3, two_body_decay, three_body_weight, three_body_decay, rcut)
+    types = element_types(X, Z, atom_counts, species)
+    return fchl_forward(X, types, cell, inv_cell, atomIDs, molIDs, atom_counts, Rs2, Rs3, prm)
+
+
+def _fchl_bwd_impl(grad, X, Z, species, atomIDs, molIDs, atom_counts, cell, inv_cell, Rs2, Rs3, eta2, eta3,
+                   two_body_decay, three_body_weight, three_body_decay, rcut):
+    prm = make_params(species.shape[0], Rs2, Rs3, eta2, eta3, two_body_decay, three_body_weight, three_body_decay, rcut)
+    types = element_types(X, Z, atom_counts, species)
+    g = fchl_vjp(grad, X, types, cell, inv_cell, atomIDs, molIDs, atom_counts, Rs2, Rs3, prm)
+    return g.reshape(X.shape)
+
+
+def _fchl_and_derivative_impl(X, Z, species, atomIDs, molIDs, atom_counts, cell, inv_cell, Rs2, Rs3, eta2, eta3,
+                              two_body_decay, three_body_weight, three_body_decay, rcut, gradients):
+    prm = make_params(species.shape[0], Rs2, Rs3, eta2, eta3, two_body_decay, three_body_weight, three_body_decay, rcut)
+    types = element_types(X, Z, atom_counts, species)
+    if gradients:
+        rep, jac = fchl_jacobian(X, types, cell, inv_cell, atomIDs, molIDs, atom_counts, Rs2, Rs3, prm)
+        return [rep, jac]
+    return [fchl_forward(X, types, cell, inv_cell, atomIDs, molIDs, atom_counts, Rs2, Rs3, prm)]
+
+
+def register_ops():
+    """Define qml_lightning_fchl::* and qml_lightning_sorf::* once per process."""
+    global _registered
+    if _registered:
+        return
+    _registered = True
+    Library = torch.library.Library
+
+    fl = Library("qml_lightning_fchl", "DEF")
+    fl.define("fchl_forwards(%s) -> Tensor" % _FCHL_SIG)
+    fl.define("fchl_backwards(Tensor grad, %s) -> Tensor" % _FCHL_SIG)
+    fl.define("get_fchl_and_derivative(%s, bool gradients) -> Tensor[]" % _FCHL_SIG)
+    fl.define("get_element_types(Tensor coordinates, Tensor charges, Tensor natom_counts, Tensor species) -> Tensor")
+    fl.define("get_num_neighbours(Tensor coordinates, Tensor natoms, Tensor rcut, Tensor lattice_vecs, "
+              "Tensor inv_lattice_vecs) -> Tensor")
+    fl.define("get_neighbour_list(Tensor coordinates, Tensor natoms, Tensor max_neighbours, Tensor rcut, "
+              "Tensor lattice_vecs, Tensor inv_lattice_vecs) -> Tensor")
+    fl.impl("fchl_forwards", _fchl_fwd_impl, "CompositeExplicitAutograd")
+    fl.impl("fchl_backwards", _fchl_bwd_impl, "CompositeExplicitAutograd")
+    fl.impl("get_fchl_and_derivative", _fchl_and_derivative_impl, "CompositeExplicitAutograd")
+    fl.impl("get_element_types", lambda X, Z, n, s: element_types(X, Z, n, s), "CompositeExplicitAutograd")
+    fl.impl("get_num_neighbours", lambda X, n, rc, c, ic: num_neighbours(X, n, rc, c, ic), "CompositeExplicitAutograd")
+    fl.impl("get_neighbour_list", lambda X, n, mx, rc, c, ic: neighbour_list(X, n, mx, rc, c, ic), "CompositeExplicitAutograd")
+
+    def fchl_setup(ctx, inputs, output):
+        ctx.save_for_backward(*inputs)
+
+    def fchl_backward(ctx, grad):
+        # autograd on X only (torchscript/FCHL19.cpp:314)
+        g = torch.ops.qml_lightning_fchl.fchl_backwards(grad.contiguous(), *ctx.saved_tensors)
+        return (g,) + (None,) * 15
+
+    torch.library.register_autograd("qml_lightning_fchl::fchl_forwards", fchl_backward, setup_context=fchl_setup,
+                                    lib=fl)
+
+    sl = Library("qml_lightning_sorf", "DEF")
+    sl.define("get_SORF_coefficients(Tensor u, Tensor d, Tensor coeff_normalisation, Tensor ntransforms) -> Tensor")
+    sl.define("get_SORF_coefficients_backward(Tensor grad, Tensor d, Tensor coeff_normalisation, Tensor ntransforms) "
+              "-> Tensor")
+    sl.define("get_cos_features(Tensor coeffs, Tensor b, Tensor nmol, Tensor batch_indexes) -> Tensor")
+    sl.define("get_cos_features_backward(Tensor grad, Tensor coeffs, Tensor b, Tensor nmol, Tensor batch_indexes) "
+              "-> Tensor")
+    sl.impl("get_SORF_coefficients",
+            lambda u, d, cn, nt: sorf_forward(u, d, _scalar(cn), int(nt.item())), "CompositeExplicitAutograd")   # SORF.cpp:85
+    sl.impl("get_SORF_coefficients_backward",
+            lambda g, d, cn, nt: sorf_adjoint(g, d, _scalar(cn), int(nt.item())), "CompositeExplicitAutograd")   # SORF.cpp:99
+    sl.impl("get_cos_features",
+            lambda c, b, nmol, idx: cos_features(c, b, int(nmol.item()), idx), "CompositeExplicitAutograd")      # SORF.cpp:118
+    sl.impl("get_cos_features_backward",
+            lambda g, c, b, nmol, idx: cos_features_backward(g, c, b, int(nmol.item()), idx), "CompositeExplicitAutograd")
+
+    def sorf_setup(ctx, inputs, output):
+        _, d, cn, nt = inputs
+        ctx.save_for_backward(d, cn, nt)
+
+    def sorf_backward(ctx, grad):
+        d, cn, nt = ctx.saved_tensors
+        return torch.ops.qml_lightning_sorf.get_SORF_coefficients_backward(grad.contiguous(), d, cn, nt), None, None, None
+
+    def cos_setup(ctx, inputs, output):
+        ctx.save_for_backward(*inputs)
+
+    def cos_backward(ctx, grad):
+        c, b, nmol, idx = ctx.saved_tensors
+        return torch.ops.qml_lightning_sorf.get_cos_features_backward(grad.contiguous(), c, b, nmol, idx), None, None, None
+
+    torch.library.register_autograd("qml_lightning_sorf::get_SORF_coefficients", sorf_backward,
+                                    setup_context=sorf_setup, lib=sl)
+    torch.library.register_autograd("qml_lightning_sorf::get_cos_features", cos_backward, setup_context=cos_setup,
+                                    lib=sl)
+    _libs.extend([fl, sl])

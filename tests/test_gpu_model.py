@@ -1,0 +1,242 @@
+"""GPU parity at the model level: the reference's Python API (FCHLCuda,
+HadamardFeaturesModel, RandomFourrierFeaturesModel, torch.ops, TorchScript, autograd
+forces, build_Z_components) against the fp64 oracle and the reference's known-answer vector."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import model as omodel
+from oracle import sorf as osorf
+from tests import helpers
+from tests.test_gpu_kernels import REL_EF, REL_REP, close, dev, make_batch, oracle_prm, t32, ti32
+
+pytestmark = pytest.mark.gpu
+
+
+def build_sorf_model(species, npcas, nstacks, ntransforms=1, sigma=2.0, fused=True, seed=10, **repkw):
+    from qml_lightning_amd.models.hadamard_features import HadamardFeaturesModel
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    rep = FCHLCuda(species=np.array(species), **repkw)
+    m = HadamardFeaturesModel(rep=rep, elements=np.array(species), ntransforms=ntransforms, sigma=sigma,
+                              llambda=1e-5, npcas=npcas, nstacks=nstacks, nbatch_train=4, nbatch_test=5, fused=fused)
+    red, D, bias, alpha = helpers.model_weights(len(species), rep.get_repsize(), npcas, nstacks, ntransforms, seed)
+    m.reductors = t32(red)
+    m.Dmat = t32(D)
+    m.bias = t32(bias)
+    m.alpha = torch.tensor(alpha, device=dev())
+    m.is_trained = True
+    return m, (red, D.astype(np.float64), bias, alpha.astype(np.float32).astype(np.float64))
+
+
+def inputs(X, Z, aid, mid, nat):
+    return t32(X), t32(Z), ti32(aid), ti32(mid), ti32(nat)
+
+
+def test_reference_known_answer_aspirin(kat):
+    """unit_tests/models/unit_test_sorf.py of the reference, run through this library."""
+    from qml_lightning_amd.models.hadamard_features import HadamardFeaturesModel
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    d = kat
+    for fused in (True, False):
+        rep = FCHLCuda(species=np.array([1, 6, 8]), rcut=6.0, nRs2=24, nRs3=22, eta2=0.28, eta3=3.2,
+                       two_body_decay=2.3, three_body_weight=18.8, three_body_decay=0.65)
+        rep.three_body_weight = torch.tensor(float(d["three_body_weight"]))
+        assert np.allclose(rep.Rs2.cpu().numpy(), d["Rs2"]) and np.allclose(rep.Rs3.cpu().numpy(), d["Rs3"])
+        m = HadamardFeaturesModel(rep=rep, elements=np.array([1, 6, 8]), ntransforms=1, sigma=2.0, llambda=1e-5,
+                                  npcas=128, nstacks=128, fused=fused)
+        m.reductors = t32(d["reductors"])
+        m.Dmat = t32(d["Dmat"].astype(np.float32))
+        m.bias = t32(d["bias"])
+        m.alpha = torch.tensor(d["alpha"], device=dev())
+        X = t32(d["coordinates"]).unsqueeze(0)
+        X.requires_grad = True
+        Z = t32(d["charges"]).unsqueeze(0)
+        n = d["coordinates"].shape[0]
+        E = m.forward(X, Z, torch.arange(n, dtype=torch.int32, device=dev()),
+                      torch.zeros(n, dtype=torch.int32, device=dev()), ti32([n]))
+        F, = torch.autograd.grad(-E.sum(), X)
+        total = d["self_energy"][d["charges"]].sum() + E.item()
+        assert np.isclose(float(d["ref_energy"]), total)                       # unit_test_sorf.py:100
+        assert abs(total - float(d["ref_energy"])) < 0.1
+        # unit_test_sorf.py:101 asserts rtol = atol = 1e-4 against values printed to 5 digits;
+        # the print alone rounds 5e1-sized entries by up to 5e-4, so allow 1e-3 absolute
+        got = F.squeeze(0).cpu().numpy()
+        assert np.abs(got - d["ref_forces"]).max() < 1e-3 + 1e-4 * np.abs(d["ref_forces"]).max()
+        assert np.isclose(d["ref_forces"], got, rtol=1e-4, atol=1e-3).all()
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("case", ["benzene_c1", "aspirin_c2", "ragged_c3"])
+def test_sorf_energy_and_forces_vs_oracle(case, fused):
+    cfg = {
+        "benzene_c1": (helpers.benzene_batch(5, 0), [1, 6], 64, 8),
+        "aspirin_c2": (helpers.fixed_composition_batch(helpers.ASPIRIN, 4, 1), [1, 6, 8], 128, 16),
+        "ragged_c3": (helpers.ragged_batch(9, 2), [1, 6, 7, 8, 9], 128, 4),
+    }[case]
+    (coords, charges), species, npcas, nstacks = cfg
+    m, (red, D, bias, alpha) = build_sorf_model(species, npcas, nstacks, fused=fused)
+    prm = oracle_prm(species)
+    X, Z, aid, mid, nat = make_batch(coords, charges)
+    E, F, Zf = omodel.sorf_energy_forces(X, Z, aid, mid, nat, prm, species, red, D, bias, alpha, 2.0)
+    gX, gZ, gaid, gmid, gnat = inputs(X, Z, aid, mid, nat)
+    e, f = m.predict_opt(gX, gZ, gaid, gmid, gnat)
+    close(e, E, REL_EF, "energies")
+    close(f, F, REL_EF, "forces")
+    for mm in range(len(nat)):
+        assert (f[mm, nat[mm]:] == 0).all()
+    e_only = m.predict_opt(gX.detach().clone(), gZ, gaid, gmid, gnat, forces=False)
+    close(e_only, E, REL_EF, "energies, no forces")
+
+
+def test_two_transforms_and_torch_ops_directly():
+    """ntransforms = 2 through the registered operators, autograd included."""
+    species = [1, 6]
+    (coords, charges) = helpers.benzene_batch(2, 3)
+    m, (red, D, bias, alpha) = build_sorf_model(species, 32, 4, ntransforms=2, fused=False)
+    prm = oracle_prm(species)
+    X, Z, aid, mid, nat = make_batch(coords, charges)
+    E, F, _ = omodel.sorf_energy_forces(X, Z, aid, mid, nat, prm, species, red, D, bias, alpha, 2.0)
+    e, f = m.predict_opt(*inputs(X, Z, aid, mid, nat))
+    close(e, E, REL_EF)
+    close(f, F, REL_EF)
+    m2, _ = build_sorf_model(species, 32, 4, ntransforms=2, fused=True)
+    e2, f2 = m2.predict_opt(*inputs(X, Z, aid, mid, nat))
+    close(e2, E, REL_EF)
+    close(f2, F, REL_EF)
+
+
+def test_torchscript_roundtrip(tmp_path):
+    species = [1, 6, 8]
+    (coords, charges) = helpers.fixed_composition_batch(helpers.ASPIRIN, 3, 1)
+    X, Z, aid, mid, nat = make_batch(coords, charges)
+    for fused in (True, False):
+        m, _ = build_sorf_model(species, 64, 8, fused=fused)
+        gX, gZ, gaid, gmid, gnat = inputs(X, Z, aid, mid, nat)
+        e0, f0 = m.predict_opt(gX, gZ, gaid, gmid, gnat)
+        path = os.path.join(tmp_path, "model_%d.pt" % fused)
+        m.save_jit_model(path)
+        loaded = torch.jit.load(path)
+        gX2 = gX.detach().clone().requires_grad_(True)
+        e1 = loaded.forward(gX2, gZ, gaid, gmid, gnat)
+        f1, = torch.autograd.grad(-e1.sum(), gX2)
+        close(e1, e0.detach().cpu().numpy(), 1e-6, "scripted energies")
+        close(f1, f0.cpu().numpy(), 1e-5, "scripted forces")
+        code = loaded.code
+        assert ("sorf_energy" in code) == fused
+        assert ("get_SORF_coefficients" in code) == (not fused)
+
+
+def test_predict_from_lists_and_predict_cuda():
+    species = [1, 6, 7, 8, 9]
+    coords, charges = helpers.ragged_batch(11, 4)
+    m, (red, D, bias, alpha) = build_sorf_model(species, 64, 4)
+    prm = oracle_prm(species)
+    c32 = [np.asarray(c, dtype=np.float32) for c in coords]
+    X, Z, aid, mid, nat = make_batch(coords, charges)
+    E, F, _ = omodel.sorf_energy_forces(X, Z, aid, mid, nat, prm, species, red, D, bias, alpha, 2.0)
+    nmax = int(nat.max())
+    e, f = m.predict(c32, charges, nmax, forces=True)
+    close(e, E, REL_EF, "predict energies")
+    close(f, F, REL_EF, "predict forces")
+    # the explicit-Jacobian route (fp64 rows times alpha) gives the same numbers
+    e2, f2 = m.predict_cuda(c32, charges, nmax, forces=True, print_info=False)
+    close(e2, E, REL_EF, "predict_cuda energies")
+    close(f2, F, REL_EF, "predict_cuda forces")
+
+
+@pytest.mark.parametrize("mode", ["EF", "E", "F"])
+def test_training_rows_and_gram_vs_oracle(mode):
+    species = [1, 6]
+    coords, charges = helpers.benzene_batch(6, 0)
+    m, (red, D, bias, alpha) = build_sorf_model(species, 16, 4)
+    prm = oracle_prm(species)
+    rng = np.random.default_rng(14)
+    E = rng.normal(size=6) if "E" in mode else None
+    Fo = [rng.normal(size=(12, 3)) for _ in range(6)] if "F" in mode else None
+    c32 = [np.asarray(c, dtype=np.float32) for c in coords]
+    rows, ys = [], []
+    for i in range(0, 6, 4):          # nbatch_train = 4
+        X, Z, aid, mid, nat = make_batch(coords[i:i + 4], charges[i:i + 4])
+        r, y = omodel.sorf_training_rows(X, Z, aid, mid, nat, prm, species, red, D, bias, 2.0,
+                                         E=E[i:i + 4] if E is not None else None,
+                                         F=np.array(Fo[i:i + 4]) if Fo is not None else None)
+        rows.append(r)
+        ys.append(y)
+    R, Y = np.concatenate(rows), np.concatenate(ys)
+    ZTZ_ref, ZTy_ref = osorf.gram(R, Y)
+    ZTZ, ZTy = m.build_Z_components(c32, charges, E=E, F=Fo, print_info=False)
+    close(ZTZ, ZTZ_ref, 2e-5, "ZTZ " + mode)      # products of 1e-5-accurate features
+    close(ZTy, ZTy_ref, 2e-5, "ZTy " + mode)
+    for kw in (dict(ntiles=3), dict(cpu_solve=True), dict(use_specialized_matmul=True),
+               dict(ntiles=2, use_specialized_matmul=True)):
+        a, b = m.build_Z_components(c32, charges, E=E, F=Fo, print_info=False, **kw)
+        close(a, ZTZ_ref, 2e-5, "ZTZ %s %s" % (mode, kw))
+        close(b, ZTy_ref, 2e-5, "ZTy %s %s" % (mode, kw))
+    if mode == "EF":
+        # rows of one batch, and the train/predict loop closing on itself
+        data = m.format_data(c32[:4], charges[:4], E=E[:4], F=Fo[:4])
+        close(m._batch_rows(data, True), rows[0], REL_REP, "rows")
+        m.train(c32, charges, E=E, F=Fo, print_info=False)
+        assert m.alpha.shape == (m.nfeatures(),) and torch.isfinite(m.alpha).all()
+
+
+def test_rff_model_vs_oracle():
+    from qml_lightning_amd.models.random_features import RandomFourrierFeaturesModel
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    species = [1, 6, 8]
+    coords, charges = helpers.fixed_composition_batch(helpers.ASPIRIN, 3, 1)
+    rep = FCHLCuda(species=np.array(species))
+    np.random.seed(5)
+    m = RandomFourrierFeaturesModel(rep=rep, elements=np.array(species), sigma=2.0, nstacks=4, npcas=32,
+                                    nbatch_train=2, nbatch_test=2)
+    red, _, _, _ = helpers.model_weights(3, rep.get_repsize(), 32, 4)
+    m.reductors = t32(red)
+    rng = np.random.default_rng(13)
+    alpha = rng.normal(size=m.nfeatures())
+    m.alpha = torch.tensor(alpha, device=dev())
+    m.is_trained = True
+    W = m.W.double().cpu().numpy()
+    b = m.b.double().cpu().numpy()
+    prm = oracle_prm(species)
+    X, Z, aid, mid, nat = make_batch(coords, charges)
+    E, F, Zf = omodel.rff_energy_forces(X, Z, aid, mid, nat, prm, species, red, W, b,
+                                        alpha.astype(np.float32).astype(np.float64))
+    e, f = m.predict_opt(*inputs(X, Z, aid, mid, nat))
+    close(e, E, REL_EF, "rff energies")
+    close(f, F, REL_EF, "rff forces")
+    # training rows (fp64 kernels) against the oracle's rows
+    c32 = [np.asarray(c, dtype=np.float32) for c in coords]
+    data = m.format_data(c32, charges)
+    rows = m._batch_rows(data, True)
+    rep_o, J, _ = omodel.representation(X, Z, aid, mid, nat, prm, jacobian=True)
+    G = np.zeros((3, 21, 3, m.nfeatures()))
+    Zc = np.zeros((3, m.nfeatures()))
+    for ei, el in enumerate(species):
+        mask = Z.astype(int) == el
+        idx = np.nonzero(mask)[0]
+        sub = osorf.project(rep_o[mask], red[ei])
+        Zc += osorf.rff_features(sub, W[ei], b[ei], idx, 3)
+        G += osorf.rff_derivative_features(sub, osorf.project(J[mask], red[ei]), W[ei], b[ei], idx, 3)
+    close(rows[:3], Zc, REL_REP, "rff Z rows")
+    close(rows[3:], G.reshape(-1, m.nfeatures()), REL_REP, "rff G rows")
+    s = torch.jit.script(m)
+    gX = t32(X).requires_grad_(True)
+    e2 = s.forward(gX, t32(Z), ti32(aid), ti32(mid), ti32(nat))
+    close(e2, E, REL_EF, "scripted rff energies")
+
+
+def test_fd_helper_matches_jacobian():
+    """FCHLCuda.rep_deriv_fd, the reference's own check of its analytic Jacobian
+    (unit_tests/representation/test_fchl_derivative.py:60-82)."""
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    coords, charges = helpers.benzene_batch(1, 2)
+    rep = FCHLCuda(species=np.array([1, 6]), nRs2=8, nRs3=6)
+    X, Z, aid, mid, nat = make_batch(coords, charges)
+    gX, gZ, gaid, gmid, gnat = inputs(X, Z, aid, mid, nat)
+    r, J = rep.get_representation_and_derivative(gX, gZ, gaid, gmid, gnat)
+    fd = rep.rep_deriv_fd(gX, gZ, gaid, gmid, gnat, dx=0.005)
+    # fp32 finite differences: the reference only prints this norm; 2 % of the scale is
+    # what fp32 cancellation at dx = 0.005 allows
+    assert (fd - J.double()).abs().max() < 0.02 * J.abs().max()

@@ -1,0 +1,75 @@
+"""Host-side logic that needs no GPU: batch formatting, targets layout, model attributes
+and TorchScript compilation of the forward methods."""
+import numpy as np
+import torch
+
+from oracle import model as omodel
+
+
+def _model(fused=True):
+    from qml_lightning_amd.models.hadamard_features import HadamardFeaturesModel
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    rep = FCHLCuda(species=np.array([1, 6, 8]))
+    return HadamardFeaturesModel(rep=rep, elements=np.array([1, 6, 8]), ntransforms=1, sigma=2.0, npcas=128,
+                                 nstacks=4, fused=fused)
+
+
+def test_fchl_hyperparameter_tensors_match_reference_layout():
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    rep = FCHLCuda(species=np.array([1, 6, 7, 8]), eta3=2.7, three_body_weight=13.4)
+    assert rep.get_repsize() == 4 * 24 + 4 * 5 * 20
+    # FCHL.py:35 -- the weight handed to the kernels carries sqrt(eta3/pi)
+    assert np.isclose(float(rep.three_body_weight), np.sqrt(2.7 / np.pi) * 13.4)
+    assert np.allclose(rep.Rs2.cpu().numpy(), np.linspace(0, 6, 25)[1:])
+    assert rep.species.dtype == torch.float32 and rep.eta2.dim() == 0
+
+
+def test_format_data_matches_oracle_layout():
+    m = _model()
+    rng = np.random.default_rng(0)
+    coords = [rng.normal(size=(n, 3)) for n in (3, 5, 2)]
+    charges = [np.array([1, 6, 8]), np.array([6, 6, 1, 1, 8]), np.array([1, 1])]
+    E = [1.0, 2.0, 3.0]
+    F = [rng.normal(size=c.shape) for c in coords]
+    d = m.format_data(coords, charges, E=E, F=F)
+    X, Z, aid, mid, nat = omodel.format_batch(coords, charges)
+    assert np.allclose(d['coordinates'].cpu().numpy(), X.astype(np.float32))
+    assert (d['charges'].cpu().numpy() == Z).all() and d['charges'].dtype == torch.float32
+    assert (d['atomIDs'].cpu().numpy() == aid).all() and d['atomIDs'].dtype == torch.int32
+    assert (d['molIDs'].cpu().numpy() == mid).all() and (d['natom_counts'].cpu().numpy() == nat).all()
+    assert d['forces'].shape == (3, 5, 3) and d['forces'].dtype == torch.float64
+    assert (d['forces'][0, 3:] == 0).all()
+    assert d['cells'].shape == (0, 3, 3)
+    flat = Z.reshape(-1).astype(int)
+    for e in (1, 6, 8):
+        assert (d['element_index'][e].cpu().numpy() == np.nonzero(flat == e)[0]).all()
+    t = m._targets(d, 3, True, True)
+    assert t.shape == (3 + 3 * 5 * 3, 1) and t[1, 0] == 2.0
+    assert np.allclose(t[3:, 0].cpu().numpy(), d['forces'].cpu().numpy().reshape(-1))
+    t = m._targets(d, 3, False, True)
+    assert (t[:3] == 0).all()
+
+
+def test_self_energy_subtraction_and_unit_conversion():
+    m = _model()
+    Q = [np.array([1, 1, 8]), np.array([6, 1, 1, 1, 1]), np.array([8, 8]), np.array([6, 8])]
+    beta = {1: -0.5, 6: -37.8, 8: -75.0}
+    E = [sum(beta[int(q)] for q in qs) for qs in Q]
+    m.calculate_self_energy(Q, E)
+    for e, v in beta.items():
+        assert np.isclose(float(m.self_energy[e]), v, atol=1e-8)
+    m.set_subtract_self_energies(True)
+    d = m.format_data([np.zeros((len(q), 3)) for q in Q], Q, E=E)
+    assert np.allclose(d['energies'].cpu().numpy(), 0.0, atol=1e-8)
+
+
+def test_forward_compiles_to_torchscript_with_the_reference_operator_names():
+    for fused in (True, False):
+        s = torch.jit.script(_model(fused))
+        code = s.code + s.rep.code
+        assert "ops.qml_lightning_fchl.fchl_forwards" in code
+        if fused:
+            assert "ops.qml_lightning_sorf.sorf_energy" in code
+        else:
+            assert "ops.qml_lightning_sorf.get_SORF_coefficients" in code
+            assert "ops.qml_lightning_sorf.get_cos_features" in code
