@@ -180,16 +180,25 @@ def gram(Zrows, y):
     return Zrows.T @ Zrows, Zrows.T @ y
 
 
-def matmul_and_reduce(A32, B32, C64):
+def matmul_and_reduce(A32, B32, C64, block=16):
     """C += double(float(A) @ float(B)) with the inner sum carried in fp32 with Kahan
-    compensation (utils_kernel.cu:104-117).  Small sizes only (Python loop over K)."""
+    compensation (utils_kernel.cu:104-117).  The reference walks K in zero-padded tiles of
+    16 (utils_kernel.cu:90-101), and a zero product still applies the pending compensation
+    (y = fma(0, 0, -c)), so the padded steps are part of the arithmetic and are kept.
+    Small sizes only (Python loop over K)."""
     A32 = np.asarray(A32, dtype=np.float32)
     B32 = np.asarray(B32, dtype=np.float32)
+    K = A32.shape[1]
+    Kpad = -(-K // block) * block
     s = np.zeros((A32.shape[0], B32.shape[1]), dtype=np.float32)
     c = np.zeros_like(s)
-    for k in range(A32.shape[1]):
-        # fma(a, b, -c): the product is not rounded before the subtraction
-        yv = (A32[:, k:k + 1].astype(np.float64) * B32[k:k + 1, :].astype(np.float64) - c.astype(np.float64)).astype(np.float32)
+    for k in range(Kpad):
+        if k < K:
+            prod = A32[:, k:k + 1].astype(np.float64) * B32[k:k + 1, :].astype(np.float64)   # exact in fp64
+        else:
+            prod = np.zeros(s.shape)
+        # fma(a, b, -c): one rounding of the exact a*b - c
+        yv = (prod - c.astype(np.float64)).astype(np.float32)
         t = (s + yv).astype(np.float32)
         c = ((t - s).astype(np.float32) - yv).astype(np.float32)
         s = t

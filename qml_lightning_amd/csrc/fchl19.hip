@@ -189,9 +189,12 @@ __device__ __forceinline__ Triple triple_geometry(const Stage& s, int j, int k) 
     t.cj = -(ax * cx + ay * cy + az * cz) * ia * ic;        // (R_i-R_j).(R_k-R_j)
     const float cc = fminf(1.0f, fmaxf(-1.0f, t.ci));
     t.cosT = cc;
-    t.sinT = sqrtf(fmaxf(0.0f, 1.0f - cc * cc));
-    const float a2b2 = (t.a * t.a) * (t.b * t.b);
-    t.guard_inv = t.a * t.b * rsqrtf(fmaxf(1e-10f, a2b2 - vi * vi));
+    // a^2 b^2 - (d_ij.d_ik)^2 = |d_ij x d_ik|^2 (Lagrange): the cross product keeps full
+    // relative accuracy near collinear triples, where the difference of squares cancels
+    const float px = ay * bz - az * by, py = az * bx - ax * bz, pz = ax * by - ay * bx;
+    const float cross2 = px * px + py * py + pz * pz;
+    t.sinT = fminf(1.0f, sqrtf(cross2) * ia * ib);
+    t.guard_inv = t.a * t.b * rsqrtf(fmaxf(1e-10f, cross2));
     t.ujk[0] = cx * ic;
     t.ujk[1] = cy * ic;
     t.ujk[2] = cz * ic;

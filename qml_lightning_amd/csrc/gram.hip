@@ -123,15 +123,15 @@ __global__ __launch_bounds__(GT) void gram_kernel(const double* __restrict__ Z, 
         }
     }
 
-    // accumulator layout of v_mfma_f64_16x16x4_f64: lane holds rows 4*(lane/16)+r, r=0..3,
-    // of column lane%16
+    // accumulator layout of v_mfma_f64_16x16x4_f64 (measured on gfx950): register r of a
+    // lane holds row lane/16 + 4r of column lane%16
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int gi = i0 + wi + p * 16 + lk * 4 + r;
+                const int gi = i0 + wi + p * 16 + lk + 4 * r;
                 const int gj = j0 + wj + q * 16 + l16;
                 if (gi < ilim && gj < F) {
                     const double v = acc[p][q][r];
