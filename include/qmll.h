@@ -153,11 +153,14 @@ int qmll_sin_coeffs_f64(const float* coeffs, const float* bias, int A, int F, do
 /* Replaces sorf_gpu.compute_molecular_featurization_derivative (hadamard_cuda.cpp:95-109,
  * launcher hadamard_kernel.cu:905-932, kernel :587-717).  cos_derivs f64 [A,F] (from
  * qmll_sin_coeffs_f64), input_derivative f32 [A,n,3,d] (projected Jacobian rows of the A
- * atoms), D f32 [T,S,d], mol_index i32 [A] -> G f64 [nmol,n,3,F] +=
- * normalisation * cos_derivs[a,s*d+p] * (prod_m (H/sqrt(d) diag(D[m,s])) u)[p],
- * accumulated with fp64 atomics into caller-owned memory. */
+ * atoms), D f32 [T,S,d] -> G f64 [nmol,n,3,F] +=
+ * normalisation * cos_derivs[a,s*d+p] * (prod_m (H/sqrt(d) diag(D[m,s])) u)[p].
+ * Two ways to say which molecule an atom belongs to:
+ *   mol_index i32 [A] (any order, seg_offsets NULL): fp64 atomics, as the reference does;
+ *   seg_offsets i32 [nmol+1] (atoms molecule-major, atoms seg[m]..seg[m+1] belong to m):
+ *   atomic-free, each G element read-modify-written once, fixed summation order. */
 int qmll_derivative_features(const double* cos_derivs, double normalisation, const int* mol_index,
-                             const float* input_derivative, const float* D,
+                             const int* seg_offsets, const float* input_derivative, const float* D,
                              int A, int n, int d, int S, int T, int nmol, double* G, qmll_stream_t stream);
 
 /* Fused predict path for one element: SORF (T = ntransforms) + cos features + energy

@@ -42,7 +42,7 @@ PROTOTYPES = {
     "qmll_cos_features_f64": [P, P, P, c_int, c_int, c_int, P, P],
     "qmll_cos_features_backward": [P, P, P, P, c_int, c_int, c_int, P, P],
     "qmll_sin_coeffs_f64": [P, P, c_int, c_int, P, P],
-    "qmll_derivative_features": [P, c_double, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, P],
+    "qmll_derivative_features": [P, c_double, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, P],
     "qmll_sorf_energy_fused": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_float, P, P, P],
     "qmll_rff_features": [P, P, P, P, c_int, c_int, c_int, c_int, P, P],
     "qmll_rff_derivative_features": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],

@@ -296,6 +296,68 @@ __global__ __launch_bounds__(SORF_THREADS) void derivative_features_kernel(
     }
 }
 
+// Segmented, atomic-free variant for molecule-major atoms: seg[mol]..seg[mol+1] are the
+// atoms of molecule `mol`.  A wavefront owns (molecule, stack): it keeps the sin
+// coefficients of a chunk of the molecule's atoms for that stack in registers, walks the
+// 3n target rows, sums the chained transforms of the chunk's atoms in registers and adds
+// the row slice into G once (each G element has exactly one owner, so a plain
+// read-modify-write is enough and the sum order is fixed).
+template <int LOG2D>
+__global__ __launch_bounds__(SORF_THREADS) void derivative_features_seg_kernel(
+    const double* __restrict__ cos_derivs, double normalisation, const int* __restrict__ seg,
+    const float* __restrict__ input_derivative, const float* __restrict__ D, int n, int S, int T, float hscale,
+    double* __restrict__ G) {
+    using Sh = Shape<LOG2D>;
+    constexpr int AC = Sh::EPL >= 16 ? 1 : (Sh::EPL >= 4 ? 4 : 8);   // atoms per register chunk
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub = lane / Sh::LANES, l = lane % Sh::LANES;
+    const int e0 = l * Sh::EPL;
+    const int mol = blockIdx.x;
+    const int a0 = seg[mol], a1 = seg[mol + 1];
+    if (a1 <= a0) return;
+    const size_t F = (size_t)S * Sh::d;
+    const int step = SORF_WAVES * gridDim.y * Sh::G;
+    const double scale = normalisation * (double)hscale;
+    for (int s = (blockIdx.y * SORF_WAVES + wave) * Sh::G + sub; s < S; s += step) {
+        for (int ac = a0; ac < a1; ac += AC) {
+            const int na = min(AC, a1 - ac);
+            float cdv[AC][Sh::EPL];
+#pragma unroll
+            for (int i = 0; i < AC; ++i)
+#pragma unroll
+                for (int q = 0; q < Sh::EPL; ++q)
+                    cdv[i][q] = i < na ? (float)cos_derivs[(size_t)(ac + i) * F + (size_t)s * Sh::d + e0 + q] : 0.0f;
+            for (int jx = 0; jx < 3 * n; ++jx) {
+                float acc[Sh::EPL];
+#pragma unroll
+                for (int q = 0; q < Sh::EPL; ++q) acc[q] = 0.0f;
+                bool any = false;
+#pragma unroll
+                for (int i = 0; i < AC; ++i) {
+                    if (i < na) {
+                        float v[Sh::EPL];
+                        load_vec<Sh::EPL>(v, input_derivative + (((size_t)(ac + i) * n) * 3 + jx) * Sh::d + e0);
+                        float nz = 0.0f;
+#pragma unroll
+                        for (int q = 0; q < Sh::EPL; ++q) nz += fabsf(v[q]);
+                        if (__ballot(nz != 0.0f) != 0ull) {
+                            any = true;
+                            chain_forward<LOG2D>(v, D, S, T, s, e0, lane);
+#pragma unroll
+                            for (int q = 0; q < Sh::EPL; ++q) acc[q] = fmaf(cdv[i][q], v[q], acc[q]);
+                        }
+                    }
+                }
+                if (any) {
+                    double* g = G + (((size_t)mol * n) * 3 + jx) * F + (size_t)s * Sh::d + e0;
+#pragma unroll
+                    for (int q = 0; q < Sh::EPL; ++q) g[q] += scale * (double)acc[q];
+                }
+            }
+        }
+    }
+}
+
 // ---- elementwise feature kernels ----------------------------------------------------
 // Thread = feature column f, workgroup = (feature tile, atom chunk).  Within its chunk a
 // thread keeps a running sum while consecutive atoms belong to the same molecule and
@@ -442,22 +504,35 @@ extern "C" int qmll_sorf_energy_fused(const float* x, const float* D, const floa
 }
 
 extern "C" int qmll_derivative_features(const double* cos_derivs, double normalisation, const int* mol_index,
-                                        const float* input_derivative, const float* D, int A, int n, int d, int S,
-                                        int T, int nmol, double* G, qmll_stream_t stream) {
+                                        const int* seg_offsets, const float* input_derivative, const float* D, int A,
+                                        int n, int d, int S, int T, int nmol, double* G, qmll_stream_t stream) {
     int rc = check_sorf("qmll_derivative_features", A, d, S, T);
     if (rc) return rc;
     QMLL_REQUIRE(n >= 0 && nmol >= 0, QMLL_ERR_INVALID, "qmll_derivative_features: bad size n=%d nmol=%d", n, nmol);
-    if (A == 0 || n == 0) return QMLL_OK;
-    QMLL_REQUIRE(cos_derivs && mol_index && input_derivative && D && G, QMLL_ERR_INVALID,
-                 "qmll_derivative_features: null pointer");
-    QMLL_REQUIRE((long long)A * n < 2147483647LL, QMLL_ERR_INVALID, "qmll_derivative_features: A*n too large");
+    if (A == 0 || n == 0 || nmol == 0) return QMLL_OK;
+    QMLL_REQUIRE(cos_derivs && input_derivative && D && G, QMLL_ERR_INVALID, "qmll_derivative_features: null pointer");
+    QMLL_REQUIRE(mol_index || seg_offsets, QMLL_ERR_INVALID,
+                 "qmll_derivative_features: need mol_index or seg_offsets");
     const float hscale = hnorm(d, T);
+    if (seg_offsets) {
+        const int G_ = d >= 64 ? 1 : 64 / d;
+        int ny = (S + SORF_WAVES * G_ - 1) / (SORF_WAVES * G_);
+        if (ny > 65535) ny = 65535;
+        dim3 grid(nmol, ny);
+#define CALL(L)                                                                                                     \
+    hipLaunchKernelGGL(derivative_features_seg_kernel<L>, grid, dim3(SORF_THREADS), 0, (hipStream_t)stream,         \
+                       cos_derivs, normalisation, seg_offsets, input_derivative, D, n, S, T, hscale, G)
+        DISPATCH_LOG2D(qmll_log2(d), CALL)
+#undef CALL
+    } else {
+        QMLL_REQUIRE((long long)A * n < 2147483647LL, QMLL_ERR_INVALID, "qmll_derivative_features: A*n too large");
 #define CALL(L)                                                                                                   \
     hipLaunchKernelGGL(derivative_features_kernel<L>, dim3((unsigned)(A * n)), dim3(SORF_THREADS), 0,             \
                        (hipStream_t)stream, cos_derivs, normalisation, mol_index, input_derivative, D, n, S, T, \
                        hscale, G)
-    DISPATCH_LOG2D(qmll_log2(d), CALL)
+        DISPATCH_LOG2D(qmll_log2(d), CALL)
 #undef CALL
+    }
     QMLL_CHECK_LAUNCH("qmll_derivative_features");
     return QMLL_OK;
 }

@@ -14,8 +14,7 @@ import numpy as np
 import torch
 
 from .. import ops
-from ..cuda.sorf_gpu import (compute_hadamard_features, compute_molecular_featurization_derivative,
-                             compute_partial_feature_derivatives, sorf_matrix_gpu)
+from ..cuda.sorf_gpu import compute_hadamard_features, compute_partial_feature_derivatives
 from ..representations.dimensionality_reduction import project_representation
 from .kernel import BaseKernel, _default_device
 
@@ -110,8 +109,9 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         if derivative_features is not None and grad is not None:
             cos_derivs = torch.empty(coeffs.shape, device=coeffs.device, dtype=torch.float64)
             compute_partial_feature_derivatives(coeffs, self.bias[element_idx], cos_derivs)
-            compute_molecular_featurization_derivative(cos_derivs, coeff_normalisation, self.Dmat[element_idx], grad,
-                                                       indexes, derivative_features)
+            # `indexes` comes from a molecule-major gather, so the atomic-free kernel applies
+            ops.derivative_features(cos_derivs, coeff_normalisation, self.Dmat[element_idx], grad, indexes,
+                                    derivative_features, molecule_major=True)
 
     def forward(self, X, Z, atomIDs, molIDs, atom_counts, cell: Optional[torch.Tensor] = None,
                 inv_cell: Optional[torch.Tensor] = None):

@@ -248,7 +248,10 @@ def sin_coeffs(coeffs, bias, out):
     return out
 
 
-def derivative_features(cos_derivs, normalisation, D, input_derivatives, mol_index, G):
+def derivative_features(cos_derivs, normalisation, D, input_derivatives, mol_index, G, molecule_major=False):
+    """G += force-feature rows of one element.  molecule_major=True promises that
+    mol_index is non-decreasing (atoms grouped by molecule): the atomic-free kernel is
+    used, with segment offsets found on the device."""
     D, u, mol_index = _f32(D), _f32(input_derivatives), _i32(mol_index)
     A, n, _, d = u.shape
     T, S, _ = D.shape
@@ -257,8 +260,13 @@ def derivative_features(cos_derivs, normalisation, D, input_derivatives, mol_ind
         raise RuntimeError("derivative features need contiguous float64 cos_derivs and output")
     if G.shape[1] != n or G.shape[3] != S * d:
         raise RuntimeError("feature_derivatives has shape %s, expected [nmol,%d,3,%d]" % (tuple(G.shape), n, S * d))
-    check(_lib.lib().qmll_derivative_features(_ptr(cos_derivs), float(normalisation), _ptr(mol_index), _ptr(u), _ptr(D),
-                                              A, n, d, S, T, int(G.shape[0]), _ptr(G), _stream()),
+    nmol = int(G.shape[0])
+    seg = None
+    if molecule_major:
+        bounds = torch.arange(nmol + 1, dtype=torch.int32, device=u.device)
+        seg = torch.searchsorted(mol_index, bounds).to(torch.int32)
+    check(_lib.lib().qmll_derivative_features(_ptr(cos_derivs), float(normalisation), _ptr(mol_index), _ptr(seg),
+                                              _ptr(u), _ptr(D), A, n, d, S, T, nmol, _ptr(G), _stream()),
           "qmll_derivative_features")
     return G
 

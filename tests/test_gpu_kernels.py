@@ -247,9 +247,11 @@ def test_derivative_features(d, S, T):
     idx = np.sort(rng.integers(0, nmol, A)).astype(np.int32)
     norm = 2.5
     ref = sorf.derivative_features(cd, norm, idx, u, D, nmol)
-    G = torch.zeros(nmol, n, 3, S * d, dtype=torch.float64, device=dev())
-    ops.derivative_features(torch.tensor(cd, device=dev()), norm, t32(D), t32(u), ti32(idx), G)
-    close(G, ref, REL_REP, "derivative features")
+    for molecule_major in (False, True):
+        G = torch.ones(nmol, n, 3, S * d, dtype=torch.float64, device=dev())      # accumulates in place
+        ops.derivative_features(torch.tensor(cd, device=dev()), norm, t32(D), t32(u), ti32(idx), G,
+                                molecule_major=molecule_major)
+        close(G - 1.0, ref, REL_REP, "derivative features, molecule_major=%s" % molecule_major)
 
 
 @pytest.mark.parametrize("d,S,T", [(8, 3, 1), (64, 5, 2), (128, 16, 1), (256, 8, 1), (512, 4, 1)])
