@@ -45,25 +45,35 @@ struct FchlArgs {
 constexpr int TCH = 256;  // triples per LDS chunk
 constexpr float PI_F = 3.14159265358979323846f;
 
+// LDS neighbour arrays of one central atom, sorted by element type (stable in j within a
+// type); goff[e]..goff[e+1] is the slice of type e.
 struct Stage {
     float* dx;
     float* dy;
     float* dz;
     float* r;
+    float* fc;    // cosine cutoff at r
+    float* dfc;   // its r-derivative
     int* el;
     int* j;
+    int* goff;    // [ns+1]
     float* next;  // first free float after the neighbour arrays
 };
 
-__device__ __forceinline__ Stage carve(float* smem, int cap) {
+constexpr int STAGE_ARRAYS = 8;   // per-neighbour arrays carved by `carve`
+
+__device__ __forceinline__ Stage carve(float* smem, int cap, int ns) {
     Stage s;
     s.dx = smem;
     s.dy = s.dx + cap;
     s.dz = s.dy + cap;
     s.r = s.dz + cap;
-    s.el = (int*)(s.r + cap);
+    s.fc = s.r + cap;
+    s.dfc = s.fc + cap;
+    s.el = (int*)(s.dfc + cap);
     s.j = s.el + cap;
-    s.next = (float*)(s.j + cap);
+    s.goff = s.j + cap;
+    s.next = (float*)(s.goff + ns + 1);
     return s;
 }
 
@@ -79,11 +89,17 @@ __device__ __forceinline__ void min_image(float& dx, float& dy, float& dz, const
     dz = c[6] * s0 + c[7] * s1 + c[8] * s2;
 }
 
-// Fill the LDS neighbour arrays of atom (m,i); returns the neighbour count.  Neighbours
-// whose element type is negative (charge not in `species`) are dropped.
+__device__ __forceinline__ float cutoff(float r, float inv_rc) { return 0.5f * (cosf(r * PI_F * inv_rc) + 1.0f); }
+__device__ __forceinline__ float dcutoff(float r, float inv_rc) { return -0.5f * PI_F * inv_rc * sinf(r * PI_F * inv_rc); }
+
+// Fill the LDS neighbour arrays of atom (m,i), sorted by element type; returns the
+// neighbour count.  Neighbours whose element type is negative (charge not in `species`)
+// are dropped.  Pass 0 counts per type (lane e keeps the count of type e), pass 1 scatters
+// each neighbour to goff[type] + its rank among the earlier neighbours of that type.
 __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i, int lane) {
     const float* Xm = a.X + (size_t)m * a.n * 3;
     const int* tm = a.types + (size_t)m * a.n;
+    const int ns = a.p.nspecies;
     const bool pbc = a.cell != nullptr;
     float c[9], ic[9];
     if (pbc) {
@@ -94,7 +110,7 @@ __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i,
     }
     const float xi = Xm[i * 3 + 0], yi = Xm[i * 3 + 1], zi = Xm[i * 3 + 2];
     const float rc2 = a.p.rcut * a.p.rcut;
-    int count = 0;
+    const float inv_rc = 1.0f / a.p.rcut;
     const bool have_list = a.nlist != nullptr;
     int total;
     const int* li = nullptr;
@@ -106,44 +122,72 @@ __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i,
         total = a.natoms[m];
         if (total > a.n) total = a.n;
     }
-    for (int base = 0; base < total; base += QMLL_WAVE) {
-        const int t = base + lane;
-        bool ok = t < total;
-        int j = 0;
-        float dx = 0.f, dy = 0.f, dz = 0.f, r2 = 0.f;
-        int e = -1;
-        if (ok) {
-            j = have_list ? li[t] : t;
-            ok = j >= 0 && j < a.n;
+    int mycount = 0;   // lane e: neighbours of type e seen so far
+    int nn = 0;
+    for (int pass = 0; pass < 2; ++pass) {
+        if (pass == 1) {
+            // exclusive prefix over the type counts -> goff
+            int incl = mycount;
+            for (int o = 1; o < 64; o <<= 1) {
+                const int up = __shfl_up(incl, o, 64);
+                if (lane >= o) incl += up;
+            }
+            if (lane < ns) s.goff[lane] = incl - mycount;
+            nn = __shfl(incl, ns - 1, 64);
+            if (nn > a.cap) nn = a.cap;
+            if (lane == 0) s.goff[ns] = nn;
+            mycount = 0;
+            __syncthreads();
         }
-        if (ok) {
-            dx = xi - Xm[j * 3 + 0];
-            dy = yi - Xm[j * 3 + 1];
-            dz = zi - Xm[j * 3 + 2];
-            if (pbc) min_image(dx, dy, dz, c, ic);
-            r2 = dx * dx + dy * dy + dz * dz;
-            e = tm[j];
-            // a supplied list is authoritative (it may be stale on purpose, e.g. finite
-            // differences with a frozen list); only the built-in search applies the cutoff
-            ok = (have_list ? (r2 > 0.0f) : (r2 < rc2 && r2 > 0.0f)) && e >= 0;
+        for (int base = 0; base < total; base += QMLL_WAVE) {
+            const int t = base + lane;
+            bool ok = t < total;
+            int j = 0;
+            float dx = 0.f, dy = 0.f, dz = 0.f, r2 = 0.f;
+            int e = -1;
+            if (ok) {
+                j = have_list ? li[t] : t;
+                ok = j >= 0 && j < a.n;
+            }
+            if (ok) {
+                dx = xi - Xm[j * 3 + 0];
+                dy = yi - Xm[j * 3 + 1];
+                dz = zi - Xm[j * 3 + 2];
+                if (pbc) min_image(dx, dy, dz, c, ic);
+                r2 = dx * dx + dy * dy + dz * dz;
+                e = tm[j];
+                // a supplied list is authoritative (it may be stale on purpose, e.g. finite
+                // differences with a frozen list); only the built-in search applies the cutoff
+                ok = (have_list ? (r2 > 0.0f) : (r2 < rc2 && r2 > 0.0f)) && e >= 0 && e < ns;
+            }
+            for (int ep = 0; ep < ns; ++ep) {
+                const unsigned long long mask = __ballot(ok && e == ep);
+                const int before = __builtin_amdgcn_readlane(mycount, ep);
+                if (pass == 1 && ok && e == ep) {
+                    const int pos = s.goff[ep] + before + __popcll(mask & ((1ull << lane) - 1ull));
+                    if (pos < a.cap) {
+                        const float r = sqrtf(r2);
+                        s.dx[pos] = dx;
+                        s.dy[pos] = dy;
+                        s.dz[pos] = dz;
+                        s.r[pos] = r;
+                        s.fc[pos] = cutoff(r, inv_rc);
+                        s.dfc[pos] = dcutoff(r, inv_rc);
+                        s.el[pos] = e;
+                        s.j[pos] = j;
+                    }
+                }
+                if (lane == ep) mycount += __popcll(mask);
+            }
         }
-        const unsigned long long mask = __ballot(ok);
-        const int pos = count + __popcll(mask & ((1ull << lane) - 1ull));
-        if (ok && pos < a.cap) {
-            s.dx[pos] = dx;
-            s.dy[pos] = dy;
-            s.dz[pos] = dz;
-            s.r[pos] = sqrtf(r2);
-            s.el[pos] = e;
-            s.j[pos] = j;
-        }
-        count += __popcll(mask);
     }
-    return count < a.cap ? count : a.cap;
+    return nn;
 }
 
-__device__ __forceinline__ float cutoff(float r, float inv_rc) { return 0.5f * (cosf(r * PI_F * inv_rc) + 1.0f); }
-__device__ __forceinline__ float dcutoff(float r, float inv_rc) { return -0.5f * PI_F * inv_rc * sinf(r * PI_F * inv_rc); }
+// 2^x and log2(x) on the transcendental unit (1 ulp)
+__device__ __forceinline__ float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float flog2(float x) { return __builtin_amdgcn_logf(x); }
+constexpr float LOG2E = 1.4426950408889634f;
 
 // row index of pair t in the list of pairs (j<k) over nn items, rows enumerated j = 0..nn-2
 __device__ __forceinline__ void unrank_pair(int t, int nn, int& j, int& k) {
@@ -203,6 +247,14 @@ __device__ __forceinline__ Triple triple_geometry(const Stage& s, int j, int k) 
 
 // ---------------------------------------------------------------------------------
 // forward
+//
+// Atomic-free: with the neighbours sorted by element type every output block is owned by
+// one loop nest.  Two-body block of type e: lanes = (neighbour sub-slot, radial bin z),
+// serial over the neighbours of type e, partial sums folded across sub-slots by lane
+// shuffles.  Three-body block of the type pair (p<=q): the pair's triples are evaluated
+// once (lane = triple) into an LDS table (rho, K cos, K sin), then lanes = (triple
+// sub-slot, radial bin l) run over the table with the bin sums in registers.  Rows go
+// straight from registers to global memory.
 // ---------------------------------------------------------------------------------
 __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* __restrict__ rep) {
     extern __shared__ float smem[];
@@ -213,17 +265,15 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     const int ns = a.p.nspecies, nRs2 = a.p.nRs2, nRs3 = a.p.nRs3;
     const int R = ns * nRs2 + ns * (ns + 1) * nRs3;
 
-    Stage s = carve(smem, a.cap);
+    float* trip = smem;             // [TCH][4]: rho, K cos, K sin, -   (first: 16-byte aligned)
+    Stage s = carve(smem + 4 * TCH, a.cap, ns);
     float* smu = s.next;            // [cap]  mu_j
-    float* sis2 = smu + a.cap;      // [cap]  1/(2 sigma_j^2)
+    float* sis2 = smu + a.cap;      // [cap]  log2(e) / (2 sigma_j^2)
     float* spre = sis2 + a.cap;     // [cap]  r^-d2 fc / (sigma sqrt(2pi))
     float* slnRs2 = spre + a.cap;   // [nRs2]
     float* sinvRs2 = slnRs2 + nRs2; // [nRs2]
     float* sRs3 = sinvRs2 + nRs2;   // [nRs3]
-    float* acc = sRs3 + nRs3;       // [R]
-    float* trip = acc + R;          // [TCH][4]: rho, Kc, Ks, bin offset
 
-    for (int t = lane; t < R; t += QMLL_WAVE) acc[t] = 0.0f;
     for (int t = lane; t < nRs2; t += QMLL_WAVE) {
         const float v = a.Rs2[t];
         slnRs2[t] = logf(v);
@@ -234,56 +284,116 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     const int nn = stage_neighbours(a, s, m, i, lane);
     __syncthreads();
 
-    const float inv_rc = 1.0f / a.p.rcut;
     // per-neighbour two-body factors
     for (int j = lane; j < nn; j += QMLL_WAVE) {
         const float r = s.r[j];
         const float s2 = logf(1.0f + a.p.eta2 / (r * r));
         smu[j] = logf(r) - 0.5f * s2;                    // ln(r / sqrt(1 + eta2/r^2))
-        sis2[j] = 0.5f / s2;
-        spre[j] = rsqrtf(s2) * 0.3989422804014327f * powf(r, -a.p.two_body_decay) * cutoff(r, inv_rc);
+        sis2[j] = 0.5f * LOG2E / s2;
+        spre[j] = rsqrtf(s2) * 0.3989422804014327f * powf(r, -a.p.two_body_decay) * s.fc[j];
     }
     __syncthreads();
-    for (int it = lane; it < nn * nRs2; it += QMLL_WAVE) {
-        const int j = it / nRs2;
-        const int z = it - j * nRs2;
-        const float u = slnRs2[z] - smu[j];
-        const float v = spre[j] * sinvRs2[z] * expf(-u * u * sis2[j]);
-        atomicAdd(&acc[s.el[j] * nRs2 + z], v);
+
+    float* out = rep + ((size_t)m * a.n + i) * R;
+
+    // ---- two-body blocks ----
+    {
+        const int W = nRs2 < 64 ? nRs2 : 64;     // lanes per neighbour sub-slot
+        const int JS = 64 / W;                   // neighbour sub-slots
+        const int jsub = lane / W, zl = lane - jsub * W;
+        for (int zb = 0; zb < nRs2; zb += W) {
+            const int z = zb + zl;
+            const bool zok = z < nRs2 && jsub < JS;
+            const float lnRs = zok ? slnRs2[z] : 0.0f;
+            const float invRs = zok ? sinvRs2[z] : 0.0f;
+            for (int e = 0; e < ns; ++e) {
+                float acc = 0.0f;
+                if (zok) {
+                    for (int j = s.goff[e] + jsub; j < s.goff[e + 1]; j += JS) {
+                        const float u = lnRs - smu[j];
+                        acc = fmaf(spre[j] * invRs, fexp2(-u * u * sis2[j]), acc);
+                    }
+                }
+                float tot = acc;
+                for (int k = 1; k < JS; ++k) tot += __shfl(acc, zl + W * k, 64);
+                if (zok && jsub == 0) out[e * nRs2 + z] = tot;
+            }
+        }
     }
 
-    // three-body
-    const int ntrip = nn * (nn - 1) / 2;
+    // ---- three-body blocks ----
     const float zeta2 = 2.0f * expf(-0.5f * PI_F * PI_F);
-    for (int c0 = 0; c0 < ntrip; c0 += TCH) {
-        const int nchunk = min(TCH, ntrip - c0);
-        __syncthreads();
-        for (int tt = lane; tt < nchunk; tt += QMLL_WAVE) {
-            int j, k;
-            unrank_pair(c0 + tt, nn, j, k);
-            const Triple t = triple_geometry(s, j, k);
-            const float ksi = a.p.three_body_weight * (1.0f + 3.0f * t.ci * t.cj * t.ck) *
-                              powf(t.a * t.b * t.c, -a.p.three_body_decay);
-            const float f = zeta2 * ksi * cutoff(t.a, inv_rc) * cutoff(t.b, inv_rc);
-            trip[tt * 4 + 0] = 0.5f * (t.a + t.b);
-            trip[tt * 4 + 1] = f * t.cosT;
-            trip[tt * 4 + 2] = f * t.sinT;
-            trip[tt * 4 + 3] = __int_as_float(pair_offset(s.el[j], s.el[k], ns, nRs2, nRs3));
-        }
-        __syncthreads();
-        for (int it = lane; it < nchunk * nRs3; it += QMLL_WAVE) {
-            const int tt = it / nRs3;
-            const int l = it - tt * nRs3;
-            const float d = trip[tt * 4 + 0] - sRs3[l];
-            const float e = expf(-a.p.eta3 * d * d);
-            const int off = __float_as_int(trip[tt * 4 + 3]) + 2 * l;
-            atomicAdd(&acc[off], e * trip[tt * 4 + 1]);
-            atomicAdd(&acc[off + 1], e * trip[tt * 4 + 2]);
+    const float k3 = a.p.eta3 * LOG2E;
+    const int W3 = nRs3 < 64 ? nRs3 : 64;
+    const int TS = 64 / W3;
+    const int tsub = lane / W3, ll = lane - tsub * W3;
+    constexpr int MAXLB = 4;                     // radial bins handled: up to 4 x 64
+    for (int p = 0; p < ns; ++p) {
+        const int op = s.goff[p], np_ = s.goff[p + 1] - op;
+        for (int q = p; q < ns; ++q) {
+            const int oq = s.goff[q], nq = s.goff[q + 1] - oq;
+            const int ntr = (p == q) ? np_ * (np_ - 1) / 2 : np_ * nq;
+            const int sbase = pair_offset(p, q, ns, nRs2, nRs3);
+            float accc[MAXLB], accs[MAXLB];
+#pragma unroll
+            for (int b = 0; b < MAXLB; ++b) accc[b] = accs[b] = 0.0f;
+            for (int t0 = 0; t0 < ntr; t0 += TCH) {
+                const int nchunk = min(TCH, ntr - t0);
+                __syncthreads();
+                for (int tt = lane; tt < nchunk; tt += QMLL_WAVE) {
+                    int ja, kb;
+                    if (p == q) {
+                        unrank_pair(t0 + tt, np_, ja, kb);
+                    } else {
+                        ja = (t0 + tt) / nq;
+                        kb = (t0 + tt) - ja * nq;
+                    }
+                    const int j = op + ja, k = oq + kb;
+                    const Triple t = triple_geometry(s, j, k);
+                    const float ksi = a.p.three_body_weight * (1.0f + 3.0f * t.ci * t.cj * t.ck) *
+                                      fexp2(-a.p.three_body_decay * flog2(t.a * t.b * t.c));
+                    const float f = zeta2 * ksi * s.fc[j] * s.fc[k];
+                    *reinterpret_cast<float4*>(trip + tt * 4) =
+                        make_float4(0.5f * (t.a + t.b), f * t.cosT, f * t.sinT, 0.0f);
+                }
+                __syncthreads();
+                if (tsub < TS) {
+#pragma unroll
+                    for (int b = 0; b < MAXLB; ++b) {
+                        const int l = b * 64 + ll;
+                        if (b * 64 < nRs3 && l < nRs3) {
+                            const float rs = sRs3[l];
+                            float c_ = accc[b], s_ = accs[b];
+                            for (int tt = tsub; tt < nchunk; tt += TS) {
+                                const float4 v = *reinterpret_cast<const float4*>(trip + tt * 4);
+                                const float d = v.x - rs;
+                                const float e = fexp2(-k3 * d * d);
+                                c_ = fmaf(e, v.y, c_);
+                                s_ = fmaf(e, v.z, s_);
+                            }
+                            accc[b] = c_;
+                            accs[b] = s_;
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int b = 0; b < MAXLB; ++b) {
+                if (b * 64 < nRs3) {
+                    float tc = accc[b], tsn = accs[b];
+                    for (int k = 1; k < TS; ++k) {
+                        tc += __shfl(accc[b], ll + W3 * k, 64);
+                        tsn += __shfl(accs[b], ll + W3 * k, 64);
+                    }
+                    const int l = b * 64 + ll;
+                    if (tsub == 0 && l < nRs3) {
+                        out[sbase + 2 * l] = tc;
+                        out[sbase + 2 * l + 1] = tsn;
+                    }
+                }
+            }
         }
     }
-    __syncthreads();
-    float* out = rep + ((size_t)m * a.n + i) * R;
-    for (int t = lane; t < R; t += QMLL_WAVE) out[t] = acc[t];
 }
 
 // ---------------------------------------------------------------------------------
@@ -293,7 +403,7 @@ struct TwoBody {
     float mu, s2, s2p, mup, pre, fc, dfc, d2_over_r;
 };
 
-__device__ __forceinline__ TwoBody two_body_setup(float r, const qmll_fchl_params& p, float inv_rc) {
+__device__ __forceinline__ TwoBody two_body_setup(float r, float fc, float dfc, const qmll_fchl_params& p) {
     TwoBody t;
     const float r2 = r * r;
     t.s2 = logf(1.0f + p.eta2 / r2);
@@ -301,8 +411,8 @@ __device__ __forceinline__ TwoBody two_body_setup(float r, const qmll_fchl_param
     t.s2p = -2.0f * p.eta2 / (r * (r2 + p.eta2));      // d sigma^2 / dr
     t.mup = 1.0f / r - 0.5f * t.s2p;                   // d mu / dr
     t.pre = rsqrtf(t.s2) * 0.3989422804014327f * powf(r, -p.two_body_decay);
-    t.fc = cutoff(r, inv_rc);
-    t.dfc = dcutoff(r, inv_rc);
+    t.fc = fc;
+    t.dfc = dfc;
     t.d2_over_r = p.two_body_decay / r;
     return t;
 }
@@ -311,7 +421,7 @@ __device__ __forceinline__ TwoBody two_body_setup(float r, const qmll_fchl_param
 __device__ __forceinline__ void two_body_bin(const TwoBody& t, float lnRs, float invRs, float& val, float& dval) {
     const float u = lnRs - t.mu;
     const float inv_s2 = 1.0f / t.s2;
-    const float Bz = t.pre * invRs * expf(-0.5f * u * u * inv_s2);
+    const float Bz = t.pre * invRs * fexp2(-0.5f * LOG2E * u * u * inv_s2);
     const float Q = -0.5f * t.s2p * inv_s2 - t.d2_over_r + u * inv_s2 * (t.mup + 0.5f * u * t.s2p * inv_s2);
     val = Bz * t.fc;
     dval = Bz * (t.fc * Q + t.dfc);
@@ -324,7 +434,8 @@ struct TripleDeriv {
     float cia, cib, cic;     // partials of cos_i
 };
 
-__device__ __forceinline__ TripleDeriv triple_derivatives(const Triple& t, const qmll_fchl_params& p, float inv_rc) {
+__device__ __forceinline__ TripleDeriv triple_derivatives(const Triple& t, const qmll_fchl_params& p, float fa,
+                                                          float dfa, float fb, float dfb) {
     TripleDeriv d;
     const float ia = 1.0f / t.a, ib = 1.0f / t.b, ic = 1.0f / t.c;
     // d cos / d distance (law of cosines)
@@ -337,9 +448,7 @@ __device__ __forceinline__ TripleDeriv triple_derivatives(const Triple& t, const
     const float Pa = 3.0f * (d.cia * t.cj * t.ck + t.ci * cja * t.ck + t.ci * t.cj * cka);
     const float Pb = 3.0f * (d.cib * t.cj * t.ck + t.ci * cjb * t.ck + t.ci * t.cj * ckb);
     const float Pc = 3.0f * (d.cic * t.cj * t.ck + t.ci * cjc * t.ck + t.ci * t.cj * ckc);
-    const float dec = p.three_body_weight * powf(t.a * t.b * t.c, -p.three_body_decay);
-    const float fa = cutoff(t.a, inv_rc), fb = cutoff(t.b, inv_rc);
-    const float dfa = dcutoff(t.a, inv_rc), dfb = dcutoff(t.b, inv_rc);
+    const float dec = p.three_body_weight * fexp2(-p.three_body_decay * flog2(t.a * t.b * t.c));
     const float ksi = dec * P;
     const float ksia = dec * (Pa - p.three_body_decay * P * ia);
     const float ksib = dec * (Pb - p.three_body_decay * P * ib);
@@ -364,7 +473,7 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
     const int ns = a.p.nspecies, nRs2 = a.p.nRs2, nRs3 = a.p.nRs3;
     const int R = ns * nRs2 + ns * (ns + 1) * nRs3;
 
-    Stage s = carve(smem, a.cap);
+    Stage s = carve(smem, a.cap, ns);
     float* sgx = s.next;             // [cap] gradient on neighbour j
     float* sgy = sgx + a.cap;
     float* sgz = sgy + a.cap;
@@ -389,13 +498,13 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
     const int nn = stage_neighbours(a, s, m, i, lane);
     __syncthreads();
 
-    const float inv_rc = 1.0f / a.p.rcut;
+    const float k3 = a.p.eta3 * LOG2E;
     float gix = 0.0f, giy = 0.0f, giz = 0.0f;
 
     // two-body: lane per neighbour, serial over bins
     for (int j = lane; j < nn; j += QMLL_WAVE) {
         const float r = s.r[j];
-        const TwoBody tb = two_body_setup(r, a.p, inv_rc);
+        const TwoBody tb = two_body_setup(r, s.fc[j], s.dfc[j], a.p);
         const float* g = gin + s.el[j] * nRs2;
         float gr = 0.0f;
         for (int z = 0; z < nRs2; ++z) {
@@ -421,13 +530,13 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
         int j, k;
         unrank_pair(tt, nn, j, k);
         const Triple t = triple_geometry(s, j, k);
-        const TripleDeriv d = triple_derivatives(t, a.p, inv_rc);
+        const TripleDeriv d = triple_derivatives(t, a.p, s.fc[j], s.dfc[j], s.fc[k], s.dfc[k]);
         const float* g = gin + pair_offset(s.el[j], s.el[k], ns, nRs2, nRs3);
         const float rho = 0.5f * (t.a + t.b);
         float Gc = 0.f, Gs = 0.f, Hc = 0.f, Hs = 0.f;
         for (int l = 0; l < nRs3; ++l) {
             const float dl = rho - sRs3[l];
-            const float e = expf(-a.p.eta3 * dl * dl);
+            const float e = fexp2(-k3 * dl * dl);
             const float de = -2.0f * a.p.eta3 * dl * e;   // d e / d rho
             const float gc = g[2 * l], gs = g[2 * l + 1];
             Gc = fmaf(gc, e, Gc);
@@ -490,7 +599,7 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
     const int ns = a.p.nspecies, nRs2 = a.p.nRs2, nRs3 = a.p.nRs3;
     const int R = ns * nRs2 + ns * (ns + 1) * nRs3;
 
-    Stage s = carve(smem, a.cap);
+    Stage s = carve(smem, a.cap, ns);
     float* slnRs2 = s.next;          // [nRs2]
     float* sinvRs2 = slnRs2 + nRs2;  // [nRs2]
     float* sRs3 = sinvRs2 + nRs2;    // [nRs3]
@@ -506,7 +615,7 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
     const int nn = stage_neighbours(a, s, m, i, lane);
     __syncthreads();
 
-    const float inv_rc = 1.0f / a.p.rcut;
+    const float k3 = a.p.eta3 * LOG2E;
     const float zeta2 = 2.0f * expf(-0.5f * PI_F * PI_F);
     float* jbase = jac + (((size_t)m * a.n + i) * a.n) * 3 * R;
 
@@ -526,7 +635,7 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
                 const int j = j0 + it / nRs2;
                 const int z = it % nRs2;
                 const float r = s.r[j];
-                const TwoBody tb = two_body_setup(r, a.p, inv_rc);
+                const TwoBody tb = two_body_setup(r, s.fc[j], s.dfc[j], a.p);
                 float v, dv;
                 two_body_bin(tb, slnRs2[z], sinvRs2[z], v, dv);
                 const float ir = sign * dv / r;
@@ -553,10 +662,10 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
                     k = o < target ? target : o;
                 }
                 const Triple t = triple_geometry(s, j, k);
-                const TripleDeriv d = triple_derivatives(t, a.p, inv_rc);
+                const TripleDeriv d = triple_derivatives(t, a.p, s.fc[j], s.dfc[j], s.fc[k], s.dfc[k]);
                 const float rho = 0.5f * (t.a + t.b);
                 const float dl = rho - sRs3[l];
-                const float e = expf(-a.p.eta3 * dl * dl);
+                const float e = fexp2(-k3 * dl * dl);
                 const float de = -a.p.eta3 * dl * e;          // (d e/d rho) * (d rho/d a)
                 // T_c = zeta2 K e cosT, T_s = zeta2 K e sinT; partials wrt a, b, c
                 const float dcos = t.sinT * t.guard_inv;       // d cosT = dcos * d cos_i
@@ -664,7 +773,7 @@ extern "C" int qmll_fchl19_forward(const float* X, const int* types, const float
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(rep != nullptr, QMLL_ERR_INVALID, "qmll_fchl19_forward: null output");
     const int R = prm->nspecies * prm->nRs2 + prm->nspecies * (prm->nspecies + 1) * prm->nRs3;
-    const size_t lds = sizeof(float) * ((size_t)9 * a.cap + 2 * prm->nRs2 + prm->nRs3 + R + 4 * TCH);
+    const size_t lds = sizeof(float) * ((size_t)(STAGE_ARRAYS + 3) * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 + 4 * TCH + 4);
     QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
                  "qmll_fchl19_forward: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R, LDS_LIMIT);
     hipLaunchKernelGGL(fchl19_forward_kernel, dim3(A), dim3(64), lds, (hipStream_t)stream, a, rep);
@@ -684,7 +793,7 @@ extern "C" int qmll_fchl19_vjp(const float* X, const int* types, const float* ce
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(grad_rep && grad_X, QMLL_ERR_INVALID, "qmll_fchl19_vjp: null gradient pointer");
     const int R = prm->nspecies * prm->nRs2 + prm->nspecies * (prm->nspecies + 1) * prm->nRs3;
-    const size_t lds = sizeof(float) * ((size_t)9 * a.cap + 2 * prm->nRs2 + prm->nRs3 + R);
+    const size_t lds = sizeof(float) * ((size_t)(STAGE_ARRAYS + 3) * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 + R);
     QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
                  "qmll_fchl19_vjp: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R, LDS_LIMIT);
     hipLaunchKernelGGL(fchl19_vjp_kernel, dim3(A), dim3(64), lds, (hipStream_t)stream, a, grad_rep, grad_X);
@@ -704,7 +813,7 @@ extern "C" int qmll_fchl19_jacobian(const float* X, const int* types, const floa
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(jac != nullptr, QMLL_ERR_INVALID, "qmll_fchl19_jacobian: null output");
     const int R = prm->nspecies * prm->nRs2 + prm->nspecies * (prm->nspecies + 1) * prm->nRs3;
-    const size_t lds = sizeof(float) * ((size_t)6 * a.cap + 2 * prm->nRs2 + prm->nRs3 + 4 * (size_t)R);
+    const size_t lds = sizeof(float) * ((size_t)STAGE_ARRAYS * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 + 4 * (size_t)R);
     QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
                  "qmll_fchl19_jacobian: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R,
                  LDS_LIMIT);
