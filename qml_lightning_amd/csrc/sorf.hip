@@ -51,10 +51,14 @@ __device__ __forceinline__ void store_vec(const float (&v)[EPL], float* __restri
     }
 }
 
+// One radix-2 stage across lanes: lanes with bit MASK clear get v + partner, the others
+// partner - v.  The own value's sign is flipped with a per-lane mask (one xor), so the
+// add can take the partner straight from the DPP / swizzle network.
 template <int MASK>
 __device__ __forceinline__ float butterfly(float v, int lane) {
     const float p = lane_xor<MASK>(v);
-    return (lane & MASK) ? p - v : v + p;
+    const int sm = (lane & MASK) ? (int)0x80000000 : 0;
+    return p + __int_as_float(__float_as_int(v) ^ sm);
 }
 
 // unnormalised Walsh-Hadamard transform of the d = EPL*LANES values held by LANES lanes
@@ -84,19 +88,28 @@ __device__ __forceinline__ void fwht_wave(float (&v)[EPL], int lane) {
     }
 }
 
-template <int LOG2D>
-struct Shape {
-    static constexpr int d = 1 << LOG2D;
-    static constexpr int EPL = d >= 64 ? d / 64 : 1;
-    static constexpr int LANES = d >= 64 ? 64 : d;
+// Two ways to lay a length-d transform over a wavefront.
+//  Wide: all 64 lanes share one transform (d >= 64), d/64 elements per lane: consecutive
+//        lanes touch consecutive memory, best for the kernels that stream coefficients.
+//  Deep: 32 elements per lane, d/32 lanes per transform, 64/(d/32) transforms side by side:
+//        five of the log2(d) stages are register-to-register and only log2(d/32) go across
+//        lanes, best for the fused kernel, which is bound by instruction issue.
+template <int D_, int EPL_>
+struct ShapeT {
+    static constexpr int d = D_;
+    static constexpr int EPL = EPL_;
+    static constexpr int LANES = D_ / EPL_;
     static constexpr int G = 64 / LANES;   // transforms per wavefront
 };
+template <int LOG2D>
+using Shape = ShapeT<(1 << LOG2D), ((1 << LOG2D) >= 64 ? (1 << LOG2D) / 64 : 1)>;
+template <int LOG2D>
+using DeepShape = ShapeT<(1 << LOG2D), ((1 << LOG2D) >= 32 ? 32 : (1 << LOG2D))>;
 
 // forward chain for stack s: v <- prod_m H diag(D[m,s]) v   (unnormalised)
-template <int LOG2D>
-__device__ __forceinline__ void chain_forward(float (&v)[Shape<LOG2D>::EPL], const float* __restrict__ D, int S, int T,
+template <typename Sh>
+__device__ __forceinline__ void chain_forward(float (&v)[Sh::EPL], const float* __restrict__ D, int S, int T,
                                               int s, int e0, int lane) {
-    using Sh = Shape<LOG2D>;
     for (int m = 0; m < T; ++m) {
         float dv[Sh::EPL];
         load_vec<Sh::EPL>(dv, D + ((size_t)m * S + s) * Sh::d + e0);
@@ -107,10 +120,9 @@ __device__ __forceinline__ void chain_forward(float (&v)[Shape<LOG2D>::EPL], con
 }
 
 // adjoint chain: v <- prod_{m=T-1..0} diag(D[m,s]) H v   (unnormalised)
-template <int LOG2D>
-__device__ __forceinline__ void chain_adjoint(float (&v)[Shape<LOG2D>::EPL], const float* __restrict__ D, int S, int T,
+template <typename Sh>
+__device__ __forceinline__ void chain_adjoint(float (&v)[Sh::EPL], const float* __restrict__ D, int S, int T,
                                               int s, int e0, int lane) {
-    using Sh = Shape<LOG2D>;
     for (int m = T - 1; m >= 0; --m) {
         fwht_wave<Sh::EPL, Sh::LANES>(v, lane);
         float dv[Sh::EPL];
@@ -140,7 +152,7 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_forward_kernel(const float*
         float v[Sh::EPL];
 #pragma unroll
         for (int q = 0; q < Sh::EPL; ++q) v[q] = xv[q];
-        chain_forward<LOG2D>(v, D, S, T, s, e0, lane);
+        chain_forward<Sh>(v, D, S, T, s, e0, lane);
 #pragma unroll
         for (int q = 0; q < Sh::EPL; ++q) v[q] *= scale;
         store_vec<Sh::EPL>(v, out + (a * S + s) * Sh::d + e0);
@@ -164,7 +176,7 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_adjoint_kernel(const float*
     for (int s = wave * Sh::G + sub; s < S; s += SORF_WAVES * Sh::G) {
         float v[Sh::EPL];
         load_vec<Sh::EPL>(v, g + (a * S + s) * Sh::d + e0);
-        chain_adjoint<LOG2D>(v, D, S, T, s, e0, lane);
+        chain_adjoint<Sh>(v, D, S, T, s, e0, lane);
 #pragma unroll
         for (int q = 0; q < Sh::EPL; ++q) acc[q] += v[q];
     }
@@ -187,6 +199,11 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_adjoint_kernel(const float*
 }
 
 // ---- fused predict path ------------------------------------------------------------
+// Wide layout (coalesced loads of D, bias and alpha).  Per stack: sign diagonal, transform,
+// one sincos per feature, energy and d(energy)/d(coefficient), adjoint transform,
+// accumulate; the four wavefronts of a workgroup split the stacks and meet in LDS.  (The
+// deep layout has fewer cross-lane stages but its 128-byte-strided per-lane loads of the
+// three per-feature arrays cost more than the butterflies save: measured 1.7x slower.)
 template <int LOG2D, bool WITH_GRAD>
 __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_fused_kernel(
     const float* __restrict__ x, const float* __restrict__ D, const float* __restrict__ bias,
@@ -205,22 +222,29 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_fused_kernel(
     for (int q = 0; q < Sh::EPL; ++q) acc[q] = 0.0f;
     float energy = 0.0f;
     for (int s = wave * Sh::G + sub; s < S; s += SORF_WAVES * Sh::G) {
-        float v[Sh::EPL], bv[Sh::EPL], av[Sh::EPL];
+        float v[Sh::EPL];
 #pragma unroll
         for (int q = 0; q < Sh::EPL; ++q) v[q] = xv[q];
-        chain_forward<LOG2D>(v, D, S, T, s, e0, lane);
-        load_vec<Sh::EPL>(bv, bias + (size_t)s * Sh::d + e0);
-        load_vec<Sh::EPL>(av, alpha + (size_t)s * Sh::d + e0);
+        chain_forward<Sh>(v, D, S, T, s, e0, lane);
+        const float* bp = bias + (size_t)s * Sh::d + e0;
+        const float* ap = alpha + (size_t)s * Sh::d + e0;
+        constexpr int CH = Sh::EPL >= 4 ? 4 : Sh::EPL;
 #pragma unroll
-        for (int q = 0; q < Sh::EPL; ++q) {
-            float sn, cs;
-            sincos_f32(fmaf(v[q], scale, bv[q]), &sn, &cs);
-            const float w = av[q] * normf;
-            energy = fmaf(w, cs, energy);
-            v[q] = -w * sn;                       // d E / d coefficient
+        for (int q0 = 0; q0 < Sh::EPL; q0 += CH) {
+            float bv[CH], av[CH];
+            load_vec<CH>(bv, bp + q0);
+            load_vec<CH>(av, ap + q0);
+#pragma unroll
+            for (int q = 0; q < CH; ++q) {
+                float sn, cs;
+                sincos_f32(fmaf(v[q0 + q], scale, bv[q]), &sn, &cs);
+                const float w = av[q] * normf;
+                energy = fmaf(w, cs, energy);
+                v[q0 + q] = -w * sn;                       // d E / d coefficient
+            }
         }
         if constexpr (WITH_GRAD) {
-            chain_adjoint<LOG2D>(v, D, S, T, s, e0, lane);
+            chain_adjoint<Sh>(v, D, S, T, s, e0, lane);
 #pragma unroll
             for (int q = 0; q < Sh::EPL; ++q) acc[q] += v[q];
         }
@@ -228,9 +252,11 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_fused_kernel(
     energy = wave_sum(energy);
     if (lane == 0) ered[wave] = energy;
     if constexpr (WITH_GRAD) {
-        if constexpr (Sh::G > 1) {
+        // fold the G transforms that ran side by side in this wavefront
 #pragma unroll
-            for (int mask = Sh::LANES; mask < 64; mask <<= 1) acc[0] += __shfl_xor(acc[0], mask, 64);
+        for (int mask = Sh::LANES; mask < 64; mask <<= 1) {
+#pragma unroll
+            for (int q = 0; q < Sh::EPL; ++q) acc[q] += __shfl_xor(acc[q], mask, 64);
         }
         if (sub == 0) {
 #pragma unroll
@@ -285,7 +311,7 @@ __global__ __launch_bounds__(SORF_THREADS) void derivative_features_kernel(
             float v[Sh::EPL];
 #pragma unroll
             for (int q = 0; q < Sh::EPL; ++q) v[q] = uv[q];
-            chain_forward<LOG2D>(v, D, S, T, s, e0, lane);
+            chain_forward<Sh>(v, D, S, T, s, e0, lane);
 #pragma unroll
             for (int q = 0; q < Sh::EPL; ++q) {
                 const size_t f = (size_t)s * Sh::d + e0 + q;
@@ -342,7 +368,7 @@ __global__ __launch_bounds__(SORF_THREADS) void derivative_features_seg_kernel(
                         for (int q = 0; q < Sh::EPL; ++q) nz += fabsf(v[q]);
                         if (__ballot(nz != 0.0f) != 0ull) {
                             any = true;
-                            chain_forward<LOG2D>(v, D, S, T, s, e0, lane);
+                            chain_forward<Sh>(v, D, S, T, s, e0, lane);
 #pragma unroll
                             for (int q = 0; q < Sh::EPL; ++q) acc[q] = fmaf(cdv[i][q], v[q], acc[q]);
                         }
