@@ -18,43 +18,66 @@
 namespace {
 
 typedef double double4_t __attribute__((ext_vector_type(4)));
+typedef double double2_t __attribute__((ext_vector_type(2)));
 
 constexpr int TILE = 128;     // C tile edge per workgroup
 constexpr int KB = 16;        // rows of Z staged per step
 constexpr int GT = 256;       // threads
-constexpr int LDS_STRIDE = TILE + 2;   // doubles per staged row (pad: spreads the 4 k-rows over banks)
+// doubles per staged row: 128 + 16, i.e. consecutive rows start 32 banks apart, so the two
+// k-rows a half-wavefront reads in one ds_read_b64 never share a bank
+constexpr int LDS_STRIDE = TILE + 16;
+constexpr int SUPER = 8;      // tiles per edge of a super-tile (L2 locality unit)
+constexpr int NXCD = 8;       // workgroup ids go round-robin over the 8 XCDs
 
-// map a linear tile id to (ti, tj) with ti <= tj, walking row by row over the upper triangle
-__device__ __forceinline__ void upper_tile(int t, int nt, int& ti, int& tj) {
-    // row ti starts at offset ti*nt - ti(ti-1)/2
-    const float b = (float)(2 * nt + 1);
-    int r = (int)((b - sqrtf(fmaxf(b * b - 8.0f * (float)t, 0.0f))) * 0.5f);
-    if (r < 0) r = 0;
-    if (r > nt - 1) r = nt - 1;
-    while (r > 0 && r * nt - (r * (r - 1)) / 2 > t) --r;
-    while (r + 1 < nt && (r + 1) * nt - ((r + 1) * r) / 2 <= t) ++r;
-    ti = r;
-    tj = r + (t - (r * nt - (r * (r - 1)) / 2));
+// Workgroup id -> C tile.  Hardware deals consecutive workgroup ids to the 8 XCDs in turn
+// and every XCD has its own L2.  The tiles are grouped in super-tiles of 8x8; super-tile
+// number g (row-major over the super-tile grid, upper triangle only in the symmetric mode)
+// goes to XCD g%8, and the k-th workgroup of an XCD works on tile k%64 of that XCD's
+// (k/64)-th super-tile.  So the ~64 tiles an XCD runs at a time share 16 panels of Z, and
+// every XCD gets the same number of super-tiles.
+template <bool SYM>
+__device__ __forceinline__ void tile_of_block(unsigned b, int nti, int ntj, int& ti, int& tj) {
+    const unsigned xcd = b % NXCD, k = b / NXCD;
+    const unsigned g = (k / (SUPER * SUPER)) * NXCD + xcd;      // super-tile number
+    const unsigned in_super = k % (SUPER * SUPER);
+    const int sr_n = (nti + SUPER - 1) / SUPER, sc_n = (ntj + SUPER - 1) / SUPER;
+    int sr, sc;
+    if (SYM) {
+        // g-th super-tile of the upper triangle, rows of length sc_n - sr
+        const float bb = (float)(2 * sc_n + 1);
+        int r = (int)((bb - sqrtf(fmaxf(bb * bb - 8.0f * (float)g, 0.0f))) * 0.5f);
+        if (r < 0) r = 0;
+        if (r > sc_n - 1) r = sc_n - 1;
+        while (r > 0 && (unsigned)(r * sc_n - (r * (r - 1)) / 2) > g) --r;
+        while (r + 1 < sc_n && (unsigned)((r + 1) * sc_n - ((r + 1) * r) / 2) <= g) ++r;
+        sr = r;
+        sc = r + (int)(g - (unsigned)(r * sc_n - (r * (r - 1)) / 2));
+        if (sc >= sc_n) sr = sr_n;   // past the last super-tile
+    } else {
+        sr = (int)(g / sc_n);
+        sc = (int)(g % sc_n);
+    }
+    ti = sr * SUPER + (int)(in_super / SUPER);
+    tj = sc * SUPER + (int)(in_super % SUPER);
+    if (sr >= sr_n || ti >= nti || tj >= ntj) ti = tj = -1;
 }
 
-// SYM: C is [F,F], tiles ti<=tj, mirrored on store.  !SYM: rows f0..f1 of C, C_tile [f1-f0, F].
-template <bool SYM>
-__global__ __launch_bounds__(GT) void gram_kernel(const double* __restrict__ Z, int M, int F, int f0, int f1,
-                                                   int ntj, double* __restrict__ C) {
-    __shared__ double sA[KB][LDS_STRIDE];
-    __shared__ double sB[KB][LDS_STRIDE];
+// GUARD: some panel sticks out of the matrix (F or the row block not a multiple of 128, or
+// odd F): every element load is bounds-checked.  !GUARD: whole panels, 16-byte vector loads.
+template <bool SYM, bool GUARD>
+__global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ Z, int M, int F, int f0, int f1,
+                                                      int nti, int ntj, double* __restrict__ C) {
+    __shared__ __attribute__((aligned(16))) double sA[KB][LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) double sB[KB][LDS_STRIDE];
 
     int ti, tj;
-    if (SYM) {
-        upper_tile(blockIdx.x, ntj, ti, tj);
-    } else {
-        ti = blockIdx.x / ntj;
-        tj = blockIdx.x % ntj;
-    }
+    tile_of_block<SYM>(blockIdx.x, nti, ntj, ti, tj);
+    if (ti < 0 || (SYM && ti > tj)) return;
     const int i0 = f0 + ti * TILE;   // first feature of the A panel (rows of C)
     const int j0 = tj * TILE;        // first feature of the B panel (columns of C)
     const int ilim = SYM ? F : f1;
     const bool same = SYM && ti == tj;
+    constexpr bool interior = !GUARD;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -67,35 +90,52 @@ __global__ __launch_bounds__(GT) void gram_kernel(const double* __restrict__ Z, 
 #pragma unroll
         for (int q = 0; q < 4; ++q) acc[p][q] = (double4_t){0.0, 0.0, 0.0, 0.0};
 
-    // global -> register staging: KB x 128 doubles per panel = 2048; 256 threads x 8
-    // thread t loads row (t / 16) , columns (t % 16) * 8 .. +8   (KB = 16)
+    // global -> register staging: KB x 128 doubles per panel = 2048 = 256 threads x 8:
+    // thread t loads row t/16, columns (t%16)*8 .. +8
     const int lr = tid >> 4;
     const int lc = (tid & 15) * 8;
-    double ra[8], rb[8];
+    double2_t ra[4], rb[4];
+    bool loaded_rowok = true;
 
     auto load_panels = [&](int m0) {
         const int m = m0 + lr;
         const bool rowok = m < M;
-        const double* zr = Z + (size_t)m * F;
+        if constexpr (interior) {
+            // rows past the end are read from the last row (always valid memory) and zeroed
+            const double* zr = Z + (size_t)(rowok ? m : M - 1) * F;
+            const double2_t* pa = reinterpret_cast<const double2_t*>(zr + i0 + lc);
+            const double2_t* pb = reinterpret_cast<const double2_t*>(zr + j0 + lc);
+            // nothing may consume the loaded values before the MFMAs of the current panel
+            // have been issued, so the zeroing of tail rows happens at the LDS store
+            loaded_rowok = rowok;
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            const int ca = i0 + lc + q;
-            ra[q] = (rowok && ca < ilim) ? zr[ca] : 0.0;
-        }
-        if (!same) {
+            for (int q = 0; q < 4; ++q) ra[q] = pa[q];
+            if (!same) {
 #pragma unroll
-            for (int q = 0; q < 8; ++q) {
-                const int cb = j0 + lc + q;
-                rb[q] = (rowok && cb < F) ? zr[cb] : 0.0;
+                for (int q = 0; q < 4; ++q) rb[q] = pb[q];
+            }
+        } else {
+            const double* zr = Z + (size_t)m * F;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int ca = i0 + lc + 2 * q;
+                ra[q].x = (rowok && ca < ilim) ? zr[ca] : 0.0;
+                ra[q].y = (rowok && ca + 1 < ilim) ? zr[ca + 1] : 0.0;
+                const int cb = j0 + lc + 2 * q;
+                rb[q].x = (rowok && cb < F) ? zr[cb] : 0.0;
+                rb[q].y = (rowok && cb + 1 < F) ? zr[cb + 1] : 0.0;
             }
         }
     };
     auto store_panels = [&]() {
+        const double2_t zero = {0.0, 0.0};
+        double2_t* da = reinterpret_cast<double2_t*>(&sA[lr][lc]);
 #pragma unroll
-        for (int q = 0; q < 8; ++q) sA[lr][lc + q] = ra[q];
+        for (int q = 0; q < 4; ++q) da[q] = loaded_rowok ? ra[q] : zero;
         if (!same) {
+            double2_t* db = reinterpret_cast<double2_t*>(&sB[lr][lc]);
 #pragma unroll
-            for (int q = 0; q < 8; ++q) sB[lr][lc + q] = rb[q];
+            for (int q = 0; q < 4; ++q) db[q] = loaded_rowok ? rb[q] : zero;
         }
     };
 
@@ -136,12 +176,8 @@ __global__ __launch_bounds__(GT) void gram_kernel(const double* __restrict__ Z, 
                 if (gi < ilim && gj < F) {
                     const double v = acc[p][q][r];
                     if (SYM) {
-                        if (same) {
-                            C[(size_t)gi * F + gj] += v;      // the full diagonal tile was computed
-                        } else {
-                            C[(size_t)gi * F + gj] += v;
-                            C[(size_t)gj * F + gi] += v;
-                        }
+                        C[(size_t)gi * F + gj] += v;
+                        if (!same) C[(size_t)gj * F + gi] += v;   // mirror of an off-diagonal tile
                     } else {
                         C[(size_t)(gi - f0) * F + gj] += v;
                     }
@@ -201,14 +237,24 @@ static int gram_launch(const double* Z, const double* y, int M, int F, int f0, i
     QMLL_REQUIRE((y == nullptr) == (ZTy == nullptr), QMLL_ERR_INVALID, "%s: y and ZTy must both be given or both be NULL",
                  who);
     const int ntj = (F + TILE - 1) / TILE;
-    if (sym) {
-        const long long ntiles = (long long)ntj * (ntj + 1) / 2;
-        QMLL_REQUIRE(ntiles < 2147483647LL, QMLL_ERR_INVALID, "%s: too many tiles", who);
-        hipLaunchKernelGGL(gram_kernel<true>, dim3((unsigned)ntiles), dim3(GT), 0, stream, Z, M, F, 0, F, ntj, C);
-    } else {
-        const int nti = (f1 - f0 + TILE - 1) / TILE;
-        hipLaunchKernelGGL(gram_kernel<false>, dim3((unsigned)(nti * ntj)), dim3(GT), 0, stream, Z, M, F, f0, f1, ntj, C);
-    }
+    const int nti = sym ? ntj : (f1 - f0 + TILE - 1) / TILE;
+    // super-tiles are dealt round-robin to the XCDs; each owns SUPER*SUPER workgroup ids,
+    // and ids of tiles outside the matrix (or below the diagonal) exit at once
+    const long long sr = (nti + SUPER - 1) / SUPER, sc = (ntj + SUPER - 1) / SUPER;
+    long long nsuper = sym ? sc * (sc + 1) / 2 : sr * sc;
+    nsuper = (nsuper + NXCD - 1) / NXCD * NXCD;
+    const long long nblocks = nsuper * SUPER * SUPER;
+    QMLL_REQUIRE(nblocks < 2147483647LL, QMLL_ERR_INVALID, "%s: too many tiles", who);
+    const bool guard = (F % TILE) != 0 || ((f1 - f0) % TILE) != 0 || (f0 % 2) != 0;
+    const dim3 grid((unsigned)nblocks), block(GT);
+    if (sym && !guard)
+        hipLaunchKernelGGL((gram_kernel<true, false>), grid, block, 0, stream, Z, M, F, 0, F, nti, ntj, C);
+    else if (sym)
+        hipLaunchKernelGGL((gram_kernel<true, true>), grid, block, 0, stream, Z, M, F, 0, F, nti, ntj, C);
+    else if (!guard)
+        hipLaunchKernelGGL((gram_kernel<false, false>), grid, block, 0, stream, Z, M, F, f0, f1, nti, ntj, C);
+    else
+        hipLaunchKernelGGL((gram_kernel<false, true>), grid, block, 0, stream, Z, M, F, f0, f1, nti, ntj, C);
     QMLL_CHECK_LAUNCH(who);
     if (y) {
         dim3 grid((f1 - f0 + 255) / 256, (M + GV_ROWS - 1) / GV_ROWS);
