@@ -61,6 +61,29 @@ __device__ __forceinline__ float butterfly(float v, int lane) {
     return p + __int_as_float(__float_as_int(v) ^ sm);
 }
 
+// Radix-2 stage across lanes 16 or 32 apart for TWO registers at once, on the gfx950 lane
+// swap instructions: v_permlane16_swap exchanges the odd 16-lane rows of `a` with the even
+// rows of `b` (v_permlane32_swap: the upper half of `a` with the lower half of `b`), after
+// which partner values sit in the same lane of a and b; one add, one subtract, and the
+// same swap again puts sums and differences back in place.  No LDS crossbar round trip.
+template <int MASK>
+__device__ __forceinline__ void butterfly_pair(float& a, float& b) {
+    typedef unsigned uint2_t __attribute__((ext_vector_type(2)));
+    uint2_t r;
+    if constexpr (MASK == 16)
+        r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    else
+        r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    const float x = __uint_as_float(r[0]), y = __uint_as_float(r[1]);
+    const float sum = x + y, dif = x - y;
+    if constexpr (MASK == 16)
+        r = __builtin_amdgcn_permlane16_swap(__float_as_uint(sum), __float_as_uint(dif), false, false);
+    else
+        r = __builtin_amdgcn_permlane32_swap(__float_as_uint(sum), __float_as_uint(dif), false, false);
+    a = __uint_as_float(r[0]);
+    b = __uint_as_float(r[1]);
+}
+
 // unnormalised Walsh-Hadamard transform of the d = EPL*LANES values held by LANES lanes
 template <int EPL, int LANES>
 __device__ __forceinline__ void fwht_wave(float (&v)[EPL], int lane) {
@@ -82,9 +105,18 @@ __device__ __forceinline__ void fwht_wave(float (&v)[EPL], int lane) {
         if constexpr (LANES > 2) t = butterfly<2>(t, lane);
         if constexpr (LANES > 4) t = butterfly<4>(t, lane);
         if constexpr (LANES > 8) t = butterfly<8>(t, lane);
-        if constexpr (LANES > 16) t = butterfly<16>(t, lane);
-        if constexpr (LANES > 32) t = butterfly<32>(t, lane);
+        if constexpr (EPL == 1) {
+            if constexpr (LANES > 16) t = butterfly<16>(t, lane);
+            if constexpr (LANES > 32) t = butterfly<32>(t, lane);
+        }
         v[q] = t;
+    }
+    if constexpr (EPL >= 2) {
+#pragma unroll
+        for (int q = 0; q < EPL; q += 2) {
+            if constexpr (LANES > 16) butterfly_pair<16>(v[q], v[q + 1]);
+            if constexpr (LANES > 32) butterfly_pair<32>(v[q], v[q + 1]);
+        }
     }
 }
 
@@ -221,32 +253,70 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_fused_kernel(
 #pragma unroll
     for (int q = 0; q < Sh::EPL; ++q) acc[q] = 0.0f;
     float energy = 0.0f;
-    for (int s = wave * Sh::G + sub; s < S; s += SORF_WAVES * Sh::G) {
-        float v[Sh::EPL];
+    constexpr int STEP = SORF_WAVES * Sh::G;
+    if (T == 1) {
+        // one transform per stack (the usual case): the sign diagonal serves the forward and
+        // the adjoint pass, and the three per-feature vectors of the NEXT stack are fetched
+        // while this stack is being computed
+        int s = wave * Sh::G + sub;
+        float dv[Sh::EPL], bv[Sh::EPL], av[Sh::EPL];
+        if (s < S) {
+            load_vec<Sh::EPL>(dv, D + (size_t)s * Sh::d + e0);
+            load_vec<Sh::EPL>(bv, bias + (size_t)s * Sh::d + e0);
+            load_vec<Sh::EPL>(av, alpha + (size_t)s * Sh::d + e0);
+        }
+        for (; s < S; s += STEP) {
+            float dn[Sh::EPL], bn[Sh::EPL], an[Sh::EPL];
+            const int sn = s + STEP < S ? s + STEP : s;      // last round re-reads its own row
+            load_vec<Sh::EPL>(dn, D + (size_t)sn * Sh::d + e0);
+            load_vec<Sh::EPL>(bn, bias + (size_t)sn * Sh::d + e0);
+            load_vec<Sh::EPL>(an, alpha + (size_t)sn * Sh::d + e0);
+            float v[Sh::EPL];
 #pragma unroll
-        for (int q = 0; q < Sh::EPL; ++q) v[q] = xv[q];
-        chain_forward<Sh>(v, D, S, T, s, e0, lane);
-        const float* bp = bias + (size_t)s * Sh::d + e0;
-        const float* ap = alpha + (size_t)s * Sh::d + e0;
-        constexpr int CH = Sh::EPL >= 4 ? 4 : Sh::EPL;
+            for (int q = 0; q < Sh::EPL; ++q) v[q] = xv[q] * dv[q];
+            fwht_wave<Sh::EPL, Sh::LANES>(v, lane);
 #pragma unroll
-        for (int q0 = 0; q0 < Sh::EPL; q0 += CH) {
-            float bv[CH], av[CH];
-            load_vec<CH>(bv, bp + q0);
-            load_vec<CH>(av, ap + q0);
-#pragma unroll
-            for (int q = 0; q < CH; ++q) {
-                float sn, cs;
-                sincos_f32(fmaf(v[q0 + q], scale, bv[q]), &sn, &cs);
+            for (int q = 0; q < Sh::EPL; ++q) {
+                float sn_, cs;
+                sincos_f32(fmaf(v[q], scale, bv[q]), &sn_, &cs);
                 const float w = av[q] * normf;
                 energy = fmaf(w, cs, energy);
-                v[q0 + q] = -w * sn;                       // d E / d coefficient
+                v[q] = -w * sn_;                          // d E / d coefficient
+            }
+            if constexpr (WITH_GRAD) {
+                fwht_wave<Sh::EPL, Sh::LANES>(v, lane);
+#pragma unroll
+                for (int q = 0; q < Sh::EPL; ++q) acc[q] = fmaf(v[q], dv[q], acc[q]);
+            }
+#pragma unroll
+            for (int q = 0; q < Sh::EPL; ++q) {
+                dv[q] = dn[q];
+                bv[q] = bn[q];
+                av[q] = an[q];
             }
         }
-        if constexpr (WITH_GRAD) {
-            chain_adjoint<Sh>(v, D, S, T, s, e0, lane);
+    } else {
+        for (int s = wave * Sh::G + sub; s < S; s += STEP) {
+            float v[Sh::EPL];
 #pragma unroll
-            for (int q = 0; q < Sh::EPL; ++q) acc[q] += v[q];
+            for (int q = 0; q < Sh::EPL; ++q) v[q] = xv[q];
+            chain_forward<Sh>(v, D, S, T, s, e0, lane);
+            float bv[Sh::EPL], av[Sh::EPL];
+            load_vec<Sh::EPL>(bv, bias + (size_t)s * Sh::d + e0);
+            load_vec<Sh::EPL>(av, alpha + (size_t)s * Sh::d + e0);
+#pragma unroll
+            for (int q = 0; q < Sh::EPL; ++q) {
+                float sn_, cs;
+                sincos_f32(fmaf(v[q], scale, bv[q]), &sn_, &cs);
+                const float w = av[q] * normf;
+                energy = fmaf(w, cs, energy);
+                v[q] = -w * sn_;
+            }
+            if constexpr (WITH_GRAD) {
+                chain_adjoint<Sh>(v, D, S, T, s, e0, lane);
+#pragma unroll
+                for (int q = 0; q < Sh::EPL; ++q) acc[q] += v[q];
+            }
         }
     }
     energy = wave_sum(energy);
@@ -385,64 +455,114 @@ __global__ __launch_bounds__(SORF_THREADS) void derivative_features_seg_kernel(
 }
 
 // ---- elementwise feature kernels ----------------------------------------------------
-// Thread = feature column f, workgroup = (feature tile, atom chunk).  Within its chunk a
-// thread keeps a running sum while consecutive atoms belong to the same molecule and
-// flushes it with one atomic when the molecule changes: atoms arrive molecule-major, so
-// this is about one atomic per (molecule, feature) instead of one per (atom, feature).
+// Thread = V consecutive feature columns (V = 4: 16-byte loads/stores; V = 1 when F is not
+// a multiple of 4), workgroup = (atom chunk, feature tile).  The forward kernel keeps a
+// running sum while consecutive atoms belong to the same molecule and flushes it with one
+// atomic when the molecule changes: atoms arrive molecule-major, so this is about one
+// atomic per (molecule, feature) instead of one per (atom, feature).
 constexpr int CF_THREADS = 256;
 constexpr int CF_ATOMS = 32;
 
-template <typename OutT>
+template <int V>
+__device__ __forceinline__ void load_f(float (&v)[V], const float* p) {
+    load_vec<V>(v, p);
+}
+
+template <typename OutT, int V>
 __global__ __launch_bounds__(CF_THREADS) void cos_features_kernel(const float* __restrict__ coeffs,
                                                                    const float* __restrict__ bias,
                                                                    const int* __restrict__ mol_index, int A, int F,
                                                                    int nmol, float normf, OutT* __restrict__ Zf) {
-    const int f = blockIdx.y * CF_THREADS + threadIdx.x;
+    const int f = (blockIdx.y * CF_THREADS + threadIdx.x) * V;
     if (f >= F) return;
     const int a0 = blockIdx.x * CF_ATOMS;
     const int a1 = min(A, a0 + CF_ATOMS);
-    const float b = bias[f];
+    float b[V];
+    load_f<V>(b, bias + f);
     int cur = -1;
-    OutT run = 0;
+    OutT run[V];
+#pragma unroll
+    for (int q = 0; q < V; ++q) run[q] = 0;
     for (int a = a0; a < a1; ++a) {
         const int mol = mol_index[a];
         if (mol != cur) {
-            if (cur >= 0 && cur < nmol) unsafeAtomicAdd(&Zf[(size_t)cur * F + f], run);
+            if (cur >= 0 && cur < nmol) {
+#pragma unroll
+                for (int q = 0; q < V; ++q) unsafeAtomicAdd(&Zf[(size_t)cur * F + f + q], run[q]);
+            }
             cur = mol;
-            run = 0;
+#pragma unroll
+            for (int q = 0; q < V; ++q) run[q] = 0;
         }
-        float sn, cs;
-        sincos_f32(coeffs[(size_t)a * F + f] + b, &sn, &cs);
-        run += (OutT)(cs * normf);
+        float c[V];
+        load_f<V>(c, coeffs + (size_t)a * F + f);
+#pragma unroll
+        for (int q = 0; q < V; ++q) {
+            float sn, cs;
+            sincos_f32(c[q] + b[q], &sn, &cs);
+            run[q] += (OutT)(cs * normf);
+        }
     }
-    if (cur >= 0 && cur < nmol) unsafeAtomicAdd(&Zf[(size_t)cur * F + f], run);
+    if (cur >= 0 && cur < nmol) {
+#pragma unroll
+        for (int q = 0; q < V; ++q) unsafeAtomicAdd(&Zf[(size_t)cur * F + f + q], run[q]);
+    }
 }
 
+template <int V>
 __global__ __launch_bounds__(CF_THREADS) void cos_features_backward_kernel(const float* __restrict__ gZ,
                                                                             const float* __restrict__ coeffs,
                                                                             const float* __restrict__ bias,
-                                                                            const int* __restrict__ mol_index, int F,
-                                                                            int nmol, float normf,
+                                                                            const int* __restrict__ mol_index, int A,
+                                                                            int F, int nmol, float normf,
                                                                             float* __restrict__ gc) {
-    const int f = blockIdx.y * CF_THREADS + threadIdx.x;
+    const int f = (blockIdx.y * CF_THREADS + threadIdx.x) * V;
     if (f >= F) return;
-    const size_t a = blockIdx.x;
-    const int mol = mol_index[a];
-    float sn, cs;
-    sincos_f32(coeffs[a * F + f] + bias[f], &sn, &cs);
-    const float gz = (mol >= 0 && mol < nmol) ? gZ[(size_t)mol * F + f] : 0.0f;
-    gc[a * F + f] = gz * -sn * normf;
+    const int a0 = blockIdx.x * CF_ATOMS;
+    const int a1 = min(A, a0 + CF_ATOMS);
+    float b[V];
+    load_f<V>(b, bias + f);
+    for (int a = a0; a < a1; ++a) {
+        const int mol = mol_index[a];
+        float c[V], g[V], o[V];
+        load_f<V>(c, coeffs + (size_t)a * F + f);
+        if (mol >= 0 && mol < nmol) {
+            load_f<V>(g, gZ + (size_t)mol * F + f);
+        } else {
+#pragma unroll
+            for (int q = 0; q < V; ++q) g[q] = 0.0f;
+        }
+#pragma unroll
+        for (int q = 0; q < V; ++q) {
+            float sn, cs;
+            sincos_f32(c[q] + b[q], &sn, &cs);
+            o[q] = g[q] * -sn * normf;
+        }
+        store_vec<V>(o, gc + (size_t)a * F + f);
+    }
 }
 
+template <int V>
 __global__ __launch_bounds__(CF_THREADS) void sin_coeffs_kernel(const float* __restrict__ coeffs,
-                                                                 const float* __restrict__ bias, int F, float normf,
-                                                                 double* __restrict__ out) {
-    const int f = blockIdx.y * CF_THREADS + threadIdx.x;
+                                                                 const float* __restrict__ bias, int A, int F,
+                                                                 float normf, double* __restrict__ out) {
+    const int f = (blockIdx.y * CF_THREADS + threadIdx.x) * V;
     if (f >= F) return;
-    const size_t a = blockIdx.x;
-    float sn, cs;
-    sincos_f32(coeffs[a * F + f] + bias[f], &sn, &cs);
-    out[a * F + f] = (double)(sn * normf);
+    const int a0 = blockIdx.x * CF_ATOMS;
+    const int a1 = min(A, a0 + CF_ATOMS);
+    float b[V];
+    load_f<V>(b, bias + f);
+    for (int a = a0; a < a1; ++a) {
+        float c[V];
+        load_f<V>(c, coeffs + (size_t)a * F + f);
+        double* o = out + (size_t)a * F + f;
+#pragma unroll
+        for (int q = 0; q < V; ++q) {
+            float sn, cs;
+            sincos_f32(c[q] + b[q], &sn, &cs);
+            o[q] = (double)(sn * normf);
+        }
+    }
 }
 
 int check_sorf(const char* who, int A, int d, int S, int T) {
@@ -569,15 +689,24 @@ static int check_feat(const char* who, int A, int F, int nmol) {
     return QMLL_OK;
 }
 
+// grid for the elementwise kernels: x = atom chunks, y = feature tiles of 256*V columns
+static dim3 feat_grid(int A, int F, int V) {
+    return dim3((A + CF_ATOMS - 1) / CF_ATOMS, (F + CF_THREADS * V - 1) / (CF_THREADS * V));
+}
+
 extern "C" int qmll_cos_features_f32(const float* coeffs, const float* bias, const int* mol_index, int A, int F,
                                      int nmol, float* Zf, qmll_stream_t stream) {
     int rc = check_feat("qmll_cos_features_f32", A, F, nmol);
     if (rc) return rc;
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(coeffs && bias && mol_index && Zf, QMLL_ERR_INVALID, "qmll_cos_features_f32: null pointer");
-    dim3 grid((A + CF_ATOMS - 1) / CF_ATOMS, (F + CF_THREADS - 1) / CF_THREADS);
-    hipLaunchKernelGGL(cos_features_kernel<float>, grid, dim3(CF_THREADS), 0, (hipStream_t)stream, coeffs, bias,
-                       mol_index, A, F, nmol, sqrtf(2.0f / (float)F), Zf);
+    const float normf = sqrtf(2.0f / (float)F);
+    if (F % 4 == 0)
+        hipLaunchKernelGGL((cos_features_kernel<float, 4>), feat_grid(A, F, 4), dim3(CF_THREADS), 0,
+                           (hipStream_t)stream, coeffs, bias, mol_index, A, F, nmol, normf, Zf);
+    else
+        hipLaunchKernelGGL((cos_features_kernel<float, 1>), feat_grid(A, F, 1), dim3(CF_THREADS), 0,
+                           (hipStream_t)stream, coeffs, bias, mol_index, A, F, nmol, normf, Zf);
     QMLL_CHECK_LAUNCH("qmll_cos_features_f32");
     return QMLL_OK;
 }
@@ -588,9 +717,13 @@ extern "C" int qmll_cos_features_f64(const float* coeffs, const float* bias, con
     if (rc) return rc;
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(coeffs && bias && mol_index && Zf, QMLL_ERR_INVALID, "qmll_cos_features_f64: null pointer");
-    dim3 grid((A + CF_ATOMS - 1) / CF_ATOMS, (F + CF_THREADS - 1) / CF_THREADS);
-    hipLaunchKernelGGL(cos_features_kernel<double>, grid, dim3(CF_THREADS), 0, (hipStream_t)stream, coeffs, bias,
-                       mol_index, A, F, nmol, sqrtf(2.0f / (float)F), Zf);
+    const float normf = sqrtf(2.0f / (float)F);
+    if (F % 4 == 0)
+        hipLaunchKernelGGL((cos_features_kernel<double, 4>), feat_grid(A, F, 4), dim3(CF_THREADS), 0,
+                           (hipStream_t)stream, coeffs, bias, mol_index, A, F, nmol, normf, Zf);
+    else
+        hipLaunchKernelGGL((cos_features_kernel<double, 1>), feat_grid(A, F, 1), dim3(CF_THREADS), 0,
+                           (hipStream_t)stream, coeffs, bias, mol_index, A, F, nmol, normf, Zf);
     QMLL_CHECK_LAUNCH("qmll_cos_features_f64");
     return QMLL_OK;
 }
@@ -602,9 +735,13 @@ extern "C" int qmll_cos_features_backward(const float* gZ, const float* coeffs, 
     if (rc) return rc;
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(gZ && coeffs && bias && mol_index && gc, QMLL_ERR_INVALID, "qmll_cos_features_backward: null pointer");
-    dim3 grid(A, (F + CF_THREADS - 1) / CF_THREADS);
-    hipLaunchKernelGGL(cos_features_backward_kernel, grid, dim3(CF_THREADS), 0, (hipStream_t)stream, gZ, coeffs, bias,
-                       mol_index, F, nmol, sqrtf(2.0f / (float)F), gc);
+    const float normf = sqrtf(2.0f / (float)F);
+    if (F % 4 == 0)
+        hipLaunchKernelGGL(cos_features_backward_kernel<4>, feat_grid(A, F, 4), dim3(CF_THREADS), 0,
+                           (hipStream_t)stream, gZ, coeffs, bias, mol_index, A, F, nmol, normf, gc);
+    else
+        hipLaunchKernelGGL(cos_features_backward_kernel<1>, feat_grid(A, F, 1), dim3(CF_THREADS), 0,
+                           (hipStream_t)stream, gZ, coeffs, bias, mol_index, A, F, nmol, normf, gc);
     QMLL_CHECK_LAUNCH("qmll_cos_features_backward");
     return QMLL_OK;
 }
@@ -615,9 +752,13 @@ extern "C" int qmll_sin_coeffs_f64(const float* coeffs, const float* bias, int A
     if (rc) return rc;
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(coeffs && bias && out, QMLL_ERR_INVALID, "qmll_sin_coeffs_f64: null pointer");
-    dim3 grid(A, (F + CF_THREADS - 1) / CF_THREADS);
-    hipLaunchKernelGGL(sin_coeffs_kernel, grid, dim3(CF_THREADS), 0, (hipStream_t)stream, coeffs, bias, F,
-                       sqrtf(2.0f / (float)F), out);
+    const float normf = sqrtf(2.0f / (float)F);
+    if (F % 4 == 0)
+        hipLaunchKernelGGL(sin_coeffs_kernel<4>, feat_grid(A, F, 4), dim3(CF_THREADS), 0, (hipStream_t)stream, coeffs,
+                           bias, A, F, normf, out);
+    else
+        hipLaunchKernelGGL(sin_coeffs_kernel<1>, feat_grid(A, F, 1), dim3(CF_THREADS), 0, (hipStream_t)stream, coeffs,
+                           bias, A, F, normf, out);
     QMLL_CHECK_LAUNCH("qmll_sin_coeffs_f64");
     return QMLL_OK;
 }

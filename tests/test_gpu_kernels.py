@@ -224,15 +224,21 @@ def test_cos_features_forward_backward_sin(scale):
     close(ops.sin_coeffs(t32(c), t32(b), out), sorf.sin_coeffs(carg, zero_b), REL_REP, "sin coeffs")
 
 
-def test_cos_features_unsorted_molecule_index():
+@pytest.mark.parametrize("F", [64, 63, 1030])
+def test_cos_features_unsorted_molecule_index(F):
     from qml_lightning_amd import ops
     rng = np.random.default_rng(4)
-    A, F, nmol = 50, 64, 7
+    A, nmol = 50, 7
     c = rng.normal(size=(A, F)).astype(np.float32)
     b = rng.uniform(0, 2 * np.pi, F).astype(np.float32)
     idx = rng.integers(0, nmol, A).astype(np.int32)
     carg = (c + b[None, :]).astype(np.float32).astype(np.float64)
     close(ops.cos_features(t32(c), t32(b), nmol, ti32(idx)), sorf.cos_features(carg, np.zeros(F), idx, nmol), REL_REP)
+    g = rng.normal(size=(nmol, F)).astype(np.float32)
+    close(ops.cos_features_backward(t32(g), t32(c), t32(b), nmol, ti32(idx)),
+          sorf.cos_features_backward(g, carg, np.zeros(F), idx), REL_REP, "cos backward, odd sizes")
+    out = torch.empty(A, F, dtype=torch.float64, device=dev())
+    close(ops.sin_coeffs(t32(c), t32(b), out), sorf.sin_coeffs(carg, np.zeros(F)), REL_REP, "sin coeffs, odd sizes")
 
 
 @pytest.mark.parametrize("d,S,T", [(16, 3, 1), (128, 8, 1), (64, 4, 2), (256, 4, 1)])
