@@ -178,6 +178,21 @@ int qmll_sorf_energy_fused(const float* x, const float* D, const float* bias, co
                            const int* out_index, int A, int d, int S, int T, float normalisation,
                            float* e_atom, float* gx, qmll_stream_t stream);
 
+/* All elements in one launch (no counterpart in the reference, which loops over elements
+ * on the host and gathers each element's atoms with boolean masks,
+ * qml_lightning/models/hadamard_features.py:99-119).  x_all f32 [N, ne*d]: row = atom slot
+ * (molecule-major, padded slots included), one d-wide block per element type holding that
+ * slot's representation projected with the element's reductor; types i32 [N] (as from
+ * qmll_element_types, -1 = element not in the model); atom_slots i32 [A]: slots of the real
+ * atoms; D f32 [ne,T,S,d]; bias f32 [ne,S*d]; alpha f32 [S*d].
+ *   -> e_slots[slot] = energy contribution of the atom in that slot (only listed slots are
+ *      written; the caller zero-fills the rest)
+ *   -> gx_all f32 [N, ne*d]: block types[slot] of a listed slot = d e_slots[slot] / d x_all
+ *      (other blocks untouched: the caller zero-fills; NULL = energies only) */
+int qmll_sorf_energy_typed(const float* x_all, const int* types, const int* atom_slots, const float* D,
+                           const float* bias, const float* alpha, int A, int N, int ne, int d, int S, int T,
+                           float normalisation, float* e_slots, float* gx_all, qmll_stream_t stream);
+
 /* ---- RFF ------------------------------------------------------------------------- */
 
 /* Replaces rff_gpu.get_rff / compute_rff (qml_lightning/cuda/random_features.cpp:11-20,

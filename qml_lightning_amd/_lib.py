@@ -44,6 +44,7 @@ PROTOTYPES = {
     "qmll_sin_coeffs_f64": [P, P, c_int, c_int, P, P],
     "qmll_derivative_features": [P, c_double, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, P],
     "qmll_sorf_energy_fused": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_float, P, P, P],
+    "qmll_sorf_energy_typed": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, P, P, P],
     "qmll_rff_features": [P, P, P, P, c_int, c_int, c_int, c_int, P, P],
     "qmll_rff_derivative_features": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
     "qmll_gram_f64": [P, P, c_int, c_int, P, P, P],

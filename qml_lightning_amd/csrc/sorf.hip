@@ -236,11 +236,17 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_adjoint_kernel(const float*
 // accumulate; the four wavefronts of a workgroup split the stacks and meet in LDS.  (The
 // deep layout has fewer cross-lane stages but its 128-byte-strided per-lane loads of the
 // three per-feature arrays cost more than the butterflies save: measured 1.7x slower.)
+//
+// Two addressing modes.  Per element (types == NULL): x is [A,d], the weights belong to
+// one element, atom a writes e_atom[out_index ? out_index[a] : a] and gx[a,:].  Typed
+// (types != NULL): x is [N, ne*d] with one d-wide block per element type, out_index[a] is
+// the slot (row) of atom a, types[slot] picks the block and the element's D / bias, and
+// the gradient goes to the same block of gx [N, ne*d]; all elements run in one launch.
 template <int LOG2D, bool WITH_GRAD>
 __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_fused_kernel(
     const float* __restrict__ x, const float* __restrict__ D, const float* __restrict__ bias,
-    const float* __restrict__ alpha, const int* __restrict__ out_index, int S, int T, float scale, float normf,
-    float* __restrict__ e_atom, float* __restrict__ gx) {
+    const float* __restrict__ alpha, const int* __restrict__ out_index, const int* __restrict__ types, int ne,
+    int S, int T, float scale, float normf, float* __restrict__ e_atom, float* __restrict__ gx) {
     using Sh = Shape<LOG2D>;
     __shared__ float red[SORF_WAVES][Sh::d];
     __shared__ float ered[SORF_WAVES];
@@ -248,8 +254,20 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_fused_kernel(
     const int sub = lane / Sh::LANES, l = lane % Sh::LANES;
     const int e0 = l * Sh::EPL;
     const size_t a = blockIdx.x;
+    const size_t slot = out_index ? (size_t)out_index[a] : a;
+    size_t xoff = a * Sh::d;          // row of x / gx that belongs to this atom
+    if (types != nullptr) {
+        const int t = types[slot];
+        if (t < 0 || t >= ne) {        // element not in the model: contributes nothing
+            if (threadIdx.x == 0) e_atom[slot] = 0.0f;
+            return;
+        }
+        xoff = (slot * ne + t) * Sh::d;
+        D += (size_t)t * T * S * Sh::d;
+        bias += (size_t)t * S * Sh::d;
+    }
     float xv[Sh::EPL], acc[Sh::EPL];
-    load_vec<Sh::EPL>(xv, x + a * Sh::d + e0);
+    load_vec<Sh::EPL>(xv, x + xoff + e0);
 #pragma unroll
     for (int q = 0; q < Sh::EPL; ++q) acc[q] = 0.0f;
     float energy = 0.0f;
@@ -338,14 +356,14 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_fused_kernel(
         float t = 0.0f;
 #pragma unroll
         for (int w = 0; w < SORF_WAVES; ++w) t += ered[w];
-        e_atom[out_index ? out_index[a] : (int)a] = t;
+        e_atom[slot] = t;
     }
     if constexpr (WITH_GRAD) {
         for (int e = threadIdx.x; e < Sh::d; e += SORF_THREADS) {
             float t = 0.0f;
 #pragma unroll
             for (int w = 0; w < SORF_WAVES; ++w) t += red[w][e];
-            gx[a * Sh::d + e] = scale * t;
+            gx[xoff + e] = scale * t;
         }
     }
 }
@@ -461,7 +479,7 @@ __global__ __launch_bounds__(SORF_THREADS) void derivative_features_seg_kernel(
 // atomic when the molecule changes: atoms arrive molecule-major, so this is about one
 // atomic per (molecule, feature) instead of one per (atom, feature).
 constexpr int CF_THREADS = 256;
-constexpr int CF_ATOMS = 32;
+constexpr int CF_ATOMS = 16;
 
 template <int V>
 __device__ __forceinline__ void load_f(float (&v)[V], const float* p) {
@@ -483,7 +501,19 @@ __global__ __launch_bounds__(CF_THREADS) void cos_features_kernel(const float* _
     OutT run[V];
 #pragma unroll
     for (int q = 0; q < V; ++q) run[q] = 0;
+    // coefficients of the next two atoms are in flight while the current one is evaluated
+    float c0[V], c1[V];
+    load_f<V>(c0, coeffs + (size_t)a0 * F + f);
+    load_f<V>(c1, coeffs + (size_t)min(a0 + 1, a1 - 1) * F + f);
     for (int a = a0; a < a1; ++a) {
+        float c[V], c2[V];
+        load_f<V>(c2, coeffs + (size_t)min(a + 2, a1 - 1) * F + f);
+#pragma unroll
+        for (int q = 0; q < V; ++q) {
+            c[q] = c0[q];
+            c0[q] = c1[q];
+            c1[q] = c2[q];
+        }
         const int mol = mol_index[a];
         if (mol != cur) {
             if (cur >= 0 && cur < nmol) {
@@ -494,8 +524,6 @@ __global__ __launch_bounds__(CF_THREADS) void cos_features_kernel(const float* _
 #pragma unroll
             for (int q = 0; q < V; ++q) run[q] = 0;
         }
-        float c[V];
-        load_f<V>(c, coeffs + (size_t)a * F + f);
 #pragma unroll
         for (int q = 0; q < V; ++q) {
             float sn, cs;
@@ -627,6 +655,24 @@ extern "C" int qmll_sorf_adjoint(const float* g, const float* D, int A, int d, i
     return QMLL_OK;
 }
 
+static int launch_fused(const char* who, const float* x, const float* D, const float* bias, const float* alpha,
+                        const int* out_index, const int* types, int ne, int A, int d, int S, int T,
+                        float normalisation, float* e_atom, float* gx, hipStream_t stream) {
+    const float scale = normalisation * hnorm(d, T);
+    const float normf = sqrtf(2.0f / ((float)S * (float)d));
+#define CALL(L)                                                                                                  \
+    if (gx)                                                                                                      \
+        hipLaunchKernelGGL((sorf_energy_fused_kernel<L, true>), dim3(A), dim3(SORF_THREADS), 0, stream, x, D,    \
+                           bias, alpha, out_index, types, ne, S, T, scale, normf, e_atom, gx);                   \
+    else                                                                                                         \
+        hipLaunchKernelGGL((sorf_energy_fused_kernel<L, false>), dim3(A), dim3(SORF_THREADS), 0, stream, x, D,   \
+                           bias, alpha, out_index, types, ne, S, T, scale, normf, e_atom, gx)
+    DISPATCH_LOG2D(qmll_log2(d), CALL)
+#undef CALL
+    QMLL_CHECK_LAUNCH(who);
+    return QMLL_OK;
+}
+
 extern "C" int qmll_sorf_energy_fused(const float* x, const float* D, const float* bias, const float* alpha,
                                       const int* out_index, int A, int d, int S, int T, float normalisation,
                                       float* e_atom, float* gx, qmll_stream_t stream) {
@@ -634,19 +680,21 @@ extern "C" int qmll_sorf_energy_fused(const float* x, const float* D, const floa
     if (rc) return rc;
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(x && D && bias && alpha && e_atom, QMLL_ERR_INVALID, "qmll_sorf_energy_fused: null pointer");
-    const float scale = normalisation * hnorm(d, T);
-    const float normf = sqrtf(2.0f / ((float)S * (float)d));
-#define CALL(L)                                                                                                      \
-    if (gx)                                                                                                          \
-        hipLaunchKernelGGL((sorf_energy_fused_kernel<L, true>), dim3(A), dim3(SORF_THREADS), 0, (hipStream_t)stream, \
-                           x, D, bias, alpha, out_index, S, T, scale, normf, e_atom, gx);                            \
-    else                                                                                                             \
-        hipLaunchKernelGGL((sorf_energy_fused_kernel<L, false>), dim3(A), dim3(SORF_THREADS), 0, (hipStream_t)stream, \
-                           x, D, bias, alpha, out_index, S, T, scale, normf, e_atom, gx)
-    DISPATCH_LOG2D(qmll_log2(d), CALL)
-#undef CALL
-    QMLL_CHECK_LAUNCH("qmll_sorf_energy_fused");
-    return QMLL_OK;
+    return launch_fused("qmll_sorf_energy_fused", x, D, bias, alpha, out_index, nullptr, 1, A, d, S, T, normalisation,
+                        e_atom, gx, (hipStream_t)stream);
+}
+
+extern "C" int qmll_sorf_energy_typed(const float* x_all, const int* types, const int* atom_slots, const float* D,
+                                      const float* bias, const float* alpha, int A, int N, int ne, int d, int S, int T,
+                                      float normalisation, float* e_slots, float* gx_all, qmll_stream_t stream) {
+    int rc = check_sorf("qmll_sorf_energy_typed", A, d, S, T);
+    if (rc) return rc;
+    QMLL_REQUIRE(N >= 0 && ne > 0, QMLL_ERR_INVALID, "qmll_sorf_energy_typed: bad size N=%d ne=%d", N, ne);
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(x_all && types && atom_slots && D && bias && alpha && e_slots, QMLL_ERR_INVALID,
+                 "qmll_sorf_energy_typed: null pointer");
+    return launch_fused("qmll_sorf_energy_typed", x_all, D, bias, alpha, atom_slots, types, ne, A, d, S, T,
+                        normalisation, e_slots, gx_all, (hipStream_t)stream);
 }
 
 extern "C" int qmll_derivative_features(const double* cos_derivs, double normalisation, const int* mol_index,

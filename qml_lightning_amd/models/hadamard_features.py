@@ -49,6 +49,24 @@ def _register_fused_op():
         return gsub, None, None, None, None, None
 
     torch.library.register_autograd("qml_lightning_sorf::sorf_energy", backward, setup_context=setup, lib=lib)
+
+    # all elements in one launch: x_all [N, ne*d] holds, per atom slot, the representation
+    # projected with every element's reductor; the kernel picks the block of the atom's type
+    lib.define("sorf_energy_typed(Tensor x_all, Tensor types, Tensor atom_slots, Tensor Dmat, Tensor bias, "
+               "Tensor alpha, Tensor coeff_normalisation, Tensor ntransforms) -> (Tensor, Tensor)")
+
+    def impl_typed(x_all, types, atom_slots, Dmat, bias, alpha, cn, nt):
+        return ops.sorf_energy_typed(x_all, types, atom_slots, Dmat, bias, alpha, ops._scalar(cn), int(nt.item()))
+
+    lib.impl("sorf_energy_typed", impl_typed, "CompositeExplicitAutograd")
+
+    def backward_typed(ctx, g_e, g_gx):
+        (gx,) = ctx.saved_tensors
+        gx_all = gx * g_e[:, None] if g_e is not None else None
+        return gx_all, None, None, None, None, None, None, None
+
+    torch.library.register_autograd("qml_lightning_sorf::sorf_energy_typed", backward_typed, setup_context=setup,
+                                    lib=lib)
     ops._libs.append(lib)
 
 
@@ -133,19 +151,19 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         alpha = self.alpha.float()
 
         if self.fused:
+            # one GEMM projects every atom slot with every element's reductor ([N,R] x [R,ne*d]);
+            # one kernel then runs SORF + cos + energy for all atoms, each on the block of its
+            # own element: no per-element gathers, no host round trips for their sizes
             nslots = X.shape[0] * X.shape[1]
             flat_rep = torch_rep.view(nslots, torch_rep.shape[2])
-            e_slots = torch.zeros(nslots, device=X.device, dtype=torch.float32)
-            for e in self.elements:
-                element_idx = self.element2index[e]
-                idx = torch.where(Z.reshape(-1).int() == e.item())[0]
-                if idx.shape[0] == 0:
-                    continue
-                sub = project_representation(flat_rep.index_select(0, idx), self.reductors[element_idx])
-                e_atom, _ = torch.ops.qml_lightning_sorf.sorf_energy(sub, self.Dmat[element_idx],
-                                                                     self.bias[element_idx], alpha,
-                                                                     coeff_normalisation, self.ntransforms)
-                e_slots = e_slots.index_put((idx,), e_atom)
+            ne = self.reductors.shape[0]
+            Ucat = self.reductors.permute(1, 0, 2).reshape(self.reductors.shape[1], ne * self.npcas)
+            x_all = torch.matmul(flat_rep, Ucat)
+            types = torch.ops.qml_lightning_fchl.get_element_types(X, Z, atom_counts, self.species)
+            slots = molIDs * X.shape[1] + atomIDs
+            e_slots, _ = torch.ops.qml_lightning_sorf.sorf_energy_typed(x_all, types.view(-1), slots, self.Dmat,
+                                                                        self.bias, alpha, coeff_normalisation,
+                                                                        self.ntransforms)
             return e_slots.view(X.shape[0], X.shape[1]).sum(dim=1)
 
         Ztest = torch.zeros(X.shape[0], self.nfeatures(), device=X.device, dtype=torch.float32)

@@ -283,6 +283,26 @@ def sorf_energy_fused(x, D, bias, alpha, out_index, normalisation, ntransforms, 
     return gx
 
 
+def sorf_energy_typed(x_all, types, atom_slots, Dmat, bias, alpha, normalisation, ntransforms, with_grad=True):
+    """All elements in one launch.  x_all [N, ne*d], types int32 [N], atom_slots int32 [A],
+    Dmat [ne,T,S,d], bias [ne,F], alpha [F] -> (e_slots [N], gx_all [N, ne*d] or None)."""
+    x_all, Dmat, bias, alpha = _f32(x_all), _f32(Dmat), _f32(bias), _f32(alpha)
+    types, atom_slots = _i32(types).reshape(-1), _i32(atom_slots)
+    ne, Tn, S, d = Dmat.shape
+    N = x_all.shape[0]
+    if x_all.shape[1] != ne * d or types.shape[0] != N:
+        raise RuntimeError("sorf_energy_typed: x_all is %s, expected [%d, %d]" % (tuple(x_all.shape), types.shape[0], ne * d))
+    T = int(ntransforms)
+    if T != Tn:
+        raise RuntimeError("sorf_energy_typed: %d diagonals stored per stack, %d transforms asked for" % (Tn, T))
+    e_slots = torch.zeros(N, dtype=torch.float32, device=x_all.device)
+    gx = torch.zeros((N, ne * d), dtype=torch.float32, device=x_all.device) if with_grad else None
+    check(_lib.lib().qmll_sorf_energy_typed(_ptr(x_all), _ptr(types), _ptr(atom_slots), _ptr(Dmat), _ptr(bias),
+                                            _ptr(alpha), int(atom_slots.shape[0]), N, ne, d, S, T, float(normalisation),
+                                            _ptr(e_slots), _ptr(gx), _stream()), "qmll_sorf_energy_typed")
+    return e_slots, gx
+
+
 # ---------------------------------------------------------------------------------------
 # RFF / Gram
 # ---------------------------------------------------------------------------------------

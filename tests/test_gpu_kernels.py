@@ -285,6 +285,35 @@ def test_fused_energy_matches_two_op_chain(d, S, T):
     close(e2, e_ref, REL_EF, "fused energy only")
 
 
+def test_typed_fused_energy_matches_per_element_calls():
+    """All elements in one launch == one fused call per element (slots, padded rows, unknown types)."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(9)
+    ne, d, S, T, N = 3, 64, 6, 1, 40
+    F = S * d
+    x_all = rng.normal(size=(N, ne * d)).astype(np.float32)
+    types = rng.integers(-1, ne, N).astype(np.int32)              # -1: element not in the model
+    slots = np.sort(rng.choice(N, size=29, replace=False)).astype(np.int32)   # the rest are padding
+    D = np.where(rng.uniform(-1, 1, (ne, T, S, d)) > 0, 1.0, -1.0).astype(np.float32)
+    b = rng.uniform(0, 2 * np.pi, (ne, F)).astype(np.float32)
+    alpha = rng.normal(size=F).astype(np.float32)
+    norm = 3.0
+    e, gx = ops.sorf_energy_typed(t32(x_all), ti32(types), ti32(slots), t32(D), t32(b), t32(alpha), norm, T)
+    e_ref = np.zeros(N)
+    g_ref = np.zeros((N, ne * d))
+    for s_ in slots:
+        t_ = types[s_]
+        if t_ < 0:
+            continue
+        xs = x_all[s_, t_ * d:(t_ + 1) * d][None, :]
+        c = sorf.sorf_coefficients(xs, D[t_], norm).reshape(1, F)
+        e_ref[s_] = (np.sqrt(2.0 / F) * np.cos(c + b[t_]) * alpha).sum()
+        gc = -np.sqrt(2.0 / F) * np.sin(c + b[t_]) * alpha
+        g_ref[s_, t_ * d:(t_ + 1) * d] = sorf.sorf_adjoint(gc.reshape(1, S, d), D[t_], norm)[0]
+    close(e, e_ref, REL_EF, "typed energies")
+    close(gx, g_ref, REL_EF, "typed gradients")
+
+
 # ---------------------------------------------------------------------------------------
 @pytest.mark.parametrize("M,F", [(37, 24), (300, 128), (1000, 384), (513, 200)])
 def test_gram_matches_fp64_matmul(M, F):
