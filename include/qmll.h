@@ -203,10 +203,14 @@ int qmll_rff_features(const float* x, const double* W, const double* b, const in
 
 /* Replaces rff_gpu.get_rff_derivatives / compute_rff_derivatives (random_features.cpp:22-33,
  * kernel random_features_kernel.cu:43-94).  grad f32 [A,n,3,d] -> G f64 [nmol,n,3,F] +=
- * sqrt(2/F) sin(x.W+b)_f * (grad[a,j,c,:].W)_f. */
+ * sqrt(2/F) sin(x.W+b)_f * (grad[a,j,c,:].W)_f.
+ * The molecule of an atom is given as for qmll_derivative_features: mol_index i32 [A] (any
+ * order, fp64 atomics) or seg_offsets i32 [nmol+1] (atoms molecule-major); with seg_offsets
+ * and d in {64,128,256} the products run on the fp64 matrix cores, atomic-free.  One of
+ * the two may be NULL (mol_index only when that matrix-core route applies). */
 int qmll_rff_derivative_features(const float* x, const float* grad, const double* W, const double* b,
-                                 const int* mol_index, int A, int n, int d, int F, int nmol, double* G,
-                                 qmll_stream_t stream);
+                                 const int* mol_index, const int* seg_offsets, int A, int n, int d, int F,
+                                 int nmol, double* G, qmll_stream_t stream);
 
 /* ---- Gram ------------------------------------------------------------------------ */
 

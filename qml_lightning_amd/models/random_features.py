@@ -5,7 +5,8 @@ from typing import Optional
 import numpy as np
 import torch
 
-from ..cuda.rff_gpu import get_rff, get_rff_derivatives
+from .. import ops
+from ..cuda.rff_gpu import get_rff
 from ..representations.dimensionality_reduction import project_representation
 from .kernel import BaseKernel, _default_device
 
@@ -48,7 +49,8 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
         W, b = self.W[idx].double(), self.b[idx].double()
         get_rff(rep, W, b, indexes, feature_matrix)
         if derivative_matrix is not None and grad is not None:
-            get_rff_derivatives(rep, grad, W, b, indexes, derivative_matrix)
+            # the batch's atoms are molecule-major: atomic-free matrix-core kernel
+            ops.rff_derivative_features(rep, grad, W, b, indexes, derivative_matrix, molecule_major=True)
 
     def forward(self, X, Z, atomIDs, molIDs, atom_counts, cell: Optional[torch.Tensor] = None,
                 inv_cell: Optional[torch.Tensor] = None):

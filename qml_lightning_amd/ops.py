@@ -316,13 +316,20 @@ def rff_features(x, W, b, mol_index, Zf):
     return Zf
 
 
-def rff_derivative_features(x, grad, W, b, mol_index, G):
+def rff_derivative_features(x, grad, W, b, mol_index, G, molecule_major=False):
+    """molecule_major=True promises that mol_index is non-decreasing: the atomic-free
+    matrix-core kernel is used (for d in 64/128/256)."""
     x, grad, mol_index = _f32(x), _f32(grad), _i32(mol_index)
     W, b = W.double().contiguous(), b.double().contiguous()
     A, n, _, d = grad.shape
     F = W.shape[1]
-    check(_lib.lib().qmll_rff_derivative_features(_ptr(x), _ptr(grad), _ptr(W), _ptr(b), _ptr(mol_index), A, n, d, F,
-                                                  int(G.shape[0]), _ptr(G), _stream()), "qmll_rff_derivative_features")
+    nmol = int(G.shape[0])
+    seg = None
+    if molecule_major:
+        bounds = torch.arange(nmol + 1, dtype=torch.int32, device=x.device)
+        seg = torch.searchsorted(mol_index, bounds).to(torch.int32)
+    check(_lib.lib().qmll_rff_derivative_features(_ptr(x), _ptr(grad), _ptr(W), _ptr(b), _ptr(mol_index), _ptr(seg), A, n,
+                                                  d, F, nmol, _ptr(G), _stream()), "qmll_rff_derivative_features")
     return G
 
 

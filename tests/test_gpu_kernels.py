@@ -378,3 +378,23 @@ def test_rff_features_and_derivatives(d, F):
     ops.rff_derivative_features(t32(x), t32(grad), torch.tensor(W, device=dev()), torch.tensor(b, device=dev()),
                                 ti32(idx), G)
     close(G, sorf.rff_derivative_features(x, grad, W, b, idx, nmol), 1e-12, "rff derivative features")
+
+
+@pytest.mark.parametrize("d,F,n", [(64, 200, 6), (128, 704, 21), (128, 130, 29), (256, 64, 9), (16, 40, 6)])
+def test_rff_derivatives_molecule_major(d, F, n):
+    """Matrix-core route (segments instead of a molecule index); accumulates onto G;
+    molecule 2 is left without atoms; n = 29 needs two row groups; d = 16 falls back."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(d + F + n)
+    A, nmol = 23, 6
+    x = rng.normal(size=(A, d)).astype(np.float32)
+    grad = rng.normal(size=(A, n, 3, d)).astype(np.float32)
+    grad[1, 2] = 0.0
+    W = rng.normal(size=(d, F)) / 8.0
+    b = rng.uniform(0, 2 * np.pi, F)
+    idx = np.sort(rng.choice([0, 1, 3, 4, 5], A)).astype(np.int32)
+    G0 = rng.normal(size=(nmol, n, 3, F))
+    G = torch.tensor(G0, device=dev())
+    ops.rff_derivative_features(t32(x), t32(grad), torch.tensor(W, device=dev()), torch.tensor(b, device=dev()),
+                                ti32(idx), G, molecule_major=True)
+    close(G, G0 + sorf.rff_derivative_features(x, grad, W, b, idx, nmol), 1e-12, "rff derivative features (segments)")
