@@ -56,6 +56,97 @@ def cpu_baseline(coords, charges, weights, nsample, cores):
     return n / dt, n, dt, out, chunks
 
 
+def other_configs(torch, dev):
+    """Short measurements of the remaining BASELINE configurations (1, 3, 4, 5) with the
+    same step definition; reported under "other_configs", never as `value`."""
+    from qml_lightning_amd.models.hadamard_features import HadamardFeaturesModel
+    from qml_lightning_amd.models.random_features import RandomFourrierFeaturesModel
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    from qml_lightning_amd.utils import synthetic
+
+    def sorf_model(species, npcas, nstacks, nbatch_train):
+        rep = FCHLCuda(species=np.array(species))
+        m = HadamardFeaturesModel(rep=rep, elements=np.array(species), ntransforms=1, sigma=SIGMA, llambda=1e-5,
+                                  npcas=npcas, nstacks=nstacks, nbatch_train=nbatch_train, nbatch_test=1 << 20)
+        red, D, bias, alpha = synthetic.model_weights(len(species), rep.get_repsize(), npcas, nstacks)
+        m.reductors, m.Dmat, m.bias = (torch.tensor(v, device=dev) for v in (red, D, bias))
+        m.alpha = torch.tensor(alpha, device=dev)
+        m.is_trained = True
+        return m
+
+    def predict_rate(model, coords, charges, forces, steps=5, warm=2):
+        data = model.format_data([c.astype(np.float32) for c in coords], charges)
+        X, Z = data['coordinates'], data['charges']
+        aid, mid, nat = data['atomIDs'], data['molIDs'], data['natom_counts']
+
+        def step():
+            if not forces:
+                with torch.no_grad():
+                    return model.forward(X, Z, aid, mid, nat)
+            Xg = X.detach().requires_grad_(True)
+            E = model.forward(Xg, Z, aid, mid, nat)
+            return torch.autograd.grad(-E.sum(), Xg)[0]
+        for _ in range(warm):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        return {"molecules": len(coords), "atoms": int(aid.shape[0]), "ms_per_step": dt * 1e3,
+                "molecules_per_s": len(coords) / dt, "outputs": "energies + forces" if forces else "energies"}
+
+    def ztz_seconds(model, coords, charges, natoms):
+        rng = np.random.default_rng(14)
+        nm = len(coords)
+        Et = rng.normal(size=nm)
+        Ft = [rng.normal(size=(natoms, 3)) for _ in range(nm)]
+        model.build_Z_components(coords[:16], charges[:16], E=Et[:16], F=Ft[:16], print_info=False)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ZTZ, ZTy = model.build_Z_components(coords, charges, E=Et, F=Ft, print_info=False)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        M, Fn = nm * (1 + 3 * natoms), model.nfeatures()
+        return {"ztz_seconds": dt, "ztz_molecules": nm, "ztz_rows": M, "ztz_features": Fn,
+                "ztz_TFLOPs_whole_build": (float(M) * Fn * (Fn + 1)) / dt / 1e12}
+
+    out = {}
+    # config 1: 100 noisy C6H6, npcas 64 x nstacks 8
+    coords, charges = synthetic.benzene_batch(100, seed=0)
+    out["config1_c6h6_100"] = predict_rate(sorf_model([1, 6], 64, 8, 64), coords, charges, True, steps=50, warm=10)
+    # config 3: 8192 ragged molecules (3..29 atoms, H C N O F), npcas 128 x nstacks 64, energies only
+    coords, charges = synthetic.ragged_batch(8192, seed=2)
+    out["config3_ragged_8192"] = predict_rate(sorf_model([1, 6, 7, 8, 9], 128, 64, 64), coords, charges, False)
+    # config 4: C12H12N2O (27 atoms), npcas 256 x nstacks 128 = 32768 features: fp64 Gram on 500, predict on 1548
+    coords, charges = synthetic.fixed_composition_batch(synthetic.C12H12N2O, 2048, seed=3, sigma=0.15)
+    m4 = sorf_model([1, 6, 7, 8], 256, 128, 250)
+    r4 = predict_rate(m4, coords[500:], charges[500:], True)
+    r4.update(ztz_seconds(m4, [c.astype(np.float32) for c in coords[:500]], charges[:500], 27))
+    out["config4_c12h12n2o"] = r4
+    del m4
+    torch.cuda.empty_cache()
+    # config 5: random Fourier features, 32768 features, projected dimension 128, C9H8O4 batch;
+    # W = N(0,1)/(2 sigma^2) as the reference samples it; SORF at the same feature count beside it
+    coords, charges = synthetic.fixed_composition_batch(synthetic.ASPIRIN, NMOL_PREDICT, seed=1)
+    np.random.seed(15)
+    rep = FCHLCuda(species=np.array(SPECIES))
+    m5 = RandomFourrierFeaturesModel(rep=rep, elements=np.array(SPECIES), sigma=SIGMA, llambda=1e-5, npcas=128,
+                                     nstacks=256, nbatch_train=500, nbatch_test=1 << 20)
+    red, _, _, alpha = synthetic.model_weights(len(SPECIES), rep.get_repsize(), 128, 256)
+    m5.reductors = torch.tensor(red, device=dev)
+    m5.alpha = torch.tensor(alpha, device=dev)
+    m5.is_trained = True
+    r5 = predict_rate(m5, coords, charges, True)
+    r5.update(ztz_seconds(m5, [c.astype(np.float32) for c in coords[:NMOL_TRAIN]], charges[:NMOL_TRAIN], 21))
+    out["config5_rff_32768"] = r5
+    del m5
+    torch.cuda.empty_cache()
+    out["config5_sorf_32768"] = predict_rate(sorf_model(SPECIES, 128, 256, 500), coords, charges, True)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -64,6 +155,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-train", action="store_true", help="skip the Z^T Z build measurement")
     ap.add_argument("--cpu-sample", type=int, default=1024)
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the short measurements of BASELINE configs 1, 3, 4 and 5")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a plain 1 GiB read + 1 GiB write elementwise kernel (reference point for "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -265,6 +358,16 @@ def main():
         "kernels": kernels,
     }
     out.update(train)
+    if "gram_f64" in kernels:
+        g = kernels["gram_f64"]
+        out["roofline_ztz"] = {"kernel": "gram_f64", "bound": "mfma", "achieved": g["TFLOPs"], "peak": FP64_PEAK_TFLOPS,
+                               "unit": "TFLOP/s", "frac": g["frac"], "traffic": g.get("traffic_bytes")}
+    if not args.no_other_configs:
+        torch.cuda.empty_cache()
+        try:
+            out["other_configs"] = other_configs(torch, dev)
+        except Exception as exc:   # the headline line must survive a failure here
+            out["other_configs"] = {"error": repr(exc)}
 
     if cpu is not None:
         rate, nsamp, secs, res, chunks, cores = cpu

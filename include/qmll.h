@@ -20,6 +20,8 @@
 #ifndef QMLL_H
 #define QMLL_H
 
+#include <stddef.h>
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -192,6 +194,47 @@ int qmll_sorf_energy_fused(const float* x, const float* D, const float* bias, co
 int qmll_sorf_energy_typed(const float* x_all, const int* types, const int* atom_slots, const float* D,
                            const float* bias, const float* alpha, int A, int N, int ne, int d, int S, int T,
                            float normalisation, float* e_slots, float* gx_all, qmll_stream_t stream);
+
+/* ---- element-sorted projection ---------------------------------------------------- */
+/* The three entry points below replace, for all elements of a batch at once, the
+ * per-element loop `sub = rep[Z == e]; sub = matmul(sub, reductors[e])` of
+ * qml_lightning/models/hadamard_features.py:99-108 (projection:
+ * qml_lightning/representations/dimensionality_reduction.py:47-72) and its autograd
+ * transpose; the fused energy kernel then consumes the compact, element-sorted rows. */
+
+/* Stable counting sort of the real atoms by element type.  types i32 [N] per atom slot (as
+ * from qmll_element_types), slots i32 [A] = slot of each real atom.
+ *   -> sorted_slots i32 [A]: slots ordered by type (original order kept within a type);
+ *      atoms whose type is outside [0,ne) are left out and the tail is filled with 0
+ *   -> type_offsets i32 [ne+1]: atoms of type t are sorted_slots[type_offsets[t] ..
+ *      type_offsets[t+1])
+ * workspace: device memory of at least qmll_sort_by_type_workspace(A, ne) bytes. ne <= 32. */
+size_t qmll_sort_by_type_workspace(int A, int ne);
+int qmll_sort_by_type(const int* types, const int* slots, int A, int ne, void* workspace, size_t workspace_bytes,
+                      int* sorted_slots, int* type_offsets, qmll_stream_t stream);
+
+/* x f32 [A,d]: row a = rep[sorted_slots[a], :] . reductors[type of a]  (rep f32 [N,R],
+ * reductors f32 [ne,R,d]); rows at and beyond type_offsets[ne] are not written. */
+int qmll_project_typed(const float* rep, const int* sorted_slots, const int* type_offsets, const float* reductors,
+                       int A, int ne, int R, int d, float* x, qmll_stream_t stream);
+
+/* Transpose of qmll_project_typed: g_rep[sorted_slots[a], :] = gx[a, :] . reductors[type]^T
+ * (g_rep f32 [N,R]).  Rows of slots that are not in the sorted list are not written, except
+ * that with types != NULL (i32 [N]) the rows of slots whose type is outside [0,ne) are set
+ * to zero. */
+int qmll_project_typed_backward(const float* gx, const int* sorted_slots, const int* type_offsets,
+                                const float* reductors, const int* types, int A, int N, int ne, int R, int d,
+                                float* g_rep, qmll_stream_t stream);
+
+/* qmll_sorf_energy_typed on compact element-sorted rows: x f32 [A,d] as written by
+ * qmll_project_typed, D f32 [ne,T,S,d], bias f32 [ne,S*d], alpha f32 [S*d].
+ *   -> e_slots[sorted_slots[a]] = energy contribution of atom a (a < type_offsets[ne];
+ *      the caller zero-fills the rest)
+ *   -> gx f32 [A,d] = d e / d x  (rows beyond type_offsets[ne] set to zero; NULL = energies
+ *      only) */
+int qmll_sorf_energy_sorted(const float* x, const int* type_offsets, const int* sorted_slots, const float* D,
+                            const float* bias, const float* alpha, int A, int ne, int d, int S, int T,
+                            float normalisation, float* e_slots, float* gx, qmll_stream_t stream);
 
 /* ---- RFF ------------------------------------------------------------------------- */
 

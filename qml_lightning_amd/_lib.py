@@ -5,7 +5,7 @@ raises; there is no CPU or eager fallback.
 """
 import ctypes
 import os
-from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_void_p
+from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_size_t, c_void_p
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("QML_LIGHTNING_AMD_LIB", os.path.join(HERE, "libqmll.so"))
@@ -45,13 +45,18 @@ PROTOTYPES = {
     "qmll_derivative_features": [P, c_double, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, P],
     "qmll_sorf_energy_fused": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_float, P, P, P],
     "qmll_sorf_energy_typed": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, P, P, P],
+    "qmll_sort_by_type_workspace": [c_int, c_int],
+    "qmll_sort_by_type": [P, P, c_int, c_int, P, c_size_t, P, P, P],
+    "qmll_project_typed": [P, P, P, P, c_int, c_int, c_int, c_int, P, P],
+    "qmll_project_typed_backward": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
+    "qmll_sorf_energy_sorted": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_float, P, P, P],
     "qmll_rff_features": [P, P, P, P, c_int, c_int, c_int, c_int, P, P],
     "qmll_rff_derivative_features": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
     "qmll_gram_f64": [P, P, c_int, c_int, P, P, P],
     "qmll_gram_tile_f64": [P, P, c_int, c_int, c_int, c_int, P, P, P],
     "qmll_matmul_and_reduce": [P, P, c_int, c_int, c_int, P, P],
 }
-_RESTYPES = {"qmll_last_error": c_char_p}
+_RESTYPES = {"qmll_last_error": c_char_p, "qmll_sort_by_type_workspace": c_size_t}
 
 _lib = None
 

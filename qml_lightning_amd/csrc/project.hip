@@ -1,0 +1,356 @@
+// Per-element projection of the representation on the fp32 matrix cores of gfx950, and
+// the element sort that feeds it.  Replaces, for the whole batch at once, the per-element
+// boolean-mask gather + torch.matmul(rep, reductor) of
+// qml_lightning/representations/dimensionality_reduction.py:47-72 as it is called from
+// qml_lightning/models/hadamard_features.py:99-108 (and its autograd transpose).
+//
+// Atoms are first ordered by element type (stable counting sort, two small kernels), so a
+// tile of 128 consecutive atoms shares one reductor.  typed_gemm_kernel then computes
+//     C[row, :] = A[row, :] . B_type      (B row-major [K,N])            forward,  or
+//     C[row, :] = A[row, :] . B_type^T    (B row-major [N,K])            backward
+// with v_mfma_f32_32x32x2f32; rows of A can be gathered and rows of C scattered through the
+// sorted slot list, so neither the gathered representation nor a zero-padded
+// [slots, elements*d] intermediate is ever materialised.  Only real atoms of known
+// elements are touched: no work is spent on padding or on the other elements' reductors.
+#include "qmll_common.h"
+
+namespace {
+
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+constexpr int MAXNE = 32;     // element types the sort supports
+constexpr int ST = 256;       // threads = atoms per workgroup of the sort
+
+// ---- sort by element type ---------------------------------------------------------------
+// counts[b*ne + e] = atoms of type e among atoms b*256 .. b*256+255
+__global__ __launch_bounds__(ST) void type_count_kernel(const int* __restrict__ types, const int* __restrict__ slots,
+                                                         int A, int ne, int* __restrict__ counts) {
+    __shared__ int wcnt[ST / 64][MAXNE];
+    const int a = blockIdx.x * ST + threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = a < A ? types[slots[a]] : -1;
+    for (int e = 0; e < ne; ++e) {
+        const unsigned long long m = __ballot(t == e);
+        if (lane == 0) wcnt[wave][e] = __popcll(m);
+    }
+    __syncthreads();
+    if (threadIdx.x < ne) {
+        int s = 0;
+#pragma unroll
+        for (int w = 0; w < ST / 64; ++w) s += wcnt[w][threadIdx.x];
+        counts[blockIdx.x * ne + threadIdx.x] = s;
+    }
+}
+
+// sorted[pos] = slot of the atom, pos = start of its type + atoms of that type before it
+// (in workgroups before this one, in wavefronts before this one, in lanes before this one)
+__global__ __launch_bounds__(ST) void type_place_kernel(const int* __restrict__ types, const int* __restrict__ slots,
+                                                         int A, int ne, const int* __restrict__ counts, int nb,
+                                                         int* __restrict__ sorted, int* __restrict__ offsets) {
+    __shared__ int before[MAXNE], total[MAXNE], start[MAXNE + 1];
+    __shared__ int wcnt[ST / 64][MAXNE];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int b = blockIdx.x;
+    if (threadIdx.x < MAXNE) before[threadIdx.x] = total[threadIdx.x] = 0;
+    __syncthreads();
+    for (int e = 0; e < ne; ++e) {
+        int sb = 0, sa = 0;
+        for (int q = threadIdx.x; q < nb; q += ST) {
+            const int c = counts[q * ne + e];
+            sa += c;
+            if (q < b) sb += c;
+        }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) {
+            sb += __shfl_xor(sb, m, 64);
+            sa += __shfl_xor(sa, m, 64);
+        }
+        if (lane == 0) {
+            atomicAdd(&before[e], sb);
+            atomicAdd(&total[e], sa);
+        }
+    }
+    const int a = b * ST + threadIdx.x;
+    const int slot = a < A ? slots[a] : 0;
+    const int t = a < A ? types[slot] : -1;
+    int rank = 0;
+    for (int e = 0; e < ne; ++e) {
+        const unsigned long long m = __ballot(t == e);
+        if (lane == 0) wcnt[wave][e] = __popcll(m);
+        if (t == e) rank = __popcll(m & ((1ull << lane) - 1ull));
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int s = 0;
+        for (int e = 0; e < ne; ++e) {
+            start[e] = s;
+            s += total[e];
+        }
+        start[ne] = s;
+    }
+    __syncthreads();
+    if (b == 0 && threadIdx.x <= ne) offsets[threadIdx.x] = start[threadIdx.x];
+    if (t >= 0 && t < ne) {
+        int pos = start[t] + before[t] + rank;
+        for (int w = 0; w < wave; ++w) pos += wcnt[w][t];
+        sorted[pos] = slot;
+    }
+    // entries past the last typed atom name a valid slot, so gathers through them stay in bounds
+    for (int i = start[ne] + a; i < A; i += nb * ST) sorted[i] = 0;
+}
+
+// ---- typed GEMM -------------------------------------------------------------------------
+constexpr int PT = 256;            // threads (4 wavefronts, each 32 rows x 64 columns)
+constexpr int PM = 128;            // rows per workgroup
+constexpr int PN = 64;             // columns per workgroup
+constexpr int PK = 32;             // contraction chunk staged in LDS
+constexpr int PKS = PK + 4;        // LDS row stride of k-contiguous tiles: 16-byte reads of 16
+                                   // consecutive rows fall into 16 distinct groups of 4 banks
+
+// which sorted rows a workgroup owns: tiles never straddle two types
+__device__ __forceinline__ bool tile_of_block(const int* __restrict__ offsets, int ne, int b, int& type, int& row0,
+                                              int& rows) {
+    for (int t = 0; t < ne; ++t) {
+        const int o0 = offsets[t], o1 = offsets[t + 1];
+        const int nt = (o1 - o0 + PM - 1) / PM;
+        if (b < nt) {
+            type = t;
+            row0 = o0 + b * PM;
+            rows = min(PM, o1 - row0);
+            return true;
+        }
+        b -= nt;
+    }
+    return false;
+}
+
+// BT = false: B_type is [K,N] row-major (ldb = row length); BT = true: B_type is [N,K].
+// VEC: all leading dimensions, K and N are multiples of 4 and the bases are 16-byte aligned.
+template <bool BT, bool VEC>
+__global__ __launch_bounds__(PT) void typed_gemm_kernel(const float* __restrict__ A, int lda,
+                                                         const int* __restrict__ a_rows, const float* __restrict__ Bm,
+                                                         size_t b_type_stride, int ldb, float* __restrict__ C, int ldc,
+                                                         const int* __restrict__ c_rows,
+                                                         const int* __restrict__ offsets, int ne, int K, int N) {
+    __shared__ __attribute__((aligned(16))) float sA[PM * PKS];
+    __shared__ __attribute__((aligned(16))) float sB[PN * PKS];   // BT: [PN][PKS]; else [PK][PN], rotated rows
+    int type, row0, rows;
+    if (!tile_of_block(offsets, ne, blockIdx.x, type, row0, rows)) return;
+    const int col0 = blockIdx.y * PN;
+    const float* Bt = Bm + (size_t)type * b_type_stride;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i = lane & 31, h = lane >> 5;
+
+    // staging: A tile 128 rows x 32 k = 1024 float4, thread -> rows tid/8 + 32v, k4 = tid%8
+    const int ar = tid >> 3, ak = (tid & 7) * 4;
+    const float* arow[4];
+    bool arow_ok[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const int r = ar + 32 * v;
+        arow_ok[v] = r < rows;
+        const int src = arow_ok[v] ? (a_rows ? a_rows[row0 + r] : row0 + r) : 0;
+        arow[v] = A + (size_t)src * lda;
+    }
+    // B tile: !BT 32 k x 64 n = 512 float4 -> k = tid/16 + 16v, n4 = tid%16
+    //          BT 64 n x 32 k = 512 float4 -> n = tid/8 + 32v,  k4 = tid%8
+    const int bk = BT ? (tid & 7) * 4 : (tid >> 4);
+    const int bn = BT ? (tid >> 3) : (tid & 15) * 4;
+
+    float4 ra[4], rb[2];
+    auto load4 = [&](const float* p, int first, int limit) -> float4 {
+        // elements first..first+3 of a row, zero beyond `limit`
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (VEC) {
+            if (first < limit) v = *reinterpret_cast<const float4*>(p + first);
+        } else {
+            if (first < limit) v.x = p[first];
+            if (first + 1 < limit) v.y = p[first + 1];
+            if (first + 2 < limit) v.z = p[first + 2];
+            if (first + 3 < limit) v.w = p[first + 3];
+        }
+        return v;
+    };
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+            ra[v] = arow_ok[v] ? load4(arow[v], k0 + ak, K) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+            if (BT) {
+                const int n = col0 + bn + 32 * v;
+                rb[v] = n < N ? load4(Bt + (size_t)n * ldb, k0 + bk, K) : make_float4(0.f, 0.f, 0.f, 0.f);
+            } else {
+                const int k = k0 + bk + 16 * v;
+                rb[v] = k < K ? load4(Bt + (size_t)k * ldb, col0 + bn, N) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) *reinterpret_cast<float4*>(&sA[(ar + 32 * v) * PKS + ak]) = ra[v];
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+            if (BT) {
+                *reinterpret_cast<float4*>(&sB[(bn + 32 * v) * PKS + bk]) = rb[v];
+            } else {
+                // rows 16..31 are rotated by 32 columns: the two wavefront halves, which read
+                // rows k and k+16 in one instruction, then use disjoint banks
+                const int k = bk + 16 * v;
+                *reinterpret_cast<float4*>(&sB[k * PN + ((bn + 32 * v) & 63)]) = rb[v];
+            }
+        }
+    };
+
+    float16_t acc[2];
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[jt][r] = 0.0f;
+
+    const int nchunks = (K + PK - 1) / PK;
+    fetch(0);
+    for (int c = 0; c < nchunks; ++c) {
+        __syncthreads();
+        stash();
+        __syncthreads();
+        if (c + 1 < nchunks) fetch((c + 1) * PK);
+        // MFMA step s contracts k = s (lanes 0-31) and k = 16 + s (lanes 32-63) of the chunk;
+        // the order of the contraction index is free, and this one lets a lane read its 16
+        // A values (and, transposed, B values) as four 16-byte LDS loads
+        float af[16];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float4 v = *reinterpret_cast<const float4*>(&sA[(32 * wave + i) * PKS + 16 * h + 4 * q]);
+            af[4 * q] = v.x; af[4 * q + 1] = v.y; af[4 * q + 2] = v.z; af[4 * q + 3] = v.w;
+        }
+        float bf[2][16];
+#pragma unroll
+        for (int jt = 0; jt < 2; ++jt) {
+            if (BT) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 v = *reinterpret_cast<const float4*>(&sB[(i + 32 * jt) * PKS + 16 * h + 4 * q]);
+                    bf[jt][4 * q] = v.x; bf[jt][4 * q + 1] = v.y; bf[jt][4 * q + 2] = v.z; bf[jt][4 * q + 3] = v.w;
+                }
+            } else {
+#pragma unroll
+                for (int s = 0; s < 16; ++s) bf[jt][s] = sB[(s + 16 * h) * PN + ((i + 32 * jt + 32 * h) & 63)];
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 16; ++s) {
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt)
+                acc[jt] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s], bf[jt][s], acc[jt], 0, 0, 0);
+        }
+    }
+
+    // accumulator register r of v_mfma_f32_32x32x2f32 holds row 8(r/4) + 4(lane/32) + r%4,
+    // column lane%32 (probed on gfx950)
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt) {
+        const int col = col0 + 32 * jt + i;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = 32 * wave + 8 * (r / 4) + 4 * h + (r % 4);
+            if (row < rows && col < N) {
+                const int dst = c_rows ? c_rows[row0 + row] : row0 + row;
+                C[(size_t)dst * ldc + col] = acc[jt][r];
+            }
+        }
+    }
+}
+
+// rows of real atoms whose element the model does not know get a zero gradient
+__global__ __launch_bounds__(256) void zero_untyped_rows_kernel(const int* __restrict__ types, int N, int ne, int R,
+                                                                float* __restrict__ out) {
+    const int slot = blockIdx.x;
+    const int t = types[slot];
+    if (t >= 0 && t < ne) return;
+    for (int c = threadIdx.x; c < R; c += 256) out[(size_t)slot * R + c] = 0.0f;
+}
+
+__global__ void zero_ints_kernel(int* __restrict__ p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+}  // namespace
+
+extern "C" size_t qmll_sort_by_type_workspace(int A, int ne) {
+    if (A <= 0 || ne <= 0) return 0;
+    return (size_t)((A + ST - 1) / ST) * (size_t)ne * sizeof(int);
+}
+
+extern "C" int qmll_sort_by_type(const int* types, const int* slots, int A, int ne, void* workspace,
+                                 size_t workspace_bytes, int* sorted_slots, int* type_offsets, qmll_stream_t stream) {
+    QMLL_REQUIRE(A >= 0 && ne > 0 && ne <= MAXNE, QMLL_ERR_INVALID, "qmll_sort_by_type: bad size A=%d ne=%d (at most %d types)",
+                 A, ne, MAXNE);
+    QMLL_REQUIRE(type_offsets, QMLL_ERR_INVALID, "qmll_sort_by_type: null pointer");
+    if (A == 0) {
+        hipLaunchKernelGGL(zero_ints_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, type_offsets, ne + 1);
+        QMLL_CHECK_LAUNCH("qmll_sort_by_type");
+        return QMLL_OK;
+    }
+    QMLL_REQUIRE(types && slots && sorted_slots && workspace, QMLL_ERR_INVALID, "qmll_sort_by_type: null pointer");
+    QMLL_REQUIRE(workspace_bytes >= qmll_sort_by_type_workspace(A, ne), QMLL_ERR_INVALID,
+                 "qmll_sort_by_type: workspace of %zu bytes, %zu needed", workspace_bytes,
+                 qmll_sort_by_type_workspace(A, ne));
+    const int nb = (A + ST - 1) / ST;
+    int* counts = static_cast<int*>(workspace);
+    hipLaunchKernelGGL(type_count_kernel, dim3(nb), dim3(ST), 0, (hipStream_t)stream, types, slots, A, ne, counts);
+    QMLL_CHECK_LAUNCH("qmll_sort_by_type");
+    hipLaunchKernelGGL(type_place_kernel, dim3(nb), dim3(ST), 0, (hipStream_t)stream, types, slots, A, ne, counts, nb,
+                       sorted_slots, type_offsets);
+    QMLL_CHECK_LAUNCH("qmll_sort_by_type");
+    return QMLL_OK;
+}
+
+extern "C" int qmll_project_typed(const float* rep, const int* sorted_slots, const int* type_offsets,
+                                  const float* reductors, int A, int ne, int R, int d, float* x,
+                                  qmll_stream_t stream) {
+    QMLL_REQUIRE(A >= 0 && ne > 0 && R > 0 && d > 0, QMLL_ERR_INVALID, "qmll_project_typed: bad size A=%d ne=%d R=%d d=%d", A,
+                 ne, R, d);
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(rep && sorted_slots && type_offsets && reductors && x, QMLL_ERR_INVALID,
+                 "qmll_project_typed: null pointer");
+    const dim3 grid((A + PM - 1) / PM + ne, (d + PN - 1) / PN);
+    const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(rep) && aligned16(reductors);
+    if (vec)
+        hipLaunchKernelGGL((typed_gemm_kernel<false, true>), grid, dim3(PT), 0, (hipStream_t)stream, rep, R, sorted_slots,
+                           reductors, (size_t)R * d, d, x, d, (const int*)nullptr, type_offsets, ne, R, d);
+    else
+        hipLaunchKernelGGL((typed_gemm_kernel<false, false>), grid, dim3(PT), 0, (hipStream_t)stream, rep, R,
+                           sorted_slots, reductors, (size_t)R * d, d, x, d, (const int*)nullptr, type_offsets, ne, R, d);
+    QMLL_CHECK_LAUNCH("qmll_project_typed");
+    return QMLL_OK;
+}
+
+extern "C" int qmll_project_typed_backward(const float* gx, const int* sorted_slots, const int* type_offsets,
+                                           const float* reductors, const int* types, int A, int N, int ne, int R,
+                                           int d, float* g_rep, qmll_stream_t stream) {
+    QMLL_REQUIRE(A >= 0 && N >= 0 && ne > 0 && R > 0 && d > 0, QMLL_ERR_INVALID,
+                 "qmll_project_typed_backward: bad size A=%d N=%d ne=%d R=%d d=%d", A, N, ne, R, d);
+    if (types && N > 0) {
+        QMLL_REQUIRE(g_rep, QMLL_ERR_INVALID, "qmll_project_typed_backward: null pointer");
+        hipLaunchKernelGGL(zero_untyped_rows_kernel, dim3(N), dim3(256), 0, (hipStream_t)stream, types, N, ne, R, g_rep);
+        QMLL_CHECK_LAUNCH("qmll_project_typed_backward");
+    }
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(gx && sorted_slots && type_offsets && reductors && g_rep, QMLL_ERR_INVALID,
+                 "qmll_project_typed_backward: null pointer");
+    const dim3 grid((A + PM - 1) / PM + ne, (R + PN - 1) / PN);
+    const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(gx) && aligned16(reductors);
+    if (vec)
+        hipLaunchKernelGGL((typed_gemm_kernel<true, true>), grid, dim3(PT), 0, (hipStream_t)stream, gx, d,
+                           (const int*)nullptr, reductors, (size_t)R * d, d, g_rep, R, sorted_slots, type_offsets, ne, d, R);
+    else
+        hipLaunchKernelGGL((typed_gemm_kernel<true, false>), grid, dim3(PT), 0, (hipStream_t)stream, gx, d,
+                           (const int*)nullptr, reductors, (size_t)R * d, d, g_rep, R, sorted_slots, type_offsets, ne, d, R);
+    QMLL_CHECK_LAUNCH("qmll_project_typed_backward");
+    return QMLL_OK;
+}

@@ -245,8 +245,9 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_adjoint_kernel(const float*
 template <int LOG2D, bool WITH_GRAD>
 __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_fused_kernel(
     const float* __restrict__ x, const float* __restrict__ D, const float* __restrict__ bias,
-    const float* __restrict__ alpha, const int* __restrict__ out_index, const int* __restrict__ types, int ne,
-    int S, int T, float scale, float normf, float* __restrict__ e_atom, float* __restrict__ gx) {
+    const float* __restrict__ alpha, const int* __restrict__ out_index, const int* __restrict__ types,
+    const int* __restrict__ type_offsets, int ne, int S, int T, float scale, float normf, float* __restrict__ e_atom,
+    float* __restrict__ gx) {
     using Sh = Shape<LOG2D>;
     __shared__ float red[SORF_WAVES][Sh::d];
     __shared__ float ered[SORF_WAVES];
@@ -256,7 +257,19 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_fused_kernel(
     const size_t a = blockIdx.x;
     const size_t slot = out_index ? (size_t)out_index[a] : a;
     size_t xoff = a * Sh::d;          // row of x / gx that belongs to this atom
-    if (types != nullptr) {
+    if (type_offsets != nullptr) {
+        // atoms sorted by element: x and gx are compact [A,d] in that order, atom a belongs to
+        // the type whose range [type_offsets[t], type_offsets[t+1]) holds it
+        if ((int)a >= type_offsets[ne]) {     // past the last atom of a known element
+            if constexpr (WITH_GRAD)
+                for (int e = threadIdx.x; e < Sh::d; e += SORF_THREADS) gx[xoff + e] = 0.0f;
+            return;
+        }
+        int t = 0;
+        while (t + 1 < ne && (int)a >= type_offsets[t + 1]) ++t;
+        D += (size_t)t * T * S * Sh::d;
+        bias += (size_t)t * S * Sh::d;
+    } else if (types != nullptr) {
         const int t = types[slot];
         if (t < 0 || t >= ne) {        // element not in the model: contributes nothing
             if (threadIdx.x == 0) e_atom[slot] = 0.0f;
@@ -656,17 +669,17 @@ extern "C" int qmll_sorf_adjoint(const float* g, const float* D, int A, int d, i
 }
 
 static int launch_fused(const char* who, const float* x, const float* D, const float* bias, const float* alpha,
-                        const int* out_index, const int* types, int ne, int A, int d, int S, int T,
-                        float normalisation, float* e_atom, float* gx, hipStream_t stream) {
+                        const int* out_index, const int* types, const int* type_offsets, int ne, int A, int d, int S,
+                        int T, float normalisation, float* e_atom, float* gx, hipStream_t stream) {
     const float scale = normalisation * hnorm(d, T);
     const float normf = sqrtf(2.0f / ((float)S * (float)d));
 #define CALL(L)                                                                                                  \
     if (gx)                                                                                                      \
         hipLaunchKernelGGL((sorf_energy_fused_kernel<L, true>), dim3(A), dim3(SORF_THREADS), 0, stream, x, D,    \
-                           bias, alpha, out_index, types, ne, S, T, scale, normf, e_atom, gx);                   \
+                           bias, alpha, out_index, types, type_offsets, ne, S, T, scale, normf, e_atom, gx);     \
     else                                                                                                         \
         hipLaunchKernelGGL((sorf_energy_fused_kernel<L, false>), dim3(A), dim3(SORF_THREADS), 0, stream, x, D,   \
-                           bias, alpha, out_index, types, ne, S, T, scale, normf, e_atom, gx)
+                           bias, alpha, out_index, types, type_offsets, ne, S, T, scale, normf, e_atom, gx)
     DISPATCH_LOG2D(qmll_log2(d), CALL)
 #undef CALL
     QMLL_CHECK_LAUNCH(who);
@@ -680,7 +693,7 @@ extern "C" int qmll_sorf_energy_fused(const float* x, const float* D, const floa
     if (rc) return rc;
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(x && D && bias && alpha && e_atom, QMLL_ERR_INVALID, "qmll_sorf_energy_fused: null pointer");
-    return launch_fused("qmll_sorf_energy_fused", x, D, bias, alpha, out_index, nullptr, 1, A, d, S, T, normalisation,
+    return launch_fused("qmll_sorf_energy_fused", x, D, bias, alpha, out_index, nullptr, nullptr, 1, A, d, S, T, normalisation,
                         e_atom, gx, (hipStream_t)stream);
 }
 
@@ -693,8 +706,21 @@ extern "C" int qmll_sorf_energy_typed(const float* x_all, const int* types, cons
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(x_all && types && atom_slots && D && bias && alpha && e_slots, QMLL_ERR_INVALID,
                  "qmll_sorf_energy_typed: null pointer");
-    return launch_fused("qmll_sorf_energy_typed", x_all, D, bias, alpha, atom_slots, types, ne, A, d, S, T,
+    return launch_fused("qmll_sorf_energy_typed", x_all, D, bias, alpha, atom_slots, types, nullptr, ne, A, d, S, T,
                         normalisation, e_slots, gx_all, (hipStream_t)stream);
+}
+
+extern "C" int qmll_sorf_energy_sorted(const float* x, const int* type_offsets, const int* sorted_slots, const float* D,
+                                       const float* bias, const float* alpha, int A, int ne, int d, int S, int T,
+                                       float normalisation, float* e_slots, float* gx, qmll_stream_t stream) {
+    int rc = check_sorf("qmll_sorf_energy_sorted", A, d, S, T);
+    if (rc) return rc;
+    QMLL_REQUIRE(ne > 0, QMLL_ERR_INVALID, "qmll_sorf_energy_sorted: bad size ne=%d", ne);
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(x && type_offsets && sorted_slots && D && bias && alpha && e_slots, QMLL_ERR_INVALID,
+                 "qmll_sorf_energy_sorted: null pointer");
+    return launch_fused("qmll_sorf_energy_sorted", x, D, bias, alpha, sorted_slots, nullptr, type_offsets, ne, A, d, S, T,
+                        normalisation, e_slots, gx, (hipStream_t)stream);
 }
 
 extern "C" int qmll_derivative_features(const double* cos_derivs, double normalisation, const int* mol_index,

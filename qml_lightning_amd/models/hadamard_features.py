@@ -53,20 +53,82 @@ def _register_fused_op():
     # all elements in one launch: x_all [N, ne*d] holds, per atom slot, the representation
     # projected with every element's reductor; the kernel picks the block of the atom's type
     lib.define("sorf_energy_typed(Tensor x_all, Tensor types, Tensor atom_slots, Tensor Dmat, Tensor bias, "
-               "Tensor alpha, Tensor coeff_normalisation, Tensor ntransforms) -> (Tensor, Tensor)")
+               "Tensor alpha, Tensor coeff_normalisation, Tensor ntransforms, bool with_grad) -> (Tensor, Tensor)")
 
-    def impl_typed(x_all, types, atom_slots, Dmat, bias, alpha, cn, nt):
-        return ops.sorf_energy_typed(x_all, types, atom_slots, Dmat, bias, alpha, ops._scalar(cn), int(nt.item()))
+    def impl_typed(x_all, types, atom_slots, Dmat, bias, alpha, cn, nt, with_grad):
+        e_slots, gx = ops.sorf_energy_typed(x_all, types, atom_slots, Dmat, bias, alpha, ops._scalar(cn),
+                                            int(nt.item()), with_grad=with_grad)
+        if gx is None:   # energies only: the adjoint transform is skipped
+            gx = torch.empty(0, dtype=torch.float32, device=x_all.device)
+        return e_slots, gx
 
     lib.impl("sorf_energy_typed", impl_typed, "CompositeExplicitAutograd")
 
     def backward_typed(ctx, g_e, g_gx):
         (gx,) = ctx.saved_tensors
-        gx_all = gx * g_e[:, None] if g_e is not None else None
-        return gx_all, None, None, None, None, None, None, None
+        if g_e is None:
+            return (None,) * 9
+        if gx.numel() == 0:
+            raise RuntimeError("sorf_energy_typed was called with with_grad=False but a gradient is requested")
+        return (gx * g_e[:, None],) + (None,) * 8
 
     torch.library.register_autograd("qml_lightning_sorf::sorf_energy_typed", backward_typed, setup_context=setup,
                                     lib=lib)
+
+    # element-sorted route: sort the atoms by type, project each with its own element's
+    # reductor on the matrix cores (compact [A,d]), run the fused kernel on those rows
+    lib.define("sort_by_type(Tensor types, Tensor slots, int ne) -> (Tensor, Tensor)")
+    lib.impl("sort_by_type", lambda types, slots, ne: ops.sort_by_type(types, slots, ne), "CompositeExplicitAutograd")
+    lib.define("project_typed(Tensor rep, Tensor sorted_slots, Tensor type_offsets, Tensor reductors, Tensor types) "
+               "-> Tensor")
+    lib.define("project_typed_backward(Tensor gx, Tensor sorted_slots, Tensor type_offsets, Tensor reductors, "
+               "Tensor types, int nslots) -> Tensor")
+    lib.impl("project_typed", lambda rep, ss, off, red, types: ops.project_typed(rep, ss, off, red),
+             "CompositeExplicitAutograd")
+    lib.impl("project_typed_backward",
+             lambda gx, ss, off, red, types, nslots: ops.project_typed_backward(gx, ss, off, red, types, nslots),
+             "CompositeExplicitAutograd")
+
+    def project_setup(ctx, inputs, output):
+        rep, ss, off, red, types = inputs
+        ctx.save_for_backward(ss, off, red, types)
+        ctx.nslots = rep.shape[0]
+
+    def project_backward(ctx, g):
+        ss, off, red, types = ctx.saved_tensors
+        g_rep = torch.ops.qml_lightning_sorf.project_typed_backward(g.contiguous(), ss, off, red, types, ctx.nslots)
+        return g_rep, None, None, None, None
+
+    torch.library.register_autograd("qml_lightning_sorf::project_typed", project_backward, setup_context=project_setup,
+                                    lib=lib)
+
+    lib.define("sorf_energy_sorted(Tensor x, Tensor type_offsets, Tensor sorted_slots, Tensor Dmat, Tensor bias, "
+               "Tensor alpha, Tensor coeff_normalisation, Tensor ntransforms, int nslots, bool with_grad) "
+               "-> (Tensor, Tensor)")
+
+    def impl_sorted(x, off, ss, Dmat, bias, alpha, cn, nt, nslots, with_grad):
+        e_slots, gx = ops.sorf_energy_sorted(x, off, ss, Dmat, bias, alpha, ops._scalar(cn), int(nt.item()), nslots,
+                                             with_grad=with_grad)
+        if gx is None:   # energies only: the adjoint transform is skipped
+            gx = torch.empty(0, dtype=torch.float32, device=x.device)
+        return e_slots, gx
+
+    lib.impl("sorf_energy_sorted", impl_sorted, "CompositeExplicitAutograd")
+
+    def setup_sorted(ctx, inputs, output):
+        ctx.save_for_backward(output[1], inputs[2])
+        ctx.set_materialize_grads(False)
+
+    def backward_sorted(ctx, g_e, g_gx):
+        gx, ss = ctx.saved_tensors
+        if g_e is None:
+            return (None,) * 10
+        if gx.numel() == 0 and ss.numel() != 0:
+            raise RuntimeError("sorf_energy_sorted was called with with_grad=False but a gradient is requested")
+        return (gx * g_e.index_select(0, ss.long())[:, None],) + (None,) * 9
+
+    torch.library.register_autograd("qml_lightning_sorf::sorf_energy_sorted", backward_sorted,
+                                    setup_context=setup_sorted, lib=lib)
     ops._libs.append(lib)
 
 
@@ -151,19 +213,19 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         alpha = self.alpha.float()
 
         if self.fused:
-            # one GEMM projects every atom slot with every element's reductor ([N,R] x [R,ne*d]);
-            # one kernel then runs SORF + cos + energy for all atoms, each on the block of its
-            # own element: no per-element gathers, no host round trips for their sizes
+            # the atoms are sorted by element on the device (no host round trip for sizes);
+            # one matrix-core kernel projects each with its own element's reductor into compact
+            # rows, and one kernel runs SORF + cos + energy (+ gradient) on those rows
             nslots = X.shape[0] * X.shape[1]
             flat_rep = torch_rep.view(nslots, torch_rep.shape[2])
-            ne = self.reductors.shape[0]
-            Ucat = self.reductors.permute(1, 0, 2).reshape(self.reductors.shape[1], ne * self.npcas)
-            x_all = torch.matmul(flat_rep, Ucat)
-            types = torch.ops.qml_lightning_fchl.get_element_types(X, Z, atom_counts, self.species)
+            types = torch.ops.qml_lightning_fchl.get_element_types(X, Z, atom_counts, self.species).view(-1)
             slots = molIDs * X.shape[1] + atomIDs
-            e_slots, _ = torch.ops.qml_lightning_sorf.sorf_energy_typed(x_all, types.view(-1), slots, self.Dmat,
-                                                                        self.bias, alpha, coeff_normalisation,
-                                                                        self.ntransforms)
+            sorted_slots, type_offsets = torch.ops.qml_lightning_sorf.sort_by_type(types, slots,
+                                                                                   self.reductors.shape[0])
+            x = torch.ops.qml_lightning_sorf.project_typed(flat_rep, sorted_slots, type_offsets, self.reductors, types)
+            e_slots, _ = torch.ops.qml_lightning_sorf.sorf_energy_sorted(x, type_offsets, sorted_slots, self.Dmat,
+                                                                         self.bias, alpha, coeff_normalisation,
+                                                                         self.ntransforms, nslots, x.requires_grad)
             return e_slots.view(X.shape[0], X.shape[1]).sum(dim=1)
 
         Ztest = torch.zeros(X.shape[0], self.nfeatures(), device=X.device, dtype=torch.float32)

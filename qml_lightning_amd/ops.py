@@ -304,6 +304,79 @@ def sorf_energy_typed(x_all, types, atom_slots, Dmat, bias, alpha, normalisation
 
 
 # ---------------------------------------------------------------------------------------
+# element-sorted projection + fused energy
+# ---------------------------------------------------------------------------------------
+def sort_by_type(types, slots, ne):
+    """Stable sort of the real atoms' slots by element type -> (sorted_slots [A], type_offsets [ne+1])."""
+    types, slots = _i32(types).reshape(-1), _i32(slots).reshape(-1)
+    A = int(slots.shape[0])
+    sorted_slots = torch.empty(A, dtype=torch.int32, device=types.device)
+    offsets = torch.empty(ne + 1, dtype=torch.int32, device=types.device)
+    nbytes = int(_lib.lib().qmll_sort_by_type_workspace(A, ne))
+    work = torch.empty(max(nbytes // 4, 1), dtype=torch.int32, device=types.device)
+    check(_lib.lib().qmll_sort_by_type(_ptr(types), _ptr(slots), A, int(ne), _ptr(work), nbytes, _ptr(sorted_slots),
+                                       _ptr(offsets), _stream()), "qmll_sort_by_type")
+    return sorted_slots, offsets
+
+
+def project_typed(rep, sorted_slots, type_offsets, reductors):
+    """x [A,d]: row a = rep[sorted_slots[a]] . reductors[type of a] (rep [N,R], reductors [ne,R,d])."""
+    rep, reductors = _f32(rep), _f32(reductors)
+    sorted_slots, type_offsets = _i32(sorted_slots), _i32(type_offsets)
+    ne, R, d = reductors.shape
+    if rep.dim() != 2 or rep.shape[1] != R or type_offsets.shape[0] != ne + 1:
+        raise RuntimeError("project_typed: rep %s, reductors %s, %d offsets do not fit together"
+                           % (tuple(rep.shape), tuple(reductors.shape), type_offsets.shape[0]))
+    A = int(sorted_slots.shape[0])
+    x = torch.empty((A, d), dtype=torch.float32, device=rep.device)
+    check(_lib.lib().qmll_project_typed(_ptr(rep), _ptr(sorted_slots), _ptr(type_offsets), _ptr(reductors), A, ne, R, d,
+                                        _ptr(x), _stream()), "qmll_project_typed")
+    return x
+
+
+def project_typed_backward(gx, sorted_slots, type_offsets, reductors, types, nslots):
+    """g_rep [nslots,R] with g_rep[sorted_slots[a]] = gx[a] . reductors[type]^T, zero elsewhere."""
+    gx, reductors = _f32(gx), _f32(reductors)
+    sorted_slots, type_offsets, types = _i32(sorted_slots), _i32(type_offsets), _i32(types).reshape(-1)
+    ne, R, d = reductors.shape
+    A, N = int(sorted_slots.shape[0]), int(nslots)
+    if gx.shape[0] != A or gx.shape[1] != d or types.shape[0] != N:
+        raise RuntimeError("project_typed_backward: gx %s for %d atoms, d=%d" % (tuple(gx.shape), A, d))
+    if A == N:
+        # every slot holds a real atom: the kernel writes every row of a known element and
+        # zeroes the rows of unknown ones
+        g_rep = torch.empty((N, R), dtype=torch.float32, device=gx.device)
+        tz = types
+    else:
+        g_rep = torch.zeros((N, R), dtype=torch.float32, device=gx.device)
+        tz = None
+    check(_lib.lib().qmll_project_typed_backward(_ptr(gx), _ptr(sorted_slots), _ptr(type_offsets), _ptr(reductors),
+                                                 _ptr(tz), A, N, ne, R, d, _ptr(g_rep), _stream()),
+          "qmll_project_typed_backward")
+    return g_rep
+
+
+def sorf_energy_sorted(x, type_offsets, sorted_slots, Dmat, bias, alpha, normalisation, ntransforms, nslots,
+                       with_grad=True):
+    """Fused SORF + cos + energy on element-sorted rows x [A,d] -> (e_slots [nslots], gx [A,d] or None)."""
+    x, Dmat, bias, alpha = _f32(x), _f32(Dmat), _f32(bias), _f32(alpha)
+    type_offsets, sorted_slots = _i32(type_offsets), _i32(sorted_slots)
+    ne, Tn, S, d = Dmat.shape
+    A = int(sorted_slots.shape[0])
+    if x.shape[0] != A or x.shape[1] != d or type_offsets.shape[0] != ne + 1:
+        raise RuntimeError("sorf_energy_sorted: x is %s, expected [%d, %d]" % (tuple(x.shape), A, d))
+    T = int(ntransforms)
+    if T != Tn:
+        raise RuntimeError("sorf_energy_sorted: %d diagonals stored per stack, %d transforms asked for" % (Tn, T))
+    e_slots = torch.zeros(int(nslots), dtype=torch.float32, device=x.device)
+    gx = torch.empty((A, d), dtype=torch.float32, device=x.device) if with_grad else None
+    check(_lib.lib().qmll_sorf_energy_sorted(_ptr(x), _ptr(type_offsets), _ptr(sorted_slots), _ptr(Dmat), _ptr(bias),
+                                             _ptr(alpha), A, ne, d, S, T, float(normalisation), _ptr(e_slots), _ptr(gx),
+                                             _stream()), "qmll_sorf_energy_sorted")
+    return e_slots, gx
+
+
+# ---------------------------------------------------------------------------------------
 # RFF / Gram
 # ---------------------------------------------------------------------------------------
 def rff_features(x, W, b, mol_index, Zf):

@@ -314,6 +314,89 @@ def test_typed_fused_energy_matches_per_element_calls():
     close(gx, g_ref, REL_EF, "typed gradients")
 
 
+@pytest.mark.parametrize("A,N,ne", [(0, 4, 3), (1, 1, 1), (255, 300, 2), (256, 256, 5), (1000, 1400, 4),
+                                    (70001, 70001, 3)])
+def test_sort_by_type_is_a_stable_counting_sort(A, N, ne):
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(A + ne)
+    types = rng.integers(-1, ne + 1, N).astype(np.int32)     # -1 and ne: elements the model does not know
+    slots = np.sort(rng.choice(N, size=A, replace=False)).astype(np.int32)
+    got_slots, got_off = ops.sort_by_type(ti32(types), ti32(slots), ne)
+    t_atoms = types[slots]
+    known = (t_atoms >= 0) & (t_atoms < ne)
+    order = np.argsort(t_atoms[known], kind="stable")
+    ref = slots[known][order]
+    off = np.concatenate([[0], np.cumsum(np.bincount(t_atoms[known], minlength=ne))])
+    assert np.array_equal(got_off.cpu().numpy(), off)
+    got = got_slots.cpu().numpy()
+    assert np.array_equal(got[:len(ref)], ref)
+    assert (got[len(ref):] == 0).all()
+
+
+@pytest.mark.parametrize("R,d,ne,N,A", [(312, 128, 3, 500, 500), (75, 64, 2, 90, 61), (720, 256, 5, 700, 523),
+                                        (10, 8, 1, 5, 3), (496, 256, 4, 130, 130)])
+def test_project_typed_forward_and_backward(R, d, ne, N, A):
+    """Element-sorted projection on the matrix cores against fp64 matmul, both directions:
+    gathered rows, tiles that end inside a type, R not a multiple of 4, unknown elements."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(R + d)
+    rep = rng.normal(size=(N, R)).astype(np.float32)
+    red = rng.normal(size=(ne, R, d)).astype(np.float32)
+    types = rng.integers(0, ne, N).astype(np.int32)
+    types[rng.choice(N, size=max(1, N // 20), replace=False)] = -1
+    slots = np.sort(rng.choice(N, size=A, replace=False)).astype(np.int32)
+    ss, off = ops.sort_by_type(ti32(types), ti32(slots), ne)
+    x = ops.project_typed(t32(rep), ss, off, t32(red))
+    ssn = ss.cpu().numpy()
+    total = int(off[-1].item())
+    x_ref = np.stack([rep[s_].astype(np.float64) @ red[types[s_]].astype(np.float64) for s_ in ssn[:total]]) \
+        if total else np.zeros((0, d))
+    close(x[:total], x_ref, REL_REP, "projection")
+    gx = rng.normal(size=(A, d)).astype(np.float32)
+    g = ops.project_typed_backward(t32(gx), ss, off, t32(red), ti32(types), N)
+    g_ref = np.zeros((N, R))
+    for a_, s_ in enumerate(ssn[:total]):
+        g_ref[s_] = gx[a_].astype(np.float64) @ red[types[s_]].astype(np.float64).T
+    close(g, g_ref, REL_REP, "projection transpose")
+    # unlisted and unknown rows are exactly zero
+    mask = np.ones(N, bool)
+    mask[ssn[:total]] = False
+    assert (g.cpu().numpy()[mask] == 0).all()
+
+
+def test_sorted_fused_energy_matches_per_atom_oracle():
+    """Element-sorted rows through the fused kernel: energies land in the atoms' slots, the
+    gradient stays in sorted order, rows past the last known atom give zero."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(19)
+    ne, d, S, T, N, A = 3, 64, 6, 1, 50, 37
+    F = S * d
+    types = rng.integers(-1, ne, N).astype(np.int32)
+    slots = np.sort(rng.choice(N, size=A, replace=False)).astype(np.int32)
+    ss, off = ops.sort_by_type(ti32(types), ti32(slots), ne)
+    ssn, total = ss.cpu().numpy(), int(off[-1].item())
+    x = rng.normal(size=(A, d)).astype(np.float32)
+    D = np.where(rng.uniform(-1, 1, (ne, T, S, d)) > 0, 1.0, -1.0).astype(np.float32)
+    b = rng.uniform(0, 2 * np.pi, (ne, F)).astype(np.float32)
+    alpha = rng.normal(size=F).astype(np.float32)
+    norm = 3.0
+    e, gx = ops.sorf_energy_sorted(t32(x), off, ss, t32(D), t32(b), t32(alpha), norm, T, N)
+    e_ref = np.zeros(N)
+    g_ref = np.zeros((A, d))
+    for a_ in range(total):
+        t_ = types[ssn[a_]]
+        c = sorf.sorf_coefficients(x[a_][None, :], D[t_], norm).reshape(1, F)
+        e_ref[ssn[a_]] = (np.sqrt(2.0 / F) * np.cos(c + b[t_]) * alpha).sum()
+        gc = -np.sqrt(2.0 / F) * np.sin(c + b[t_]) * alpha
+        g_ref[a_] = sorf.sorf_adjoint(gc.reshape(1, S, d), D[t_], norm)[0]
+    close(e, e_ref, REL_EF, "sorted energies")
+    close(gx, g_ref, REL_EF, "sorted gradients")
+    assert (gx[total:] == 0).all()
+    e2, g2 = ops.sorf_energy_sorted(t32(x), off, ss, t32(D), t32(b), t32(alpha), norm, T, N, with_grad=False)
+    assert g2 is None
+    close(e2, e_ref, REL_EF, "sorted energies only")
+
+
 # ---------------------------------------------------------------------------------------
 @pytest.mark.parametrize("M,F", [(37, 24), (300, 128), (1000, 384), (513, 200)])
 def test_gram_matches_fp64_matmul(M, F):
