@@ -255,6 +255,18 @@ int qmll_rff_derivative_features(const float* x, const float* grad, const double
                                  const int* mol_index, const int* seg_offsets, int A, int n, int d, int F,
                                  int nmol, double* G, qmll_stream_t stream);
 
+/* Fused RFF predict path on element-sorted rows (x f32 [A,d] from qmll_project_typed).
+ * Replaces, for all elements at once, the loop body of the reference's TorchScript forward
+ * (qml_lightning/models/random_features.py:88-102: matmul(sub, W[e]) + b, cos, index_add,
+ * matmul(Ztest, alpha)) and its autograd transpose; the [atoms,F] feature matrix is never
+ * written.  W f32 [ne,d,F], b f32 [ne,F], alpha f32 [F]; d is 64 or 128, F a multiple of 32.
+ *   -> e_slots[sorted_slots[a]] = sqrt(2/F) sum_f alpha_f cos(x_a . W_t[:,f] + b_t[f])
+ *      (only atoms a < type_offsets[ne]; the caller zero-fills the rest)
+ *   -> gx f32 [A,d] = d e / d x (rows beyond type_offsets[ne] zero; NULL = energies only) */
+int qmll_rff_energy_sorted(const float* x, const int* type_offsets, const int* sorted_slots, const float* W,
+                           const float* b, const float* alpha, int A, int ne, int d, int F, float* e_slots,
+                           float* gx, qmll_stream_t stream);
+
 /* ---- Gram ------------------------------------------------------------------------ */
 
 /* Replaces the Gram accumulation of BaseKernel.build_Z_components

@@ -52,6 +52,7 @@ PROTOTYPES = {
     "qmll_sorf_energy_sorted": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_float, P, P, P],
     "qmll_rff_features": [P, P, P, P, c_int, c_int, c_int, c_int, P, P],
     "qmll_rff_derivative_features": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
+    "qmll_rff_energy_sorted": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, P, P, P],
     "qmll_gram_f64": [P, P, c_int, c_int, P, P, P],
     "qmll_gram_tile_f64": [P, P, c_int, c_int, c_int, c_int, P, P, P],
     "qmll_matmul_and_reduce": [P, P, c_int, c_int, c_int, P, P],

@@ -129,6 +129,29 @@ def _register_fused_op():
 
     torch.library.register_autograd("qml_lightning_sorf::sorf_energy_sorted", backward_sorted,
                                     setup_context=setup_sorted, lib=lib)
+
+    # random Fourier features on the same element-sorted rows
+    lib.define("rff_energy_sorted(Tensor x, Tensor type_offsets, Tensor sorted_slots, Tensor W, Tensor b, "
+               "Tensor alpha, int nslots, bool with_grad) -> (Tensor, Tensor)")
+
+    def impl_rff(x, off, ss, W, b, alpha, nslots, with_grad):
+        e_slots, gx = ops.rff_energy_sorted(x, off, ss, W, b, alpha, nslots, with_grad=with_grad)
+        if gx is None:
+            gx = torch.empty(0, dtype=torch.float32, device=x.device)
+        return e_slots, gx
+
+    lib.impl("rff_energy_sorted", impl_rff, "CompositeExplicitAutograd")
+
+    def backward_rff(ctx, g_e, g_gx):
+        gx, ss = ctx.saved_tensors
+        if g_e is None:
+            return (None,) * 8
+        if gx.numel() == 0 and ss.numel() != 0:
+            raise RuntimeError("rff_energy_sorted was called with with_grad=False but a gradient is requested")
+        return (gx * g_e.index_select(0, ss.long())[:, None],) + (None,) * 7
+
+    torch.library.register_autograd("qml_lightning_sorf::rff_energy_sorted", backward_rff, setup_context=setup_sorted,
+                                    lib=lib)
     ops._libs.append(lib)
 
 

@@ -1,6 +1,6 @@
 """RandomFourrierFeaturesModel (qml_lightning/models/random_features.py:17-236): features
 sqrt(2/F) cos(x W + b) with W ~ N(0,1)/(2 sigma^2) per element."""
-from typing import Optional
+from typing import Final, Optional
 
 import numpy as np
 import torch
@@ -8,17 +8,24 @@ import torch
 from .. import ops
 from ..cuda.rff_gpu import get_rff
 from ..representations.dimensionality_reduction import project_representation
+from . import hadamard_features  # noqa: F401  (registers the fused operators)
 from .kernel import BaseKernel, _default_device
 
 
 class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
+    """`fused=True` (default where the kernel applies: npcas 64 or 128, a multiple of 32
+    features) runs forward() through one matrix-core kernel that never writes the
+    [atoms, nfeatures] matrix; `fused=False` is the reference's own operator sequence."""
+
+    fused: Final[bool]
 
     def __init__(self, rep=None, elements=np.array([1, 6, 7, 8]), sigma=2.0, llambda=1e-10,
-                 nstacks=8192, npcas=128, nbatch_train=64, nbatch_test=64):
+                 nstacks=8192, npcas=128, nbatch_train=64, nbatch_test=64, fused=True):
         torch.nn.Module.__init__(self)
         BaseKernel.__init__(self, rep, npcas, elements, sigma, llambda)
         self.device = _default_device()
         self.npcas = npcas
+        self.fused = bool(fused) and npcas in (64, 128) and (nstacks * npcas) % 32 == 0
         self.nbatch_train = nbatch_train
         self.nbatch_test = nbatch_test
         self._nfeatures = nstacks * self.npcas
@@ -63,6 +70,19 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
         assert X.is_cuda, "X tensor must reside on GPU"
         assert Z.is_cuda, "Z tensor must reside on GPU"
         torch_rep = self.rep.forward(X, Z, atomIDs, molIDs, atom_counts, cell, inv_cell)
+        if self.fused:
+            # atoms sorted by element on the device, projected with their own reductor into
+            # compact rows, then one kernel for x.W + b -> cos -> alpha contraction (+ gradient)
+            nslots = X.shape[0] * X.shape[1]
+            flat_rep = torch_rep.view(nslots, torch_rep.shape[2])
+            types = torch.ops.qml_lightning_fchl.get_element_types(X, Z, atom_counts, self.species).view(-1)
+            slots = molIDs * X.shape[1] + atomIDs
+            sorted_slots, type_offsets = torch.ops.qml_lightning_sorf.sort_by_type(types, slots,
+                                                                                   self.reductors.shape[0])
+            x = torch.ops.qml_lightning_sorf.project_typed(flat_rep, sorted_slots, type_offsets, self.reductors, types)
+            e_slots, _ = torch.ops.qml_lightning_sorf.rff_energy_sorted(x, type_offsets, sorted_slots, self.W, self.b,
+                                                                        self.alpha.float(), nslots, x.requires_grad)
+            return e_slots.view(X.shape[0], X.shape[1]).sum(dim=1)
         Ztest = torch.zeros(X.shape[0], self.nfeatures(), device=X.device, dtype=torch.float32)
         for e in self.elements:
             indexes = Z.int() == e.item()

@@ -406,6 +406,24 @@ def rff_derivative_features(x, grad, W, b, mol_index, G, molecule_major=False):
     return G
 
 
+def rff_energy_sorted(x, type_offsets, sorted_slots, W, b, alpha, nslots, with_grad=True):
+    """Fused RFF energy (and gradient) on element-sorted rows x [A,d]; W [ne,d,F], b [ne,F],
+    alpha [F] fp32 -> (e_slots [nslots], gx [A,d] or None)."""
+    x, W, b, alpha = _f32(x), _f32(W), _f32(b), _f32(alpha)
+    type_offsets, sorted_slots = _i32(type_offsets), _i32(sorted_slots)
+    ne, d, F = W.shape
+    A = int(sorted_slots.shape[0])
+    if x.shape[0] != A or x.shape[1] != d or type_offsets.shape[0] != ne + 1 or b.shape[0] != ne or b.shape[1] != F:
+        raise RuntimeError("rff_energy_sorted: x %s, W %s, b %s do not fit together"
+                           % (tuple(x.shape), tuple(W.shape), tuple(b.shape)))
+    e_slots = torch.zeros(int(nslots), dtype=torch.float32, device=x.device)
+    gx = torch.empty((A, d), dtype=torch.float32, device=x.device) if with_grad else None
+    check(_lib.lib().qmll_rff_energy_sorted(_ptr(x), _ptr(type_offsets), _ptr(sorted_slots), _ptr(W), _ptr(b),
+                                            _ptr(alpha), A, ne, d, F, _ptr(e_slots), _ptr(gx), _stream()),
+          "qmll_rff_energy_sorted")
+    return e_slots, gx
+
+
 def gram(Zrows, y, ZTZ, ZTy, f0=None, f1=None):
     """ZTZ += Z^T Z (or the row block f0:f1 of it), ZTy += Z^T y, fp64, in place."""
     if Zrows.dtype != torch.float64 or not Zrows.is_contiguous():

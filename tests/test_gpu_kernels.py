@@ -463,6 +463,38 @@ def test_rff_features_and_derivatives(d, F):
     close(G, sorf.rff_derivative_features(x, grad, W, b, idx, nmol), 1e-12, "rff derivative features")
 
 
+@pytest.mark.parametrize("d,F,ne,A", [(64, 64, 1, 5), (128, 192, 3, 300), (64, 640, 2, 131)])
+def test_rff_energy_sorted_kernel(d, F, ne, A):
+    """Fused x.W + b -> cos -> alpha contraction and its gradient on element-sorted rows."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(d + F)
+    N = A + 9
+    types = rng.integers(0, ne, N).astype(np.int32)
+    types[rng.choice(N, size=3, replace=False)] = -1
+    slots = np.sort(rng.choice(N, size=A, replace=False)).astype(np.int32)
+    ss, off = ops.sort_by_type(ti32(types), ti32(slots), ne)
+    ssn, total = ss.cpu().numpy(), int(off[-1].item())
+    x = rng.normal(size=(A, d)).astype(np.float32)
+    W = (rng.normal(size=(ne, d, F)) / 8.0).astype(np.float32)
+    b = rng.uniform(0, 2 * np.pi, (ne, F)).astype(np.float32)
+    alpha = rng.normal(size=F).astype(np.float32)
+    e, gx = ops.rff_energy_sorted(t32(x), off, ss, t32(W), t32(b), t32(alpha), N)
+    e_ref = np.zeros(N)
+    g_ref = np.zeros((A, d))
+    nf = np.sqrt(2.0 / F)
+    for a_ in range(total):
+        t_ = types[ssn[a_]]
+        arg = x[a_].astype(np.float64) @ W[t_].astype(np.float64) + b[t_]
+        e_ref[ssn[a_]] = nf * (alpha * np.cos(arg)).sum()
+        g_ref[a_] = -nf * W[t_].astype(np.float64) @ (alpha * np.sin(arg))
+    close(e, e_ref, REL_EF, "fused rff energies")
+    close(gx, g_ref, REL_EF, "fused rff gradient")
+    assert (gx[total:] == 0).all()
+    e2, g2 = ops.rff_energy_sorted(t32(x), off, ss, t32(W), t32(b), t32(alpha), N, with_grad=False)
+    assert g2 is None
+    close(e2, e_ref, REL_EF, "fused rff energies only")
+
+
 @pytest.mark.parametrize("d,F,n", [(64, 200, 6), (128, 704, 21), (128, 130, 29), (256, 64, 9), (16, 40, 6)])
 def test_rff_derivatives_molecule_major(d, F, n):
     """Matrix-core route (segments instead of a molecule index); accumulates onto G;

@@ -227,6 +227,43 @@ def test_rff_model_vs_oracle():
     close(e2, E, REL_EF, "scripted rff energies")
 
 
+@pytest.mark.parametrize("npcas,nstacks,case", [(64, 3, "aspirin"), (128, 2, "ragged")])
+def test_rff_fused_forward_vs_oracle(npcas, nstacks, case):
+    """The single-kernel RFF predict path (energies, autograd forces, energies only, TorchScript)."""
+    from qml_lightning_amd.models.random_features import RandomFourrierFeaturesModel
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    if case == "aspirin":
+        species = [1, 6, 8]
+        coords, charges = helpers.fixed_composition_batch(helpers.ASPIRIN, 7, 1)
+    else:
+        species = [1, 6, 7, 8, 9]
+        coords, charges = helpers.ragged_batch(11, 2)
+    rep = FCHLCuda(species=np.array(species))
+    np.random.seed(6)
+    m = RandomFourrierFeaturesModel(rep=rep, elements=np.array(species), sigma=2.0, nstacks=nstacks, npcas=npcas)
+    assert m.fused
+    red, _, _, _ = helpers.model_weights(len(species), rep.get_repsize(), npcas, nstacks)
+    m.reductors = t32(red)
+    alpha = np.random.default_rng(14).normal(size=m.nfeatures())
+    m.alpha = torch.tensor(alpha, device=dev())
+    m.is_trained = True
+    prm = oracle_prm(species)
+    X, Z, aid, mid, nat = make_batch(coords, charges)
+    E, F, _ = omodel.rff_energy_forces(X, Z, aid, mid, nat, prm, species, red, m.W.double().cpu().numpy(),
+                                       m.b.double().cpu().numpy(), alpha.astype(np.float32).astype(np.float64))
+    e, f = m.predict_opt(*inputs(X, Z, aid, mid, nat))
+    close(e, E, REL_EF, "fused rff energies")
+    close(f, F, REL_EF, "fused rff forces")
+    e_only = m.predict_opt(*inputs(X, Z, aid, mid, nat), forces=False)
+    close(e_only, E, REL_EF, "fused rff energies, no forces")
+    s = torch.jit.script(m)
+    gX = t32(X).requires_grad_(True)
+    e2 = s.forward(gX, t32(Z), ti32(aid), ti32(mid), ti32(nat))
+    f2, = torch.autograd.grad(-e2.sum(), gX)
+    close(e2, E, REL_EF, "scripted fused rff energies")
+    close(f2, F, REL_EF, "scripted fused rff forces")
+
+
 def test_fd_helper_matches_jacobian():
     """FCHLCuda.rep_deriv_fd, the reference's own check of its analytic Jacobian
     (unit_tests/representation/test_fchl_derivative.py:60-82)."""
