@@ -463,6 +463,10 @@ __device__ __forceinline__ TripleDeriv triple_derivatives(const Triple& t, const
 // ---------------------------------------------------------------------------------
 // VJP
 // ---------------------------------------------------------------------------------
+// TABLE: the per-triple forces on the two neighbours go to an LDS table [6][ntrip] and are
+// summed per neighbour afterwards (each triple index is computed, never searched), instead
+// of LDS atomics, which serialise badly here: the 64 triples of a pass share 3-4 values of j.
+template <bool TABLE>
 __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float* __restrict__ grad_rep,
                                                          float* __restrict__ grad_X) {
     extern __shared__ float smem[];
@@ -481,6 +485,7 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
     float* sinvRs2 = slnRs2 + nRs2;  // [nRs2]
     float* sRs3 = sinvRs2 + nRs2;    // [nRs3]
     float* gin = sRs3 + nRs3;        // [R]
+    float* tab = gin + R;            // TABLE: [6][ntrip]
 
     const float* gsrc = grad_rep + ((size_t)m * a.n + i) * R;
     for (int t = lane; t < R; t += QMLL_WAVE) gin[t] = gsrc[t];
@@ -501,25 +506,36 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
     const float k3 = a.p.eta3 * LOG2E;
     float gix = 0.0f, giy = 0.0f, giz = 0.0f;
 
-    // two-body: lane per neighbour, serial over bins
-    for (int j = lane; j < nn; j += QMLL_WAVE) {
-        const float r = s.r[j];
-        const TwoBody tb = two_body_setup(r, s.fc[j], s.dfc[j], a.p);
-        const float* g = gin + s.el[j] * nRs2;
-        float gr = 0.0f;
-        for (int z = 0; z < nRs2; ++z) {
-            float val, dval;
-            two_body_bin(tb, slnRs2[z], sinvRs2[z], val, dval);
-            gr = fmaf(g[z], dval, gr);
+    // two-body: lanes = (bin group g, neighbour j); group g takes the bins z = g, g+G, ...
+    {
+        const int G = (nn > 0 && nn < 64) ? 64 / nn : 1;
+        for (int base = 0; base < nn; base += QMLL_WAVE) {
+            const int g = G > 1 ? lane / nn : 0;
+            const int j = G > 1 ? lane - g * nn : base + lane;
+            const bool active = g < G && j < nn;
+            float gr = 0.0f;
+            if (active) {
+                const TwoBody tb = two_body_setup(s.r[j], s.fc[j], s.dfc[j], a.p);
+                const float* gz = gin + s.el[j] * nRs2;
+                for (int z = g; z < nRs2; z += G) {
+                    float val, dval;
+                    two_body_bin(tb, slnRs2[z], sinvRs2[z], val, dval);
+                    gr = fmaf(gz[z], dval, gr);
+                }
+            }
+            float tot = gr;
+            for (int k = 1; k < G; ++k) tot += __shfl(gr, (lane + nn * k) & 63, 64);
+            if (active && g == 0) {
+                const float ir = 1.0f / s.r[j];
+                const float ux = s.dx[j] * ir, uy = s.dy[j] * ir, uz = s.dz[j] * ir;   // dr/dR_i
+                gix += tot * ux;
+                giy += tot * uy;
+                giz += tot * uz;
+                sgx[j] -= tot * ux;   // each lane owns its own j here
+                sgy[j] -= tot * uy;
+                sgz[j] -= tot * uz;
+            }
         }
-        const float ir = 1.0f / r;
-        const float ux = s.dx[j] * ir, uy = s.dy[j] * ir, uz = s.dz[j] * ir;   // dr/dR_i
-        gix += gr * ux;
-        giy += gr * uy;
-        giz += gr * uz;
-        sgx[j] -= gr * ux;   // each lane owns its own j here
-        sgy[j] -= gr * uy;
-        sgz[j] -= gr * uz;
     }
     __syncthreads();
 
@@ -556,12 +572,21 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
         gix += Ea * uax + Eb * ubx;
         giy += Ea * uay + Eb * uby;
         giz += Ea * uaz + Eb * ubz;
-        atomicAdd(&sgx[j], -Ea * uax + Ec * t.ujk[0]);
-        atomicAdd(&sgy[j], -Ea * uay + Ec * t.ujk[1]);
-        atomicAdd(&sgz[j], -Ea * uaz + Ec * t.ujk[2]);
-        atomicAdd(&sgx[k], -Eb * ubx - Ec * t.ujk[0]);
-        atomicAdd(&sgy[k], -Eb * uby - Ec * t.ujk[1]);
-        atomicAdd(&sgz[k], -Eb * ubz - Ec * t.ujk[2]);
+        if constexpr (TABLE) {
+            tab[0 * ntrip + tt] = -Ea * uax + Ec * t.ujk[0];
+            tab[1 * ntrip + tt] = -Ea * uay + Ec * t.ujk[1];
+            tab[2 * ntrip + tt] = -Ea * uaz + Ec * t.ujk[2];
+            tab[3 * ntrip + tt] = -Eb * ubx - Ec * t.ujk[0];
+            tab[4 * ntrip + tt] = -Eb * uby - Ec * t.ujk[1];
+            tab[5 * ntrip + tt] = -Eb * ubz - Ec * t.ujk[2];
+        } else {
+            atomicAdd(&sgx[j], -Ea * uax + Ec * t.ujk[0]);
+            atomicAdd(&sgy[j], -Ea * uay + Ec * t.ujk[1]);
+            atomicAdd(&sgz[j], -Ea * uaz + Ec * t.ujk[2]);
+            atomicAdd(&sgx[k], -Eb * ubx - Ec * t.ujk[0]);
+            atomicAdd(&sgy[k], -Eb * uby - Ec * t.ujk[1]);
+            atomicAdd(&sgz[k], -Eb * ubz - Ec * t.ujk[2]);
+        }
     }
     __syncthreads();
     gix = wave_sum(gix);
@@ -573,11 +598,25 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
         atomicAdd(&gm[i * 3 + 1], giy);
         atomicAdd(&gm[i * 3 + 2], giz);
     }
-    for (int j = lane; j < nn; j += QMLL_WAVE) {
-        const int jj = s.j[j];
-        atomicAdd(&gm[jj * 3 + 0], sgx[j]);
-        atomicAdd(&gm[jj * 3 + 1], sgy[j]);
-        atomicAdd(&gm[jj * 3 + 2], sgz[j]);
+    if constexpr (TABLE) {
+        // lane = (neighbour x, component c): triples (x,k) are the run starting at off(x),
+        // triples (j,x) sit at off(j) + x - j - 1, with off(j) = j (2 nn - j - 1) / 2
+        for (int it = lane; it < 3 * nn; it += QMLL_WAVE) {
+            const int x = it / 3, c = it - 3 * x;
+            float sum = c == 0 ? sgx[x] : (c == 1 ? sgy[x] : sgz[x]);
+            const float* tj = tab + c * ntrip + (x * (2 * nn - x - 1)) / 2;
+            for (int q = 0; q < nn - 1 - x; ++q) sum += tj[q];
+            const float* tk = tab + (3 + c) * ntrip + x - 1;
+            for (int j = 0; j < x; ++j) sum += tk[(j * (2 * nn - j - 1)) / 2 - j];
+            atomicAdd(&gm[s.j[x] * 3 + c], sum);
+        }
+    } else {
+        for (int j = lane; j < nn; j += QMLL_WAVE) {
+            const int jj = s.j[j];
+            atomicAdd(&gm[jj * 3 + 0], sgx[j]);
+            atomicAdd(&gm[jj * 3 + 1], sgy[j]);
+            atomicAdd(&gm[jj * 3 + 2], sgz[j]);
+        }
     }
 }
 
@@ -793,10 +832,17 @@ extern "C" int qmll_fchl19_vjp(const float* X, const int* types, const float* ce
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(grad_rep && grad_X, QMLL_ERR_INVALID, "qmll_fchl19_vjp: null gradient pointer");
     const int R = prm->nspecies * prm->nRs2 + prm->nspecies * (prm->nspecies + 1) * prm->nRs3;
-    const size_t lds = sizeof(float) * ((size_t)(STAGE_ARRAYS + 3) * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 + R);
+    size_t lds = sizeof(float) * ((size_t)(STAGE_ARRAYS + 3) * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 + R);
     QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
                  "qmll_fchl19_vjp: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R, LDS_LIMIT);
-    hipLaunchKernelGGL(fchl19_vjp_kernel, dim3(A), dim3(64), lds, (hipStream_t)stream, a, grad_rep, grad_X);
+    // per-triple force table [6][cap (cap-1) / 2] while it stays small; LDS atomics beyond
+    const size_t table = sizeof(float) * 6 * ((size_t)a.cap * (a.cap - 1) / 2);
+    if (table <= 16 * 1024 && lds + table <= LDS_LIMIT) {
+        lds += table;
+        hipLaunchKernelGGL(fchl19_vjp_kernel<true>, dim3(A), dim3(64), lds, (hipStream_t)stream, a, grad_rep, grad_X);
+    } else {
+        hipLaunchKernelGGL(fchl19_vjp_kernel<false>, dim3(A), dim3(64), lds, (hipStream_t)stream, a, grad_rep, grad_X);
+    }
     QMLL_CHECK_LAUNCH("qmll_fchl19_vjp");
     return QMLL_OK;
 }

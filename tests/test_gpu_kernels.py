@@ -65,6 +65,9 @@ CASES = {
     "aspirin_c2": lambda: (helpers.fixed_composition_batch(helpers.ASPIRIN, 3, 1), [1, 6, 8], {}),
     "ragged_c3": lambda: (helpers.ragged_batch(12, 2), [1, 6, 7, 8, 9], {}),
     "flexible_c4": lambda: (helpers.fixed_composition_batch(helpers.C12H12N2O, 2, 3, sigma=0.15), [1, 6, 7, 8], {}),
+    # 40 atoms: more neighbours than the backward kernel's per-triple table holds (its other path)
+    "big_molecule": lambda: (helpers.fixed_composition_batch(np.array([6] * 14 + [1] * 20 + [8] * 6), 1, 11, box=8.0),
+                             [1, 6, 8], {}),
     "short_cutoff": lambda: (helpers.fixed_composition_batch(helpers.ASPIRIN, 2, 5), [1, 6, 8],
                              {"rcut": 3.1, "nRs2": 7, "nRs3": 5}),
 }
