@@ -89,8 +89,6 @@ __device__ __forceinline__ void min_image(float& dx, float& dy, float& dz, const
     dz = c[6] * s0 + c[7] * s1 + c[8] * s2;
 }
 
-__device__ __forceinline__ float cutoff(float r, float inv_rc) { return 0.5f * (cosf(r * PI_F * inv_rc) + 1.0f); }
-__device__ __forceinline__ float dcutoff(float r, float inv_rc) { return -0.5f * PI_F * inv_rc * sinf(r * PI_F * inv_rc); }
 
 // Fill the LDS neighbour arrays of atom (m,i), sorted by element type; returns the
 // neighbour count.  Neighbours whose element type is negative (charge not in `species`)
@@ -171,8 +169,11 @@ __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i,
                         s.dy[pos] = dy;
                         s.dz[pos] = dz;
                         s.r[pos] = r;
-                        s.fc[pos] = cutoff(r, inv_rc);
-                        s.dfc[pos] = dcutoff(r, inv_rc);
+                        // fc = (cos(pi r/rc) + 1)/2 and its r-derivative from one polynomial sincos
+                        float sn, cs;
+                        sincos_f32(r * PI_F * inv_rc, &sn, &cs);
+                        s.fc[pos] = 0.5f * (cs + 1.0f);
+                        s.dfc[pos] = -0.5f * PI_F * inv_rc * sn;
                         s.el[pos] = e;
                         s.j[pos] = j;
                     }
@@ -290,7 +291,7 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
         const float s2 = logf(1.0f + a.p.eta2 / (r * r));
         smu[j] = logf(r) - 0.5f * s2;                    // ln(r / sqrt(1 + eta2/r^2))
         sis2[j] = 0.5f * LOG2E / s2;
-        spre[j] = rsqrtf(s2) * 0.3989422804014327f * powf(r, -a.p.two_body_decay) * s.fc[j];
+        spre[j] = rsqrtf(s2) * 0.3989422804014327f * fexp2(-a.p.two_body_decay * flog2(r)) * s.fc[j];
     }
     __syncthreads();
 
@@ -322,7 +323,7 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     }
 
     // ---- three-body blocks ----
-    const float zeta2 = 2.0f * expf(-0.5f * PI_F * PI_F);
+    const float zeta2 = 0.014383766711652736f;   // 2 exp(-pi^2 / 2)
     const float k3 = a.p.eta3 * LOG2E;
     const int W3 = nRs3 < 64 ? nRs3 : 64;
     const int TS = 64 / W3;
@@ -410,7 +411,7 @@ __device__ __forceinline__ TwoBody two_body_setup(float r, float fc, float dfc, 
     t.mu = logf(r) - 0.5f * t.s2;
     t.s2p = -2.0f * p.eta2 / (r * (r2 + p.eta2));      // d sigma^2 / dr
     t.mup = 1.0f / r - 0.5f * t.s2p;                   // d mu / dr
-    t.pre = rsqrtf(t.s2) * 0.3989422804014327f * powf(r, -p.two_body_decay);
+    t.pre = rsqrtf(t.s2) * 0.3989422804014327f * fexp2(-p.two_body_decay * flog2(r));
     t.fc = fc;
     t.dfc = dfc;
     t.d2_over_r = p.two_body_decay / r;
@@ -541,7 +542,7 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
 
     // three-body: lane per triple, serial over radial bins
     const int ntrip = nn * (nn - 1) / 2;
-    const float zeta2 = 2.0f * expf(-0.5f * PI_F * PI_F);
+    const float zeta2 = 0.014383766711652736f;   // 2 exp(-pi^2 / 2)
     for (int tt = lane; tt < ntrip; tt += QMLL_WAVE) {
         int j, k;
         unrank_pair(tt, nn, j, k);
@@ -655,7 +656,7 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
     __syncthreads();
 
     const float k3 = a.p.eta3 * LOG2E;
-    const float zeta2 = 2.0f * expf(-0.5f * PI_F * PI_F);
+    const float zeta2 = 0.014383766711652736f;   // 2 exp(-pi^2 / 2)
     float* jbase = jac + (((size_t)m * a.n + i) * a.n) * 3 * R;
 
     // target = -1: central atom; target = 0..nn-1: neighbour at that list position
