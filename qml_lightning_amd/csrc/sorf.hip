@@ -381,24 +381,23 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_fused_kernel(
     }
 }
 
-// ---- fused kernel, instruction-lean variant (one transform per stack, d >= 128) ---------
-// The generic kernel above spends ~75 vector instructions per coefficient; this one ~45:
-//  * the four butterfly stages inside a row of 16 lanes are ONE v_fmac_f32_dpp each,
-//    w += c * w[partner], c = +-1 per lane.  Lanes that should hold (partner - own) hold its
-//    negative instead; the pending sign of a lane is the same after every full transform
-//    (parity of its four stage bits), so it is folded into per-lane constants.  The third
-//    stage pairs lane i with i^7 (row_half_mirror, a single DPP control; i^4 is none), which
-//    is the standard transform if logical index bits (c0,c1,c2,c3) sit at lane
-//    (c0^c2) + 2(c1^c2) + 4 c2 + 8 c3: a fixed permutation of where each lane loads from.
-//  * the stages across rows (lanes 16 and 32 apart) use v_permlane16/32_swap on register
-//    pairs WITHOUT swapping back: each such step leaves one index bit exchanged between the
-//    register number and the lane number.  The forward transform therefore ends in a permuted
-//    layout; bias and alpha are simply loaded in that layout, and the adjoint transform, run
-//    with its two swap stages in the opposite order, ends in the original layout again.
+// ---- fused kernel, instruction-lean variant (one transform per stack, 64 <= d <= 256) ----
+// The generic kernel above spends ~75 vector instructions per coefficient; this one ~40:
+//  * a transform lives in ONE ROW of 16 lanes, d/16 registers per lane, so the four rows of a
+//    wavefront hold four atoms and only four butterfly stages cross lanes (none crosses rows);
+//    the other log2(d/16) stages are register-to-register.
+//  * each cross-lane stage is ONE v_fmac_f32_dpp, w += c * w[partner], c = +-1 per lane.
+//    Lanes that should hold (partner - own) hold its negative instead; the pending sign of a
+//    lane is the same after every full transform (parity of its four stage bits), so it is
+//    folded into per-lane constants.  The third stage pairs lane i with i^7 (row_half_mirror,
+//    a single DPP control; i^4 is none), which is the standard transform if logical index
+//    bits (c0,c1,c2,c3) sit at lane (c0^c2) + 2(c1^c2) + 4 c2 + 8 c3: a fixed permutation of
+//    where each lane loads from.
 //  * sin and cos come from a reduction by pi (not pi/2): both carry the same sign (-1)^k,
 //    which is applied once to the weight alpha that multiplies both; no quadrant swap.
-//  * two stacks are in flight per wavefront (d = 128), so the dependent DPP chains of one
-//    hide the latency of the other.
+//  * the four atoms of a workgroup share each stack's sign diagonal, bias and alpha (one
+//    load serves all rows), which divides the L2 traffic for those vectors -- the limit of a
+//    one-atom-per-workgroup mapping -- by four.
 #define QMLL_DPP_STAGE4(CTRL, w0, w1, w2, w3, c)                                                 \
     asm("s_nop 1\n\t"                                                                            \
         "v_fmac_f32_dpp %0, %0, %4 " CTRL " row_mask:0xf bank_mask:0xf\n\t"                      \
@@ -422,21 +421,6 @@ __device__ __forceinline__ void row_stages(float (&w)[NV], const float (&cs)[4])
     for (int g = 0; g < NV; g += 4) QMLL_DPP_STAGE4("row_ror:8", w[g], w[g + 1], w[g + 2], w[g + 3], cs[3]);
 }
 
-// butterfly between lanes 16 (or 32) apart for a register pair; afterwards the pair's index
-// bit and that lane bit have changed places (no swap back)
-template <int MASK>
-__device__ __forceinline__ void swap_butterfly(float& a, float& b) {
-    typedef unsigned uint2_t __attribute__((ext_vector_type(2)));
-    uint2_t r;
-    if constexpr (MASK == 16)
-        r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
-    else
-        r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
-    const float x = __uint_as_float(r[0]), y = __uint_as_float(r[1]);
-    a = x + y;
-    b = x - y;
-}
-
 template <int EPL>
 __device__ __forceinline__ void register_stages(float* v) {
 #pragma unroll
@@ -452,10 +436,21 @@ __device__ __forceinline__ void register_stages(float* v) {
     }
 }
 
+// sum over the 16 lanes of a row, result in every lane of the row
+__device__ __forceinline__ float row_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false));   // row_half_mirror
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));   // row_ror:8
+    return v;
+}
+
 // sin and cos of x = r + k pi, |r| <= pi/2, WITHOUT the factor (-1)^k, which is returned as
 // a sign-bit mask.  Polynomials of degree 9 / 10 on [-pi/2, pi/2]: 1.3e-7 absolute.
 __device__ __forceinline__ void sincos_pi(float x, float* s, float* c, int* signmask) {
-    const float kf = rintf(x * 0.31830988618379067154f);
+    // k = round(x / pi) by adding 1.5 * 2^23: the sum's lowest mantissa bit is the parity of k
+    const float t = fmaf(x, 0.31830988618379067154f, 12582912.0f);
+    const float kf = t - 12582912.0f;
     float r = fmaf(kf, -3.1415920257568359375f, x);              // pi split in two fp32 parts
     r = fmaf(kf, -6.2783295e-07f, r);
     const float r2 = r * r;
@@ -468,23 +463,20 @@ __device__ __forceinline__ void sincos_pi(float x, float* s, float* c, int* sign
     pc = fmaf(pc, r2, 0.04166664183139801f);
     pc = fmaf(pc, r2, -0.5f);
     *c = fmaf(pc, r2, 1.0f);
-    *signmask = (int)kf << 31;
+    *signmask = __float_as_int(t) << 31;
 }
 
-// NA atoms of one element share a workgroup: each wavefront loads the sign diagonal, bias and
-// alpha of a stack once and applies them to all NA atoms, which divides the L2 traffic for
-// those vectors (re-read by every atom otherwise, the limit of a one-atom-per-workgroup
-// mapping) by NA and gives NA * d/64 independent butterfly chains per wavefront.
-template <int LOG2D, int NA, bool WITH_GRAD>
-__global__ __launch_bounds__(SORF_THREADS) void sorf_energy_lean_kernel(
+constexpr int ROWS_NA = 4;   // atoms per workgroup = rows of 16 lanes per wavefront
+
+template <int LOG2D, bool WITH_GRAD>
+__global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
     const float* __restrict__ x, const float* __restrict__ D, const float* __restrict__ bias,
     const float* __restrict__ alpha, const int* __restrict__ out_index, const int* __restrict__ type_offsets, int ne,
     int A, int S, float scale, float normf, float* __restrict__ e_atom, float* __restrict__ gx) {
     constexpr int d = 1 << LOG2D;
-    constexpr int EPL = d / 64;                 // registers per lane per transform
-    constexpr int M = LOG2D - 6;                // log2(EPL)
-    constexpr int NV = NA * EPL;
-    static_assert(EPL >= 2 && NV % 4 == 0, "needs register pairs and groups of four chains");
+    constexpr int EPL = d / 16;                 // registers per lane
+    constexpr int NA = ROWS_NA;
+    static_assert(EPL >= 4 && EPL % 4 == 0, "groups of four butterfly chains per lane");
     __shared__ float red[SORF_WAVES][NA][d];
     __shared__ float ered[SORF_WAVES][NA];
     const int lane = threadIdx.x & 63;
@@ -514,122 +506,86 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_lean_kernel(
         if (rows <= 0) return;
     }
 
-    // where this lane's registers sit in the vector: original layout (x, D, gradient) and the
-    // layout the forward transform ends in (bias, alpha)
-    const int i16 = lane & 15, l4 = (lane >> 4) & 1, l5 = lane >> 5;
+    // this lane's row (atom) and the EPL consecutive vector elements it holds
+    const int row = lane >> 4, i16 = lane & 15;
     const int c2 = (i16 >> 2) & 1, c0 = (i16 & 1) ^ c2, c1 = ((i16 >> 1) & 1) ^ c2, c3 = i16 >> 3;
-    const int cidx = c0 | (c1 << 1) | (c2 << 2) | (c3 << 3);
-    const int e0 = (cidx + 16 * l4 + 32 * l5) * EPL;
-    unsigned e1b[EPL];                          // byte offsets in the permuted layout
-#pragma unroll
-    for (int p = 0; p < EPL; ++p)
-        e1b[p] = 4u * (unsigned)(l4 | ((p >> 1) << 1) | (cidx << M) | (l5 << (M + 4)) | ((p & 1) << (M + 5)));
+    const int e0 = (c0 | (c1 << 1) | (c2 << 2) | (c3 << 3)) * EPL;
     const float cs[4] = {c0 ? -1.0f : 1.0f, c1 ? -1.0f : 1.0f, c2 ? -1.0f : 1.0f, c3 ? -1.0f : 1.0f};
     const float sigma = ((c0 + c1 + c2 + c3) & 1) ? -1.0f : 1.0f;   // pending sign after a transform
     const float scale_l = scale * sigma;
+    const bool valid = row < rows;
 
-    float xv[NV], acc[NV], energy[NA];
+    float xv[EPL], acc[EPL];
+    load_vec<EPL>(xv, x + (size_t)(row0 + (valid ? row : 0)) * d + e0);
 #pragma unroll
-    for (int j = 0; j < NA; ++j) {
-        float t[EPL];
-        load_vec<EPL>(t, x + (size_t)(row0 + (j < rows ? j : 0)) * d + e0);
-#pragma unroll
-        for (int p = 0; p < EPL; ++p) {
-            xv[j * EPL + p] = j < rows ? t[p] : 0.0f;
-            acc[j * EPL + p] = 0.0f;
-        }
-        energy[j] = 0.0f;
+    for (int p = 0; p < EPL; ++p) {
+        if (!valid) xv[p] = 0.0f;
+        acc[p] = 0.0f;
     }
+    float energy = 0.0f;
 
+    // per stack: the sign diagonal is fetched one stack ahead (it is the first thing a stack
+    // needs), bias and alpha at the start of their own stack (needed after the transform)
     float dv[EPL], bv[EPL], av[EPL];
-    auto fetch = [&](int stack, float (&dd)[EPL], float (&bb)[EPL], float (&aa)[EPL]) {
-        const size_t row = (size_t)stack * d;               // wave-uniform
-        load_vec<EPL>(dd, D + row + e0);
-        const char* brow = reinterpret_cast<const char*>(bias + row);
-        const char* arow = reinterpret_cast<const char*>(alpha + row);
+    int s = wave;
+    if (s < S) load_vec<EPL>(dv, D + (size_t)s * d + e0);
+    for (; s < S; s += SORF_WAVES) {
+        const size_t off = (size_t)s * d + e0;               // the same for the four rows
+        load_vec<EPL>(bv, bias + off);
+        load_vec<EPL>(av, alpha + off);
+        float dn[EPL];
+        load_vec<EPL>(dn, D + (size_t)(s + SORF_WAVES < S ? s + SORF_WAVES : s) * d + e0);
+
+        float v[EPL];
+#pragma unroll
+        for (int p = 0; p < EPL; ++p) v[p] = xv[p] * dv[p];
+        register_stages<EPL>(v);
+        row_stages<EPL>(v, cs);
+
+        float arg[EPL], amax = 0.0f;
 #pragma unroll
         for (int p = 0; p < EPL; ++p) {
-            bb[p] = *reinterpret_cast<const float*>(brow + e1b[p]);
-            aa[p] = *reinterpret_cast<const float*>(arow + e1b[p]);
-        }
-    };
-    int s = wave;
-    if (s < S) fetch(s, dv, bv, av);
-    for (; s < S; s += SORF_WAVES) {
-        float dn[EPL], bn[EPL], an[EPL];
-        fetch(s + SORF_WAVES < S ? s + SORF_WAVES : s, dn, bn, an);   // the last round re-reads its own rows
-
-        float v[NV];
-#pragma unroll
-        for (int j = 0; j < NA; ++j)
-#pragma unroll
-            for (int p = 0; p < EPL; ++p) v[j * EPL + p] = xv[j * EPL + p] * dv[p];
-        // forward transform: register stages, in-row stages, then rows 16 and 32 apart
-#pragma unroll
-        for (int j = 0; j < NA; ++j) register_stages<EPL>(v + j * EPL);
-        row_stages<NV>(v, cs);
-#pragma unroll
-        for (int q = 0; q < NV; q += 2) swap_butterfly<16>(v[q], v[q + 1]);
-#pragma unroll
-        for (int q = 0; q < NV; q += 2) swap_butterfly<32>(v[q], v[q + 1]);
-
-        float arg[NV], amax = 0.0f;
-#pragma unroll
-        for (int q = 0; q < NV; ++q) {
-            arg[q] = fmaf(v[q], scale_l, bv[q % EPL]);
-            amax = fmaxf(amax, fabsf(arg[q]));
+            arg[p] = fmaf(v[p], scale_l, bv[p]);
+            amax = fmaxf(amax, fabsf(arg[p]));
         }
 #pragma unroll
-        for (int q = 0; q < NV; ++q) {
+        for (int p = 0; p < EPL; ++p) {
             float sn, cs_;
             int sm;
-            sincos_pi(arg[q], &sn, &cs_, &sm);
-            const float w = __int_as_float(__float_as_int(av[q % EPL]) ^ sm);
-            energy[q / EPL] = fmaf(w, cs_, energy[q / EPL]);
-            v[q] = w * sn;                                   // -(d E / d coefficient) / normf
+            sincos_pi(arg[p], &sn, &cs_, &sm);
+            const float w = __int_as_float(__float_as_int(av[p]) ^ sm);
+            energy = fmaf(w, cs_, energy);
+            v[p] = w * sn;                                   // -(d E / d coefficient) / normf
         }
         if (__builtin_expect(__any(amax > 32000.0f), 0)) {
             // arguments the two-term reduction cannot handle: redo those with the library routine
 #pragma unroll
-            for (int q = 0; q < NV; ++q) {
-                if (fabsf(arg[q]) > 32000.0f) {
+            for (int p = 0; p < EPL; ++p) {
+                if (fabsf(arg[p]) > 32000.0f) {
                     float sn, cs_, s0, c0_;
                     int sm;
-                    sincos_pi(arg[q], &s0, &c0_, &sm);
-                    const float w0 = __int_as_float(__float_as_int(av[q % EPL]) ^ sm);
-                    sincos_large(arg[q], &sn, &cs_);
-                    energy[q / EPL] += av[q % EPL] * cs_ - w0 * c0_;
-                    v[q] = av[q % EPL] * sn;
+                    sincos_pi(arg[p], &s0, &c0_, &sm);
+                    const float w0 = __int_as_float(__float_as_int(av[p]) ^ sm);
+                    sincos_large(arg[p], &sn, &cs_);
+                    energy += av[p] * cs_ - w0 * c0_;
+                    v[p] = av[p] * sn;
                 }
             }
         }
         if constexpr (WITH_GRAD) {
-            // adjoint transform from the permuted layout back to the original one
+            register_stages<EPL>(v);
+            row_stages<EPL>(v, cs);
 #pragma unroll
-            for (int j = 0; j < NA; ++j) register_stages<EPL>(v + j * EPL);
-            row_stages<NV>(v, cs);
-#pragma unroll
-            for (int q = 0; q < NV; q += 2) swap_butterfly<32>(v[q], v[q + 1]);
-#pragma unroll
-            for (int q = 0; q < NV; q += 2) swap_butterfly<16>(v[q], v[q + 1]);
-#pragma unroll
-            for (int q = 0; q < NV; ++q) acc[q] = fmaf(v[q], dv[q % EPL], acc[q]);
+            for (int p = 0; p < EPL; ++p) acc[p] = fmaf(v[p], dv[p], acc[p]);
         }
 #pragma unroll
-        for (int p = 0; p < EPL; ++p) {
-            dv[p] = dn[p];
-            bv[p] = bn[p];
-            av[p] = an[p];
-        }
+        for (int p = 0; p < EPL; ++p) dv[p] = dn[p];
     }
+    energy = row_sum(energy);
+    if (i16 == 0) ered[wave][row] = energy;
+    if constexpr (WITH_GRAD) {
 #pragma unroll
-    for (int j = 0; j < NA; ++j) {
-        const float e = wave_sum(energy[j]);
-        if (lane == 0) ered[wave][j] = e;
-        if constexpr (WITH_GRAD) {
-#pragma unroll
-            for (int p = 0; p < EPL; ++p) red[wave][j][e0 + p] = acc[j * EPL + p] * sigma;
-        }
+        for (int p = 0; p < EPL; ++p) red[wave][row][e0 + p] = acc[p] * sigma;
     }
     __syncthreads();
     if (threadIdx.x < rows) {
@@ -951,26 +907,24 @@ static int launch_fused(const char* who, const float* x, const float* D, const f
                         int T, float normalisation, float* e_atom, float* gx, hipStream_t stream) {
     const float scale = normalisation * hnorm(d, T);
     const float normf = sqrtf(2.0f / ((float)S * (float)d));
-    if (T == 1 && d >= 128 && d <= 512 && types == nullptr) {
-        // one transform per stack, two to eight registers per lane, atoms groupable by element:
-        // the instruction-lean kernel, several atoms per workgroup
-#define CALL_LEAN(L, NA)                                                                                             \
-    {                                                                                                                \
-        const dim3 grid((A + NA - 1) / NA + (type_offsets ? ne : 0));                                                \
-        if (gx)                                                                                                      \
-            hipLaunchKernelGGL((sorf_energy_lean_kernel<L, NA, true>), grid, dim3(SORF_THREADS), 0, stream, x, D,    \
-                               bias, alpha, out_index, type_offsets, ne, A, S, scale, normf, e_atom, gx);            \
-        else                                                                                                         \
-            hipLaunchKernelGGL((sorf_energy_lean_kernel<L, NA, false>), grid, dim3(SORF_THREADS), 0, stream, x, D,   \
-                               bias, alpha, out_index, type_offsets, ne, A, S, scale, normf, e_atom, gx);            \
-    }
+    if (T == 1 && d >= 64 && d <= 256 && types == nullptr) {
+        // one transform per stack, 4 to 16 registers per lane, atoms groupable by element: the
+        // instruction-lean kernel (four atoms per workgroup)
+        const dim3 grid((A + ROWS_NA - 1) / ROWS_NA + (type_offsets ? ne : 0));
+#define CALL_ROWS(L)                                                                                                 \
+    if (gx)                                                                                                          \
+        hipLaunchKernelGGL((sorf_energy_rows_kernel<L, true>), grid, dim3(SORF_THREADS), 0, stream, x, D, bias,      \
+                           alpha, out_index, type_offsets, ne, A, S, scale, normf, e_atom, gx);                      \
+    else                                                                                                             \
+        hipLaunchKernelGGL((sorf_energy_rows_kernel<L, false>), grid, dim3(SORF_THREADS), 0, stream, x, D, bias,     \
+                           alpha, out_index, type_offsets, ne, A, S, scale, normf, e_atom, gx)
         switch (qmll_log2(d)) {
-            case 7: CALL_LEAN(7, 4) break;
-            case 8: CALL_LEAN(8, 4) break;
-            case 9: CALL_LEAN(9, 2) break;
+            case 6: { CALL_ROWS(6); } break;
+            case 7: { CALL_ROWS(7); } break;
+            case 8: { CALL_ROWS(8); } break;
             default: break;
         }
-#undef CALL_LEAN
+#undef CALL_ROWS
         QMLL_CHECK_LAUNCH(who);
         if (gx && type_offsets) {
             hipLaunchKernelGGL(zero_tail_rows_kernel, dim3(64), dim3(256), 0, stream, type_offsets, ne, A, d, gx);
