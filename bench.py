@@ -268,9 +268,6 @@ def main():
         idx = data['element_index'][e]
         sub = torch.matmul(flat_rep.index_select(0, idx), model.reductors[ei])
         Ae = sub.shape[0]
-        e_atom = torch.empty(Ae, device=dev)
-        t_fused += timed(lambda: ops.sorf_energy_fused(sub, model.Dmat[ei], model.bias[ei], alpha32, None, norm, 1,
-                                                       e_atom))
         # the reference's two-op contract, kernel by kernel (coefficients materialised)
         molidx = torch.div(idx, n, rounding_mode='floor').to(torch.int32)
         t_sorf += timed(lambda: ops.sorf_forward(sub, model.Dmat[ei], norm, 1))
@@ -283,11 +280,33 @@ def main():
         del coeffs, gc
     d = NPCAS
     log2d = int(np.log2(d))
+    # the predict step's own launches: sort by element, projection (and its transpose), fused kernel
+    ne = len(SPECIES)
+    slots = mid * n + aid
+    tflat = types.view(-1)
+    ss, off = ops.sort_by_type(tflat, slots, ne)
+    x_sorted = ops.project_typed(flat_rep, ss, off, model.reductors)
+    gx_sorted = torch.randn_like(x_sorted)
+    t_sort = timed(lambda: ops.sort_by_type(tflat, slots, ne))
+    t_proj = timed(lambda: ops.project_typed(flat_rep, ss, off, model.reductors))
+    t_projb = timed(lambda: ops.project_typed_backward(gx_sorted, ss, off, model.reductors, tflat, B * n))
+    t_fused = timed(lambda: ops.sorf_energy_sorted(x_sorted, off, ss, model.Dmat, model.bias, alpha32, norm, 1, B * n))
+    proj_flops = 2.0 * A * R * d
+    kernels["sort_by_type"] = {"seconds": t_sort, "bound": "latency"}
+    kernels["project_typed"] = {"seconds": t_proj, "bound": "mfma", "TFLOPs": proj_flops / t_proj / 1e12,
+                                "frac": proj_flops / t_proj / 1e12 / FP32_PEAK_TFLOPS,
+                                "GBs": A * 4 * (R + d) / t_proj / 1e9}
+    kernels["project_typed_backward"] = {"seconds": t_projb, "bound": "mfma", "TFLOPs": proj_flops / t_projb / 1e12,
+                                         "frac": proj_flops / t_projb / 1e12 / FP32_PEAK_TFLOPS,
+                                         "GBs": A * 4 * (R + d) / t_projb / 1e9}
     # fused kernel, algorithmic flops per atom: forward+adjoint butterflies 2*F*log2(d), D multiplies 2F,
     # scale+bias FMA 2F, one sin and one cos per feature 2F, energy FMA 2F, alpha*norm*sin 2F
     fused_flops = A * F * (2 * log2d + 10)
+    # 37.5 vector instructions per coefficient in the kernel's main loop (d = 128; counted in its ISA);
+    # plain fp32 VOP2 instructions issue at 1.0e12 wavefront-instructions/s on this GPU (measured)
     kernels["sorf_energy_fused"] = {"seconds": t_fused, "bound": "valu", "TFLOPs": fused_flops / t_fused / 1e12,
-                                    "sincos_per_s": A * F / t_fused}
+                                    "sincos_per_s": A * F / t_fused,
+                                    "valu_wave_instr_per_s": 37.5 * A * F / 64 / t_fused}
     kernels["sorf_forward"] = {"seconds": t_sorf, "bound": "hbm", "GBs": A * (4 * d + 4 * F) / t_sorf / 1e9}
     kernels["cos_features_f32"] = {"seconds": t_cos, "bound": "hbm", "GBs": (A * 4 * F + B * 4 * F) / t_cos / 1e9}
     kernels["cos_features_backward"] = {"seconds": t_cosb, "bound": "hbm", "GBs": A * 8 * F / t_cosb / 1e9}
@@ -302,6 +321,11 @@ def main():
         Ft = [rng.normal(size=(21, 3)) for _ in range(NMOL_TRAIN)]
         model.build_Z_components(tc[:64], tq[:64], E=Et[:64], F=Ft[:64], print_info=False)   # warm-up
         torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for b0 in range(0, NMOL_TRAIN, 500):                 # the host formatting the build repeats per batch
+            model.format_data(tc[b0:b0 + 500], tq[b0:b0 + 500], E=Et[b0:b0 + 500], F=Ft[b0:b0 + 500])
+        torch.cuda.synchronize()
+        t_format = time.perf_counter() - t0
         t0 = time.perf_counter()
         ZTZ, ZTy = model.build_Z_components(tc, tq, E=Et, F=Ft, print_info=False)
         torch.cuda.synchronize()
@@ -319,6 +343,7 @@ def main():
                                "frac": gram_flops / t_gram / 1e12 / FP64_PEAK_TFLOPS}
         train = {"ztz_seconds": t_build, "ztz_molecules": NMOL_TRAIN, "ztz_rows": M, "ztz_features": F,
                  "ztz_includes": "host format_data + FCHL19 Jacobian + projection + SORF rows + Gram, 500 molecules per batch",
+                 "ztz_seconds_excluding_format_data": t_build - t_format, "format_data_seconds": t_format,
                  "gram_kernel_seconds": t_gram}
         del rows, yv, ZTZ, ZTy
 
@@ -338,9 +363,11 @@ def main():
                     "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": kernels[dominant]["TFLOPs"] / FP32_PEAK_TFLOPS,
                     "traffic": kernels[dominant].get("traffic_bytes"),
                     "note": "fused FWHT+sincos kernel: neither HBM nor MFMA bounds it (8d bytes per atom, no "
-                            "contraction); algorithmic flops count one flop per sin and per cos, a 1-ulp sincos "
-                            "costs ~26 VALU ops, so 0.10 of the fp32 FMA peak is ~0.8 of the instruction-issue "
-                            "rate (DESIGN.md section 6); traffic = bytes per launch from profiles/pmc_traffic.json"}
+                            "contraction); it is bound by vector instruction issue.  Algorithmic flops count one "
+                            "flop per sin and per cos, while a 1-ulp sincos costs ~19 instructions and the cross-lane "
+                            "butterflies issue at half rate, so the fraction of the fp32 FMA peak understates it: "
+                            "valu_wave_instr_per_s against the measured 1.0e12/s for plain fp32 instructions is the "
+                            "issue-rate fraction; traffic = bytes per launch from profiles/pmc_traffic.json"}
     else:
         roofline = {"kernel": dominant, "bound": "valu", "achieved": kernels[dominant]["exp_per_s"] / 1e12,
                     "peak": 256 * 4 * 16 * 2.4e9 / 4 / 1e12, "unit": "Texp/s",

@@ -190,12 +190,23 @@ class BaseKernel():
         if cpu_solve:
             self.alpha = torch.linalg.solve(ZTZ, ZtrainY.cpu())[:, 0].to(self.device)
         else:
-            self.alpha = torch.linalg.solve(ZTZ, ZtrainY)[:, 0]
+            self.alpha = self._solve_spd(ZTZ, ZtrainY)[:, 0]
         end.record()
         torch.cuda.synchronize()
         if print_info:
             print("coefficients time: ", start.elapsed_time(end), "ms")
         self.is_trained = True
+
+    @staticmethod
+    def _solve_spd(A, b):
+        """x = A^-1 b for the regularised normal matrix.  The reference calls
+        torch.linalg.solve (LU, kernel.py:231); Z^T Z + lambda I is symmetric positive definite,
+        so a Cholesky factorisation gives the same solution for half the flops; LU remains the
+        fallback when rounding has left the matrix numerically indefinite."""
+        L, info = torch.linalg.cholesky_ex(A)
+        if int(info.item()) == 0:
+            return torch.cholesky_solve(b, L)
+        return torch.linalg.solve(A, b)
 
     def hyperparam_opt_nested_cv(self, X, Q, E, F=None, cells=None, inv_cells=None,
                                  sigmas=np.linspace(1.5, 12.5, 10), lambdas=np.logspace(-11, -5, 9), kfolds=5,
