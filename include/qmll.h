@@ -128,18 +128,29 @@ int qmll_sorf_forward(const float* x, const float* D, int A, int d, int S, int T
 int qmll_sorf_adjoint(const float* g, const float* D, int A, int d, int S, int T, float normalisation,
                       float* gx, qmll_stream_t stream);
 
+/* Segment table of a molecule-major atom list, the form in which the reference builds
+ * batch_indexes (torch.where(Z == e)[0], hadamard_features.py:101-107; ordering in
+ * kernel.py:143-149).  mol_index i32 [A] -> seg i32 [nmol+2], zero-filled by the caller:
+ * seg[m] = first atom of molecule m (seg[nmol] = A); seg[nmol+1] becomes non-zero when
+ * mol_index is not ascending or leaves [0,nmol), in which case the table must not be used
+ * (the feature kernels below check the flag on the device, no host round trip). */
+int qmll_segment_offsets(const int* mol_index, int A, int nmol, int* seg, qmll_stream_t stream);
+
 /* Replaces sorf_gpu.CosFeaturesCUDA / cos_features_gpu (hadamard_cuda.cpp:23-32; kernel
  * hadamard_kernel.cu:778-800).  coeffs f32 [A,F], bias f32 [F], mol_index i32 [A]
  * (row of Zf each atom adds to, values in [0,nmol)) -> Zf f32 [nmol,F] +=
- * sqrt(2/F) cos(coeffs+bias), accumulated with atomics into caller-zeroed memory. */
-int qmll_cos_features_f32(const float* coeffs, const float* bias, const int* mol_index, int A, int F, int nmol,
-                          float* Zf, qmll_stream_t stream);
+ * sqrt(2/F) cos(coeffs+bias), into caller-zeroed memory.  seg: NULL, or the table from
+ * qmll_segment_offsets for the same mol_index: each molecule's atoms are then summed in
+ * registers in atom order and added once (deterministic, no atomics); without a table, or
+ * with one flagged invalid, partial sums are added with atomics in any order. */
+int qmll_cos_features_f32(const float* coeffs, const float* bias, const int* mol_index, const int* seg, int A, int F,
+                          int nmol, float* Zf, qmll_stream_t stream);
 
 /* Replaces sorf_gpu.compute_hadamard_features / compute_molecular_featurization
  * (hadamard_cuda.cpp:89-93; kernel hadamard_kernel.cu:541-563): same as above but every
  * fp32 feature value is widened and accumulated into Zf f64 [nmol,F] (in place). */
-int qmll_cos_features_f64(const float* coeffs, const float* bias, const int* mol_index, int A, int F, int nmol,
-                          double* Zf, qmll_stream_t stream);
+int qmll_cos_features_f64(const float* coeffs, const float* bias, const int* mol_index, const int* seg, int A, int F,
+                          int nmol, double* Zf, qmll_stream_t stream);
 
 /* Replaces sorf_gpu.CosDerivativeFeaturesCUDA / cos_derivative_features_gpu
  * (hadamard_cuda.cpp:34-45; kernel hadamard_kernel.cu:816-839).  gZ f32 [nmol,F] ->

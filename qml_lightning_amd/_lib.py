@@ -38,8 +38,9 @@ PROTOTYPES = {
     "qmll_fchl19_jacobian": _FCHL_COMMON + [P, P, P],
     "qmll_sorf_forward": [P, P, c_int, c_int, c_int, c_int, c_float, P, P],
     "qmll_sorf_adjoint": [P, P, c_int, c_int, c_int, c_int, c_float, P, P],
-    "qmll_cos_features_f32": [P, P, P, c_int, c_int, c_int, P, P],
-    "qmll_cos_features_f64": [P, P, P, c_int, c_int, c_int, P, P],
+    "qmll_segment_offsets": [P, c_int, c_int, P, P],
+    "qmll_cos_features_f32": [P, P, P, P, c_int, c_int, c_int, P, P],
+    "qmll_cos_features_f64": [P, P, P, P, c_int, c_int, c_int, P, P],
     "qmll_cos_features_backward": [P, P, P, P, c_int, c_int, c_int, P, P],
     "qmll_sin_coeffs_f64": [P, P, c_int, c_int, P, P],
     "qmll_derivative_features": [P, c_double, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, P],

@@ -382,7 +382,8 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_fused_kernel(
 }
 
 // ---- fused kernel, instruction-lean variant (one transform per stack, 64 <= d <= 256) ----
-// The generic kernel above spends ~75 vector instructions per coefficient; this one ~40:
+// The generic kernel above spends ~75 vector instructions per coefficient; this one ~28 plus two
+// transcendental issues:
 //  * a transform lives in ONE ROW of 16 lanes, d/16 registers per lane, so the four rows of a
 //    wavefront hold four atoms and only four butterfly stages cross lanes (none crosses rows);
 //    the other log2(d/16) stages are register-to-register.
@@ -393,8 +394,7 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_fused_kernel(
 //    a single DPP control; i^4 is none), which is the standard transform if logical index
 //    bits (c0,c1,c2,c3) sit at lane (c0^c2) + 2(c1^c2) + 4 c2 + 8 c3: a fixed permutation of
 //    where each lane loads from.
-//  * sin and cos come from a reduction by pi (not pi/2): both carry the same sign (-1)^k,
-//    which is applied once to the weight alpha that multiplies both; no quadrant swap.
+//  * sin and cos come from the transcendental unit after an exact reduction by 2 pi.
 //  * the four atoms of a workgroup share each stack's sign diagonal, bias and alpha (one
 //    load serves all rows), which divides the L2 traffic for those vectors -- the limit of a
 //    one-atom-per-workgroup mapping -- by four.
@@ -445,25 +445,65 @@ __device__ __forceinline__ float row_sum(float v) {
     return v;
 }
 
-// sin and cos of x = r + k pi, |r| <= pi/2, WITHOUT the factor (-1)^k, which is returned as
-// a sign-bit mask.  Polynomials of degree 9 / 10 on [-pi/2, pi/2]: 1.3e-7 absolute.
-__device__ __forceinline__ void sincos_pi(float x, float* s, float* c, int* signmask) {
-    // k = round(x / pi) by adding 1.5 * 2^23: the sum's lowest mantissa bit is the parity of k
-    const float t = fmaf(x, 0.31830988618379067154f, 12582912.0f);
+// Per-lane constants of the 16-lanes-per-transform layout: which row (transform) of the
+// wavefront the lane belongs to, where its elements sit in the vector, the +-1 factors of
+// the four in-row stages and the sign left pending after a full transform.  A lane holds
+// EPL/4 groups of four consecutive elements, group q at q*64 + 4*pos (pos = the lane's
+// permuted place in the row, which makes row_half_mirror a radix-2 stage): a 16-byte
+// access per lane then covers 256 contiguous bytes per row.  Index bits 0-1 and the bits
+// from 6 up are the register stages, bits 2-5 the in-row stages; the stages of a
+// Walsh-Hadamard transform commute, so the natural-order result is unchanged.
+template <int EPL>
+struct RowLanes {
+    int row, i16, e0;
+    float cs[4];
+    float sigma;
+    __device__ __forceinline__ explicit RowLanes(int lane) {
+        row = lane >> 4;
+        i16 = lane & 15;
+        const int c2 = (i16 >> 2) & 1, c0 = (i16 & 1) ^ c2, c1 = ((i16 >> 1) & 1) ^ c2, c3 = i16 >> 3;
+        e0 = (c0 | (c1 << 1) | (c2 << 2) | (c3 << 3)) * 4;
+        cs[0] = c0 ? -1.0f : 1.0f;
+        cs[1] = c1 ? -1.0f : 1.0f;
+        cs[2] = c2 ? -1.0f : 1.0f;
+        cs[3] = c3 ? -1.0f : 1.0f;
+        sigma = ((c0 + c1 + c2 + c3) & 1) ? -1.0f : 1.0f;
+    }
+};
+
+// the lane's EPL elements of the vector at p (p already includes the lane's e0)
+template <int EPL>
+__device__ __forceinline__ void load_row(float (&v)[EPL], const float* __restrict__ p) {
+#pragma unroll
+    for (int q = 0; q < EPL / 4; ++q) {
+        const float4 t = *reinterpret_cast<const float4*>(p + q * 64);
+        v[4 * q + 0] = t.x;
+        v[4 * q + 1] = t.y;
+        v[4 * q + 2] = t.z;
+        v[4 * q + 3] = t.w;
+    }
+}
+
+template <int EPL>
+__device__ __forceinline__ void store_row(const float (&v)[EPL], float* __restrict__ p) {
+#pragma unroll
+    for (int q = 0; q < EPL / 4; ++q)
+        *reinterpret_cast<float4*>(p + q * 64) = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+}
+
+// sin and cos on the transcendental unit (v_sin_f32 / v_cos_f32 take revolutions): the
+// argument is first reduced to |r| <= pi by a Cody-Waite step with 2 pi split in two fp32
+// parts (exact for |x| <= 3.2e4), so the conversion to revolutions loses nothing.  Measured
+// against fp64 over |x| < 1500: 3.7e-7 maximum, 7.5e-8 rms absolute error.  Two
+// transcendental issues and five plain instructions replace the 17 of a polynomial pair.
+__device__ __forceinline__ void sincos_hw(float x, float* s, float* c) {
+    const float t = fmaf(x, 0.15915494309189535f, 12582912.0f);   // + 1.5 * 2^23: rounds x / 2 pi
     const float kf = t - 12582912.0f;
-    float r = fmaf(kf, -3.1415920257568359375f, x);              // pi split in two fp32 parts
-    r = fmaf(kf, -6.2783295e-07f, r);
-    const float r2 = r * r;
-    float ps = fmaf(r2, 2.599247636680957e-06f, -0.00019806188356596977f);
-    ps = fmaf(ps, r2, 0.008333010599017143f);
-    ps = fmaf(ps, r2, -0.16666656732559204f);
-    *s = fmaf(ps * r2, r, r);
-    float pc = fmaf(r2, -2.607318947411841e-07f, 2.4761640815995634e-05f);
-    pc = fmaf(pc, r2, -0.001388839795254171f);
-    pc = fmaf(pc, r2, 0.04166664183139801f);
-    pc = fmaf(pc, r2, -0.5f);
-    *c = fmaf(pc, r2, 1.0f);
-    *signmask = __float_as_int(t) << 31;
+    float r = fmaf(kf, -6.2831840515136719f, x);
+    r = fmaf(kf, -1.2556659e-06f, r);
+    const float u = r * 0.15915494309189535f;
+    *s = __builtin_amdgcn_sinf(u);
+    *c = __builtin_amdgcn_cosf(u);
 }
 
 constexpr int ROWS_NA = 4;   // atoms per workgroup = rows of 16 lanes per wavefront
@@ -506,17 +546,16 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
         if (rows <= 0) return;
     }
 
-    // this lane's row (atom) and the EPL consecutive vector elements it holds
-    const int row = lane >> 4, i16 = lane & 15;
-    const int c2 = (i16 >> 2) & 1, c0 = (i16 & 1) ^ c2, c1 = ((i16 >> 1) & 1) ^ c2, c3 = i16 >> 3;
-    const int e0 = (c0 | (c1 << 1) | (c2 << 2) | (c3 << 3)) * EPL;
-    const float cs[4] = {c0 ? -1.0f : 1.0f, c1 ? -1.0f : 1.0f, c2 ? -1.0f : 1.0f, c3 ? -1.0f : 1.0f};
-    const float sigma = ((c0 + c1 + c2 + c3) & 1) ? -1.0f : 1.0f;   // pending sign after a transform
+    // this lane's row (atom) and the vector elements it holds
+    const RowLanes<EPL> L(lane);
+    const int row = L.row, i16 = L.i16, e0 = L.e0;
+    const float (&cs)[4] = L.cs;
+    const float sigma = L.sigma;                                     // pending sign after a transform
     const float scale_l = scale * sigma;
     const bool valid = row < rows;
 
     float xv[EPL], acc[EPL];
-    load_vec<EPL>(xv, x + (size_t)(row0 + (valid ? row : 0)) * d + e0);
+    load_row<EPL>(xv, x + (size_t)(row0 + (valid ? row : 0)) * d + e0);
 #pragma unroll
     for (int p = 0; p < EPL; ++p) {
         if (!valid) xv[p] = 0.0f;
@@ -528,13 +567,13 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
     // needs), bias and alpha at the start of their own stack (needed after the transform)
     float dv[EPL], bv[EPL], av[EPL];
     int s = wave;
-    if (s < S) load_vec<EPL>(dv, D + (size_t)s * d + e0);
+    if (s < S) load_row<EPL>(dv, D + (size_t)s * d + e0);
     for (; s < S; s += SORF_WAVES) {
         const size_t off = (size_t)s * d + e0;               // the same for the four rows
-        load_vec<EPL>(bv, bias + off);
-        load_vec<EPL>(av, alpha + off);
+        load_row<EPL>(bv, bias + off);
+        load_row<EPL>(av, alpha + off);
         float dn[EPL];
-        load_vec<EPL>(dn, D + (size_t)(s + SORF_WAVES < S ? s + SORF_WAVES : s) * d + e0);
+        load_row<EPL>(dn, D + (size_t)(s + SORF_WAVES < S ? s + SORF_WAVES : s) * d + e0);
 
         float v[EPL];
 #pragma unroll
@@ -551,11 +590,9 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
 #pragma unroll
         for (int p = 0; p < EPL; ++p) {
             float sn, cs_;
-            int sm;
-            sincos_pi(arg[p], &sn, &cs_, &sm);
-            const float w = __int_as_float(__float_as_int(av[p]) ^ sm);
-            energy = fmaf(w, cs_, energy);
-            v[p] = w * sn;                                   // -(d E / d coefficient) / normf
+            sincos_hw(arg[p], &sn, &cs_);
+            energy = fmaf(av[p], cs_, energy);
+            v[p] = av[p] * sn;                               // -(d E / d coefficient) / normf
         }
         if (__builtin_expect(__any(amax > 32000.0f), 0)) {
             // arguments the two-term reduction cannot handle: redo those with the library routine
@@ -563,11 +600,9 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
             for (int p = 0; p < EPL; ++p) {
                 if (fabsf(arg[p]) > 32000.0f) {
                     float sn, cs_, s0, c0_;
-                    int sm;
-                    sincos_pi(arg[p], &s0, &c0_, &sm);
-                    const float w0 = __int_as_float(__float_as_int(av[p]) ^ sm);
+                    sincos_hw(arg[p], &s0, &c0_);
                     sincos_large(arg[p], &sn, &cs_);
-                    energy += av[p] * cs_ - w0 * c0_;
+                    energy += av[p] * (cs_ - c0_);
                     v[p] = av[p] * sn;
                 }
             }
@@ -585,7 +620,7 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
     if (i16 == 0) ered[wave][row] = energy;
     if constexpr (WITH_GRAD) {
 #pragma unroll
-        for (int p = 0; p < EPL; ++p) red[wave][row][e0 + p] = acc[p] * sigma;
+        for (int p = 0; p < EPL; ++p) red[wave][row][(p >> 2) * 64 + e0 + (p & 3)] = acc[p] * sigma;
     }
     __syncthreads();
     if (threadIdx.x < rows) {
@@ -613,6 +648,119 @@ __global__ void zero_tail_rows_kernel(const int* __restrict__ type_offsets, int 
     const size_t n = (size_t)(A - total) * d;
     for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (size_t)gridDim.x * blockDim.x)
         gx[(size_t)total * d + t] = 0.0f;
+}
+
+// ---- two-op contract in the 16-lane-row layout (64 <= d <= 256) ---------------------------
+// The four rows of a wavefront carry four consecutive stacks of ONE atom, so a workgroup has
+// 16 stacks in flight and every lane moves d/16 consecutive floats (16-byte accesses, a row
+// covers one contiguous d-float vector).  Eight or more independent butterfly chains per
+// lane and the next stack's operands in flight hide the memory latency that bounds a
+// one-transform-per-wavefront mapping.
+constexpr int ROWS_STACKS = SORF_WAVES * 4;   // stacks in flight per workgroup
+
+template <int LOG2D>
+__global__ __launch_bounds__(SORF_THREADS) void sorf_forward_rows_kernel(const float* __restrict__ x,
+                                                                          const float* __restrict__ D, int S, int T,
+                                                                          float scale, float* __restrict__ out) {
+    constexpr int d = 1 << LOG2D;
+    constexpr int EPL = d / 16;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const RowLanes<EPL> L(lane);
+    const size_t a = blockIdx.x;
+    float xv[EPL];
+    load_row<EPL>(xv, x + a * d + L.e0);
+    const int step = ROWS_STACKS * gridDim.y;
+    const float fin = scale * L.sigma;
+    int sb = blockIdx.y * ROWS_STACKS + wave * 4;          // first stack of this wavefront's four
+    if (sb >= S) return;
+    int s = min(sb + L.row, S - 1);
+    float dv[EPL];
+    load_row<EPL>(dv, D + (size_t)s * d + L.e0);
+    for (; sb < S; sb += step) {
+        const bool live = sb + L.row < S;
+        const int sn = min(sb + step + L.row, S - 1);
+        float dn[EPL];
+        load_row<EPL>(dn, D + (size_t)sn * d + L.e0);       // first diagonal of the next round
+        float v[EPL];
+#pragma unroll
+        for (int p = 0; p < EPL; ++p) v[p] = xv[p] * dv[p];
+        register_stages<EPL>(v);
+        row_stages<EPL>(v, L.cs);
+        for (int m = 1; m < T; ++m) {
+            float dm[EPL];
+            load_row<EPL>(dm, D + ((size_t)m * S + s) * d + L.e0);
+#pragma unroll
+            for (int p = 0; p < EPL; ++p) v[p] *= dm[p] * L.sigma;
+            register_stages<EPL>(v);
+            row_stages<EPL>(v, L.cs);
+        }
+#pragma unroll
+        for (int p = 0; p < EPL; ++p) v[p] *= fin;
+        if (live) store_row<EPL>(v, out + (a * S + s) * d + L.e0);
+        s = sn;
+#pragma unroll
+        for (int p = 0; p < EPL; ++p) dv[p] = dn[p];
+    }
+}
+
+template <int LOG2D>
+__global__ __launch_bounds__(SORF_THREADS) void sorf_adjoint_rows_kernel(const float* __restrict__ g,
+                                                                          const float* __restrict__ D, int S, int T,
+                                                                          float scale, float* __restrict__ gx) {
+    constexpr int d = 1 << LOG2D;
+    constexpr int EPL = d / 16;
+    __shared__ float red[ROWS_STACKS][d];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const RowLanes<EPL> L(lane);
+    const size_t a = blockIdx.x;
+    float acc[EPL];
+#pragma unroll
+    for (int p = 0; p < EPL; ++p) acc[p] = 0.0f;
+    int sb = wave * 4;
+    if (sb < S) {
+        int s = min(sb + L.row, S - 1);
+        float v[EPL], dv[EPL];
+        load_row<EPL>(v, g + (a * S + s) * d + L.e0);
+        load_row<EPL>(dv, D + ((size_t)(T - 1) * S + s) * d + L.e0);
+        for (; sb < S; sb += ROWS_STACKS) {
+            const bool live = sb + L.row < S;
+            const int sn = min(sb + ROWS_STACKS + L.row, S - 1);
+            float vn[EPL], dn[EPL];
+            load_row<EPL>(vn, g + (a * S + sn) * d + L.e0);
+            load_row<EPL>(dn, D + ((size_t)(T - 1) * S + sn) * d + L.e0);
+            register_stages<EPL>(v);
+            row_stages<EPL>(v, L.cs);
+            for (int m = T - 1; m > 0; --m) {
+                // v <- true value of diag(D[m]) H v, then the next transform
+#pragma unroll
+                for (int p = 0; p < EPL; ++p) v[p] *= dv[p] * L.sigma;
+                load_row<EPL>(dv, D + ((size_t)(m - 1) * S + s) * d + L.e0);
+                register_stages<EPL>(v);
+                row_stages<EPL>(v, L.cs);
+            }
+            if (live) {
+#pragma unroll
+                for (int p = 0; p < EPL; ++p) acc[p] = fmaf(v[p], dv[p], acc[p]);
+            }
+            s = sn;
+#pragma unroll
+            for (int p = 0; p < EPL; ++p) {
+                v[p] = vn[p];
+                dv[p] = dn[p];
+            }
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < EPL; ++p) red[wave * 4 + L.row][(p >> 2) * 64 + L.e0 + (p & 3)] = acc[p] * L.sigma;
+    __syncthreads();
+    for (int e = threadIdx.x; e < d; e += SORF_THREADS) {
+        float t = 0.0f;
+#pragma unroll
+        for (int w = 0; w < ROWS_STACKS; ++w) t += red[w][e];
+        gx[a * d + e] = scale * t;
+    }
 }
 
 // ---- derivative (force) features ----------------------------------------------------
@@ -736,8 +884,11 @@ __device__ __forceinline__ void load_f(float (&v)[V], const float* p) {
 template <typename OutT, int V>
 __global__ __launch_bounds__(CF_THREADS) void cos_features_kernel(const float* __restrict__ coeffs,
                                                                    const float* __restrict__ bias,
-                                                                   const int* __restrict__ mol_index, int A, int F,
+                                                                   const int* __restrict__ mol_index,
+                                                                   const int* __restrict__ seg, int A, int F,
                                                                    int nmol, float normf, OutT* __restrict__ Zf) {
+    // with a segment table this kernel only runs when the table is flagged invalid
+    if (seg != nullptr && seg[nmol + 1] == 0) return;
     const int f = (blockIdx.y * CF_THREADS + threadIdx.x) * V;
     if (f >= F) return;
     const int a0 = blockIdx.x * CF_ATOMS;
@@ -784,6 +935,63 @@ __global__ __launch_bounds__(CF_THREADS) void cos_features_kernel(const float* _
     }
 }
 
+// Offsets of the molecule segments of a molecule-major atom list: seg[m] = first atom whose
+// molecule index is >= m (seg[nmol] = A).  seg[nmol+1] is raised when the list is not
+// ascending or holds an index outside [0,nmol): the segments are then meaningless.  The
+// caller zero-fills seg; one thread per boundary (A+1 of them) writes the entries it owns.
+__global__ void segment_offsets_kernel(const int* __restrict__ mol_index, int A, int nmol, int* __restrict__ seg) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t > A) return;
+    const int prev = t == 0 ? -1 : mol_index[t - 1];
+    const int cur = t == A ? nmol : mol_index[t];
+    if (prev > cur || cur < 0 || cur > nmol || (t < A && cur == nmol)) {
+        seg[nmol + 1] = 1;
+        return;
+    }
+    for (int m = prev + 1; m <= cur; ++m) seg[m] = t;
+}
+
+// Segmented, atomic-free cos features for molecule-major atoms: workgroup = (molecule,
+// feature tile); the molecule's atoms are streamed with four rows in flight, summed in
+// registers in atom order and added into Zf once (each Zf element has one owner).  Does
+// nothing when the segment table is flagged invalid; the atomic kernel then does the work.
+template <typename OutT, int V>
+__global__ __launch_bounds__(CF_THREADS) void cos_features_seg_kernel(const float* __restrict__ coeffs,
+                                                                       const float* __restrict__ bias,
+                                                                       const int* __restrict__ seg, int F, int nmol,
+                                                                       float normf, OutT* __restrict__ Zf) {
+    if (seg[nmol + 1] != 0) return;
+    const int mol = blockIdx.x;
+    const int f = (blockIdx.y * CF_THREADS + threadIdx.x) * V;
+    const int a0 = seg[mol], a1 = seg[mol + 1];
+    if (f >= F || a1 <= a0) return;
+    float b[V];
+    load_f<V>(b, bias + f);
+    OutT run[V];
+#pragma unroll
+    for (int q = 0; q < V; ++q) run[q] = 0;
+    constexpr int U = 4;
+    for (int a = a0; a < a1; a += U) {
+        float c[U][V];
+#pragma unroll
+        for (int u = 0; u < U; ++u) load_f<V>(c[u], coeffs + (size_t)min(a + u, a1 - 1) * F + f);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (a + u < a1) {
+#pragma unroll
+                for (int q = 0; q < V; ++q) {
+                    float sn, cs;
+                    sincos_f32(c[u][q] + b[q], &sn, &cs);
+                    run[q] += (OutT)(cs * normf);
+                }
+            }
+        }
+    }
+    OutT* z = Zf + (size_t)mol * F + f;
+#pragma unroll
+    for (int q = 0; q < V; ++q) z[q] += run[q];
+}
+
 template <int V>
 __global__ __launch_bounds__(CF_THREADS) void cos_features_backward_kernel(const float* __restrict__ gZ,
                                                                             const float* __restrict__ coeffs,
@@ -797,23 +1005,34 @@ __global__ __launch_bounds__(CF_THREADS) void cos_features_backward_kernel(const
     const int a1 = min(A, a0 + CF_ATOMS);
     float b[V];
     load_f<V>(b, bias + f);
-    for (int a = a0; a < a1; ++a) {
-        const int mol = mol_index[a];
-        float c[V], g[V], o[V];
-        load_f<V>(c, coeffs + (size_t)a * F + f);
-        if (mol >= 0 && mol < nmol) {
-            load_f<V>(g, gZ + (size_t)mol * F + f);
-        } else {
+    constexpr int U = 4;   // atoms in flight per thread
+    for (int a = a0; a < a1; a += U) {
+        float c[U][V], g[U][V];
 #pragma unroll
-            for (int q = 0; q < V; ++q) g[q] = 0.0f;
+        for (int u = 0; u < U; ++u) {
+            const int aa = min(a + u, a1 - 1);
+            const int mol = mol_index[aa];
+            load_f<V>(c[u], coeffs + (size_t)aa * F + f);
+            if (mol >= 0 && mol < nmol) {
+                load_f<V>(g[u], gZ + (size_t)mol * F + f);
+            } else {
+#pragma unroll
+                for (int q = 0; q < V; ++q) g[u][q] = 0.0f;
+            }
         }
 #pragma unroll
-        for (int q = 0; q < V; ++q) {
-            float sn, cs;
-            sincos_f32(c[q] + b[q], &sn, &cs);
-            o[q] = g[q] * -sn * normf;
+        for (int u = 0; u < U; ++u) {
+            if (a + u < a1) {
+                float o[V];
+#pragma unroll
+                for (int q = 0; q < V; ++q) {
+                    float sn, cs;
+                    sincos_f32(c[u][q] + b[q], &sn, &cs);
+                    o[q] = g[u][q] * -sn * normf;
+                }
+                store_vec<V>(o, gc + (size_t)(a + u) * F + f);
+            }
         }
-        store_vec<V>(o, gc + (size_t)a * F + f);
     }
 }
 
@@ -875,6 +1094,18 @@ extern "C" int qmll_sorf_forward(const float* x, const float* D, int A, int d, i
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(x && D && out, QMLL_ERR_INVALID, "qmll_sorf_forward: null pointer");
     const float scale = normalisation * hnorm(d, T);
+    if (d >= 64 && d <= 256) {
+        int ny = (S + ROWS_STACKS - 1) / ROWS_STACKS;
+        if (ny > 2) ny = 2;   // a workgroup streams at least half of an atom's stacks
+        const dim3 grid(A, ny);
+        switch (qmll_log2(d)) {
+            case 6: hipLaunchKernelGGL(sorf_forward_rows_kernel<6>, grid, dim3(SORF_THREADS), 0, (hipStream_t)stream, x, D, S, T, scale, out); break;
+            case 7: hipLaunchKernelGGL(sorf_forward_rows_kernel<7>, grid, dim3(SORF_THREADS), 0, (hipStream_t)stream, x, D, S, T, scale, out); break;
+            default: hipLaunchKernelGGL(sorf_forward_rows_kernel<8>, grid, dim3(SORF_THREADS), 0, (hipStream_t)stream, x, D, S, T, scale, out); break;
+        }
+        QMLL_CHECK_LAUNCH("qmll_sorf_forward");
+        return QMLL_OK;
+    }
     const int G = d >= 64 ? 1 : 64 / d;
     int ny = (S + SORF_WAVES * G - 1) / (SORF_WAVES * G);
     if (ny > 8) ny = 8;   // each wavefront streams >= S/32 stacks: keeps the x row and D hot
@@ -894,6 +1125,15 @@ extern "C" int qmll_sorf_adjoint(const float* g, const float* D, int A, int d, i
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(g && D && gx, QMLL_ERR_INVALID, "qmll_sorf_adjoint: null pointer");
     const float scale = normalisation * hnorm(d, T);
+    if (d >= 64 && d <= 256) {
+        switch (qmll_log2(d)) {
+            case 6: hipLaunchKernelGGL(sorf_adjoint_rows_kernel<6>, dim3(A), dim3(SORF_THREADS), 0, (hipStream_t)stream, g, D, S, T, scale, gx); break;
+            case 7: hipLaunchKernelGGL(sorf_adjoint_rows_kernel<7>, dim3(A), dim3(SORF_THREADS), 0, (hipStream_t)stream, g, D, S, T, scale, gx); break;
+            default: hipLaunchKernelGGL(sorf_adjoint_rows_kernel<8>, dim3(A), dim3(SORF_THREADS), 0, (hipStream_t)stream, g, D, S, T, scale, gx); break;
+        }
+        QMLL_CHECK_LAUNCH("qmll_sorf_adjoint");
+        return QMLL_OK;
+    }
 #define CALL(L) \
     hipLaunchKernelGGL(sorf_adjoint_kernel<L>, dim3(A), dim3(SORF_THREADS), 0, (hipStream_t)stream, g, D, S, T, scale, gx)
     DISPATCH_LOG2D(qmll_log2(d), CALL)
@@ -1027,38 +1267,56 @@ static dim3 feat_grid(int A, int F, int V) {
     return dim3((A + CF_ATOMS - 1) / CF_ATOMS, (F + CF_THREADS * V - 1) / (CF_THREADS * V));
 }
 
-extern "C" int qmll_cos_features_f32(const float* coeffs, const float* bias, const int* mol_index, int A, int F,
-                                     int nmol, float* Zf, qmll_stream_t stream) {
-    int rc = check_feat("qmll_cos_features_f32", A, F, nmol);
+// launches of the forward feature kernels: segmented when a segment table is given (with
+// the atomic kernel behind it for a table flagged invalid), atomic otherwise
+template <typename OutT>
+static int launch_cos_features(const char* who, const float* coeffs, const float* bias, const int* mol_index,
+                               const int* seg, int A, int F, int nmol, OutT* Zf, hipStream_t stream) {
+    int rc = check_feat(who, A, F, nmol);
     if (rc) return rc;
     if (A == 0) return QMLL_OK;
-    QMLL_REQUIRE(coeffs && bias && mol_index && Zf, QMLL_ERR_INVALID, "qmll_cos_features_f32: null pointer");
+    QMLL_REQUIRE(coeffs && bias && mol_index && Zf, QMLL_ERR_INVALID, "%s: null pointer", who);
     const float normf = sqrtf(2.0f / (float)F);
+    if (seg != nullptr && nmol > 0) {
+        // small batches take one column per thread so that the grid still fills the device
+        const bool wide = F % 4 == 0 && (long long)nmol * ((F + CF_THREADS * 4 - 1) / (CF_THREADS * 4)) >= 2048;
+        if (wide)
+            hipLaunchKernelGGL((cos_features_seg_kernel<OutT, 4>), dim3(nmol, (F + CF_THREADS * 4 - 1) / (CF_THREADS * 4)),
+                               dim3(CF_THREADS), 0, stream, coeffs, bias, seg, F, nmol, normf, Zf);
+        else
+            hipLaunchKernelGGL((cos_features_seg_kernel<OutT, 1>), dim3(nmol, (F + CF_THREADS - 1) / CF_THREADS),
+                               dim3(CF_THREADS), 0, stream, coeffs, bias, seg, F, nmol, normf, Zf);
+        QMLL_CHECK_LAUNCH(who);
+    }
     if (F % 4 == 0)
-        hipLaunchKernelGGL((cos_features_kernel<float, 4>), feat_grid(A, F, 4), dim3(CF_THREADS), 0,
-                           (hipStream_t)stream, coeffs, bias, mol_index, A, F, nmol, normf, Zf);
+        hipLaunchKernelGGL((cos_features_kernel<OutT, 4>), feat_grid(A, F, 4), dim3(CF_THREADS), 0, stream, coeffs,
+                           bias, mol_index, seg, A, F, nmol, normf, Zf);
     else
-        hipLaunchKernelGGL((cos_features_kernel<float, 1>), feat_grid(A, F, 1), dim3(CF_THREADS), 0,
-                           (hipStream_t)stream, coeffs, bias, mol_index, A, F, nmol, normf, Zf);
-    QMLL_CHECK_LAUNCH("qmll_cos_features_f32");
+        hipLaunchKernelGGL((cos_features_kernel<OutT, 1>), feat_grid(A, F, 1), dim3(CF_THREADS), 0, stream, coeffs,
+                           bias, mol_index, seg, A, F, nmol, normf, Zf);
+    QMLL_CHECK_LAUNCH(who);
     return QMLL_OK;
 }
 
-extern "C" int qmll_cos_features_f64(const float* coeffs, const float* bias, const int* mol_index, int A, int F,
-                                     int nmol, double* Zf, qmll_stream_t stream) {
-    int rc = check_feat("qmll_cos_features_f64", A, F, nmol);
-    if (rc) return rc;
-    if (A == 0) return QMLL_OK;
-    QMLL_REQUIRE(coeffs && bias && mol_index && Zf, QMLL_ERR_INVALID, "qmll_cos_features_f64: null pointer");
-    const float normf = sqrtf(2.0f / (float)F);
-    if (F % 4 == 0)
-        hipLaunchKernelGGL((cos_features_kernel<double, 4>), feat_grid(A, F, 4), dim3(CF_THREADS), 0,
-                           (hipStream_t)stream, coeffs, bias, mol_index, A, F, nmol, normf, Zf);
-    else
-        hipLaunchKernelGGL((cos_features_kernel<double, 1>), feat_grid(A, F, 1), dim3(CF_THREADS), 0,
-                           (hipStream_t)stream, coeffs, bias, mol_index, A, F, nmol, normf, Zf);
-    QMLL_CHECK_LAUNCH("qmll_cos_features_f64");
+extern "C" int qmll_segment_offsets(const int* mol_index, int A, int nmol, int* seg, qmll_stream_t stream) {
+    QMLL_REQUIRE(A >= 0 && nmol >= 0, QMLL_ERR_INVALID, "qmll_segment_offsets: bad size A=%d nmol=%d", A, nmol);
+    QMLL_REQUIRE(seg && (mol_index || A == 0), QMLL_ERR_INVALID, "qmll_segment_offsets: null pointer");
+    hipLaunchKernelGGL(segment_offsets_kernel, dim3(A / 256 + 1), dim3(256), 0, (hipStream_t)stream, mol_index, A, nmol,
+                       seg);
+    QMLL_CHECK_LAUNCH("qmll_segment_offsets");
     return QMLL_OK;
+}
+
+extern "C" int qmll_cos_features_f32(const float* coeffs, const float* bias, const int* mol_index, const int* seg,
+                                     int A, int F, int nmol, float* Zf, qmll_stream_t stream) {
+    return launch_cos_features<float>("qmll_cos_features_f32", coeffs, bias, mol_index, seg, A, F, nmol, Zf,
+                                      (hipStream_t)stream);
+}
+
+extern "C" int qmll_cos_features_f64(const float* coeffs, const float* bias, const int* mol_index, const int* seg,
+                                     int A, int F, int nmol, double* Zf, qmll_stream_t stream) {
+    return launch_cos_features<double>("qmll_cos_features_f64", coeffs, bias, mol_index, seg, A, F, nmol, Zf,
+                                       (hipStream_t)stream);
 }
 
 extern "C" int qmll_cos_features_backward(const float* gZ, const float* coeffs, const float* bias,

@@ -213,6 +213,16 @@ def sorf_adjoint(g, D, normalisation, ntransforms):
     return out
 
 
+def segment_offsets(mol_index, nmol):
+    """int32 [nmol+2]: first atom of each molecule of an ascending molecule index, then a
+    flag that is non-zero when the index is not ascending (checked on the device)."""
+    mol_index = _i32(mol_index)
+    seg = torch.zeros(int(nmol) + 2, dtype=torch.int32, device=mol_index.device)
+    check(_lib.lib().qmll_segment_offsets(_ptr(mol_index), int(mol_index.shape[0]), int(nmol), _ptr(seg), _stream()),
+          "qmll_segment_offsets")
+    return seg
+
+
 def cos_features(coeffs, bias, nmol, mol_index, out=None):
     """f32 [nmol,F] (new, zero-initialised) or accumulate into a given f32/f64 tensor."""
     _need_cuda(coeffs, "coeffs")
@@ -225,7 +235,8 @@ def cos_features(coeffs, bias, nmol, mol_index, out=None):
     if not out.is_contiguous():
         raise RuntimeError("feature matrix must be contiguous")
     fn = _lib.lib().qmll_cos_features_f64 if out.dtype == torch.float64 else _lib.lib().qmll_cos_features_f32
-    check(fn(_ptr(coeffs), _ptr(bias), _ptr(mol_index), A, F, int(out.shape[0]), _ptr(out), _stream()),
+    seg = segment_offsets(mol_index, out.shape[0]) if A > 0 else None
+    check(fn(_ptr(coeffs), _ptr(bias), _ptr(mol_index), _ptr(seg), A, F, int(out.shape[0]), _ptr(out), _stream()),
           "qmll_cos_features")
     return out
 
