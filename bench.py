@@ -302,11 +302,15 @@ def main():
     # fused kernel, algorithmic flops per atom: forward+adjoint butterflies 2*F*log2(d), D multiplies 2F,
     # scale+bias FMA 2F, one sin and one cos per feature 2F, energy FMA 2F, alpha*norm*sin 2F
     fused_flops = A * F * (2 * log2d + 10)
-    # 37.5 vector instructions per coefficient in the kernel's main loop (d = 128; counted in its ISA);
-    # plain fp32 VOP2 instructions issue at 1.0e12 wavefront-instructions/s on this GPU (measured)
+    # 26.5 vector instructions per coefficient in the kernel's main loop (d = 128; counted in its ISA):
+    # 16.5 plain fp32 (measured issue cost 2.3 clocks each), 8 DPP butterflies (4.1 clocks) and
+    # v_sin_f32 + v_cos_f32 (8.1 clocks each) = 87 SIMD clocks per wavefront-coefficient
+    simd_clocks = 1024 * 2.4e9
     kernels["sorf_energy_fused"] = {"seconds": t_fused, "bound": "valu", "TFLOPs": fused_flops / t_fused / 1e12,
                                     "sincos_per_s": A * F / t_fused,
-                                    "valu_wave_instr_per_s": 37.5 * A * F / 64 / t_fused}
+                                    "valu_wave_instr_per_s": 26.5 * A * F / 64 / t_fused,
+                                    "issue_model_clocks_per_coefficient": 87.0,
+                                    "issue_bound_frac": 87.0 * A * F / 64 / simd_clocks / t_fused}
     kernels["sorf_forward"] = {"seconds": t_sorf, "bound": "hbm", "GBs": A * (4 * d + 4 * F) / t_sorf / 1e9}
     kernels["cos_features_f32"] = {"seconds": t_cos, "bound": "hbm", "GBs": (A * 4 * F + B * 4 * F) / t_cos / 1e9}
     kernels["cos_features_backward"] = {"seconds": t_cosb, "bound": "hbm", "GBs": A * 8 * F / t_cosb / 1e9}
@@ -364,10 +368,11 @@ def main():
                     "traffic": kernels[dominant].get("traffic_bytes"),
                     "note": "fused FWHT+sincos kernel: neither HBM nor MFMA bounds it (8d bytes per atom, no "
                             "contraction); it is bound by vector instruction issue.  Algorithmic flops count one "
-                            "flop per sin and per cos, while a 1-ulp sincos costs ~19 instructions and the cross-lane "
-                            "butterflies issue at half rate, so the fraction of the fp32 FMA peak understates it: "
-                            "valu_wave_instr_per_s against the measured 1.0e12/s for plain fp32 instructions is the "
-                            "issue-rate fraction; traffic = bytes per launch from profiles/pmc_traffic.json"}
+                            "flop per sin and per cos and per butterfly add, while a butterfly across lanes issues "
+                            "at half rate and v_sin/v_cos at quarter rate, none of them an FMA, so the fraction of "
+                            "the fp32 FMA peak understates it: kernels.sorf_energy_fused.issue_bound_frac is the "
+                            "kernel's instruction mix priced at the measured issue costs, over the launch time; "
+                            "traffic = bytes per launch from profiles/pmc_traffic.json"}
     else:
         roofline = {"kernel": dominant, "bound": "valu", "achieved": kernels[dominant]["exp_per_s"] / 1e12,
                     "peak": 256 * 4 * 16 * 2.4e9 / 4 / 1e12, "unit": "Texp/s",
