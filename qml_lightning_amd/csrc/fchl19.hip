@@ -37,12 +37,14 @@ struct FchlArgs {
     int n;
     int B;
     int cap;  // capacity of the LDS neighbour arrays
+    int tcap; // capacity (entries) of the forward kernel's LDS triple table
     const float* Rs2;
     const float* Rs3;
     qmll_fchl_params p;
 };
 
-constexpr int TCH = 256;  // triples per LDS chunk
+constexpr int TCH = 256;      // smallest triple table
+constexpr int TCH_MAX = 1024; // largest (16 KB): beyond, element pairs are processed in chunks
 constexpr float PI_F = 3.14159265358979323846f;
 
 // LDS neighbour arrays of one central atom, sorted by element type (stable in j within a
@@ -266,14 +268,15 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     const int ns = a.p.nspecies, nRs2 = a.p.nRs2, nRs3 = a.p.nRs3;
     const int R = ns * nRs2 + ns * (ns + 1) * nRs3;
 
-    float* trip = smem;             // [TCH][4]: rho, K cos, K sin, -   (first: 16-byte aligned)
-    Stage s = carve(smem + 4 * TCH, a.cap, ns);
+    float* trip = smem;             // [tcap][4]: sk3 rho, K cos, K sin, -   (first: 16-byte aligned)
+    Stage s = carve(smem + 4 * a.tcap, a.cap, ns);
     float* smu = s.next;            // [cap]  mu_j
     float* sis2 = smu + a.cap;      // [cap]  log2(e) / (2 sigma_j^2)
     float* spre = sis2 + a.cap;     // [cap]  r^-d2 fc / (sigma sqrt(2pi))
     float* slnRs2 = spre + a.cap;   // [nRs2]
     float* sinvRs2 = slnRs2 + nRs2; // [nRs2]
     float* sRs3 = sinvRs2 + nRs2;   // [nRs3]
+    int* pbase = (int*)(sRs3 + nRs3);   // [ns*ns] first table entry of each element pair
 
     for (int t = lane; t < nRs2; t += QMLL_WAVE) {
         const float v = a.Rs2[t];
@@ -325,21 +328,112 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     // ---- three-body blocks ----
     const float zeta2 = 0.014383766711652736f;   // 2 exp(-pi^2 / 2)
     const float k3 = a.p.eta3 * LOG2E;
+    const float sk3 = sqrtf(k3);                 // exp(-eta3 (rho - Rs)^2) = exp2(-(sk3 rho - sk3 Rs)^2)
     const int W3 = nRs3 < 64 ? nRs3 : 64;
     const int TS = 64 / W3;
     const int tsub = lane / W3, ll = lane - tsub * W3;
     constexpr int MAXLB = 4;                     // radial bins handled: up to 4 x 64
+
+    // one table entry per triple: (sk3 rho, K cos, K sin, -)
+    auto table_entry = [&](int j, int k) -> float4 {
+        const Triple t = triple_geometry(s, j, k);
+        const float ksi = a.p.three_body_weight * (1.0f + 3.0f * t.ci * t.cj * t.ck) *
+                          fexp2(-a.p.three_body_decay * flog2(t.a * t.b * t.c));
+        const float f = zeta2 * ksi * s.fc[j] * s.fc[k];
+        return make_float4(sk3 * 0.5f * (t.a + t.b), f * t.cosT, f * t.sinT, 0.0f);
+    };
+    // bin sums of `count` table entries starting at `first`, added to the accumulators
+    auto accumulate = [&](int first, int count, float (&accc)[MAXLB], float (&accs)[MAXLB]) {
+        if (tsub >= TS) return;
+#pragma unroll
+        for (int b = 0; b < MAXLB; ++b) {
+            const int l = b * 64 + ll;
+            if (b * 64 < nRs3 && l < nRs3) {
+                const float rs = sk3 * sRs3[l];
+                float c_ = accc[b], s_ = accs[b];
+                for (int tt = tsub; tt < count; tt += TS) {
+                    const float4 v = *reinterpret_cast<const float4*>(trip + (first + tt) * 4);
+                    const float d = v.x - rs;
+                    const float e = fexp2(-d * d);
+                    c_ = fmaf(e, v.y, c_);
+                    s_ = fmaf(e, v.z, s_);
+                }
+                accc[b] = c_;
+                accs[b] = s_;
+            }
+        }
+    };
+    // fold the triple sub-slots and store the block of pair (p,q)
+    auto store_block = [&](int sbase, const float (&accc)[MAXLB], const float (&accs)[MAXLB]) {
+#pragma unroll
+        for (int b = 0; b < MAXLB; ++b) {
+            if (b * 64 < nRs3) {
+                float tc = accc[b], tsn = accs[b];
+                for (int k = 1; k < TS; ++k) {
+                    tc += __shfl(accc[b], ll + W3 * k, 64);
+                    tsn += __shfl(accs[b], ll + W3 * k, 64);
+                }
+                const int l = b * 64 + ll;
+                if (tsub == 0 && l < nRs3) {
+                    out[sbase + 2 * l] = tc;
+                    out[sbase + 2 * l + 1] = tsn;
+                }
+            }
+        }
+    };
+
+    const int ntrip = nn * (nn - 1) / 2;
+    if (ntrip <= a.tcap) {
+        // All triples at once (three passes of 64 lanes at 20 neighbours instead of one or
+        // more per element pair): the table is ordered by element pair, pbase[p*ns+q] is
+        // the first entry of pair (p<=q), and a triple's slot follows from its position in
+        // the sorted list.
+        if (lane == 0) {
+            int acc = 0;
+            for (int p = 0; p < ns; ++p) {
+                const int np_ = s.goff[p + 1] - s.goff[p];
+                for (int q = p; q < ns; ++q) {
+                    pbase[p * ns + q] = acc;
+                    acc += (p == q) ? np_ * (np_ - 1) / 2 : np_ * (s.goff[q + 1] - s.goff[q]);
+                }
+            }
+        }
+        __syncthreads();
+        for (int tt = lane; tt < ntrip; tt += QMLL_WAVE) {
+            int j, k;
+            unrank_pair(tt, nn, j, k);
+            const int p = s.el[j], q = s.el[k];           // p <= q: the list is sorted by type
+            const int jl = j - s.goff[p], kl = k - s.goff[q];
+            const int np_ = s.goff[p + 1] - s.goff[p], nq = s.goff[q + 1] - s.goff[q];
+            const int local = (p == q) ? (jl * (2 * np_ - jl - 1)) / 2 + (kl - jl - 1) : jl * nq + kl;
+            *reinterpret_cast<float4*>(trip + (pbase[p * ns + q] + local) * 4) = table_entry(j, k);
+        }
+        __syncthreads();
+        for (int p = 0; p < ns; ++p) {
+            const int np_ = s.goff[p + 1] - s.goff[p];
+            for (int q = p; q < ns; ++q) {
+                const int nq = s.goff[q + 1] - s.goff[q];
+                const int ntr = (p == q) ? np_ * (np_ - 1) / 2 : np_ * nq;
+                float accc[MAXLB], accs[MAXLB];
+#pragma unroll
+                for (int b = 0; b < MAXLB; ++b) accc[b] = accs[b] = 0.0f;
+                accumulate(pbase[p * ns + q], ntr, accc, accs);
+                store_block(pair_offset(p, q, ns, nRs2, nRs3), accc, accs);
+            }
+        }
+        return;
+    }
+    // more triples than the table holds: element pair by element pair, in chunks of the table
     for (int p = 0; p < ns; ++p) {
         const int op = s.goff[p], np_ = s.goff[p + 1] - op;
         for (int q = p; q < ns; ++q) {
             const int oq = s.goff[q], nq = s.goff[q + 1] - oq;
             const int ntr = (p == q) ? np_ * (np_ - 1) / 2 : np_ * nq;
-            const int sbase = pair_offset(p, q, ns, nRs2, nRs3);
             float accc[MAXLB], accs[MAXLB];
 #pragma unroll
             for (int b = 0; b < MAXLB; ++b) accc[b] = accs[b] = 0.0f;
-            for (int t0 = 0; t0 < ntr; t0 += TCH) {
-                const int nchunk = min(TCH, ntr - t0);
+            for (int t0 = 0; t0 < ntr; t0 += a.tcap) {
+                const int nchunk = min(a.tcap, ntr - t0);
                 __syncthreads();
                 for (int tt = lane; tt < nchunk; tt += QMLL_WAVE) {
                     int ja, kb;
@@ -349,50 +443,12 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
                         ja = (t0 + tt) / nq;
                         kb = (t0 + tt) - ja * nq;
                     }
-                    const int j = op + ja, k = oq + kb;
-                    const Triple t = triple_geometry(s, j, k);
-                    const float ksi = a.p.three_body_weight * (1.0f + 3.0f * t.ci * t.cj * t.ck) *
-                                      fexp2(-a.p.three_body_decay * flog2(t.a * t.b * t.c));
-                    const float f = zeta2 * ksi * s.fc[j] * s.fc[k];
-                    *reinterpret_cast<float4*>(trip + tt * 4) =
-                        make_float4(0.5f * (t.a + t.b), f * t.cosT, f * t.sinT, 0.0f);
+                    *reinterpret_cast<float4*>(trip + tt * 4) = table_entry(op + ja, oq + kb);
                 }
                 __syncthreads();
-                if (tsub < TS) {
-#pragma unroll
-                    for (int b = 0; b < MAXLB; ++b) {
-                        const int l = b * 64 + ll;
-                        if (b * 64 < nRs3 && l < nRs3) {
-                            const float rs = sRs3[l];
-                            float c_ = accc[b], s_ = accs[b];
-                            for (int tt = tsub; tt < nchunk; tt += TS) {
-                                const float4 v = *reinterpret_cast<const float4*>(trip + tt * 4);
-                                const float d = v.x - rs;
-                                const float e = fexp2(-k3 * d * d);
-                                c_ = fmaf(e, v.y, c_);
-                                s_ = fmaf(e, v.z, s_);
-                            }
-                            accc[b] = c_;
-                            accs[b] = s_;
-                        }
-                    }
-                }
+                accumulate(0, nchunk, accc, accs);
             }
-#pragma unroll
-            for (int b = 0; b < MAXLB; ++b) {
-                if (b * 64 < nRs3) {
-                    float tc = accc[b], tsn = accs[b];
-                    for (int k = 1; k < TS; ++k) {
-                        tc += __shfl(accc[b], ll + W3 * k, 64);
-                        tsn += __shfl(accs[b], ll + W3 * k, 64);
-                    }
-                    const int l = b * 64 + ll;
-                    if (tsub == 0 && l < nRs3) {
-                        out[sbase + 2 * l] = tc;
-                        out[sbase + 2 * l + 1] = tsn;
-                    }
-                }
-            }
+            store_block(pair_offset(p, q, ns, nRs2, nRs3), accc, accs);
         }
     }
 }
@@ -792,6 +848,7 @@ int fill_args(FchlArgs& a, const float* X, const int* types, const float* cell, 
     a.B = B;
     a.cap = nlist ? nn_stride : n;
     if (a.cap < 1) a.cap = 1;
+    a.tcap = TCH;
     a.Rs2 = Rs2;
     a.Rs3 = Rs3;
     a.p = *prm;
@@ -813,7 +870,11 @@ extern "C" int qmll_fchl19_forward(const float* X, const int* types, const float
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(rep != nullptr, QMLL_ERR_INVALID, "qmll_fchl19_forward: null output");
     const int R = prm->nspecies * prm->nRs2 + prm->nspecies * (prm->nspecies + 1) * prm->nRs3;
-    const size_t lds = sizeof(float) * ((size_t)(STAGE_ARRAYS + 3) * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 + 4 * TCH + 4);
+    // table for every triple of a full neighbourhood when that stays small
+    const long long alltrip = (long long)a.cap * (a.cap - 1) / 2;
+    a.tcap = alltrip <= TCH ? TCH : (alltrip <= TCH_MAX ? (int)alltrip : TCH);
+    const size_t lds = sizeof(float) * ((size_t)(STAGE_ARRAYS + 3) * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 +
+                                        4 * (size_t)a.tcap + (size_t)prm->nspecies * prm->nspecies + 4);
     QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
                  "qmll_fchl19_forward: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R, LDS_LIMIT);
     hipLaunchKernelGGL(fchl19_forward_kernel, dim3(A), dim3(64), lds, (hipStream_t)stream, a, rep);
