@@ -38,6 +38,7 @@ struct FchlArgs {
     int B;
     int cap;  // capacity of the LDS neighbour arrays
     int tcap; // capacity (entries) of the forward kernel's LDS triple table
+    int tpad; // extra entries for the zero padding between the table's segments
     const float* Rs2;
     const float* Rs3;
     qmll_fchl_params p;
@@ -94,8 +95,9 @@ __device__ __forceinline__ void min_image(float& dx, float& dy, float& dz, const
 
 // Fill the LDS neighbour arrays of atom (m,i), sorted by element type; returns the
 // neighbour count.  Neighbours whose element type is negative (charge not in `species`)
-// are dropped.  Pass 0 counts per type (lane e keeps the count of type e), pass 1 scatters
-// each neighbour to goff[type] + its rank among the earlier neighbours of that type.
+// are dropped.  Up to 64 candidates take a single pass; beyond, pass 0 counts per type (lane e
+// keeps the count of type e) and pass 1 scatters each neighbour to goff[type] + its rank among
+// the earlier neighbours of that type.
 __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i, int lane) {
     const float* Xm = a.X + (size_t)m * a.n * 3;
     const int* tm = a.types + (size_t)m * a.n;
@@ -109,6 +111,11 @@ __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i,
         }
     }
     const float xi = Xm[i * 3 + 0], yi = Xm[i * 3 + 1], zi = Xm[i * 3 + 2];
+    // atom `lane` of the molecule, fetched before the atom count is known: without a
+    // neighbour list it is this lane's candidate, and the loads overlap the count's
+    const int own = lane < a.n ? lane : 0;
+    const float xo = Xm[own * 3 + 0], yo = Xm[own * 3 + 1], zo = Xm[own * 3 + 2];
+    const int eo = tm[own];
     const float rc2 = a.p.rcut * a.p.rcut;
     const float inv_rc = 1.0f / a.p.rcut;
     const bool have_list = a.nlist != nullptr;
@@ -121,6 +128,55 @@ __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i,
     } else {
         total = a.natoms[m];
         if (total > a.n) total = a.n;
+    }
+    if (total <= QMLL_WAVE) {
+        // One candidate per lane: a single pass.  The loads below depend only on the molecule
+        // index, so they are issued together; the count of each type is the population of a
+        // ballot, known to every lane, and a lane's slot is the running start of its type
+        // plus its rank among the earlier lanes of that type.
+        const int t = lane;
+        const int j = have_list ? (t < total ? li[t] : -1) : t;
+        const bool jok = t < total && j >= 0 && j < a.n;
+        float xj = xo, yj = yo, zj = zo;
+        int e = eo;
+        if (have_list) {
+            const int jj = jok ? j : 0;
+            xj = Xm[jj * 3 + 0];
+            yj = Xm[jj * 3 + 1];
+            zj = Xm[jj * 3 + 2];
+            e = tm[jj];
+        }
+        float dx = xi - xj, dy = yi - yj, dz = zi - zj;
+        if (pbc) min_image(dx, dy, dz, c, ic);
+        const float r2 = dx * dx + dy * dy + dz * dz;
+        // a supplied list is authoritative (it may be stale on purpose, e.g. finite
+        // differences with a frozen list); only the built-in search applies the cutoff
+        const bool ok = jok && (have_list ? (r2 > 0.0f) : (r2 < rc2 && r2 > 0.0f)) && e >= 0 && e < ns;
+        int start = 0, pos = 0;
+        const unsigned long long below = (1ull << lane) - 1ull;
+        for (int ep = 0; ep < ns; ++ep) {
+            const unsigned long long mask = __ballot(ok && e == ep);
+            if (lane == 0) s.goff[ep] = start;
+            if (e == ep) pos = start + __popcll(mask & below);
+            start += __popcll(mask);
+        }
+        const int nn = start < a.cap ? start : a.cap;
+        if (lane == 0) s.goff[ns] = nn;
+        if (ok && pos < a.cap) {
+            const float r = sqrtf(r2);
+            s.dx[pos] = dx;
+            s.dy[pos] = dy;
+            s.dz[pos] = dz;
+            s.r[pos] = r;
+            // fc = (cos(pi r/rc) + 1)/2 and its r-derivative from one sine / cosine pair
+            float sn, cs;
+            sincos_hw(r * PI_F * inv_rc, &sn, &cs);
+            s.fc[pos] = 0.5f * (cs + 1.0f);
+            s.dfc[pos] = -0.5f * PI_F * inv_rc * sn;
+            s.el[pos] = e;
+            s.j[pos] = j;
+        }
+        return nn;
     }
     int mycount = 0;   // lane e: neighbours of type e seen so far
     int nn = 0;
@@ -269,7 +325,7 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     const int R = ns * nRs2 + ns * (ns + 1) * nRs3;
 
     float* trip = smem;             // [tcap][4]: sk3 rho, K cos, K sin, -   (first: 16-byte aligned)
-    Stage s = carve(smem + 4 * a.tcap, a.cap, ns);
+    Stage s = carve(smem + 4 * (a.tcap + a.tpad), a.cap, ns);
     float* smu = s.next;            // [cap]  mu_j
     float* sis2 = smu + a.cap;      // [cap]  log2(e) / (2 sigma_j^2)
     float* spre = sis2 + a.cap;     // [cap]  r^-d2 fc / (sigma sqrt(2pi))
@@ -284,6 +340,9 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
         sinvRs2[t] = 1.0f / v;
     }
     for (int t = lane; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
+    // the table starts as zero entries: the padding between its segments contributes nothing
+    for (int t = lane; t < a.tcap + a.tpad; t += QMLL_WAVE)
+        reinterpret_cast<float4*>(trip)[t] = make_float4(0.f, 0.f, 0.f, 0.f);
 
     const int nn = stage_neighbours(a, s, m, i, lane);
     __syncthreads();
@@ -342,17 +401,21 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
         const float f = zeta2 * ksi * s.fc[j] * s.fc[k];
         return make_float4(sk3 * 0.5f * (t.a + t.b), f * t.cosT, f * t.sinT, 0.0f);
     };
-    // bin sums of `count` table entries starting at `first`, added to the accumulators
+    // bin sums of `count` table entries starting at `first`, added to the accumulators.  The
+    // entries up to the next multiple of TS are zero entries, so every sub-slot runs the same
+    // number of rounds and the loop is wavefront-uniform (scalar control, unrollable).
     auto accumulate = [&](int first, int count, float (&accc)[MAXLB], float (&accs)[MAXLB]) {
-        if (tsub >= TS) return;
+        const int rounds = (count + TS - 1) / TS;
+        const float4* src = reinterpret_cast<const float4*>(trip) + first + (tsub < TS ? tsub : 0);
 #pragma unroll
         for (int b = 0; b < MAXLB; ++b) {
             const int l = b * 64 + ll;
-            if (b * 64 < nRs3 && l < nRs3) {
-                const float rs = sk3 * sRs3[l];
+            if (b * 64 < nRs3) {
+                const float rs = sk3 * sRs3[l < nRs3 ? l : 0];
                 float c_ = accc[b], s_ = accs[b];
-                for (int tt = tsub; tt < count; tt += TS) {
-                    const float4 v = *reinterpret_cast<const float4*>(trip + (first + tt) * 4);
+#pragma unroll 4
+                for (int it = 0; it < rounds; ++it) {
+                    const float4 v = src[it * TS];
                     const float d = v.x - rs;
                     const float e = fexp2(-d * d);
                     c_ = fmaf(e, v.y, c_);
@@ -394,7 +457,8 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
                 const int np_ = s.goff[p + 1] - s.goff[p];
                 for (int q = p; q < ns; ++q) {
                     pbase[p * ns + q] = acc;
-                    acc += (p == q) ? np_ * (np_ - 1) / 2 : np_ * (s.goff[q + 1] - s.goff[q]);
+                    const int ntr = (p == q) ? np_ * (np_ - 1) / 2 : np_ * (s.goff[q + 1] - s.goff[q]);
+                    acc += (ntr + TS - 1) / TS * TS;       // segments start on a multiple of TS
                 }
             }
         }
@@ -445,6 +509,8 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
                     }
                     *reinterpret_cast<float4*>(trip + tt * 4) = table_entry(op + ja, oq + kb);
                 }
+                if (lane < (nchunk + TS - 1) / TS * TS - nchunk)
+                    *reinterpret_cast<float4*>(trip + (nchunk + lane) * 4) = make_float4(0.f, 0.f, 0.f, 0.f);
                 __syncthreads();
                 accumulate(0, nchunk, accc, accs);
             }
@@ -849,6 +915,7 @@ int fill_args(FchlArgs& a, const float* X, const int* types, const float* cell, 
     a.cap = nlist ? nn_stride : n;
     if (a.cap < 1) a.cap = 1;
     a.tcap = TCH;
+    a.tpad = 0;
     a.Rs2 = Rs2;
     a.Rs3 = Rs3;
     a.p = *prm;
@@ -873,8 +940,11 @@ extern "C" int qmll_fchl19_forward(const float* X, const int* types, const float
     // table for every triple of a full neighbourhood when that stays small
     const long long alltrip = (long long)a.cap * (a.cap - 1) / 2;
     a.tcap = alltrip <= TCH ? TCH : (alltrip <= TCH_MAX ? (int)alltrip : TCH);
+    // each of the ns (ns+1)/2 segments is padded to a multiple of the triple sub-slot count
+    const int tsub_slots = prm->nRs3 < 64 ? 64 / prm->nRs3 : 1;
+    a.tpad = prm->nspecies * (prm->nspecies + 1) / 2 * (tsub_slots - 1);
     const size_t lds = sizeof(float) * ((size_t)(STAGE_ARRAYS + 3) * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 +
-                                        4 * (size_t)a.tcap + (size_t)prm->nspecies * prm->nspecies + 4);
+                                        4 * (size_t)(a.tcap + a.tpad) + (size_t)prm->nspecies * prm->nspecies + 4);
     QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
                  "qmll_fchl19_forward: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R, LDS_LIMIT);
     hipLaunchKernelGGL(fchl19_forward_kernel, dim3(A), dim3(64), lds, (hipStream_t)stream, a, rep);
