@@ -3,7 +3,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 One step = energies + forces (FCHL19 -> PCA projection -> SORF -> cos features -> E, and
--dE/dX by autograd) for the 4096-molecule C9H8O4 batch of BASELINE config 2 (21 atoms,
+-dE/dX; `model.energies_and_forces`, the body of the reference-shaped `predict_opt`; the
+differentiable `forward` + `autograd.grad` route of a TorchScript caller is timed beside
+it) for the 4096-molecule C9H8O4 batch of BASELINE config 2 (21 atoms,
 species {1,6,8}, npcas 128, nstacks 128 = 16384 features, fp32), inputs resident in HBM.
 Prints one JSON line: molecules/s, the per-kernel rooflines measured with HIP events on
 the launch stream, the time to build Z^T Z / Z^T y for 1000 such molecules with forces,
@@ -80,12 +82,7 @@ def other_configs(torch, dev):
         aid, mid, nat = data['atomIDs'], data['molIDs'], data['natom_counts']
 
         def step():
-            if not forces:
-                with torch.no_grad():
-                    return model.forward(X, Z, aid, mid, nat)
-            Xg = X.detach().requires_grad_(True)
-            E = model.forward(Xg, Z, aid, mid, nat)
-            return torch.autograd.grad(-E.sum(), Xg)[0]
+            return model.energies_and_forces(X, Z, aid, mid, nat, forces=forces)
         for _ in range(warm):
             step()
         torch.cuda.synchronize()
@@ -214,10 +211,13 @@ def main():
         torch.cuda.synchronize()
 
     def step():
+        return model.energies_and_forces(X, Z, aid, mid, nat)
+
+    def step_autograd():
         Xg = X.detach().requires_grad_(True)
-        E = model.forward(Xg, Z, aid, mid, nat)
-        Fr, = torch.autograd.grad(-E.sum(), Xg)
-        return E, Fr
+        Ea = model.forward(Xg, Z, aid, mid, nat)
+        Fa, = torch.autograd.grad(-Ea.sum(), Xg)
+        return Ea, Fa
 
     for _ in range(args.warmup):
         step()
@@ -229,6 +229,18 @@ def main():
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
     value = B * args.steps / dt
+    # the same step through forward + autograd.grad (the route of a TorchScript caller)
+    for _ in range(args.warmup):
+        step_autograd()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        Ea, Fa = step_autograd()
+    torch.cuda.synchronize()
+    ms_autograd = (time.perf_counter() - t0) / args.steps * 1e3
+    autograd_route = {"ms_per_step": ms_autograd, "molecules_per_s": B / ms_autograd * 1e3,
+                      "max_abs_diff_energy": float((Ea.detach() - E).abs().max()),
+                      "max_abs_diff_force": float((Fa - Fr).abs().max())}
 
     # ---- per-kernel timing with HIP events on the launch stream ----------------------------
     def timed(fn, iters=5):
@@ -387,6 +399,7 @@ def main():
                                "nRs2 24 nRs3 20, SORF npcas 128 x nstacks 128 = 16384 features, energies + forces",
                    "molecules_per_step": B, "atoms_per_step": A},
         "roofline": roofline,
+        "autograd_route": autograd_route,
         "kernels": kernels,
     }
     out.update(train)

@@ -269,12 +269,41 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         return torch.matmul(Ztest, alpha)
 
     @torch.jit.unused
+    def energies_and_forces(self, coordinates, charges, atomIDs, molIDs, natom_counts, cells=None, inv_cells=None,
+                            forces=True):
+        """(energies [B], forces [B,n,3] or None) for device tensors through the fused route,
+        asynchronously on the current stream.  The fused kernel returns dE/dx itself, so the
+        forces need no autograd graph: same numbers as `forward` + `autograd.grad`."""
+        norm = float(np.sqrt(self.npcas) / self.sigma)
+        alpha = self.alpha.float()
+        T = int(self.ntransforms)
+
+        def energy_fn(x, type_offsets, sorted_slots, nslots, with_grad):
+            return ops.sorf_energy_sorted(x, type_offsets, sorted_slots, self.Dmat, self.bias, alpha, norm, T, nslots,
+                                          with_grad=with_grad)
+
+        with torch.no_grad():
+            return self._direct_energy_forces(coordinates.detach(), charges, atomIDs, molIDs, natom_counts, cells,
+                                              inv_cells, forces, energy_fn)
+
+    @torch.jit.unused
     def predict_opt(self, coordinates, charges, atomIDs, molIDs, natom_counts, cells=None, inv_cells=None,
                     forces=True, print_info=False, profiler=False):
         """Energies (and forces = -dE/dX by autograd) for tensors already on the device
         (hadamard_features.py:125-179)."""
         if self.is_trained is False:
             raise RuntimeError("Error: must train the model first by calling train()!")
+        if self.fused and not profiler:
+            start = torch.cuda.Event(enable_timing=True)
+            end = torch.cuda.Event(enable_timing=True)
+            start.record()
+            result = self.energies_and_forces(coordinates, charges, atomIDs, molIDs, natom_counts, cells, inv_cells,
+                                              forces=forces)
+            end.record()
+            torch.cuda.synchronize()
+            if print_info:
+                print("prediction for", coordinates.shape[0], "molecules time: ", start.elapsed_time(end), "ms")
+            return result if forces else result[0]
         with torch.autograd.profiler.profile(enabled=profiler, use_device='cuda', with_stack=True) as prof:
             start = torch.cuda.Event(enable_timing=True)
             end = torch.cuda.Event(enable_timing=True)

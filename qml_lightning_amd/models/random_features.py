@@ -98,6 +98,22 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
         return torch.matmul(Ztest, self.alpha.float())
 
     @torch.jit.unused
+    def energies_and_forces(self, coordinates, charges, atomIDs, molIDs, natom_counts, cells=None, inv_cells=None,
+                            forces=True):
+        """(energies [B], forces [B,n,3] or None) for device tensors through the fused route,
+        asynchronously on the current stream; no autograd graph (the fused kernel returns
+        dE/dx itself)."""
+        alpha = self.alpha.float()
+
+        def energy_fn(x, type_offsets, sorted_slots, nslots, with_grad):
+            return ops.rff_energy_sorted(x, type_offsets, sorted_slots, self.W, self.b, alpha, nslots,
+                                         with_grad=with_grad)
+
+        with torch.no_grad():
+            return self._direct_energy_forces(coordinates.detach(), charges, atomIDs, molIDs, natom_counts, cells,
+                                              inv_cells, forces, energy_fn)
+
+    @torch.jit.unused
     def predict_opt(self, coordinates, charges, atomIDs, molIDs, natom_counts, zcells=None, zinv_cells=None,
                     forces=True, print_info=False, profiler=False):
         if self.is_trained is False:
@@ -105,6 +121,14 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
         start = torch.cuda.Event(enable_timing=True)
         end = torch.cuda.Event(enable_timing=True)
         start.record()
+        if self.fused:
+            result = self.energies_and_forces(coordinates, charges, atomIDs, molIDs, natom_counts, zcells, zinv_cells,
+                                              forces=forces)
+            end.record()
+            torch.cuda.synchronize()
+            if print_info:
+                print("prediction for", coordinates.shape[0], "molecules time: ", start.elapsed_time(end), "ms")
+            return result if forces else result[0]
         if forces:
             coordinates.requires_grad = True
         total_energies = self.forward(coordinates, charges, atomIDs, molIDs, natom_counts, zcells, zinv_cells)

@@ -88,6 +88,12 @@ def test_sorf_energy_and_forces_vs_oracle(case, fused):
         assert (f[mm, nat[mm]:] == 0).all()
     e_only = m.predict_opt(gX.detach().clone(), gZ, gaid, gmid, gnat, forces=False)
     close(e_only, E, REL_EF, "energies, no forces")
+    # the differentiable route (what a TorchScript caller runs): forward + autograd
+    gX2 = gX.detach().clone().requires_grad_(True)
+    e2 = m.forward(gX2, gZ, gaid, gmid, gnat)
+    f2, = torch.autograd.grad(-e2.sum(), gX2)
+    close(e2, E, REL_EF, "energies, autograd route")
+    close(f2, F, REL_EF, "forces, autograd route")
 
 
 def test_two_transforms_and_torch_ops_directly():
