@@ -5,7 +5,7 @@
 One step = energies + forces (FCHL19 -> PCA projection -> SORF -> cos features -> E, and
 -dE/dX; `model.energies_and_forces`, the body of the reference-shaped `predict_opt`; the
 differentiable `forward` + `autograd.grad` route of a TorchScript caller is timed beside
-it) for the 4096-molecule C9H8O4 batch of BASELINE config 2 (21 atoms,
+it) for the 4096-molecule C9H8O4 batch of the benchmark's second configuration (21 atoms,
 species {1,6,8}, npcas 128, nstacks 128 = 16384 features, fp32), inputs resident in HBM.
 Prints one JSON line: molecules/s, the per-kernel rooflines measured with HIP events on
 the launch stream, the time to build Z^T Z / Z^T y for 1000 such molecules with forces,
@@ -59,7 +59,7 @@ def cpu_baseline(coords, charges, weights, nsample, cores):
 
 
 def other_configs(torch, dev):
-    """Short measurements of the remaining BASELINE configurations (1, 3, 4, 5) with the
+    """Short measurements of the other benchmark configurations (1, 3, 4, 5) with the
     same step definition; reported under "other_configs", never as `value`."""
     from qml_lightning_amd.models.hadamard_features import HadamardFeaturesModel
     from qml_lightning_amd.models.random_features import RandomFourrierFeaturesModel
@@ -153,14 +153,14 @@ def main():
     ap.add_argument("--no-train", action="store_true", help="skip the Z^T Z build measurement")
     ap.add_argument("--cpu-sample", type=int, default=1024)
     ap.add_argument("--no-other-configs", action="store_true",
-                    help="skip the short measurements of BASELINE configs 1, 3, 4 and 5")
+                    help="skip the short measurements of configurations 1, 3, 4 and 5")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a plain 1 GiB read + 1 GiB write elementwise kernel (reference point for "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; run with --gpus 1 (molecules shard trivially across GPUs, "
-              "see DESIGN.md, but no multi-GPU figure is produced here)", file=sys.stderr)
+              "but no multi-GPU figure is produced here)", file=sys.stderr)
         sys.exit(2)
 
     import torch
@@ -170,7 +170,7 @@ def main():
     from qml_lightning_amd.representations.FCHL import FCHLCuda
     from qml_lightning_amd.utils import synthetic
 
-    # ---- workload (BASELINE config 2) ---------------------------------------------------
+    # ---- workload (configuration 2) ---------------------------------------------------------
     coords, charges = synthetic.fixed_composition_batch(synthetic.ASPIRIN, NMOL_PREDICT, seed=1)
     coords = [c.astype(np.float32) for c in coords]
     nrep = len(SPECIES) * 24 + len(SPECIES) * (len(SPECIES) + 1) * 20
@@ -395,7 +395,7 @@ def main():
         "value": value, "unit": "molecules/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "BASELINE config 2: 4096 x C9H8O4 (21 atoms), species {1,6,8}, FCHL19 rcut 6 "
+        "config": {"workload": "config 2: 4096 x C9H8O4 (21 atoms), species {1,6,8}, FCHL19 rcut 6 "
                                "nRs2 24 nRs3 20, SORF npcas 128 x nstacks 128 = 16384 features, energies + forces",
                    "molecules_per_step": B, "atoms_per_step": A},
         "roofline": roofline,
