@@ -68,6 +68,10 @@ CASES = {
     # 40 atoms: more neighbours than the backward kernel's per-triple table holds (its other path)
     "big_molecule": lambda: (helpers.fixed_composition_batch(np.array([6] * 14 + [1] * 20 + [8] * 6), 1, 11, box=8.0),
                              [1, 6, 8], {}),
+    # 72 atoms, up to 60 neighbours: more candidates than one wavefront pass stages and more
+    # triples (1770) than the forward kernel's table holds (its chunked path)
+    "many_atoms": lambda: (helpers.fixed_composition_batch(np.array([6] * 26 + [1] * 36 + [8] * 10), 1, 12, box=9.0),
+                           [1, 6, 8], {}),
     "short_cutoff": lambda: (helpers.fixed_composition_batch(helpers.ASPIRIN, 2, 5), [1, 6, 8],
                              {"rcut": 3.1, "nRs2": 7, "nRs3": 5}),
 }
