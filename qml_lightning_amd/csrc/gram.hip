@@ -67,8 +67,10 @@ __device__ __forceinline__ void tile_of_block(unsigned b, int nti, int ntj, int&
 template <bool SYM, bool GUARD>
 __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ Z, int M, int F, int f0, int f1,
                                                       int nti, int ntj, double* __restrict__ C) {
-    __shared__ __attribute__((aligned(16))) double sA[KB][LDS_STRIDE];
-    __shared__ __attribute__((aligned(16))) double sB[KB][LDS_STRIDE];
+    // two copies of each staged panel: the next one is written while the current one is read,
+    // one barrier per step (2 x 2 x 18 KB per workgroup, two workgroups per CU)
+    __shared__ __attribute__((aligned(16))) double sA[2][KB][LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) double sB[2][KB][LDS_STRIDE];
 
     int ti, tj;
     tile_of_block<SYM>(blockIdx.x, nti, ntj, ti, tj);
@@ -127,13 +129,13 @@ __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ 
             }
         }
     };
-    auto store_panels = [&]() {
+    auto store_panels = [&](int buf) {
         const double2_t zero = {0.0, 0.0};
-        double2_t* da = reinterpret_cast<double2_t*>(&sA[lr][lc]);
+        double2_t* da = reinterpret_cast<double2_t*>(&sA[buf][lr][lc]);
 #pragma unroll
         for (int q = 0; q < 4; ++q) da[q] = loaded_rowok ? ra[q] : zero;
         if (!same) {
-            double2_t* db = reinterpret_cast<double2_t*>(&sB[lr][lc]);
+            double2_t* db = reinterpret_cast<double2_t*>(&sB[buf][lr][lc]);
 #pragma unroll
             for (int q = 0; q < 4; ++q) db[q] = loaded_rowok ? rb[q] : zero;
         }
@@ -141,12 +143,12 @@ __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ 
 
     const int nsteps = (M + KB - 1) / KB;
     load_panels(0);
-    const double(*pa)[LDS_STRIDE] = sA;
-    const double(*pb)[LDS_STRIDE] = same ? sA : sB;
+    store_panels(0);
+    __syncthreads();
     for (int step = 0; step < nsteps; ++step) {
-        __syncthreads();                 // everyone is done reading the previous panel
-        store_panels();
-        __syncthreads();
+        const int cur = step & 1;
+        const double(*pa)[LDS_STRIDE] = sA[cur];
+        const double(*pb)[LDS_STRIDE] = same ? sA[cur] : sB[cur];
         if (step + 1 < nsteps) load_panels((step + 1) * KB);   // in flight during the MFMAs
 #pragma unroll
         for (int kk = 0; kk < KB; kk += 4) {
@@ -161,6 +163,10 @@ __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ 
                 for (int q = 0; q < 4; ++q)
                     acc[p][q] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[p], fb[q], acc[p][q], 0, 0, 0);
         }
+        // the other copy was last read in the previous step, which every wavefront left
+        // through the barrier below
+        if (step + 1 < nsteps) store_panels(cur ^ 1);
+        __syncthreads();
     }
 
     // accumulator layout of v_mfma_f64_16x16x4_f64 (measured on gfx950): register r of a
