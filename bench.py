@@ -242,6 +242,18 @@ def main():
                       "max_abs_diff_energy": float((Ea.detach() - E).abs().max()),
                       "max_abs_diff_force": float((Fa - Fr).abs().max())}
 
+    # the same batch handed over as host arrays (lists of numpy coordinates / charges): batch
+    # formatting on the host, upload over PCIe, predict, results left on the device
+    model.predict(coords[:64], charges[:64], n, forces=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(3):
+        model.predict(coords, charges, n, forces=True)
+    torch.cuda.synchronize()
+    ms_host = (time.perf_counter() - t0) / 3 * 1e3
+    from_host = {"ms_per_step": ms_host, "molecules_per_s": B / ms_host * 1e3,
+                 "includes": "format_data on the host + host-to-device copies + predict; never the headline value"}
+
     # ---- per-kernel timing with HIP events on the launch stream ----------------------------
     def timed(fn, iters=5):
         fn()
@@ -400,6 +412,7 @@ def main():
                    "molecules_per_step": B, "atoms_per_step": A},
         "roofline": roofline,
         "autograd_route": autograd_route,
+        "from_host_arrays": from_host,
         "kernels": kernels,
     }
     out.update(train)

@@ -392,13 +392,16 @@ class BaseKernel():
         zbatch = len(X)
         counts = np.array([np.asarray(x).shape[0] for x in X], dtype=np.int32)
         n = int(counts.max()) if zbatch else 0
+        # one concatenation and one scatter instead of a Python loop over molecules
+        molIDs = np.repeat(np.arange(zbatch, dtype=np.int32), counts)
+        starts = np.cumsum(counts) - counts
+        atomIDs = (np.arange(int(counts.sum()), dtype=np.int64) - np.repeat(starts, counts)).astype(np.int32)
+        flat = molIDs.astype(np.int64) * n + atomIDs
         coords = np.zeros((zbatch, n, 3), dtype=np.float32)
         charges = np.zeros((zbatch, n), dtype=np.float32)
-        for j in range(zbatch):
-            coords[j, :counts[j]] = np.asarray(X[j], dtype=np.float32)
-            charges[j, :counts[j]] = np.asarray(Q[j], dtype=np.float32)
-        molIDs = np.repeat(np.arange(zbatch, dtype=np.int32), counts)
-        atomIDs = np.concatenate([np.arange(c, dtype=np.int32) for c in counts]) if zbatch else np.zeros(0, np.int32)
+        if zbatch:
+            coords.reshape(-1, 3)[flat] = np.concatenate([np.asarray(x, dtype=np.float32).reshape(-1, 3) for x in X])
+            charges.reshape(-1)[flat] = np.concatenate([np.asarray(q, dtype=np.float32).reshape(-1) for q in Q])
         data = {
             'coordinates': torch.from_numpy(coords).to(dev),
             'charges': torch.from_numpy(charges).to(dev),
@@ -419,13 +422,12 @@ class BaseKernel():
                 energies *= self.hartree2kcalmol
             if self.subtract_self_energies():
                 se = self.self_energy.numpy()
-                for j in range(zbatch):
-                    energies[j] -= se[np.asarray(Q[j]).astype(np.int64)].sum()
+                energies -= np.bincount(molIDs, weights=se[flat_q[flat]], minlength=zbatch)
             data['energies'] = torch.from_numpy(energies).to(dev)
         if F is not None:
             forces = np.zeros((zbatch, n, 3), dtype=np.float64)
-            for j in range(zbatch):
-                forces[j, :counts[j]] = np.asarray(F[j], dtype=np.float64)
+            if zbatch:
+                forces.reshape(-1, 3)[flat] = np.concatenate([np.asarray(f, dtype=np.float64).reshape(-1, 3) for f in F])
             if self.convert_hartree2kcal():
                 forces *= self.hartree2kcalmol
             data['forces'] = torch.from_numpy(forces).to(dev)

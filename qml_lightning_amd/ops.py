@@ -23,7 +23,13 @@ _P = ctypes.c_void_p
 
 
 def _ptr(t):
-    return _P(t.data_ptr()) if t is not None else _P(0)
+    """Device address of a tensor for the C ABI (NULL for None).  A host tensor is refused
+    here, whatever the caller checked: its address handed to a kernel is a GPU memory fault."""
+    if t is None:
+        return _P(0)
+    if not t.is_cuda:
+        raise RuntimeError("expected a CUDA tensor, got one on %s" % t.device)
+    return _P(t.data_ptr())
 
 
 def _stream():
