@@ -1,4 +1,5 @@
-"""Build libqmll.so (the C-ABI HIP library) for gfx950 with hipcc, in-tree.
+"""Build, in-tree: libqmll.so (the C-ABI HIP library, hipcc for gfx950) and
+libqmll_torch.so (the TORCH_LIBRARY operator registrations over that C ABI, host C++ only).
 
     python -m qml_lightning_amd.build        # or: from qml_lightning_amd.build import build; build()
 """
@@ -9,6 +10,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libqmll.so")
+TORCH_LIB = os.path.join(HERE, "libqmll_torch.so")
 SOURCES = ["qmll_core.cpp", "neighbours.hip", "fchl19.hip", "sorf.hip", "project.hip", "rff.hip", "gram.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-munsafe-fp-atomics",
@@ -35,7 +37,26 @@ def build(verbose=True, jobs=6):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
+    build_torch_ops(verbose)
     return LIB
+
+
+def build_torch_ops(verbose=True):
+    """Compile csrc/torch_ops.cpp against the installed libtorch and link it to libqmll.so
+    (found next to it at run time through an $ORIGIN run path)."""
+    import torch
+    tdir = os.path.dirname(torch.__file__)
+    abi = int(torch.compiled_with_cxx11_abi())
+    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O2", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1",
+           "-DUSE_ROCM=1", "-D_GLIBCXX_USE_CXX11_ABI=%d" % abi,
+           "-I" + os.path.join(tdir, "include"), "-I" + os.path.join(tdir, "include", "torch", "csrc", "api", "include"),
+           "-I/opt/rocm/include", os.path.join(CSRC, "torch_ops.cpp"), "-o", TORCH_LIB,
+           "-L" + os.path.join(tdir, "lib"), "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip",
+           "-L" + HERE, "-lqmll", "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return TORCH_LIB
 
 
 def _drain(procs):

@@ -28,6 +28,8 @@ def _register_fused_op():
     if _fused_registered:
         return
     _fused_registered = True
+    if ops.OPS_BACKEND == "c++":     # libqmll_torch.so has registered these operators already
+        return
     lib = torch.library.Library("qml_lightning_sorf", "FRAGMENT")
     lib.define("sorf_energy(Tensor sub, Tensor D, Tensor bias, Tensor alpha, Tensor coeff_normalisation, "
                "Tensor ntransforms) -> (Tensor, Tensor)")

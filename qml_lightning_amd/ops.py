@@ -13,6 +13,7 @@ there is no CPU implementation.
 """
 import ctypes
 import math
+import os
 
 import torch
 
@@ -478,6 +479,8 @@ _FCHL_SIG = ("Tensor X, Tensor Z, Tensor species, Tensor atomIDs, Tensor molIDs,
 
 _registered = False
 _libs = []
+TORCH_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libqmll_torch.so")
+OPS_BACKEND = None   # "c++" (libqmll_torch.so) or "python" (the torch.library definitions below)
 
 
 def _fchl_fwd_impl(X, Z, species, atomIDs, molIDs, atom_counts, cell, inv_cell, Rs2, Rs3, eta2, eta3, two_body_decay,
@@ -510,10 +513,21 @@ def _fchl_and_derivative_impl(X, Z, species, atomIDs, molIDs, atom_counts, cell,
 
 def register_ops():
     """Define qml_lightning_fchl::* and qml_lightning_sorf::* once per process."""
-    global _registered
+    global _registered, OPS_BACKEND
     if _registered:
         return
     _registered = True
+    # The operators live in libqmll_torch.so (TORCH_LIBRARY from C++, as in the reference: low
+    # dispatch cost, usable by hosts without Python).  The definitions below do the same from
+    # Python over the same kernels; they serve when that library has not been built, when
+    # QML_LIGHTNING_AMD_PY_OPS=1 asks for them, or when QML_LIGHTNING_AMD_LIB points to another
+    # copy of libqmll.so (the C++ library is linked to the copy beside it).
+    want_python = os.environ.get("QML_LIGHTNING_AMD_PY_OPS") == "1" or "QML_LIGHTNING_AMD_LIB" in os.environ
+    if not want_python and os.path.exists(TORCH_LIB_PATH) and os.path.exists(_lib.LIB_PATH):
+        torch.ops.load_library(TORCH_LIB_PATH)
+        OPS_BACKEND = "c++"
+        return
+    OPS_BACKEND = "python"
     Library = torch.library.Library
 
     fl = Library("qml_lightning_fchl", "DEF")

@@ -79,3 +79,27 @@ def test_ops_are_registered_and_refuse_cpu_tensors():
     with pytest.raises(RuntimeError, match="CUDA tensor"):
         torch.ops.qml_lightning_sorf.get_SORF_coefficients(torch.zeros(2, 8), torch.ones(1, 2, 8), torch.tensor(1.0),
                                                            torch.tensor(1))
+
+
+def test_cpp_operator_library_registers_every_operator():
+    """libqmll_torch.so (TORCH_LIBRARY from C++, as the reference's torchscript_*.so) is what
+    `import qml_lightning_amd` loads; the Python definitions are only its stand-in."""
+    import torch
+    import qml_lightning_amd  # noqa: F401
+    from qml_lightning_amd import ops
+    if os.environ.get("QML_LIGHTNING_AMD_PY_OPS") == "1" or "QML_LIGHTNING_AMD_LIB" in os.environ:
+        pytest.skip("the Python operator definitions were asked for")
+    assert os.path.exists(ops.TORCH_LIB_PATH), "libqmll_torch.so has not been built"
+    assert ops.OPS_BACKEND == "c++"
+    for name in ("fchl_forwards", "fchl_backwards", "get_fchl_and_derivative", "get_element_types",
+                 "get_num_neighbours", "get_neighbour_list"):
+        assert hasattr(torch.ops.qml_lightning_fchl, name), name
+    for name in ("get_SORF_coefficients", "get_SORF_coefficients_backward", "get_cos_features",
+                 "get_cos_features_backward", "sorf_energy", "sorf_energy_typed", "sort_by_type", "project_typed",
+                 "project_typed_backward", "sorf_energy_sorted", "rff_energy_sorted"):
+        assert hasattr(torch.ops.qml_lightning_sorf, name), name
+    # schemas as TorchScript sees them: positional tensors, as in the reference
+    schema = str(torch.ops.qml_lightning_fchl.fchl_forwards.default._schema)
+    assert schema.count("Tensor") == 17      # 16 inputs, 1 output
+    handle = ctypes.CDLL(ops.TORCH_LIB_PATH)
+    assert handle.qmll_torch_ops_version() >= 1
