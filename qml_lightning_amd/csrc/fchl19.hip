@@ -334,17 +334,26 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     float* sRs3 = sinvRs2 + nRs2;   // [nRs3]
     int* pbase = (int*)(sRs3 + nRs3);   // [ns*ns] first table entry of each element pair
 
-    for (int t = lane; t < nRs2; t += QMLL_WAVE) {
-        const float v = a.Rs2[t];
-        slnRs2[t] = logf(v);
-        sinvRs2[t] = 1.0f / v;
-    }
-    for (int t = lane; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
+    // Global loads that do not depend on the neighbourhood are issued first and consumed after
+    // the staging, so their latency overlaps the staging's own loads.
+    const float rs2v = lane < nRs2 ? a.Rs2[lane] : 1.0f;
+    const float rs3v = lane < nRs3 ? a.Rs3[lane] : 0.0f;
     // the table starts as zero entries: the padding between its segments contributes nothing
     for (int t = lane; t < a.tcap + a.tpad; t += QMLL_WAVE)
         reinterpret_cast<float4*>(trip)[t] = make_float4(0.f, 0.f, 0.f, 0.f);
 
     const int nn = stage_neighbours(a, s, m, i, lane);
+    if (lane < nRs2) {
+        slnRs2[lane] = logf(rs2v);
+        sinvRs2[lane] = 1.0f / rs2v;
+    }
+    if (lane < nRs3) sRs3[lane] = rs3v;
+    for (int t = lane + QMLL_WAVE; t < nRs2; t += QMLL_WAVE) {
+        const float v = a.Rs2[t];
+        slnRs2[t] = logf(v);
+        sinvRs2[t] = 1.0f / v;
+    }
+    for (int t = lane + QMLL_WAVE; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
     __syncthreads();
 
     // per-neighbour two-body factors
@@ -610,20 +619,37 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
     float* gin = sRs3 + nRs3;        // [R]
     float* tab = gin + R;            // TABLE: [6][ntrip]
 
+    // Global loads that do not depend on the neighbourhood (grid tables, the incoming gradient
+    // row) are issued first and consumed after the staging, so their latency overlaps the
+    // staging's own loads.
     const float* gsrc = grad_rep + ((size_t)m * a.n + i) * R;
-    for (int t = lane; t < R; t += QMLL_WAVE) gin[t] = gsrc[t];
-    for (int t = lane; t < nRs2; t += QMLL_WAVE) {
-        const float v = a.Rs2[t];
-        slnRs2[t] = logf(v);
-        sinvRs2[t] = 1.0f / v;
-    }
-    for (int t = lane; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
+    constexpr int GREG = 8;                      // gradient values per lane held in registers
+    float gr[GREG];
+#pragma unroll
+    for (int k = 0; k < GREG; ++k) gr[k] = lane + QMLL_WAVE * k < R ? gsrc[lane + QMLL_WAVE * k] : 0.0f;
+    const float rs2v = lane < nRs2 ? a.Rs2[lane] : 1.0f;
+    const float rs3v = lane < nRs3 ? a.Rs3[lane] : 0.0f;
     for (int t = lane; t < a.cap; t += QMLL_WAVE) {
         sgx[t] = 0.0f;
         sgy[t] = 0.0f;
         sgz[t] = 0.0f;
     }
     const int nn = stage_neighbours(a, s, m, i, lane);
+#pragma unroll
+    for (int k = 0; k < GREG; ++k)
+        if (lane + QMLL_WAVE * k < R) gin[lane + QMLL_WAVE * k] = gr[k];
+    for (int t = lane + QMLL_WAVE * GREG; t < R; t += QMLL_WAVE) gin[t] = gsrc[t];
+    if (lane < nRs2) {
+        slnRs2[lane] = logf(rs2v);
+        sinvRs2[lane] = 1.0f / rs2v;
+    }
+    if (lane < nRs3) sRs3[lane] = rs3v;
+    for (int t = lane + QMLL_WAVE; t < nRs2; t += QMLL_WAVE) {
+        const float v = a.Rs2[t];
+        slnRs2[t] = logf(v);
+        sinvRs2[t] = 1.0f / v;
+    }
+    for (int t = lane + QMLL_WAVE; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
     __syncthreads();
 
     const float k3 = a.p.eta3 * LOG2E;
