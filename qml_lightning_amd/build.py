@@ -38,6 +38,7 @@ def build(verbose=True, jobs=6):
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
     build_torch_ops(verbose)
+    build_host_check(verbose)
     return LIB
 
 
@@ -69,6 +70,28 @@ def _drain(procs):
             raise RuntimeError("hipcc failed on %s" % src)
         if out.strip():
             print(out)
+
+
+
+
+def build_host_check(verbose=True):
+    """tests/cpp/run_scripted: a C++ program (libtorch only, no Python) that loads a saved model
+    through libqmll_torch.so; the GPU tests run it as a child process."""
+    import torch
+    tdir = os.path.dirname(torch.__file__)
+    src = os.path.join(os.path.dirname(HERE), "tests", "cpp", "run_scripted.cpp")
+    if not os.path.exists(src):
+        return None
+    out = os.path.splitext(src)[0]
+    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O1", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch.compiled_with_cxx11_abi()),
+           "-I" + os.path.join(tdir, "include"), "-I" + os.path.join(tdir, "include", "torch", "csrc", "api", "include"),
+           src, "-o", out, "-L" + os.path.join(tdir, "lib"), "-Wl,--no-as-needed", "-ltorch", "-ltorch_cpu", "-lc10",
+           "-ltorch_hip", "-lc10_hip", "-ldl", "-Wl,-rpath," + os.path.join(tdir, "lib")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return out
 
 
 if __name__ == "__main__":

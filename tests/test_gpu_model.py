@@ -283,3 +283,45 @@ def test_fd_helper_matches_jacobian():
     # fp32 finite differences: the reference only prints this norm; 2 % of the scale is
     # what fp32 cancellation at dx = 0.005 allows
     assert (fd - J.double()).abs().max() < 0.02 * J.abs().max()
+
+
+def test_scripted_model_runs_in_a_host_without_python(tmp_path):
+    """tests/cpp/run_scripted (libtorch only) loads libqmll_torch.so, a model file saved here and
+    a batch, and must print the energies and forces this process computes."""
+    import subprocess
+    from qml_lightning_amd import ops
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "cpp", "run_scripted")
+    if ops.OPS_BACKEND != "c++" or not os.path.exists(exe):
+        pytest.skip("needs libqmll_torch.so and tests/cpp/run_scripted (python -m qml_lightning_amd.build)")
+    species = [1, 6, 8]
+    (coords, charges) = helpers.fixed_composition_batch(helpers.ASPIRIN, 3, 1)
+    X, Z, aid, mid, nat = make_batch(coords, charges)
+    gX, gZ, gaid, gmid, gnat = inputs(X, Z, aid, mid, nat)
+
+    class Batch(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            for name, t in (("X", gX), ("Z", gZ), ("atomIDs", gaid), ("molIDs", gmid), ("atom_counts", gnat)):
+                self.register_buffer(name, t.detach().clone())
+
+        def forward(self):
+            return self.X
+
+    batch_path = os.path.join(tmp_path, "batch.pt")
+    torch.jit.script(Batch()).save(batch_path)
+    for fused in (True, False):
+        m, _ = build_sorf_model(species, 64, 8, fused=fused)
+        e0, f0 = m.predict_opt(gX.detach().clone(), gZ, gaid, gmid, gnat)
+        path = os.path.join(tmp_path, "model_%d.pt" % fused)
+        m.save_jit_model(path)
+        torch.cuda.synchronize()
+        res = subprocess.run([exe, ops.TORCH_LIB_PATH, path, batch_path], capture_output=True, text=True, timeout=300)
+        assert res.returncode == 0, res.stderr[-2000:]
+        lines = res.stdout.split()
+        ne = int(lines[1])
+        e = np.array(lines[2:2 + ne], dtype=np.float64)
+        nf = int(lines[3 + ne])
+        f = np.array(lines[4 + ne:4 + ne + nf], dtype=np.float64).reshape(f0.shape)
+        close(e, e0.detach().cpu().numpy(), 1e-6, "energies from the C++ host")
+        close(f, f0.cpu().numpy(), 1e-5, "forces from the C++ host")
