@@ -272,7 +272,8 @@ int qmll_rff_derivative_features(const float* x, const float* grad, const double
  * matmul(Ztest, alpha)) and its autograd transpose; the [atoms,F] feature matrix is never
  * written.  W f32 [ne,d,F], b f32 [ne,F], alpha f32 [F]; d is 64 or 128, F a multiple of 32.
  *   -> e_slots[sorted_slots[a]] = sqrt(2/F) sum_f alpha_f cos(x_a . W_t[:,f] + b_t[f])
- *      (only atoms a < type_offsets[ne]; the caller zero-fills the rest)
+ *      (only atoms a < type_offsets[ne]; e_slots must arrive zero-filled: the launch may
+ *      split the features in two halves that add into it)
  *   -> gx f32 [A,d] = d e / d x (rows beyond type_offsets[ne] zero; NULL = energies only) */
 int qmll_rff_energy_sorted(const float* x, const int* type_offsets, const int* sorted_slots, const float* W,
                            const float* b, const float* alpha, int A, int ne, int d, int F, float* e_slots,

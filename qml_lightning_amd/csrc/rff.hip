@@ -287,8 +287,11 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
         for (int v = 0; v < NV; ++v)
             stage[v] = *reinterpret_cast<const float4*>(Wt + (size_t)(sk + KSTEP * v) * F + f0 + sf);
     };
-    fetch(0);
-    for (int f0 = 0; f0 < F; f0 += RE_FC) {
+    // feature range of this workgroup: gridDim.y splits of F (each a multiple of RE_FC)
+    const int fsplit = F / (int)gridDim.y;
+    const int fbeg = (int)blockIdx.y * fsplit, fend = fbeg + fsplit;
+    fetch(fbeg);
+    for (int f0 = fbeg; f0 < fend; f0 += RE_FC) {
         __syncthreads();
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
@@ -303,7 +306,7 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
             sa[tid] = alpha[f0 + tid] * norm;
         }
         __syncthreads();
-        if (f0 + RE_FC < F) fetch(f0 + RE_FC);
+        if (f0 + RE_FC < fend) fetch(f0 + RE_FC);
 
         // one block of 32 features at a time
 #pragma unroll
@@ -330,7 +333,9 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     float sn, cs;
-                    sincos_f32(sacc[4 * q + e] + bq[e], &sn, &cs);
+                    const float arg = sacc[4 * q + e] + bq[e];
+                    sincos_hw(arg, &sn, &cs);
+                    if (__builtin_expect(fabsf(arg) > 32000.0f, 0)) sincos_large(arg, &sn, &cs);
                     energy = fmaf(aq[e], cs, energy);
                     sacc[4 * q + e] = -aq[e] * sn;
                 }
@@ -351,18 +356,37 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
     }
 
     energy += __shfl_xor(energy, 32, 64);
-    if (h == 0 && aok) e_slots[sorted_slots[row0 + arow]] = energy;
-    if constexpr (WITH_GRAD) {
-        if (aok) {
-            float* gr = gx + (size_t)(row0 + arow) * D;
+    if (gridDim.y == 1) {
+        if (h == 0 && aok) e_slots[sorted_slots[row0 + arow]] = energy;
+        if constexpr (WITH_GRAD) {
+            if (aok) {
+                float* gr = gx + (size_t)(row0 + arow) * D;
 #pragma unroll
-            for (int blk = 0; blk < D / 32; ++blk)
+                for (int blk = 0; blk < D / 32; ++blk)
 #pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    *reinterpret_cast<float4*>(gr + 32 * blk + 8 * q + 4 * h) =
-                        make_float4(gacc[blk][4 * q], gacc[blk][4 * q + 1], gacc[blk][4 * q + 2], gacc[blk][4 * q + 3]);
+                    for (int q = 0; q < 4; ++q)
+                        *reinterpret_cast<float4*>(gr + 32 * blk + 8 * q + 4 * h) =
+                            make_float4(gacc[blk][4 * q], gacc[blk][4 * q + 1], gacc[blk][4 * q + 2], gacc[blk][4 * q + 3]);
+            }
+        }
+    } else {
+        // two feature halves add into zero-filled outputs: a sum of two terms does not depend
+        // on their order, so the result stays reproducible
+        if (h == 0 && aok) atomicAdd(&e_slots[sorted_slots[row0 + arow]], energy);
+        if constexpr (WITH_GRAD) {
+            if (aok) {
+                float* gr = gx + (size_t)(row0 + arow) * D;
+#pragma unroll
+                for (int blk = 0; blk < D / 32; ++blk)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) atomicAdd(gr + 32 * blk + 8 * (r / 4) + 4 * h + (r % 4), gacc[blk][r]);
+            }
         }
     }
+}
+
+__global__ void zero_fill_kernel(float* __restrict__ p, size_t n) {
+    for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (size_t)gridDim.x * blockDim.x) p[t] = 0.0f;
 }
 
 // rows past the last atom of a known element carry a zero gradient
@@ -442,8 +466,18 @@ extern "C" int qmll_rff_energy_sorted(const float* x, const int* type_offsets, c
     QMLL_REQUIRE((((uintptr_t)x | (uintptr_t)W | (uintptr_t)gx) & 15) == 0, QMLL_ERR_INVALID,
                  "qmll_rff_energy_sorted: x, W and gx must be 16-byte aligned");
     const float norm = sqrtf(2.0f / (float)F);
-    const dim3 grid((A + RE_M - 1) / RE_M + ne);
     hipStream_t st = (hipStream_t)stream;
+    // Two workgroups fit a CU (two wavefronts per SIMD): when the tiles fill the last round of
+    // those slots badly, the features are split in two halves over twice the workgroups, which
+    // add their energies and gradients into zero-filled outputs.
+    const int tiles = (A + RE_M - 1) / RE_M, slots = 2 * 256;
+    auto fill = [&](int k) { return (double)tiles * k / (double)(((long long)tiles * k + slots - 1) / slots * slots); };
+    const int fs = (F % (2 * RE_FC) == 0 && fill(2) > fill(1) + 0.05) ? 2 : 1;
+    const dim3 grid(tiles + ne, fs);
+    if (fs > 1 && gx) {
+        hipLaunchKernelGGL(zero_fill_kernel, dim3(1024), dim3(256), 0, st, gx, (size_t)A * d);
+        QMLL_CHECK_LAUNCH("qmll_rff_energy_sorted");
+    }
 #define CALL(DD)                                                                                                     \
     if (gx)                                                                                                          \
         hipLaunchKernelGGL((rff_energy_sorted_kernel<DD, true>), grid, dim3(RE_T), 0, st, x, type_offsets, sorted_slots, \
