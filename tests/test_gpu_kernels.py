@@ -248,6 +248,24 @@ def test_cos_features_unsorted_molecule_index(F):
     close(ops.sin_coeffs(t32(c), t32(b), out), sorf.sin_coeffs(carg, np.zeros(F)), REL_REP, "sin coeffs, odd sizes")
 
 
+def test_segment_offsets_table_and_validity_flag():
+    """Segment table of an ascending molecule index (== numpy searchsorted); the flag in the
+    last entry is raised for an index that is not ascending or leaves [0, nmol)."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(8)
+    for nmol, A in ((1, 5), (7, 40), (300, 2500), (50, 3)):       # the last: mostly empty molecules
+        idx = np.sort(rng.integers(0, nmol, A)).astype(np.int32)
+        seg = ops.segment_offsets(ti32(idx), nmol).cpu().numpy()
+        assert seg[nmol + 1] == 0
+        assert (seg[:nmol + 1] == np.searchsorted(idx, np.arange(nmol + 1), side="left")).all()
+    idx = np.array([0, 1, 1, 3, 2, 4], dtype=np.int32)            # not ascending
+    assert ops.segment_offsets(ti32(idx), 5).cpu().numpy()[6] != 0
+    idx = np.array([0, 1, 5], dtype=np.int32)                     # 5 is outside [0, 5)
+    assert ops.segment_offsets(ti32(idx), 5).cpu().numpy()[6] != 0
+    idx = np.array([-1, 0, 1], dtype=np.int32)
+    assert ops.segment_offsets(ti32(idx), 5).cpu().numpy()[6] != 0
+
+
 @pytest.mark.parametrize("d,S,T", [(16, 3, 1), (128, 8, 1), (64, 4, 2), (256, 4, 1)])
 def test_derivative_features(d, S, T):
     from qml_lightning_amd import ops
