@@ -96,6 +96,32 @@ def test_sorf_energy_and_forces_vs_oracle(case, fused):
     close(f2, F, REL_EF, "forces, autograd route")
 
 
+def test_periodic_cell_energy_and_forces_both_routes():
+    """Minimum-image neighbours through the whole model: `predict_opt` (no autograd graph) and
+    `forward` + autograd against the oracle."""
+    species = [1, 8]
+    rng = np.random.default_rng(8)
+    cellm = np.array([[5.0, 0.0, 0.0], [0.5, 5.2, 0.0], [0.2, 0.3, 4.9]]).T.astype(np.float32).astype(np.float64)
+    inv = np.linalg.inv(cellm).astype(np.float32).astype(np.float64)
+    coords = [helpers.random_geometry(rng, 6, 4.8, 1.2), helpers.random_geometry(rng, 5, 4.8, 1.2)]
+    charges = [np.array([8, 1, 1, 8, 1, 1]), np.array([8, 1, 1, 1, 8])]
+    X, Z, aid, mid, nat = make_batch(coords, charges)
+    cell, icell = np.stack([cellm, cellm]), np.stack([inv, inv])
+    m, (red, D, bias, alpha) = build_sorf_model(species, 64, 4, rcut=2.4, nRs2=10, nRs3=8)
+    prm = oracle_prm(species, rcut=2.4, nRs2=10, nRs3=8)
+    E, F, _ = omodel.sorf_energy_forces(X, Z, aid, mid, nat, prm, species, red, D, bias, alpha, 2.0, cell=cell,
+                                        inv_cell=icell)
+    gX, gZ, gaid, gmid, gnat = inputs(X, Z, aid, mid, nat)
+    e, f = m.predict_opt(gX, gZ, gaid, gmid, gnat, t32(cell), t32(icell))
+    close(e, E, REL_EF, "periodic energies")
+    close(f, F, REL_EF, "periodic forces")
+    gX2 = gX.detach().clone().requires_grad_(True)
+    e2 = m.forward(gX2, gZ, gaid, gmid, gnat, t32(cell), t32(icell))
+    f2, = torch.autograd.grad(-e2.sum(), gX2)
+    close(e2, E, REL_EF, "periodic energies, autograd route")
+    close(f2, F, REL_EF, "periodic forces, autograd route")
+
+
 def test_two_transforms_and_torch_ops_directly():
     """ntransforms = 2 through the registered operators, autograd included."""
     species = [1, 6]
