@@ -326,15 +326,15 @@ def main():
     # fused kernel, algorithmic flops per atom: forward+adjoint butterflies 2*F*log2(d), D multiplies 2F,
     # scale+bias FMA 2F, one sin and one cos per feature 2F, energy FMA 2F, alpha*norm*sin 2F
     fused_flops = A * F * (2 * log2d + 10)
-    # 26.5 vector instructions per coefficient in the kernel's main loop (d = 128; counted in its ISA):
-    # 16.5 plain fp32 (measured issue cost 2.3 clocks each), 8 DPP butterflies (4.1 clocks) and
-    # v_sin_f32 + v_cos_f32 (8.1 clocks each) = 87 SIMD clocks per wavefront-coefficient
+    # 23.5 vector instructions per coefficient in the kernel's main loop (d = 128; counted in its ISA):
+    # 13.5 plain fp32 (measured issue cost 2.3 clocks each), 8 DPP butterflies (4.1 clocks) and
+    # v_sin_f32 + v_cos_f32 (8.1 clocks each) = 80 SIMD clocks per wavefront-coefficient
     simd_clocks = 1024 * 2.4e9
     kernels["sorf_energy_fused"] = {"seconds": t_fused, "bound": "valu", "TFLOPs": fused_flops / t_fused / 1e12,
                                     "sincos_per_s": A * F / t_fused,
-                                    "valu_wave_instr_per_s": 26.5 * A * F / 64 / t_fused,
-                                    "issue_model_clocks_per_coefficient": 87.0,
-                                    "issue_bound_frac": 87.0 * A * F / 64 / simd_clocks / t_fused}
+                                    "valu_wave_instr_per_s": 23.5 * A * F / 64 / t_fused,
+                                    "issue_model_clocks_per_coefficient": 80.0,
+                                    "issue_bound_frac": 80.0 * A * F / 64 / simd_clocks / t_fused}
     kernels["sorf_forward"] = {"seconds": t_sorf, "bound": "hbm", "GBs": A * (4 * d + 4 * F) / t_sorf / 1e9}
     kernels["cos_features_f32"] = {"seconds": t_cos, "bound": "hbm", "GBs": (A * 4 * F + B * 4 * F) / t_cos / 1e9}
     kernels["cos_features_backward"] = {"seconds": t_cosb, "bound": "hbm", "GBs": A * 8 * F / t_cosb / 1e9}
