@@ -133,7 +133,7 @@ __global__ __launch_bounds__(PT) void typed_gemm_kernel(const float* __restrict_
                                                          const int* __restrict__ c_rows,
                                                          const int* __restrict__ offsets, int ne, int K, int N) {
     __shared__ __attribute__((aligned(16))) float sA[PM * PKS];
-    __shared__ __attribute__((aligned(16))) float sB[PN * PKS];   // BT: [PN][PKS]; else [PK][PN], rotated rows
+    __shared__ __attribute__((aligned(16))) float sB[BT ? PN * PKS : PK * PN];   // BT: [PN][PKS]; else [PK][PN], rotated rows
     int type, row0, rows;
     if (!tile_of_block(offsets, ne, blockIdx.x, type, row0, rows)) return;
     const int col0 = blockIdx.y * PN;
