@@ -127,7 +127,9 @@ __device__ __forceinline__ bool tile_of_block(const int* __restrict__ offsets, i
 // BT = false: B_type is [K,N] row-major (ldb = row length); BT = true: B_type is [N,K].
 // VEC: all leading dimensions, K and N are multiples of 4 and the bases are 16-byte aligned.
 template <bool BT, bool VEC>
-__global__ __launch_bounds__(PT) void typed_gemm_kernel(const float* __restrict__ A, int lda,
+// the forward kernel gains 15 % from a fifth wavefront per SIMD (at most 96 registers); the
+// transpose does not fit more than four
+__global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(BT ? 4 : 5))) void typed_gemm_kernel(const float* __restrict__ A, int lda,
                                                          const int* __restrict__ a_rows, const float* __restrict__ Bm,
                                                          size_t b_type_stride, int ldb, float* __restrict__ C, int ldc,
                                                          const int* __restrict__ c_rows,
@@ -219,31 +221,29 @@ __global__ __launch_bounds__(PT) void typed_gemm_kernel(const float* __restrict_
         // MFMA step s contracts k = s (lanes 0-31) and k = 16 + s (lanes 32-63) of the chunk;
         // the order of the contraction index is free, and this one lets a lane read its 16
         // A values (and, transposed, B values) as four 16-byte LDS loads
-        float af[16];
+        // four k-steps at a time: 4 A values and 2 x 4 B values live, not the whole chunk
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const float4 v = *reinterpret_cast<const float4*>(&sA[(32 * wave + i) * PKS + 16 * h + 4 * q]);
-            af[4 * q] = v.x; af[4 * q + 1] = v.y; af[4 * q + 2] = v.z; af[4 * q + 3] = v.w;
-        }
-        float bf[2][16];
+            const float4 va = *reinterpret_cast<const float4*>(&sA[(32 * wave + i) * PKS + 16 * h + 4 * q]);
+            const float af[4] = {va.x, va.y, va.z, va.w};
+            float bf[2][4];
 #pragma unroll
-        for (int jt = 0; jt < 2; ++jt) {
-            if (BT) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
+            for (int jt = 0; jt < 2; ++jt) {
+                if (BT) {
                     const float4 v = *reinterpret_cast<const float4*>(&sB[(i + 32 * jt) * PKS + 16 * h + 4 * q]);
-                    bf[jt][4 * q] = v.x; bf[jt][4 * q + 1] = v.y; bf[jt][4 * q + 2] = v.z; bf[jt][4 * q + 3] = v.w;
+                    bf[jt][0] = v.x; bf[jt][1] = v.y; bf[jt][2] = v.z; bf[jt][3] = v.w;
+                } else {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+                        bf[jt][s] = sB[(4 * q + s + 16 * h) * PN + ((i + 32 * jt + 32 * h) & 63)];
                 }
-            } else {
-#pragma unroll
-                for (int s = 0; s < 16; ++s) bf[jt][s] = sB[(s + 16 * h) * PN + ((i + 32 * jt + 32 * h) & 63)];
             }
-        }
 #pragma unroll
-        for (int s = 0; s < 16; ++s) {
+            for (int s = 0; s < 4; ++s) {
 #pragma unroll
-            for (int jt = 0; jt < 2; ++jt)
-                acc[jt] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s], bf[jt][s], acc[jt], 0, 0, 0);
+                for (int jt = 0; jt < 2; ++jt)
+                    acc[jt] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s], bf[jt][s], acc[jt], 0, 0, 0);
+            }
         }
     }
 
