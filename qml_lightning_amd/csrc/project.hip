@@ -264,12 +264,19 @@ __global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(BT ? 4 : 5))
 }
 
 // rows of real atoms whose element the model does not know get a zero gradient
+// (lane = slot; the rare untyped slots of a wavefront are then zeroed row by row by all lanes)
 __global__ __launch_bounds__(256) void zero_untyped_rows_kernel(const int* __restrict__ types, int N, int ne, int R,
                                                                 float* __restrict__ out) {
-    const int slot = blockIdx.x;
-    const int t = types[slot];
-    if (t >= 0 && t < ne) return;
-    for (int c = threadIdx.x; c < R; c += 256) out[(size_t)slot * R + c] = 0.0f;
+    const int slot = blockIdx.x * 256 + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int t = slot < N ? types[slot] : 0;
+    unsigned long long todo = __ballot(slot < N && (t < 0 || t >= ne));
+    while (todo) {
+        const int l = __ffsll((long long)todo) - 1;
+        todo &= todo - 1;
+        const size_t row = (size_t)(slot - lane + l) * R;
+        for (int c = lane; c < R; c += 64) out[row + c] = 0.0f;
+    }
 }
 
 __global__ void zero_ints_kernel(int* __restrict__ p, int n) {
@@ -337,7 +344,8 @@ extern "C" int qmll_project_typed_backward(const float* gx, const int* sorted_sl
                  "qmll_project_typed_backward: bad size A=%d N=%d ne=%d R=%d d=%d", A, N, ne, R, d);
     if (types && N > 0) {
         QMLL_REQUIRE(g_rep, QMLL_ERR_INVALID, "qmll_project_typed_backward: null pointer");
-        hipLaunchKernelGGL(zero_untyped_rows_kernel, dim3(N), dim3(256), 0, (hipStream_t)stream, types, N, ne, R, g_rep);
+        hipLaunchKernelGGL(zero_untyped_rows_kernel, dim3((N + 255) / 256), dim3(256), 0, (hipStream_t)stream, types, N, ne,
+                           R, g_rep);
         QMLL_CHECK_LAUNCH("qmll_project_typed_backward");
     }
     if (A == 0) return QMLL_OK;
