@@ -933,6 +933,95 @@ __global__ __launch_bounds__(SORF_THREADS) void derivative_features_seg_kernel(
     }
 }
 
+// The same in the 16-lane-row layout (64 <= d <= 256): the four rows of a wavefront are four
+// consecutive stacks, whose sign diagonals stay in registers for the whole molecule; every
+// lane runs d/16 independent butterfly chains with single-instruction DPP stages (28 issue
+// clocks per element instead of 60 for the one-transform-per-wavefront form), the projected
+// derivative row of an atom is loaded once for the four stacks, and the sine coefficients of
+// up to DF_AC atoms sit in registers while the 3n target rows are walked.
+template <int LOG2D>
+__global__ __launch_bounds__(SORF_THREADS) void derivative_features_rows_kernel(
+    const double* __restrict__ cos_derivs, double normalisation, const int* __restrict__ seg,
+    const float* __restrict__ input_derivative, const float* __restrict__ D, int n, int S, int T, float hscale,
+    double* __restrict__ G) {
+    constexpr int d = 1 << LOG2D;
+    constexpr int EPL = d / 16;
+    constexpr int AC = EPL >= 16 ? 4 : 8;       // atoms whose sine coefficients are held in registers
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const RowLanes<EPL> L(lane);
+    const int mol = blockIdx.x;
+    const int a0 = seg[mol], a1 = seg[mol + 1];
+    if (a1 <= a0) return;
+    const size_t F = (size_t)S * d;
+    const double scale = normalisation * (double)hscale;
+    const int step = ROWS_STACKS * gridDim.y;
+    for (int sb = blockIdx.y * ROWS_STACKS + wave * 4; sb < S; sb += step) {
+        const bool live = sb + L.row < S;
+        const int s = min(sb + L.row, S - 1);
+        float dv[EPL];
+        load_row<EPL>(dv, D + (size_t)s * d + L.e0);                 // first diagonal of the chain
+        for (int ac = a0; ac < a1; ac += AC) {
+            const int na = min(AC, a1 - ac);
+            float cdv[AC][EPL];
+#pragma unroll
+            for (int i = 0; i < AC; ++i) {
+                const double* src = cos_derivs + (size_t)(ac + min(i, na - 1)) * F + (size_t)s * d + L.e0;
+#pragma unroll
+                for (int p = 0; p < EPL; ++p)
+                    cdv[i][p] = i < na ? (float)src[(p >> 2) * 64 + (p & 3)] * L.sigma : 0.0f;   // pending sign folded in
+            }
+            for (int jx = 0; jx < 3 * n; ++jx) {
+                float acc[EPL];
+#pragma unroll
+                for (int p = 0; p < EPL; ++p) acc[p] = 0.0f;
+                bool any = false;
+#pragma unroll
+                for (int i = 0; i < AC; ++i) {
+                    if (i < na) {
+                        float v[EPL];
+                        load_row<EPL>(v, input_derivative + (((size_t)(ac + i) * n) * 3 + jx) * d + L.e0);
+                        float nz = 0.0f;
+#pragma unroll
+                        for (int p = 0; p < EPL; ++p) nz += fabsf(v[p]);
+                        if (__ballot(nz != 0.0f) != 0ull) {              // an all-zero row adds nothing
+                            any = true;
+#pragma unroll
+                            for (int p = 0; p < EPL; ++p) v[p] *= dv[p];
+                            register_stages<EPL>(v);
+                            row_stages<EPL>(v, L.cs);
+                            for (int m = 1; m < T; ++m) {
+                                float dm[EPL];
+                                load_row<EPL>(dm, D + ((size_t)m * S + s) * d + L.e0);
+#pragma unroll
+                                for (int p = 0; p < EPL; ++p) v[p] *= dm[p] * L.sigma;
+                                register_stages<EPL>(v);
+                                row_stages<EPL>(v, L.cs);
+                            }
+#pragma unroll
+                            for (int p = 0; p < EPL; ++p) acc[p] = fmaf(cdv[i][p], v[p], acc[p]);
+                        }
+                    }
+                }
+                if (any && live) {
+                    double* g = G + (((size_t)mol * n) * 3 + jx) * F + (size_t)s * d + L.e0;
+#pragma unroll
+                    for (int q = 0; q < EPL / 4; ++q) {
+                        double2* gq = reinterpret_cast<double2*>(g + q * 64);
+                        double2 lo = gq[0], hi = gq[1];
+                        lo.x += scale * (double)acc[4 * q];
+                        lo.y += scale * (double)acc[4 * q + 1];
+                        hi.x += scale * (double)acc[4 * q + 2];
+                        hi.y += scale * (double)acc[4 * q + 3];
+                        gq[0] = lo;
+                        gq[1] = hi;
+                    }
+                }
+            }
+        }
+    }
+}
+
 // ---- elementwise feature kernels ----------------------------------------------------
 // Thread = V consecutive feature columns (V = 4: 16-byte loads/stores; V = 1 when F is not
 // a multiple of 4), workgroup = (atom chunk, feature tile).  The forward kernel keeps a
@@ -1300,7 +1389,18 @@ extern "C" int qmll_derivative_features(const double* cos_derivs, double normali
     QMLL_REQUIRE(mol_index || seg_offsets, QMLL_ERR_INVALID,
                  "qmll_derivative_features: need mol_index or seg_offsets");
     const float hscale = hnorm(d, T);
-    if (seg_offsets) {
+    if (seg_offsets && d >= 64 && d <= 256) {
+        // 16 stacks in flight per workgroup; the stacks are split over enough workgroups to
+        // keep a few thousand of them in the launch
+        int ny = (4096 + nmol - 1) / nmol;
+        if (ny > (S + ROWS_STACKS - 1) / ROWS_STACKS) ny = (S + ROWS_STACKS - 1) / ROWS_STACKS;
+        const dim3 grid(nmol, ny);
+        switch (qmll_log2(d)) {
+            case 6: hipLaunchKernelGGL(derivative_features_rows_kernel<6>, grid, dim3(SORF_THREADS), 0, (hipStream_t)stream, cos_derivs, normalisation, seg_offsets, input_derivative, D, n, S, T, hscale, G); break;
+            case 7: hipLaunchKernelGGL(derivative_features_rows_kernel<7>, grid, dim3(SORF_THREADS), 0, (hipStream_t)stream, cos_derivs, normalisation, seg_offsets, input_derivative, D, n, S, T, hscale, G); break;
+            default: hipLaunchKernelGGL(derivative_features_rows_kernel<8>, grid, dim3(SORF_THREADS), 0, (hipStream_t)stream, cos_derivs, normalisation, seg_offsets, input_derivative, D, n, S, T, hscale, G); break;
+        }
+    } else if (seg_offsets) {
         const int G_ = d >= 64 ? 1 : 64 / d;
         int ny = (S + SORF_WAVES * G_ - 1) / (SORF_WAVES * G_);
         if (ny > 65535) ny = 65535;
