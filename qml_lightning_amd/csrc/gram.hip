@@ -130,14 +130,23 @@ __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ 
         }
     };
     auto store_panels = [&](int buf) {
-        const double2_t zero = {0.0, 0.0};
         double2_t* da = reinterpret_cast<double2_t*>(&sA[buf][lr][lc]);
+        double2_t* db = reinterpret_cast<double2_t*>(&sB[buf][lr][lc]);
+        if (__builtin_expect(loaded_rowok, 1)) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) da[q] = loaded_rowok ? ra[q] : zero;
-        if (!same) {
-            double2_t* db = reinterpret_cast<double2_t*>(&sB[buf][lr][lc]);
+            for (int q = 0; q < 4; ++q) da[q] = ra[q];
+            if (!same) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) db[q] = loaded_rowok ? rb[q] : zero;
+                for (int q = 0; q < 4; ++q) db[q] = rb[q];
+            }
+        } else {   // a row past the end of Z (last step only) contributes zeros
+            const double2_t zero = {0.0, 0.0};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) da[q] = zero;
+            if (!same) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) db[q] = zero;
+            }
         }
     };
 
