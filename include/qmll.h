@@ -287,6 +287,17 @@ int qmll_rff_energy_sorted(const float* x, const int* type_offsets, const int* s
  * triangles written), ZTy f64 [F] += Z^T y.  fp64 MFMA. */
 int qmll_gram_f64(const double* Z, const double* y, int M, int F, double* ZTZ, double* ZTy, qmll_stream_t stream);
 
+/* qmll_gram_f64 without its last pass: only the tiles (128 x 128) on or above the diagonal of
+ * ZTZ are accumulated; the strictly lower tiles are left as they are.  For a caller that
+ * accumulates several row batches (the loop of build_Z_components, kernel.py:93-192): add
+ * every batch with this entry, then call qmll_gram_mirror_f64 once. */
+int qmll_gram_upper_f64(const double* Z, const double* y, int M, int F, double* ZTZ, double* ZTy,
+                        qmll_stream_t stream);
+
+/* ZTZ[j,i] = ZTZ[i,j] for the tiles strictly above the diagonal: completes a matrix built with
+ * qmll_gram_upper_f64 (both triangles bit-identical). */
+int qmll_gram_mirror_f64(double* ZTZ, int F, qmll_stream_t stream);
+
 /* Feature-tiled variant (kernel.py:172-181, ntiles > 1): ZTZ_tile f64 [f1-f0, F] +=
  * Z[:, f0:f1]^T Z, ZTy f64 [F] (rows f0..f1 updated) += Z[:, f0:f1]^T y. */
 int qmll_gram_tile_f64(const double* Z, const double* y, int M, int F, int f0, int f1, double* ZTZ_tile, double* ZTy,

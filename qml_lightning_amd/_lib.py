@@ -55,6 +55,8 @@ PROTOTYPES = {
     "qmll_rff_derivative_features": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
     "qmll_rff_energy_sorted": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, P, P, P],
     "qmll_gram_f64": [P, P, c_int, c_int, P, P, P],
+    "qmll_gram_upper_f64": [P, P, c_int, c_int, P, P, P],
+    "qmll_gram_mirror_f64": [P, c_int, P],
     "qmll_gram_tile_f64": [P, P, c_int, c_int, c_int, c_int, P, P, P],
     "qmll_matmul_and_reduce": [P, P, c_int, c_int, c_int, P, P],
 }

@@ -9,8 +9,8 @@
 // each wavefront keeps a 64x64 sub-tile (4x4 MFMA tiles, 128 accumulator registers) and
 // the two 128-wide column panels of Z are staged through LDS KB rows at a time with the
 // next panel's global loads in flight during the MFMAs.  In the symmetric mode only tiles
-// on or above the diagonal are computed and the mirror image is written from the same
-// accumulators.  Algorithmic work: M*F*(F+1) flops, 8*M*F bytes read once (re-reads of a
+// on or above the diagonal are computed; the mirror image is copied by a separate pass
+// (gram_mirror_kernel), once per call or once after the caller's last batch.  Algorithmic work: M*F*(F+1) flops, 8*M*F bytes read once (re-reads of a
 // panel by the tiles of one row/column are served from L2: consecutive workgroup ids walk
 // along a tile row).
 #include "qmll_common.h"
@@ -30,50 +30,69 @@ constexpr int SUPER = 8;      // tiles per edge of a super-tile (L2 locality uni
 constexpr int NXCD = 8;       // workgroup ids go round-robin over the 8 XCDs
 
 // Workgroup id -> C tile.  Hardware deals consecutive workgroup ids to the 8 XCDs in turn
-// and every XCD has its own L2.  The tiles are grouped in super-tiles of 8x8; super-tile
-// number g (row-major over the super-tile grid, upper triangle only in the symmetric mode)
-// goes to XCD g%8, and the k-th workgroup of an XCD works on tile k%64 of that XCD's
-// (k/64)-th super-tile.  So the ~64 tiles an XCD runs at a time share 16 panels of Z, and
-// every XCD gets the same number of super-tiles.
+// and every XCD has its own L2.  The tiles are grouped in super-tiles of 8x8, dealt to the
+// XCDs round-robin; the k-th workgroup of an XCD works on tile k%64 of that XCD's (k/64)-th
+// super-tile, so the ~64 tiles an XCD runs at a time share 16 panels of Z.
+// Symmetric mode: every XCD must get the same number of REAL tiles per id range, because
+// ids are handed out in order and a full XCD holds back the ids of the others.  So the
+// super-tiles strictly above the diagonal (64 tiles each) are dealt first, then the diagonal
+// super-tiles, whose 36 tiles on or above the diagonal are numbered without gaps.
+constexpr int DIAG_TILES = SUPER * (SUPER + 1) / 2;
+
+struct TileMap {
+    int off_per;    // strictly-upper super-tiles per XCD (symmetric) / all super-tiles per XCD
+    int diag_per;   // diagonal super-tiles per XCD (symmetric mode only)
+};
+
 template <bool SYM>
-__device__ __forceinline__ void tile_of_block(unsigned b, int nti, int ntj, int& ti, int& tj) {
+__device__ __forceinline__ void tile_of_block(unsigned b, int nti, int ntj, TileMap tm, int& ti, int& tj) {
     const unsigned xcd = b % NXCD, k = b / NXCD;
-    const unsigned g = (k / (SUPER * SUPER)) * NXCD + xcd;      // super-tile number
-    const unsigned in_super = k % (SUPER * SUPER);
     const int sr_n = (nti + SUPER - 1) / SUPER, sc_n = (ntj + SUPER - 1) / SUPER;
-    int sr, sc;
-    if (SYM) {
-        // g-th super-tile of the upper triangle, rows of length sc_n - sr
-        const float bb = (float)(2 * sc_n + 1);
+    ti = tj = -1;
+    if (!SYM) {
+        const unsigned g = (k / (SUPER * SUPER)) * NXCD + xcd;
+        const unsigned in_super = k % (SUPER * SUPER);
+        const int sr = (int)(g / sc_n), sc = (int)(g % sc_n);
+        if (sr >= sr_n) return;
+        ti = sr * SUPER + (int)(in_super / SUPER);
+        tj = sc * SUPER + (int)(in_super % SUPER);
+    } else if (k < (unsigned)tm.off_per * (SUPER * SUPER)) {
+        const unsigned g = (k / (SUPER * SUPER)) * NXCD + xcd;
+        const unsigned in_super = k % (SUPER * SUPER);
+        const int n1 = sc_n - 1;                                // row r holds n1 - r super-tiles
+        if (g >= (unsigned)(sc_n * n1 / 2)) return;
+        const float bb = (float)(2 * n1 + 1);
         int r = (int)((bb - sqrtf(fmaxf(bb * bb - 8.0f * (float)g, 0.0f))) * 0.5f);
-        if (r < 0) r = 0;
-        if (r > sc_n - 1) r = sc_n - 1;
-        while (r > 0 && (unsigned)(r * sc_n - (r * (r - 1)) / 2) > g) --r;
-        while (r + 1 < sc_n && (unsigned)((r + 1) * sc_n - ((r + 1) * r) / 2) <= g) ++r;
-        sr = r;
-        sc = r + (int)(g - (unsigned)(r * sc_n - (r * (r - 1)) / 2));
-        if (sc >= sc_n) sr = sr_n;   // past the last super-tile
+        r = min(max(r, 0), n1 - 1);
+        while (r > 0 && (unsigned)(r * n1 - (r * (r - 1)) / 2) > g) --r;
+        while (r + 1 < n1 && (unsigned)((r + 1) * n1 - ((r + 1) * r) / 2) <= g) ++r;
+        const int sc = r + 1 + (int)(g - (unsigned)(r * n1 - (r * (r - 1)) / 2));
+        ti = r * SUPER + (int)(in_super / SUPER);
+        tj = sc * SUPER + (int)(in_super % SUPER);
     } else {
-        sr = (int)(g / sc_n);
-        sc = (int)(g % sc_n);
+        const unsigned k2 = k - (unsigned)tm.off_per * (SUPER * SUPER);
+        const unsigned dg = (k2 / DIAG_TILES) * NXCD + xcd;
+        if (dg >= (unsigned)sc_n) return;
+        int t = (int)(k2 % DIAG_TILES), a = 0;
+        while (t >= SUPER - a) { t -= SUPER - a; ++a; }         // row a of the triangle holds 8 - a tiles
+        ti = (int)dg * SUPER + a;
+        tj = (int)dg * SUPER + a + t;
     }
-    ti = sr * SUPER + (int)(in_super / SUPER);
-    tj = sc * SUPER + (int)(in_super % SUPER);
-    if (sr >= sr_n || ti >= nti || tj >= ntj) ti = tj = -1;
+    if (ti >= nti || tj >= ntj) ti = tj = -1;
 }
 
 // GUARD: some panel sticks out of the matrix (F or the row block not a multiple of 128, or
 // odd F): every element load is bounds-checked.  !GUARD: whole panels, 16-byte vector loads.
 template <bool SYM, bool GUARD>
 __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ Z, int M, int F, int f0, int f1,
-                                                      int nti, int ntj, double* __restrict__ C) {
+                                                      int nti, int ntj, TileMap tm, double* __restrict__ C) {
     // two copies of each staged panel: the next one is written while the current one is read,
     // one barrier per step (2 x 2 x 18 KB per workgroup, two workgroups per CU)
     __shared__ __attribute__((aligned(16))) double sA[2][KB][LDS_STRIDE];
     __shared__ __attribute__((aligned(16))) double sB[2][KB][LDS_STRIDE];
 
     int ti, tj;
-    tile_of_block<SYM>(blockIdx.x, nti, ntj, ti, tj);
+    tile_of_block<SYM>(blockIdx.x, nti, ntj, tm, ti, tj);
     if (ti < 0 || (SYM && ti > tj)) return;
     const int i0 = f0 + ti * TILE;   // first feature of the A panel (rows of C)
     const int j0 = tj * TILE;        // first feature of the B panel (columns of C)
@@ -191,14 +210,34 @@ __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ 
                 if (gi < ilim && gj < F) {
                     const double v = acc[p][q][r];
                     if (SYM) {
-                        C[(size_t)gi * F + gj] += v;
-                        if (!same) C[(size_t)gj * F + gi] += v;   // mirror of an off-diagonal tile
+                        C[(size_t)gi * F + gj] += v;               // the mirror image is a separate pass
                     } else {
                         C[(size_t)(gi - f0) * F + gj] += v;
                     }
                 }
             }
         }
+    }
+}
+
+// C[j,i] = C[i,j] for every element of the tiles strictly above the diagonal (32x32 blocks
+// transposed through LDS, both sides coalesced).  The symmetric kernel accumulates only tiles
+// on or above the diagonal; copying instead of adding twice keeps the two triangles
+// bit-identical and replaces 128-byte-strided read-modify-writes in the kernel's epilogue.
+constexpr int MT = 32;
+__global__ __launch_bounds__(256) void gram_mirror_kernel(double* __restrict__ C, int F) {
+    __shared__ double t[MT][MT + 1];
+    const int bi = blockIdx.y, bj = blockIdx.x;            // block row / column, 32 x 32 each
+    if (bi / (TILE / MT) >= bj / (TILE / MT)) return;      // only tiles strictly above the diagonal
+    const int tx = threadIdx.x % MT, ty = threadIdx.x / MT;
+    for (int r = ty; r < MT; r += 256 / MT) {
+        const int gi = bi * MT + r, gj = bj * MT + tx;
+        t[r][tx] = (gi < F && gj < F) ? C[(size_t)gi * F + gj] : 0.0;
+    }
+    __syncthreads();
+    for (int r = ty; r < MT; r += 256 / MT) {
+        const int gj = bj * MT + r, gi = bi * MT + tx;
+        if (gi < F && gj < F) C[(size_t)gj * F + gi] = t[tx][r];
     }
 }
 
@@ -243,7 +282,7 @@ __global__ __launch_bounds__(MR* MR) void matmul_and_reduce_kernel(const float* 
 
 }  // namespace
 
-static int gram_launch(const double* Z, const double* y, int M, int F, int f0, int f1, bool sym, double* C,
+static int gram_launch(const double* Z, const double* y, int M, int F, int f0, int f1, bool sym, bool mirror, double* C,
                        double* ZTy, hipStream_t stream, const char* who) {
     QMLL_REQUIRE(M >= 0 && F > 0, QMLL_ERR_INVALID, "%s: bad size M=%d F=%d", who, M, F);
     QMLL_REQUIRE(0 <= f0 && f0 < f1 && f1 <= F, QMLL_ERR_INVALID, "%s: bad feature range [%d,%d) of %d", who, f0, f1, F);
@@ -253,24 +292,37 @@ static int gram_launch(const double* Z, const double* y, int M, int F, int f0, i
                  who);
     const int ntj = (F + TILE - 1) / TILE;
     const int nti = sym ? ntj : (f1 - f0 + TILE - 1) / TILE;
-    // super-tiles are dealt round-robin to the XCDs; each owns SUPER*SUPER workgroup ids,
-    // and ids of tiles outside the matrix (or below the diagonal) exit at once
+    // super-tiles are dealt round-robin to the XCDs; ids of tiles outside the matrix exit at once
     const long long sr = (nti + SUPER - 1) / SUPER, sc = (ntj + SUPER - 1) / SUPER;
-    long long nsuper = sym ? sc * (sc + 1) / 2 : sr * sc;
-    nsuper = (nsuper + NXCD - 1) / NXCD * NXCD;
-    const long long nblocks = nsuper * SUPER * SUPER;
+    TileMap tm;
+    long long per_xcd;
+    if (sym) {
+        tm.off_per = (int)((sc * (sc - 1) / 2 + NXCD - 1) / NXCD);
+        tm.diag_per = (int)((sc + NXCD - 1) / NXCD);
+        per_xcd = (long long)tm.off_per * SUPER * SUPER + (long long)tm.diag_per * DIAG_TILES;
+    } else {
+        tm.off_per = (int)((sr * sc + NXCD - 1) / NXCD);
+        tm.diag_per = 0;
+        per_xcd = (long long)tm.off_per * SUPER * SUPER;
+    }
+    const long long nblocks = per_xcd * NXCD;
     QMLL_REQUIRE(nblocks < 2147483647LL, QMLL_ERR_INVALID, "%s: too many tiles", who);
     const bool guard = (F % TILE) != 0 || ((f1 - f0) % TILE) != 0 || (f0 % 2) != 0;
     const dim3 grid((unsigned)nblocks), block(GT);
     if (sym && !guard)
-        hipLaunchKernelGGL((gram_kernel<true, false>), grid, block, 0, stream, Z, M, F, 0, F, nti, ntj, C);
+        hipLaunchKernelGGL((gram_kernel<true, false>), grid, block, 0, stream, Z, M, F, 0, F, nti, ntj, tm, C);
     else if (sym)
-        hipLaunchKernelGGL((gram_kernel<true, true>), grid, block, 0, stream, Z, M, F, 0, F, nti, ntj, C);
+        hipLaunchKernelGGL((gram_kernel<true, true>), grid, block, 0, stream, Z, M, F, 0, F, nti, ntj, tm, C);
     else if (!guard)
-        hipLaunchKernelGGL((gram_kernel<false, false>), grid, block, 0, stream, Z, M, F, f0, f1, nti, ntj, C);
+        hipLaunchKernelGGL((gram_kernel<false, false>), grid, block, 0, stream, Z, M, F, f0, f1, nti, ntj, tm, C);
     else
-        hipLaunchKernelGGL((gram_kernel<false, true>), grid, block, 0, stream, Z, M, F, f0, f1, nti, ntj, C);
+        hipLaunchKernelGGL((gram_kernel<false, true>), grid, block, 0, stream, Z, M, F, f0, f1, nti, ntj, tm, C);
     QMLL_CHECK_LAUNCH(who);
+    if (sym && mirror) {
+        const unsigned nb = (unsigned)((F + MT - 1) / MT);
+        hipLaunchKernelGGL(gram_mirror_kernel, dim3(nb, nb), dim3(256), 0, stream, C, F);
+        QMLL_CHECK_LAUNCH(who);
+    }
     if (y) {
         dim3 grid((f1 - f0 + 255) / 256, (M + GV_ROWS - 1) / GV_ROWS);
         hipLaunchKernelGGL(gemv_t_kernel, grid, dim3(256), 0, stream, Z, y, M, F, f0, f1, ZTy);
@@ -281,12 +333,27 @@ static int gram_launch(const double* Z, const double* y, int M, int F, int f0, i
 
 extern "C" int qmll_gram_f64(const double* Z, const double* y, int M, int F, double* ZTZ, double* ZTy,
                              qmll_stream_t stream) {
-    return gram_launch(Z, y, M, F, 0, F > 0 ? F : 1, true, ZTZ, ZTy, (hipStream_t)stream, "qmll_gram_f64");
+    return gram_launch(Z, y, M, F, 0, F > 0 ? F : 1, true, true, ZTZ, ZTy, (hipStream_t)stream, "qmll_gram_f64");
+}
+
+extern "C" int qmll_gram_upper_f64(const double* Z, const double* y, int M, int F, double* ZTZ, double* ZTy,
+                                   qmll_stream_t stream) {
+    return gram_launch(Z, y, M, F, 0, F > 0 ? F : 1, true, false, ZTZ, ZTy, (hipStream_t)stream, "qmll_gram_upper_f64");
+}
+
+extern "C" int qmll_gram_mirror_f64(double* ZTZ, int F, qmll_stream_t stream) {
+    QMLL_REQUIRE(F > 0, QMLL_ERR_INVALID, "qmll_gram_mirror_f64: bad size F=%d", F);
+    QMLL_REQUIRE(ZTZ, QMLL_ERR_INVALID, "qmll_gram_mirror_f64: null pointer");
+    const unsigned nb = (unsigned)((F + MT - 1) / MT);
+    QMLL_REQUIRE(nb <= 65535, QMLL_ERR_INVALID, "qmll_gram_mirror_f64: F=%d too large", F);
+    hipLaunchKernelGGL(gram_mirror_kernel, dim3(nb, nb), dim3(256), 0, (hipStream_t)stream, ZTZ, F);
+    QMLL_CHECK_LAUNCH("qmll_gram_mirror_f64");
+    return QMLL_OK;
 }
 
 extern "C" int qmll_gram_tile_f64(const double* Z, const double* y, int M, int F, int f0, int f1, double* ZTZ_tile,
                                   double* ZTy, qmll_stream_t stream) {
-    return gram_launch(Z, y, M, F, f0, f1, false, ZTZ_tile, ZTy, (hipStream_t)stream, "qmll_gram_tile_f64");
+    return gram_launch(Z, y, M, F, f0, f1, false, false, ZTZ_tile, ZTy, (hipStream_t)stream, "qmll_gram_tile_f64");
 }
 
 extern "C" int qmll_matmul_and_reduce(const float* A, const float* B, int Ar, int K, int Bc, double* C,

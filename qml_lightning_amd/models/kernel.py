@@ -147,6 +147,7 @@ class BaseKernel():
         ZTZ = torch.zeros(nf, nf, device=torch.device('cpu') if cpu_solve else dev, dtype=torch.float64)
         ZtrainY = torch.zeros(nf, 1, device=dev, dtype=torch.float64)
         start.record()
+        mirror_pending = False
         nsub = int(np.ceil(nf / ntiles))
         for tile in range(ntiles):
             lo, hi = tile * nsub, min(nsub * (tile + 1), nf)
@@ -178,10 +179,13 @@ class BaseKernel():
                     matmul_and_reduce(r32.T.contiguous(), r32, ZTZ)
                     ZtrainY += torch.matmul(rows.T, targets)
                 else:
-                    ops.gram(rows, targets, ZTZ, ZtrainY)
+                    ops.gram(rows, targets, ZTZ, ZtrainY, mirror=False)    # upper tiles; mirrored once below
+                    mirror_pending = True
                 del rows
             if ntiles > 1:
                 ZTZ[lo:hi, :] += ZTZ_tile.cpu() if cpu_solve else ZTZ_tile
+        if mirror_pending:
+            ops.gram_mirror(ZTZ)
         end.record()
         torch.cuda.synchronize()
         if print_info:

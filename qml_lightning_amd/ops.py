@@ -442,8 +442,18 @@ def rff_energy_sorted(x, type_offsets, sorted_slots, W, b, alpha, nslots, with_g
     return e_slots, gx
 
 
-def gram(Zrows, y, ZTZ, ZTy, f0=None, f1=None):
-    """ZTZ += Z^T Z (or the row block f0:f1 of it), ZTy += Z^T y, fp64, in place."""
+def gram_mirror(ZTZ):
+    """Copy the upper triangle of ZTZ onto the lower one (after `gram(..., mirror=False)` calls)."""
+    if ZTZ.dtype != torch.float64 or not ZTZ.is_contiguous() or ZTZ.shape[0] != ZTZ.shape[1]:
+        raise RuntimeError("gram_mirror needs a contiguous square float64 matrix")
+    check(_lib.lib().qmll_gram_mirror_f64(_ptr(ZTZ), int(ZTZ.shape[0]), _stream()), "qmll_gram_mirror_f64")
+    return ZTZ
+
+
+def gram(Zrows, y, ZTZ, ZTy, f0=None, f1=None, mirror=True):
+    """ZTZ += Z^T Z (or the row block f0:f1 of it), ZTy += Z^T y, fp64, in place.
+    mirror=False (full matrix only) accumulates just the tiles on or above the diagonal: a
+    caller adding several batches finishes with one `gram_mirror(ZTZ)`."""
     if Zrows.dtype != torch.float64 or not Zrows.is_contiguous():
         raise RuntimeError("gram needs a contiguous float64 row matrix")
     M, F = Zrows.shape
@@ -454,7 +464,8 @@ def gram(Zrows, y, ZTZ, ZTy, f0=None, f1=None):
             raise RuntimeError("targets have %d rows, features have %d" % (yv.shape[0], M))
     zty = ZTy if ZTy is not None else None
     if f0 is None:
-        check(_lib.lib().qmll_gram_f64(_ptr(Zrows), _ptr(yv), M, F, _ptr(ZTZ), _ptr(zty), _stream()), "qmll_gram_f64")
+        fn = _lib.lib().qmll_gram_f64 if mirror else _lib.lib().qmll_gram_upper_f64
+        check(fn(_ptr(Zrows), _ptr(yv), M, F, _ptr(ZTZ), _ptr(zty), _stream()), "qmll_gram_f64")
     else:
         check(_lib.lib().qmll_gram_tile_f64(_ptr(Zrows), _ptr(yv), M, F, int(f0), int(f1), _ptr(ZTZ), _ptr(zty),
                                             _stream()), "qmll_gram_tile_f64")

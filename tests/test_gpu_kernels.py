@@ -423,7 +423,7 @@ def test_sorted_fused_energy_matches_per_atom_oracle():
 
 
 # ---------------------------------------------------------------------------------------
-@pytest.mark.parametrize("M,F", [(37, 24), (300, 128), (1000, 384), (513, 200)])
+@pytest.mark.parametrize("M,F", [(37, 24), (300, 128), (1000, 384), (513, 200), (40, 2176), (33, 3000), (20, 4224)])
 def test_gram_matches_fp64_matmul(M, F):
     from qml_lightning_amd import ops
     rng = np.random.default_rng(M)
@@ -450,6 +450,29 @@ def test_gram_matches_fp64_matmul(M, F):
         full[lo:hi] = tile
     close(full, Zr.T @ Zr, 1e-13, "tiled ZTZ")
     close(zty, Zr.T @ y, 1e-13, "tiled ZTy")
+
+
+@pytest.mark.parametrize("F", [200, 384])
+def test_gram_upper_batches_then_one_mirror(F):
+    """Two row batches added with the upper-tile entry and mirrored once equal two full calls bit for bit."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(F)
+    batches = [torch.tensor(rng.normal(size=(m, F)), device=dev()) for m in (130, 77)]
+    ys = [torch.tensor(rng.normal(size=(b.shape[0], 1)), device=dev()) for b in batches]
+    full = torch.zeros(F, F, dtype=torch.float64, device=dev())
+    fy = torch.zeros(F, 1, dtype=torch.float64, device=dev())
+    up = torch.full((F, F), 7.0, dtype=torch.float64, device=dev()).tril(-128).contiguous()   # junk below the tiles
+    uy = torch.zeros(F, 1, dtype=torch.float64, device=dev())
+    for b, y in zip(batches, ys):
+        ops.gram(b, y, full, fy)
+        ops.gram(b, y, up, uy, mirror=False)
+    lower_tiles = torch.ones(F, F, device=dev()).tril(-1).bool() & \
+        ((torch.arange(F, device=dev())[:, None] // 128) > (torch.arange(F, device=dev())[None, :] // 128))
+    assert (up[lower_tiles] == 7.0).sum() > 0              # untouched until mirrored
+    ops.gram_mirror(up)
+    assert torch.equal(up, full) and torch.equal(uy, fy)
+    ref = sum(b.cpu().numpy().T @ b.cpu().numpy() for b in batches)
+    close(up, ref, 1e-13, "batched ZTZ")
 
 
 def test_matmul_and_reduce_is_the_reference_kahan_sum():
