@@ -298,6 +298,24 @@ int qmll_gram_upper_f64(const double* Z, const double* y, int M, int F, double* 
  * qmll_gram_upper_f64 (both triangles bit-identical). */
 int qmll_gram_mirror_f64(double* ZTZ, int F, qmll_stream_t stream);
 
+/* ---- regularised solve: replaces torch.linalg.solve(ZTZ + lambda I, ZtrainY) of
+ * qml_lightning/models/kernel.py:226-234 (LU there; the matrix is symmetric positive definite) ---- */
+
+/* Bytes of device workspace qmll_cholesky_f64 / qmll_cholesky_solve_f64 need for an F x F matrix. */
+size_t qmll_cholesky_workspace_bytes(int F);
+
+/* In-place fp64 Cholesky factorisation A = U^T U of the F x F matrix A (row-major, row stride ld
+ * doubles, ld even).  Reads only elements on or above the diagonal; on exit they hold U.  Below
+ * the diagonal, the lower halves of the 128 x 128 diagonal tiles are overwritten with junk, the
+ * rest is untouched.  workspace (qmll_cholesky_workspace_bytes(F), 16-byte aligned) receives the
+ * reciprocal diagonal of U and must be passed unchanged to qmll_cholesky_solve_f64.
+ * info (device int, zeroed by the caller): 0 on success, else 1 + the index of the first pivot
+ * that is not positive; U is then unusable. */
+int qmll_cholesky_f64(double* A, int F, long long ld, void* workspace, int* info, qmll_stream_t stream);
+
+/* b <- (U^T U)^-1 b for one right-hand side b[F], U and workspace from qmll_cholesky_f64. */
+int qmll_cholesky_solve_f64(const double* U, int F, long long ld, void* workspace, double* b, qmll_stream_t stream);
+
 /* Feature-tiled variant (kernel.py:172-181, ntiles > 1): ZTZ_tile f64 [f1-f0, F] +=
  * Z[:, f0:f1]^T Z, ZTy f64 [F] (rows f0..f1 updated) += Z[:, f0:f1]^T y. */
 int qmll_gram_tile_f64(const double* Z, const double* y, int M, int F, int f0, int f1, double* ZTZ_tile, double* ZTy,

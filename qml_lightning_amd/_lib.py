@@ -5,7 +5,7 @@ raises; there is no CPU or eager fallback.
 """
 import ctypes
 import os
-from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_size_t, c_void_p
+from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_longlong, c_size_t, c_void_p
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("QML_LIGHTNING_AMD_LIB", os.path.join(HERE, "libqmll.so"))
@@ -57,10 +57,14 @@ PROTOTYPES = {
     "qmll_gram_f64": [P, P, c_int, c_int, P, P, P],
     "qmll_gram_upper_f64": [P, P, c_int, c_int, P, P, P],
     "qmll_gram_mirror_f64": [P, c_int, P],
+    "qmll_cholesky_workspace_bytes": [c_int],
+    "qmll_cholesky_f64": [P, c_int, c_longlong, P, P, P],
+    "qmll_cholesky_solve_f64": [P, c_int, c_longlong, P, P, P],
     "qmll_gram_tile_f64": [P, P, c_int, c_int, c_int, c_int, P, P, P],
     "qmll_matmul_and_reduce": [P, P, c_int, c_int, c_int, P, P],
 }
-_RESTYPES = {"qmll_last_error": c_char_p, "qmll_sort_by_type_workspace": c_size_t}
+_RESTYPES = {"qmll_last_error": c_char_p, "qmll_sort_by_type_workspace": c_size_t,
+             "qmll_cholesky_workspace_bytes": c_size_t}
 
 _lib = None
 

@@ -85,7 +85,9 @@ __device__ __forceinline__ void tile_of_block(unsigned b, int nti, int ntj, Tile
 // odd F): every element load is bounds-checked.  !GUARD: whole panels, 16-byte vector loads.
 template <bool SYM, bool GUARD>
 __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ Z, int M, int F, int f0, int f1,
-                                                      int nti, int ntj, TileMap tm, double* __restrict__ C) {
+                                                      int nti, int ntj, TileMap tm, double* __restrict__ C,
+                                                      long long ldz, long long ldc, double sign,
+                                                      const double* __restrict__ Za, long long lda, int overwrite) {
     // two copies of each staged panel: the next one is written while the current one is read,
     // one barrier per step (2 x 2 x 18 KB per workgroup, two workgroups per CU)
     __shared__ __attribute__((aligned(16))) double sA[2][KB][LDS_STRIDE];
@@ -123,9 +125,9 @@ __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ 
         const bool rowok = m < M;
         if constexpr (interior) {
             // rows past the end are read from the last row (always valid memory) and zeroed
-            const double* zr = Z + (size_t)(rowok ? m : M - 1) * F;
-            const double2_t* pa = reinterpret_cast<const double2_t*>(zr + i0 + lc);
-            const double2_t* pb = reinterpret_cast<const double2_t*>(zr + j0 + lc);
+            const size_t mr = (size_t)(rowok ? m : M - 1);
+            const double2_t* pa = reinterpret_cast<const double2_t*>(Za + mr * lda + i0 + lc);
+            const double2_t* pb = reinterpret_cast<const double2_t*>(Z + mr * ldz + j0 + lc);
             // nothing may consume the loaded values before the MFMAs of the current panel
             // have been issued, so the zeroing of tail rows happens at the LDS store
             loaded_rowok = rowok;
@@ -136,12 +138,13 @@ __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ 
                 for (int q = 0; q < 4; ++q) rb[q] = pb[q];
             }
         } else {
-            const double* zr = Z + (size_t)m * F;
+            const double* zr = Z + (size_t)m * ldz;
+            const double* zar = Za + (size_t)m * lda;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int ca = i0 + lc + 2 * q;
-                ra[q].x = (rowok && ca < ilim) ? zr[ca] : 0.0;
-                ra[q].y = (rowok && ca + 1 < ilim) ? zr[ca + 1] : 0.0;
+                ra[q].x = (rowok && ca < ilim) ? zar[ca] : 0.0;
+                ra[q].y = (rowok && ca + 1 < ilim) ? zar[ca + 1] : 0.0;
                 const int cb = j0 + lc + 2 * q;
                 rb[q].x = (rowok && cb < F) ? zr[cb] : 0.0;
                 rb[q].y = (rowok && cb + 1 < F) ? zr[cb + 1] : 0.0;
@@ -208,11 +211,13 @@ __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ 
                 const int gi = i0 + wi + p * 16 + lk + 4 * r;
                 const int gj = j0 + wj + q * 16 + l16;
                 if (gi < ilim && gj < F) {
-                    const double v = acc[p][q][r];
+                    const double v = sign * acc[p][q][r];
                     if (SYM) {
-                        C[(size_t)gi * F + gj] += v;               // the mirror image is a separate pass
+                        C[(size_t)gi * ldc + gj] += v;             // the mirror image is a separate pass
+                    } else if (overwrite) {
+                        C[(size_t)(gi - f0) * ldc + gj] = v;
                     } else {
-                        C[(size_t)(gi - f0) * F + gj] += v;
+                        C[(size_t)(gi - f0) * ldc + gj] += v;
                     }
                 }
             }
@@ -282,10 +287,19 @@ __global__ __launch_bounds__(MR* MR) void matmul_and_reduce_kernel(const float* 
 
 }  // namespace
 
+// Z: M rows of F used columns, row stride ldz; C: row stride ldc; C += sign * Z^T Z
 static int gram_launch(const double* Z, const double* y, int M, int F, int f0, int f1, bool sym, bool mirror, double* C,
-                       double* ZTy, hipStream_t stream, const char* who) {
+                       double* ZTy, hipStream_t stream, const char* who, long long ldz = 0, long long ldc = 0,
+                       double sign = 1.0, const double* Za = nullptr, long long lda = 0, int overwrite = 0) {
+    if (ldz == 0) ldz = F;
+    if (ldc == 0) ldc = F;
+    if (!Za) {   // the Gram product: both operands are Z
+        Za = Z;
+        lda = ldz;
+    }
     QMLL_REQUIRE(M >= 0 && F > 0, QMLL_ERR_INVALID, "%s: bad size M=%d F=%d", who, M, F);
-    QMLL_REQUIRE(0 <= f0 && f0 < f1 && f1 <= F, QMLL_ERR_INVALID, "%s: bad feature range [%d,%d) of %d", who, f0, f1, F);
+    QMLL_REQUIRE(0 <= f0 && f0 < f1 && (f1 <= F || (Za && Za != Z)), QMLL_ERR_INVALID,
+                 "%s: bad feature range [%d,%d) of %d", who, f0, f1, F);
     if (M == 0) return QMLL_OK;
     QMLL_REQUIRE(Z && C, QMLL_ERR_INVALID, "%s: null pointer", who);
     QMLL_REQUIRE((y == nullptr) == (ZTy == nullptr), QMLL_ERR_INVALID, "%s: y and ZTy must both be given or both be NULL",
@@ -307,18 +321,20 @@ static int gram_launch(const double* Z, const double* y, int M, int F, int f0, i
     }
     const long long nblocks = per_xcd * NXCD;
     QMLL_REQUIRE(nblocks < 2147483647LL, QMLL_ERR_INVALID, "%s: too many tiles", who);
-    const bool guard = (F % TILE) != 0 || ((f1 - f0) % TILE) != 0 || (f0 % 2) != 0;
+    const bool guard = (F % TILE) != 0 || ((f1 - f0) % TILE) != 0 || (f0 % 2) != 0 || (ldz % 2) != 0 ||
+                       (lda % 2) != 0 || (reinterpret_cast<uintptr_t>(Z) % 16) != 0 ||
+                       (reinterpret_cast<uintptr_t>(Za) % 16) != 0;
     const dim3 grid((unsigned)nblocks), block(GT);
     if (sym && !guard)
-        hipLaunchKernelGGL((gram_kernel<true, false>), grid, block, 0, stream, Z, M, F, 0, F, nti, ntj, tm, C);
+        hipLaunchKernelGGL((gram_kernel<true, false>), grid, block, 0, stream, Z, M, F, 0, F, nti, ntj, tm, C, ldz, ldc, sign, Za, lda, overwrite);
     else if (sym)
-        hipLaunchKernelGGL((gram_kernel<true, true>), grid, block, 0, stream, Z, M, F, 0, F, nti, ntj, tm, C);
+        hipLaunchKernelGGL((gram_kernel<true, true>), grid, block, 0, stream, Z, M, F, 0, F, nti, ntj, tm, C, ldz, ldc, sign, Za, lda, overwrite);
     else if (!guard)
-        hipLaunchKernelGGL((gram_kernel<false, false>), grid, block, 0, stream, Z, M, F, f0, f1, nti, ntj, tm, C);
+        hipLaunchKernelGGL((gram_kernel<false, false>), grid, block, 0, stream, Z, M, F, f0, f1, nti, ntj, tm, C, ldz, ldc, sign, Za, lda, overwrite);
     else
-        hipLaunchKernelGGL((gram_kernel<false, true>), grid, block, 0, stream, Z, M, F, f0, f1, nti, ntj, tm, C);
+        hipLaunchKernelGGL((gram_kernel<false, true>), grid, block, 0, stream, Z, M, F, f0, f1, nti, ntj, tm, C, ldz, ldc, sign, Za, lda, overwrite);
     QMLL_CHECK_LAUNCH(who);
-    if (sym && mirror) {
+    if (sym && mirror && ldc == F) {
         const unsigned nb = (unsigned)((F + MT - 1) / MT);
         hipLaunchKernelGGL(gram_mirror_kernel, dim3(nb, nb), dim3(256), 0, stream, C, F);
         QMLL_CHECK_LAUNCH(who);
@@ -366,4 +382,20 @@ extern "C" int qmll_matmul_and_reduce(const float* A, const float* B, int Ar, in
     hipLaunchKernelGGL(matmul_and_reduce_kernel, grid, dim3(MR * MR), 0, (hipStream_t)stream, A, B, Ar, K, Bc, C);
     QMLL_CHECK_LAUNCH("qmll_matmul_and_reduce");
     return QMLL_OK;
+}
+
+// used by solve.hip: tiles on or above the diagonal of C[n,n] += sign * Z^T Z with strided operands
+int qmll_internal_syrk_upper(const double* Z, int M, int n, long long ldz, double* C, long long ldc, double sign,
+                             hipStream_t stream) {
+    return gram_launch(Z, nullptr, M, n, 0, n, true, false, C, nullptr, stream, "qmll_cholesky_f64", ldz, ldc, sign);
+}
+
+// used by solve.hip: C[ra, n] (row stride ldc) = or += sign * Za^T Zb, Za = M rows of ra columns
+// (row stride lda), Zb = M rows of n columns (row stride ldb).  With overwrite set and
+// ra <= 128, C may be Zb itself: one workgroup owns each 128-column strip and reads all of it
+// before it writes.
+int qmll_internal_gemm_tn(const double* Za, long long lda, int ra, const double* Zb, long long ldb, int n, int M,
+                          double* C, long long ldc, double sign, int overwrite, hipStream_t stream) {
+    return gram_launch(Zb, nullptr, M, n, 0, ra, false, false, C, nullptr, stream, "qmll_cholesky_f64", ldb, ldc, sign,
+                       Za, lda, overwrite);
 }

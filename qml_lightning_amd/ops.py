@@ -442,6 +442,29 @@ def rff_energy_sorted(x, type_offsets, sorted_slots, W, b, alpha, nslots, with_g
     return e_slots, gx
 
 
+def cholesky_solve_spd(A, b, overwrite_a=False):
+    """x = A^-1 b for a symmetric positive definite fp64 A [F,F] and b [F] or [F,1], by the
+    in-place upper Cholesky factorisation of the library.  Only the upper triangle of A is read.
+    Returns (x, info): info is a device int32 tensor, 0 on success, else 1 + the index of the first
+    non-positive pivot (x is then meaningless).  A is destroyed when overwrite_a is True."""
+    if A.dtype != torch.float64 or A.dim() != 2 or A.shape[0] != A.shape[1] or A.stride(1) != 1:
+        raise RuntimeError("cholesky_solve_spd needs a square float64 matrix with contiguous rows")
+    F = int(A.shape[0])
+    if b.dtype != torch.float64 or b.numel() != F:
+        raise RuntimeError("cholesky_solve_spd: b must hold F float64 values")
+    U = A if overwrite_a else A.clone()
+    ld = int(U.stride(0))
+    if ld % 2 != 0:
+        raise RuntimeError("cholesky_solve_spd: the row stride must be even")
+    L = _lib.lib()
+    work = torch.empty(int(L.qmll_cholesky_workspace_bytes(F)) // 8 + 1, dtype=torch.float64, device=A.device)
+    info = torch.zeros(1, dtype=torch.int32, device=A.device)
+    x = b.detach().clone().contiguous()
+    check(L.qmll_cholesky_f64(_ptr(U), F, ld, _ptr(work), _ptr(info), _stream()), "qmll_cholesky_f64")
+    check(L.qmll_cholesky_solve_f64(_ptr(U), F, ld, _ptr(work), _ptr(x), _stream()), "qmll_cholesky_solve_f64")
+    return x, info
+
+
 def gram_mirror(ZTZ):
     """Copy the upper triangle of ZTZ onto the lower one (after `gram(..., mirror=False)` calls)."""
     if ZTZ.dtype != torch.float64 or not ZTZ.is_contiguous() or ZTZ.shape[0] != ZTZ.shape[1]:

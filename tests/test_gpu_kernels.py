@@ -475,6 +475,48 @@ def test_gram_upper_batches_then_one_mirror(F):
     close(up, ref, 1e-13, "batched ZTZ")
 
 
+@pytest.mark.parametrize("F", [6, 100, 128, 300, 1064, 2176])
+def test_cholesky_solve_matches_lapack(F):
+    """(Z^T Z + lambda I) x = b by the library's blocked Cholesky against numpy's LU solve (the
+    reference's route, kernel.py:231) and numpy's factor; conditioning as in training (few rows
+    more than features, small lambda)."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(F)
+    Zr = rng.normal(size=(F + 20, F))
+    A = Zr.T @ Zr + 1e-6 * np.eye(F)
+    b = rng.normal(size=(F, 1))
+    At = torch.tensor(A, device=dev())
+    keep = At.clone()
+    x, info = ops.cholesky_solve_spd(At, torch.tensor(b, device=dev()))
+    assert int(info.item()) == 0
+    assert torch.equal(At, keep)                                   # the input is left alone
+    x_ref = np.linalg.solve(A, b)
+    resid = np.abs(A @ x.cpu().numpy() - b).max()
+    resid_ref = np.abs(A @ x_ref - b).max()
+    assert resid <= 10 * resid_ref + 1e-9, (resid, resid_ref)
+    assert np.abs(x.cpu().numpy() - x_ref).max() <= 1e-6 * np.abs(x_ref).max() * max(1.0, np.linalg.cond(A) * 1e-9)
+    # the factor itself: in place, upper triangle = chol(A)^T
+    U = At.clone()
+    work = torch.empty(int(ops._lib.lib().qmll_cholesky_workspace_bytes(F)) // 8 + 1, dtype=torch.float64, device=dev())
+    info2 = torch.zeros(1, dtype=torch.int32, device=dev())
+    ops.check(ops._lib.lib().qmll_cholesky_f64(ops._ptr(U), F, F, ops._ptr(work), ops._ptr(info2), ops._stream()), "chol")
+    Uref = np.linalg.cholesky(A).T
+    got = np.triu(U.cpu().numpy())
+    assert np.abs(got - Uref).max() <= 1e-9 * np.abs(Uref).max()
+    assert int(info2.item()) == 0
+
+
+def test_cholesky_reports_a_matrix_that_is_not_positive_definite():
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(5)
+    F = 200
+    Zr = rng.normal(size=(F + 20, F))
+    A = Zr.T @ Zr
+    A[150, 150] = -1.0                                             # pivot 150 cannot be positive
+    x, info = ops.cholesky_solve_spd(torch.tensor(A, device=dev()), torch.zeros(F, 1, dtype=torch.float64, device=dev()))
+    assert int(info.item()) == 151
+
+
 def test_matmul_and_reduce_is_the_reference_kahan_sum():
     from qml_lightning_amd import ops
     rng = np.random.default_rng(3)
