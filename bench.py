@@ -358,7 +358,21 @@ def main():
         ZTZ, ZTy = model.build_Z_components(tc, tq, E=Et, F=Ft, print_info=False)
         torch.cuda.synchronize()
         t_build = time.perf_counter() - t0
-        del ZTZ, ZTy
+        # the step after the build: (Z^T Z + lambda I) alpha = Z^T y by the library's blocked
+        # Cholesky, with the torch (rocSOLVER) factorisation of the same matrix beside it
+        ZTZ.diagonal().add_(1e-5)
+        t_solve = timed(lambda: ops.cholesky_solve_spd(ZTZ, ZTy), iters=2)
+        xs, info = ops.cholesky_solve_spd(ZTZ, ZTy)
+        solve_resid = float((ZTZ @ xs - ZTy).abs().max() / ZTy.abs().max())
+        def torch_route():
+            L, _ = torch.linalg.cholesky_ex(ZTZ)
+            return torch.cholesky_solve(ZTy, L)
+        t_solve_torch = timed(torch_route, iters=2)
+        solve = {"solve_seconds": t_solve, "solve_TFLOPs": F ** 3 / 3.0 / t_solve / 1e12,
+                 "solve_info": int(info.item()), "solve_relative_residual": solve_resid,
+                 "solve_seconds_torch_cholesky": t_solve_torch,
+                 "solve_includes": "copy of Z^T Z + Cholesky factorisation + two triangular solves"}
+        del ZTZ, ZTy, xs
         # the Gram kernel alone, at the full training shape
         M = NMOL_TRAIN * (1 + 3 * n)
         rows = torch.randn(M, F, dtype=torch.float64, device=dev)
@@ -373,6 +387,7 @@ def main():
                  "ztz_includes": "host format_data + FCHL19 Jacobian + projection + SORF rows + Gram, 500 molecules per batch",
                  "ztz_seconds_excluding_format_data": t_build - t_format, "format_data_seconds": t_format,
                  "gram_kernel_seconds": t_gram}
+        train.update(solve)
         del rows, yv, ZTZ, ZTy
 
     # HBM-side bytes per launch come from separate rocprofv3 --pmc runs of this script (they

@@ -75,7 +75,12 @@ __global__ __launch_bounds__(256) void potrf_block_kernel(double* __restrict__ A
                 if (tid == 0) *info = k0 + j + 1;
                 return;
             }
-            const double ip = 1.0 / piv;
+            // reciprocal by the hardware estimate and two Newton steps (full fp64 accuracy up to a
+            // couple of ulps) instead of the much longer IEEE division sequence: this sits on the
+            // serial path of every step
+            double ip = __builtin_amdgcn_rcp(piv);
+            ip = fma(fma(-piv, ip, 1.0), ip, ip);
+            ip = fma(fma(-piv, ip, 1.0), ip, ip);
             double rv[8], tv[8], f[8];
 #pragma unroll
             for (int b = ja; b < 8; ++b) rv[b] = rowS[buf][b * G + tj];
@@ -197,6 +202,31 @@ extern "C" size_t qmll_cholesky_workspace_bytes(int F) {
     return (nblk * 2 * NB * NB + (size_t)F) * sizeof(double) + 256;
 }
 
+namespace {
+
+// rows [k0, k0+nb) of the panel that starts at P0: update from the panel's rows above, factor the
+// diagonal block, solve the row strip to its right
+int factor_block(double* A, int F, long long ld, int P0, int k0, double* invs, int* info, hipStream_t stream) {
+    const int nb = F - k0 < NB ? F - k0 : NB;
+    double* inv = invs + (size_t)(k0 / NB) * 2 * NB * NB;
+    if (k0 > P0) {
+        const double* above = A + (size_t)P0 * ld + k0;
+        const int rc = qmll_internal_gemm_tn(above, ld, nb, above, ld, F - k0, k0 - P0, A + (size_t)k0 * ld + k0, ld,
+                                             -1.0, 0, stream);
+        if (rc != QMLL_OK) return rc;
+    }
+    hipLaunchKernelGGL(potrf_block_kernel, dim3(1), dim3(256), 0, stream, A, ld, k0, nb, inv, inv + NB * NB, info);
+    QMLL_CHECK_LAUNCH("qmll_cholesky_f64");
+    const int n = F - k0 - nb;
+    if (n > 0) {
+        double* A12 = A + (size_t)k0 * ld + k0 + NB;
+        return qmll_internal_gemm_tn(inv, NB, NB, A12, ld, n, NB, A12, ld, 1.0, 1, stream);
+    }
+    return QMLL_OK;
+}
+
+}  // namespace
+
 extern "C" int qmll_cholesky_f64(double* A, int F, long long ld, void* workspace, int* info, qmll_stream_t stream_) {
     hipStream_t stream = (hipStream_t)stream_;
     QMLL_REQUIRE(F > 0 && ld >= F, QMLL_ERR_INVALID, "qmll_cholesky_f64: bad size F=%d ld=%lld", F, ld);
@@ -205,32 +235,15 @@ extern "C" int qmll_cholesky_f64(double* A, int F, long long ld, void* workspace
                  "qmll_cholesky_f64: the workspace must be 16-byte aligned");
     double* invs = reinterpret_cast<double*>(workspace);
     for (int P0 = 0; P0 < F; P0 += OB) {
-        const int pend = P0 + OB < F ? P0 + OB : F;
+        const int pend = P0 + OB < F ? P0 + OB : F;           // this panel: rows [P0, pend)
         for (int k0 = P0; k0 < pend; k0 += NB) {
-            const int nb = F - k0 < NB ? F - k0 : NB;
-            double* inv = invs + (size_t)(k0 / NB) * 2 * NB * NB;
-            if (k0 > P0) {
-                // rows of this block, columns k0..F: subtract the product of the panel's rows above
-                const double* above = A + (size_t)P0 * ld + k0;
-                const int rc = qmll_internal_gemm_tn(above, ld, nb, above, ld, F - k0, k0 - P0,
-                                                     A + (size_t)k0 * ld + k0, ld, -1.0, 0, stream);
-                if (rc != QMLL_OK) return rc;
-            }
-            hipLaunchKernelGGL(potrf_block_kernel, dim3(1), dim3(256), 0, stream, A, ld, k0, nb, inv, inv + NB * NB, info);
-            QMLL_CHECK_LAUNCH("qmll_cholesky_f64");
-            const int n = F - k0 - nb;
-            if (n > 0) {
-                double* A12 = A + (size_t)k0 * ld + k0 + NB;
-                const int rc = qmll_internal_gemm_tn(inv, NB, NB, A12, ld, n, NB, A12, ld, 1.0, 1, stream);
-                if (rc != QMLL_OK) return rc;
-            }
-        }
-        const int n2 = F - pend;
-        if (n2 > 0) {
-            const int rc = qmll_internal_syrk_upper(A + (size_t)P0 * ld + pend, pend - P0, n2, ld,
-                                                    A + (size_t)pend * ld + pend, ld, -1.0, stream);
+            const int rc = factor_block(A, F, ld, P0, k0, invs, info, stream);
             if (rc != QMLL_OK) return rc;
         }
+        if (pend >= F) break;
+        const int rc = qmll_internal_syrk_upper(A + (size_t)P0 * ld + pend, pend - P0, F - pend, ld,
+                                                A + (size_t)pend * ld + pend, ld, -1.0, stream);
+        if (rc != QMLL_OK) return rc;
     }
     return QMLL_OK;
 }

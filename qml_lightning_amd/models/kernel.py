@@ -232,8 +232,13 @@ class BaseKernel():
     def _solve_spd(A, b):
         """x = A^-1 b for the regularised normal matrix.  The reference calls
         torch.linalg.solve (LU, kernel.py:231); Z^T Z + lambda I is symmetric positive definite,
-        so a Cholesky factorisation gives the same solution for half the flops; LU remains the
-        fallback when rounding has left the matrix numerically indefinite."""
+        so the library's blocked Cholesky factorisation gives the same solution for half the
+        flops; LU remains the fallback when rounding has left the matrix numerically indefinite."""
+        if A.is_cuda and b.dim() == 2 and b.shape[1] == 1 and A.stride(1) == 1 and A.stride(0) % 2 == 0:
+            x, info = ops.cholesky_solve_spd(A, b)
+            if int(info.item()) == 0:
+                return x
+            return torch.linalg.solve(A, b)
         L, info = torch.linalg.cholesky_ex(A)
         if int(info.item()) == 0:
             return torch.cholesky_solve(b, L)
@@ -246,31 +251,41 @@ class BaseKernel():
         from sklearn.model_selection import KFold
         kf = KFold(n_splits=kfolds, shuffle=False)
         best = (None, None, np.inf)
+        pick = lambda seq, ids: [seq[z] for z in ids]
+        err = torch.sqrt if use_rmse else (lambda v: v)
+        red = (lambda d: torch.mean(d * d)) if use_rmse else (lambda d: torch.mean(torch.abs(d)))
         for sigma in sigmas:
-            for llambda in lambdas:
-                fold_error = 0.0
-                for train_index, test_index in kf.split(X):
-                    pick = lambda seq, ids: [seq[z] for z in ids]
-                    self.sigma, self.llambda = sigma, llambda
-                    self.train(pick(X, train_index), pick(Q, train_index), pick(E, train_index),
-                               pick(F, train_index) if F is not None else None, cells, inv_cells, print_info=False)
-                    Xt, Qt = pick(X, test_index), pick(Q, test_index)
-                    data = self.format_data(Xt, Qt, pick(E, test_index), pick(F, test_index) if F is not None else None,
-                                            cells=cells, inv_cells=inv_cells)
-                    max_natoms = int(data['natom_counts'].max().item())
-                    err = torch.sqrt if use_rmse else (lambda v: v)
-                    red = (lambda d: torch.mean(d * d)) if use_rmse else (lambda d: torch.mean(torch.abs(d)))
+            # Z^T Z and Z^T y do not depend on lambda: one build per (sigma, fold) serves the
+            # whole lambda row of the grid (the reference rebuilds them for every grid point)
+            fold_errors = np.zeros(len(lambdas))
+            for train_index, test_index in kf.split(X):
+                self.sigma = sigma
+                ZTZ, ZtrainY = self.build_Z_components(pick(X, train_index), pick(Q, train_index),
+                                                       pick(E, train_index),
+                                                       pick(F, train_index) if F is not None else None, cells,
+                                                       inv_cells, print_info=False)
+                Xt, Qt = pick(X, test_index), pick(Q, test_index)
+                data = self.format_data(Xt, Qt, pick(E, test_index), pick(F, test_index) if F is not None else None,
+                                        cells=cells, inv_cells=inv_cells)
+                max_natoms = int(data['natom_counts'].max().item())
+                diag = ZTZ.diagonal().clone()
+                for li, llambda in enumerate(lambdas):
+                    self.llambda = llambda
+                    ZTZ.diagonal().copy_(diag + llambda)
+                    self.alpha = self._solve_spd(ZTZ, ZtrainY)[:, 0]
+                    self.is_trained = True
                     if F is not None:
                         ep, fp = self.predict(Xt, Qt, max_natoms, cells=cells, inv_cells=inv_cells, forces=True,
                                               print_info=False)
                         e_err = err(red(ep - data['energies']))
                         f_err = err(red(fp - data['forces']))
-                        fold_error += 0.5 * float(e_err + f_err)
+                        fold_errors[li] += 0.5 * float(e_err + f_err)
                     else:
                         ep = self.predict(Xt, Qt, max_natoms, cells=cells, inv_cells=inv_cells, forces=False,
                                           print_info=False)
-                        fold_error += float(err(red(ep - data['energies'])))
-                fold_error /= kfolds
+                        fold_errors[li] += float(err(red(ep - data['energies'])))
+            for li, llambda in enumerate(lambdas):
+                fold_error = fold_errors[li] / kfolds
                 if print_info:
                     print("sigma", sigma, "lambda", llambda, "error", fold_error)
                 if fold_error < best[2]:

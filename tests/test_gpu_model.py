@@ -214,6 +214,47 @@ def test_training_rows_and_gram_vs_oracle(mode):
         assert m.alpha.shape == (m.nfeatures(),) and torch.isfinite(m.alpha).all()
 
 
+def test_grid_search_shares_the_gram_matrix_across_lambdas():
+    """hyperparam_opt_nested_cv (kernel.py:249-347) builds Z^T Z once per (sigma, fold); every grid
+    point must score exactly as a fresh train() + predict() at that point does."""
+    species = [1, 6]
+    coords, charges = helpers.benzene_batch(8, 3)
+    c32 = [np.asarray(c, dtype=np.float32) for c in coords]
+    rng = np.random.default_rng(21)
+    E = rng.normal(size=8)
+    Fo = [rng.normal(size=(12, 3)) for _ in range(8)]
+    sigmas, lambdas, kfolds = [2.0, 3.0], [1e-3, 1e-1], 2
+    m, _ = build_sorf_model(species, 16, 4)
+    printed = []
+    import builtins
+    real_print = builtins.print
+    builtins.print = lambda *a, **k: printed.append(a)
+    try:
+        best = m.hyperparam_opt_nested_cv(c32, charges, E, Fo, sigmas=sigmas, lambdas=lambdas, kfolds=kfolds)
+    finally:
+        builtins.print = real_print
+    got = {(a[1], a[3]): a[5] for a in printed if a and a[0] == "sigma"}
+    from sklearn.model_selection import KFold
+    expect = {}
+    for sg in sigmas:
+        for lm in lambdas:
+            m2, _ = build_sorf_model(species, 16, 4, sigma=sg)
+            m2.llambda = lm
+            tot = 0.0
+            for tr, te in KFold(n_splits=kfolds, shuffle=False).split(c32):
+                pick = lambda seq, ids: [seq[i] for i in ids]
+                m2.train(pick(c32, tr), pick(charges, tr), pick(E, tr), pick(Fo, tr), print_info=False)
+                ep, fp = m2.predict(pick(c32, te), pick(charges, te), 12, forces=True, print_info=False)
+                et = torch.tensor(np.array(pick(E, te)), device=dev())
+                ft = torch.tensor(np.array(pick(Fo, te)), device=dev())
+                tot += 0.5 * float(torch.mean(torch.abs(ep - et)) + torch.mean(torch.abs(fp - ft)))
+            expect[(sg, lm)] = tot / kfolds
+    assert set(got) == set(expect)
+    for k in expect:      # two builds of Z^T Z differ in summation order; the solve amplifies that
+        assert abs(got[k] - expect[k]) <= 1e-6 * max(1.0, abs(expect[k])), (k, got[k], expect[k])
+    assert best == min(expect, key=expect.get)
+
+
 def test_rff_model_vs_oracle():
     from qml_lightning_amd.models.random_features import RandomFourrierFeaturesModel
     from qml_lightning_amd.representations.FCHL import FCHLCuda
