@@ -83,11 +83,19 @@ __device__ __forceinline__ void tile_of_block(unsigned b, int nti, int ntj, Tile
 
 // GUARD: some panel sticks out of the matrix (F or the row block not a multiple of 128, or
 // odd F): every element load is bounds-checked.  !GUARD: whole panels, 16-byte vector loads.
-template <bool SYM, bool GUARD>
+// GEN: general operands for the Cholesky updates (separate A operand Za, row strides, sign,
+// overwrite).  !GEN is the Gram product proper: both operands are Z, every stride is F, C += Z^T Z;
+// the strides and the second pointer are then compile-time aliases, which keeps its address
+// arithmetic and register use as they were tuned.
+template <bool SYM, bool GUARD, bool GEN>
 __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ Z, int M, int F, int f0, int f1,
                                                       int nti, int ntj, TileMap tm, double* __restrict__ C,
-                                                      long long ldz, long long ldc, double sign,
-                                                      const double* __restrict__ Za, long long lda, int overwrite) {
+                                                      long long ldz_, long long ldc_, double sign_,
+                                                      const double* __restrict__ Za_, long long lda_, int overwrite_) {
+    const long long ldz = GEN ? ldz_ : (long long)F, ldc = GEN ? ldc_ : (long long)F, lda = GEN ? lda_ : (long long)F;
+    const double sign = GEN ? sign_ : 1.0;
+    const double* __restrict__ Za = GEN ? Za_ : Z;
+    const int overwrite = GEN ? overwrite_ : 0;
     // two copies of each staged panel: the next one is written while the current one is read,
     // one barrier per step (2 x 2 x 18 KB per workgroup, two workgroups per CU)
     __shared__ __attribute__((aligned(16))) double sA[2][KB][LDS_STRIDE];
@@ -325,14 +333,22 @@ static int gram_launch(const double* Z, const double* y, int M, int F, int f0, i
                        (lda % 2) != 0 || (reinterpret_cast<uintptr_t>(Z) % 16) != 0 ||
                        (reinterpret_cast<uintptr_t>(Za) % 16) != 0;
     const dim3 grid((unsigned)nblocks), block(GT);
-    if (sym && !guard)
-        hipLaunchKernelGGL((gram_kernel<true, false>), grid, block, 0, stream, Z, M, F, 0, F, nti, ntj, tm, C, ldz, ldc, sign, Za, lda, overwrite);
-    else if (sym)
-        hipLaunchKernelGGL((gram_kernel<true, true>), grid, block, 0, stream, Z, M, F, 0, F, nti, ntj, tm, C, ldz, ldc, sign, Za, lda, overwrite);
-    else if (!guard)
-        hipLaunchKernelGGL((gram_kernel<false, false>), grid, block, 0, stream, Z, M, F, f0, f1, nti, ntj, tm, C, ldz, ldc, sign, Za, lda, overwrite);
-    else
-        hipLaunchKernelGGL((gram_kernel<false, true>), grid, block, 0, stream, Z, M, F, f0, f1, nti, ntj, tm, C, ldz, ldc, sign, Za, lda, overwrite);
+    const bool gen = Za != Z || ldz != F || ldc != F || lda != F || sign != 1.0 || overwrite != 0;
+#define QMLL_GRAM_LAUNCH(S, G, E)                                                                              \
+    hipLaunchKernelGGL((gram_kernel<S, G, E>), grid, block, 0, stream, Z, M, F, sym ? 0 : f0, sym ? F : f1, nti, \
+                       ntj, tm, C, ldz, ldc, sign, Za, lda, overwrite)
+    if (gen) {
+        if (sym && !guard) QMLL_GRAM_LAUNCH(true, false, true);
+        else if (sym) QMLL_GRAM_LAUNCH(true, true, true);
+        else if (!guard) QMLL_GRAM_LAUNCH(false, false, true);
+        else QMLL_GRAM_LAUNCH(false, true, true);
+    } else {
+        if (sym && !guard) QMLL_GRAM_LAUNCH(true, false, false);
+        else if (sym) QMLL_GRAM_LAUNCH(true, true, false);
+        else if (!guard) QMLL_GRAM_LAUNCH(false, false, false);
+        else QMLL_GRAM_LAUNCH(false, true, false);
+    }
+#undef QMLL_GRAM_LAUNCH
     QMLL_CHECK_LAUNCH(who);
     if (sym && mirror && ldc == F) {
         const unsigned nb = (unsigned)((F + MT - 1) / MT);

@@ -398,6 +398,40 @@ class BaseKernel():
         print("Self Energies: ", self.self_energy)
 
     # -- batch formatting -------------------------------------------------------------------
+    def _format_padded_arrays(self, X, Q, cells=None, inv_cells=None):
+        """format_data for a batch that already is one zero-padded array pair X [B,n,3], Q [B,n]
+        (charge 0 = padding, real atoms first in every row: the layout format_data itself
+        produces, kernel.py:630-695).  Two uploads; counts, atom and molecule indices are built
+        on the device, with no Python loop over molecules."""
+        dev = self.device
+        B, n = Q.shape
+        coords = torch.from_numpy(np.ascontiguousarray(X, dtype=np.float32)).to(dev)
+        charges = torch.from_numpy(np.ascontiguousarray(Q, dtype=np.float32)).to(dev)
+        mask = charges > 0
+        counts = mask.sum(dim=1, dtype=torch.int32)
+        if bool(mask.all()):                               # fixed composition: no search needed
+            flat = torch.arange(B * n, device=dev)
+        else:
+            # padding must trail the real atoms of its row
+            if bool((mask[:, 1:] & ~mask[:, :-1]).any()):
+                raise RuntimeError("format_data: padded rows must hold their real atoms first")
+            flat = mask.reshape(-1).nonzero()[:, 0]
+        data = {
+            'coordinates': coords,
+            'charges': charges,
+            'natom_counts': counts,
+            'atomIDs': (flat % n).to(torch.int32),
+            'molIDs': (flat // n).to(torch.int32),
+            'energies': None,
+            'forces': None,
+            'cells': torch.empty((0, 3, 3), device=dev),
+            'inv_cells': torch.empty((0, 3, 3), device=dev),
+        }   # no 'element_index': the per-element lists are searched on the device when a caller needs them
+        if cells is not None:
+            data['cells'] = torch.from_numpy(np.asarray(cells, dtype=np.float32).reshape(B, 3, 3)).to(dev)
+            data['inv_cells'] = torch.from_numpy(np.asarray(inv_cells, dtype=np.float32).reshape(B, 3, 3)).to(dev)
+        return data
+
     def format_data(self, X, Q, E=None, F=None, cells=None, inv_cells=None):
         """Lists of per-molecule arrays -> zero-padded device tensors with the keys
         coordinates / charges / natom_counts / atomIDs / molIDs / energies / forces /
@@ -409,6 +443,9 @@ class BaseKernel():
                                "contributes to the potential energy.")
         dev = self.device
         zbatch = len(X)
+        if (isinstance(X, np.ndarray) and X.ndim == 3 and isinstance(Q, np.ndarray) and Q.ndim == 2
+                and E is None and F is None and not self.subtract_self_energies()):
+            return self._format_padded_arrays(X, Q, cells, inv_cells)
         counts = np.array([np.asarray(x).shape[0] for x in X], dtype=np.int32)
         n = int(counts.max()) if zbatch else 0
         # one concatenation and one scatter instead of a Python loop over molecules

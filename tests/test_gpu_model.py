@@ -214,6 +214,40 @@ def test_training_rows_and_gram_vs_oracle(mode):
         assert m.alpha.shape == (m.nfeatures(),) and torch.isfinite(m.alpha).all()
 
 
+@pytest.mark.parametrize("ragged", [False, True])
+def test_format_data_of_padded_arrays_equals_the_list_route(ragged):
+    """One zero-padded array pair goes through the device-side formatter; lists of per-molecule
+    arrays through the host one (kernel.py:601-722).  Same tensors, same predictions."""
+    species = [1, 6, 8]
+    coords, charges = helpers.fixed_composition_batch(helpers.ASPIRIN, 5, 1)
+    if ragged:
+        keep = [21, 9, 15, 21, 4]
+        coords = [c[:k] for c, k in zip(coords, keep)]
+        charges = [q[:k] for q, k in zip(charges, keep)]
+    m, _ = build_sorf_model(species, 32, 4)
+    c32 = [np.asarray(c, dtype=np.float32) for c in coords]
+    n = max(len(q) for q in charges)
+    Xp = np.zeros((len(c32), n, 3), dtype=np.float32)
+    Qp = np.zeros((len(c32), n), dtype=np.float32)
+    for i, (c, q) in enumerate(zip(c32, charges)):
+        Xp[i, :len(q)] = c
+        Qp[i, :len(q)] = q
+    a = m.format_data(c32, charges)
+    b = m.format_data(Xp, Qp)
+    for key in ("coordinates", "charges", "natom_counts", "atomIDs", "molIDs"):
+        assert a[key].dtype == b[key].dtype and torch.equal(a[key], b[key]), key
+    for e in species:
+        assert torch.equal(m._element_index(a, a["charges"], e), m._element_index(b, b["charges"], e))
+    ea, fa = m.predict(c32, charges, n, forces=True, print_info=False)
+    eb, fb = m.predict(Xp, Qp, n, forces=True, print_info=False)
+    assert torch.equal(ea, eb)
+    assert (fa - fb).abs().max() <= 1e-6 * fa.abs().max()   # the force sums use float atomics: order varies
+    bad = Qp.copy()
+    bad[0, 0] = 0.0                                      # a hole before real atoms
+    with pytest.raises(RuntimeError):
+        m.format_data(Xp, bad)
+
+
 def test_grid_search_shares_the_gram_matrix_across_lambdas():
     """hyperparam_opt_nested_cv (kernel.py:249-347) builds Z^T Z once per (sigma, fold); every grid
     point must score exactly as a fresh train() + predict() at that point does."""
