@@ -356,7 +356,7 @@ class BaseKernel():
             if not chunks:
                 continue
             mat = torch.cat(chunks)
-            U, S, _ = torch.linalg.svd(mat.T, full_matrices=False)
+            U, S = self._left_singular_vectors(mat)
             reductor = U[:, :npcas]
             if print_info:
                 cev = 100 - (S.sum() - S[:npcas].sum()) / S.sum() * 100
@@ -366,6 +366,25 @@ class BaseKernel():
                 raise RuntimeError(f"ERROR - not enough atomic environments in input dataset for element {int(e)}. "
                                    "Either increase npca_choice or provide more structures.")
             self.reductors[element_idx] = reductor
+
+    @staticmethod
+    def _left_singular_vectors(mat):
+        """Left singular vectors and singular values of mat.T for mat [nsamples, repsize], in
+        descending order: what torch.linalg.svd(mat.T) returns in the reference (kernel.py:509).
+        Computed as the eigenvectors of the repsize x repsize fp64 matrix mat^T mat (the library's
+        Gram kernel, then a small symmetric eigensolve) instead of an SVD of the tall matrix.
+        The sign of a singular vector is arbitrary in any SVD; here its largest component is
+        made positive, so equal inputs give equal reductors."""
+        rows = mat.double().contiguous()
+        R = rows.shape[1]
+        cov = torch.zeros(R, R, dtype=torch.float64, device=rows.device)
+        ops.gram(rows, None, cov, None)
+        w, V = torch.linalg.eigh(cov)
+        w, V = w.flip(0), V.flip(1)
+        lead = V.gather(0, V.abs().argmax(dim=0, keepdim=True))
+        V = V * torch.where(lead < 0, -1.0, 1.0)
+        k = min(rows.shape)                      # an SVD of [repsize, nsamples] has min(...) vectors
+        return V[:, :k].to(mat.dtype), torch.sqrt(w[:k].clamp_min(0.0)).to(mat.dtype)
 
     # -- unit conversion / self energies ----------------------------------------------------
     def set_subtract_self_energies(self, subtract):

@@ -248,6 +248,42 @@ def test_format_data_of_padded_arrays_equals_the_list_route(ragged):
         m.format_data(Xp, bad)
 
 
+def test_reductor_fit_matches_an_svd_of_the_samples():
+    """get_reductors (kernel.py:447-540): per element the leading left singular vectors of the
+    sampled representations; here via the Gram matrix and an eigensolve, checked against numpy's SVD."""
+    from qml_lightning_amd.models.kernel import BaseKernel
+    rng = np.random.default_rng(2)
+    mat = (rng.normal(size=(700, 60)) * np.logspace(0, -3, 60)).astype(np.float32)
+    U, S = BaseKernel._left_singular_vectors(torch.tensor(mat, device=dev()))
+    Un, Sn, _ = np.linalg.svd(mat.astype(np.float64).T, full_matrices=False)
+    assert U.shape == (60, 60) and U.dtype == torch.float32
+    close(S, Sn, 1e-5, "singular values")
+    Ud = U.double().cpu().numpy()
+    for k in (1, 8, 32):                                   # same leading subspaces
+        assert np.abs(Ud[:, :k] @ Ud[:, :k].T - Un[:, :k] @ Un[:, :k].T).max() < 1e-5
+    assert np.abs(Ud.T @ Ud - np.eye(60)).max() < 1e-5
+    assert (Ud[np.abs(Ud).argmax(axis=0), np.arange(60)] > 0).all()     # the sign convention
+
+    species = [1, 6, 8]
+    coords, charges = helpers.fixed_composition_batch(helpers.ASPIRIN, 12, 1)
+    c32 = [np.asarray(c, dtype=np.float32) for c in coords]
+    m, _ = build_sorf_model(species, 32, 4)
+    m.reductors = torch.zeros_like(m.reductors)
+    np.random.seed(0)
+    torch.manual_seed(0)
+    m.get_reductors(c32, charges, npcas=32, print_info=False)
+    first = m.reductors.clone()
+    for e in range(3):
+        P = first[e].double()
+        assert (P.T @ P - torch.eye(32, dtype=torch.float64, device=dev())).abs().max() < 1e-5
+    np.random.seed(0)
+    torch.manual_seed(0)
+    m.get_reductors(c32, charges, npcas=32, print_info=False)
+    assert torch.equal(first, m.reductors)                  # seeded selection, deterministic vectors
+    with pytest.raises(RuntimeError):                       # 4 oxygens x 2 molecules < 32 components
+        m.get_reductors(c32[:2], charges[:2], npcas=32, print_info=False)
+
+
 def test_grid_search_shares_the_gram_matrix_across_lambdas():
     """hyperparam_opt_nested_cv (kernel.py:249-347) builds Z^T Z once per (sigma, fold); every grid
     point must score exactly as a fresh train() + predict() at that point does."""
