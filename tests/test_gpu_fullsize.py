@@ -1,0 +1,181 @@
+"""The benchmark configurations at their full sizes, checked through properties that do not need
+the CPU oracle (which takes minutes at these sizes): the result of one large batch equals the
+results of its parts, energies are invariant and forces covariant under rigid motions, forces are
+the directional derivative of the energy, the Gram matrix satisfies its checksum identities and the
+solve its residual bound.  Small-size parity against the oracle is in test_gpu_kernels.py /
+test_gpu_model.py."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def sorf_model(species, npcas, nstacks, sigma=2.0):
+    from qml_lightning_amd.models.hadamard_features import HadamardFeaturesModel
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    from qml_lightning_amd.utils import synthetic
+    rep = FCHLCuda(species=np.array(species))
+    m = HadamardFeaturesModel(rep=rep, elements=np.array(species), ntransforms=1, sigma=sigma, llambda=1e-5,
+                              npcas=npcas, nstacks=nstacks, nbatch_train=500, nbatch_test=1 << 20)
+    red, D, bias, alpha = synthetic.model_weights(len(species), rep.get_repsize(), npcas, nstacks)
+    m.reductors, m.Dmat, m.bias = (torch.tensor(v, device=dev()) for v in (red, D, bias))
+    m.alpha = torch.tensor(alpha, device=dev())
+    m.is_trained = True
+    return m
+
+
+def step(m, coords, charges, forces=True):
+    data = m.format_data([np.asarray(c, dtype=np.float32) for c in coords], charges)
+    out = m.energies_and_forces(data['coordinates'], data['charges'], data['atomIDs'], data['molIDs'],
+                                data['natom_counts'], forces=forces)
+    if isinstance(out, tuple):
+        return out[0], (out[1] if forces else None)
+    return out, None
+
+
+def within(a, b, tol, what):
+    """max |a - b| <= tol * max |b|, with a short message."""
+    err, scale = float((a - b).abs().max()), float(b.abs().max())
+    assert err <= tol * scale, "%s: max abs diff %.3e over scale %.3e (allowed %.1e relative)" % (what, err, scale, tol)
+
+
+def random_rotation(rng):
+    q, r = np.linalg.qr(rng.normal(size=(3, 3)))
+    q = q * np.sign(np.diag(r))
+    if np.linalg.det(q) < 0:
+        q[:, 0] = -q[:, 0]
+    return q
+
+
+def test_config2_batch_of_4096_equals_its_parts_and_respects_rigid_motions():
+    """4096 x C9H8O4, 16384 features, energies + forces (the timed workload)."""
+    from qml_lightning_amd.utils import synthetic
+    species = [1, 6, 8]
+    coords, charges = synthetic.fixed_composition_batch(synthetic.ASPIRIN, 4096, seed=1)
+    m = sorf_model(species, 128, 128)
+    E, F = step(m, coords, charges)
+    assert E.shape == (4096,) and F.shape == (4096, 21, 3)
+    assert torch.isfinite(E).all() and torch.isfinite(F).all()
+    escale, fscale = float(E.abs().max()), float(F.abs().max())
+    # the same molecules in batches of 500 and in reversed order
+    for lo in range(0, 4096, 500):
+        e, f = step(m, coords[lo:lo + 500], charges[lo:lo + 500])
+        within(e, E[lo:lo + 500], 1e-5, "e")
+        within(f, F[lo:lo + 500], 1e-5, "f")
+    e, f = step(m, coords[::-1], charges[::-1])
+    within(e.flip(0), E, 1e-5, "e.flip(0)")
+    within(f.flip(0), F, 1e-5, "f.flip(0)")
+    # permuting the atoms inside every molecule permutes the forces and leaves the energies
+    rng = np.random.default_rng(0)
+    perm = rng.permutation(21)
+    e, f = step(m, [c[perm] for c in coords], [q[perm] for q in charges])
+    within(e, E, 2e-5, "e")
+    within(f, F[:, perm], 2e-5, "f")
+    # rotation + translation: fp32 coordinates are re-rounded, so the tolerance is that of the
+    # representation (1e-5) times the conditioning of the sum over 21 atoms
+    R = random_rotation(rng)
+    shift = np.array([0.7, -1.1, 0.4])
+    e, f = step(m, [c @ R.T + shift for c in coords], charges)
+    within(e, E, 1e-4, "e")
+    Frot = F.double() @ torch.tensor(R.T, device=dev())
+    within(f.double(), Frot, 1e-4, "rotated forces")
+    # no net force on any molecule
+    assert float(F.sum(dim=1).abs().max()) <= 1e-4 * fscale
+    # forces are minus the directional derivative of the energies (central difference in fp32
+    # coordinates, h = 2^-8 so that x +- h v is exact for |x| < 8 and v in {-1, 0, 1}^3)
+    h = 2.0 ** -8
+    v = [rng.integers(-1, 2, size=c.shape).astype(np.float64) for c in coords[:512]]
+    ep, _ = step(m, [c + h * d for c, d in zip(coords[:512], v)], charges[:512], forces=False)
+    em, _ = step(m, [c - h * d for c, d in zip(coords[:512], v)], charges[:512], forces=False)
+    dE = (ep.double() - em.double()) / (2 * h)
+    proj = -(F[:512].double() * torch.tensor(np.array(v), device=dev())).sum(dim=(1, 2))
+    within(dE, proj, 2e-3, "directional derivative vs forces")
+
+
+def test_config3_ragged_8192_energies_equal_their_parts():
+    """8192 molecules of 3..29 atoms over H, C, N, O, F, 8192 features, energies only."""
+    from qml_lightning_amd.utils import synthetic
+    coords, charges = synthetic.ragged_batch(8192, seed=2)
+    m = sorf_model([1, 6, 7, 8, 9], 128, 64)
+    E, _ = step(m, coords, charges, forces=False)
+    assert E.shape == (8192,) and torch.isfinite(E).all()
+    scale = float(E.abs().max())
+    for lo in (0, 3000, 8000):
+        e, _ = step(m, coords[lo:lo + 192], charges[lo:lo + 192], forces=False)
+        within(e, E[lo:lo + 192], 1e-5, "e")
+    order = np.random.default_rng(1).permutation(8192)
+    e, _ = step(m, [coords[i] for i in order], [charges[i] for i in order], forces=False)
+    within(e, E[torch.tensor(order, device=dev())], 1e-5, "e")
+
+
+def test_config4_32768_features_batch_equals_its_parts():
+    """1548 x C12H12N2O (27 atoms), npcas 256 x nstacks 128."""
+    from qml_lightning_amd.utils import synthetic
+    coords, charges = synthetic.fixed_composition_batch(synthetic.C12H12N2O, 1548, seed=3, sigma=0.15)
+    m = sorf_model([1, 6, 7, 8], 256, 128)
+    E, F = step(m, coords, charges)
+    assert torch.isfinite(E).all() and torch.isfinite(F).all()
+    e, f = step(m, coords[1000:1300], charges[1000:1300])
+    within(e, E[1000:1300], 1e-5, "e")
+    within(f, F[1000:1300], 1e-5, "f")
+    assert float(F.sum(dim=1).abs().max()) <= 1e-4 * float(F.abs().max())
+
+
+def test_config5_rff_32768_features_batch_equals_its_parts():
+    from qml_lightning_amd.models.random_features import RandomFourrierFeaturesModel
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    from qml_lightning_amd.utils import synthetic
+    species = [1, 6, 8]
+    coords, charges = synthetic.fixed_composition_batch(synthetic.ASPIRIN, 2048, seed=1)
+    np.random.seed(15)
+    rep = FCHLCuda(species=np.array(species))
+    m = RandomFourrierFeaturesModel(rep=rep, elements=np.array(species), sigma=2.0, llambda=1e-5, npcas=128,
+                                    nstacks=256, nbatch_train=500, nbatch_test=1 << 20)
+    red, _, _, alpha = synthetic.model_weights(3, rep.get_repsize(), 128, 256)
+    m.reductors = torch.tensor(red, device=dev())
+    m.alpha = torch.tensor(alpha, device=dev())
+    m.is_trained = True
+    E, F = step(m, coords, charges)
+    assert torch.isfinite(E).all() and torch.isfinite(F).all()
+    e, f = step(m, coords[700:900], charges[700:900])
+    # 32768 fp32 terms per energy, summed in an order that depends on the batch size
+    within(e, E[700:900], 5e-5, "rff energies, part vs whole")
+    within(f, F[700:900], 5e-5, "rff forces, part vs whole")
+    assert float(F.sum(dim=1).abs().max()) <= 1e-4 * float(F.abs().max())
+
+
+def test_gram_16384_features_checksums_and_solve_residual():
+    """Z^T Z at the training width (16384 features) in two row batches: symmetry, trace = |Z|_F^2,
+    (Z^T Z) v = Z^T (Z v), Z^T y; then the regularised solve on it."""
+    from qml_lightning_amd import ops
+    F = 16384
+    g = torch.Generator(device=dev()).manual_seed(3)
+    ZTZ = torch.zeros(F, F, dtype=torch.float64, device=dev())
+    ZTy = torch.zeros(F, 1, dtype=torch.float64, device=dev())
+    v = torch.randn(F, 1, dtype=torch.float64, device=dev(), generator=g)
+    ref_v = torch.zeros_like(v)
+    ref_y = torch.zeros_like(v)
+    fro = 0.0
+    for M in (12000, 9001):                                  # the second batch ends in a partial panel
+        Z = torch.randn(M, F, dtype=torch.float64, device=dev(), generator=g)
+        y = torch.randn(M, 1, dtype=torch.float64, device=dev(), generator=g)
+        ops.gram(Z, y, ZTZ, ZTy, mirror=False)
+        ref_v += Z.T @ (Z @ v)
+        ref_y += Z.T @ y
+        fro += float((Z * Z).sum())
+        del Z, y
+    ops.gram_mirror(ZTZ)
+    assert torch.equal(ZTZ, ZTZ.T)
+    assert abs(float(ZTZ.diagonal().sum()) - fro) <= 1e-12 * fro
+    within(ZTZ @ v, ref_v, 1e-11, "ZTZ @ v")
+    within(ZTy, ref_y, 1e-12, "ZTy")
+    ZTZ.diagonal().add_(1e-5)
+    x, info = ops.cholesky_solve_spd(ZTZ, ZTy)
+    assert int(info.item()) == 0
+    resid = float((ZTZ @ x - ZTy).abs().max() / ZTy.abs().max())
+    assert resid <= 1e-10, resid
