@@ -506,6 +506,27 @@ def test_cholesky_solve_matches_lapack(F):
     assert int(info2.item()) == 0
 
 
+def test_cholesky_in_place_on_a_strided_view():
+    """overwrite_a=True factors inside a wider buffer (row stride 700 for a 300 x 300 matrix) and
+    touches nothing outside the matrix."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(9)
+    F, W = 300, 700
+    Zr = rng.normal(size=(F + 20, F))
+    A = Zr.T @ Zr + 1e-6 * np.eye(F)
+    b = rng.normal(size=(F, 1))
+    big = torch.full((F + 3, W), 5.0, dtype=torch.float64, device=dev())
+    view = big[1:F + 1, 100:100 + F]
+    view.copy_(torch.tensor(A, device=dev()))
+    x, info = ops.cholesky_solve_spd(view, torch.tensor(b, device=dev()), overwrite_a=True)
+    assert int(info.item()) == 0
+    assert np.abs(A @ x.cpu().numpy() - b).max() <= 1e-7 * np.abs(b).max()
+    assert np.abs(np.triu(view.cpu().numpy()) - np.linalg.cholesky(A).T).max() <= 1e-9 * np.abs(A).max() ** 0.5
+    outside = big.clone()
+    outside[1:F + 1, 100:100 + F] = 5.0
+    assert (outside == 5.0).all()
+
+
 def test_cholesky_reports_a_matrix_that_is_not_positive_definite():
     from qml_lightning_amd import ops
     rng = np.random.default_rng(5)
