@@ -560,11 +560,14 @@ __device__ __forceinline__ void store_row(const float (&v)[EPL], float* __restri
 
 constexpr int ROWS_NA = 4;   // atoms per workgroup = rows of 16 lanes per wavefront
 
-template <int LOG2D, bool WITH_GRAD>
+// MULTI: more than one transform per stack (T > 1); the first sign diagonal stays in registers
+// as for T = 1, the later ones are fetched where they are used (forward and again in the adjoint).
+template <int LOG2D, bool WITH_GRAD, bool MULTI>
 __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
     const float* __restrict__ x, const float* __restrict__ D, const float* __restrict__ bias,
     const float* __restrict__ alpha, const int* __restrict__ out_index, const int* __restrict__ type_offsets, int ne,
-    int A, int S, float scale, float normf, float* __restrict__ e_atom, float* __restrict__ gx) {
+    int A, int S, int T_, float scale, float normf, float* __restrict__ e_atom, float* __restrict__ gx) {
+    const int T = MULTI ? T_ : 1;
     constexpr int d = 1 << LOG2D;
     constexpr int EPL = d / 16;                 // registers per lane
     constexpr int NA = ROWS_NA;
@@ -590,7 +593,7 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
             b -= nt;
         }
         if (rows == 0) return;
-        D += (size_t)t * S * d;
+        D += (size_t)t * T * S * d;
         bias += (size_t)t * S * d;
     } else {
         row0 = blockIdx.x * NA;
@@ -632,6 +635,16 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
         for (int p = 0; p < EPL; ++p) v[p] = xv[p] * dv[p];
         register_stages<EPL>(v);
         row_stages<EPL>(v, cs);
+        if constexpr (MULTI) {
+            for (int m = 1; m < T; ++m) {
+                float dm[EPL];
+                load_row<EPL>(dm, D + ((size_t)m * S + s) * d + e0);
+#pragma unroll
+                for (int p = 0; p < EPL; ++p) v[p] *= dm[p] * sigma;
+                register_stages<EPL>(v);
+                row_stages<EPL>(v, cs);
+            }
+        }
 
         float arg[EPL], amax = 0.0f;
 #pragma unroll
@@ -668,6 +681,16 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
         if constexpr (WITH_GRAD) {
             register_stages<EPL>(v);
             row_stages<EPL>(v, cs);
+            if constexpr (MULTI) {
+                for (int m = T - 1; m >= 1; --m) {
+                    float dm[EPL];
+                    load_row<EPL>(dm, D + ((size_t)m * S + s) * d + e0);
+#pragma unroll
+                    for (int p = 0; p < EPL; ++p) v[p] *= dm[p] * sigma;
+                    register_stages<EPL>(v);
+                    row_stages<EPL>(v, cs);
+                }
+            }
 #pragma unroll
             for (int p = 0; p < EPL; ++p) acc[p] = fmaf(v[p], dv[p], acc[p]);
         }
@@ -1303,23 +1326,25 @@ static int launch_fused(const char* who, const float* x, const float* D, const f
                         int T, float normalisation, float* e_atom, float* gx, hipStream_t stream) {
     const float scale = normalisation * hnorm(d, T);
     const float normf = sqrtf(2.0f / ((float)S * (float)d));
-    if (T == 1 && d >= 64 && d <= 256 && types == nullptr) {
-        // one transform per stack, 4 to 16 registers per lane, atoms groupable by element: the
-        // instruction-lean kernel (four atoms per workgroup)
+    if (d >= 64 && d <= 256 && types == nullptr) {
+        // 4 to 16 registers per lane, atoms groupable by element: the instruction-lean kernel
+        // (four atoms per workgroup)
         const dim3 grid((A + ROWS_NA - 1) / ROWS_NA + (type_offsets ? ne : 0));
-#define CALL_ROWS(L)                                                                                                 \
-    if (gx)                                                                                                          \
-        hipLaunchKernelGGL((sorf_energy_rows_kernel<L, true>), grid, dim3(SORF_THREADS), 0, stream, x, D, bias,      \
-                           alpha, out_index, type_offsets, ne, A, S, scale, normf, e_atom, gx);                      \
-    else                                                                                                             \
-        hipLaunchKernelGGL((sorf_energy_rows_kernel<L, false>), grid, dim3(SORF_THREADS), 0, stream, x, D, bias,     \
-                           alpha, out_index, type_offsets, ne, A, S, scale, normf, e_atom, gx)
+#define LAUNCH_ROWS(L, G, M)                                                                                       \
+    hipLaunchKernelGGL((sorf_energy_rows_kernel<L, G, M>), grid, dim3(SORF_THREADS), 0, stream, x, D, bias, alpha, \
+                       out_index, type_offsets, ne, A, S, T, scale, normf, e_atom, gx)
+#define CALL_ROWS(L)                                  \
+    if (gx && T == 1) LAUNCH_ROWS(L, true, false);    \
+    else if (gx) LAUNCH_ROWS(L, true, true);          \
+    else if (T == 1) LAUNCH_ROWS(L, false, false);    \
+    else LAUNCH_ROWS(L, false, true)
         switch (qmll_log2(d)) {
             case 6: { CALL_ROWS(6); } break;
             case 7: { CALL_ROWS(7); } break;
             case 8: { CALL_ROWS(8); } break;
             default: break;
         }
+#undef LAUNCH_ROWS
 #undef CALL_ROWS
         QMLL_CHECK_LAUNCH(who);
         if (gx && type_offsets) {

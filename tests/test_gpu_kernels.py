@@ -285,7 +285,8 @@ def test_derivative_features(d, S, T):
         close(G - 1.0, ref, REL_REP, "derivative features, molecule_major=%s" % molecule_major)
 
 
-@pytest.mark.parametrize("d,S,T", [(8, 3, 1), (64, 5, 2), (128, 16, 1), (256, 8, 1), (512, 4, 1)])
+@pytest.mark.parametrize("d,S,T", [(8, 3, 1), (64, 5, 2), (128, 16, 1), (128, 9, 2), (128, 5, 3), (256, 8, 1), (256, 6, 2),
+                                   (512, 4, 1), (512, 3, 2)])
 def test_fused_energy_matches_two_op_chain(d, S, T):
     from qml_lightning_amd import ops
     rng = np.random.default_rng(d + S)
@@ -389,12 +390,13 @@ def test_project_typed_forward_and_backward(R, d, ne, N, A):
     assert (g.cpu().numpy()[mask] == 0).all()
 
 
-def test_sorted_fused_energy_matches_per_atom_oracle():
+@pytest.mark.parametrize("T", [1, 2])
+def test_sorted_fused_energy_matches_per_atom_oracle(T):
     """Element-sorted rows through the fused kernel: energies land in the atoms' slots, the
     gradient stays in sorted order, rows past the last known atom give zero."""
     from qml_lightning_amd import ops
     rng = np.random.default_rng(19)
-    ne, d, S, T, N, A = 3, 64, 6, 1, 50, 37
+    ne, d, S, N, A = 3, 64, 6, 50, 37
     F = S * d
     types = rng.integers(-1, ne, N).astype(np.int32)
     slots = np.sort(rng.choice(N, size=A, replace=False)).astype(np.int32)
