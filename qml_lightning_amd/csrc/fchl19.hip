@@ -962,6 +962,8 @@ extern "C" int qmll_fchl19_forward(const float* X, const int* types, const float
     if (rc) return rc;
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(rep != nullptr, QMLL_ERR_INVALID, "qmll_fchl19_forward: null output");
+    QMLL_REQUIRE(prm->nRs3 <= 256, QMLL_ERR_INVALID,
+                 "qmll_fchl19_forward: nRs3=%d: at most 256 three-body radial bins are supported", prm->nRs3);
     const int R = prm->nspecies * prm->nRs2 + prm->nspecies * (prm->nspecies + 1) * prm->nRs3;
     // table for every triple of a full neighbourhood when that stays small
     const long long alltrip = (long long)a.cap * (a.cap - 1) / 2;

@@ -156,6 +156,15 @@ def test_fchl_periodic_cell():
     close(ops.fchl_jacobian(*args)[1], J, REL_REP, "pbc jacobian")
 
 
+def test_fchl_forward_refuses_more_radial_bins_than_it_handles():
+    from qml_lightning_amd import ops
+    prm = oracle_prm([1, 6], nRs3=300)
+    args = (t32(np.zeros((1, 2, 3))), ti32([[1, 0]]), None, None, ti32([0, 1]), ti32([0, 0]), ti32([2]), t32(prm.Rs2),
+            t32(prm.Rs3), gpu_prm(prm))
+    with pytest.raises(RuntimeError, match="nRs3"):
+        ops.fchl_forward(*args)
+
+
 def test_fchl_single_atom_and_empty_batch():
     from qml_lightning_amd import ops
     prm = oracle_prm([1, 6])
