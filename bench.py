@@ -58,6 +58,23 @@ def cpu_baseline(coords, charges, weights, nsample, cores):
     return n / dt, n, dt, out, chunks
 
 
+def bench_solve(torch, ops, timed, ZTZ, ZTy, F):
+    """(Z^T Z + lambda I) alpha = Z^T y on the matrix just built: the library's blocked Cholesky,
+    with the torch (rocSOLVER) factorisation of the same matrix beside it."""
+    ZTZ.diagonal().add_(1e-5)
+    t_solve = timed(lambda: ops.cholesky_solve_spd(ZTZ, ZTy), iters=2)
+    xs, info = ops.cholesky_solve_spd(ZTZ, ZTy)
+    resid = float((ZTZ @ xs - ZTy).abs().max() / ZTy.abs().max())
+
+    def torch_route():
+        L, _ = torch.linalg.cholesky_ex(ZTZ)
+        return torch.cholesky_solve(ZTy, L)
+    t_torch = timed(torch_route, iters=2)
+    return {"solve_seconds": t_solve, "solve_TFLOPs": F ** 3 / 3.0 / t_solve / 1e12, "solve_info": int(info.item()),
+            "solve_relative_residual": resid, "solve_seconds_torch_cholesky": t_torch,
+            "solve_includes": "copy of Z^T Z + Cholesky factorisation + two triangular solves"}
+
+
 def other_configs(torch, dev):
     """Short measurements of the other benchmark configurations (1, 3, 4, 5) with the
     same step definition; reported under "other_configs", never as `value`."""
@@ -151,6 +168,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-train", action="store_true", help="skip the Z^T Z build measurement")
+    ap.add_argument("--no-solve", action="store_true", help="skip the regularised solve after the Z^T Z build")
     ap.add_argument("--cpu-sample", type=int, default=1024)
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the short measurements of configurations 1, 3, 4 and 5")
@@ -372,19 +390,10 @@ def main():
         t_build = time.perf_counter() - t0
         # the step after the build: (Z^T Z + lambda I) alpha = Z^T y by the library's blocked
         # Cholesky, with the torch (rocSOLVER) factorisation of the same matrix beside it
-        ZTZ.diagonal().add_(1e-5)
-        t_solve = timed(lambda: ops.cholesky_solve_spd(ZTZ, ZTy), iters=2)
-        xs, info = ops.cholesky_solve_spd(ZTZ, ZTy)
-        solve_resid = float((ZTZ @ xs - ZTy).abs().max() / ZTy.abs().max())
-        def torch_route():
-            L, _ = torch.linalg.cholesky_ex(ZTZ)
-            return torch.cholesky_solve(ZTy, L)
-        t_solve_torch = timed(torch_route, iters=2)
-        solve = {"solve_seconds": t_solve, "solve_TFLOPs": F ** 3 / 3.0 / t_solve / 1e12,
-                 "solve_info": int(info.item()), "solve_relative_residual": solve_resid,
-                 "solve_seconds_torch_cholesky": t_solve_torch,
-                 "solve_includes": "copy of Z^T Z + Cholesky factorisation + two triangular solves"}
-        del ZTZ, ZTy, xs
+        solve = {}
+        if not args.no_solve:
+            solve = bench_solve(torch, ops, timed, ZTZ, ZTy, F)
+        del ZTZ, ZTy
         # the Gram kernel alone, at the full training shape
         M = NMOL_TRAIN * (1 + 3 * n)
         rows = torch.randn(M, F, dtype=torch.float64, device=dev)
