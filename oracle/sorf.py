@@ -10,6 +10,7 @@ Follows (paths relative to the reference tree):
   * sin coefficients ................... qml_lightning/cuda/hadamard_kernel.cu:565-585
   * derivative features ................ qml_lightning/cuda/hadamard_kernel.cu:587-717
   * model-level feature assembly ....... qml_lightning/models/hadamard_features.py:66-121
+  * regularised solve .................. qml_lightning/models/kernel.py:226-234
   * Gram accumulation, targets ......... qml_lightning/models/kernel.py:118-192
   * fp32-Kahan -> fp64 product ......... qml_lightning/cuda/utils_kernel.cu:70-119
   * RFF features / derivative .......... qml_lightning/cuda/random_features_kernel.cu:5-94,
@@ -178,6 +179,16 @@ def training_rows(Z, G, E=None, F=None):
 def gram(Zrows, y):
     """ZTZ = Z^T Z, ZTy = Z^T y in fp64 (kernel.py:190-192)."""
     return Zrows.T @ Zrows, Zrows.T @ y
+
+
+def regularised_solve(ZTZ, ZTy, llambda):
+    """alpha of the regularised normal equations, the way train() gets it: lambda added to the
+    diagonal of Z^T Z, then a general (LU) solve (qml_lightning/models/kernel.py:226-234).
+    Pinned by the identity it solves: tests check the residual and the agreement with a Cholesky
+    factorisation of the same matrix."""
+    A = np.array(ZTZ, dtype=np.float64, copy=True)
+    A[np.diag_indices_from(A)] += llambda
+    return np.linalg.solve(A, np.asarray(ZTy, dtype=np.float64))
 
 
 def matmul_and_reduce(A32, B32, C64, block=16):

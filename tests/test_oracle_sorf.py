@@ -117,6 +117,25 @@ def test_training_rows_variants_and_gram():
     assert np.allclose(np.concatenate(tiles, 0), ZTZ)
 
 
+def test_regularised_solve_satisfies_the_normal_equations():
+    """alpha minimises |Z a - y|^2 + lambda |a|^2: the gradient vanishes, the Cholesky route agrees,
+    and for lambda -> 0 with full column rank it is the least-squares solution."""
+    rng = np.random.default_rng(4)
+    Z = rng.normal(size=(90, 40))
+    y = rng.normal(size=(90, 1))
+    ZTZ, ZTy = sorf.gram(Z, y)
+    lam = 1e-3
+    a = sorf.regularised_solve(ZTZ, ZTy, lam)
+    grad = Z.T @ (Z @ a - y) + lam * a
+    assert np.abs(grad).max() < 1e-10
+    L = np.linalg.cholesky(ZTZ + lam * np.eye(40))
+    a_chol = np.linalg.solve(L.T, np.linalg.solve(L, ZTy))
+    assert np.abs(a - a_chol).max() < 1e-12
+    a0 = sorf.regularised_solve(ZTZ, ZTy, 0.0)
+    assert np.abs(a0 - np.linalg.lstsq(Z, y, rcond=None)[0]).max() < 1e-10
+    assert np.array_equal(ZTZ, Z.T @ Z)                    # the input is not modified
+
+
 def test_matmul_and_reduce_close_to_fp64():
     rng = np.random.default_rng(3)
     A = rng.normal(size=(16, 200)).astype(np.float32)
