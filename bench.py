@@ -260,6 +260,26 @@ def main():
                       "max_abs_diff_energy": float((Ea.detach() - E).abs().max()),
                       "max_abs_diff_force": float((Fa - Fr).abs().max())}
 
+    # the same step through the reference's two-operator contract (get_SORF_coefficients +
+    # get_cos_features with autograd, the only operators a model file saved by the reference calls):
+    # the [atoms, features] coefficient array goes through HBM four times
+    model.fused = False
+    for _ in range(2):
+        step_autograd()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        E2, F2 = step_autograd()
+    torch.cuda.synchronize()
+    ms_two_op = (time.perf_counter() - t0) / 5 * 1e3
+    model.fused = True
+    two_op_route = {"ms_per_step": ms_two_op, "molecules_per_s": B / ms_two_op * 1e3,
+                    "max_abs_diff_energy": float((E2.detach() - E).abs().max()),
+                    "max_abs_diff_force": float((F2 - Fr).abs().max()),
+                    "hbm_bytes_per_step_algorithmic": float(A) * (20.0 * F + 8.0 * NPCAS)}
+    del E2, F2
+    torch.cuda.empty_cache()
+
     # the same batch handed over as host arrays (lists of numpy coordinates / charges): batch
     # formatting on the host, upload over PCIe, predict, results left on the device
     model.predict(coords[:64], charges[:64], n, forces=True)
@@ -448,6 +468,7 @@ def main():
                    "molecules_per_step": B, "atoms_per_step": A},
         "roofline": roofline,
         "autograd_route": autograd_route,
+        "two_op_route": two_op_route,
         "from_host_arrays": from_host,
         "kernels": kernels,
     }
