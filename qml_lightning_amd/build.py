@@ -17,7 +17,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-munsafe-fp-ato
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-value"]
 
 
-def build(verbose=True, jobs=6):
+def build(verbose=True, jobs=8):
     """Compile every source to an object (in parallel) and link libqmll.so."""
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
