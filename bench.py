@@ -429,6 +429,10 @@ def main():
                  "ztz_seconds_excluding_format_data": t_build - t_format, "format_data_seconds": t_format,
                  "gram_kernel_seconds": t_gram}
         train.update(solve)
+        if solve:
+            kernels["cholesky_solve_f64"] = {"seconds": solve["solve_seconds"], "bound": "mfma",
+                                             "TFLOPs": solve["solve_TFLOPs"],
+                                             "frac": solve["solve_TFLOPs"] / FP64_PEAK_TFLOPS}
         del rows, yv, ZTZ, ZTy
 
     # HBM-side bytes per launch come from separate rocprofv3 --pmc runs of this script (they
