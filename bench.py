@@ -339,7 +339,7 @@ def main():
     t_sorf = t_cos = t_cosb = t_adj = 0.0
     two_op_bytes = 0
     for ei, e in enumerate(SPECIES):
-        idx = data['element_index'][e]
+        idx = model._element_index(data, data['charges'], e)
         sub = torch.matmul(flat_rep.index_select(0, idx), model.reductors[ei])
         Ae = sub.shape[0]
         # the reference's two-op contract, kernel by kernel (coefficients materialised)

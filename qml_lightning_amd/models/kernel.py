@@ -451,6 +451,19 @@ class BaseKernel():
             data['inv_cells'] = torch.from_numpy(np.asarray(inv_cells, dtype=np.float32).reshape(B, 3, 3)).to(dev)
         return data
 
+    @staticmethod
+    def _concat_rows(items, width, dtype):
+        """All per-molecule arrays stacked into one [total_atoms, width] array.  One
+        np.concatenate over the sequence (a C loop) when the items already have the expected
+        shape; a per-item conversion only for odd inputs (nested lists, flattened rows)."""
+        try:
+            out = np.concatenate(items)
+            if out.ndim == (2 if width > 1 else 1) and (width == 1 or out.shape[1] == width):
+                return out.astype(dtype, copy=False).reshape(-1, width)
+        except ValueError:
+            pass
+        return np.concatenate([np.asarray(v, dtype=dtype).reshape(-1, width) for v in items])
+
     def format_data(self, X, Q, E=None, F=None, cells=None, inv_cells=None):
         """Lists of per-molecule arrays -> zero-padded device tensors with the keys
         coordinates / charges / natom_counts / atomIDs / molIDs / energies / forces /
@@ -465,7 +478,7 @@ class BaseKernel():
         if (isinstance(X, np.ndarray) and X.ndim == 3 and isinstance(Q, np.ndarray) and Q.ndim == 2
                 and E is None and F is None and not self.subtract_self_energies()):
             return self._format_padded_arrays(X, Q, cells, inv_cells)
-        counts = np.array([np.asarray(x).shape[0] for x in X], dtype=np.int32)
+        counts = np.fromiter(map(len, X), dtype=np.int32, count=zbatch)
         n = int(counts.max()) if zbatch else 0
         # one concatenation and one scatter instead of a Python loop over molecules
         molIDs = np.repeat(np.arange(zbatch, dtype=np.int32), counts)
@@ -475,8 +488,8 @@ class BaseKernel():
         coords = np.zeros((zbatch, n, 3), dtype=np.float32)
         charges = np.zeros((zbatch, n), dtype=np.float32)
         if zbatch:
-            coords.reshape(-1, 3)[flat] = np.concatenate([np.asarray(x, dtype=np.float32).reshape(-1, 3) for x in X])
-            charges.reshape(-1)[flat] = np.concatenate([np.asarray(q, dtype=np.float32).reshape(-1) for q in Q])
+            coords.reshape(-1, 3)[flat] = self._concat_rows(X, 3, np.float32)
+            charges.reshape(-1)[flat] = self._concat_rows(Q, 1, np.float32).reshape(-1)
         data = {
             'coordinates': torch.from_numpy(coords).to(dev),
             'charges': torch.from_numpy(charges).to(dev),
@@ -489,8 +502,11 @@ class BaseKernel():
             'inv_cells': torch.empty((0, 3, 3), device=dev),
         }
         flat_q = charges.reshape(-1).astype(np.int64)
-        data['element_index'] = {int(e): torch.from_numpy(np.nonzero(flat_q == int(e))[0]).to(dev)
-                                 for e in self.elements}
+        if E is not None or F is not None:
+            # training batches gather rows per element: the index lists are cheap to build here on
+            # the host; a predict batch never needs them (its atoms are sorted on the device)
+            data['element_index'] = {int(e): torch.from_numpy(np.nonzero(flat_q == int(e))[0]).to(dev)
+                                     for e in self.elements}
         if E is not None:
             energies = np.array(E, dtype=np.float64).reshape(zbatch).copy()
             if self.convert_hartree2kcal():
@@ -502,7 +518,7 @@ class BaseKernel():
         if F is not None:
             forces = np.zeros((zbatch, n, 3), dtype=np.float64)
             if zbatch:
-                forces.reshape(-1, 3)[flat] = np.concatenate([np.asarray(f, dtype=np.float64).reshape(-1, 3) for f in F])
+                forces.reshape(-1, 3)[flat] = self._concat_rows(F, 3, np.float64)
             if self.convert_hartree2kcal():
                 forces *= self.hartree2kcalmol
             data['forces'] = torch.from_numpy(forces).to(dev)
