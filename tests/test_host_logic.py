@@ -48,6 +48,16 @@ def test_format_data_matches_oracle_layout():
     assert np.allclose(t[3:, 0].cpu().numpy(), d['forces'].cpu().numpy().reshape(-1))
     t = m._targets(d, 3, False, True)
     assert (t[:3] == 0).all()
+    # nested Python lists give the same tensors; a predict batch carries no per-element index lists
+    d2 = m.format_data([c.tolist() for c in coords], [q.tolist() for q in charges])
+    for key in ("coordinates", "charges", "atomIDs", "molIDs", "natom_counts"):
+        assert torch.equal(d2[key], d[key]), key
+    assert 'element_index' not in d2 and d2['energies'] is None and d2['forces'] is None
+    for e in (1, 6, 8):
+        assert torch.equal(m._element_index(d2, d2['charges'], e), d['element_index'][e])
+    # the fallback for rows that do not stack directly (a flattened force array)
+    rows = m._concat_rows([np.arange(6.0), np.arange(9.0).reshape(3, 3)], 3, np.float64)
+    assert rows.shape == (5, 3) and rows[1, 0] == 3.0 and rows[2, 1] == 1.0
 
 
 def test_self_energy_subtraction_and_unit_conversion():
