@@ -336,9 +336,18 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
             sl = slice(i, i + self.nbatch_test)
             data = self.format_data(X[sl], Z[sl], cells=cells[sl] if cells is not None else None,
                                     inv_cells=inv_cells[sl] if cells is not None else None)
-            result = self.predict_opt(data['coordinates'], data['charges'], data['atomIDs'], data['molIDs'],
-                                      data['natom_counts'], data['cells'], data['inv_cells'], forces=forces,
-                                      print_info=False, profiler=False)
+            if self.fused:
+                # no synchronisation per batch: the host formats the next batch while this one runs
+                if self.is_trained is False:
+                    raise RuntimeError("Error: must train the model first by calling train()!")
+                result = self.energies_and_forces(data['coordinates'], data['charges'], data['atomIDs'],
+                                                  data['molIDs'], data['natom_counts'], data['cells'],
+                                                  data['inv_cells'], forces=forces)
+                result = result if forces else result[0]
+            else:
+                result = self.predict_opt(data['coordinates'], data['charges'], data['atomIDs'], data['molIDs'],
+                                          data['natom_counts'], data['cells'], data['inv_cells'], forces=forces,
+                                          print_info=False, profiler=False)
             if forces:
                 predict_energies[sl] = result[0].detach()
                 n = result[1].shape[1]
