@@ -33,7 +33,16 @@ def _ptr(t):
     return _P(t.data_ptr())
 
 
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_RAW_DEVICE = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream():
+    """Handle of torch's current stream on the current device.  The raw accessors cost well under a
+    microsecond; torch.cuda.current_stream() builds a Stream object and re-checks device
+    availability on every call (8 us), seven times per predict step."""
+    if _RAW_STREAM is not None and _RAW_DEVICE is not None:
+        return _P(_RAW_STREAM(_RAW_DEVICE()))
     return _P(torch.cuda.current_stream().cuda_stream)
 
 

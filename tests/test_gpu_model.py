@@ -248,6 +248,28 @@ def test_format_data_of_padded_arrays_equals_the_list_route(ragged):
         m.format_data(Xp, bad)
 
 
+def test_kernels_follow_the_current_stream():
+    """Every launch goes to torch's current stream: the same step issued inside a side-stream
+    context (after that stream has been made to wait for the inputs) gives the same numbers, and
+    nothing is left running on the default stream."""
+    species = [1, 6, 8]
+    coords, charges = helpers.fixed_composition_batch(helpers.ASPIRIN, 6, 1)
+    m, _ = build_sorf_model(species, 64, 8)
+    X, Z, aid, mid, nat = make_batch(coords, charges)
+    args = inputs(X, Z, aid, mid, nat)
+    e0, f0 = m.energies_and_forces(*args)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        e1, f1 = m.energies_and_forces(*args)
+        done = torch.cuda.Event()
+        done.record(side)
+    done.synchronize()
+    assert torch.equal(e0, e1)
+    assert (f0 - f1).abs().max() <= 1e-6 * f0.abs().max()
+
+
 def test_reductor_fit_matches_an_svd_of_the_samples():
     """get_reductors (kernel.py:447-540): per element the leading left singular vectors of the
     sampled representations; here via the Gram matrix and an eigensolve, checked against numpy's SVD."""
