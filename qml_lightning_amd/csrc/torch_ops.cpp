@@ -526,6 +526,66 @@ std::tuple<Tensor, Tensor> rff_energy_sorted(const Tensor& x, const Tensor& off,
     return {r[0], r[1]};
 }
 
+// ---- the whole fused predict chain as one operator ---------------------------------------
+// energies [B] of forward(X, Z, atomIDs, molIDs, atom_counts) (models/hadamard_features.py:82-123):
+// representation, sort by element, projection, SORF + cos + energy, and -- when the coordinates
+// require a gradient -- the backward chain as well (the fused kernel returns dE/dx itself, the
+// projection transpose and the representation VJP follow), saved for one autograd node.  One
+// dispatch and one node instead of five of each: what a TorchScript caller that evaluates a single
+// molecule per step pays for is dispatch, not kernels.
+#define MODEL_TENSORS                                                                                   \
+    const Tensor &reductors, const Tensor &Dmat, const Tensor &bias, const Tensor &alpha, const Tensor &cn, \
+        const Tensor &nt
+
+Tensor fchl_sorf_energy_impl(FCHL_TENSORS, MODEL_TENSORS, bool with_grad, Tensor* gX_out) {
+    FchlInputs in = prepare(FCHL_PASS);
+    Tensor rep = at::zeros({in.B, in.n, in.R}, in.X.options());
+    check(qmll_fchl19_forward(FCHL_ABI(in), rep.data_ptr<float>(), stream()), "qmll_fchl19_forward");
+    const int64_t nslots = (int64_t)in.B * in.n;
+    Tensor slots = in.molIDs * in.n + in.atomIDs;
+    auto sorted = sort_by_type(in.types, slots, reductors.size(0));
+    const Tensor& ss = std::get<0>(sorted);
+    const Tensor& off = std::get<1>(sorted);
+    Tensor x = project_typed_impl(rep.view({nslots, in.R}), ss, off, reductors);
+    auto eg = sorf_energy_sorted_impl(x, off, ss, Dmat, bias, alpha, cn, nt, nslots, with_grad);
+    Tensor energies = std::get<0>(eg).view({in.B, in.n}).sum(1);
+    if (with_grad) {
+        Tensor g_rep = project_typed_backward(std::get<1>(eg), ss, off, reductors, in.types, nslots);
+        Tensor gX = at::zeros({in.B, in.n, 3}, in.X.options());
+        check(qmll_fchl19_vjp(FCHL_ABI(in), fp(g_rep), gX.data_ptr<float>(), stream()), "qmll_fchl19_vjp");
+        *gX_out = gX;
+    }
+    return energies;
+}
+
+struct FchlSorfEnergyFn : public Function<FchlSorfEnergyFn> {
+    static variable_list forward(AutogradContext* ctx, FCHL_TENSORS, MODEL_TENSORS, bool with_grad) {
+        Tensor gX;
+        Tensor e = fchl_sorf_energy_impl(FCHL_PASS, reductors, Dmat, bias, alpha, cn, nt, with_grad, &gX);
+        if (!with_grad) gX = empty_like_none(e);
+        ctx->save_for_backward({gX});
+        ctx->mark_non_differentiable({gX});
+        ctx->set_materialize_grads(false);
+        ctx->saved_data["xdim"] = X.dim();
+        return {e, gX};
+    }
+    static variable_list backward(AutogradContext* ctx, variable_list grads) {
+        variable_list out(23);
+        if (!grads[0].defined()) return out;
+        const Tensor gX = ctx->get_saved_variables()[0];                 // [B,n,3], dE_m/dX of each molecule
+        TORCH_CHECK(gX.dim() == 3, "fchl_sorf_energy was called with with_grad=False but a gradient is requested");
+        Tensor g = gX * grads[0].reshape({-1, 1, 1});
+        out[0] = ctx->saved_data["xdim"].toInt() == 2 ? g.squeeze(0) : g;
+        return out;
+    }
+};
+
+// returns (energies [B], dE/dX [B,n,3] or an empty tensor when with_grad is false)
+std::tuple<Tensor, Tensor> fchl_sorf_energy(FCHL_TENSORS, MODEL_TENSORS, bool with_grad) {
+    auto r = FchlSorfEnergyFn::apply(FCHL_PASS, reductors, Dmat, bias, alpha, cn, nt, with_grad);
+    return {r[0], r[1]};
+}
+
 }  // namespace
 
 // operator names and argument order of the reference (torchscript/FCHL19.cpp:318-333)
@@ -551,6 +611,7 @@ TORCH_LIBRARY(qml_lightning_sorf, m) {
     m.def("project_typed_backward", &project_typed_backward);
     m.def("sorf_energy_sorted", &sorf_energy_sorted);
     m.def("rff_energy_sorted", &rff_energy_sorted);
+    m.def("fchl_sorf_energy", &fchl_sorf_energy);
 }
 
 // names the loader can test for

@@ -154,6 +154,51 @@ def _register_fused_op():
 
     torch.library.register_autograd("qml_lightning_sorf::rff_energy_sorted", backward_rff, setup_context=setup_sorted,
                                     lib=lib)
+    # the whole fused chain as one operator: one dispatch and one autograd node per evaluation
+    lib.define("fchl_sorf_energy(%s, Tensor reductors, Tensor Dmat, Tensor bias, Tensor alpha, "
+               "Tensor coeff_normalisation, Tensor ntransforms, bool with_grad) -> (Tensor, Tensor)" % ops._FCHL_SIG)
+
+    def impl_chain(X, Z, species, atomIDs, molIDs, atom_counts, cell, inv_cell, Rs2, Rs3, eta2, eta3, two_body_decay,
+                   three_body_weight, three_body_decay, rcut, reductors, Dmat, bias, alpha, cn, nt, with_grad):
+        Xb, Zb = ops._batched(X, Z)
+        B, n = Zb.shape
+        nslots = B * n
+        prm = ops.make_params(species.shape[0], Rs2, Rs3, eta2, eta3, two_body_decay, three_body_weight,
+                              three_body_decay, rcut)
+        types = ops.element_types(Xb, Zb, atom_counts, species)
+        cell_ = cell if cell.numel() > 0 else None
+        inv_cell_ = inv_cell if inv_cell.numel() > 0 else None
+        fargs = (Xb, types, cell_, inv_cell_, atomIDs, molIDs, atom_counts, Rs2, Rs3, prm)
+        rep = ops.fchl_forward(*fargs)
+        tflat = types.view(-1)
+        ss, off = ops.sort_by_type(tflat, molIDs * n + atomIDs, reductors.shape[0])
+        x = ops.project_typed(rep.view(nslots, -1), ss, off, reductors)
+        e_slots, gx = ops.sorf_energy_sorted(x, off, ss, Dmat, bias, alpha, ops._scalar(cn), int(nt.item()), nslots,
+                                             with_grad=with_grad)
+        energies = e_slots.view(B, n).sum(dim=1)
+        if not with_grad:
+            return energies, torch.empty(0, dtype=torch.float32, device=X.device)
+        g_rep = ops.project_typed_backward(gx, ss, off, reductors, tflat, nslots)
+        return energies, ops.fchl_vjp(g_rep.view(rep.shape), *fargs)
+
+    lib.impl("fchl_sorf_energy", impl_chain, "CompositeExplicitAutograd")
+
+    def setup_chain(ctx, inputs, output):
+        ctx.save_for_backward(output[1])
+        ctx.xdim = inputs[0].dim()
+        ctx.set_materialize_grads(False)
+
+    def backward_chain(ctx, g_e, g_gx):
+        (gX,) = ctx.saved_tensors
+        if g_e is None:
+            return (None,) * 23
+        if gX.dim() != 3:
+            raise RuntimeError("fchl_sorf_energy was called with with_grad=False but a gradient is requested")
+        g = gX * g_e.reshape(-1, 1, 1)
+        return (g.squeeze(0) if ctx.xdim == 2 else g,) + (None,) * 22
+
+    torch.library.register_autograd("qml_lightning_sorf::fchl_sorf_energy", backward_chain, setup_context=setup_chain,
+                                    lib=lib)
     ops._libs.append(lib)
 
 
@@ -163,9 +208,10 @@ _register_fused_op()
 class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
 
     fused: Final[bool]
+    separate_ops: Final[bool]
 
     def __init__(self, rep=None, elements=np.array([1, 6, 7, 8]), ntransforms=2, sigma=3.0, llambda=1e-11, npcas=128,
-                 nbatch_train=64, nbatch_test=64, nstacks=32, fused=True):
+                 nbatch_train=64, nbatch_test=64, nstacks=32, fused=True, separate_ops=False):
         torch.nn.Module.__init__(self)
         BaseKernel.__init__(self, rep, npcas, elements, sigma, llambda)
         self.device = _default_device()
@@ -176,6 +222,7 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         self.species = torch.from_numpy(np.asarray(elements)).float().to(self.device)
         self.npcas = npcas
         self.fused = fused
+        self.separate_ops = separate_ops   # fused route as five operators (one node each) instead of one
         self.Dmat = torch.zeros((len(elements), ntransforms, nstacks, npcas), dtype=torch.float32, device=self.device)
         self.get_SORF_diagonals(elements, ntransforms, nstacks, npcas)
         self.bias = torch.zeros((len(elements), self.nfeatures()), dtype=torch.float32, device=self.device)
@@ -234,8 +281,19 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         assert inv_cell.is_cuda, "inv_cell tensor must reside on GPU"
 
         coeff_normalisation = torch.sqrt(torch.tensor(self.npcas)) / self.sigma
-        torch_rep = self.rep.forward(X, Z, atomIDs, molIDs, atom_counts, cell, inv_cell)
         alpha = self.alpha.float()
+
+        if self.fused and not self.separate_ops:
+            # the whole chain below (representation, sort by element, projection, SORF + cos +
+            # energy and, for a gradient, its backward) as ONE operator and one autograd node
+            energies, _ = torch.ops.qml_lightning_sorf.fchl_sorf_energy(
+                X, Z, self.rep.species, atomIDs, molIDs, atom_counts, cell, inv_cell, self.rep.Rs2, self.rep.Rs3,
+                self.rep.eta2, self.rep.eta3, self.rep.two_body_decay, self.rep.three_body_weight,
+                self.rep.three_body_decay, self.rep.rcut, self.reductors, self.Dmat, self.bias, alpha,
+                coeff_normalisation, self.ntransforms, X.requires_grad)
+            return energies
+
+        torch_rep = self.rep.forward(X, Z, atomIDs, molIDs, atom_counts, cell, inv_cell)
 
         if self.fused:
             # the atoms are sorted by element on the device (no host round trip for sizes);

@@ -122,6 +122,44 @@ def test_periodic_cell_energy_and_forces_both_routes():
     close(f2, F, REL_EF, "periodic forces, autograd route")
 
 
+def test_forward_routes_agree_under_autograd():
+    """forward + autograd.grad through the one-operator chain, the same chain operator by operator,
+    and the reference's two-operator route: same energies, same gradients for a weighted sum of the
+    energies (the upstream gradient differs per molecule), also for a single unbatched molecule."""
+    species = [1, 6, 8]
+    coords, charges = helpers.ragged_batch(5, 4)
+    species = [1, 6, 7, 8, 9]
+    X, Z, aid, mid, nat = make_batch(coords, charges)
+    prm = oracle_prm(species)
+    w = torch.tensor([0.5, -1.0, 2.0, 0.0, 1.5], device=dev())
+    results = []
+    for kw in (dict(fused=True), dict(fused=True, separate_ops=True), dict(fused=False)):
+        sep = kw.pop("separate_ops", False)
+        m, (red, D, bias, alpha) = build_sorf_model(species, 32, 4, **kw)
+        m.separate_ops = sep
+        gX, gZ, gaid, gmid, gnat = inputs(X, Z, aid, mid, nat)
+        gX.requires_grad_(True)
+        e = m.forward(gX, gZ, gaid, gmid, gnat)
+        g, = torch.autograd.grad((e * w).sum(), gX)
+        results.append((e.detach(), g))
+        with torch.no_grad():                                  # no gradient asked: energies only
+            e_ng = m.forward(gX.detach(), gZ, gaid, gmid, gnat)
+        assert torch.equal(e_ng, e.detach())
+    E, F, _ = omodel.sorf_energy_forces(X, Z, aid, mid, nat, prm, species, red, D, bias, alpha, 2.0)
+    for e, g in results:
+        close(e, E, REL_EF, "energies")
+        close(g, -F * w.cpu().numpy()[:, None, None], REL_EF, "weighted gradient")
+    # one molecule handed over unbatched: X [n,3], Z [n]
+    m, _ = build_sorf_model(species, 32, 4)
+    n0 = int(nat[0])
+    x1 = t32(X[0, :n0]).requires_grad_(True)
+    e1 = m.forward(x1, t32(Z[0, :n0]), ti32(aid[:n0]), ti32(mid[:n0]), ti32(nat[:1]))
+    g1, = torch.autograd.grad(e1.sum(), x1)
+    assert g1.shape == x1.shape
+    close(e1, E[:1], REL_EF, "unbatched energy")
+    close(g1, -F[0, :n0], REL_EF, "unbatched gradient")
+
+
 def test_two_transforms_and_torch_ops_directly():
     """ntransforms = 2 through the registered operators, autograd included."""
     species = [1, 6]

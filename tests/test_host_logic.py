@@ -79,7 +79,12 @@ def test_forward_compiles_to_torchscript_with_the_reference_operator_names():
         code = s.code + s.rep.code
         assert "ops.qml_lightning_fchl.fchl_forwards" in code
         if fused:
-            assert "ops.qml_lightning_sorf.sorf_energy" in code
+            assert "ops.qml_lightning_sorf.fchl_sorf_energy" in code      # the whole chain, one operator
         else:
             assert "ops.qml_lightning_sorf.get_SORF_coefficients" in code
             assert "ops.qml_lightning_sorf.get_cos_features" in code
+    m = _model(True)
+    m.separate_ops = True                                                 # the fused route operator by operator
+    code = torch.jit.script(m).code
+    for name in ("sort_by_type", "project_typed", "sorf_energy_sorted"):
+        assert "ops.qml_lightning_sorf." + name in code
