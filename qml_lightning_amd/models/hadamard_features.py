@@ -334,17 +334,19 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         """(energies [B], forces [B,n,3] or None) for device tensors through the fused route,
         asynchronously on the current stream.  The fused kernel returns dE/dx itself, so the
         forces need no autograd graph: same numbers as `forward` + `autograd.grad`."""
-        norm = float(np.sqrt(self.npcas) / self.sigma)
-        alpha = self.alpha.float()
-        T = int(self.ntransforms)
-
-        def energy_fn(x, type_offsets, sorted_slots, nslots, with_grad):
-            return ops.sorf_energy_sorted(x, type_offsets, sorted_slots, self.Dmat, self.bias, alpha, norm, T, nslots,
-                                          with_grad=with_grad)
-
+        # one call of the operator that runs the whole chain (what `forward` dispatches to), outside
+        # autograd: it returns the energies and dE/dX
+        if cells is None or inv_cells is None:
+            cells = torch.empty(0, 3, 3, device=coordinates.device)
+            inv_cells = cells
+        coeff_normalisation = torch.sqrt(torch.tensor(self.npcas)) / self.sigma
+        rep = self.rep
         with torch.no_grad():
-            return self._direct_energy_forces(coordinates.detach(), charges, atomIDs, molIDs, natom_counts, cells,
-                                              inv_cells, forces, energy_fn)
+            energies, gX = torch.ops.qml_lightning_sorf.fchl_sorf_energy(
+                coordinates, charges, rep.species, atomIDs, molIDs, natom_counts, cells, inv_cells, rep.Rs2, rep.Rs3,
+                rep.eta2, rep.eta3, rep.two_body_decay, rep.three_body_weight, rep.three_body_decay, rep.rcut,
+                self.reductors, self.Dmat, self.bias, self.alpha.float(), coeff_normalisation, self.ntransforms, forces)
+        return energies, (gX.neg_() if forces else None)
 
     @torch.jit.unused
     def predict_opt(self, coordinates, charges, atomIDs, molIDs, natom_counts, cells=None, inv_cells=None,
