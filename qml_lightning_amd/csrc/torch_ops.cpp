@@ -537,7 +537,8 @@ std::tuple<Tensor, Tensor> rff_energy_sorted(const Tensor& x, const Tensor& off,
     const Tensor &reductors, const Tensor &Dmat, const Tensor &bias, const Tensor &alpha, const Tensor &cn, \
         const Tensor &nt
 
-Tensor fchl_sorf_energy_impl(FCHL_TENSORS, MODEL_TENSORS, bool with_grad, Tensor* gX_out) {
+// rff = true: `Dmat` holds W [ne,d,F], `bias` holds b [ne,F]; cn and nt are unused
+Tensor fchl_sorf_energy_impl(FCHL_TENSORS, MODEL_TENSORS, bool with_grad, Tensor* gX_out, bool rff = false) {
     FchlInputs in = prepare(FCHL_PASS);
     Tensor rep = at::zeros({in.B, in.n, in.R}, in.X.options());
     check(qmll_fchl19_forward(FCHL_ABI(in), rep.data_ptr<float>(), stream()), "qmll_fchl19_forward");
@@ -547,7 +548,8 @@ Tensor fchl_sorf_energy_impl(FCHL_TENSORS, MODEL_TENSORS, bool with_grad, Tensor
     const Tensor& ss = std::get<0>(sorted);
     const Tensor& off = std::get<1>(sorted);
     Tensor x = project_typed_impl(rep.view({nslots, in.R}), ss, off, reductors);
-    auto eg = sorf_energy_sorted_impl(x, off, ss, Dmat, bias, alpha, cn, nt, nslots, with_grad);
+    auto eg = rff ? rff_energy_sorted_impl(x, off, ss, Dmat, bias, alpha, nslots, with_grad)
+                  : sorf_energy_sorted_impl(x, off, ss, Dmat, bias, alpha, cn, nt, nslots, with_grad);
     Tensor energies = std::get<0>(eg).view({in.B, in.n}).sum(1);
     if (with_grad) {
         Tensor g_rep = project_typed_backward(std::get<1>(eg), ss, off, reductors, in.types, nslots);
@@ -586,6 +588,36 @@ std::tuple<Tensor, Tensor> fchl_sorf_energy(FCHL_TENSORS, MODEL_TENSORS, bool wi
     return {r[0], r[1]};
 }
 
+// the same chain with random Fourier features (models/random_features.py:82-102)
+struct FchlRffEnergyFn : public Function<FchlRffEnergyFn> {
+    static variable_list forward(AutogradContext* ctx, FCHL_TENSORS, const Tensor& reductors, const Tensor& W,
+                                 const Tensor& b, const Tensor& alpha, bool with_grad) {
+        Tensor gX;
+        Tensor e = fchl_sorf_energy_impl(FCHL_PASS, reductors, W, b, alpha, Tensor(), Tensor(), with_grad, &gX, true);
+        if (!with_grad) gX = empty_like_none(e);
+        ctx->save_for_backward({gX});
+        ctx->mark_non_differentiable({gX});
+        ctx->set_materialize_grads(false);
+        ctx->saved_data["xdim"] = X.dim();
+        return {e, gX};
+    }
+    static variable_list backward(AutogradContext* ctx, variable_list grads) {
+        variable_list out(21);
+        if (!grads[0].defined()) return out;
+        const Tensor gX = ctx->get_saved_variables()[0];
+        TORCH_CHECK(gX.dim() == 3, "fchl_rff_energy was called with with_grad=False but a gradient is requested");
+        Tensor g = gX * grads[0].reshape({-1, 1, 1});
+        out[0] = ctx->saved_data["xdim"].toInt() == 2 ? g.squeeze(0) : g;
+        return out;
+    }
+};
+
+std::tuple<Tensor, Tensor> fchl_rff_energy(FCHL_TENSORS, const Tensor& reductors, const Tensor& W, const Tensor& b,
+                                           const Tensor& alpha, bool with_grad) {
+    auto r = FchlRffEnergyFn::apply(FCHL_PASS, reductors, W, b, alpha, with_grad);
+    return {r[0], r[1]};
+}
+
 }  // namespace
 
 // operator names and argument order of the reference (torchscript/FCHL19.cpp:318-333)
@@ -612,6 +644,7 @@ TORCH_LIBRARY(qml_lightning_sorf, m) {
     m.def("sorf_energy_sorted", &sorf_energy_sorted);
     m.def("rff_energy_sorted", &rff_energy_sorted);
     m.def("fchl_sorf_energy", &fchl_sorf_energy);
+    m.def("fchl_rff_energy", &fchl_rff_energy);
 }
 
 // names the loader can test for

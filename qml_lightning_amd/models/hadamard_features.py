@@ -183,6 +183,33 @@ def _register_fused_op():
 
     lib.impl("fchl_sorf_energy", impl_chain, "CompositeExplicitAutograd")
 
+    # the same chain with random Fourier features: W in place of the diagonals, b in place of the bias
+    lib.define("fchl_rff_energy(%s, Tensor reductors, Tensor W, Tensor b, Tensor alpha, bool with_grad) "
+               "-> (Tensor, Tensor)" % ops._FCHL_SIG)
+
+    def impl_chain_rff(X, Z, species, atomIDs, molIDs, atom_counts, cell, inv_cell, Rs2, Rs3, eta2, eta3,
+                       two_body_decay, three_body_weight, three_body_decay, rcut, reductors, W, b, alpha, with_grad):
+        Xb, Zb = ops._batched(X, Z)
+        B, n = Zb.shape
+        nslots = B * n
+        prm = ops.make_params(species.shape[0], Rs2, Rs3, eta2, eta3, two_body_decay, three_body_weight,
+                              three_body_decay, rcut)
+        types = ops.element_types(Xb, Zb, atom_counts, species)
+        fargs = (Xb, types, cell if cell.numel() > 0 else None, inv_cell if inv_cell.numel() > 0 else None, atomIDs,
+                 molIDs, atom_counts, Rs2, Rs3, prm)
+        rep = ops.fchl_forward(*fargs)
+        tflat = types.view(-1)
+        ss, off = ops.sort_by_type(tflat, molIDs * n + atomIDs, reductors.shape[0])
+        x = ops.project_typed(rep.view(nslots, -1), ss, off, reductors)
+        e_slots, gx = ops.rff_energy_sorted(x, off, ss, W, b, alpha, nslots, with_grad=with_grad)
+        energies = e_slots.view(B, n).sum(dim=1)
+        if not with_grad:
+            return energies, torch.empty(0, dtype=torch.float32, device=X.device)
+        g_rep = ops.project_typed_backward(gx, ss, off, reductors, tflat, nslots)
+        return energies, ops.fchl_vjp(g_rep.view(rep.shape), *fargs)
+
+    lib.impl("fchl_rff_energy", impl_chain_rff, "CompositeExplicitAutograd")
+
     def setup_chain(ctx, inputs, output):
         ctx.save_for_backward(output[1])
         ctx.xdim = inputs[0].dim()
@@ -199,6 +226,18 @@ def _register_fused_op():
 
     torch.library.register_autograd("qml_lightning_sorf::fchl_sorf_energy", backward_chain, setup_context=setup_chain,
                                     lib=lib)
+
+    def backward_chain_rff(ctx, g_e, g_gx):
+        (gX,) = ctx.saved_tensors
+        if g_e is None:
+            return (None,) * 21
+        if gX.dim() != 3:
+            raise RuntimeError("fchl_rff_energy was called with with_grad=False but a gradient is requested")
+        g = gX * g_e.reshape(-1, 1, 1)
+        return (g.squeeze(0) if ctx.xdim == 2 else g,) + (None,) * 20
+
+    torch.library.register_autograd("qml_lightning_sorf::fchl_rff_energy", backward_chain_rff,
+                                    setup_context=setup_chain, lib=lib)
     ops._libs.append(lib)
 
 

@@ -18,14 +18,17 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
     [atoms, nfeatures] matrix; `fused=False` is the reference's own operator sequence."""
 
     fused: Final[bool]
+    separate_ops: Final[bool]
 
     def __init__(self, rep=None, elements=np.array([1, 6, 7, 8]), sigma=2.0, llambda=1e-10,
-                 nstacks=8192, npcas=128, nbatch_train=64, nbatch_test=64, fused=True):
+                 nstacks=8192, npcas=128, nbatch_train=64, nbatch_test=64, fused=True,
+                 separate_ops=False):
         torch.nn.Module.__init__(self)
         BaseKernel.__init__(self, rep, npcas, elements, sigma, llambda)
         self.device = _default_device()
         self.npcas = npcas
         self.fused = bool(fused) and npcas in (64, 128) and (nstacks * npcas) % 32 == 0
+        self.separate_ops = separate_ops   # fused route as five operators (one node each) instead of one
         self.nbatch_train = nbatch_train
         self.nbatch_test = nbatch_test
         self._nfeatures = nstacks * self.npcas
@@ -69,6 +72,14 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
             inv_cell = torch.empty(0, 3, 3, device=X.device)
         assert X.is_cuda, "X tensor must reside on GPU"
         assert Z.is_cuda, "Z tensor must reside on GPU"
+        if self.fused and not self.separate_ops:
+            # the whole chain below as ONE operator and one autograd node
+            energies, _ = torch.ops.qml_lightning_sorf.fchl_rff_energy(
+                X, Z, self.rep.species, atomIDs, molIDs, atom_counts, cell, inv_cell, self.rep.Rs2, self.rep.Rs3,
+                self.rep.eta2, self.rep.eta3, self.rep.two_body_decay, self.rep.three_body_weight,
+                self.rep.three_body_decay, self.rep.rcut, self.reductors, self.W, self.b, self.alpha.float(),
+                X.requires_grad)
+            return energies
         torch_rep = self.rep.forward(X, Z, atomIDs, molIDs, atom_counts, cell, inv_cell)
         if self.fused:
             # atoms sorted by element on the device, projected with their own reductor into
@@ -103,15 +114,16 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
         """(energies [B], forces [B,n,3] or None) for device tensors through the fused route,
         asynchronously on the current stream; no autograd graph (the fused kernel returns
         dE/dx itself)."""
-        alpha = self.alpha.float()
-
-        def energy_fn(x, type_offsets, sorted_slots, nslots, with_grad):
-            return ops.rff_energy_sorted(x, type_offsets, sorted_slots, self.W, self.b, alpha, nslots,
-                                         with_grad=with_grad)
-
+        if cells is None or inv_cells is None:
+            cells = torch.empty(0, 3, 3, device=coordinates.device)
+            inv_cells = cells
+        rep = self.rep
         with torch.no_grad():
-            return self._direct_energy_forces(coordinates.detach(), charges, atomIDs, molIDs, natom_counts, cells,
-                                              inv_cells, forces, energy_fn)
+            energies, gX = torch.ops.qml_lightning_sorf.fchl_rff_energy(
+                coordinates, charges, rep.species, atomIDs, molIDs, natom_counts, cells, inv_cells, rep.Rs2, rep.Rs3,
+                rep.eta2, rep.eta3, rep.two_body_decay, rep.three_body_weight, rep.three_body_decay, rep.rcut,
+                self.reductors, self.W, self.b, self.alpha.float(), forces)
+        return energies, (gX.neg_() if forces else None)
 
     @torch.jit.unused
     def predict_opt(self, coordinates, charges, atomIDs, molIDs, natom_counts, zcells=None, zinv_cells=None,

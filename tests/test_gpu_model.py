@@ -465,6 +465,13 @@ def test_rff_fused_forward_vs_oracle(npcas, nstacks, case):
     f2, = torch.autograd.grad(-e2.sum(), gX)
     close(e2, E, REL_EF, "scripted fused rff energies")
     close(f2, F, REL_EF, "scripted fused rff forces")
+    # the same chain operator by operator
+    m.separate_ops = True
+    gX3 = t32(X).requires_grad_(True)
+    e3 = m.forward(gX3, t32(Z), ti32(aid), ti32(mid), ti32(nat))
+    f3, = torch.autograd.grad(-e3.sum(), gX3)
+    close(e3, E, REL_EF, "rff energies, separate operators")
+    close(f3, F, REL_EF, "rff forces, separate operators")
 
 
 def test_fd_helper_matches_jacobian():

@@ -96,7 +96,8 @@ def test_cpp_operator_library_registers_every_operator():
         assert hasattr(torch.ops.qml_lightning_fchl, name), name
     for name in ("get_SORF_coefficients", "get_SORF_coefficients_backward", "get_cos_features",
                  "get_cos_features_backward", "sorf_energy", "sorf_energy_typed", "sort_by_type", "project_typed",
-                 "project_typed_backward", "sorf_energy_sorted", "rff_energy_sorted", "fchl_sorf_energy"):
+                 "project_typed_backward", "sorf_energy_sorted", "rff_energy_sorted", "fchl_sorf_energy",
+                 "fchl_rff_energy"):
         assert hasattr(torch.ops.qml_lightning_sorf, name), name
     # schemas as TorchScript sees them: positional tensors, as in the reference
     schema = str(torch.ops.qml_lightning_fchl.fchl_forwards.default._schema)
