@@ -51,33 +51,6 @@ class BaseKernel():
         raise NotImplementedError("Abstract method only.")
 
     # -- rows of one batch ----------------------------------------------------------------
-    def _direct_energy_forces(self, X, Z, atomIDs, molIDs, natom_counts, cells, inv_cells, forces, energy_fn):
-        """Energies [B] and, with `forces`, forces [B,n,3] = -dE/dX of the element-sorted fused
-        route, as a straight chain of kernel launches: representation, sort by element,
-        projection, `energy_fn(x, type_offsets, sorted_slots, nslots, with_grad)` -> (per-slot
-        energies, dE/dx), projection transpose, representation VJP.  The same numbers as
-        `forward` + `autograd.grad` (the fused kernel already returns dE/dx), without the
-        autograd graph: 0.13 ms instead of 0.65 ms for a single molecule."""
-        rep = self.rep
-        X, Z = ops._batched(X, Z)
-        B, n = Z.shape
-        nslots = B * n
-        prm = ops.make_params(rep.nspecies, rep.Rs2, rep.Rs3, rep.eta2, rep.eta3, rep.two_body_decay,
-                              rep.three_body_weight, rep.three_body_decay, rep.rcut)
-        types = ops.element_types(X, Z, natom_counts, rep.species)
-        fargs = (X, types, cells, inv_cells, atomIDs, molIDs, natom_counts, rep.Rs2, rep.Rs3, prm)
-        representation = ops.fchl_forward(*fargs)
-        tflat = types.view(-1)
-        sorted_slots, type_offsets = ops.sort_by_type(tflat, molIDs * n + atomIDs, self.reductors.shape[0])
-        x = ops.project_typed(representation.view(nslots, -1), sorted_slots, type_offsets, self.reductors)
-        e_slots, gx = energy_fn(x, type_offsets, sorted_slots, nslots, forces)
-        energies = e_slots.view(B, n).sum(dim=1)
-        if not forces:
-            return energies, None
-        g_rep = ops.project_typed_backward(gx, sorted_slots, type_offsets, self.reductors, tflat, nslots)
-        gX = ops.fchl_vjp(g_rep.view(representation.shape), *fargs)
-        return energies, gX.neg_()
-
     def _batch_rows(self, data, with_forces, zero_energy_rows=False):
         """fp64 row matrix [B (+ B*n*3), F] of one formatted batch: B energy rows, then the
         B*n*3 force rows in (molecule, atom, xyz) order (kernel.py:134-170)."""
