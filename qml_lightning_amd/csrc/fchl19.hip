@@ -777,6 +777,12 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
 // in an LDS row buffer and streams them out coalesced.  For a neighbour target only the
 // triples that contain it contribute; for the self row all triples do.
 // ---------------------------------------------------------------------------------
+// TABLE: everything of a triple that does not depend on the radial bin (geometry, the partials of
+// the angular and decay factors, the unit vectors) is computed once per triple into an LDS table
+// of JT floats; the (triple, radial bin) items of every target pass then only read it.  Without
+// the table each item recomputes its triple, nRs3 times over and again in the neighbour passes.
+constexpr int JT = 20;   // rho, bin offset, 6 alpha, 2 beta, u_ij, u_ik, u_jk, pad
+template <bool TABLE>
 __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* __restrict__ rep,
                                                               float* __restrict__ jac) {
     extern __shared__ float smem[];
@@ -793,6 +799,8 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
     float* sRs3 = sinvRs2 + nRs2;    // [nRs3]
     float* row = sRs3 + nRs3;        // [3][R] rows being assembled (+ [R] value row)
     float* val = row + 3 * R;        // [R]   representation row (self pass only)
+    // TABLE: [ntrip][JT], 16-byte aligned behind the rows
+    float* ttab = val + R + ((4 - ((size_t)(val + R - smem) & 3)) & 3);
 
     for (int t = lane; t < nRs2; t += QMLL_WAVE) {
         const float v = a.Rs2[t];
@@ -806,6 +814,34 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
     const float k3 = a.p.eta3 * LOG2E;
     const float zeta2 = 0.014383766711652736f;   // 2 exp(-pi^2 / 2)
     float* jbase = jac + (((size_t)m * a.n + i) * a.n) * 3 * R;
+
+    if constexpr (TABLE) {
+        // T_c = zeta2 K e cosT, T_s = zeta2 K e sinT with e = exp(-eta3 (rho - Rs_l)^2): their partials
+        // with respect to the three distances are e * alpha + (de/drho) * beta, alpha and beta per triple
+        const int ntrip = nn * (nn - 1) / 2;
+        for (int tt = lane; tt < ntrip; tt += QMLL_WAVE) {
+            int j, k;
+            unrank_pair(tt, nn, j, k);
+            const Triple t = triple_geometry(s, j, k);
+            const TripleDeriv d = triple_derivatives(t, a.p, s.fc[j], s.dfc[j], s.fc[k], s.dfc[k]);
+            const float dcos = t.sinT * t.guard_inv;       // d cosT = dcos * d cos_i
+            const float dsin = -t.cosT * t.guard_inv;      // d sinT = dsin * d cos_i
+            const float ia = 1.0f / t.a, ib = 1.0f / t.b;
+            float4* e4 = reinterpret_cast<float4*>(ttab + (size_t)tt * JT);
+            e4[0] = make_float4(0.5f * (t.a + t.b),
+                                __int_as_float(pair_offset(s.el[j], s.el[k], ns, nRs2, nRs3)),
+                                zeta2 * (d.Ka * t.cosT + d.K * dcos * d.cia),
+                                zeta2 * (d.Kb * t.cosT + d.K * dcos * d.cib));
+            e4[1] = make_float4(zeta2 * (d.Kc * t.cosT + d.K * dcos * d.cic),
+                                zeta2 * (d.Ka * t.sinT + d.K * dsin * d.cia),
+                                zeta2 * (d.Kb * t.sinT + d.K * dsin * d.cib),
+                                zeta2 * (d.Kc * t.sinT + d.K * dsin * d.cic));
+            e4[2] = make_float4(zeta2 * d.K * t.cosT, zeta2 * d.K * t.sinT, s.dx[j] * ia, s.dy[j] * ia);
+            e4[3] = make_float4(s.dz[j] * ia, s.dx[k] * ib, s.dy[k] * ib, s.dz[k] * ib);
+            e4[4] = make_float4(t.ujk[0], t.ujk[1], t.ujk[2], 0.0f);
+        }
+        __syncthreads();
+    }
 
     // target = -1: central atom; target = 0..nn-1: neighbour at that list position
     for (int target = -1; target < nn; ++target) {
@@ -834,8 +870,114 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
                 if (target < 0) atomicAdd(&val[bin], v);
             }
         }
-        // three-body: items (triple, radial bin l)
-        {
+        // three-body with the table: owner computes.  Lanes = (triple sub-slot, radial bin l); a lane
+        // sums its bin over the triples of one element pair in registers (no LDS atomics, which run
+        // at one lane per clock), sub-slots are folded with shuffles, sub-slot 0 stores the bin.
+        if constexpr (TABLE) {
+            const int W3 = nRs3 < 64 ? nRs3 : 64;
+            const int TS = 64 / W3;
+            const int tsub = lane / W3, ll = lane - tsub * W3;
+            // the triples of one block: index it -> neighbour positions j < k
+            auto block = [&](int off_pair, int count, int p, int q) {
+                const int op = s.goff[p], oq = s.goff[q];
+                const int np_ = s.goff[p + 1] - op, nq = s.goff[q + 1] - oq;
+                for (int lb = 0; lb * 64 < nRs3; ++lb) {
+                    const int l = lb * 64 + ll;
+                    const bool lok = l < nRs3 && tsub < TS;
+                    const float rs = sRs3[lok ? l : 0];
+                    float gc[3] = {0.f, 0.f, 0.f}, gs[3] = {0.f, 0.f, 0.f}, vc = 0.f, vs = 0.f;
+                    for (int it = tsub; it < count && lok; it += TS) {
+                        int j, k;
+                        if (target < 0) {
+                            if (p == q) {
+                                unrank_pair(it, np_, j, k);
+                                j += op;
+                                k += op;
+                            } else {
+                                j = op + it / nq;
+                                k = oq + it - (it / nq) * nq;
+                            }
+                        } else {   // q is the element of the other neighbour o; p that of the target
+                            int o = oq + it;
+                            if (p == q && o >= target) ++o;
+                            j = o < target ? o : target;
+                            k = o < target ? target : o;
+                        }
+                        const float4* e4 = reinterpret_cast<const float4*>(
+                            ttab + (size_t)((j * (2 * nn - j - 1)) / 2 + (k - j - 1)) * JT);
+                        const float4 q0 = e4[0], q1 = e4[1], q2 = e4[2], q3 = e4[3], q4 = e4[4];
+                        const float dl = q0.x - rs;
+                        const float e = fexp2(-k3 * dl * dl);
+                        const float de = -a.p.eta3 * dl * e;      // (d e/d rho) * (d rho/d a)
+                        const float Tca = fmaf(e, q0.z, de * q2.x), Tcb = fmaf(e, q0.w, de * q2.x), Tcc = e * q1.x;
+                        const float Tsa = fmaf(e, q1.y, de * q2.y), Tsb = fmaf(e, q1.z, de * q2.y), Tsc = e * q1.w;
+                        const float ua[3] = {q2.z, q2.w, q3.x};
+                        const float ub[3] = {q3.y, q3.z, q3.w};
+                        const float uc[3] = {q4.x, q4.y, q4.z};
+                        if (target < 0) {            // d/dR_i, and the value itself
+                            vc = fmaf(e, q2.x, vc);
+                            vs = fmaf(e, q2.y, vs);
+#pragma unroll
+                            for (int x = 0; x < 3; ++x) {
+                                gc[x] += Tca * ua[x] + Tcb * ub[x];
+                                gs[x] += Tsa * ua[x] + Tsb * ub[x];
+                            }
+                        } else if (j == target) {    // d/dR_j
+#pragma unroll
+                            for (int x = 0; x < 3; ++x) {
+                                gc[x] += -Tca * ua[x] + Tcc * uc[x];
+                                gs[x] += -Tsa * ua[x] + Tsc * uc[x];
+                            }
+                        } else {                     // d/dR_k
+#pragma unroll
+                            for (int x = 0; x < 3; ++x) {
+                                gc[x] += -Tcb * ub[x] - Tcc * uc[x];
+                                gs[x] += -Tsb * ub[x] - Tsc * uc[x];
+                            }
+                        }
+                    }
+                    // fold the sub-slots: totals apart from the partial sums the other lanes read
+                    float tc[3] = {gc[0], gc[1], gc[2]}, tsn[3] = {gs[0], gs[1], gs[2]}, tvc = vc, tvs = vs;
+                    for (int kk = 1; kk < TS; ++kk) {
+                        const int src = ll + W3 * kk;
+#pragma unroll
+                        for (int x = 0; x < 3; ++x) {
+                            tc[x] += __shfl(gc[x], src, 64);
+                            tsn[x] += __shfl(gs[x], src, 64);
+                        }
+                        tvc += __shfl(vc, src, 64);
+                        tvs += __shfl(vs, src, 64);
+                    }
+                    if (tsub == 0 && l < nRs3) {
+                        const int off = off_pair + 2 * l;
+#pragma unroll
+                        for (int x = 0; x < 3; ++x) {
+                            row[x * R + off] = tc[x];
+                            row[x * R + off + 1] = tsn[x];
+                        }
+                        if (target < 0) {
+                            val[off] = tvc;
+                            val[off + 1] = tvs;
+                        }
+                    }
+                }
+            };
+            if (target < 0) {
+                for (int p = 0; p < ns; ++p) {
+                    const int np_ = s.goff[p + 1] - s.goff[p];
+                    for (int q = p; q < ns; ++q) {
+                        const int nq = s.goff[q + 1] - s.goff[q];
+                        block(pair_offset(p, q, ns, nRs2, nRs3), p == q ? np_ * (np_ - 1) / 2 : np_ * nq, p, q);
+                    }
+                }
+            } else {
+                const int p = s.el[target];
+                for (int q = 0; q < ns; ++q) {
+                    const int nq = s.goff[q + 1] - s.goff[q];
+                    block(pair_offset(p, q, ns, nRs2, nRs3), nq - (p == q ? 1 : 0), p, q);
+                }
+            }
+        } else {
             // self: all pairs (j<k); neighbour target: the nn-1 pairs {target, other}
             const int ntr = target < 0 ? nn * (nn - 1) / 2 : nn - 1;
             for (int it = lane; it < ntr * nRs3; it += QMLL_WAVE) {
@@ -1019,11 +1161,20 @@ extern "C" int qmll_fchl19_jacobian(const float* X, const int* types, const floa
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(jac != nullptr, QMLL_ERR_INVALID, "qmll_fchl19_jacobian: null output");
     const int R = prm->nspecies * prm->nRs2 + prm->nspecies * (prm->nspecies + 1) * prm->nRs3;
-    const size_t lds = sizeof(float) * ((size_t)STAGE_ARRAYS * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 + 4 * (size_t)R);
+    size_t lds = sizeof(float) * ((size_t)STAGE_ARRAYS * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 + 4 * (size_t)R);
     QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
                  "qmll_fchl19_jacobian: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R,
                  LDS_LIMIT);
-    hipLaunchKernelGGL(fchl19_jacobian_kernel, dim3(A), dim3(64), lds, (hipStream_t)stream, a, rep, jac);
+    // per-triple table while it fits: an atom has at most cap neighbours from a given list and at
+    // most max_atoms - 1 otherwise
+    const size_t maxnn = nlist ? (size_t)a.cap : (size_t)(a.cap > 1 ? a.cap - 1 : 1);
+    const size_t table = sizeof(float) * (JT * (maxnn * (maxnn - 1) / 2) + 4);
+    if (lds + table <= LDS_LIMIT) {
+        lds += table;
+        hipLaunchKernelGGL(fchl19_jacobian_kernel<true>, dim3(A), dim3(64), lds, (hipStream_t)stream, a, rep, jac);
+    } else {
+        hipLaunchKernelGGL(fchl19_jacobian_kernel<false>, dim3(A), dim3(64), lds, (hipStream_t)stream, a, rep, jac);
+    }
     QMLL_CHECK_LAUNCH("qmll_fchl19_jacobian");
     return QMLL_OK;
 }
