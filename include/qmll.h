@@ -176,6 +176,25 @@ int qmll_derivative_features(const double* cos_derivs, double normalisation, con
                              const int* seg_offsets, const float* input_derivative, const float* D,
                              int A, int n, int d, int S, int T, int nmol, double* G, qmll_stream_t stream);
 
+/* One element's inputs of qmll_derivative_features_typed: sine coefficients f64 [A_e, S*d], projected
+ * Jacobian rows f32 [A_e, n, 3, d], sign diagonals f32 [T, S, d], and the first atom of each molecule
+ * in the element's molecule-major atom list, i32 [nmol + 1] (all device pointers). */
+typedef struct {
+    const double* cos_derivs;
+    const float* input_derivative;
+    const float* D;
+    const int* seg_offsets;
+} qmll_df_element;
+
+/* qmll_derivative_features for every element of the batch in ONE launch (the loop over elements of
+ * calculate_features, qml_lightning/models/hadamard_features.py:66-80, around
+ * compute_molecular_featurization_derivative, cuda/hadamard_kernel.cu:587-717): G f64 [nmol, n, 3, S*d]
+ * += the force-feature rows of all `ne` elements (host array `elements`, ne <= 8), each G element read
+ * and written once; with overwrite != 0, G = those rows (never read, so it need not be cleared first:
+ * the reference's loop starts from torch.zeros, kernel.py:134-137).  64 <= d <= 256. */
+int qmll_derivative_features_typed(const qmll_df_element* elements, int ne, double normalisation, int n, int d, int S,
+                                   int T, int nmol, int overwrite, double* G, qmll_stream_t stream);
+
 /* Fused predict path for one element: SORF (T = ntransforms) + cos features + energy
  * contraction + the gradient with respect to the projected representation, without ever
  * materialising the [A,F] coefficients.  The result equals the chain

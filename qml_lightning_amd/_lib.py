@@ -23,6 +23,11 @@ class FchlParams(Structure):
                 ("rcut", c_float)]
 
 
+class DfElement(Structure):
+    """Mirror of struct qmll_df_element (device pointers)."""
+    _fields_ = [("cos_derivs", c_void_p), ("input_derivative", c_void_p), ("D", c_void_p), ("seg_offsets", c_void_p)]
+
+
 P = c_void_p  # every device pointer and the stream travel as void*
 _FCHL_COMMON = [P, P, P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, P, P, POINTER(FchlParams)]
 
@@ -44,6 +49,7 @@ PROTOTYPES = {
     "qmll_cos_features_backward": [P, P, P, P, c_int, c_int, c_int, P, P],
     "qmll_sin_coeffs_f64": [P, P, c_int, c_int, P, P],
     "qmll_derivative_features": [P, c_double, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, P],
+    "qmll_derivative_features_typed": [POINTER(DfElement), c_int, c_double, c_int, c_int, c_int, c_int, c_int, c_int, P, P],
     "qmll_sorf_energy_fused": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_float, P, P, P],
     "qmll_sorf_energy_typed": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, P, P, P],
     "qmll_sort_by_type_workspace": [c_int, c_int],

@@ -1045,6 +1045,154 @@ __global__ __launch_bounds__(SORF_THREADS) void derivative_features_rows_kernel(
     }
 }
 
+// All elements of a batch in one launch.  The per-element form above walks G once per element
+// and per chunk of DF_AC atoms (read + write of the molecule's 3n x F block each time: four
+// passes for C9H8O4), which is what bounds it.  Here a workgroup owns (molecule, four stacks):
+// the sine coefficients of ALL the molecule's atoms for those stacks sit in LDS (read from
+// memory once), its wavefronts share out the 3n target rows, each row's sum over the atoms
+// stays in registers, and every G element is written once (overwrite) or read and written once.
+// Workgroup ids are dealt round-robin over the 8 XCDs, so the id keeps a molecule's stack
+// groups on one XCD: the molecule's projected Jacobian rows (read by every stack group) then
+// come out of that XCD's L2.
+constexpr int DF_MAXE = 8;
+constexpr int DFT_THREADS = 512;
+constexpr int DFT_WAVES = DFT_THREADS / 64;
+constexpr int DFT_LDS_BYTES = 64 * 1024;      // most that one workgroup takes; a molecule with more atoms takes several passes
+struct DfElements {
+    const double* cd[DF_MAXE];   // sine coefficients [A_e, F]
+    const float* id[DF_MAXE];    // projected Jacobian rows [A_e, n, 3, d]
+    const float* D[DF_MAXE];     // sign diagonals [T, S, d]
+    const int* seg[DF_MAXE];     // first atom of each molecule in the element's list [nmol + 1]
+    int ne;
+};
+
+template <int LOG2D>
+__global__ __launch_bounds__(DFT_THREADS) void derivative_features_typed_rows_kernel(
+    DfElements E, double normalisation, int n, int S, int T, float hscale, int nmol, int ngroups, int cap,
+    int overwrite, double* __restrict__ G) {
+    constexpr int d = 1 << LOG2D;
+    constexpr int EPL = d / 16;
+    constexpr int Q = EPL / 4;
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    extern __shared__ f4 dft_cdv[];              // [cap][Q][64 lanes]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const RowLanes<EPL> L(lane);
+    const int b = blockIdx.x;
+    const int mol = (b / (8 * ngroups)) * 8 + (b & 7);
+    if (mol >= nmol) return;
+    const int sb = ((b >> 3) % ngroups) * 4;
+    const bool live = sb + L.row < S;
+    const int s = min(sb + L.row, S - 1);
+    const size_t F = (size_t)S * d;
+    const double scale = normalisation * (double)hscale;
+    const int nrows = 3 * n;
+    const size_t rstride = (size_t)n * 3 * d;    // between the Jacobian rows of consecutive atoms
+    int ntot = 0;
+    for (int e = 0; e < E.ne; ++e) ntot += E.seg[e][mol + 1] - E.seg[e][mol];
+    int c0 = 0;
+    do {
+        const int c1 = min(c0 + cap, ntot);
+        if (c0 > 0) __syncthreads();
+        // sine coefficients of atoms c0..c1 (counted element by element) -> LDS, sign folded in
+        int base = 0;
+        for (int e = 0; e < E.ne; ++e) {
+            const int a0 = E.seg[e][mol], cnt = E.seg[e][mol + 1] - a0;
+            const int lo = max(c0, base), hi = min(c1, base + cnt);
+            for (int t = lo + ((wave - (lo - c0)) & (DFT_WAVES - 1)); t < hi; t += DFT_WAVES) {
+                const double* src = E.cd[e] + (size_t)(a0 + t - base) * F + (size_t)s * d + L.e0;
+#pragma unroll
+                for (int q = 0; q < Q; ++q) {
+                    const double2 x = *reinterpret_cast<const double2*>(src + q * 64);
+                    const double2 y = *reinterpret_cast<const double2*>(src + q * 64 + 2);
+                    f4 c = {(float)x.x * L.sigma, (float)x.y * L.sigma, (float)y.x * L.sigma, (float)y.y * L.sigma};
+                    dft_cdv[((t - c0) * Q + q) * 64 + lane] = c;
+                }
+            }
+            base += cnt;
+        }
+        __syncthreads();
+        for (int jx = wave; jx < nrows; jx += DFT_WAVES) {
+            float acc[EPL];
+#pragma unroll
+            for (int p = 0; p < EPL; ++p) acc[p] = 0.0f;
+            bool any = false;
+            base = 0;
+            for (int e = 0; e < E.ne; ++e) {
+                const int a0 = E.seg[e][mol], cnt = E.seg[e][mol + 1] - a0;
+                const int lo = max(c0, base), hi = min(c1, base + cnt);
+                if (lo < hi) {
+                    const float* De = E.D[e];
+                    float dv[EPL];
+                    load_row<EPL>(dv, De + (size_t)s * d + L.e0);         // first diagonal of the chain
+                    const float* row = E.id[e] + ((size_t)(a0 + lo - base) * n * 3 + jx) * d + L.e0;
+                    float v[EPL];
+                    load_row<EPL>(v, row);
+                    for (int t = lo; t < hi; ++t) {
+                        float vn[EPL];                                     // next atom's row, in flight
+                        row += rstride;
+                        if (t + 1 < hi) {
+                            load_row<EPL>(vn, row);
+                        } else {
+#pragma unroll
+                            for (int p = 0; p < EPL; ++p) vn[p] = 0.0f;
+                        }
+                        float nz = 0.0f;
+#pragma unroll
+                        for (int p = 0; p < EPL; ++p) nz += fabsf(v[p]);
+                        if (__ballot(nz != 0.0f) != 0ull) {                // an all-zero row adds nothing
+                            any = true;
+#pragma unroll
+                            for (int p = 0; p < EPL; ++p) v[p] *= dv[p];
+                            register_stages<EPL>(v);
+                            row_stages<EPL>(v, L.cs);
+                            for (int m = 1; m < T; ++m) {
+                                float dm[EPL];
+                                load_row<EPL>(dm, De + ((size_t)m * S + s) * d + L.e0);
+#pragma unroll
+                                for (int p = 0; p < EPL; ++p) v[p] *= dm[p] * L.sigma;
+                                register_stages<EPL>(v);
+                                row_stages<EPL>(v, L.cs);
+                            }
+#pragma unroll
+                            for (int q = 0; q < Q; ++q) {
+                                const f4 c = dft_cdv[((t - c0) * Q + q) * 64 + lane];
+                                acc[4 * q] = fmaf(c[0], v[4 * q], acc[4 * q]);
+                                acc[4 * q + 1] = fmaf(c[1], v[4 * q + 1], acc[4 * q + 1]);
+                                acc[4 * q + 2] = fmaf(c[2], v[4 * q + 2], acc[4 * q + 2]);
+                                acc[4 * q + 3] = fmaf(c[3], v[4 * q + 3], acc[4 * q + 3]);
+                            }
+                        }
+#pragma unroll
+                        for (int p = 0; p < EPL; ++p) v[p] = vn[p];
+                    }
+                }
+                base += cnt;
+            }
+            const bool fresh = overwrite && c0 == 0;                       // G holds nothing yet
+            if (live && (any || fresh)) {
+                double* g = G + (((size_t)mol * n) * 3 + jx) * F + (size_t)s * d + L.e0;
+#pragma unroll
+                for (int q = 0; q < Q; ++q) {
+                    double2* gq = reinterpret_cast<double2*>(g + q * 64);
+                    double2 lo2 = {0.0, 0.0}, hi2 = {0.0, 0.0};
+                    if (!fresh) {
+                        lo2 = gq[0];
+                        hi2 = gq[1];
+                    }
+                    lo2.x += scale * (double)acc[4 * q];
+                    lo2.y += scale * (double)acc[4 * q + 1];
+                    hi2.x += scale * (double)acc[4 * q + 2];
+                    hi2.y += scale * (double)acc[4 * q + 3];
+                    gq[0] = lo2;
+                    gq[1] = hi2;
+                }
+            }
+        }
+        c0 += cap;
+    } while (c0 < ntot);
+}
+
 // ---- elementwise feature kernels ----------------------------------------------------
 // Thread = V consecutive feature columns (V = 4: 16-byte loads/stores; V = 1 when F is not
 // a multiple of 4), workgroup = (atom chunk, feature tile).  The forward kernel keeps a
@@ -1445,6 +1593,59 @@ extern "C" int qmll_derivative_features(const double* cos_derivs, double normali
 #undef CALL
     }
     QMLL_CHECK_LAUNCH("qmll_derivative_features");
+    return QMLL_OK;
+}
+
+extern "C" int qmll_derivative_features_typed(const qmll_df_element* elements, int ne, double normalisation, int n,
+                                              int d, int S, int T, int nmol, int overwrite, double* G,
+                                              qmll_stream_t stream) {
+    int rc = check_sorf("qmll_derivative_features_typed", 0, d, S, T);
+    if (rc) return rc;
+    QMLL_REQUIRE(n >= 0 && nmol >= 0 && ne >= 0, QMLL_ERR_INVALID,
+                 "qmll_derivative_features_typed: bad size n=%d nmol=%d ne=%d", n, nmol, ne);
+    QMLL_REQUIRE(ne <= DF_MAXE, QMLL_ERR_INVALID, "qmll_derivative_features_typed: at most %d elements per call (got %d)",
+                 DF_MAXE, ne);
+    QMLL_REQUIRE(d >= 64 && d <= 256, QMLL_ERR_INVALID,
+                 "qmll_derivative_features_typed: projected dimension %d outside [64, 256]", d);
+    if (n == 0 || nmol == 0) return QMLL_OK;
+    if (ne == 0 && !overwrite) return QMLL_OK;       // with overwrite, no element still means G = 0
+    QMLL_REQUIRE(G && (elements || ne == 0), QMLL_ERR_INVALID, "qmll_derivative_features_typed: null pointer");
+    DfElements E;
+    E.ne = ne;
+    for (int e = 0; e < ne; ++e) {
+        QMLL_REQUIRE(elements[e].cos_derivs && elements[e].input_derivative && elements[e].D && elements[e].seg_offsets,
+                     QMLL_ERR_INVALID, "qmll_derivative_features_typed: null pointer in element %d", e);
+        E.cd[e] = elements[e].cos_derivs;
+        E.id[e] = elements[e].input_derivative;
+        E.D[e] = elements[e].D;
+        E.seg[e] = elements[e].seg_offsets;
+    }
+    for (int e = ne; e < DF_MAXE; ++e) {
+        E.cd[e] = nullptr;
+        E.id[e] = nullptr;
+        E.D[e] = nullptr;
+        E.seg[e] = nullptr;
+    }
+    const float hscale = hnorm(d, T);
+    const int ngroups = (S + 3) / 4;
+    const int per_atom = 4 * d * (int)sizeof(float);             // LDS bytes of one atom's four stacks
+    int cap = DFT_LDS_BYTES / per_atom;               // atoms per pass over the target rows
+    if (cap > n) cap = n;
+    const long long nblocks = (long long)((nmol + 7) / 8) * 8 * ngroups;
+    QMLL_REQUIRE(nblocks <= 0x7fffffffLL, QMLL_ERR_INVALID,
+                 "qmll_derivative_features_typed: %d molecules x %d stacks exceed the grid", nmol, S);
+    const dim3 grid((unsigned)nblocks);
+    const size_t lds = (size_t)cap * per_atom;
+#define CALL(L)                                                                                                    \
+    hipLaunchKernelGGL(derivative_features_typed_rows_kernel<L>, grid, dim3(DFT_THREADS), lds, (hipStream_t)stream, \
+                       E, normalisation, n, S, T, hscale, nmol, ngroups, cap, overwrite, G)
+    switch (qmll_log2(d)) {
+        case 6: CALL(6); break;
+        case 7: CALL(7); break;
+        default: CALL(8); break;
+    }
+#undef CALL
+    QMLL_CHECK_LAUNCH("qmll_derivative_features_typed");
     return QMLL_OK;
 }
 

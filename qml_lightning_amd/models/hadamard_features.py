@@ -262,6 +262,7 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         self.npcas = npcas
         self.fused = fused
         self.separate_ops = separate_ops   # fused route as five operators (one node each) instead of one
+        self._pending_derivative_features = []
         self.Dmat = torch.zeros((len(elements), ntransforms, nstacks, npcas), dtype=torch.float32, device=self.device)
         self.get_SORF_diagonals(elements, ntransforms, nstacks, npcas)
         self.bias = torch.zeros((len(elements), self.nfeatures()), dtype=torch.float32, device=self.device)
@@ -300,9 +301,27 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         if derivative_features is not None and grad is not None:
             cos_derivs = torch.empty(coeffs.shape, device=coeffs.device, dtype=torch.float64)
             compute_partial_feature_derivatives(coeffs, self.bias[element_idx], cos_derivs)
+            if self._queue_force_rows:
+                # all elements go through ONE launch once the batch's loop over elements is done
+                # (finish_features): every element of the force-feature block is then read and
+                # written once instead of once per element and atom chunk
+                self._pending_derivative_features.append((cos_derivs, self.Dmat[element_idx], grad, indexes))
+                return
             # `indexes` comes from a molecule-major gather, so the atomic-free kernel applies
             ops.derivative_features(cos_derivs, coeff_normalisation, self.Dmat[element_idx], grad, indexes,
                                     derivative_features, molecule_major=True)
+
+    @torch.jit.unused
+    def writes_force_rows(self):
+        return 64 <= self.npcas <= 256 and len(self.elements) <= 8
+
+    @torch.jit.unused
+    def finish_features(self, derivative_features=None, overwrite=False):
+        """Force-feature rows of the elements queued by calculate_features, in one launch."""
+        pending, self._pending_derivative_features = self._pending_derivative_features, []
+        if derivative_features is not None and (pending or overwrite):
+            ops.derivative_features_typed(pending, float(np.sqrt(self.npcas) / self.sigma), derivative_features,
+                                          overwrite=overwrite)
 
     def forward(self, X, Z, atomIDs, molIDs, atom_counts, cell: Optional[torch.Tensor] = None,
                 inv_cell: Optional[torch.Tensor] = None):

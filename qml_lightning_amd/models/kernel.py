@@ -39,8 +39,19 @@ class BaseKernel():
         self._subtract_self_energies = False
         self.sigma = sigma
         self.llambda = llambda
+        self._queue_force_rows = False
 
     # -- to be provided by the feature model -------------------------------------------
+    def finish_features(self, derivative_matrix=None, overwrite=False):
+        """Called once per batch after the loop over elements; models that queue work in
+        calculate_features run it here."""
+        return None
+
+    def writes_force_rows(self):
+        """True when finish_features writes every element of the force-feature block itself
+        (overwrite=True), so that the block need not be cleared first."""
+        return False
+
     def calculate_features(self, rep, element, indexes, feature_matrix, grad=None, derivative_matrix=None):
         raise NotImplementedError("Abstract method only.")
 
@@ -67,11 +78,17 @@ class BaseKernel():
                                                          inv_cells)
             rep_derivative = None
         nrows = B + (B * n * 3 if with_forces else 0)
-        rows = torch.zeros(nrows, F, device=coordinates.device, dtype=torch.float64)
+        own_force_rows = with_forces and self.writes_force_rows()
+        if own_force_rows:
+            rows = torch.empty(nrows, F, device=coordinates.device, dtype=torch.float64)
+            rows[:B].zero_()
+        else:
+            rows = torch.zeros(nrows, F, device=coordinates.device, dtype=torch.float64)
         Zenergy = rows[:B]
         G = rows[B:].view(B, n, 3, F) if with_forces else None
         flat_rep = representation.view(B * n, -1)
         flat_jac = rep_derivative.view(B * n, n, 3, -1) if with_forces else None
+        self._queue_force_rows = own_force_rows     # calculate_features may queue; finish_features runs the queue
         for e in self.elements:
             idx = self._element_index(data, charges, int(e))
             if idx.shape[0] == 0:
@@ -83,6 +100,8 @@ class BaseKernel():
             if with_forces:
                 sub_grad = project_derivative(flat_jac.index_select(0, idx), self.reductors[element_idx])
             self.calculate_features(sub, e, batch_indexes, Zenergy, sub_grad, G)
+        self._queue_force_rows = False
+        self.finish_features(G, overwrite=own_force_rows)
         if zero_energy_rows:
             Zenergy.fill_(0)        # energy rows stay, as zeros, so the row count is unchanged (kernel.py:164-165)
         return rows

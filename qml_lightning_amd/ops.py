@@ -298,6 +298,42 @@ def derivative_features(cos_derivs, normalisation, D, input_derivatives, mol_ind
     return G
 
 
+def derivative_features_typed(items, normalisation, G, overwrite=False):
+    """G += force-feature rows of every element of the batch in one launch.  items: one tuple
+    (cos_derivs f64 [A_e,F], D f32 [T,S,d], input_derivatives f32 [A_e,n,3,d], mol_index i32 [A_e],
+    non-decreasing) per element.  Each G element is read and written once, instead of once per
+    element and atom chunk as with `derivative_features`; with overwrite, G = those rows and is
+    only written (it may come from torch.empty).  64 <= d <= 256, at most 8 elements."""
+    if not items:
+        return G.zero_() if overwrite else G
+    if G.dtype != torch.float64 or not G.is_contiguous():
+        raise RuntimeError("derivative features need a contiguous float64 output")
+    nmol, n = int(G.shape[0]), int(G.shape[1])
+    keep, structs = [], (_lib.DfElement * len(items))()
+    T = S = d = None
+    bounds = torch.arange(nmol + 1, dtype=torch.int32, device=G.device)
+    for k, (cos_derivs, D, u, mol_index) in enumerate(items):
+        D, u, mol_index = _f32(D), _f32(u), _i32(mol_index)
+        if cos_derivs.dtype != torch.float64 or not cos_derivs.is_contiguous():
+            raise RuntimeError("derivative features need contiguous float64 cos_derivs")
+        if T is None:
+            T, S, d = (int(v) for v in D.shape)
+        if tuple(D.shape) != (T, S, d) or tuple(u.shape[1:]) != (n, 3, d) or cos_derivs.shape != (u.shape[0], S * d):
+            raise RuntimeError("derivative_features_typed: element %d does not fit [T,S,d] = %s, n = %d" % (k, (T, S, d), n))
+        seg = torch.searchsorted(mol_index, bounds).to(torch.int32)
+        keep.append((cos_derivs, D, u, seg))
+        structs[k].cos_derivs = cos_derivs.data_ptr()
+        structs[k].input_derivative = u.data_ptr()
+        structs[k].D = D.data_ptr()
+        structs[k].seg_offsets = seg.data_ptr()
+    if G.shape[3] != S * d:
+        raise RuntimeError("feature_derivatives has shape %s, expected [nmol,%d,3,%d]" % (tuple(G.shape), n, S * d))
+    check(_lib.lib().qmll_derivative_features_typed(structs, len(items), float(normalisation), n, d, S, T, nmol,
+                                                    int(bool(overwrite)), _ptr(G), _stream()),
+          "qmll_derivative_features_typed")
+    return G
+
+
 def sorf_energy_fused(x, D, bias, alpha, out_index, normalisation, ntransforms, e_atom, with_grad=True):
     """Per-atom energies written into e_atom[out_index]; returns d e_atom / d x or None."""
     x, D, bias, alpha = _f32(x), _f32(D), _f32(bias), _f32(alpha)

@@ -294,6 +294,39 @@ def test_derivative_features(d, S, T):
         close(G - 1.0, ref, REL_REP, "derivative features, molecule_major=%s" % molecule_major)
 
 
+@pytest.mark.parametrize("d,S,T,ne", [(64, 5, 2, 3), (128, 17, 1, 3), (128, 8, 1, 1), (256, 6, 1, 5), (128, 4, 3, 8)])
+def test_derivative_features_all_elements_in_one_launch(d, S, T, ne):
+    """The typed entry (every element of the batch in one launch) against the oracle summed over the
+    elements, with molecules that lack an element, more atoms in a molecule than one pass holds,
+    rows that are not neighbours, and G either holding earlier contributions (add) or garbage
+    (overwrite)."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(d + S + ne)
+    n, nmol = 7, 6
+    norm = 1.75
+    ref = np.zeros((nmol, n, 3, S * d))
+    items = []
+    for e in range(ne):
+        A = int(rng.integers(1, 30)) if e else 23          # the first element: up to 23 atoms in few molecules
+        idx = np.sort(rng.integers(0, nmol if e else 2, A)).astype(np.int32)
+        u = rng.normal(size=(A, n, 3, d)).astype(np.float32)
+        u[rng.integers(0, A), rng.integers(0, n)] = 0.0
+        D = np.where(rng.uniform(-1, 1, (T, S, d)) > 0, 1.0, -1.0).astype(np.float32)
+        cd = rng.normal(size=(A, S * d))
+        ref += sorf.derivative_features(cd, norm, idx, u, D, nmol)
+        items.append((torch.tensor(cd, device=dev()), t32(D), t32(u), ti32(idx)))
+    G = torch.full((nmol, n, 3, S * d), 0.5, dtype=torch.float64, device=dev())
+    ops.derivative_features_typed(items, norm, G)
+    close(G - 0.5, ref, REL_REP, "typed derivative features")
+    G = torch.full((nmol, n, 3, S * d), float("nan"), dtype=torch.float64, device=dev())
+    ops.derivative_features_typed(items, norm, G, overwrite=True)
+    close(G, ref, REL_REP, "typed derivative features, overwrite")
+    ops.derivative_features_typed([], norm, G, overwrite=True)
+    assert float(G.abs().max()) == 0.0
+    with pytest.raises(RuntimeError):
+        ops.derivative_features_typed(items * 9, norm, G)          # more than 8 elements
+
+
 @pytest.mark.parametrize("d,S,T", [(8, 3, 1), (64, 5, 2), (128, 16, 1), (128, 9, 2), (128, 5, 3), (256, 8, 1), (256, 6, 2),
                                    (512, 4, 1), (512, 3, 2)])
 def test_fused_energy_matches_two_op_chain(d, S, T):
