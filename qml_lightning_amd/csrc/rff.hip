@@ -370,8 +370,7 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
             }
         }
     } else {
-        // two feature halves add into zero-filled outputs: a sum of two terms does not depend
-        // on their order, so the result stays reproducible
+        // the feature parts add into zero-filled outputs
         if (h == 0 && aok) atomicAdd(&e_slots[sorted_slots[row0 + arow]], energy);
         if constexpr (WITH_GRAD) {
             if (aok) {
@@ -467,12 +466,18 @@ extern "C" int qmll_rff_energy_sorted(const float* x, const int* type_offsets, c
                  "qmll_rff_energy_sorted: x, W and gx must be 16-byte aligned");
     const float norm = sqrtf(2.0f / (float)F);
     hipStream_t st = (hipStream_t)stream;
-    // Two workgroups fit a CU (two wavefronts per SIMD): when the tiles fill the last round of
-    // those slots badly, the features are split in two halves over twice the workgroups, which
-    // add their energies and gradients into zero-filled outputs.
+    // Two workgroups fit a CU (two wavefronts per SIMD), and a workgroup's time is set by the
+    // matrix pipe, so the launch takes ceil(workgroups / 512) rounds of 1/fs of a tile's work
+    // when the features are split over fs workgroups per tile.  fs is the power of two up to
+    // 64 with the shortest estimate (a larger one has to win by 5 %): 672 tiles take 2 rounds
+    // with fs = 1 and 21/16 with fs = 16; one molecule takes 1/64 instead of 1.  For fs > 1
+    // the parts add their energies and gradients into zero-filled outputs with fp32 atomics
+    // (from fs = 4 on the order of the terms, hence the last bit, varies from run to run).
     const int tiles = (A + RE_M - 1) / RE_M, slots = 2 * 256;
-    auto fill = [&](int k) { return (double)tiles * k / (double)(((long long)tiles * k + slots - 1) / slots * slots); };
-    const int fs = (F % (2 * RE_FC) == 0 && fill(2) > fill(1) + 0.05) ? 2 : 1;
+    auto rounds = [&](int k) { return (double)(((long long)(tiles + ne) * k + slots - 1) / slots) / k; };
+    int fs = 1;
+    for (int k = 2; k <= 64 && F % (k * RE_FC) == 0; k *= 2)
+        if (rounds(k) < 0.95 * rounds(fs)) fs = k;
     const dim3 grid(tiles + ne, fs);
     if (fs > 1 && gx) {
         hipLaunchKernelGGL(zero_fill_kernel, dim3(1024), dim3(256), 0, st, gx, (size_t)A * d);
