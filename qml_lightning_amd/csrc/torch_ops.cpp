@@ -540,10 +540,12 @@ std::tuple<Tensor, Tensor> rff_energy_sorted(const Tensor& x, const Tensor& off,
 // rff = true: `Dmat` holds W [ne,d,F], `bias` holds b [ne,F]; cn and nt are unused
 Tensor fchl_sorf_energy_impl(FCHL_TENSORS, MODEL_TENSORS, bool with_grad, Tensor* gX_out, bool rff = false) {
     FchlInputs in = prepare(FCHL_PASS);
-    Tensor rep = at::zeros({in.B, in.n, in.R}, in.X.options());
+    // the forward kernel writes every bin of a listed atom's row, and only the rows of listed
+    // atoms are read below, so the padded rows need no clearing here
+    Tensor rep = at::empty({in.B, in.n, in.R}, in.X.options());
     check(qmll_fchl19_forward(FCHL_ABI(in), rep.data_ptr<float>(), stream()), "qmll_fchl19_forward");
     const int64_t nslots = (int64_t)in.B * in.n;
-    Tensor slots = in.molIDs * in.n + in.atomIDs;
+    Tensor slots = at::add(in.atomIDs, in.molIDs, in.n);      // molIDs * n + atomIDs in one launch
     auto sorted = sort_by_type(in.types, slots, reductors.size(0));
     const Tensor& ss = std::get<0>(sorted);
     const Tensor& off = std::get<1>(sorted);

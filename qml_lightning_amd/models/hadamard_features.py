@@ -16,7 +16,7 @@ import torch
 from .. import ops
 from ..cuda.sorf_gpu import compute_hadamard_features, compute_partial_feature_derivatives
 from ..representations.dimensionality_reduction import project_representation
-from .kernel import BaseKernel, _default_device
+from .kernel import BaseKernel, _default_device, alpha_f32
 
 _fused_registered = False
 
@@ -397,13 +397,16 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         if cells is None or inv_cells is None:
             cells = torch.empty(0, 3, 3, device=coordinates.device)
             inv_cells = cells
-        coeff_normalisation = torch.sqrt(torch.tensor(self.npcas)) / self.sigma
+        if isinstance(self.sigma, float):       # sqrt(npcas) / sigma in fp32, as the tensor expression gives it
+            coeff_normalisation = torch.tensor(float(np.sqrt(np.float32(self.npcas)) / np.float32(self.sigma)))
+        else:
+            coeff_normalisation = torch.sqrt(torch.tensor(self.npcas)) / self.sigma
         rep = self.rep
         with torch.no_grad():
             energies, gX = torch.ops.qml_lightning_sorf.fchl_sorf_energy(
                 coordinates, charges, rep.species, atomIDs, molIDs, natom_counts, cells, inv_cells, rep.Rs2, rep.Rs3,
                 rep.eta2, rep.eta3, rep.two_body_decay, rep.three_body_weight, rep.three_body_decay, rep.rcut,
-                self.reductors, self.Dmat, self.bias, self.alpha.float(), coeff_normalisation, self.ntransforms, forces)
+                self.reductors, self.Dmat, self.bias, alpha_f32(self), coeff_normalisation, self.ntransforms, forces)
         return energies, (gX.neg_() if forces else None)
 
     @torch.jit.unused

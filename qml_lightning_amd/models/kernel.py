@@ -9,6 +9,8 @@ views of it, no concatenation copy), per-element atom indices built once on the 
 `format_data` (no boolean-mask device syncs), the hand-written fp64 MFMA Gram kernel, and
 no `empty_cache()` between batches.
 """
+import weakref
+
 import numpy as np
 import torch
 
@@ -19,6 +21,22 @@ from ..representations.dimensionality_reduction import project_derivative, proje
 
 def _default_device():
     return torch.device("cuda" if torch.cuda.is_available() else "cpu")
+
+
+_ALPHA32 = weakref.WeakKeyDictionary()    # model -> (alpha it was made from, its version, fp32 copy)
+
+
+def alpha_f32(model):
+    """model.alpha as fp32 (what the predict routes contract with), converted once per value of
+    alpha instead of once per call: one launch less per step, which counts for single molecules."""
+    a = model.alpha
+    if a.dtype == torch.float32:
+        return a
+    hit = _ALPHA32.get(model)
+    if hit is None or hit[0] is not a or hit[1] != a._version:
+        hit = (a, a._version, a.float())
+        _ALPHA32[model] = hit
+    return hit[2]
 
 
 class BaseKernel():

@@ -9,7 +9,7 @@ from .. import ops
 from ..cuda.rff_gpu import get_rff
 from ..representations.dimensionality_reduction import project_representation
 from . import hadamard_features  # noqa: F401  (registers the fused operators)
-from .kernel import BaseKernel, _default_device
+from .kernel import BaseKernel, _default_device, alpha_f32
 
 
 class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
@@ -122,7 +122,7 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
             energies, gX = torch.ops.qml_lightning_sorf.fchl_rff_energy(
                 coordinates, charges, rep.species, atomIDs, molIDs, natom_counts, cells, inv_cells, rep.Rs2, rep.Rs3,
                 rep.eta2, rep.eta3, rep.two_body_decay, rep.three_body_weight, rep.three_body_decay, rep.rcut,
-                self.reductors, self.W, self.b, self.alpha.float(), forces)
+                self.reductors, self.W, self.b, alpha_f32(self), forces)
         return energies, (gX.neg_() if forces else None)
 
     @torch.jit.unused
