@@ -102,7 +102,7 @@ __global__ __launch_bounds__(ST) void type_place_kernel(const int* __restrict__ 
 // ---- typed GEMM -------------------------------------------------------------------------
 constexpr int PT = 256;            // threads (4 wavefronts, each 32 rows x 64 columns)
 constexpr int PM = 128;            // rows per workgroup
-constexpr int PN = 64;             // columns per workgroup
+constexpr int PN = 64;             // columns per workgroup (PNT = 128 where the caller picks the wide tile)
 constexpr int PK = 32;             // contraction chunk staged in LDS
 constexpr int PKS = PK + 4;        // LDS row stride of k-contiguous tiles: 16-byte reads of 16
                                    // consecutive rows fall into 16 distinct groups of 4 banks
@@ -126,19 +126,22 @@ __device__ __forceinline__ bool tile_of_block(const int* __restrict__ offsets, i
 
 // BT = false: B_type is [K,N] row-major (ldb = row length); BT = true: B_type is [N,K].
 // VEC: all leading dimensions, K and N are multiples of 4 and the bases are 16-byte aligned.
-template <bool BT, bool VEC>
+// PNT: columns per workgroup, 64 or 128.  The wide tile reads the A rows once instead of twice
+// and halves the number of workgroups, each twice as long.
+template <bool BT, bool VEC, int PNT>
 // the forward kernel gains 15 % from a fifth wavefront per SIMD (at most 96 registers); the
-// transpose does not fit more than four
-__global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(BT ? 4 : 5))) void typed_gemm_kernel(const float* __restrict__ A, int lda,
+// transpose does not fit more than four, the wide tile three
+__global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(PNT > 64 ? 3 : (BT ? 4 : 5)))) void typed_gemm_kernel(const float* __restrict__ A, int lda,
                                                          const int* __restrict__ a_rows, const float* __restrict__ Bm,
                                                          size_t b_type_stride, int ldb, float* __restrict__ C, int ldc,
                                                          const int* __restrict__ c_rows,
                                                          const int* __restrict__ offsets, int ne, int K, int N) {
     __shared__ __attribute__((aligned(16))) float sA[PM * PKS];
-    __shared__ __attribute__((aligned(16))) float sB[BT ? PN * PKS : PK * PN];   // BT: [PN][PKS]; else [PK][PN], rotated rows
+    constexpr int NJ = PNT / 32;       // 32-column MFMA blocks per wavefront
+    __shared__ __attribute__((aligned(16))) float sB[BT ? PNT * PKS : PK * PNT];   // BT: [PNT][PKS]; else [PK][PNT], rotated rows
     int type, row0, rows;
     if (!tile_of_block(offsets, ne, blockIdx.x, type, row0, rows)) return;
-    const int col0 = blockIdx.y * PN;
+    const int col0 = blockIdx.y * PNT;
     const float* Bt = Bm + (size_t)type * b_type_stride;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -155,12 +158,14 @@ __global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(BT ? 4 : 5))
         const int src = arow_ok[v] ? (a_rows ? a_rows[row0 + r] : row0 + r) : 0;
         arow[v] = A + (size_t)src * lda;
     }
-    // B tile: !BT 32 k x 64 n = 512 float4 -> k = tid/16 + 16v, n4 = tid%16
-    //          BT 64 n x 32 k = 512 float4 -> n = tid/8 + 32v,  k4 = tid%8
-    const int bk = BT ? (tid & 7) * 4 : (tid >> 4);
-    const int bn = BT ? (tid >> 3) : (tid & 15) * 4;
+    // B tile: !BT 32 k x PNT n = 8 PNT float4 -> k = tid/(PNT/4) + (1024/PNT) v, n4 = tid%(PNT/4)
+    //          BT PNT n x 32 k = 8 PNT float4 -> n = tid/8 + 32v,  k4 = tid%8
+    constexpr int NQ = PNT / 4;        // float4 per B row (!BT)
+    constexpr int KV = PT / NQ;        // B rows staged per pass (!BT): 16 or 8
+    const int bk = BT ? (tid & 7) * 4 : (tid / NQ);
+    const int bn = BT ? (tid >> 3) : (tid % NQ) * 4;
 
-    float4 ra[4], rb[2];
+    float4 ra[4], rb[NJ];
     auto load4 = [&](const float* p, int first, int limit) -> float4 {
         // elements first..first+3 of a row, zero beyond `limit`
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -179,12 +184,12 @@ __global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(BT ? 4 : 5))
         for (int v = 0; v < 4; ++v)
             ra[v] = arow_ok[v] ? load4(arow[v], k0 + ak, K) : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-        for (int v = 0; v < 2; ++v) {
+        for (int v = 0; v < NJ; ++v) {
             if (BT) {
                 const int n = col0 + bn + 32 * v;
                 rb[v] = n < N ? load4(Bt + (size_t)n * ldb, k0 + bk, K) : make_float4(0.f, 0.f, 0.f, 0.f);
             } else {
-                const int k = k0 + bk + 16 * v;
+                const int k = k0 + bk + KV * v;
                 rb[v] = k < K ? load4(Bt + (size_t)k * ldb, col0 + bn, N) : make_float4(0.f, 0.f, 0.f, 0.f);
             }
         }
@@ -193,21 +198,21 @@ __global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(BT ? 4 : 5))
 #pragma unroll
         for (int v = 0; v < 4; ++v) *reinterpret_cast<float4*>(&sA[(ar + 32 * v) * PKS + ak]) = ra[v];
 #pragma unroll
-        for (int v = 0; v < 2; ++v) {
+        for (int v = 0; v < NJ; ++v) {
             if (BT) {
                 *reinterpret_cast<float4*>(&sB[(bn + 32 * v) * PKS + bk]) = rb[v];
             } else {
                 // rows 16..31 are rotated by 32 columns: the two wavefront halves, which read
                 // rows k and k+16 in one instruction, then use disjoint banks
-                const int k = bk + 16 * v;
-                *reinterpret_cast<float4*>(&sB[k * PN + ((bn + 32 * v) & 63)]) = rb[v];
+                const int k = bk + KV * v;
+                *reinterpret_cast<float4*>(&sB[k * PNT + ((bn + (k >= 16 ? 32 : 0)) & (PNT - 1))]) = rb[v];
             }
         }
     };
 
-    float16_t acc[2];
+    float16_t acc[NJ];
 #pragma unroll
-    for (int jt = 0; jt < 2; ++jt)
+    for (int jt = 0; jt < NJ; ++jt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[jt][r] = 0.0f;
 
@@ -226,22 +231,22 @@ __global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(BT ? 4 : 5))
         for (int q = 0; q < 4; ++q) {
             const float4 va = *reinterpret_cast<const float4*>(&sA[(32 * wave + i) * PKS + 16 * h + 4 * q]);
             const float af[4] = {va.x, va.y, va.z, va.w};
-            float bf[2][4];
+            float bf[NJ][4];
 #pragma unroll
-            for (int jt = 0; jt < 2; ++jt) {
+            for (int jt = 0; jt < NJ; ++jt) {
                 if (BT) {
                     const float4 v = *reinterpret_cast<const float4*>(&sB[(i + 32 * jt) * PKS + 16 * h + 4 * q]);
                     bf[jt][0] = v.x; bf[jt][1] = v.y; bf[jt][2] = v.z; bf[jt][3] = v.w;
                 } else {
 #pragma unroll
                     for (int s = 0; s < 4; ++s)
-                        bf[jt][s] = sB[(4 * q + s + 16 * h) * PN + ((i + 32 * jt + 32 * h) & 63)];
+                        bf[jt][s] = sB[(4 * q + s + 16 * h) * PNT + ((i + 32 * jt + 32 * h) & (PNT - 1))];
                 }
             }
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
 #pragma unroll
-                for (int jt = 0; jt < 2; ++jt)
+                for (int jt = 0; jt < NJ; ++jt)
                     acc[jt] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s], bf[jt][s], acc[jt], 0, 0, 0);
             }
         }
@@ -250,7 +255,7 @@ __global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(BT ? 4 : 5))
     // accumulator register r of v_mfma_f32_32x32x2f32 holds row 8(r/4) + 4(lane/32) + r%4,
     // column lane%32 (probed on gfx950)
 #pragma unroll
-    for (int jt = 0; jt < 2; ++jt) {
+    for (int jt = 0; jt < NJ; ++jt) {
         const int col = col0 + 32 * jt + i;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -325,13 +330,19 @@ extern "C" int qmll_project_typed(const float* rep, const int* sorted_slots, con
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(rep && sorted_slots && type_offsets && reductors && x, QMLL_ERR_INVALID,
                  "qmll_project_typed: null pointer");
-    const dim3 grid((A + PM - 1) / PM + ne, (d + PN - 1) / PN);
     const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(rep) && aligned16(reductors);
-    if (vec)
-        hipLaunchKernelGGL((typed_gemm_kernel<false, true>), grid, dim3(PT), 0, (hipStream_t)stream, rep, R, sorted_slots,
+    const int tiles = (A + PM - 1) / PM + ne;
+    // the wide tile when it wastes no columns and still leaves every CU a few workgroups
+    const bool wide = vec && d % 128 == 0 && (long long)tiles * (d / 128) >= 2 * 256;
+    const dim3 grid(tiles, wide ? d / 128 : (d + PN - 1) / PN);
+    if (wide)
+        hipLaunchKernelGGL((typed_gemm_kernel<false, true, 128>), grid, dim3(PT), 0, (hipStream_t)stream, rep, R,
+                           sorted_slots, reductors, (size_t)R * d, d, x, d, (const int*)nullptr, type_offsets, ne, R, d);
+    else if (vec)
+        hipLaunchKernelGGL((typed_gemm_kernel<false, true, PN>), grid, dim3(PT), 0, (hipStream_t)stream, rep, R, sorted_slots,
                            reductors, (size_t)R * d, d, x, d, (const int*)nullptr, type_offsets, ne, R, d);
     else
-        hipLaunchKernelGGL((typed_gemm_kernel<false, false>), grid, dim3(PT), 0, (hipStream_t)stream, rep, R,
+        hipLaunchKernelGGL((typed_gemm_kernel<false, false, PN>), grid, dim3(PT), 0, (hipStream_t)stream, rep, R,
                            sorted_slots, reductors, (size_t)R * d, d, x, d, (const int*)nullptr, type_offsets, ne, R, d);
     QMLL_CHECK_LAUNCH("qmll_project_typed");
     return QMLL_OK;
@@ -354,10 +365,10 @@ extern "C" int qmll_project_typed_backward(const float* gx, const int* sorted_sl
     const dim3 grid((A + PM - 1) / PM + ne, (R + PN - 1) / PN);
     const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(gx) && aligned16(reductors);
     if (vec)
-        hipLaunchKernelGGL((typed_gemm_kernel<true, true>), grid, dim3(PT), 0, (hipStream_t)stream, gx, d,
+        hipLaunchKernelGGL((typed_gemm_kernel<true, true, PN>), grid, dim3(PT), 0, (hipStream_t)stream, gx, d,
                            (const int*)nullptr, reductors, (size_t)R * d, d, g_rep, R, sorted_slots, type_offsets, ne, d, R);
     else
-        hipLaunchKernelGGL((typed_gemm_kernel<true, false>), grid, dim3(PT), 0, (hipStream_t)stream, gx, d,
+        hipLaunchKernelGGL((typed_gemm_kernel<true, false, PN>), grid, dim3(PT), 0, (hipStream_t)stream, gx, d,
                            (const int*)nullptr, reductors, (size_t)R * d, d, g_rep, R, sorted_slots, type_offsets, ne, d, R);
     QMLL_CHECK_LAUNCH("qmll_project_typed_backward");
     return QMLL_OK;
