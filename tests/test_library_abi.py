@@ -56,6 +56,19 @@ def test_bad_arguments_are_refused_on_the_host():
     prm = _lib.FchlParams(0, 24, 20, 0.32, 2.7, 1.8, 13.4, 0.57, 6.0)
     args = [null] * 9 + [0, 5, 1, 12, null, null, ctypes.byref(prm), null, null]
     assert L.qmll_fchl19_forward(*args) == _lib.QMLL_ERR_INVALID
+    # the all-elements force-feature entry: element count, projected dimension, null output
+    elems = (_lib.DfElement * 9)()
+    assert L.qmll_derivative_features_typed(elems, 9, 1.0, 3, 128, 4, 1, 2, 0, ctypes.c_void_p(8), null) == _lib.QMLL_ERR_INVALID
+    assert b"at most 8" in L.qmll_last_error()
+    assert L.qmll_derivative_features_typed(elems, 2, 1.0, 3, 512, 4, 1, 2, 0, ctypes.c_void_p(8), null) == _lib.QMLL_ERR_INVALID
+    assert L.qmll_derivative_features_typed(elems, 2, 1.0, 3, 96, 4, 1, 2, 0, ctypes.c_void_p(8), null) == _lib.QMLL_ERR_NOT_POW2
+    assert L.qmll_derivative_features_typed(elems, 2, 1.0, 3, 128, 4, 1, 2, 0, null, null) == _lib.QMLL_ERR_INVALID
+    assert L.qmll_derivative_features_typed(elems, 2, 1.0, 3, 128, 4, 1, 2, 0, ctypes.c_void_p(8), null) == _lib.QMLL_ERR_INVALID  # null element pointers
+    assert L.qmll_derivative_features_typed(elems, 2, 1.0, 3, 128, 4, 1, 0, 0, null, null) == _lib.QMLL_OK   # no molecules
+    # the Cholesky entries
+    assert L.qmll_cholesky_workspace_bytes(0) == 0 and L.qmll_cholesky_workspace_bytes(300) > 300 * 8
+    assert L.qmll_cholesky_f64(null, 16, 16, null, null, null) == _lib.QMLL_ERR_INVALID
+    assert L.qmll_cholesky_f64(ctypes.c_void_p(16), 16, 8, ctypes.c_void_p(16), ctypes.c_void_p(16), null) == _lib.QMLL_ERR_INVALID
     # empty inputs are fine and launch nothing
     assert L.qmll_sorf_forward(null, null, 0, 16, 2, 1, 1.0, null, null) == _lib.QMLL_OK
     assert L.qmll_gram_f64(null, null, 0, 16, null, null, null) == _lib.QMLL_OK
