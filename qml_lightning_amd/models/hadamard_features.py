@@ -453,8 +453,9 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         start.record()
         predict_energies = torch.zeros(len(X), device=self.device, dtype=torch.float32)
         predict_forces = torch.zeros(len(X), max_natoms, 3, device=self.device, dtype=torch.float32)
-        for i in self._progress(range(0, len(X), self.nbatch_test), print_info):
-            sl = slice(i, i + self.nbatch_test)
+        step = self._fused_batch(max_natoms) if self.fused else self.nbatch_test
+        for i in self._progress(range(0, len(X), step), print_info):
+            sl = slice(i, i + step)
             data = self.format_data(X[sl], Z[sl], cells=cells[sl] if cells is not None else None,
                                     inv_cells=inv_cells[sl] if cells is not None else None)
             if self.fused:

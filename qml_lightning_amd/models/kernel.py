@@ -304,6 +304,16 @@ class BaseKernel():
             print("Best error: ", best[2], "sigma = ", best[0], "lambda = ", best[1])
         return best[0], best[1]
 
+    #: atoms the fused predict route aims to put into one launch chain (see _fused_batch)
+    fused_batch_atoms = 131072
+
+    def _fused_batch(self, max_natoms):
+        """Molecules per batch of the list-route `predict` on the fused route: nbatch_test, raised
+        to about `fused_batch_atoms` atoms.  nbatch_test bounds the reference's per-batch
+        [atoms, features] arrays (64 by default, hadamard_features.py:17); the fused chain keeps
+        none of them (some 6 KB per atom), and batches of 64 molecules leave the chip mostly idle."""
+        return max(int(self.nbatch_test), self.fused_batch_atoms // max(int(max_natoms), 1))
+
     # -- explicit-Jacobian predict route ----------------------------------------------------
     def predict_cuda(self, X, Q, max_natoms, cells=None, inv_cells=None, forces=False, print_info=True):
         """fp64 energies [N] (and forces [N,max_natoms,3]) as Z.alpha and G.alpha

@@ -207,9 +207,15 @@ def test_predict_from_lists_and_predict_cuda():
     X, Z, aid, mid, nat = make_batch(coords, charges)
     E, F, _ = omodel.sorf_energy_forces(X, Z, aid, mid, nat, prm, species, red, D, bias, alpha, 2.0)
     nmax = int(nat.max())
-    e, f = m.predict(c32, charges, nmax, forces=True)
+    e, f = m.predict(c32, charges, nmax, forces=True)          # one batch: the fused route widens nbatch_test
     close(e, E, REL_EF, "predict energies")
     close(f, F, REL_EF, "predict forces")
+    assert m._fused_batch(nmax) == m.fused_batch_atoms // nmax
+    m.fused_batch_atoms = 0                                    # batches of nbatch_test = 5 molecules: 5 + 5 + 1
+    assert m._fused_batch(nmax) == 5
+    e, f = m.predict(c32, charges, nmax, forces=True)
+    close(e, E, REL_EF, "predict energies, three batches")
+    close(f, F, REL_EF, "predict forces, three batches")
     # the explicit-Jacobian route (fp64 rows times alpha) gives the same numbers
     e2, f2 = m.predict_cuda(c32, charges, nmax, forces=True, print_info=False)
     close(e2, E, REL_EF, "predict_cuda energies")
