@@ -22,6 +22,16 @@
 #include "qmll_common.h"
 
 namespace {
+// 1-ulp forms on the transcendental unit (operands here are distances and widths, far from the
+// denormal range): a correctly rounded division, square root or logarithm costs ten or more
+// instructions each, several times per neighbour and per triple
+__device__ __forceinline__ float frcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ float fsqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
+__device__ __forceinline__ float flog(float x) { return __builtin_amdgcn_logf(x) * 0.6931471805599453f; }
+// floor(x / d) for 0 <= x < 1e6, 0 < d: (x + 0.5) / d is at least 0.5 / d away from an integer,
+// far more than the rounding of the 1-ulp reciprocal, so the truncation is exact; five
+// instructions where the integer division expands to about twenty-five
+__device__ __forceinline__ int idiv_small(int x, int d) { return (int)(((float)x + 0.5f) * frcp((float)d)); }
 
 struct FchlArgs {
     const float* X;
@@ -117,7 +127,7 @@ __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i,
     const float xo = Xm[own * 3 + 0], yo = Xm[own * 3 + 1], zo = Xm[own * 3 + 2];
     const int eo = tm[own];
     const float rc2 = a.p.rcut * a.p.rcut;
-    const float inv_rc = 1.0f / a.p.rcut;
+    const float inv_rc = frcp(a.p.rcut);
     const bool have_list = a.nlist != nullptr;
     int total;
     const int* li = nullptr;
@@ -163,7 +173,7 @@ __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i,
         const int nn = start < a.cap ? start : a.cap;
         if (lane == 0) s.goff[ns] = nn;
         if (ok && pos < a.cap) {
-            const float r = sqrtf(r2);
+            const float r = fsqrt(r2);
             s.dx[pos] = dx;
             s.dy[pos] = dy;
             s.dz[pos] = dz;
@@ -222,7 +232,7 @@ __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i,
                 if (pass == 1 && ok && e == ep) {
                     const int pos = s.goff[ep] + before + __popcll(mask & ((1ull << lane) - 1ull));
                     if (pos < a.cap) {
-                        const float r = sqrtf(r2);
+                        const float r = fsqrt(r2);
                         s.dx[pos] = dx;
                         s.dy[pos] = dy;
                         s.dz[pos] = dz;
@@ -284,8 +294,8 @@ __device__ __forceinline__ Triple triple_geometry(const Stage& s, int j, int k) 
     t.a = s.r[j];
     t.b = s.r[k];
     const float c2 = cx * cx + cy * cy + cz * cz;
-    t.c = sqrtf(c2);
-    const float ia = 1.0f / t.a, ib = 1.0f / t.b, ic = 1.0f / t.c;
+    t.c = fsqrt(c2);
+    const float ia = frcp(t.a), ib = frcp(t.b), ic = frcp(t.c);
     const float vi = ax * bx + ay * by + az * bz;           // (R_j-R_i).(R_k-R_i)
     t.ci = vi * ia * ib;
     t.ck = (cx * bx + cy * by + cz * bz) * ic * ib;         // (R_j-R_k).(R_i-R_k)
@@ -296,7 +306,7 @@ __device__ __forceinline__ Triple triple_geometry(const Stage& s, int j, int k) 
     // relative accuracy near collinear triples, where the difference of squares cancels
     const float px = ay * bz - az * by, py = az * bx - ax * bz, pz = ax * by - ay * bx;
     const float cross2 = px * px + py * py + pz * pz;
-    t.sinT = fminf(1.0f, sqrtf(cross2) * ia * ib);
+    t.sinT = fminf(1.0f, fsqrt(cross2) * ia * ib);
     t.guard_inv = t.a * t.b * rsqrtf(fmaxf(1e-10f, cross2));
     t.ujk[0] = cx * ic;
     t.ujk[1] = cy * ic;
@@ -345,13 +355,13 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     const int nn = stage_neighbours(a, s, m, i, lane);
     if (lane < nRs2) {
         slnRs2[lane] = logf(rs2v);
-        sinvRs2[lane] = 1.0f / rs2v;
+        sinvRs2[lane] = frcp(rs2v);
     }
     if (lane < nRs3) sRs3[lane] = rs3v;
     for (int t = lane + QMLL_WAVE; t < nRs2; t += QMLL_WAVE) {
         const float v = a.Rs2[t];
         slnRs2[t] = logf(v);
-        sinvRs2[t] = 1.0f / v;
+        sinvRs2[t] = frcp(v);
     }
     for (int t = lane + QMLL_WAVE; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
     __syncthreads();
@@ -359,9 +369,9 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     // per-neighbour two-body factors
     for (int j = lane; j < nn; j += QMLL_WAVE) {
         const float r = s.r[j];
-        const float s2 = logf(1.0f + a.p.eta2 / (r * r));
-        smu[j] = logf(r) - 0.5f * s2;                    // ln(r / sqrt(1 + eta2/r^2))
-        sis2[j] = 0.5f * LOG2E / s2;
+        const float s2 = flog(1.0f + a.p.eta2 * frcp(r * r));
+        smu[j] = flog(r) - 0.5f * s2;                    // ln(r / sqrt(1 + eta2/r^2))
+        sis2[j] = 0.5f * LOG2E * frcp(s2);
         spre[j] = rsqrtf(s2) * 0.3989422804014327f * fexp2(-a.p.two_body_decay * flog2(r)) * s.fc[j];
     }
     __syncthreads();
@@ -371,8 +381,8 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     // ---- two-body blocks ----
     {
         const int W = nRs2 < 64 ? nRs2 : 64;     // lanes per neighbour sub-slot
-        const int JS = 64 / W;                   // neighbour sub-slots
-        const int jsub = lane / W, zl = lane - jsub * W;
+        const int JS = idiv_small(64, W);        // neighbour sub-slots
+        const int jsub = idiv_small(lane, W), zl = lane - jsub * W;
         for (int zb = 0; zb < nRs2; zb += W) {
             const int z = zb + zl;
             const bool zok = z < nRs2 && jsub < JS;
@@ -396,10 +406,10 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     // ---- three-body blocks ----
     const float zeta2 = 0.014383766711652736f;   // 2 exp(-pi^2 / 2)
     const float k3 = a.p.eta3 * LOG2E;
-    const float sk3 = sqrtf(k3);                 // exp(-eta3 (rho - Rs)^2) = exp2(-(sk3 rho - sk3 Rs)^2)
+    const float sk3 = fsqrt(k3);                 // exp(-eta3 (rho - Rs)^2) = exp2(-(sk3 rho - sk3 Rs)^2)
     const int W3 = nRs3 < 64 ? nRs3 : 64;
-    const int TS = 64 / W3;
-    const int tsub = lane / W3, ll = lane - tsub * W3;
+    const int TS = idiv_small(64, W3);
+    const int tsub = idiv_small(lane, W3), ll = lane - tsub * W3;
     constexpr int MAXLB = 4;                     // radial bins handled: up to 4 x 64
 
     // one table entry per triple: (sk3 rho, K cos, K sin, -)
@@ -414,7 +424,7 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     // entries up to the next multiple of TS are zero entries, so every sub-slot runs the same
     // number of rounds and the loop is wavefront-uniform (scalar control, unrollable).
     auto accumulate = [&](int first, int count, float (&accc)[MAXLB], float (&accs)[MAXLB]) {
-        const int rounds = (count + TS - 1) / TS;
+        const int rounds = idiv_small(count + TS - 1, TS);
         const float4* src = reinterpret_cast<const float4*>(trip) + first + (tsub < TS ? tsub : 0);
 #pragma unroll
         for (int b = 0; b < MAXLB; ++b) {
@@ -467,7 +477,7 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
                 for (int q = p; q < ns; ++q) {
                     pbase[p * ns + q] = acc;
                     const int ntr = (p == q) ? np_ * (np_ - 1) / 2 : np_ * (s.goff[q + 1] - s.goff[q]);
-                    acc += (ntr + TS - 1) / TS * TS;       // segments start on a multiple of TS
+                    acc += idiv_small(ntr + TS - 1, TS) * TS;   // segments start on a multiple of TS
                 }
             }
         }
@@ -518,7 +528,7 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
                     }
                     *reinterpret_cast<float4*>(trip + tt * 4) = table_entry(op + ja, oq + kb);
                 }
-                if (lane < (nchunk + TS - 1) / TS * TS - nchunk)
+                if (lane < idiv_small(nchunk + TS - 1, TS) * TS - nchunk)
                     *reinterpret_cast<float4*>(trip + (nchunk + lane) * 4) = make_float4(0.f, 0.f, 0.f, 0.f);
                 __syncthreads();
                 accumulate(0, nchunk, accc, accs);
@@ -538,21 +548,21 @@ struct TwoBody {
 __device__ __forceinline__ TwoBody two_body_setup(float r, float fc, float dfc, const qmll_fchl_params& p) {
     TwoBody t;
     const float r2 = r * r;
-    t.s2 = logf(1.0f + p.eta2 / r2);
-    t.mu = logf(r) - 0.5f * t.s2;
-    t.s2p = -2.0f * p.eta2 / (r * (r2 + p.eta2));      // d sigma^2 / dr
-    t.mup = 1.0f / r - 0.5f * t.s2p;                   // d mu / dr
+    t.s2 = flog(1.0f + p.eta2 * frcp(r2));
+    t.mu = flog(r) - 0.5f * t.s2;
+    t.s2p = -2.0f * p.eta2 * frcp(r * (r2 + p.eta2));      // d sigma^2 / dr
+    t.mup = frcp(r) - 0.5f * t.s2p;                   // d mu / dr
     t.pre = rsqrtf(t.s2) * 0.3989422804014327f * fexp2(-p.two_body_decay * flog2(r));
     t.fc = fc;
     t.dfc = dfc;
-    t.d2_over_r = p.two_body_decay / r;
+    t.d2_over_r = p.two_body_decay * frcp(r);
     return t;
 }
 
 // value and r-derivative of bin z
 __device__ __forceinline__ void two_body_bin(const TwoBody& t, float lnRs, float invRs, float& val, float& dval) {
     const float u = lnRs - t.mu;
-    const float inv_s2 = 1.0f / t.s2;
+    const float inv_s2 = frcp(t.s2);
     const float Bz = t.pre * invRs * fexp2(-0.5f * LOG2E * u * u * inv_s2);
     const float Q = -0.5f * t.s2p * inv_s2 - t.d2_over_r + u * inv_s2 * (t.mup + 0.5f * u * t.s2p * inv_s2);
     val = Bz * t.fc;
@@ -569,7 +579,7 @@ struct TripleDeriv {
 __device__ __forceinline__ TripleDeriv triple_derivatives(const Triple& t, const qmll_fchl_params& p, float fa,
                                                           float dfa, float fb, float dfb) {
     TripleDeriv d;
-    const float ia = 1.0f / t.a, ib = 1.0f / t.b, ic = 1.0f / t.c;
+    const float ia = frcp(t.a), ib = frcp(t.b), ic = frcp(t.c);
     // d cos / d distance (law of cosines)
     d.cia = ib - t.ci * ia;
     d.cib = ia - t.ci * ib;
@@ -641,13 +651,13 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
     for (int t = lane + QMLL_WAVE * GREG; t < R; t += QMLL_WAVE) gin[t] = gsrc[t];
     if (lane < nRs2) {
         slnRs2[lane] = logf(rs2v);
-        sinvRs2[lane] = 1.0f / rs2v;
+        sinvRs2[lane] = frcp(rs2v);
     }
     if (lane < nRs3) sRs3[lane] = rs3v;
     for (int t = lane + QMLL_WAVE; t < nRs2; t += QMLL_WAVE) {
         const float v = a.Rs2[t];
         slnRs2[t] = logf(v);
-        sinvRs2[t] = 1.0f / v;
+        sinvRs2[t] = frcp(v);
     }
     for (int t = lane + QMLL_WAVE; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
     __syncthreads();
@@ -657,9 +667,9 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
 
     // two-body: lanes = (bin group g, neighbour j); group g takes the bins z = g, g+G, ...
     {
-        const int G = (nn > 0 && nn < 64) ? 64 / nn : 1;
+        const int G = (nn > 0 && nn < 64) ? idiv_small(64, nn) : 1;
         for (int base = 0; base < nn; base += QMLL_WAVE) {
-            const int g = G > 1 ? lane / nn : 0;
+            const int g = G > 1 ? idiv_small(lane, nn) : 0;
             const int j = G > 1 ? lane - g * nn : base + lane;
             const bool active = g < G && j < nn;
             float gr = 0.0f;
@@ -675,7 +685,7 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
             float tot = gr;
             for (int k = 1; k < G; ++k) tot += __shfl(gr, (lane + nn * k) & 63, 64);
             if (active && g == 0) {
-                const float ir = 1.0f / s.r[j];
+                const float ir = frcp(s.r[j]);
                 const float ux = s.dx[j] * ir, uy = s.dy[j] * ir, uz = s.dz[j] * ir;   // dr/dR_i
                 gix += tot * ux;
                 giy += tot * uy;
@@ -715,7 +725,7 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
         const float Ea = zeta2 * (d.Ka * S0 + d.K * (S1 + Sth * d.cia));
         const float Eb = zeta2 * (d.Kb * S0 + d.K * (S1 + Sth * d.cib));
         const float Ec = zeta2 * (d.Kc * S0 + d.K * (Sth * d.cic));
-        const float ia = 1.0f / t.a, ib = 1.0f / t.b;
+        const float ia = frcp(t.a), ib = frcp(t.b);
         const float uax = s.dx[j] * ia, uay = s.dy[j] * ia, uaz = s.dz[j] * ia;   // u_ij
         const float ubx = s.dx[k] * ib, uby = s.dy[k] * ib, ubz = s.dz[k] * ib;   // u_ik
         gix += Ea * uax + Eb * ubx;
@@ -805,7 +815,7 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
     for (int t = lane; t < nRs2; t += QMLL_WAVE) {
         const float v = a.Rs2[t];
         slnRs2[t] = logf(v);
-        sinvRs2[t] = 1.0f / v;
+        sinvRs2[t] = frcp(v);
     }
     for (int t = lane; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
     const int nn = stage_neighbours(a, s, m, i, lane);
@@ -826,7 +836,7 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
             const TripleDeriv d = triple_derivatives(t, a.p, s.fc[j], s.dfc[j], s.fc[k], s.dfc[k]);
             const float dcos = t.sinT * t.guard_inv;       // d cosT = dcos * d cos_i
             const float dsin = -t.cosT * t.guard_inv;      // d sinT = dsin * d cos_i
-            const float ia = 1.0f / t.a, ib = 1.0f / t.b;
+            const float ia = frcp(t.a), ib = frcp(t.b);
             float4* e4 = reinterpret_cast<float4*>(ttab + (size_t)tt * JT);
             e4[0] = make_float4(0.5f * (t.a + t.b),
                                 __int_as_float(pair_offset(s.el[j], s.el[k], ns, nRs2, nRs3)),
@@ -862,7 +872,7 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
                 const TwoBody tb = two_body_setup(r, s.fc[j], s.dfc[j], a.p);
                 float v, dv;
                 two_body_bin(tb, slnRs2[z], sinvRs2[z], v, dv);
-                const float ir = sign * dv / r;
+                const float ir = sign * dv * frcp(r);
                 const int bin = s.el[j] * nRs2 + z;
                 atomicAdd(&row[0 * R + bin], ir * s.dx[j]);
                 atomicAdd(&row[1 * R + bin], ir * s.dy[j]);
@@ -1018,7 +1028,7 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
                         atomicAdd(&val[off + 1], Ke * t.sinT);
                     }
                 }
-                const float ia = 1.0f / t.a, ib = 1.0f / t.b;
+                const float ia = frcp(t.a), ib = frcp(t.b);
                 const float ua[3] = {s.dx[j] * ia, s.dy[j] * ia, s.dz[j] * ia};
                 const float ub[3] = {s.dx[k] * ib, s.dy[k] * ib, s.dz[k] * ib};
                 const int off = pair_offset(s.el[j], s.el[k], ns, nRs2, nRs3) + 2 * l;
