@@ -261,7 +261,7 @@ constexpr float LOG2E = 1.4426950408889634f;
 // row index of pair t in the list of pairs (j<k) over nn items, rows enumerated j = 0..nn-2
 __device__ __forceinline__ void unrank_pair(int t, int nn, int& j, int& k) {
     const float b = (float)(2 * nn - 1);
-    int jj = (int)((b - sqrtf(fmaxf(b * b - 8.0f * (float)t, 0.0f))) * 0.5f);
+    int jj = (int)((b - fsqrt(fmaxf(b * b - 8.0f * (float)t, 0.0f))) * 0.5f);   // first guess; corrected below
     if (jj < 0) jj = 0;
     if (jj > nn - 2) jj = nn - 2;
     // offset(j) = j (2nn - j - 1) / 2
@@ -354,13 +354,13 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
 
     const int nn = stage_neighbours(a, s, m, i, lane);
     if (lane < nRs2) {
-        slnRs2[lane] = logf(rs2v);
+        slnRs2[lane] = flog(rs2v);
         sinvRs2[lane] = frcp(rs2v);
     }
     if (lane < nRs3) sRs3[lane] = rs3v;
     for (int t = lane + QMLL_WAVE; t < nRs2; t += QMLL_WAVE) {
         const float v = a.Rs2[t];
-        slnRs2[t] = logf(v);
+        slnRs2[t] = flog(v);
         sinvRs2[t] = frcp(v);
     }
     for (int t = lane + QMLL_WAVE; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
@@ -650,19 +650,22 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
         if (lane + QMLL_WAVE * k < R) gin[lane + QMLL_WAVE * k] = gr[k];
     for (int t = lane + QMLL_WAVE * GREG; t < R; t += QMLL_WAVE) gin[t] = gsrc[t];
     if (lane < nRs2) {
-        slnRs2[lane] = logf(rs2v);
+        slnRs2[lane] = flog(rs2v);
         sinvRs2[lane] = frcp(rs2v);
     }
-    if (lane < nRs3) sRs3[lane] = rs3v;
+    const float k3 = a.p.eta3 * LOG2E;
+    const float sk3 = fsqrt(k3);                       // the radial grid of the triples is kept as sk3 Rs3
+    const float hfac = -2.0f * a.p.eta3 * frcp(sk3);
+    if (lane < nRs3) sRs3[lane] = sk3 * rs3v;
     for (int t = lane + QMLL_WAVE; t < nRs2; t += QMLL_WAVE) {
         const float v = a.Rs2[t];
-        slnRs2[t] = logf(v);
+        slnRs2[t] = flog(v);
         sinvRs2[t] = frcp(v);
     }
-    for (int t = lane + QMLL_WAVE; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
+    for (int t = lane + QMLL_WAVE; t < nRs3; t += QMLL_WAVE) sRs3[t] = sk3 * a.Rs3[t];
     __syncthreads();
 
-    const float k3 = a.p.eta3 * LOG2E;
+
     float gix = 0.0f, giy = 0.0f, giz = 0.0f;
 
     // two-body: lanes = (bin group g, neighbour j); group g takes the bins z = g, g+G, ...
@@ -707,18 +710,23 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
         const Triple t = triple_geometry(s, j, k);
         const TripleDeriv d = triple_derivatives(t, a.p, s.fc[j], s.dfc[j], s.fc[k], s.dfc[k]);
         const float* g = gin + pair_offset(s.el[j], s.el[k], ns, nRs2, nRs3);
-        const float rho = 0.5f * (t.a + t.b);
+        // exp(-eta3 (rho - Rs)^2) = exp2(-(sk3 rho - sk3 Rs)^2) with the grid stored pre-scaled;
+        // d e / d rho = -2 eta3 (rho - Rs) e = hfac (sk3 rho - sk3 Rs) e, the factor applied after the sums
+        const float rho = sk3 * 0.5f * (t.a + t.b);
         float Gc = 0.f, Gs = 0.f, Hc = 0.f, Hs = 0.f;
+#pragma unroll 4
         for (int l = 0; l < nRs3; ++l) {
             const float dl = rho - sRs3[l];
-            const float e = fexp2(-k3 * dl * dl);
-            const float de = -2.0f * a.p.eta3 * dl * e;   // d e / d rho
+            const float e = fexp2(-(dl * dl));
+            const float de = dl * e;
             const float gc = g[2 * l], gs = g[2 * l + 1];
             Gc = fmaf(gc, e, Gc);
             Gs = fmaf(gs, e, Gs);
             Hc = fmaf(gc, de, Hc);
             Hs = fmaf(gs, de, Hs);
         }
+        Hc *= hfac;
+        Hs *= hfac;
         const float S0 = Gc * t.cosT + Gs * t.sinT;
         const float S1 = 0.5f * (Hc * t.cosT + Hs * t.sinT);                      // d rho/da = d rho/db = 1/2
         const float Sth = (Gc * t.sinT - Gs * t.cosT) * t.guard_inv;               // multiplies d cos_i
@@ -814,7 +822,7 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
 
     for (int t = lane; t < nRs2; t += QMLL_WAVE) {
         const float v = a.Rs2[t];
-        slnRs2[t] = logf(v);
+        slnRs2[t] = flog(v);
         sinvRs2[t] = frcp(v);
     }
     for (int t = lane; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
