@@ -874,8 +874,9 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
             const int j1 = target < 0 ? nn : target + 1;
             const float sign = target < 0 ? 1.0f : -1.0f;   // dr/dR_i = u_ij, dr/dR_j = -u_ij
             for (int it = lane; it < (j1 - j0) * nRs2; it += QMLL_WAVE) {
-                const int j = j0 + it / nRs2;
-                const int z = it % nRs2;
+                const int jq = idiv_small(it, nRs2);
+                const int j = j0 + jq;
+                const int z = it - jq * nRs2;
                 const float r = s.r[j];
                 const TwoBody tb = two_body_setup(r, s.fc[j], s.dfc[j], a.p);
                 float v, dv;
@@ -893,8 +894,8 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
         // at one lane per clock), sub-slots are folded with shuffles, sub-slot 0 stores the bin.
         if constexpr (TABLE) {
             const int W3 = nRs3 < 64 ? nRs3 : 64;
-            const int TS = 64 / W3;
-            const int tsub = lane / W3, ll = lane - tsub * W3;
+            const int TS = idiv_small(64, W3);
+            const int tsub = idiv_small(lane, W3), ll = lane - tsub * W3;
             // the triples of one block: index it -> neighbour positions j < k
             auto block = [&](int off_pair, int count, int p, int q) {
                 const int op = s.goff[p], oq = s.goff[q];
@@ -999,7 +1000,7 @@ __global__ __launch_bounds__(64) void fchl19_jacobian_kernel(FchlArgs a, float* 
             // self: all pairs (j<k); neighbour target: the nn-1 pairs {target, other}
             const int ntr = target < 0 ? nn * (nn - 1) / 2 : nn - 1;
             for (int it = lane; it < ntr * nRs3; it += QMLL_WAVE) {
-                const int tt = it / nRs3;
+                const int tt = idiv_small(it, nRs3);
                 const int l = it - tt * nRs3;
                 int j, k;
                 if (target < 0) {
