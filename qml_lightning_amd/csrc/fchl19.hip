@@ -772,9 +772,15 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
             const int x = it / 3, c = it - 3 * x;
             float sum = c == 0 ? sgx[x] : (c == 1 ? sgy[x] : sgz[x]);
             const float* tj = tab + c * ntrip + (x * (2 * nn - x - 1)) / 2;
+#pragma unroll 4
             for (int q = 0; q < nn - 1 - x; ++q) sum += tj[q];
             const float* tk = tab + (3 + c) * ntrip + x - 1;
-            for (int j = 0; j < x; ++j) sum += tk[(j * (2 * nn - j - 1)) / 2 - j];
+            int idx = 0;                                   // off(j) - j, which grows by nn - j - 2 per step
+#pragma unroll 4
+            for (int j = 0; j < x; ++j) {
+                sum += tk[idx];
+                idx += nn - j - 2;
+            }
             atomicAdd(&gm[s.j[x] * 3 + c], sum);
         }
     } else {
