@@ -104,3 +104,17 @@ def test_free_self_energy_fit_matches_the_model_method():
     for z, v in true.items():
         assert abs(float(se[z]) - v) <= 1e-9 * abs(v)
     assert float(se[[0, 2, 3, 4, 5, 7]].abs().max()) == 0.0
+
+
+def test_small_integer_division_through_a_float_reciprocal_is_exact():
+    """The FCHL19 kernels divide small non-negative integers as int((x + 0.5f) * rcp(d)) with the
+    1-ulp hardware reciprocal (csrc/fchl19.hip, idiv_small).  Emulated here in fp32 with the
+    reciprocal pushed one ulp either way: equal to x // d over the range the kernels use
+    (lanes, triple counts, bin items: below 2^17; divisors up to 128)."""
+    x = np.arange(0, 1 << 17, dtype=np.int64)
+    xf = x.astype(np.float32) + np.float32(0.5)
+    for d in range(1, 129):
+        r0 = np.float32(1.0) / np.float32(d)
+        for r in (np.nextafter(r0, np.float32(0)), r0, np.nextafter(r0, np.float32(2))):
+            q = (xf * r).astype(np.int64)
+            assert np.array_equal(q, x // d), d
