@@ -243,6 +243,20 @@ size_t qmll_sort_by_type_workspace(int A, int ne);
 int qmll_sort_by_type(const int* types, const int* slots, int A, int ne, void* workspace, size_t workspace_bytes,
                       int* sorted_slots, int* type_offsets, qmll_stream_t stream);
 
+/* qmll_sort_by_type for callers that cannot allocate device memory or carry a workspace: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference (whose wrappers allocate with torch::zeros on every call).
+ * Same inputs, outputs and results as qmll_sort_by_type; the per-workgroup counters live in a
+ * device array built into the library (QMLL_SORT_NOALLOC_MAX_COUNTS ints = 512 KiB, held on
+ * every GPU the library runs on until the process ends), so ceil(A/256)*ne must not exceed
+ * QMLL_SORT_NOALLOC_MAX_COUNTS (QMLL_ERR_INVALID otherwise).  Calls no hipMalloc / hipFree.
+ * All calls on one GPU share that array: two calls that overlap on one GPU (different
+ * streams or host threads) race; calls on one stream are ordered and safe.  The first call
+ * on a device looks the array's address up (hipGetSymbolAddress): make it outside capture. */
+#define QMLL_SORT_NOALLOC_MAX_COUNTS 131072
+int qmll_sort_by_type_noalloc(const int* types, const int* slots, int A, int ne, int* sorted_slots,
+                              int* type_offsets, qmll_stream_t stream);
+
 /* x f32 [A,d]: row a = rep[sorted_slots[a], :] . reductors[type of a]  (rep f32 [N,R],
  * reductors f32 [ne,R,d]); rows at and beyond type_offsets[ne] are not written. */
 int qmll_project_typed(const float* rep, const int* sorted_slots, const int* type_offsets, const float* reductors,

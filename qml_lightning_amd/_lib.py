@@ -54,6 +54,7 @@ PROTOTYPES = {
     "qmll_sorf_energy_typed": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, P, P, P],
     "qmll_sort_by_type_workspace": [c_int, c_int],
     "qmll_sort_by_type": [P, P, c_int, c_int, P, c_size_t, P, P, P],
+    "qmll_sort_by_type_noalloc": [P, P, c_int, c_int, P, P, P],
     "qmll_project_typed": [P, P, P, P, c_int, c_int, c_int, c_int, P, P],
     "qmll_project_typed_backward": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
     "qmll_sorf_energy_sorted": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_float, P, P, P],

@@ -12,6 +12,8 @@
 // sorted slot list, so neither the gathered representation nor a zero-padded
 // [slots, elements*d] intermediate is ever materialised.  Only real atoms of known
 // elements are touched: no work is spent on padding or on the other elements' reductors.
+#include <mutex>
+
 #include "qmll_common.h"
 
 namespace {
@@ -320,6 +322,57 @@ extern "C" int qmll_sort_by_type(const int* types, const int* slots, int A, int 
                        sorted_slots, type_offsets);
     QMLL_CHECK_LAUNCH("qmll_sort_by_type");
     return QMLL_OK;
+}
+
+// ---- the same sort for callers that cannot allocate -------------------------------------
+// The per-workgroup counts live in a file-scope device array instead of a caller workspace.
+// Every GPU the library runs on holds its own copy at its own address until the process
+// ends; the address is looked up once per device and only that pointer is ever handed to a
+// kernel (the array's name in host code is a host-side stand-in, not a device address).
+constexpr int SCRATCH_INTS = QMLL_SORT_NOALLOC_MAX_COUNTS;
+constexpr int MAX_DEVICES = 64;
+static __device__ __align__(256) int scratch[SCRATCH_INTS];
+
+namespace {
+std::mutex scratch_mutex;
+int* scratch_ptr[MAX_DEVICES] = {};
+
+// device address of `scratch` on the current device (nullptr + error text on failure)
+int* scratch_of_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        qmll_set_error("qmll_sort_by_type_noalloc: no usable current device (%d)", dev);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            qmll_set_error("qmll_sort_by_type_noalloc: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        scratch_ptr[dev] = static_cast<int*>(p);
+    }
+    return scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" int qmll_sort_by_type_noalloc(const int* types, const int* slots, int A, int ne, int* sorted_slots,
+                                         int* type_offsets, qmll_stream_t stream) {
+    QMLL_REQUIRE(A >= 0 && ne > 0 && ne <= MAXNE, QMLL_ERR_INVALID,
+                 "qmll_sort_by_type_noalloc: bad size A=%d ne=%d (at most %d types)", A, ne, MAXNE);
+    const long long need = (long long)((A + ST - 1) / ST) * ne;
+    QMLL_REQUIRE(need <= (long long)SCRATCH_INTS, QMLL_ERR_INVALID,
+                 "qmll_sort_by_type_noalloc: A=%d atoms of ne=%d types need %lld counters, the built-in scratch holds %d "
+                 "(ceil(A/%d)*ne must not exceed it); use qmll_sort_by_type with a workspace",
+                 A, ne, need, SCRATCH_INTS, ST);
+    int* counts = scratch_of_current_device();
+    if (!counts) return QMLL_ERR_LAUNCH;
+    // every counter the placement kernel reads is written by the counting kernel of the same
+    // call, so nothing of the previous call's contents needs clearing
+    return qmll_sort_by_type(types, slots, A, ne, counts, (size_t)SCRATCH_INTS * sizeof(int), sorted_slots, type_offsets,
+                             stream);
 }
 
 extern "C" int qmll_project_typed(const float* rep, const int* sorted_slots, const int* type_offsets,

@@ -69,6 +69,10 @@ def test_bad_arguments_are_refused_on_the_host():
     assert L.qmll_cholesky_workspace_bytes(0) == 0 and L.qmll_cholesky_workspace_bytes(300) > 300 * 8
     assert L.qmll_cholesky_f64(null, 16, 16, null, null, null) == _lib.QMLL_ERR_INVALID
     assert L.qmll_cholesky_f64(ctypes.c_void_p(16), 16, 8, ctypes.c_void_p(16), ctypes.c_void_p(16), null) == _lib.QMLL_ERR_INVALID
+    # the sort without a workspace refuses what its built-in counters cannot hold (ceil(A/256)*ne > 131072)
+    assert L.qmll_sort_by_type_noalloc(ctypes.c_void_p(8), ctypes.c_void_p(8), 4097 * 256, 32, ctypes.c_void_p(8),
+                                       ctypes.c_void_p(8), null) == _lib.QMLL_ERR_INVALID
+    assert b"scratch" in L.qmll_last_error()
     # empty inputs are fine and launch nothing
     assert L.qmll_sorf_forward(null, null, 0, 16, 2, 1, 1.0, null, null) == _lib.QMLL_OK
     assert L.qmll_gram_f64(null, null, 0, 16, null, null, null) == _lib.QMLL_OK
