@@ -205,6 +205,8 @@ Tensor sorf_coefficients_impl(const Tensor& u, const Tensor& D, const Tensor& cn
     Tensor uu = f32(u), DD = f32(D);
     const int A = (int)uu.size(0), d = (int)uu.size(1), S = (int)DD.size(1), T = nt.item<int>();   // SORF.cpp:85
     TORCH_CHECK(T <= DD.size(0), "ntransforms (", T, ") exceeds the ", DD.size(0), " diagonals given");
+    TORCH_CHECK(uu.dim() == 2 && DD.dim() == 3 && DD.size(2) == d, "get_SORF_coefficients: input is [", uu.sizes(),
+                "], diagonals are [", DD.sizes(), "]: the last dimensions must agree");
     Tensor out = at::empty({A, S, d}, uu.options());
     check(qmll_sorf_forward(fp(uu), fp(DD), A, d, S, T, scalar(cn), A ? out.data_ptr<float>() : nullptr, stream()),
           "qmll_sorf_forward");
@@ -217,6 +219,8 @@ Tensor sorf_coefficients_backward(const Tensor& grad, const Tensor& D, const Ten
     Tensor g = f32(grad), DD = f32(D);
     const int A = (int)g.size(0), S = (int)g.size(1), d = (int)g.size(2), T = nt.item<int>();       // SORF.cpp:99
     TORCH_CHECK(T <= DD.size(0), "ntransforms (", T, ") exceeds the ", DD.size(0), " diagonals given");
+    TORCH_CHECK(DD.dim() == 3 && DD.size(1) == S && DD.size(2) == d, "get_SORF_coefficients_backward: gradient is [",
+                g.sizes(), "], diagonals are [", DD.sizes(), "]");
     Tensor out = at::empty({A, d}, g.options());
     check(qmll_sorf_adjoint(fp(g), fp(DD), A, d, S, T, scalar(cn), A ? out.data_ptr<float>() : nullptr, stream()),
           "qmll_sorf_adjoint");
@@ -246,6 +250,8 @@ Tensor cos_features_impl(const Tensor& coeffs, const Tensor& b, const Tensor& nm
     need_cuda(batch_indexes, "batch_indexes");
     Tensor c = f32(coeffs), bb = f32(b), idx = i32(batch_indexes);
     const int A = (int)c.size(0), F = (int)c.size(1), nmol = nmol_t.item<int>();                     // SORF.cpp:118
+    TORCH_CHECK(bb.numel() == F && idx.numel() == A, "get_cos_features: coefficients are [", c.sizes(), "], bias has ",
+                bb.numel(), " entries, batch_indexes ", idx.numel());
     Tensor out = at::zeros({nmol, F}, c.options());
     if (A == 0) return out;
     // segment table of the (ascending) molecule index, validated on the device
@@ -261,6 +267,9 @@ Tensor cos_features_backward(const Tensor& grad, const Tensor& coeffs, const Ten
     Tensor g = f32(grad), c = f32(coeffs), bb = f32(b), idx = i32(batch_indexes);
     const int A = (int)c.size(0), F = (int)c.size(1), nmol = (int)g.size(0);
     (void)nmol_t;
+    TORCH_CHECK(bb.numel() == F && idx.numel() == A && g.dim() == 2 && g.size(1) == F,
+                "get_cos_features_backward: coefficients are [", c.sizes(), "], gradient [", g.sizes(), "], bias has ",
+                bb.numel(), " entries, batch_indexes ", idx.numel());
     Tensor out = at::empty({A, F}, c.options());
     if (A == 0) return out;
     check(qmll_cos_features_backward(fp(g), fp(c), fp(bb), ip(idx), A, F, nmol, out.data_ptr<float>(), stream()),
@@ -296,6 +305,10 @@ std::tuple<Tensor, Tensor> sorf_energy_impl(const Tensor& sub, const Tensor& D, 
     Tensor x = f32(sub), DD = f32(D), bb = f32(bias), al = f32(alpha);
     need_cuda(x, "sub");
     const int A = (int)x.size(0), d = (int)x.size(1), S = (int)DD.size(1), T = nt.item<int>();
+    TORCH_CHECK(DD.dim() == 3 && DD.size(2) == d && T <= DD.size(0) && bb.numel() == (int64_t)S * d &&
+                    al.numel() == (int64_t)S * d,
+                "sorf_energy: x [", x.sizes(), "], diagonals [", DD.sizes(), "], bias ", bb.numel(), " and alpha ",
+                al.numel(), " entries do not fit together");
     Tensor e = at::empty({A}, x.options()), gx = at::empty({A, d}, x.options());
     check(qmll_sorf_energy_fused(fp(x), fp(DD), fp(bb), fp(al), nullptr, A, d, S, T, scalar(cn),
                                  A ? e.data_ptr<float>() : nullptr, A ? gx.data_ptr<float>() : nullptr, stream()),
@@ -336,6 +349,9 @@ std::tuple<Tensor, Tensor> sorf_energy_typed_impl(const Tensor& x_all, const Ten
     TORCH_CHECK(x.size(1) == (int64_t)ne * d && ty.size(0) == N, "sorf_energy_typed: x_all is [", x.size(0), ", ",
                 x.size(1), "], expected [", ty.size(0), ", ", ne * d, "]");
     TORCH_CHECK(T == Tn, "sorf_energy_typed: ", Tn, " diagonals stored per stack, ", T, " transforms asked for");
+    TORCH_CHECK(bb.dim() == 2 && bb.size(0) == ne && bb.size(1) == (int64_t)S * d && al.numel() == (int64_t)S * d,
+                "sorf_energy_typed: bias [", bb.sizes(), "] / alpha with ", al.numel(), " entries do not fit ", ne,
+                " elements and ", S * d, " features");
     Tensor e = at::zeros({N}, x.options());
     Tensor gx = with_grad ? at::zeros({N, (int64_t)ne * d}, x.options()) : empty_like_none(x);
     check(qmll_sorf_energy_typed(fp(x), ip(ty), ip(sl), fp(DD), fp(bb), fp(al), (int)sl.size(0), N, ne, d, S, T,
@@ -445,6 +461,9 @@ std::tuple<Tensor, Tensor> sorf_energy_sorted_impl(const Tensor& x_, const Tenso
     TORCH_CHECK(x.size(0) == A && x.size(1) == d && off.size(0) == ne + 1, "sorf_energy_sorted: x is [", x.size(0), ", ",
                 x.size(1), "], expected [", A, ", ", d, "]");
     TORCH_CHECK(T == Tn, "sorf_energy_sorted: ", Tn, " diagonals stored per stack, ", T, " transforms asked for");
+    TORCH_CHECK(bb.dim() == 2 && bb.size(0) == ne && bb.size(1) == (int64_t)S * d && al.numel() == (int64_t)S * d,
+                "sorf_energy_sorted: bias [", bb.sizes(), "] / alpha with ", al.numel(), " entries do not fit ", ne,
+                " elements and ", S * d, " features");
     Tensor e = at::zeros({nslots}, x.options());
     Tensor gx = with_grad ? at::empty({A, d}, x.options()) : empty_like_none(x);
     check(qmll_sorf_energy_sorted(fp(x), ip(off), ip(ss), fp(DD), fp(bb), fp(al), A, ne, d, S, T, scalar(cn),
@@ -497,6 +516,7 @@ std::tuple<Tensor, Tensor> rff_energy_sorted_impl(const Tensor& x_, const Tensor
     const int ne = (int)WW.size(0), d = (int)WW.size(1), F = (int)WW.size(2), A = (int)ss.size(0);
     TORCH_CHECK(x.size(0) == A && x.size(1) == d && off.size(0) == ne + 1 && bb.size(0) == ne && bb.size(1) == F,
                 "rff_energy_sorted: x, W and b do not fit together");
+    TORCH_CHECK(al.numel() == F, "rff_energy_sorted: alpha has ", al.numel(), " entries for ", F, " features");
     Tensor e = at::zeros({nslots}, x.options());
     Tensor gx = with_grad ? at::empty({A, d}, x.options()) : empty_like_none(x);
     check(qmll_rff_energy_sorted(fp(x), ip(off), ip(ss), fp(WW), fp(bb), fp(al), A, ne, d, F,
@@ -535,18 +555,34 @@ std::tuple<Tensor, Tensor> rff_energy_sorted(const Tensor& x, const Tensor& off,
 // molecule per step pays for is dispatch, not kernels.
 #define MODEL_TENSORS                                                                                   \
     const Tensor &reductors, const Tensor &Dmat, const Tensor &bias, const Tensor &alpha, const Tensor &cn, \
-        const Tensor &nt
+        const Tensor &nt, const Tensor &model_species
 
-// rff = true: `Dmat` holds W [ne,d,F], `bias` holds b [ne,F]; cn and nt are unused
+// rff = true: `Dmat` holds W [ne,d,F], `bias` holds b [ne,F]; cn and nt are unused.
+// model_species: the charges of the model's own elements in the order of its reductors / Dmat /
+// bias rows (the reference selects each element's atoms with Z == e over the MODEL's elements,
+// models/hadamard_features.py:99-107, while the representation indexes its bins by the
+// REPRESENTATION's species); an empty tensor says the two lists are the same.
 Tensor fchl_sorf_energy_impl(FCHL_TENSORS, MODEL_TENSORS, bool with_grad, Tensor* gX_out, bool rff = false) {
     FchlInputs in = prepare(FCHL_PASS);
+    TORCH_CHECK(reductors.dim() == 3 && reductors.size(1) == in.R, "fchl_sorf_energy: reductors are [",
+                reductors.sizes(), "], the representation has ", in.R, " entries per atom");
+    const int64_t ne_model = reductors.size(0);
+    if (model_species.numel() == 0) {
+        TORCH_CHECK(ne_model == in.prm.nspecies, "fchl_sorf_energy: the model has ", ne_model,
+                    " elements, the representation ", in.prm.nspecies, " species, and no model species were given");
+    } else {
+        TORCH_CHECK(model_species.numel() == ne_model, "fchl_sorf_energy: ", model_species.numel(),
+                    " model species for ", ne_model, " reductors");
+    }
+    // which reductor / Dmat / bias row an atom takes
+    const Tensor sort_types = model_species.numel() == 0 ? in.types : element_types(in.X, Z, in.natoms, model_species);
     // the forward kernel writes every bin of a listed atom's row, and only the rows of listed
     // atoms are read below, so the padded rows need no clearing here
     Tensor rep = at::empty({in.B, in.n, in.R}, in.X.options());
     check(qmll_fchl19_forward(FCHL_ABI(in), rep.data_ptr<float>(), stream()), "qmll_fchl19_forward");
     const int64_t nslots = (int64_t)in.B * in.n;
     Tensor slots = at::add(in.atomIDs, in.molIDs, in.n);      // molIDs * n + atomIDs in one launch
-    auto sorted = sort_by_type(in.types, slots, reductors.size(0));
+    auto sorted = sort_by_type(sort_types, slots, ne_model);
     const Tensor& ss = std::get<0>(sorted);
     const Tensor& off = std::get<1>(sorted);
     Tensor x = project_typed_impl(rep.view({nslots, in.R}), ss, off, reductors);
@@ -554,7 +590,7 @@ Tensor fchl_sorf_energy_impl(FCHL_TENSORS, MODEL_TENSORS, bool with_grad, Tensor
                   : sorf_energy_sorted_impl(x, off, ss, Dmat, bias, alpha, cn, nt, nslots, with_grad);
     Tensor energies = std::get<0>(eg).view({in.B, in.n}).sum(1);
     if (with_grad) {
-        Tensor g_rep = project_typed_backward(std::get<1>(eg), ss, off, reductors, in.types, nslots);
+        Tensor g_rep = project_typed_backward(std::get<1>(eg), ss, off, reductors, sort_types, nslots);
         Tensor gX = at::zeros({in.B, in.n, 3}, in.X.options());
         check(qmll_fchl19_vjp(FCHL_ABI(in), fp(g_rep), gX.data_ptr<float>(), stream()), "qmll_fchl19_vjp");
         *gX_out = gX;
@@ -565,7 +601,7 @@ Tensor fchl_sorf_energy_impl(FCHL_TENSORS, MODEL_TENSORS, bool with_grad, Tensor
 struct FchlSorfEnergyFn : public Function<FchlSorfEnergyFn> {
     static variable_list forward(AutogradContext* ctx, FCHL_TENSORS, MODEL_TENSORS, bool with_grad) {
         Tensor gX;
-        Tensor e = fchl_sorf_energy_impl(FCHL_PASS, reductors, Dmat, bias, alpha, cn, nt, with_grad, &gX);
+        Tensor e = fchl_sorf_energy_impl(FCHL_PASS, reductors, Dmat, bias, alpha, cn, nt, model_species, with_grad, &gX);
         if (!with_grad) gX = empty_like_none(e);
         ctx->save_for_backward({gX});
         ctx->mark_non_differentiable({gX});
@@ -574,7 +610,7 @@ struct FchlSorfEnergyFn : public Function<FchlSorfEnergyFn> {
         return {e, gX};
     }
     static variable_list backward(AutogradContext* ctx, variable_list grads) {
-        variable_list out(23);
+        variable_list out(24);
         if (!grads[0].defined()) return out;
         const Tensor gX = ctx->get_saved_variables()[0];                 // [B,n,3], dE_m/dX of each molecule
         TORCH_CHECK(gX.dim() == 3, "fchl_sorf_energy was called with with_grad=False but a gradient is requested");
@@ -586,16 +622,17 @@ struct FchlSorfEnergyFn : public Function<FchlSorfEnergyFn> {
 
 // returns (energies [B], dE/dX [B,n,3] or an empty tensor when with_grad is false)
 std::tuple<Tensor, Tensor> fchl_sorf_energy(FCHL_TENSORS, MODEL_TENSORS, bool with_grad) {
-    auto r = FchlSorfEnergyFn::apply(FCHL_PASS, reductors, Dmat, bias, alpha, cn, nt, with_grad);
+    auto r = FchlSorfEnergyFn::apply(FCHL_PASS, reductors, Dmat, bias, alpha, cn, nt, model_species, with_grad);
     return {r[0], r[1]};
 }
 
 // the same chain with random Fourier features (models/random_features.py:82-102)
 struct FchlRffEnergyFn : public Function<FchlRffEnergyFn> {
     static variable_list forward(AutogradContext* ctx, FCHL_TENSORS, const Tensor& reductors, const Tensor& W,
-                                 const Tensor& b, const Tensor& alpha, bool with_grad) {
+                                 const Tensor& b, const Tensor& alpha, const Tensor& model_species, bool with_grad) {
         Tensor gX;
-        Tensor e = fchl_sorf_energy_impl(FCHL_PASS, reductors, W, b, alpha, Tensor(), Tensor(), with_grad, &gX, true);
+        Tensor e = fchl_sorf_energy_impl(FCHL_PASS, reductors, W, b, alpha, Tensor(), Tensor(), model_species, with_grad,
+                                         &gX, true);
         if (!with_grad) gX = empty_like_none(e);
         ctx->save_for_backward({gX});
         ctx->mark_non_differentiable({gX});
@@ -604,7 +641,7 @@ struct FchlRffEnergyFn : public Function<FchlRffEnergyFn> {
         return {e, gX};
     }
     static variable_list backward(AutogradContext* ctx, variable_list grads) {
-        variable_list out(21);
+        variable_list out(22);
         if (!grads[0].defined()) return out;
         const Tensor gX = ctx->get_saved_variables()[0];
         TORCH_CHECK(gX.dim() == 3, "fchl_rff_energy was called with with_grad=False but a gradient is requested");
@@ -615,8 +652,8 @@ struct FchlRffEnergyFn : public Function<FchlRffEnergyFn> {
 };
 
 std::tuple<Tensor, Tensor> fchl_rff_energy(FCHL_TENSORS, const Tensor& reductors, const Tensor& W, const Tensor& b,
-                                           const Tensor& alpha, bool with_grad) {
-    auto r = FchlRffEnergyFn::apply(FCHL_PASS, reductors, W, b, alpha, with_grad);
+                                           const Tensor& alpha, const Tensor& model_species, bool with_grad) {
+    auto r = FchlRffEnergyFn::apply(FCHL_PASS, reductors, W, b, alpha, model_species, with_grad);
     return {r[0], r[1]};
 }
 

@@ -1,6 +1,8 @@
 """Drop-in for the reference's `fchl_gpu` extension (qml_lightning/cuda/fchl_cuda.cpp:204-212).
-Argument order is the reference's; the charges argument is accepted and unused by the
-kernels there too (element types carry the information)."""
+Argument order is the reference's; the kernels there do not read the charges argument (element
+types carry the information), here it only supplies the atom counts."""
+import torch
+
 from .. import ops
 
 
@@ -19,7 +21,7 @@ def get_fchl_representation(coordinates, charges, species, element_types, cell, 
     prm = _prm(species, two_body_gridpoints, three_body_gridpoints, eta2, eta3, two_body_decay, three_body_weight,
                three_body_decay, rcut)
     return ops.fchl_forward(coordinates, element_types, cell, inv_cell, blockAtomIDs, blockMolIDs,
-                            _counts(coordinates, nneighbours), two_body_gridpoints, three_body_gridpoints, prm,
+                            _counts(coordinates, charges), two_body_gridpoints, three_body_gridpoints, prm,
                             neighbourlist, nneighbours)
 
 
@@ -29,7 +31,7 @@ def get_fchl_derivative(coordinates, charges, species, element_types, cell, inv_
     prm = _prm(species, two_body_gridpoints, three_body_gridpoints, eta2, eta3, two_body_decay, three_body_weight,
                three_body_decay, rcut)
     _, jac = ops.fchl_jacobian(coordinates, element_types, cell, inv_cell, blockAtomIDs, blockMolIDs,
-                               _counts(coordinates, nneighbours), two_body_gridpoints, three_body_gridpoints, prm,
+                               _counts(coordinates, charges), two_body_gridpoints, three_body_gridpoints, prm,
                                neighbourlist, nneighbours, with_rep=False)
     return jac
 
@@ -39,7 +41,7 @@ def get_fchl_and_derivative(coordinates, charges, species, element_types, cell, 
                             two_body_decay, three_body_weight, three_body_decay, rcut, gradients):
     prm = _prm(species, two_body_gridpoints, three_body_gridpoints, eta2, eta3, two_body_decay, three_body_weight,
                three_body_decay, rcut)
-    counts = _counts(coordinates, nneighbours)
+    counts = _counts(coordinates, charges)
     if gradients:
         rep, jac = ops.fchl_jacobian(coordinates, element_types, cell, inv_cell, blockAtomIDs, blockMolIDs, counts,
                                      two_body_gridpoints, three_body_gridpoints, prm, neighbourlist, nneighbours)
@@ -54,14 +56,15 @@ def fchl_backwards(coordinates, charges, species, element_types, cell, inv_cell,
     prm = _prm(species, two_body_gridpoints, three_body_gridpoints, eta2, eta3, two_body_decay, three_body_weight,
                three_body_decay, rcut)
     return ops.fchl_vjp(grad_in, coordinates, element_types, cell, inv_cell, blockAtomIDs, blockMolIDs,
-                        _counts(coordinates, nneighbours), two_body_gridpoints, three_body_gridpoints, prm,
+                        _counts(coordinates, charges), two_body_gridpoints, three_body_gridpoints, prm,
                         neighbourlist, nneighbours)
 
 
-def _counts(coordinates, nneighbours):
-    """The reference's signatures carry no atom counts: with a neighbour list given they are
-    not needed (the list is authoritative), so any int32 [B] tensor does."""
-    import torch
-    B = coordinates.shape[0] if coordinates.dim() == 3 else 1
-    n = coordinates.shape[-2]
-    return torch.full((B,), n, dtype=torch.int32, device=coordinates.device)
+def _counts(coordinates, charges):
+    """The reference's signatures carry no atom counts (its kernels only walk the neighbour list
+    they are given).  Here they are recovered from the zero-padded charges (a real atom has a
+    positive charge, models/kernel.py:631-648), so that a call without a list, where the kernel
+    finds the neighbours itself, does not take padded slots for atoms at the origin."""
+    if charges.dim() == 1:
+        charges = charges.unsqueeze(0)
+    return (charges > 0).sum(dim=1, dtype=torch.int32)

@@ -156,10 +156,29 @@ def _register_fused_op():
                                     lib=lib)
     # the whole fused chain as one operator: one dispatch and one autograd node per evaluation
     lib.define("fchl_sorf_energy(%s, Tensor reductors, Tensor Dmat, Tensor bias, Tensor alpha, "
-               "Tensor coeff_normalisation, Tensor ntransforms, bool with_grad) -> (Tensor, Tensor)" % ops._FCHL_SIG)
+               "Tensor coeff_normalisation, Tensor ntransforms, Tensor model_species, bool with_grad) "
+               "-> (Tensor, Tensor)" % ops._FCHL_SIG)
+
+    def sort_types(Xb, Zb, atom_counts, types, species, model_species, reductors, R):
+        """Row of the model's reductors / diagonals / bias each atom takes: its index among the
+        MODEL's elements (hadamard_features.py:99-107 selects with Z == e over them), which
+        differs from the representation's species index when the two lists differ."""
+        if reductors.dim() != 3 or reductors.shape[1] != R:
+            raise RuntimeError("fchl_sorf_energy: reductors are %s, the representation has %d entries per atom"
+                               % (tuple(reductors.shape), R))
+        if model_species.numel() == 0:
+            if reductors.shape[0] != species.shape[0]:
+                raise RuntimeError("fchl_sorf_energy: the model has %d elements, the representation %d species, and "
+                                   "no model species were given" % (reductors.shape[0], species.shape[0]))
+            return types
+        if model_species.numel() != reductors.shape[0]:
+            raise RuntimeError("fchl_sorf_energy: %d model species for %d reductors"
+                               % (model_species.numel(), reductors.shape[0]))
+        return ops.element_types(Xb, Zb, atom_counts, model_species)
 
     def impl_chain(X, Z, species, atomIDs, molIDs, atom_counts, cell, inv_cell, Rs2, Rs3, eta2, eta3, two_body_decay,
-                   three_body_weight, three_body_decay, rcut, reductors, Dmat, bias, alpha, cn, nt, with_grad):
+                   three_body_weight, three_body_decay, rcut, reductors, Dmat, bias, alpha, cn, nt, model_species,
+                   with_grad):
         Xb, Zb = ops._batched(X, Z)
         B, n = Zb.shape
         nslots = B * n
@@ -170,7 +189,7 @@ def _register_fused_op():
         inv_cell_ = inv_cell if inv_cell.numel() > 0 else None
         fargs = (Xb, types, cell_, inv_cell_, atomIDs, molIDs, atom_counts, Rs2, Rs3, prm)
         rep = ops.fchl_forward(*fargs)
-        tflat = types.view(-1)
+        tflat = sort_types(Xb, Zb, atom_counts, types, species, model_species, reductors, ops.repsize(prm)).view(-1)
         ss, off = ops.sort_by_type(tflat, molIDs * n + atomIDs, reductors.shape[0])
         x = ops.project_typed(rep.view(nslots, -1), ss, off, reductors)
         e_slots, gx = ops.sorf_energy_sorted(x, off, ss, Dmat, bias, alpha, ops._scalar(cn), int(nt.item()), nslots,
@@ -184,11 +203,12 @@ def _register_fused_op():
     lib.impl("fchl_sorf_energy", impl_chain, "CompositeExplicitAutograd")
 
     # the same chain with random Fourier features: W in place of the diagonals, b in place of the bias
-    lib.define("fchl_rff_energy(%s, Tensor reductors, Tensor W, Tensor b, Tensor alpha, bool with_grad) "
-               "-> (Tensor, Tensor)" % ops._FCHL_SIG)
+    lib.define("fchl_rff_energy(%s, Tensor reductors, Tensor W, Tensor b, Tensor alpha, Tensor model_species, "
+               "bool with_grad) -> (Tensor, Tensor)" % ops._FCHL_SIG)
 
     def impl_chain_rff(X, Z, species, atomIDs, molIDs, atom_counts, cell, inv_cell, Rs2, Rs3, eta2, eta3,
-                       two_body_decay, three_body_weight, three_body_decay, rcut, reductors, W, b, alpha, with_grad):
+                       two_body_decay, three_body_weight, three_body_decay, rcut, reductors, W, b, alpha,
+                       model_species, with_grad):
         Xb, Zb = ops._batched(X, Z)
         B, n = Zb.shape
         nslots = B * n
@@ -198,7 +218,7 @@ def _register_fused_op():
         fargs = (Xb, types, cell if cell.numel() > 0 else None, inv_cell if inv_cell.numel() > 0 else None, atomIDs,
                  molIDs, atom_counts, Rs2, Rs3, prm)
         rep = ops.fchl_forward(*fargs)
-        tflat = types.view(-1)
+        tflat = sort_types(Xb, Zb, atom_counts, types, species, model_species, reductors, ops.repsize(prm)).view(-1)
         ss, off = ops.sort_by_type(tflat, molIDs * n + atomIDs, reductors.shape[0])
         x = ops.project_typed(rep.view(nslots, -1), ss, off, reductors)
         e_slots, gx = ops.rff_energy_sorted(x, off, ss, W, b, alpha, nslots, with_grad=with_grad)
@@ -218,11 +238,11 @@ def _register_fused_op():
     def backward_chain(ctx, g_e, g_gx):
         (gX,) = ctx.saved_tensors
         if g_e is None:
-            return (None,) * 23
+            return (None,) * 24
         if gX.dim() != 3:
             raise RuntimeError("fchl_sorf_energy was called with with_grad=False but a gradient is requested")
         g = gX * g_e.reshape(-1, 1, 1)
-        return (g.squeeze(0) if ctx.xdim == 2 else g,) + (None,) * 22
+        return (g.squeeze(0) if ctx.xdim == 2 else g,) + (None,) * 23
 
     torch.library.register_autograd("qml_lightning_sorf::fchl_sorf_energy", backward_chain, setup_context=setup_chain,
                                     lib=lib)
@@ -230,11 +250,11 @@ def _register_fused_op():
     def backward_chain_rff(ctx, g_e, g_gx):
         (gX,) = ctx.saved_tensors
         if g_e is None:
-            return (None,) * 21
+            return (None,) * 22
         if gX.dim() != 3:
             raise RuntimeError("fchl_rff_energy was called with with_grad=False but a gradient is requested")
         g = gX * g_e.reshape(-1, 1, 1)
-        return (g.squeeze(0) if ctx.xdim == 2 else g,) + (None,) * 20
+        return (g.squeeze(0) if ctx.xdim == 2 else g,) + (None,) * 21
 
     torch.library.register_autograd("qml_lightning_sorf::fchl_rff_energy", backward_chain_rff,
                                     setup_context=setup_chain, lib=lib)
@@ -242,6 +262,15 @@ def _register_fused_op():
 
 
 _register_fused_op()
+
+
+def model_species_for_sort(species, rep):
+    """What the one-operator predict chain gets as `model_species`: the model's element list
+    when it differs from the representation's species list (a subset, another order), else an
+    empty tensor, which lets the chain reuse the representation's element types."""
+    if rep is not None and tuple(rep.species.shape) == tuple(species.shape) and bool((rep.species.cpu() == species.cpu()).all()):
+        return torch.empty(0, dtype=torch.float32, device=species.device)
+    return species
 
 
 class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
@@ -259,6 +288,7 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         self.nbatch_train = nbatch_train
         self.nbatch_test = nbatch_test
         self.species = torch.from_numpy(np.asarray(elements)).float().to(self.device)
+        self.sort_species = model_species_for_sort(self.species, rep)
         self.npcas = npcas
         self.fused = fused
         self.separate_ops = separate_ops   # fused route as five operators (one node each) instead of one
@@ -348,7 +378,7 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
                 X, Z, self.rep.species, atomIDs, molIDs, atom_counts, cell, inv_cell, self.rep.Rs2, self.rep.Rs3,
                 self.rep.eta2, self.rep.eta3, self.rep.two_body_decay, self.rep.three_body_weight,
                 self.rep.three_body_decay, self.rep.rcut, self.reductors, self.Dmat, self.bias, alpha,
-                coeff_normalisation, self.ntransforms, X.requires_grad)
+                coeff_normalisation, self.ntransforms, self.sort_species, X.requires_grad)
             return energies
 
         torch_rep = self.rep.forward(X, Z, atomIDs, molIDs, atom_counts, cell, inv_cell)
@@ -406,7 +436,8 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
             energies, gX = torch.ops.qml_lightning_sorf.fchl_sorf_energy(
                 coordinates, charges, rep.species, atomIDs, molIDs, natom_counts, cells, inv_cells, rep.Rs2, rep.Rs3,
                 rep.eta2, rep.eta3, rep.two_body_decay, rep.three_body_weight, rep.three_body_decay, rep.rcut,
-                self.reductors, self.Dmat, self.bias, alpha_f32(self), coeff_normalisation, self.ntransforms, forces)
+                self.reductors, self.Dmat, self.bias, alpha_f32(self), coeff_normalisation, self.ntransforms,
+                self.sort_species, forces)
         return energies, (gX.neg_() if forces else None)
 
     @torch.jit.unused

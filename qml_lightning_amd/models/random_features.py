@@ -33,6 +33,7 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
         self.nbatch_test = nbatch_test
         self._nfeatures = nstacks * self.npcas
         self.species = torch.from_numpy(np.asarray(elements)).float().to(self.device)
+        self.sort_species = hadamard_features.model_species_for_sort(self.species, rep)
         self.sample_elemental_basis()
         self.feature_normalisation = float(np.sqrt(2.0 / self._nfeatures))
         self.is_trained = False
@@ -78,7 +79,7 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
                 X, Z, self.rep.species, atomIDs, molIDs, atom_counts, cell, inv_cell, self.rep.Rs2, self.rep.Rs3,
                 self.rep.eta2, self.rep.eta3, self.rep.two_body_decay, self.rep.three_body_weight,
                 self.rep.three_body_decay, self.rep.rcut, self.reductors, self.W, self.b, self.alpha.float(),
-                X.requires_grad)
+                self.sort_species, X.requires_grad)
             return energies
         torch_rep = self.rep.forward(X, Z, atomIDs, molIDs, atom_counts, cell, inv_cell)
         if self.fused:
@@ -122,7 +123,7 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
             energies, gX = torch.ops.qml_lightning_sorf.fchl_rff_energy(
                 coordinates, charges, rep.species, atomIDs, molIDs, natom_counts, cells, inv_cells, rep.Rs2, rep.Rs3,
                 rep.eta2, rep.eta3, rep.two_body_decay, rep.three_body_weight, rep.three_body_decay, rep.rcut,
-                self.reductors, self.W, self.b, alpha_f32(self), forces)
+                self.reductors, self.W, self.b, alpha_f32(self), self.sort_species, forces)
         return energies, (gX.neg_() if forces else None)
 
     @torch.jit.unused

@@ -210,6 +210,9 @@ def sorf_forward(u, D, normalisation, ntransforms):
     T, S = int(ntransforms), int(D.shape[1])
     if T > D.shape[0]:
         raise RuntimeError("ntransforms (%d) exceeds the %d diagonals given" % (T, D.shape[0]))
+    if D.dim() != 3 or D.shape[2] != d:
+        raise RuntimeError("sorf_forward: input is %s, diagonals are %s: the last dimensions must agree"
+                           % (tuple(u.shape), tuple(D.shape)))
     out = torch.empty((A, S, d), dtype=torch.float32, device=u.device)
     check(_lib.lib().qmll_sorf_forward(_ptr(u), _ptr(D), A, d, S, T, float(normalisation), _ptr(out), _stream()),
           "qmll_sorf_forward")
@@ -223,6 +226,8 @@ def sorf_adjoint(g, D, normalisation, ntransforms):
     g, D = _f32(g), _f32(D)
     A, S, d = g.shape
     T = int(ntransforms)
+    if D.dim() != 3 or T > D.shape[0] or D.shape[1] != S or D.shape[2] != d:
+        raise RuntimeError("sorf_adjoint: gradient is %s, diagonals are %s, %d transforms" % (tuple(g.shape), tuple(D.shape), T))
     out = torch.empty((A, d), dtype=torch.float32, device=g.device)
     check(_lib.lib().qmll_sorf_adjoint(_ptr(g), _ptr(D), A, d, S, T, float(normalisation), _ptr(out), _stream()),
           "qmll_sorf_adjoint")
@@ -246,10 +251,13 @@ def cos_features(coeffs, bias, nmol, mol_index, out=None):
     _need_cuda(mol_index, "batch_indexes")
     coeffs, bias, mol_index = _f32(coeffs), _f32(bias), _i32(mol_index)
     A, F = coeffs.shape
+    if bias.numel() != F or mol_index.numel() != A:
+        raise RuntimeError("cos_features: coefficients are %s, bias has %d entries, batch_indexes %d"
+                           % (tuple(coeffs.shape), bias.numel(), mol_index.numel()))
     if out is None:
         out = torch.zeros((int(nmol), F), dtype=torch.float32, device=coeffs.device)
-    if not out.is_contiguous():
-        raise RuntimeError("feature matrix must be contiguous")
+    if not out.is_contiguous() or out.dim() != 2 or out.shape[1] != F:
+        raise RuntimeError("feature matrix must be contiguous with %d columns" % F)
     fn = _lib.lib().qmll_cos_features_f64 if out.dtype == torch.float64 else _lib.lib().qmll_cos_features_f32
     seg = segment_offsets(mol_index, out.shape[0]) if A > 0 else None
     check(fn(_ptr(coeffs), _ptr(bias), _ptr(mol_index), _ptr(seg), A, F, int(out.shape[0]), _ptr(out), _stream()),
@@ -260,6 +268,9 @@ def cos_features(coeffs, bias, nmol, mol_index, out=None):
 def cos_features_backward(gZ, coeffs, bias, nmol, mol_index):
     gZ, coeffs, bias, mol_index = _f32(gZ), _f32(coeffs), _f32(bias), _i32(mol_index)
     A, F = coeffs.shape
+    if bias.numel() != F or mol_index.numel() != A or gZ.dim() != 2 or gZ.shape[1] != F:
+        raise RuntimeError("cos_features_backward: coefficients are %s, gradient %s, bias has %d entries, batch_indexes %d"
+                           % (tuple(coeffs.shape), tuple(gZ.shape), bias.numel(), mol_index.numel()))
     out = torch.empty((A, F), dtype=torch.float32, device=coeffs.device)
     check(_lib.lib().qmll_cos_features_backward(_ptr(gZ), _ptr(coeffs), _ptr(bias), _ptr(mol_index), A, F,
                                                 int(gZ.shape[0]), _ptr(out), _stream()), "qmll_cos_features_backward")
@@ -269,6 +280,8 @@ def cos_features_backward(gZ, coeffs, bias, nmol, mol_index):
 def sin_coeffs(coeffs, bias, out):
     coeffs, bias = _f32(coeffs), _f32(bias)
     A, F = coeffs.shape
+    if bias.numel() != F:
+        raise RuntimeError("sin_coeffs: bias has %d entries for %d features" % (bias.numel(), F))
     if out.dtype != torch.float64 or not out.is_contiguous() or tuple(out.shape) != (A, F):
         raise RuntimeError("sin_coeffs output must be a contiguous float64 [A,F] tensor")
     check(_lib.lib().qmll_sin_coeffs_f64(_ptr(coeffs), _ptr(bias), A, F, _ptr(out), _stream()), "qmll_sin_coeffs_f64")
@@ -339,6 +352,9 @@ def sorf_energy_fused(x, D, bias, alpha, out_index, normalisation, ntransforms, 
     x, D, bias, alpha = _f32(x), _f32(D), _f32(bias), _f32(alpha)
     A, d = x.shape
     S, T = int(D.shape[1]), int(ntransforms)
+    if D.dim() != 3 or D.shape[2] != d or T > D.shape[0] or bias.numel() != S * d or alpha.numel() != S * d:
+        raise RuntimeError("sorf_energy_fused: x %s, diagonals %s, bias with %d and alpha with %d entries do not fit together"
+                           % (tuple(x.shape), tuple(D.shape), bias.numel(), alpha.numel()))
     gx = torch.empty((A, d), dtype=torch.float32, device=x.device) if with_grad else None
     check(_lib.lib().qmll_sorf_energy_fused(_ptr(x), _ptr(D), _ptr(bias), _ptr(alpha), _ptr(out_index), A, d, S, T,
                                             float(normalisation), _ptr(e_atom), _ptr(gx), _stream()),
@@ -358,6 +374,9 @@ def sorf_energy_typed(x_all, types, atom_slots, Dmat, bias, alpha, normalisation
     T = int(ntransforms)
     if T != Tn:
         raise RuntimeError("sorf_energy_typed: %d diagonals stored per stack, %d transforms asked for" % (Tn, T))
+    if tuple(bias.shape) != (ne, S * d) or alpha.numel() != S * d:
+        raise RuntimeError("sorf_energy_typed: bias %s / alpha with %d entries do not fit %d elements and %d features"
+                           % (tuple(bias.shape), alpha.numel(), ne, S * d))
     e_slots = torch.zeros(N, dtype=torch.float32, device=x_all.device)
     gx = torch.zeros((N, ne * d), dtype=torch.float32, device=x_all.device) if with_grad else None
     check(_lib.lib().qmll_sorf_energy_typed(_ptr(x_all), _ptr(types), _ptr(atom_slots), _ptr(Dmat), _ptr(bias),
@@ -431,6 +450,9 @@ def sorf_energy_sorted(x, type_offsets, sorted_slots, Dmat, bias, alpha, normali
     T = int(ntransforms)
     if T != Tn:
         raise RuntimeError("sorf_energy_sorted: %d diagonals stored per stack, %d transforms asked for" % (Tn, T))
+    if tuple(bias.shape) != (ne, S * d) or alpha.numel() != S * d:
+        raise RuntimeError("sorf_energy_sorted: bias %s / alpha with %d entries do not fit %d elements and %d features"
+                           % (tuple(bias.shape), alpha.numel(), ne, S * d))
     e_slots = torch.zeros(int(nslots), dtype=torch.float32, device=x.device)
     gx = torch.empty((A, d), dtype=torch.float32, device=x.device) if with_grad else None
     check(_lib.lib().qmll_sorf_energy_sorted(_ptr(x), _ptr(type_offsets), _ptr(sorted_slots), _ptr(Dmat), _ptr(bias),
@@ -447,6 +469,9 @@ def rff_features(x, W, b, mol_index, Zf):
     W, b = W.double().contiguous(), b.double().contiguous()
     A, d = x.shape
     F = W.shape[1]
+    if W.shape[0] != d or b.numel() != F or mol_index.numel() != A or Zf.dtype != torch.float64 or Zf.shape[1] != F:
+        raise RuntimeError("rff_features: x %s, W %s, b with %d entries, features %s do not fit together"
+                           % (tuple(x.shape), tuple(W.shape), b.numel(), tuple(Zf.shape)))
     check(_lib.lib().qmll_rff_features(_ptr(x), _ptr(W), _ptr(b), _ptr(mol_index), A, d, F, int(Zf.shape[0]), _ptr(Zf),
                                        _stream()), "qmll_rff_features")
     return Zf
@@ -459,6 +484,10 @@ def rff_derivative_features(x, grad, W, b, mol_index, G, molecule_major=False):
     W, b = W.double().contiguous(), b.double().contiguous()
     A, n, _, d = grad.shape
     F = W.shape[1]
+    if (tuple(x.shape) != (A, d) or W.shape[0] != d or b.numel() != F or mol_index.numel() != A
+            or G.dtype != torch.float64 or tuple(G.shape[1:]) != (n, 3, F)):
+        raise RuntimeError("rff_derivative_features: x %s, grad %s, W %s, b with %d entries, output %s do not fit together"
+                           % (tuple(x.shape), tuple(grad.shape), tuple(W.shape), b.numel(), tuple(G.shape)))
     nmol = int(G.shape[0])
     seg = None
     if molecule_major:
@@ -479,6 +508,8 @@ def rff_energy_sorted(x, type_offsets, sorted_slots, W, b, alpha, nslots, with_g
     if x.shape[0] != A or x.shape[1] != d or type_offsets.shape[0] != ne + 1 or b.shape[0] != ne or b.shape[1] != F:
         raise RuntimeError("rff_energy_sorted: x %s, W %s, b %s do not fit together"
                            % (tuple(x.shape), tuple(W.shape), tuple(b.shape)))
+    if alpha.numel() != F:
+        raise RuntimeError("rff_energy_sorted: alpha has %d entries for %d features" % (alpha.numel(), F))
     e_slots = torch.zeros(int(nslots), dtype=torch.float32, device=x.device)
     gx = torch.empty((A, d), dtype=torch.float32, device=x.device) if with_grad else None
     check(_lib.lib().qmll_rff_energy_sorted(_ptr(x), _ptr(type_offsets), _ptr(sorted_slots), _ptr(W), _ptr(b),

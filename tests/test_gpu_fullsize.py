@@ -124,6 +124,21 @@ def test_config4_32768_features_batch_equals_its_parts():
     within(e, E[1000:1300], 1e-5, "e")
     within(f, F[1000:1300], 1e-5, "f")
     assert float(F.sum(dim=1).abs().max()) <= 1e-4 * float(F.abs().max())
+    # the training route at this width (Jacobian -> projected rows -> force-feature rows, fp64)
+    # against the predict route (fused kernel + VJP, fp32): rows . alpha = energies and forces
+    rows_times_alpha_equals_prediction(m, coords[:48], charges[:48], E[:48], F[:48])
+
+
+def rows_times_alpha_equals_prediction(m, coords, charges, E, F):
+    data = m.format_data([np.asarray(c, dtype=np.float32) for c in coords], charges, E=[0.0] * len(coords),
+                         F=[np.zeros((len(q), 3)) for q in charges])
+    rows = m._batch_rows(data, True)
+    B = len(coords)
+    assert rows.shape == (B + F[0].numel() * B, m.nfeatures()) and rows.dtype == torch.float64
+    out = rows @ m.alpha.double()
+    within(out[:B], E.double(), 1e-4, "rows . alpha vs predicted energies")
+    within(out[B:].reshape(F.shape), F.double(), 1e-4, "rows . alpha vs predicted forces")
+    return rows
 
 
 def test_config5_rff_32768_features_batch_equals_its_parts():
@@ -131,7 +146,7 @@ def test_config5_rff_32768_features_batch_equals_its_parts():
     from qml_lightning_amd.representations.FCHL import FCHLCuda
     from qml_lightning_amd.utils import synthetic
     species = [1, 6, 8]
-    coords, charges = synthetic.fixed_composition_batch(synthetic.ASPIRIN, 2048, seed=1)
+    coords, charges = synthetic.fixed_composition_batch(synthetic.ASPIRIN, 4096, seed=1)
     np.random.seed(15)
     rep = FCHLCuda(species=np.array(species))
     m = RandomFourrierFeaturesModel(rep=rep, elements=np.array(species), sigma=2.0, llambda=1e-5, npcas=128,
@@ -146,7 +161,26 @@ def test_config5_rff_32768_features_batch_equals_its_parts():
     # 32768 fp32 terms per energy, summed in an order that depends on the batch size
     within(e, E[700:900], 5e-5, "rff energies, part vs whole")
     within(f, F[700:900], 5e-5, "rff forces, part vs whole")
+    e, f = step(m, coords[4000:], charges[4000:])
+    within(e, E[4000:], 5e-5, "rff energies, last part vs whole")
+    within(f, F[4000:], 5e-5, "rff forces, last part vs whole")
     assert float(F.sum(dim=1).abs().max()) <= 1e-4 * float(F.abs().max())
+    # training rows at 32768 features (fp64 feature and matrix-core derivative kernels) against the
+    # fused fp32 predict kernel, then Z^T Z / Z^T y of those rows through build_Z_components
+    rows = rows_times_alpha_equals_prediction(m, coords[:96], charges[:96], E[:96], F[:96])
+    rng = np.random.default_rng(4)
+    Et = rng.normal(size=96)
+    Ft = [rng.normal(size=(21, 3)) for _ in range(96)]
+    m.nbatch_train = 48
+    ZTZ, ZTy = m.build_Z_components([np.asarray(c, dtype=np.float32) for c in coords[:96]], charges[:96], E=Et, F=Ft,
+                                    print_info=False)
+    y = torch.tensor(np.concatenate([Et, np.array(Ft).reshape(-1)]), device=dev())
+    v = torch.randn(m.nfeatures(), dtype=torch.float64, device=dev(), generator=torch.Generator(device=dev()).manual_seed(1))
+    assert torch.equal(ZTZ, ZTZ.T)
+    fro = float((rows * rows).sum())
+    assert abs(float(ZTZ.diagonal().sum()) - fro) <= 1e-11 * fro
+    within(ZTZ @ v, rows.T @ (rows @ v), 1e-10, "rff ZTZ @ v")
+    within(ZTy[:, 0], rows.T @ y, 1e-10, "rff ZTy")      # a sum over rows: the split into two batches does not matter
 
 
 def test_gram_16384_features_checksums_and_solve_residual():
@@ -179,3 +213,33 @@ def test_gram_16384_features_checksums_and_solve_residual():
     assert int(info.item()) == 0
     resid = float((ZTZ @ x - ZTy).abs().max() / ZTy.abs().max())
     assert resid <= 1e-10, resid
+
+
+def test_gram_32768_features_41000_rows_checksums():
+    """Z^T Z at the width and row count of the 32768-feature training configuration (500 molecules
+    of 27 atoms with forces: 41000 rows) in its two batches of 250 molecules (20500 rows each):
+    symmetry, trace = |Z|_F^2, (Z^T Z) v = Z^T (Z v), Z^T y."""
+    from qml_lightning_amd import ops
+    F, M = 32768, 250 * (1 + 27 * 3)
+    g = torch.Generator(device=dev()).manual_seed(5)
+    ZTZ = torch.zeros(F, F, dtype=torch.float64, device=dev())
+    ZTy = torch.zeros(F, 1, dtype=torch.float64, device=dev())
+    v = torch.randn(F, 1, dtype=torch.float64, device=dev(), generator=g)
+    ref_v = torch.zeros_like(v)
+    ref_y = torch.zeros_like(v)
+    fro = 0.0
+    for _ in range(2):
+        Z = torch.randn(M, F, dtype=torch.float64, device=dev(), generator=g)
+        y = torch.randn(M, 1, dtype=torch.float64, device=dev(), generator=g)
+        ops.gram(Z, y, ZTZ, ZTy, mirror=False)
+        ref_v += Z.T @ (Z @ v)
+        ref_y += Z.T @ y
+        fro += float((Z * Z).sum())
+        del Z, y
+    ops.gram_mirror(ZTZ)
+    # symmetry in row blocks (a transposed view of the whole 8.6 GB matrix need not be materialised)
+    for lo in range(0, F, 4096):
+        assert torch.equal(ZTZ[lo:lo + 4096], ZTZ[:, lo:lo + 4096].T)
+    assert abs(float(ZTZ.diagonal().sum()) - fro) <= 1e-12 * fro
+    within(ZTZ @ v, ref_v, 1e-11, "ZTZ @ v")
+    within(ZTy, ref_y, 1e-12, "ZTy")

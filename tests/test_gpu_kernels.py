@@ -550,6 +550,51 @@ def test_cholesky_solve_matches_lapack(F):
     assert int(info2.item()) == 0
 
 
+@pytest.mark.parametrize("llambda", [1e-11, 1e-10])
+@pytest.mark.parametrize("kind", ["fewer_rows", "smooth_columns"])
+def test_regularised_solve_of_a_numerically_rank_deficient_gram_matrix(kind, llambda):
+    """The shipped default is lambda = 1e-11 (HadamardFeaturesModel), where Z^T Z + lambda I has a
+    condition number near 1 / eps: fewer rows than features (exactly rank deficient before lambda)
+    and smooth, strongly correlated columns.  BaseKernel._solve_spd (blocked Cholesky with
+    explicitly inverted diagonal blocks, LU when a pivot is not positive) must leave a residual
+    no worse than ten times that of the reference's LU route (kernel.py:231) on the same matrix."""
+    from qml_lightning_amd.models.kernel import BaseKernel
+    rng = np.random.default_rng(17)
+    F = 700
+    if kind == "fewer_rows":
+        Zr = rng.normal(size=(F // 2, F))
+    else:
+        t = np.linspace(0.0, 1.0, F)[None, :]
+        Zr = np.cos(rng.uniform(0.5, 3.0, (F + 50, 1)) * t + rng.uniform(0, 6.28, (F + 50, 1)))
+    A = Zr.T @ Zr
+    b = Zr.T @ rng.normal(size=(Zr.shape[0], 1))
+    A[np.diag_indices(F)] += llambda
+    x = BaseKernel._solve_spd(torch.tensor(A, device=dev()), torch.tensor(b, device=dev())).cpu().numpy()
+    x_lu = np.linalg.solve(A, b)
+    resid = np.abs(A @ x - b).max()
+    resid_lu = np.abs(A @ x_lu - b).max()
+    print("%s lambda %.0e: cond %.1e, residual %.2e (LU %.2e), |x| %.2e" % (kind, llambda, np.linalg.cond(A), resid,
+                                                                           resid_lu, np.abs(x).max()))
+    assert np.isfinite(x).all()
+    assert resid <= 10 * resid_lu + 1e-12 * np.abs(b).max(), (resid, resid_lu)
+
+
+def test_solve_falls_back_to_lu_when_a_pivot_is_not_positive():
+    """A symmetric matrix that rounding has left indefinite: the Cholesky route reports the pivot
+    and _solve_spd returns the LU solution."""
+    from qml_lightning_amd.models.kernel import BaseKernel
+    rng = np.random.default_rng(6)
+    F = 300
+    Q, _ = np.linalg.qr(rng.normal(size=(F, F)))
+    w = np.linspace(1.0, 2.0, F)
+    w[123] = -1e-3                                          # one slightly negative eigenvalue
+    A = (Q * w) @ Q.T
+    A = 0.5 * (A + A.T)
+    b = rng.normal(size=(F, 1))
+    x = BaseKernel._solve_spd(torch.tensor(A, device=dev()), torch.tensor(b, device=dev())).cpu().numpy()
+    assert np.abs(A @ x - b).max() <= 1e-9 * np.abs(x).max()
+
+
 def test_cholesky_in_place_on_a_strided_view():
     """overwrite_a=True factors inside a wider buffer (row stride 700 for a 300 x 300 matrix) and
     touches nothing outside the matrix."""

@@ -68,12 +68,14 @@ def test_reference_known_answer_aspirin(kat):
 
 
 @pytest.mark.parametrize("fused", [True, False])
-@pytest.mark.parametrize("case", ["benzene_c1", "aspirin_c2", "ragged_c3"])
+@pytest.mark.parametrize("case", ["benzene_c1", "aspirin_c2", "ragged_c3", "flexible_c4"])
 def test_sorf_energy_and_forces_vs_oracle(case, fused):
     cfg = {
         "benzene_c1": (helpers.benzene_batch(5, 0), [1, 6], 64, 8),
         "aspirin_c2": (helpers.fixed_composition_batch(helpers.ASPIRIN, 4, 1), [1, 6, 8], 128, 16),
         "ragged_c3": (helpers.ragged_batch(9, 2), [1, 6, 7, 8, 9], 128, 4),
+        # the shape of the 32768-feature configuration: four species, 27 atoms, 256 components
+        "flexible_c4": (helpers.fixed_composition_batch(helpers.C12H12N2O, 2, 3, sigma=0.15), [1, 6, 7, 8], 256, 4),
     }[case]
     (coords, charges), species, npcas, nstacks = cfg
     m, (red, D, bias, alpha) = build_sorf_model(species, npcas, nstacks, fused=fused)

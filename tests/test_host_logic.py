@@ -118,3 +118,46 @@ def test_small_integer_division_through_a_float_reciprocal_is_exact():
         for r in (np.nextafter(r0, np.float32(0)), r0, np.nextafter(r0, np.float32(2))):
             q = (xf * r).astype(np.int64)
             assert np.array_equal(q, x // d), d
+
+
+def test_rff_model_draws_its_basis_as_the_reference_does():
+    """W = N(0, 1) / (2 sigma^2) per element and feature, b ~ U(0, 2 pi)
+    (models/random_features.py:38,54-55): sample moments of a 16 x 4096 draw per element."""
+    from qml_lightning_amd.models.random_features import RandomFourrierFeaturesModel
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    np.random.seed(3)
+    rep = FCHLCuda(species=np.array([1, 6, 8]))
+    for sigma in (2.0, 0.7):
+        m = RandomFourrierFeaturesModel(rep=rep, elements=np.array([1, 6, 8]), sigma=sigma, nstacks=256, npcas=16)
+        assert m.W.shape == (3, 16, 4096) and m.b.shape == (3, 4096) and m.W.dtype == torch.float32
+        s = 1.0 / (2.0 * sigma ** 2)
+        for e in range(3):
+            W = m.W[e].double().cpu().numpy()
+            b = m.b[e].double().cpu().numpy()
+            n = W.size
+            assert abs(W.std() - s) < 4 * s / np.sqrt(2 * n)          # 4 sigma of the sample std
+            assert abs(W.mean()) < 4 * s / np.sqrt(n)
+            assert b.min() >= 0.0 and b.max() < 2 * np.pi + 1e-6
+            assert abs(b.mean() - np.pi) < 4 * (2 * np.pi / np.sqrt(12)) / np.sqrt(b.size)
+            assert abs(b.std() - 2 * np.pi / np.sqrt(12)) < 0.05
+        assert np.isclose(m.feature_normalisation, np.sqrt(2.0 / 4096))
+        assert not np.allclose(m.W[0].cpu().numpy(), m.W[1].cpu().numpy())        # a draw of its own per element
+
+
+def test_model_species_for_the_element_sort():
+    """The one-operator predict chain indexes reductors / diagonals / bias by the MODEL's element
+    list; the representation indexes its bins by ITS species list.  Equal lists: an empty tensor
+    (the chain reuses the representation's element types); a subset or another order: the model's
+    own list travels with the call."""
+    from qml_lightning_amd.models.hadamard_features import HadamardFeaturesModel, model_species_for_sort
+    from qml_lightning_amd.models.random_features import RandomFourrierFeaturesModel
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    rep = FCHLCuda(species=np.array([1, 6, 7, 8]))
+    same = HadamardFeaturesModel(rep=rep, elements=np.array([1, 6, 7, 8]), ntransforms=1, npcas=16, nstacks=2)
+    assert same.sort_species.numel() == 0
+    sub = HadamardFeaturesModel(rep=rep, elements=np.array([1, 6, 8]), ntransforms=1, npcas=16, nstacks=2)
+    assert sub.sort_species.tolist() == [1.0, 6.0, 8.0] and sub.reductors.shape[0] == 3
+    perm = RandomFourrierFeaturesModel(rep=rep, elements=np.array([8, 1, 6, 7]), nstacks=2, npcas=64)
+    assert perm.sort_species.tolist() == [8.0, 1.0, 6.0, 7.0]
+    assert model_species_for_sort(torch.tensor([1.0, 6.0]), None).tolist() == [1.0, 6.0]
+    assert "sort_species" in torch.jit.script(sub).code

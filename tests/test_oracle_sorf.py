@@ -179,3 +179,40 @@ def test_rff_closed_form_and_forces():
     Ep = model.rff_energy_forces(Xp, Z, aid, mid, nat, prm, [1, 6], red, W, b, alpha, forces=False)[0]
     Em = model.rff_energy_forces(Xm, Z, aid, mid, nat, prm, [1, 6], red, W, b, alpha, forces=False)[0]
     assert np.isclose(Fr[1, 4, 1], -(Ep - Em).sum() / (2 * h), rtol=1e-5)
+
+
+def test_rff_normalisation_is_pinned_by_the_gaussian_kernel_identity():
+    """Random Fourier features approximate a Gaussian kernel (Rahimi & Recht 2007): for W with
+    independent N(0, s^2) entries and b ~ U(0, 2 pi), z(x) = sqrt(2/F) cos(x W + b) satisfies
+    E[z(x).z(y)] = exp(-s^2 |x - y|^2 / 2), so z(x).z(x) -> 1.  A wrong feature normalisation
+    (sqrt(1/F), 2/F, a missing factor) or a wrong use of W or b moves these by O(1); the sampling
+    error at F = 1e5 is sqrt(1/(2F)) = 2.2e-3 for z(x).z(x) and below 3.2e-3 for z(x).z(y):
+    the 1e-2 bound below is three of those.  The reference draws W = N(0,1) / (2 sigma^2)
+    (models/random_features.py:54), i.e. s = 1 / (2 sigma^2)."""
+    rng = np.random.default_rng(42)
+    F, d, sigma = 100000, 6, 0.6
+    s = 1.0 / (2.0 * sigma ** 2)
+    W = rng.normal(size=(d, F)) * s
+    b = rng.uniform(0.0, 2.0 * np.pi, F)
+    x = rng.normal(size=(5, d)) * 0.5
+    # one atom per molecule: row a of the feature matrix is z(x_a)
+    Z = sorf.rff_features(x, W, b, np.arange(5), 5)
+    K = Z @ Z.T
+    d2 = ((x[:, None, :] - x[None, :, :]) ** 2).sum(-1)
+    expect = np.exp(-0.5 * s * s * d2)
+    assert expect.min() < 0.5                      # the test points are not all on top of each other
+    assert np.abs(np.diag(K) - 1.0).max() < 1e-2
+    assert np.abs(K - expect).max() < 1e-2
+    # two atoms in one molecule add their feature vectors (random_features_kernel.cu:28-40)
+    Z2 = sorf.rff_features(x[:2], W, b, np.array([0, 0]), 1)
+    assert np.allclose(Z2[0], Z[0] + Z[1])
+    # the force-feature rows are minus the derivative of the features along the given rows
+    grad = np.eye(d).reshape(1, 2, 3, d)             # row (j, c) of the "Jacobian" is the unit vector 3 j + c
+    G = sorf.rff_derivative_features(x[:1], grad, W, b, np.array([0]), 1)
+    h = 1e-6
+    for k in (0, 4):
+        xp, xm = x[:1].copy(), x[:1].copy()
+        xp[0, k] += h
+        xm[0, k] -= h
+        fd = (sorf.rff_features(xp, W, b, np.array([0]), 1) - sorf.rff_features(xm, W, b, np.array([0]), 1)) / (2 * h)
+        assert np.abs(G[0, k // 3, k % 3] + fd[0]).max() < 1e-8
