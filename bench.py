@@ -43,6 +43,38 @@ def cpu_baseline_worker(args):
     return E, F
 
 
+def cpu_config1_worker(args):
+    """Configuration 1 (the CPU-reference configuration): energies + forces of C6H6 copies, fp64 oracle."""
+    coords, charges, weights = args
+    from oracle import fchl19, model as omodel
+    red, D, bias, alpha = weights
+    prm = fchl19.FCHLParams([1, 6])
+    X, Z, aid, mid, nat = omodel.format_batch(coords, charges)
+    return omodel.sorf_energy_forces(X, Z, aid, mid, nat, prm, [1, 6], red, D.astype(np.float64), bias, alpha, SIGMA)[:2]
+
+
+def cpu_config1(cores):
+    """The whole of configuration 1 on the host: 100 noisy C6H6, npcas 64, nstacks 8, fp64."""
+    import multiprocessing as mp
+    from qml_lightning_amd.utils import synthetic
+    coords, charges = synthetic.benzene_batch(100, seed=0)
+    coords = [c.astype(np.float32).astype(np.float64) for c in coords]      # the values the GPU side receives
+    red, D, bias, alpha = synthetic.model_weights(2, 2 * 24 + 2 * 3 * 20, 64, 8)
+    weights = (red, D, bias, alpha.astype(np.float32).astype(np.float64))
+    chunks = [(coords[i::cores], charges[i::cores], weights) for i in range(cores)]
+    ctx = mp.get_context("fork")
+    with ctx.Pool(cores) as pool:
+        pool.map(cpu_config1_worker, [(c[0][:1], c[1][:1], c[2]) for c in chunks])      # import + warm
+        t0 = time.perf_counter()
+        res = pool.map(cpu_config1_worker, chunks)
+        dt = time.perf_counter() - t0
+    E = np.zeros(100)
+    F = np.zeros((100, 12, 3))
+    for i, (e, f) in enumerate(res):
+        E[i::cores], F[i::cores] = e, f
+    return {"seconds": dt, "E": E, "F": F, "cores": cores}
+
+
 def cpu_baseline(coords, charges, weights, nsample, cores):
     """The oracle ("port") on `cores` host processes over the first `nsample` molecules."""
     import multiprocessing as mp
@@ -129,7 +161,12 @@ def other_configs(torch, dev):
     out = {}
     # config 1: 100 noisy C6H6, npcas 64 x nstacks 8
     coords, charges = synthetic.benzene_batch(100, seed=0)
-    out["config1_c6h6_100"] = predict_rate(sorf_model([1, 6], 64, 8, 64), coords, charges, True, steps=50, warm=10)
+    m1 = sorf_model([1, 6], 64, 8, 64)
+    out["config1_c6h6_100"] = predict_rate(m1, coords, charges, True, steps=50, warm=10)
+    d1 = m1.format_data([c.astype(np.float32) for c in coords], charges)
+    e1, f1 = m1.energies_and_forces(d1['coordinates'], d1['charges'], d1['atomIDs'], d1['molIDs'], d1['natom_counts'])
+    out["config1_c6h6_100"]["_E"] = e1.double().cpu().numpy()
+    out["config1_c6h6_100"]["_F"] = f1.double().cpu().numpy()
     # config 3: 8192 ragged molecules (3..29 atoms, H C N O F), npcas 128 x nstacks 64, energies only
     coords, charges = synthetic.ragged_batch(8192, seed=2)
     out["config3_ragged_8192"] = predict_rate(sorf_model([1, 6, 7, 8, 9], 128, 64, 64), coords, charges, False)
@@ -196,8 +233,10 @@ def main():
 
     # ---- CPU baseline first: its worker processes are forked before the GPU is initialised --
     cpu = None
+    cpu_c1 = None
     if not args.no_cpu_baseline:
         cores = min(os.cpu_count() or 1, 16)
+        cpu_c1 = cpu_config1(cores)
         c64 = [c.astype(np.float64) for c in coords[:args.cpu_sample]]
         cpu = cpu_baseline(c64, charges[:args.cpu_sample], (red, D, bias, alpha.astype(np.float32).astype(np.float64)),
                            args.cpu_sample, cores) + (cores,)
@@ -222,11 +261,19 @@ def main():
     R = rep.get_repsize()
 
     if args.calibration_copy:
-        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)      # 1 GiB
+        # a plain copy of known size (1 GiB read, 1 GiB written): the reference point for the
+        # FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this script
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
         for _ in range(3):
-            dst = src + 1.0
+            ops.check(ops._lib.lib().qmll_probe_copy(ops._ptr(src), ops._ptr(dst), src.numel(), ops._stream()), "copy")
         del src, dst
         torch.cuda.synchronize()
+    # ceilings measured on this very device (a few ms each), next to the nominal ones
+    from qml_lightning_amd.utils import peaks as peaks_mod
+    peaks = peaks_mod.measure()
+    peaks["nominal"] = dict(peaks_mod.NOMINAL)
+    torch.cuda.empty_cache()
 
     def step():
         return model.energies_and_forces(X, Z, aid, mid, nat)
@@ -272,8 +319,22 @@ def main():
         E2, F2 = step_autograd()
     torch.cuda.synchronize()
     ms_two_op = (time.perf_counter() - t0) / 5 * 1e3
+    # GPU time of the same step as the sum of its kernels' durations (one profiled step): what the
+    # route costs when the host keeps up; the difference to the wall time is host time
+    kernel_sum_ms = None
+    try:
+        from torch.profiler import ProfilerActivity, profile
+        with profile(activities=[ProfilerActivity.CUDA]) as prof:
+            step_autograd()
+            torch.cuda.synchronize()
+        kernel_sum_ms = sum(ev.self_device_time_total for ev in prof.key_averages()) / 1e3
+    except Exception as exc:      # the profiler is optional; the wall time stands on its own
+        kernel_sum_ms = None
+        print("bench.py: two-op kernel sum not measured: %r" % (exc,), file=sys.stderr)
     model.fused = True
     two_op_route = {"ms_per_step": ms_two_op, "molecules_per_s": B / ms_two_op * 1e3,
+                    "kernel_sum_ms": kernel_sum_ms,
+                    "gpu_share_of_wall": (kernel_sum_ms / ms_two_op) if kernel_sum_ms else None,
                     "max_abs_diff_energy": float((E2.detach() - E).abs().max()),
                     "max_abs_diff_force": float((F2 - Fr).abs().max()),
                     "hbm_bytes_per_step_algorithmic": float(A) * (20.0 * F + 8.0 * NPCAS)}
@@ -337,21 +398,24 @@ def main():
     norm = float(np.sqrt(NPCAS) / SIGMA)
     t_fused = 0.0
     t_sorf = t_cos = t_cosb = t_adj = 0.0
-    two_op_bytes = 0
+    big = {"atoms": 0}          # the launches of the element with the most atoms: what the profiler's per-launch bytes refer to
     for ei, e in enumerate(SPECIES):
         idx = model._element_index(data, data['charges'], e)
         sub = torch.matmul(flat_rep.index_select(0, idx), model.reductors[ei])
         Ae = sub.shape[0]
         # the reference's two-op contract, kernel by kernel (coefficients materialised)
         molidx = torch.div(idx, n, rounding_mode='floor').to(torch.int32)
-        t_sorf += timed(lambda: ops.sorf_forward(sub, model.Dmat[ei], norm, 1))
+        te_sorf = timed(lambda: ops.sorf_forward(sub, model.Dmat[ei], norm, 1))
         coeffs = ops.sorf_forward(sub, model.Dmat[ei], norm, 1).view(Ae, F)
-        t_cos += timed(lambda: ops.cos_features(coeffs, model.bias[ei], B, molidx))
+        te_cos = timed(lambda: ops.cos_features(coeffs, model.bias[ei], B, molidx))
         gZ = alpha32[None, :].expand(B, F).contiguous()
-        t_cosb += timed(lambda: ops.cos_features_backward(gZ, coeffs, model.bias[ei], B, molidx))
+        te_cosb = timed(lambda: ops.cos_features_backward(gZ, coeffs, model.bias[ei], B, molidx))
         gc = ops.cos_features_backward(gZ, coeffs, model.bias[ei], B, molidx).view(Ae, NSTACKS, NPCAS)
-        t_adj += timed(lambda: ops.sorf_adjoint(gc, model.Dmat[ei], norm, 1))
+        te_adj = timed(lambda: ops.sorf_adjoint(gc, model.Dmat[ei], norm, 1))
         del coeffs, gc
+        t_sorf, t_cos, t_cosb, t_adj = t_sorf + te_sorf, t_cos + te_cos, t_cosb + te_cosb, t_adj + te_adj
+        if Ae > big["atoms"]:
+            big = {"atoms": Ae, "element": int(e), "sorf": te_sorf, "cos": te_cos, "cosb": te_cosb, "adj": te_adj}
     d = NPCAS
     log2d = int(np.log2(d))
     # the predict step's own launches: sort by element, projection (and its transpose), fused kernel
@@ -385,10 +449,17 @@ def main():
                                     "valu_wave_instr_per_s": 23.5 * A * F / 64 / t_fused,
                                     "issue_model_clocks_per_coefficient": 80.0,
                                     "issue_bound_frac": 80.0 * A * F / 64 / simd_clocks / t_fused}
-    kernels["sorf_forward"] = {"seconds": t_sorf, "bound": "hbm", "GBs": A * (4 * d + 4 * F) / t_sorf / 1e9}
-    kernels["cos_features_f32"] = {"seconds": t_cos, "bound": "hbm", "GBs": (A * 4 * F + B * 4 * F) / t_cos / 1e9}
-    kernels["cos_features_backward"] = {"seconds": t_cosb, "bound": "hbm", "GBs": A * 8 * F / t_cosb / 1e9}
-    kernels["sorf_adjoint"] = {"seconds": t_adj, "bound": "hbm", "GBs": A * (4 * F + 4 * d) / t_adj / 1e9}
+    # the two-operator contract, kernel by kernel: `seconds` and the bytes are those of ONE launch, the
+    # element with the most atoms (the launch the profiler's per-dispatch counters describe);
+    # `seconds_all_elements` sums the launches of the three elements of one step
+    Ab = big["atoms"]
+    for key, tk, tall, nbytes in (("sorf_forward", "sorf", t_sorf, Ab * (4 * d + 4 * F)),
+                                  ("cos_features_f32", "cos", t_cos, Ab * 4 * F + B * 8 * F),
+                                  ("cos_features_backward", "cosb", t_cosb, Ab * 8 * F),
+                                  ("sorf_adjoint", "adj", t_adj, Ab * (4 * F + 4 * d))):
+        kernels[key] = {"seconds": big[tk], "bound": "hbm", "atoms": Ab, "element": big["element"],
+                        "algorithmic_bytes": float(nbytes), "GBs": nbytes / big[tk] / 1e9,
+                        "frac": nbytes / big[tk] / 1e9 / HBM_PEAK_GBS, "seconds_all_elements": tall}
 
     # ---- Z^T Z / Z^T y for 1000 molecules with forces --------------------------------------
     train = {}
@@ -445,10 +516,25 @@ def main():
         if k in traffic:
             kernels[k]["traffic_bytes"] = traffic[k]["read_bytes"] + traffic[k]["written_bytes"]
 
+    # every fraction against the ceiling measured on this device as well as the nominal one
+    exp_nominal = 256 * 4 * 16 * 2.4e9 / 4          # one v_exp_f32 per lane per 4 clocks on 16-lane SIMDs
+    for k, v in kernels.items():
+        if v["bound"] == "hbm" and "GBs" in v:
+            v["frac_of_measured"] = v["GBs"] / max(peaks["hbm_fill_GBs"], peaks["hbm_copy_GBs"])
+        elif v["bound"] == "mfma":
+            ref = peaks["mfma_f64_TFLOPs"] if k in ("gram_f64", "cholesky_solve_f64") else peaks["mfma_f32_TFLOPs"]
+            v["frac_of_measured"] = v["TFLOPs"] / ref
+        elif "exp_per_s" in v:
+            v["frac"] = v["exp_per_s"] / exp_nominal
+            v["frac_of_measured"] = v["exp_per_s"] / peaks["exp_per_s"]
+    kernels["sorf_energy_fused"]["frac"] = kernels["sorf_energy_fused"]["TFLOPs"] / FP32_PEAK_TFLOPS
+    kernels["sorf_energy_fused"]["sincos_frac_of_measured_exp_rate"] = (
+        2.0 * kernels["sorf_energy_fused"]["sincos_per_s"] / peaks["exp_per_s"])
     dominant = max(("fchl19_forward", "fchl19_vjp", "sorf_energy_fused"), key=lambda k: kernels[k]["seconds"])
     if dominant == "sorf_energy_fused":
         roofline = {"kernel": dominant, "bound": "valu", "achieved": kernels[dominant]["TFLOPs"],
                     "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": kernels[dominant]["TFLOPs"] / FP32_PEAK_TFLOPS,
+                    "issue_bound_frac": kernels[dominant]["issue_bound_frac"],
                     "traffic": kernels[dominant].get("traffic_bytes"),
                     "note": "fused FWHT+sincos kernel: neither HBM nor MFMA bounds it (8d bytes per atom, no "
                             "contraction); it is bound by vector instruction issue.  Algorithmic flops count one "
@@ -459,8 +545,8 @@ def main():
                             "traffic = bytes per launch from profiles/pmc_traffic.json"}
     else:
         roofline = {"kernel": dominant, "bound": "valu", "achieved": kernels[dominant]["exp_per_s"] / 1e12,
-                    "peak": 256 * 4 * 16 * 2.4e9 / 4 / 1e12, "unit": "Texp/s",
-                    "frac": kernels[dominant]["exp_per_s"] / (256 * 4 * 16 * 2.4e9 / 4), "traffic": None}
+                    "peak": exp_nominal / 1e12, "unit": "Texp/s", "frac": kernels[dominant]["exp_per_s"] / exp_nominal,
+                    "frac_of_measured": kernels[dominant]["frac_of_measured"], "traffic": None}
 
     out = {
         "metric": "molecules/s (FCHL19+SORF energy+force predict); Z^T Z build time, 16384 feats",
@@ -471,6 +557,7 @@ def main():
                                "nRs2 24 nRs3 20, SORF npcas 128 x nstacks 128 = 16384 features, energies + forces",
                    "molecules_per_step": B, "atoms_per_step": A},
         "roofline": roofline,
+        "peaks_measured": peaks,
         "autograd_route": autograd_route,
         "two_op_route": two_op_route,
         "from_host_arrays": from_host,
@@ -480,7 +567,8 @@ def main():
     if "gram_f64" in kernels:
         g = kernels["gram_f64"]
         out["roofline_ztz"] = {"kernel": "gram_f64", "bound": "mfma", "achieved": g["TFLOPs"], "peak": FP64_PEAK_TFLOPS,
-                               "unit": "TFLOP/s", "frac": g["frac"], "traffic": g.get("traffic_bytes")}
+                               "unit": "TFLOP/s", "frac": g["frac"], "frac_of_measured": g["frac_of_measured"],
+                               "peak_measured": peaks["mfma_f64_TFLOPs"], "traffic": g.get("traffic_bytes")}
     if not args.no_other_configs:
         torch.cuda.empty_cache()
         try:
@@ -488,6 +576,21 @@ def main():
         except Exception as exc:   # the headline line must survive a failure here
             out["other_configs"] = {"error": repr(exc)}
 
+    c1 = out.get("other_configs", {}).get("config1_c6h6_100")
+    E1 = c1.pop("_E", None) if isinstance(c1, dict) else None
+    F1 = c1.pop("_F", None) if isinstance(c1, dict) else None
+    if cpu_c1 is not None:
+        # configuration 1 is the CPU-reference configuration: the oracle on all of it, and the GPU
+        # result of the same 100 molecules checked against it
+        out["cpu_baseline_c1"] = {"value": 100.0 / cpu_c1["seconds"], "unit": "molecules/s", "cores": cpu_c1["cores"],
+                                  "kind": "port", "seconds": cpu_c1["seconds"],
+                                  "sample": "configuration 1 in full: 100 noisy C6H6 (12 atoms), species {1,6}, npcas 64 x "
+                                            "nstacks 8 = 512 features, energies + forces, fp64 NumPy oracle"}
+        if E1 is not None:
+            out["cpu_baseline_c1"]["gpu_molecules_per_s"] = c1["molecules_per_s"]
+            out["parity_vs_oracle_c1"] = {
+                "energy_rel_err": float(np.abs(E1 - cpu_c1["E"]).max() / np.abs(cpu_c1["E"]).max()),
+                "force_rel_err": float(np.abs(F1 - cpu_c1["F"]).max() / np.abs(cpu_c1["F"]).max()), "molecules": 100}
     if cpu is not None:
         rate, nsamp, secs, res, chunks, cores = cpu
         # the sample doubles as a parity check of this very run

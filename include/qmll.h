@@ -359,6 +359,22 @@ int qmll_gram_tile_f64(const double* Z, const double* y, int M, int F, int f0, i
  * K-sum carried in fp32 with Kahan compensation. */
 int qmll_matmul_and_reduce(const float* A, const float* B, int Ar, int K, int Bc, double* C, qmll_stream_t stream);
 
+/* ---- measured ceilings of the device (no counterpart in the reference; the benchmark divides
+ * each kernel's rate by these next to the nominal peaks) ------------------------------------- */
+
+/* dst[0..nfloats) = value with plain 16-byte stores; dst = src with plain 16-byte loads and stores
+ * (nfloats a multiple of 4, pointers 16-byte aligned).  The copy is also the known-size reference
+ * for scaling a profiler's FETCH_SIZE / WRITE_SIZE counters. */
+int qmll_probe_fill(float* dst, size_t nfloats, float value, qmll_stream_t stream);
+int qmll_probe_copy(const float* src, float* dst, size_t nfloats, qmll_stream_t stream);
+
+/* A loop of `iters` rounds of independent instructions on every SIMD of the chip: which = 0
+ * v_mfma_f64_16x16x4_f64, 1 v_mfma_f32_32x32x2_f32, 2 v_exp_f32.  out: device scratch of
+ * qmll_probe_out_bytes() bytes.  Returns the number of operations the launch performs (flop, or
+ * exponentials for which = 2), to be divided by the measured duration; negative on error. */
+size_t qmll_probe_out_bytes(void);
+double qmll_probe_rate(int which, int iters, void* out, qmll_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

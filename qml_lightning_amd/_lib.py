@@ -69,9 +69,13 @@ PROTOTYPES = {
     "qmll_cholesky_solve_f64": [P, c_int, c_longlong, P, P, P],
     "qmll_gram_tile_f64": [P, P, c_int, c_int, c_int, c_int, P, P, P],
     "qmll_matmul_and_reduce": [P, P, c_int, c_int, c_int, P, P],
+    "qmll_probe_fill": [P, c_size_t, c_float, P],
+    "qmll_probe_copy": [P, P, c_size_t, P],
+    "qmll_probe_out_bytes": [],
+    "qmll_probe_rate": [c_int, c_int, P, P],
 }
 _RESTYPES = {"qmll_last_error": c_char_p, "qmll_sort_by_type_workspace": c_size_t,
-             "qmll_cholesky_workspace_bytes": c_size_t}
+             "qmll_cholesky_workspace_bytes": c_size_t, "qmll_probe_out_bytes": c_size_t, "qmll_probe_rate": c_double}
 
 _lib = None
 

@@ -11,7 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libqmll.so")
 TORCH_LIB = os.path.join(HERE, "libqmll_torch.so")
-SOURCES = ["qmll_core.cpp", "neighbours.hip", "fchl19.hip", "sorf.hip", "project.hip", "rff.hip", "gram.hip", "solve.hip"]
+SOURCES = ["qmll_core.cpp", "neighbours.hip", "fchl19.hip", "sorf.hip", "project.hip", "rff.hip", "gram.hip", "solve.hip", "probe.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-munsafe-fp-atomics",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-value"]

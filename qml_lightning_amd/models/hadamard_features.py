@@ -399,20 +399,29 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
                                                                          self.ntransforms, nslots, x.requires_grad)
             return e_slots.view(X.shape[0], X.shape[1]).sum(dim=1)
 
-        Ztest = torch.zeros(X.shape[0], self.nfeatures(), device=X.device, dtype=torch.float32)
+        # The reference's operator sequence (hadamard_features.py:99-121) with nothing but its own
+        # operators and plain torch, so a file saved from here loads wherever the reference's
+        # libraries are.  Each element's atoms are looked up ONCE (one host round trip for the
+        # count) and gathered with index_select, whose backward is an index_add: the boolean-mask
+        # forms `rep[Z == e]` and `where(Z == e)` of the reference each search again, forward and
+        # backward (nine round trips per step for three elements instead of three).
+        nmol, natoms_max = torch_rep.shape[0], torch_rep.shape[1]      # [1, n] for one unbatched molecule
+        Ztest = torch.zeros(nmol, self.nfeatures(), device=X.device, dtype=torch.float32)
+        flat_rep = torch_rep.view(nmol * natoms_max, torch_rep.shape[2])
+        flat_charges = Z.int().view(-1)
         for e in self.elements:
-            indexes = Z.int() == e.item()
             element_idx = self.element2index[e]
-            batch_indexes = torch.where(indexes)[0].type(torch.int)
-            sub = torch_rep[indexes]
-            if sub.shape[0] == 0:
+            atom_rows = torch.nonzero(flat_charges == e.item())[:, 0]      # ascending: molecule-major
+            if atom_rows.shape[0] == 0:
                 continue
+            batch_indexes = torch.div(atom_rows, natoms_max, rounding_mode='floor').type(torch.int)
+            sub = flat_rep.index_select(0, atom_rows)
             sub = project_representation(sub, self.reductors[element_idx])
             coeffs = torch.ops.qml_lightning_sorf.get_SORF_coefficients(sub, self.Dmat[element_idx],
                                                                         coeff_normalisation, self.ntransforms)
             coeffs = coeffs.view(coeffs.shape[0], coeffs.shape[1] * coeffs.shape[2])
             features = torch.ops.qml_lightning_sorf.get_cos_features(coeffs, self.bias[element_idx],
-                                                                     torch.tensor(X.shape[0]), batch_indexes)
+                                                                     torch.tensor(nmol), batch_indexes)
             Ztest = Ztest + features
         return torch.matmul(Ztest, alpha)
 

@@ -80,14 +80,14 @@ class BaseKernel():
         raise NotImplementedError("Abstract method only.")
 
     # -- rows of one batch ----------------------------------------------------------------
-    def _batch_rows(self, data, with_forces, zero_energy_rows=False):
-        """fp64 row matrix [B (+ B*n*3), F] of one formatted batch: B energy rows, then the
-        B*n*3 force rows in (molecule, atom, xyz) order (kernel.py:134-170)."""
+    def _batch_projected(self, data, with_forces):
+        """Everything of a formatted batch that does not depend on sigma: per element the projected
+        representation rows [A_e, npcas] (and projected Jacobian rows [A_e, n, 3, npcas]) with the
+        molecule index of each row (kernel.py:141-160 up to the call of calculate_features)."""
         coordinates, charges = data['coordinates'], data['charges']
         atomIDs, molIDs, natom_counts = data['atomIDs'], data['molIDs'], data['natom_counts']
         cells, inv_cells = data['cells'], data['inv_cells']
         B, n = charges.shape
-        F = self.nfeatures()
         if with_forces:
             representation, rep_derivative = self.rep.get_representation_and_derivative(
                 coordinates, charges, atomIDs, molIDs, natom_counts, cells, inv_cells)
@@ -95,18 +95,9 @@ class BaseKernel():
             representation = self.rep.get_representation(coordinates, charges, atomIDs, molIDs, natom_counts, cells,
                                                          inv_cells)
             rep_derivative = None
-        nrows = B + (B * n * 3 if with_forces else 0)
-        own_force_rows = with_forces and self.writes_force_rows()
-        if own_force_rows:
-            rows = torch.empty(nrows, F, device=coordinates.device, dtype=torch.float64)
-            rows[:B].zero_()
-        else:
-            rows = torch.zeros(nrows, F, device=coordinates.device, dtype=torch.float64)
-        Zenergy = rows[:B]
-        G = rows[B:].view(B, n, 3, F) if with_forces else None
         flat_rep = representation.view(B * n, -1)
         flat_jac = rep_derivative.view(B * n, n, 3, -1) if with_forces else None
-        self._queue_force_rows = own_force_rows     # calculate_features may queue; finish_features runs the queue
+        items = []
         for e in self.elements:
             idx = self._element_index(data, charges, int(e))
             if idx.shape[0] == 0:
@@ -117,12 +108,35 @@ class BaseKernel():
             sub_grad = None
             if with_forces:
                 sub_grad = project_derivative(flat_jac.index_select(0, idx), self.reductors[element_idx])
-            self.calculate_features(sub, e, batch_indexes, Zenergy, sub_grad, G)
+            items.append((e, batch_indexes, sub, sub_grad))
+        return {'B': B, 'n': n, 'device': coordinates.device, 'items': items}
+
+    def _rows_from_projected(self, proj, with_forces, zero_energy_rows=False):
+        """fp64 row matrix [B (+ B*n*3), F] from the projected rows of one batch, at the current
+        sigma: B energy rows, then the B*n*3 force rows in (molecule, atom, xyz) order
+        (kernel.py:134-170)."""
+        B, n, F = proj['B'], proj['n'], self.nfeatures()
+        nrows = B + (B * n * 3 if with_forces else 0)
+        own_force_rows = with_forces and self.writes_force_rows()
+        if own_force_rows:
+            rows = torch.empty(nrows, F, device=proj['device'], dtype=torch.float64)
+            rows[:B].zero_()
+        else:
+            rows = torch.zeros(nrows, F, device=proj['device'], dtype=torch.float64)
+        Zenergy = rows[:B]
+        G = rows[B:].view(B, n, 3, F) if with_forces else None
+        self._queue_force_rows = own_force_rows     # calculate_features may queue; finish_features runs the queue
+        for e, batch_indexes, sub, sub_grad in proj['items']:
+            self.calculate_features(sub, e, batch_indexes, Zenergy, sub_grad if with_forces else None, G)
         self._queue_force_rows = False
         self.finish_features(G, overwrite=own_force_rows)
         if zero_energy_rows:
             Zenergy.fill_(0)        # energy rows stay, as zeros, so the row count is unchanged (kernel.py:164-165)
         return rows
+
+    def _batch_rows(self, data, with_forces, zero_energy_rows=False):
+        """Rows of one formatted batch: representation (+ Jacobian), projection, features."""
+        return self._rows_from_projected(self._batch_projected(data, with_forces), with_forces, zero_energy_rows)
 
     @staticmethod
     def _element_index(data, charges, e):
@@ -264,20 +278,34 @@ class BaseKernel():
         pick = lambda seq, ids: [seq[z] for z in ids]
         err = torch.sqrt if use_rmse else (lambda v: v)
         red = (lambda d: torch.mean(d * d)) if use_rmse else (lambda d: torch.mean(torch.abs(d)))
-        for sigma in sigmas:
-            # Z^T Z and Z^T y do not depend on lambda: one build per (sigma, fold) serves the
-            # whole lambda row of the grid (the reference rebuilds them for every grid point)
-            fold_errors = np.zeros(len(lambdas))
-            for train_index, test_index in kf.split(X):
+        # sigma enters through the coefficient normalisation alone (hadamard_features.py:68,93), so
+        # per fold the representation, its Jacobian and the projected rows are built ONCE and kept;
+        # per sigma only the features and Z^T Z / Z^T y are redone, and those serve the whole lambda
+        # row (the reference rebuilds everything for every grid point).  For the RFF model W is drawn
+        # with the sigma of construction (random_features.py:54): assigning self.sigma here does not
+        # change it, as in the reference; call sample_elemental_basis() per sigma for a real scan.
+        nf = self.nfeatures()
+        fold_errors = np.zeros((len(sigmas), len(lambdas)))
+        for train_index, test_index in kf.split(X):
+            Xtr, Qtr, Etr = pick(X, train_index), pick(Q, train_index), pick(E, train_index)
+            Ftr = pick(F, train_index) if F is not None else None
+            cached = self._projected_batches(Xtr, Qtr, Etr, Ftr, cells, inv_cells)
+            Xt, Qt = pick(X, test_index), pick(Q, test_index)
+            data = self.format_data(Xt, Qt, pick(E, test_index), pick(F, test_index) if F is not None else None,
+                                    cells=cells, inv_cells=inv_cells)
+            max_natoms = int(data['natom_counts'].max().item())
+            for si, sigma in enumerate(sigmas):
                 self.sigma = sigma
-                ZTZ, ZtrainY = self.build_Z_components(pick(X, train_index), pick(Q, train_index),
-                                                       pick(E, train_index),
-                                                       pick(F, train_index) if F is not None else None, cells,
-                                                       inv_cells, print_info=False)
-                Xt, Qt = pick(X, test_index), pick(Q, test_index)
-                data = self.format_data(Xt, Qt, pick(E, test_index), pick(F, test_index) if F is not None else None,
-                                        cells=cells, inv_cells=inv_cells)
-                max_natoms = int(data['natom_counts'].max().item())
+                if cached is None:          # the projected rows of this fold would not fit the cache budget
+                    ZTZ, ZtrainY = self.build_Z_components(Xtr, Qtr, Etr, Ftr, cells, inv_cells, print_info=False)
+                else:
+                    ZTZ = torch.zeros(nf, nf, device=self.device, dtype=torch.float64)
+                    ZtrainY = torch.zeros(nf, 1, device=self.device, dtype=torch.float64)
+                    for proj, targets in cached:
+                        rows = self._rows_from_projected(proj, F is not None)
+                        ops.gram(rows, targets, ZTZ, ZtrainY, mirror=False)
+                        del rows
+                    ops.gram_mirror(ZTZ)
                 diag = ZTZ.diagonal().clone()
                 for li, llambda in enumerate(lambdas):
                     self.llambda = llambda
@@ -289,13 +317,16 @@ class BaseKernel():
                                               print_info=False)
                         e_err = err(red(ep - data['energies']))
                         f_err = err(red(fp - data['forces']))
-                        fold_errors[li] += 0.5 * float(e_err + f_err)
+                        fold_errors[si, li] += 0.5 * float(e_err + f_err)
                     else:
                         ep = self.predict(Xt, Qt, max_natoms, cells=cells, inv_cells=inv_cells, forces=False,
                                           print_info=False)
-                        fold_errors[li] += float(err(red(ep - data['energies'])))
+                        fold_errors[si, li] += float(err(red(ep - data['energies'])))
+                del ZTZ, ZtrainY
+            del cached
+        for si, sigma in enumerate(sigmas):
             for li, llambda in enumerate(lambdas):
-                fold_error = fold_errors[li] / kfolds
+                fold_error = fold_errors[si, li] / kfolds
                 if print_info:
                     print("sigma", sigma, "lambda", llambda, "error", fold_error)
                 if fold_error < best[2]:
@@ -303,6 +334,28 @@ class BaseKernel():
         if print_info:
             print("Best error: ", best[2], "sigma = ", best[0], "lambda = ", best[1])
         return best[0], best[1]
+
+    #: bytes of projected rows (all training batches of one fold) the grid search keeps on the device
+    grid_search_cache_bytes = 64 << 30
+
+    def _projected_batches(self, X, Q, E, F, cells, inv_cells):
+        """[(projected rows, targets)] of every training batch, or None when they would take more
+        than `grid_search_cache_bytes` (per atom: npcas floats, times 1 + 3 n with forces)."""
+        nmax = max((len(q) for q in Q), default=0)
+        natoms = sum(len(q) for q in Q)
+        need = 4 * self.npcas * natoms * (1 + (3 * nmax if F is not None else 0))
+        if need > self.grid_search_cache_bytes:
+            return None
+        out = []
+        for i in range(0, len(X), self.nbatch_train):
+            sl = slice(i, i + self.nbatch_train)
+            data = self.format_data(X[sl], Q[sl], E=E[sl] if E is not None else None,
+                                    F=F[sl] if F is not None else None,
+                                    cells=cells[sl] if cells is not None else None,
+                                    inv_cells=inv_cells[sl] if cells is not None else None)
+            targets = self._targets(data, data['charges'].shape[0], E is not None, F is not None)
+            out.append((self._batch_projected(data, F is not None), targets))
+        return out
 
     #: atoms the fused predict route aims to put into one launch chain (see _fused_batch)
     fused_batch_atoms = 131072

@@ -95,14 +95,19 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
             e_slots, _ = torch.ops.qml_lightning_sorf.rff_energy_sorted(x, type_offsets, sorted_slots, self.W, self.b,
                                                                         self.alpha.float(), nslots, x.requires_grad)
             return e_slots.view(X.shape[0], X.shape[1]).sum(dim=1)
-        Ztest = torch.zeros(X.shape[0], self.nfeatures(), device=X.device, dtype=torch.float32)
+        # the reference's sequence (random_features.py:86-102); each element's atoms are looked up
+        # once and gathered with index_select (backward: index_add, no second search)
+        nmol, natoms_max = torch_rep.shape[0], torch_rep.shape[1]      # [1, n] for one unbatched molecule
+        Ztest = torch.zeros(nmol, self.nfeatures(), device=X.device, dtype=torch.float32)
+        flat_rep = torch_rep.view(nmol * natoms_max, torch_rep.shape[2])
+        flat_charges = Z.int().view(-1)
         for e in self.elements:
-            indexes = Z.int() == e.item()
             element_idx = self.element2index[e]
-            batch_indexes = torch.where(indexes)[0]
-            sub = torch_rep[indexes]
-            if sub.shape[0] == 0:
+            atom_rows = torch.nonzero(flat_charges == e.item())[:, 0]
+            if atom_rows.shape[0] == 0:
                 continue
+            batch_indexes = torch.div(atom_rows, natoms_max, rounding_mode='floor')
+            sub = flat_rep.index_select(0, atom_rows)
             sub = project_representation(sub, self.reductors[element_idx])
             feats = self.feature_normalisation * torch.cos(torch.matmul(sub, self.W[element_idx])
                                                            + self.b[element_idx][None, :])

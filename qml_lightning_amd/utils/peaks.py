@@ -1,0 +1,53 @@
+"""Measured ceilings of the GPU the library runs on, next to the nominal ones: fill and copy
+bandwidth, fp64 / fp32 matrix-core rate, transcendental rate.  Each probe is a few milliseconds
+of the library's own probe kernels, timed with HIP events on the current stream."""
+import ctypes
+
+import torch
+
+from .. import _lib
+from ..ops import _ptr, _stream
+
+NOMINAL = {"hbm_GBs": 8000.0, "mfma_f64_TFLOPs": 78.6, "mfma_f32_TFLOPs": 157.3}
+
+
+def _timed(fn, iters):
+    fn()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / iters * 1e-3
+
+
+def measure(nbytes=1 << 30, device="cuda:0"):
+    """{'hbm_fill_GBs', 'hbm_copy_GBs' (bytes read + written), 'mfma_f64_TFLOPs',
+    'mfma_f32_TFLOPs', 'exp_per_s'} of the current device."""
+    L = _lib.lib()
+    n = nbytes // 4
+    src = torch.empty(n, dtype=torch.float32, device=device)
+    dst = torch.empty(n, dtype=torch.float32, device=device)
+
+    def fill():
+        _lib.check(L.qmll_probe_fill(_ptr(src), n, 1.0, _stream()), "qmll_probe_fill")
+
+    def copy():
+        _lib.check(L.qmll_probe_copy(_ptr(src), _ptr(dst), n, _stream()), "qmll_probe_copy")
+
+    out = {"hbm_fill_GBs": nbytes / _timed(fill, 10) / 1e9, "hbm_copy_GBs": 2.0 * nbytes / _timed(copy, 10) / 1e9}
+    del src, dst
+    scratch = torch.empty(int(L.qmll_probe_out_bytes()) // 8, dtype=torch.float64, device=device)
+    for key, which, iters, scale in (("mfma_f64_TFLOPs", 0, 4000, 1e12), ("mfma_f32_TFLOPs", 1, 4000, 1e12),
+                                     ("exp_per_s", 2, 4000, 1.0)):
+        ops = [0.0]
+
+        def run():
+            ops[0] = float(L.qmll_probe_rate(which, iters, _ptr(scratch), _stream()))
+            if ops[0] < 0:
+                _lib.check(-1, "qmll_probe_rate")
+        t = _timed(run, 3)
+        out[key] = ops[0] / t / scale
+    return out

@@ -353,16 +353,20 @@ def test_reductor_fit_matches_an_svd_of_the_samples():
 
 
 def test_grid_search_shares_the_gram_matrix_across_lambdas():
-    """hyperparam_opt_nested_cv (kernel.py:249-347) builds Z^T Z once per (sigma, fold); every grid
-    point must score exactly as a fresh train() + predict() at that point does."""
+    """hyperparam_opt_nested_cv (kernel.py:249-347) builds the representation, its Jacobian and the
+    projected rows once per fold, the features and Z^T Z once per (sigma, fold); every grid point
+    must score exactly as a fresh train() + predict() at that point does."""
     species = [1, 6]
     coords, charges = helpers.benzene_batch(8, 3)
     c32 = [np.asarray(c, dtype=np.float32) for c in coords]
     rng = np.random.default_rng(21)
     E = rng.normal(size=8)
     Fo = [rng.normal(size=(12, 3)) for _ in range(8)]
-    sigmas, lambdas, kfolds = [2.0, 3.0], [1e-3, 1e-1], 2
+    sigmas, lambdas, kfolds = [2.0, 3.0, 4.5], [1e-3, 1e-1], 2
     m, _ = build_sorf_model(species, 16, 4)
+    jacobian_calls = []
+    real_jacobian = m.rep.get_representation_and_derivative
+    m.rep.get_representation_and_derivative = lambda *a, **k: (jacobian_calls.append(1), real_jacobian(*a, **k))[1]
     printed = []
     import builtins
     real_print = builtins.print
@@ -372,6 +376,9 @@ def test_grid_search_shares_the_gram_matrix_across_lambdas():
     finally:
         builtins.print = real_print
     got = {(a[1], a[3]): a[5] for a in printed if a and a[0] == "sigma"}
+    # 4 training molecules per fold = one batch of nbatch_train = 4: one Jacobian launch per fold,
+    # whatever the number of sigmas and lambdas
+    assert len(jacobian_calls) == kfolds
     from sklearn.model_selection import KFold
     expect = {}
     for sg in sigmas:
@@ -391,6 +398,19 @@ def test_grid_search_shares_the_gram_matrix_across_lambdas():
     for k in expect:      # two builds of Z^T Z differ in summation order; the solve amplifies that
         assert abs(got[k] - expect[k]) <= 1e-6 * max(1.0, abs(expect[k])), (k, got[k], expect[k])
     assert best == min(expect, key=expect.get)
+    # without room for the cache the search falls back to one full build per (sigma, fold): same scores
+    m3, _ = build_sorf_model(species, 16, 4)
+    m3.grid_search_cache_bytes = 0
+    printed.clear()
+    builtins.print = lambda *a, **k: printed.append(a)
+    try:
+        best3 = m3.hyperparam_opt_nested_cv(c32, charges, E, Fo, sigmas=sigmas, lambdas=lambdas, kfolds=kfolds)
+    finally:
+        builtins.print = real_print
+    got3 = {(a[1], a[3]): a[5] for a in printed if a and a[0] == "sigma"}
+    for k in expect:
+        assert abs(got3[k] - expect[k]) <= 1e-6 * max(1.0, abs(expect[k])), (k, got3[k], expect[k])
+    assert best3 == best
 
 
 def test_rff_model_vs_oracle():

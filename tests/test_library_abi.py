@@ -14,7 +14,7 @@ def declared():
     h = open(os.path.join(ROOT, "include", "qmll.h")).read()
     h = re.sub(r"/\*.*?\*/", "", h, flags=re.S)
     out = {}
-    for m in re.finditer(r"^(?:int|size_t|const char\*)\s+(qmll_\w+)\s*\(([^;]*?)\)\s*;", h, re.M | re.S):
+    for m in re.finditer(r"^(?:int|size_t|double|const char\*)\s+(qmll_\w+)\s*\(([^;]*?)\)\s*;", h, re.M | re.S):
         args = m.group(2).strip()
         out[m.group(1)] = 0 if args in ("", "void") else len(args.split(","))
     return out
