@@ -517,7 +517,7 @@ def main():
             kernels[k]["traffic_bytes"] = traffic[k]["read_bytes"] + traffic[k]["written_bytes"]
 
     # every fraction against the ceiling measured on this device as well as the nominal one
-    exp_nominal = 256 * 4 * 16 * 2.4e9 / 4          # one v_exp_f32 per lane per 4 clocks on 16-lane SIMDs
+    exp_nominal = 1024 * 64 / 8.0 * 2.4e9           # 1024 SIMDs, one 64-lane v_exp_f32 per 8 clocks (a quarter of the plain fp32 rate)
     for k, v in kernels.items():
         if v["bound"] == "hbm" and "GBs" in v:
             v["frac_of_measured"] = v["GBs"] / max(peaks["hbm_fill_GBs"], peaks["hbm_copy_GBs"])

@@ -369,11 +369,12 @@ int qmll_probe_fill(float* dst, size_t nfloats, float value, qmll_stream_t strea
 int qmll_probe_copy(const float* src, float* dst, size_t nfloats, qmll_stream_t stream);
 
 /* A loop of `iters` rounds of independent instructions on every SIMD of the chip: which = 0
- * v_mfma_f64_16x16x4_f64, 1 v_mfma_f32_32x32x2_f32, 2 v_exp_f32.  out: device scratch of
+ * v_mfma_f64_16x16x4_f64, 1 v_mfma_f32_32x32x2_f32, 2 v_exp_f32; blocks_per_cu (1..16) workgroups
+ * of four wavefronts per compute unit, i.e. that many wavefronts per SIMD.  out: device scratch of
  * qmll_probe_out_bytes() bytes.  Returns the number of operations the launch performs (flop, or
  * exponentials for which = 2), to be divided by the measured duration; negative on error. */
 size_t qmll_probe_out_bytes(void);
-double qmll_probe_rate(int which, int iters, void* out, qmll_stream_t stream);
+double qmll_probe_rate(int which, int iters, int blocks_per_cu, void* out, qmll_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -12,28 +12,63 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 
 constexpr int PT = 256;
 
-__global__ __launch_bounds__(PT) void probe_fill_kernel(float4* __restrict__ dst, size_t n4, float v) {
-    const float4 val = make_float4(v, v, v, v);
-    for (size_t i = (size_t)blockIdx.x * PT + threadIdx.x; i < n4; i += (size_t)gridDim.x * PT) dst[i] = val;
-}
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+constexpr int UNR = 4;   // 16-byte accesses in flight per thread: a workgroup moves 16 KB
 
-__global__ __launch_bounds__(PT) void probe_copy_kernel(const float4* __restrict__ src, float4* __restrict__ dst,
-                                                         size_t n4) {
-    for (size_t i = (size_t)blockIdx.x * PT + threadIdx.x; i < n4; i += (size_t)gridDim.x * PT) dst[i] = src[i];
-}
-
-// four independent accumulator tiles per wavefront, so the matrix pipe never waits for a result
-__global__ __launch_bounds__(PT) void probe_mfma_f64_kernel(int iters, double* __restrict__ out) {
-    const double a = 1e-3 * (double)(threadIdx.x & 7), b = 1e-3 * (double)(threadIdx.x & 3);
-    double4_t c0 = {0, 0, 0, 0}, c1 = c0, c2 = c0, c3 = c0;
-    for (int it = 0; it < iters; ++it) {
-        c0 = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c0, 0, 0, 0);
-        c1 = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c1, 0, 0, 0);
-        c2 = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c2, 0, 0, 0);
-        c3 = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c3, 0, 0, 0);
+// streaming kernels: every thread issues UNR independent 16-byte accesses (consecutive threads
+// touch consecutive 16 bytes), with the nontemporal hint the library's own streaming kernels use
+__global__ __launch_bounds__(PT) void probe_fill_kernel(floatx4* __restrict__ dst, size_t n4, float v) {
+    const floatx4 val = {v, v, v, v};
+    const size_t base = (size_t)blockIdx.x * (PT * UNR) + threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+        const size_t i = base + (size_t)u * PT;
+        if (i < n4) __builtin_nontemporal_store(val, dst + i);
     }
-    const double4_t s = c0 + c1 + c2 + c3;
-    out[(size_t)blockIdx.x * PT + threadIdx.x] = s[0] + s[1] + s[2] + s[3];
+}
+
+__global__ __launch_bounds__(PT) void probe_copy_kernel(const floatx4* __restrict__ src, floatx4* __restrict__ dst,
+                                                         size_t n4) {
+    const size_t base = (size_t)blockIdx.x * (PT * UNR) + threadIdx.x;
+    floatx4 v[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+        const size_t i = base + (size_t)u * PT;
+        if (i < n4) v[u] = __builtin_nontemporal_load(src + i);
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+        const size_t i = base + (size_t)u * PT;
+        if (i < n4) __builtin_nontemporal_store(v[u], dst + i);
+    }
+}
+
+// sixteen independent accumulator tiles per wavefront fed from four A and four B fragments, the
+// shape of a 64 x 64 sub-tile of a matrix product: the matrix pipe never waits for a result
+__global__ __launch_bounds__(PT, 2) void probe_mfma_f64_kernel(int iters, double* __restrict__ out) {
+    double fa[4], fb[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        fa[p] = 1e-3 * (double)((threadIdx.x & 7) + p + 1);
+        fb[p] = 1e-3 * (double)((threadIdx.x & 3) + 2 * p + 1);
+    }
+    double4_t acc[4][4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[p][q] = (double4_t){0, 0, 0, 0};
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[p][q] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[p], fb[q], acc[p][q], 0, 0, 0);
+    }
+    double s = 0.0;
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) s += acc[p][q][0] + acc[p][q][1] + acc[p][q][2] + acc[p][q][3];
+    out[(size_t)blockIdx.x * PT + threadIdx.x] = s;
 }
 
 __global__ __launch_bounds__(PT) void probe_mfma_f32_kernel(int iters, float* __restrict__ out) {
@@ -68,7 +103,8 @@ __global__ __launch_bounds__(PT) void probe_exp_kernel(int iters, float* __restr
     out[(size_t)blockIdx.x * PT + threadIdx.x] = s;
 }
 
-constexpr int PROBE_BLOCKS = 256 * 16;   // 16 workgroups of 4 wavefronts per CU: 16 wavefronts per SIMD queued, 8 resident
+constexpr int PROBE_CUS = 256;
+constexpr int PROBE_MAX_BLOCKS_PER_CU = 16;
 
 }  // namespace
 
@@ -76,8 +112,9 @@ extern "C" int qmll_probe_fill(float* dst, size_t nfloats, float value, qmll_str
     QMLL_REQUIRE(dst && nfloats % 4 == 0 && ((uintptr_t)dst & 15) == 0, QMLL_ERR_INVALID,
                  "qmll_probe_fill: needs a 16-byte aligned buffer of a multiple of 4 floats");
     if (nfloats == 0) return QMLL_OK;
-    hipLaunchKernelGGL(probe_fill_kernel, dim3(256 * 32), dim3(PT), 0, (hipStream_t)stream, reinterpret_cast<float4*>(dst),
-                       nfloats / 4, value);
+    const size_t n4 = nfloats / 4;
+    hipLaunchKernelGGL(probe_fill_kernel, dim3((unsigned)((n4 + PT * UNR - 1) / (PT * UNR))), dim3(PT), 0, (hipStream_t)stream,
+                       reinterpret_cast<floatx4*>(dst), n4, value);
     QMLL_CHECK_LAUNCH("qmll_probe_fill");
     return QMLL_OK;
 }
@@ -86,26 +123,30 @@ extern "C" int qmll_probe_copy(const float* src, float* dst, size_t nfloats, qml
     QMLL_REQUIRE(src && dst && nfloats % 4 == 0 && (((uintptr_t)dst | (uintptr_t)src) & 15) == 0, QMLL_ERR_INVALID,
                  "qmll_probe_copy: needs 16-byte aligned buffers of a multiple of 4 floats");
     if (nfloats == 0) return QMLL_OK;
-    hipLaunchKernelGGL(probe_copy_kernel, dim3(256 * 32), dim3(PT), 0, (hipStream_t)stream,
-                       reinterpret_cast<const float4*>(src), reinterpret_cast<float4*>(dst), nfloats / 4);
+    const size_t n4 = nfloats / 4;
+    hipLaunchKernelGGL(probe_copy_kernel, dim3((unsigned)((n4 + PT * UNR - 1) / (PT * UNR))), dim3(PT), 0, (hipStream_t)stream,
+                       reinterpret_cast<const floatx4*>(src), reinterpret_cast<floatx4*>(dst), n4);
     QMLL_CHECK_LAUNCH("qmll_probe_copy");
     return QMLL_OK;
 }
 
-extern "C" size_t qmll_probe_out_bytes(void) { return (size_t)PROBE_BLOCKS * PT * sizeof(double); }
+extern "C" size_t qmll_probe_out_bytes(void) {
+    return (size_t)PROBE_CUS * PROBE_MAX_BLOCKS_PER_CU * PT * sizeof(double);
+}
 
-extern "C" double qmll_probe_rate(int which, int iters, void* out, qmll_stream_t stream) {
+extern "C" double qmll_probe_rate(int which, int iters, int blocks_per_cu, void* out, qmll_stream_t stream) {
     // returns the number of operations the launch performs (flop for the matrix loops,
     // exponentials for which = 2); negative on error
-    if (!out || iters <= 0) {
-        qmll_set_error("qmll_probe_rate: null output or no iterations");
+    if (!out || iters <= 0 || blocks_per_cu < 1 || blocks_per_cu > PROBE_MAX_BLOCKS_PER_CU) {
+        qmll_set_error("qmll_probe_rate: null output, no iterations, or blocks_per_cu outside 1..%d", PROBE_MAX_BLOCKS_PER_CU);
         return -1.0;
     }
+    const int PROBE_BLOCKS = PROBE_CUS * blocks_per_cu;
     const double waves = (double)PROBE_BLOCKS * (PT / 64);
     double ops;
     if (which == 0) {
         hipLaunchKernelGGL(probe_mfma_f64_kernel, dim3(PROBE_BLOCKS), dim3(PT), 0, (hipStream_t)stream, iters, (double*)out);
-        ops = waves * iters * 4.0 * (2.0 * 16 * 16 * 4);
+        ops = waves * iters * 16.0 * (2.0 * 16 * 16 * 4);
     } else if (which == 1) {
         hipLaunchKernelGGL(probe_mfma_f32_kernel, dim3(PROBE_BLOCKS), dim3(PT), 0, (hipStream_t)stream, iters, (float*)out);
         ops = waves * iters * 4.0 * (2.0 * 32 * 32 * 2);
