@@ -73,9 +73,11 @@ PROTOTYPES = {
     "qmll_probe_copy": [P, P, c_size_t, P],
     "qmll_probe_out_bytes": [],
     "qmll_probe_rate": [c_int, c_int, c_int, P, P],
+    "qmll_probe_mix": [c_int, c_int, c_int, P, P],
 }
 _RESTYPES = {"qmll_last_error": c_char_p, "qmll_sort_by_type_workspace": c_size_t,
-             "qmll_cholesky_workspace_bytes": c_size_t, "qmll_probe_out_bytes": c_size_t, "qmll_probe_rate": c_double}
+             "qmll_cholesky_workspace_bytes": c_size_t, "qmll_probe_out_bytes": c_size_t, "qmll_probe_rate": c_double,
+             "qmll_probe_mix": c_double}
 
 _lib = None
 

@@ -103,6 +103,85 @@ __global__ __launch_bounds__(PT) void probe_exp_kernel(int iters, float* __restr
     out[(size_t)blockIdx.x * PT + threadIdx.x] = s;
 }
 
+// ---- instruction mixes -------------------------------------------------------------------
+// Straight-line loops of the instruction classes the fused SORF kernel issues, alone and mixed,
+// on independent registers: what a wavefront instruction of each class costs a SIMD, and how far
+// the matrix pipe runs beside the vector pipe.  One iteration of a mix stands for one stack of
+// one wavefront of that kernel at 128 components (8 registers per lane, four atoms per wavefront):
+//   MIX_FUSED      108 plain fp32 + 64 DPP fmac + 16 transcendental (the kernel as it is)
+//   MIX_MFMA_TRIAL 124 plain fp32 + 16 transcendental + 16 v_mfma_f32_16x16x4_f32: the in-row stages
+//                  (a 16-point +-1 Hadamard block per 16 lanes, forward and adjoint, 2 x 2 tiles x K = 16)
+//                  on the matrix pipe, 16 plain instructions for the operand layout, no data movement
+enum { MIX_PLAIN = 0, MIX_DPP = 1, MIX_TRANS = 2, MIX_MFMA16 = 3, MIX_FUSED = 4, MIX_MFMA_TRIAL = 5, MIX_COUNT = 6 };
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+template <int N>
+__device__ __forceinline__ void plain_ops(float (&v)[8], float c) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) v[k & 7] = fmaf(v[k & 7], c, 0.25f);
+}
+template <int N>
+__device__ __forceinline__ void dpp_ops(float (&v)[8], float c) {
+#pragma unroll
+    for (int k = 0; k < N; ++k)
+        asm volatile("v_fmac_f32_dpp %0, %0, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf" : "+v"(v[k & 7]) : "v"(c));
+}
+template <int N>
+__device__ __forceinline__ void trans_ops(float (&v)[8]) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) v[k & 7] = __builtin_amdgcn_sinf(v[k & 7]);
+}
+template <int N>
+__device__ __forceinline__ void mfma_ops(float4_t (&acc)[4], float a, float b) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) acc[k & 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[k & 3], 0, 0, 0);
+}
+
+template <int MIX>
+__global__ __launch_bounds__(PT) void probe_mix_kernel(int iters, float* __restrict__ out) {
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = 0.001f * (float)((threadIdx.x & 31) + k);
+    const float c = (threadIdx.x & 1) ? -0.5f : 0.5f;
+    float4_t acc[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    const float a = 1e-3f * (float)(threadIdx.x & 7), b = (threadIdx.x & 2) ? 1.0f : -1.0f;
+    for (int it = 0; it < iters; ++it) {
+        if constexpr (MIX == MIX_PLAIN) plain_ops<128>(v, c);
+        if constexpr (MIX == MIX_DPP) dpp_ops<128>(v, c);
+        if constexpr (MIX == MIX_TRANS) trans_ops<128>(v);
+        if constexpr (MIX == MIX_MFMA16) mfma_ops<32>(acc, a, b);
+        if constexpr (MIX == MIX_FUSED) {
+            // forward: sign multiply + register stages, in-row stages, argument, sincos, products;
+            // adjoint: register stages, in-row stages, accumulate
+            plain_ops<32>(v, c);
+            dpp_ops<32>(v, c);
+            plain_ops<22>(v, c);
+            trans_ops<16>(v);
+            plain_ops<22>(v, c);
+            dpp_ops<32>(v, c);
+            plain_ops<32>(v, c);
+        }
+        if constexpr (MIX == MIX_MFMA_TRIAL) {
+            plain_ops<40>(v, c);
+            mfma_ops<8>(acc, a, b);
+            plain_ops<22>(v, c);
+            trans_ops<16>(v);
+            plain_ops<22>(v, c);
+            mfma_ops<8>(acc, a, b);
+            plain_ops<40>(v, c);
+        }
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) s += v[k];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) s += acc[k][0] + acc[k][1] + acc[k][2] + acc[k][3];
+    out[(size_t)blockIdx.x * PT + threadIdx.x] = s;
+}
+
 constexpr int PROBE_CUS = 256;
 constexpr int PROBE_MAX_BLOCKS_PER_CU = 16;
 
@@ -162,4 +241,30 @@ extern "C" double qmll_probe_rate(int which, int iters, int blocks_per_cu, void*
         return -1.0;
     }
     return ops;
+}
+
+extern "C" double qmll_probe_mix(int mix, int iters, int blocks_per_cu, void* out, qmll_stream_t stream) {
+    // returns the number of wavefront-iterations per SIMD the launch performs (wavefronts per SIMD
+    // x iters): duration x clock / that = SIMD clocks per iteration of the mix; negative on error
+    if (!out || iters <= 0 || blocks_per_cu < 1 || blocks_per_cu > PROBE_MAX_BLOCKS_PER_CU || mix < 0 || mix >= MIX_COUNT) {
+        qmll_set_error("qmll_probe_mix: mix outside 0..%d, null output, no iterations, or blocks_per_cu outside 1..%d",
+                       MIX_COUNT - 1, PROBE_MAX_BLOCKS_PER_CU);
+        return -1.0;
+    }
+    const dim3 grid(PROBE_CUS * blocks_per_cu), block(PT);
+    float* o = (float*)out;
+    hipStream_t st = (hipStream_t)stream;
+    switch (mix) {
+        case MIX_PLAIN: hipLaunchKernelGGL(probe_mix_kernel<MIX_PLAIN>, grid, block, 0, st, iters, o); break;
+        case MIX_DPP: hipLaunchKernelGGL(probe_mix_kernel<MIX_DPP>, grid, block, 0, st, iters, o); break;
+        case MIX_TRANS: hipLaunchKernelGGL(probe_mix_kernel<MIX_TRANS>, grid, block, 0, st, iters, o); break;
+        case MIX_MFMA16: hipLaunchKernelGGL(probe_mix_kernel<MIX_MFMA16>, grid, block, 0, st, iters, o); break;
+        case MIX_FUSED: hipLaunchKernelGGL(probe_mix_kernel<MIX_FUSED>, grid, block, 0, st, iters, o); break;
+        default: hipLaunchKernelGGL(probe_mix_kernel<MIX_MFMA_TRIAL>, grid, block, 0, st, iters, o); break;
+    }
+    if (hipGetLastError() != hipSuccess) {
+        qmll_set_error("qmll_probe_mix: launch failed");
+        return -1.0;
+    }
+    return (double)blocks_per_cu * iters;
 }

@@ -618,6 +618,100 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
     }
     float energy = 0.0f;
 
+    if constexpr (!MULTI) {
+        // One transform per stack.  The coefficients are carried in REVOLUTIONS: x is scaled by
+        // scale / 2 pi once per atom, so the argument of v_sin_f32 / v_cos_f32 is a single fma per
+        // coefficient.  The network leaves sigma * (H v) in a lane (sigma = the lane's pending
+        // sign); instead of multiplying it out, the lane works with u' = sigma * u:
+        //     u' = (H v)_computed + (sigma / 2 pi) * bias,   cos(u') = cos(u),  sin(u') = sigma sin(u).
+        // The gradient entering the adjoint transform is then sigma * g.  The transposed network
+        // (the same stages with the stage constants negated: (I + diag(c) P)^T = I - diag(c) P,
+        // because the partner lane has the opposite stage bit) computes H (sigma * in), i.e. H g
+        // itself, with no sign left pending.
+        constexpr float INV2PI = 0.15915494309189535f;
+        const float xs = scale * INV2PI;
+        const float csig = sigma * INV2PI;
+        const float ncs[4] = {-cs[0], -cs[1], -cs[2], -cs[3]};
+#pragma unroll
+        for (int p = 0; p < EPL; ++p) xv[p] *= xs;
+        // v_sin_f32 / v_cos_f32 reduce the range themselves up to 256 revolutions.  The rounding of
+        // the argument, |arg| * 6e-8 radians, is the size of the rounding of an fp32 argument in
+        // radians; measured against fp64 the energies and gradients are as close as with an exact
+        // Cody-Waite reduction in front (5e-7 at |arg| ~ 16, 2e-6 at ~100).  Beyond 1500 radians the
+        // whole revolutions are taken off first: u - rint(u) is exact in fp32.
+        constexpr float UMAX = 1500.0f * INV2PI;
+        auto stack = [&](const float (&dcur)[EPL], const float (&bv)[EPL], const float (&av)[EPL]) {
+            float v[EPL];
+#pragma unroll
+            for (int p = 0; p < EPL; ++p) v[p] = xv[p] * dcur[p];
+            register_stages<EPL>(v);
+            row_stages<EPL>(v, cs);
+            float u[EPL], umax = 0.0f;
+#pragma unroll
+            for (int p = 0; p < EPL; ++p) {
+                u[p] = fmaf(bv[p], csig, v[p]);
+                umax = fmaxf(umax, fabsf(u[p]));
+            }
+#pragma unroll
+            for (int p = 0; p < EPL; ++p) {
+                const float sn = __builtin_amdgcn_sinf(u[p]), cs_ = __builtin_amdgcn_cosf(u[p]);
+                energy = fmaf(av[p], cs_, energy);
+                v[p] = av[p] * sn;                           // sigma * (-(d E / d coefficient) / normf)
+            }
+            if (__builtin_expect(__any(umax > UMAX), 0)) {
+#pragma unroll
+                for (int p = 0; p < EPL; ++p) {
+                    if (fabsf(u[p]) > UMAX) {
+                        const float c0_ = __builtin_amdgcn_cosf(u[p]);
+                        const float ur = u[p] - rintf(u[p]);
+                        const float sn = __builtin_amdgcn_sinf(ur), cs_ = __builtin_amdgcn_cosf(ur);
+                        energy += av[p] * (cs_ - c0_);
+                        v[p] = av[p] * sn;
+                    }
+                }
+            }
+            if constexpr (WITH_GRAD) {
+                register_stages<EPL>(v);
+                row_stages<EPL>(v, ncs);
+#pragma unroll
+                for (int p = 0; p < EPL; ++p) acc[p] = fmaf(v[p], dcur[p], acc[p]);
+            }
+        };
+        // two stacks per round with the sign diagonals in two register sets that swap roles: the
+        // diagonal of a stack is fetched one stack ahead (it is the first thing a stack needs),
+        // bias and alpha at the start of their own stack (needed after the transform)
+        float d0[EPL], d1[EPL];
+        int s = wave;
+        if (s < S) load_row<EPL>(d0, D + (size_t)s * d + e0);
+        while (s < S) {
+            {
+                float bv[EPL], av[EPL];
+                const size_t off = (size_t)s * d + e0;               // the same for the four rows
+                load_row<EPL>(bv, bias + off);
+                load_row<EPL>(av, alpha + off);
+                load_row<EPL>(d1, D + (size_t)(s + SORF_WAVES < S ? s + SORF_WAVES : s) * d + e0);
+                stack(d0, bv, av);
+            }
+            s += SORF_WAVES;
+            if (s >= S) break;
+            {
+                float bv[EPL], av[EPL];
+                const size_t off = (size_t)s * d + e0;
+                load_row<EPL>(bv, bias + off);
+                load_row<EPL>(av, alpha + off);
+                load_row<EPL>(d0, D + (size_t)(s + SORF_WAVES < S ? s + SORF_WAVES : s) * d + e0);
+                stack(d1, bv, av);
+            }
+            s += SORF_WAVES;
+        }
+        energy = row_sum(energy);
+        if (i16 == 0) ered[wave][row] = energy;
+        if constexpr (WITH_GRAD) {
+            // no sign is pending, and the scaling of x does not enter d E / d coefficient
+#pragma unroll
+            for (int p = 0; p < EPL; ++p) red[wave][row][(p >> 2) * 64 + e0 + (p & 3)] = acc[p];
+        }
+    } else {
     // per stack: the sign diagonal is fetched one stack ahead (it is the first thing a stack
     // needs), bias and alpha at the start of their own stack (needed after the transform)
     float dv[EPL], bv[EPL], av[EPL];
@@ -635,15 +729,13 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
         for (int p = 0; p < EPL; ++p) v[p] = xv[p] * dv[p];
         register_stages<EPL>(v);
         row_stages<EPL>(v, cs);
-        if constexpr (MULTI) {
-            for (int m = 1; m < T; ++m) {
-                float dm[EPL];
-                load_row<EPL>(dm, D + ((size_t)m * S + s) * d + e0);
+        for (int m = 1; m < T; ++m) {
+            float dm[EPL];
+            load_row<EPL>(dm, D + ((size_t)m * S + s) * d + e0);
 #pragma unroll
-                for (int p = 0; p < EPL; ++p) v[p] *= dm[p] * sigma;
-                register_stages<EPL>(v);
-                row_stages<EPL>(v, cs);
-            }
+            for (int p = 0; p < EPL; ++p) v[p] *= dm[p] * sigma;
+            register_stages<EPL>(v);
+            row_stages<EPL>(v, cs);
         }
 
         float arg[EPL], amax = 0.0f;
@@ -652,11 +744,7 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
             arg[p] = fmaf(v[p], scale_l, bv[p]);
             amax = fmaxf(amax, fabsf(arg[p]));
         }
-        // v_sin_f32 / v_cos_f32 take revolutions and reduce the range themselves up to 256
-        // revolutions: arg / 2 pi goes in directly.  Its rounding, |arg| * 6e-8 radians, is the
-        // size of the rounding of the fp32 argument itself; measured against fp64 the energies
-        // and gradients are as close as with an exact Cody-Waite reduction in front (5e-7 at
-        // |arg| ~ 16, 2e-6 at ~100), for five instructions less per coefficient.
+        // arg / 2 pi goes to the transcendental unit directly (see the one-transform branch)
 #pragma unroll
         for (int p = 0; p < EPL; ++p) {
             const float u = arg[p] * 0.15915494309189535f;
@@ -681,15 +769,13 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
         if constexpr (WITH_GRAD) {
             register_stages<EPL>(v);
             row_stages<EPL>(v, cs);
-            if constexpr (MULTI) {
-                for (int m = T - 1; m >= 1; --m) {
-                    float dm[EPL];
-                    load_row<EPL>(dm, D + ((size_t)m * S + s) * d + e0);
+            for (int m = T - 1; m >= 1; --m) {
+                float dm[EPL];
+                load_row<EPL>(dm, D + ((size_t)m * S + s) * d + e0);
 #pragma unroll
-                    for (int p = 0; p < EPL; ++p) v[p] *= dm[p] * sigma;
-                    register_stages<EPL>(v);
-                    row_stages<EPL>(v, cs);
-                }
+                for (int p = 0; p < EPL; ++p) v[p] *= dm[p] * sigma;
+                register_stages<EPL>(v);
+                row_stages<EPL>(v, cs);
             }
 #pragma unroll
             for (int p = 0; p < EPL; ++p) acc[p] = fmaf(v[p], dv[p], acc[p]);
@@ -702,6 +788,7 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
     if constexpr (WITH_GRAD) {
 #pragma unroll
         for (int p = 0; p < EPL; ++p) red[wave][row][(p >> 2) * 64 + e0 + (p & 3)] = acc[p] * sigma;
+    }
     }
     __syncthreads();
     if (threadIdx.x < rows) {

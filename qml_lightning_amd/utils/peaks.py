@@ -57,3 +57,28 @@ def measure(nbytes=1 << 30, device="cuda:0"):
             out.setdefault(key + "_by_wavefronts_per_simd", {})[str(per_cu)] = ops[0] / t / scale
         out[key] = best
     return out
+
+
+MIXES = ("plain_fp32_x128", "dpp_fmac_x128", "transcendental_x128", "mfma_f32_16x16x4_x32", "fused_kernel_stack",
+         "fused_kernel_stack_mfma_trial")
+
+
+def instruction_mixes(device="cuda:0", iters=2000):
+    """Seconds per wavefront-iteration per SIMD of each instruction mix of the library's probe
+    (see qmll_probe_mix), at 1, 2, 4 and 8 wavefronts per SIMD: {'name': {'1': s, ...}}.  Times a
+    clock frequency these are SIMD clocks per iteration; the ratios between mixes need no clock."""
+    L = _lib.lib()
+    scratch = torch.empty(int(L.qmll_probe_out_bytes()) // 8, dtype=torch.float64, device=device)
+    out = {}
+    for mix, name in enumerate(MIXES):
+        out[name] = {}
+        for per_cu in (1, 2, 4, 8):
+            units = [0.0]
+
+            def run():
+                units[0] = float(L.qmll_probe_mix(mix, iters, per_cu, _ptr(scratch), _stream()))
+                if units[0] < 0:
+                    _lib.check(-1, "qmll_probe_mix")
+            t = _timed(run, 2)
+            out[name][str(per_cu)] = t / units[0]
+    return out

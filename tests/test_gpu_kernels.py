@@ -353,6 +353,52 @@ def test_fused_energy_matches_two_op_chain(d, S, T):
     close(e2, e_ref, REL_EF, "fused energy only")
 
 
+@pytest.mark.parametrize("d", [64, 128, 256])
+def test_fused_energy_large_arguments(d):
+    """Arguments of hundreds to tens of thousands of radians (beyond the range the sine / cosine
+    unit reduces itself).  A one-hot input makes the transform exact in fp32 (every coefficient is
+    +-x_k times the scale), so the fp32 argument the kernel forms is known: one rounding of
+    x * (scale / 2 pi), one fused multiply-add with the bias, in revolutions.  Energies and
+    gradients must match the fp64 cosine / sine of exactly that argument."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(d)
+    S = 5
+    F = S * d
+    norm = np.float32(8.0)
+    # the kernel's scale is normalisation * 2^(-log2(d) / 2) in fp32 (the transform itself is unnormalised)
+    scale = np.float32(norm * np.float32(2.0 ** (-0.5 * np.log2(d))))
+    mags = (np.array([0.1, 8.0, 56.0, 320.0, 1280.0, 7200.0, 36000.0]) / scale).astype(np.float32)   # coefficients in radians
+    A = len(mags)
+    hot = rng.integers(0, d, A)
+    x = np.zeros((A, d), dtype=np.float32)
+    x[np.arange(A), hot] = mags * np.where(rng.uniform(size=A) > 0.5, 1, -1)
+    D = np.where(rng.uniform(-1, 1, (1, S, d)) > 0, 1.0, -1.0).astype(np.float32)
+    b = rng.uniform(0, 2 * np.pi, F).astype(np.float32)
+    alpha = rng.normal(size=F).astype(np.float32)
+    inv2pi = np.float32(0.15915494309189535)
+    xs = np.float32(scale * inv2pi)
+    from scipy.linalg import hadamard
+    H = hadamard(d).astype(np.float64)
+    u = np.zeros((A, F))
+    for a_ in range(A):
+        w32 = np.float32(x[a_, hot[a_]] * xs)                                    # one rounding
+        for s_ in range(S):
+            w = H[:, hot[a_]] * float(D[0, s_, hot[a_]]) * float(w32)            # exact: +-w32
+            u[a_, s_ * d:(s_ + 1) * d] = (w + b[s_ * d:(s_ + 1) * d].astype(np.float64) * float(inv2pi)).astype(np.float32)
+    arg = 2.0 * np.pi * u
+    assert np.abs(arg).max() > 32000 and (np.abs(arg).max(axis=1) < 7.0).any()
+    nf = np.sqrt(2.0 / F)
+    e_ref = (nf * np.cos(arg) * alpha).sum(1)
+    gc = -nf * np.sin(arg) * alpha
+    gx_ref = sorf.sorf_adjoint(gc.reshape(A, S, d), D, float(norm))
+    e = torch.zeros(A, device=dev())
+    gx = ops.sorf_energy_fused(t32(x), t32(D), t32(b), t32(alpha), None, float(norm), 1, e)
+    e_scale = nf * np.abs(alpha).sum()                 # what the per-atom sums are made of
+    assert np.abs(e.double().cpu().numpy() - e_ref).max() <= 2e-6 * e_scale
+    for a_ in range(A):                                # per atom: the gradient scales differ by orders of magnitude
+        close(gx[a_], gx_ref[a_], REL_EF, "fused gradient, |arg| up to %.0f" % np.abs(arg[a_]).max())
+
+
 def test_typed_fused_energy_matches_per_element_calls():
     """All elements in one launch == one fused call per element (slots, padded rows, unknown types)."""
     from qml_lightning_amd import ops
