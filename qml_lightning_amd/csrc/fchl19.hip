@@ -271,6 +271,22 @@ __device__ __forceinline__ void unrank_pair(int t, int nn, int& j, int& k) {
     k = jj + 1 + (t - (jj * (2 * nn - jj - 1)) / 2);
 }
 
+// pair t of the list of pairs (j<k) enumerated k-major: t = k (k - 1) / 2 + j, 0 <= j < k.  No
+// search: k = floor((1 + sqrt(8 t + 1)) / 2) from the 1-ulp square root, put right by one
+// comparison either way; all quantities are integers below 2^24, exact in fp32 (t < 2^20).
+__device__ __forceinline__ void unrank_pair_kmajor(int t, int& j, int& k) {
+    const float tf = (float)t;
+    float kf = floorf(0.5f + 0.5f * fsqrt(fmaf(8.0f, tf, 1.0f)));
+    float tri = 0.5f * fmaf(kf, kf, -kf);                 // k (k - 1) / 2
+    kf -= tri > tf ? 1.0f : 0.0f;
+    tri = 0.5f * fmaf(kf, kf, -kf);
+    const float up = tri + kf <= tf ? 1.0f : 0.0f;        // (k + 1) k / 2 <= t
+    tri += up * kf;
+    kf += up;
+    k = (int)kf;
+    j = (int)(tf - tri);
+}
+
 __device__ __forceinline__ int pair_offset(int ej, int ek, int ns, int nRs2, int nRs3) {
     const int p = ej < ek ? ej : ek;
     const int q = ej < ek ? ek : ej;
@@ -336,10 +352,10 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
 
     float* trip = smem;             // [tcap][4]: sk3 rho, K cos, K sin, -   (first: 16-byte aligned)
     Stage s = carve(smem + 4 * (a.tcap + a.tpad), a.cap, ns);
-    float* smu = s.next;            // [cap]  mu_j
-    float* sis2 = smu + a.cap;      // [cap]  log2(e) / (2 sigma_j^2)
-    float* spre = sis2 + a.cap;     // [cap]  r^-d2 fc / (sigma sqrt(2pi))
-    float* slnRs2 = spre + a.cap;   // [nRs2]
+    // [cap][4] per neighbour: mu_j, log2(e) / (2 sigma_j^2), r^-d2 fc / (sigma sqrt(2pi)), -
+    // (16-byte aligned: one LDS read per neighbour in the two-body loop)
+    float* s2b = s.next + ((4 - ((size_t)(s.next - smem) & 3)) & 3);
+    float* slnRs2 = s2b + 4 * a.cap;   // [nRs2]
     float* sinvRs2 = slnRs2 + nRs2; // [nRs2]
     float* sRs3 = sinvRs2 + nRs2;   // [nRs3]
     int* pbase = (int*)(sRs3 + nRs3);   // [ns*ns] first table entry of each element pair
@@ -370,9 +386,10 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     for (int j = lane; j < nn; j += QMLL_WAVE) {
         const float r = s.r[j];
         const float s2 = flog(1.0f + a.p.eta2 * frcp(r * r));
-        smu[j] = flog(r) - 0.5f * s2;                    // ln(r / sqrt(1 + eta2/r^2))
-        sis2[j] = 0.5f * LOG2E * frcp(s2);
-        spre[j] = rsqrtf(s2) * 0.3989422804014327f * fexp2(-a.p.two_body_decay * flog2(r)) * s.fc[j];
+        reinterpret_cast<float4*>(s2b)[j] = make_float4(
+            flog(r) - 0.5f * s2,                         // ln(r / sqrt(1 + eta2/r^2))
+            0.5f * LOG2E * frcp(s2),
+            rsqrtf(s2) * 0.3989422804014327f * fexp2(-a.p.two_body_decay * flog2(r)) * s.fc[j], 0.0f);
     }
     __syncthreads();
 
@@ -389,13 +406,20 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
             const float lnRs = zok ? slnRs2[z] : 0.0f;
             const float invRs = zok ? sinvRs2[z] : 0.0f;
             for (int e = 0; e < ns; ++e) {
+                // the same number of rounds for every lane (the loop stays scalar and unrolls);
+                // a sub-slot past the end of the type's neighbours reads a valid entry with weight 0
+                const int j0 = s.goff[e], j1 = s.goff[e + 1];
+                const int rounds = idiv_small(j1 - j0 + JS - 1, JS);
                 float acc = 0.0f;
-                if (zok) {
-                    for (int j = s.goff[e] + jsub; j < s.goff[e + 1]; j += JS) {
-                        const float u = lnRs - smu[j];
-                        acc = fmaf(spre[j] * invRs, fexp2(-u * u * sis2[j]), acc);
-                    }
+#pragma unroll 2
+                for (int it = 0; it < rounds; ++it) {
+                    const int j = j0 + jsub + it * JS;
+                    const bool jok = zok && j < j1;
+                    const float4 f = reinterpret_cast<const float4*>(s2b)[jok ? j : j0];
+                    const float u = lnRs - f.x;
+                    acc = fmaf(jok ? f.z : 0.0f, fexp2(-u * u * f.y), acc);
                 }
+                acc *= invRs;
                 float tot = acc;
                 for (int k = 1; k < JS; ++k) tot += __shfl(acc, zl + W * k, 64);
                 if (zok && jsub == 0) out[e * nRs2 + z] = tot;
@@ -484,11 +508,11 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
         __syncthreads();
         for (int tt = lane; tt < ntrip; tt += QMLL_WAVE) {
             int j, k;
-            unrank_pair(tt, nn, j, k);
+            unrank_pair_kmajor(tt, j, k);
             const int p = s.el[j], q = s.el[k];           // p <= q: the list is sorted by type
             const int jl = j - s.goff[p], kl = k - s.goff[q];
-            const int np_ = s.goff[p + 1] - s.goff[p], nq = s.goff[q + 1] - s.goff[q];
-            const int local = (p == q) ? (jl * (2 * np_ - jl - 1)) / 2 + (kl - jl - 1) : jl * nq + kl;
+            // any one-to-one numbering of a pair's triples does: k-major within one type, row by row else
+            const int local = (p == q) ? (kl * (kl - 1)) / 2 + jl : kl * (s.goff[p + 1] - s.goff[p]) + jl;
             *reinterpret_cast<float4*>(trip + (pbase[p * ns + q] + local) * 4) = table_entry(j, k);
         }
         __syncthreads();
@@ -706,7 +730,7 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
     const float zeta2 = 0.014383766711652736f;   // 2 exp(-pi^2 / 2)
     for (int tt = lane; tt < ntrip; tt += QMLL_WAVE) {
         int j, k;
-        unrank_pair(tt, nn, j, k);
+        unrank_pair_kmajor(tt, j, k);                     // tt = k (k - 1) / 2 + j
         const Triple t = triple_geometry(s, j, k);
         const TripleDeriv d = triple_derivatives(t, a.p, s.fc[j], s.dfc[j], s.fc[k], s.dfc[k]);
         const float* g = gin + pair_offset(s.el[j], s.el[k], ns, nRs2, nRs3);
@@ -766,20 +790,21 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
         atomicAdd(&gm[i * 3 + 2], giz);
     }
     if constexpr (TABLE) {
-        // lane = (neighbour x, component c): triples (x,k) are the run starting at off(x),
-        // triples (j,x) sit at off(j) + x - j - 1, with off(j) = j (2 nn - j - 1) / 2
+        // lane = (neighbour x, component c).  Triple (j,k) sits at k (k - 1) / 2 + j: the triples
+        // (j,x) with x second are the run of x entries starting at x (x - 1) / 2; the triples (x,k)
+        // with x first sit at k (k - 1) / 2 + x for k = x+1 .. nn-1, k entries further each step
         for (int it = lane; it < 3 * nn; it += QMLL_WAVE) {
-            const int x = it / 3, c = it - 3 * x;
+            const int x = idiv_small(it, 3), c = it - 3 * x;
             float sum = c == 0 ? sgx[x] : (c == 1 ? sgy[x] : sgz[x]);
-            const float* tj = tab + c * ntrip + (x * (2 * nn - x - 1)) / 2;
+            const float* tk = tab + (3 + c) * ntrip + (x * (x - 1)) / 2;
 #pragma unroll 4
-            for (int q = 0; q < nn - 1 - x; ++q) sum += tj[q];
-            const float* tk = tab + (3 + c) * ntrip + x - 1;
-            int idx = 0;                                   // off(j) - j, which grows by nn - j - 2 per step
+            for (int q = 0; q < x; ++q) sum += tk[q];
+            const float* tj = tab + c * ntrip + x;
+            int idx = ((x + 1) * x) / 2;
 #pragma unroll 4
-            for (int j = 0; j < x; ++j) {
-                sum += tk[idx];
-                idx += nn - j - 2;
+            for (int k = x + 1; k < nn; ++k) {
+                sum += tj[idx];
+                idx += k;
             }
             atomicAdd(&gm[s.j[x] * 3 + c], sum);
         }
@@ -1138,7 +1163,9 @@ extern "C" int qmll_fchl19_forward(const float* X, const int* types, const float
     // each of the ns (ns+1)/2 segments is padded to a multiple of the triple sub-slot count
     const int tsub_slots = prm->nRs3 < 64 ? 64 / prm->nRs3 : 1;
     a.tpad = prm->nspecies * (prm->nspecies + 1) / 2 * (tsub_slots - 1);
-    const size_t lds = sizeof(float) * ((size_t)(STAGE_ARRAYS + 3) * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 +
+    // triple table, neighbour arrays + type offsets, per-neighbour two-body factors [cap][4] (behind up
+    // to 3 floats of alignment), the radial grids, the table's segment starts
+    const size_t lds = sizeof(float) * ((size_t)(STAGE_ARRAYS + 4) * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 +
                                         4 * (size_t)(a.tcap + a.tpad) + (size_t)prm->nspecies * prm->nspecies + 4);
     QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
                  "qmll_fchl19_forward: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R, LDS_LIMIT);
