@@ -273,6 +273,20 @@ def main():
     from qml_lightning_amd.utils import peaks as peaks_mod
     peaks = peaks_mod.measure()
     peaks["nominal"] = dict(peaks_mod.NOMINAL)
+    # what a wavefront instruction of each class costs a SIMD, and the per-stack instruction mix of the
+    # fused SORF kernel next to the same mix with its in-row butterfly stages on the matrix pipe
+    mixes = peaks_mod.instruction_mixes()
+    best = {k: min(v.values()) for k, v in mixes.items()}
+    instruction_mixes = {
+        "ns_per_wavefront_iteration_per_simd": {k: {w: t * 1e9 for w, t in v.items()} for k, v in mixes.items()},
+        "ns_per_instruction": {"plain_fp32": best["plain_fp32_x128"] / 128 * 1e9, "dpp_fmac": best["dpp_fmac_x128"] / 128 * 1e9,
+                               "transcendental": best["transcendental_x128"] / 128 * 1e9,
+                               "mfma_f32_16x16x4": best["mfma_f32_16x16x4_x32"] / 32 * 1e9},
+        "fused_kernel_stack_ns": best["fused_kernel_stack"] * 1e9,
+        "fused_kernel_stack_mfma_trial_ns": best["fused_kernel_stack_mfma_trial"] * 1e9,
+        "note": "one iteration of fused_kernel_stack = 92 plain + 64 DPP + 16 transcendental wavefront instructions = one "
+                "stack of four atoms at 128 components; the trial replaces the 64 DPP by 16 v_mfma_f32_16x16x4_f32 + 16 plain",
+    }
     torch.cuda.empty_cache()
 
     def step():
@@ -440,15 +454,11 @@ def main():
     # fused kernel, algorithmic flops per atom: forward+adjoint butterflies 2*F*log2(d), D multiplies 2F,
     # scale+bias FMA 2F, one sin and one cos per feature 2F, energy FMA 2F, alpha*norm*sin 2F
     fused_flops = A * F * (2 * log2d + 10)
-    # 23.5 vector instructions per coefficient in the kernel's main loop (d = 128; counted in its ISA):
-    # 13.5 plain fp32 (measured issue cost 2.3 clocks each), 8 DPP butterflies (4.1 clocks) and
-    # v_sin_f32 + v_cos_f32 (8.1 clocks each) = 80 SIMD clocks per wavefront-coefficient
-    simd_clocks = 1024 * 2.4e9
+    # 172 vector instructions per wavefront and stack in the kernel's main loop at d = 128 (8 coefficients
+    # per lane; counted in its ISA): 92 plain fp32, 64 DPP butterflies, 8 v_sin_f32 + 8 v_cos_f32
     kernels["sorf_energy_fused"] = {"seconds": t_fused, "bound": "valu", "TFLOPs": fused_flops / t_fused / 1e12,
                                     "sincos_per_s": A * F / t_fused,
-                                    "valu_wave_instr_per_s": 23.5 * A * F / 64 / t_fused,
-                                    "issue_model_clocks_per_coefficient": 80.0,
-                                    "issue_bound_frac": 80.0 * A * F / 64 / simd_clocks / t_fused}
+                                    "valu_wave_instr_per_s": 172.0 / 8.0 * A * F / 64 / t_fused}
     # the two-operator contract, kernel by kernel: `seconds` and the bytes are those of ONE launch, the
     # element with the most atoms (the launch the profiler's per-dispatch counters describe);
     # `seconds_all_elements` sums the launches of the three elements of one step
@@ -528,20 +538,28 @@ def main():
             v["frac"] = v["exp_per_s"] / exp_nominal
             v["frac_of_measured"] = v["exp_per_s"] / peaks["exp_per_s"]
     kernels["sorf_energy_fused"]["frac"] = kernels["sorf_energy_fused"]["TFLOPs"] / FP32_PEAK_TFLOPS
+    # a wavefront of the fused kernel carries four atoms through one stack per iteration: its time per
+    # wavefront-stack per SIMD against the bare instruction mix of such an iteration (probe kernel)
+    wave_stacks_per_simd = (A / 4.0) * NSTACKS / 1024.0
+    kernels["sorf_energy_fused"]["ns_per_wavefront_stack_per_simd"] = t_fused / wave_stacks_per_simd * 1e9
+    kernels["sorf_energy_fused"]["instruction_mix_ns"] = instruction_mixes["fused_kernel_stack_ns"]
+    kernels["sorf_energy_fused"]["frac_of_instruction_mix"] = (
+        instruction_mixes["fused_kernel_stack_ns"] / kernels["sorf_energy_fused"]["ns_per_wavefront_stack_per_simd"])
     kernels["sorf_energy_fused"]["sincos_frac_of_measured_exp_rate"] = (
         2.0 * kernels["sorf_energy_fused"]["sincos_per_s"] / peaks["exp_per_s"])
     dominant = max(("fchl19_forward", "fchl19_vjp", "sorf_energy_fused"), key=lambda k: kernels[k]["seconds"])
     if dominant == "sorf_energy_fused":
         roofline = {"kernel": dominant, "bound": "valu", "achieved": kernels[dominant]["TFLOPs"],
                     "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": kernels[dominant]["TFLOPs"] / FP32_PEAK_TFLOPS,
-                    "issue_bound_frac": kernels[dominant]["issue_bound_frac"],
+                    "frac_of_instruction_mix": kernels[dominant]["frac_of_instruction_mix"],
                     "traffic": kernels[dominant].get("traffic_bytes"),
                     "note": "fused FWHT+sincos kernel: neither HBM nor MFMA bounds it (8d bytes per atom, no "
                             "contraction); it is bound by vector instruction issue.  Algorithmic flops count one "
                             "flop per sin and per cos and per butterfly add, while a butterfly across lanes issues "
                             "at half rate and v_sin/v_cos at quarter rate, none of them an FMA, so the fraction of "
-                            "the fp32 FMA peak understates it: kernels.sorf_energy_fused.issue_bound_frac is the "
-                            "kernel's instruction mix priced at the measured issue costs, over the launch time; "
+                            "the fp32 FMA peak understates it: frac_of_instruction_mix is the time a probe kernel needs for the "
+                            "bare instruction mix of one wavefront-stack (92 plain + 64 DPP + 16 transcendental, independent "
+                            "registers, no memory access) over the kernel's own time per wavefront-stack, both measured in this run; "
                             "traffic = bytes per launch from profiles/pmc_traffic.json"}
     else:
         roofline = {"kernel": dominant, "bound": "valu", "achieved": kernels[dominant]["exp_per_s"] / 1e12,
@@ -558,6 +576,7 @@ def main():
                    "molecules_per_step": B, "atoms_per_step": A},
         "roofline": roofline,
         "peaks_measured": peaks,
+        "instruction_mixes": instruction_mixes,
         "autograd_route": autograd_route,
         "two_op_route": two_op_route,
         "from_host_arrays": from_host,

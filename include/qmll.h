@@ -378,7 +378,7 @@ double qmll_probe_rate(int which, int iters, int blocks_per_cu, void* out, qmll_
 
 /* Straight-line loops of the instruction classes the fused SORF kernel issues, on independent
  * registers: mix = 0 128 plain fp32, 1 128 DPP fmac, 2 128 v_sin_f32, 3 32 v_mfma_f32_16x16x4_f32,
- * 4 the per-stack mix of the fused kernel at 128 components (108 plain + 64 DPP + 16
+ * 4 the per-stack mix of the fused kernel at 128 components (92 plain + 64 DPP + 16
  * transcendental), 5 the same with the in-row stages as 16 matrix instructions and 16 more plain
  * ones instead of the 64 DPP.  Returns wavefront-iterations per SIMD (blocks_per_cu x iters), so
  * duration x clock / that = SIMD clocks per iteration; negative on error. */

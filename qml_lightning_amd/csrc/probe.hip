@@ -108,8 +108,8 @@ __global__ __launch_bounds__(PT) void probe_exp_kernel(int iters, float* __restr
 // on independent registers: what a wavefront instruction of each class costs a SIMD, and how far
 // the matrix pipe runs beside the vector pipe.  One iteration of a mix stands for one stack of
 // one wavefront of that kernel at 128 components (8 registers per lane, four atoms per wavefront):
-//   MIX_FUSED      108 plain fp32 + 64 DPP fmac + 16 transcendental (the kernel as it is)
-//   MIX_MFMA_TRIAL 124 plain fp32 + 16 transcendental + 16 v_mfma_f32_16x16x4_f32: the in-row stages
+//   MIX_FUSED      92 plain fp32 + 64 DPP fmac + 16 transcendental (the kernel as it is, counted in its ISA)
+//   MIX_MFMA_TRIAL 108 plain fp32 + 16 transcendental + 16 v_mfma_f32_16x16x4_f32: the in-row stages
 //                  (a 16-point +-1 Hadamard block per 16 lanes, forward and adjoint, 2 x 2 tiles x K = 16)
 //                  on the matrix pipe, 16 plain instructions for the operand layout, no data movement
 enum { MIX_PLAIN = 0, MIX_DPP = 1, MIX_TRANS = 2, MIX_MFMA16 = 3, MIX_FUSED = 4, MIX_MFMA_TRIAL = 5, MIX_COUNT = 6 };
@@ -156,22 +156,22 @@ __global__ __launch_bounds__(PT) void probe_mix_kernel(int iters, float* __restr
         if constexpr (MIX == MIX_FUSED) {
             // forward: sign multiply + register stages, in-row stages, argument, sincos, products;
             // adjoint: register stages, in-row stages, accumulate
-            plain_ops<32>(v, c);
+            plain_ops<28>(v, c);
             dpp_ops<32>(v, c);
-            plain_ops<22>(v, c);
+            plain_ops<18>(v, c);
             trans_ops<16>(v);
-            plain_ops<22>(v, c);
+            plain_ops<18>(v, c);
             dpp_ops<32>(v, c);
-            plain_ops<32>(v, c);
+            plain_ops<28>(v, c);
         }
         if constexpr (MIX == MIX_MFMA_TRIAL) {
-            plain_ops<40>(v, c);
+            plain_ops<36>(v, c);
             mfma_ops<8>(acc, a, b);
-            plain_ops<22>(v, c);
+            plain_ops<18>(v, c);
             trans_ops<16>(v);
-            plain_ops<22>(v, c);
+            plain_ops<18>(v, c);
             mfma_ops<8>(acc, a, b);
-            plain_ops<40>(v, c);
+            plain_ops<36>(v, c);
         }
     }
     float s = 0.0f;

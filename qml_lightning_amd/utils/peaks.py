@@ -82,3 +82,18 @@ def instruction_mixes(device="cuda:0", iters=2000):
             t = _timed(run, 2)
             out[name][str(per_cu)] = t / units[0]
     return out
+
+
+if __name__ == "__main__":
+    # python -m qml_lightning_amd.utils.peaks [mixes|peaks]: one JSON line (what a profiler run of the
+    # probe kernels is pointed at)
+    import json
+    import sys
+    import qml_lightning_amd  # noqa: F401
+    what = sys.argv[1] if len(sys.argv) > 1 else "both"
+    out = {}
+    if what in ("peaks", "both"):
+        out["peaks"] = measure()
+    if what in ("mixes", "both"):
+        out["instruction_mixes_seconds_per_wavefront_iteration"] = instruction_mixes()
+    print(json.dumps(out))

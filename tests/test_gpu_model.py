@@ -557,3 +557,73 @@ def test_scripted_model_runs_in_a_host_without_python(tmp_path):
         f = np.array(lines[4 + ne:4 + ne + nf], dtype=np.float64).reshape(f0.shape)
         close(e, e0.detach().cpu().numpy(), 1e-6, "energies from the C++ host")
         close(f, f0.cpu().numpy(), 1e-5, "forces from the C++ host")
+
+
+@pytest.mark.parametrize("nmol,npcas,nstacks", [(12, 16, 4), (4, 64, 8)])
+def test_training_at_the_default_regularisation_vs_fp64_oracle_rows(nmol, npcas, nstacks):
+    """train() at the shipped default lambda = 1e-11 (hadamard_features.py:16): alpha solved from the
+    library's rows (force-feature rows summed over a molecule's atoms in fp32 before they are widened;
+    the reference widens every product, cuda/hadamard_kernel.cu:710) against alpha solved in numpy from
+    the fp64 oracle rows.  Both the overdetermined case (444 rows, 64 features) and the underdetermined
+    one (148 rows, 512 features: Z^T Z + lambda I has a condition number near 1 / eps).  alpha itself is
+    not comparable there (the normal matrix amplifies rounding by its condition number); what a user
+    sees is: the fit reproduces its training targets equally well, and held-out molecules are predicted
+    alike, to well below the fit's own error."""
+    species = [1, 6]
+    coords, charges = helpers.benzene_batch(nmol + 3, 5)
+    m, (red, D, bias, _) = build_sorf_model(species, npcas, nstacks)
+    m.llambda = 1e-11
+    m.nbatch_train = 5
+    prm = oracle_prm(species)
+    rng = np.random.default_rng(3)
+    c32 = [np.asarray(c, dtype=np.float32) for c in coords]
+    # smooth targets: a fixed random model's own energies and forces plus a little noise
+    _, _, _, a_true = helpers.model_weights(2, prm.repsize, npcas, nstacks, 1, 77)
+    X, Z, aid, mid, nat = make_batch(coords, charges)
+    E_all, F_all, _ = omodel.sorf_energy_forces(X, Z, aid, mid, nat, prm, species, red, D, bias, 0.05 * a_true, 2.0)
+    E_all = E_all + 1e-3 * rng.normal(size=E_all.shape)
+    F_all = F_all + 1e-3 * rng.normal(size=F_all.shape)
+    tr, te = slice(0, nmol), slice(nmol, nmol + 3)
+    m.train(c32[tr], charges[tr], E=list(E_all[tr]), F=[f for f in F_all[tr]], print_info=False)
+    rows, y = omodel.sorf_training_rows(*make_batch(coords[tr], charges[tr]), prm, species, red, D, bias, 2.0,
+                                        E=E_all[tr], F=F_all[tr])
+    ZTZ, ZTy = osorf.gram(rows, y)
+    a_ref = osorf.regularised_solve(ZTZ, ZTy, 1e-11)[:, 0]
+    a_gpu = m.alpha.double().cpu().numpy()
+    # the fit on its own training rows (fp64 rows of the oracle, both alphas)
+    res_gpu = np.abs(rows @ a_gpu - y[:, 0]).max()
+    res_ref = np.abs(rows @ a_ref - y[:, 0]).max()
+    scale = np.abs(y).max()
+    print("default lambda, %d rows x %d features: training residual gpu %.2e, oracle %.2e (targets up to %.2e)"
+          % (rows.shape[0], rows.shape[1], res_gpu, res_ref, scale))
+    assert res_gpu <= max(3.0 * res_ref, 2e-4 * scale)
+    # held-out molecules through the fp64 oracle with either alpha, and through the library's predict
+    Xt, Zt, at, mt, nt = make_batch(coords[te], charges[te])
+    E_ref, F_ref, _ = omodel.sorf_energy_forces(Xt, Zt, at, mt, nt, prm, species, red, D, bias, a_ref, 2.0)
+    E_g, F_g, _ = omodel.sorf_energy_forces(Xt, Zt, at, mt, nt, prm, species, red, D, bias, a_gpu, 2.0)
+    e_dev = np.abs(E_g - E_ref).max() / np.abs(E_ref).max()
+    f_dev = np.abs(F_g - F_ref).max() / np.abs(F_ref).max()
+    # the yardstick: the same solve from the oracle's rows with noise of 1e-7 of their largest entry, a
+    # hundredth of the parity tolerance of the features and the size of fp32 rounding in a feature
+    # value (the reference computes every feature value in fp32 too, cuda/hadamard_kernel.cu:561,583)
+    noisy = rows + 1e-7 * np.abs(rows).max() * np.random.default_rng(9).normal(size=rows.shape)
+    a_n = osorf.regularised_solve(*osorf.gram(noisy, y), 1e-11)[:, 0]
+    E_p, F_p, _ = omodel.sorf_energy_forces(Xt, Zt, at, mt, nt, prm, species, red, D, bias, a_n, 2.0)
+    e_yard = np.abs(E_p - E_ref).max() / np.abs(E_ref).max()
+    f_yard = np.abs(F_p - F_ref).max() / np.abs(F_ref).max()
+    print("held-out predictions vs the fp64-trained alpha: library-trained energies %.2e forces %.2e; "
+          "oracle rows with 1e-7 noise: energies %.2e forces %.2e" % (e_dev, f_dev, e_yard, f_yard))
+    assert e_dev <= max(1e-3, 3.0 * e_yard) and f_dev <= max(1e-3, 3.0 * f_yard)
+    # and the rows themselves: the force-feature rows (fp32 sum over a molecule's atoms) are as close to
+    # the fp64 oracle as the energy rows (every value widened before it is added)
+    if nmol <= 5:                      # one batch of nbatch_train = 5 molecules holds them all
+        data = m.format_data(c32[tr], charges[tr], E=list(E_all[tr]), F=[f for f in F_all[tr]])
+        got = m._batch_rows(data, True).cpu().numpy()
+        err = np.abs(got - rows)
+        rms_e = np.sqrt((err[:nmol] ** 2).mean()) / np.abs(rows[:nmol]).max()
+        rms_f = np.sqrt((err[nmol:] ** 2).mean()) / np.abs(rows[nmol:]).max()
+        print("rows vs oracle, rms error over largest entry: energy rows %.2e, force rows %.2e" % (rms_e, rms_f))
+        assert rms_f <= max(2.0 * rms_e, 1e-7) and rms_e <= 5e-7
+    e, f = m.predict(c32[te], charges[te], 12, forces=True, print_info=False)
+    close(e, E_g, 5e-4, "library predict with its own alpha, energies")     # fp32 contraction with an alpha of large entries
+    close(f, F_g, 5e-4, "library predict with its own alpha, forces")
