@@ -19,6 +19,8 @@
 // da/dR_i = u_ij, da/dR_j = -u_ij, db/dR_i = u_ik, db/dR_k = -u_ik, dc/dR_j = u_jk,
 // dc/dR_k = -u_jk.  This is algebraically the reference's 40-term expansion; the
 // degenerate-angle guard sqrt(max(1e-10, a^2 b^2 - (d_ij.d_ik)^2)) is kept.
+#include <type_traits>
+
 #include "qmll_common.h"
 
 namespace {
@@ -57,6 +59,9 @@ struct FchlArgs {
 constexpr int TCH = 256;      // smallest triple table
 constexpr int TCH_MAX = 1024; // largest (16 KB): beyond, element pairs are processed in chunks
 constexpr float PI_F = 3.14159265358979323846f;
+// three floats read from a 16-byte-aligned LDS entry with a single 12-byte instruction (a 16-byte
+// read of the same entry occupies the LDS pipe a third longer)
+typedef float float3v __attribute__((ext_vector_type(3)));
 
 // LDS neighbour arrays of one central atom, sorted by element type (stable in j within a
 // type); goff[e]..goff[e+1] is the slice of type e.
@@ -237,9 +242,9 @@ __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i,
                         s.dy[pos] = dy;
                         s.dz[pos] = dz;
                         s.r[pos] = r;
-                        // fc = (cos(pi r/rc) + 1)/2 and its r-derivative from one polynomial sincos
+                        // fc = (cos(pi r/rc) + 1)/2 and its r-derivative from one sine / cosine pair
                         float sn, cs;
-                        sincos_f32(r * PI_F * inv_rc, &sn, &cs);
+                        sincos_hw(r * PI_F * inv_rc, &sn, &cs);
                         s.fc[pos] = 0.5f * (cs + 1.0f);
                         s.dfc[pos] = -0.5f * PI_F * inv_rc * sn;
                         s.el[pos] = e;
@@ -272,19 +277,12 @@ __device__ __forceinline__ void unrank_pair(int t, int nn, int& j, int& k) {
 }
 
 // pair t of the list of pairs (j<k) enumerated k-major: t = k (k - 1) / 2 + j, 0 <= j < k.  No
-// search: k = floor((1 + sqrt(8 t + 1)) / 2) from the 1-ulp square root, put right by one
-// comparison either way; all quantities are integers below 2^24, exact in fp32 (t < 2^20).
+// search and no correction step: for t in [k (k - 1) / 2, (k + 1) k / 2) the value 2 t + 1.25 lies in
+// [(k - 1/2)^2 + 1, (k + 1/2)^2 - 1], so 1/2 + sqrt(2 t + 1.25) stays at least 1 / (2 k) inside
+// (k, k + 1), hundreds of ulps for every t < 2^20 (k < 1449) even with a root two ulps off.
 __device__ __forceinline__ void unrank_pair_kmajor(int t, int& j, int& k) {
-    const float tf = (float)t;
-    float kf = floorf(0.5f + 0.5f * fsqrt(fmaf(8.0f, tf, 1.0f)));
-    float tri = 0.5f * fmaf(kf, kf, -kf);                 // k (k - 1) / 2
-    kf -= tri > tf ? 1.0f : 0.0f;
-    tri = 0.5f * fmaf(kf, kf, -kf);
-    const float up = tri + kf <= tf ? 1.0f : 0.0f;        // (k + 1) k / 2 <= t
-    tri += up * kf;
-    kf += up;
-    k = (int)kf;
-    j = (int)(tf - tri);
+    k = (int)(0.5f + fsqrt(fmaf(2.0f, (float)t, 1.25f)));
+    j = t - (__mul24(k, k - 1) >> 1);
 }
 
 __device__ __forceinline__ int pair_offset(int ej, int ek, int ns, int nRs2, int nRs3) {
@@ -355,10 +353,15 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     // [cap][4] per neighbour: mu_j, log2(e) / (2 sigma_j^2), r^-d2 fc / (sigma sqrt(2pi)), -
     // (16-byte aligned: one LDS read per neighbour in the two-body loop)
     float* s2b = s.next + ((4 - ((size_t)(s.next - smem) & 3)) & 3);
-    float* slnRs2 = s2b + 4 * a.cap;   // [nRs2]
+    // [cap][4] per neighbour, read with one instruction each by the triples: (d_ij, 1 / r) and
+    // (sk3 r / 2, fc r^-d3, element type, index within the type | neighbours of the type << 16)
+    float* recA = s2b + 4 * a.cap;
+    float* recB = recA + 4 * a.cap;
+    float* slnRs2 = recB + 4 * a.cap;  // [nRs2]
     float* sinvRs2 = slnRs2 + nRs2; // [nRs2]
     float* sRs3 = sinvRs2 + nRs2;   // [nRs3]
     int* pbase = (int*)(sRs3 + nRs3);   // [ns*ns] first table entry of each element pair
+    int* prounds = pbase + ns * ns;     // [ns*ns] rounds of each element pair's segment
 
     // Global loads that do not depend on the neighbourhood are issued first and consumed after
     // the staging, so their latency overlaps the staging's own loads.
@@ -382,14 +385,23 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     for (int t = lane + QMLL_WAVE; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
     __syncthreads();
 
-    // per-neighbour two-body factors
+    const float zeta2 = 0.014383766711652736f;   // 2 exp(-pi^2 / 2)
+    const float k3 = a.p.eta3 * LOG2E;
+    const float sk3 = fsqrt(k3);                 // exp(-eta3 (rho - Rs)^2) = exp2(-(sk3 rho - sk3 Rs)^2)
+    // per-neighbour factors of the two-body bins and of the triples
     for (int j = lane; j < nn; j += QMLL_WAVE) {
-        const float r = s.r[j];
-        const float s2 = flog(1.0f + a.p.eta2 * frcp(r * r));
+        const float r = s.r[j], fc = s.fc[j];
+        const float ir = frcp(r), l2r = flog2(r);
+        const float s2 = flog(fmaf(a.p.eta2 * ir, ir, 1.0f));
         reinterpret_cast<float4*>(s2b)[j] = make_float4(
-            flog(r) - 0.5f * s2,                         // ln(r / sqrt(1 + eta2/r^2))
+            fmaf(l2r, 0.6931471805599453f, -0.5f * s2),   // ln(r / sqrt(1 + eta2/r^2))
             0.5f * LOG2E * frcp(s2),
-            rsqrtf(s2) * 0.3989422804014327f * fexp2(-a.p.two_body_decay * flog2(r)) * s.fc[j], 0.0f);
+            rsqrtf(s2) * 0.3989422804014327f * fexp2(-a.p.two_body_decay * l2r) * fc, 0.0f);
+        const int e = s.el[j], g0 = s.goff[e];
+        reinterpret_cast<float4*>(recA)[j] = make_float4(s.dx[j], s.dy[j], s.dz[j], ir);
+        reinterpret_cast<float4*>(recB)[j] = make_float4(sk3 * 0.5f * r, fc * fexp2(-a.p.three_body_decay * l2r),
+                                                         __int_as_float(e),
+                                                         __int_as_float((j - g0) | ((s.goff[e + 1] - g0) << 16)));
     }
     __syncthreads();
 
@@ -415,7 +427,7 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
                 for (int it = 0; it < rounds; ++it) {
                     const int j = j0 + jsub + it * JS;
                     const bool jok = zok && j < j1;
-                    const float4 f = reinterpret_cast<const float4*>(s2b)[jok ? j : j0];
+                    const float3v f = *reinterpret_cast<const float3v*>(s2b + 4 * (jok ? j : j0));   // one 12-byte LDS read
                     const float u = lnRs - f.x;
                     acc = fmaf(jok ? f.z : 0.0f, fexp2(-u * u * f.y), acc);
                 }
@@ -428,47 +440,39 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     }
 
     // ---- three-body blocks ----
-    const float zeta2 = 0.014383766711652736f;   // 2 exp(-pi^2 / 2)
-    const float k3 = a.p.eta3 * LOG2E;
-    const float sk3 = fsqrt(k3);                 // exp(-eta3 (rho - Rs)^2) = exp2(-(sk3 rho - sk3 Rs)^2)
     const int W3 = nRs3 < 64 ? nRs3 : 64;
     const int TS = idiv_small(64, W3);
     const int tsub = idiv_small(lane, W3), ll = lane - tsub * W3;
     constexpr int MAXLB = 4;                     // radial bins handled: up to 4 x 64
 
-    // one table entry per triple: (sk3 rho, K cos, K sin, -)
-    auto table_entry = [&](int j, int k) -> float4 {
-        const Triple t = triple_geometry(s, j, k);
-        const float ksi = a.p.three_body_weight * (1.0f + 3.0f * t.ci * t.cj * t.ck) *
-                          fexp2(-a.p.three_body_decay * flog2(t.a * t.b * t.c));
-        const float f = zeta2 * ksi * s.fc[j] * s.fc[k];
-        return make_float4(sk3 * 0.5f * (t.a + t.b), f * t.cosT, f * t.sinT, 0.0f);
+    // one table entry per triple: (sk3 rho, K cos, K sin, -) from the two neighbours' records.  With
+    // a = d_ij, b = d_ik, c = b - a: cos_i cos_j cos_k = -(a.b)(a.c)(c.b) / (|a| |b| |c|)^2, the decay
+    // (|a| |b| |c|)^-d3 is the product of the neighbours' factors and |c|^-d3 = exp2(-d3 log2(c.c) / 2);
+    // sin_i = |a x b| / (|a| |b|) keeps full relative accuracy near collinear triples.
+    const float zw3 = zeta2 * a.p.three_body_weight, hd3 = -0.5f * a.p.three_body_decay;
+    auto table_entry = [&](const float4 Aj, const float4 Bj, const float4 Ak, const float4 Bk) -> float4 {
+        const float cx = Ak.x - Aj.x, cy = Ak.y - Aj.y, cz = Ak.z - Aj.z;
+        const float c2 = cx * cx + cy * cy + cz * cz;
+        const float vi = Aj.x * Ak.x + Aj.y * Ak.y + Aj.z * Ak.z;
+        const float dac = Aj.x * cx + Aj.y * cy + Aj.z * cz;
+        const float dcb = cx * Ak.x + cy * Ak.y + cz * Ak.z;
+        const float w = Aj.w * Ak.w;
+        const float W = w * rsqrtf(c2);
+        const float px = Aj.y * Ak.z - Aj.z * Ak.y, py = Aj.z * Ak.x - Aj.x * Ak.z, pz = Aj.x * Ak.y - Aj.y * Ak.x;
+        const float f = zw3 * fmaf(-3.0f * vi * dac, dcb * W * W, 1.0f) * Bj.y * Bk.y * fexp2(hd3 * flog2(c2));
+        const float cosT = fminf(1.0f, fmaxf(-1.0f, vi * w));
+        const float sinT = fminf(1.0f, fsqrt(px * px + py * py + pz * pz) * w);
+        return make_float4(Bj.x + Bk.x, f * cosT, f * sinT, 0.0f);
     };
-    // bin sums of `count` table entries starting at `first`, added to the accumulators.  The
-    // entries up to the next multiple of TS are zero entries, so every sub-slot runs the same
-    // number of rounds and the loop is wavefront-uniform (scalar control, unrollable).
-    auto accumulate = [&](int first, int count, float (&accc)[MAXLB], float (&accs)[MAXLB]) {
-        const int rounds = idiv_small(count + TS - 1, TS);
-        const float4* src = reinterpret_cast<const float4*>(trip) + first + (tsub < TS ? tsub : 0);
+    const float4* rA = reinterpret_cast<const float4*>(recA);
+    const float4* rB = reinterpret_cast<const float4*>(recB);
+    // this lane's radial grid points, pre-scaled
+    float rsl[MAXLB];
 #pragma unroll
-        for (int b = 0; b < MAXLB; ++b) {
-            const int l = b * 64 + ll;
-            if (b * 64 < nRs3) {
-                const float rs = sk3 * sRs3[l < nRs3 ? l : 0];
-                float c_ = accc[b], s_ = accs[b];
-#pragma unroll 4
-                for (int it = 0; it < rounds; ++it) {
-                    const float4 v = src[it * TS];
-                    const float d = v.x - rs;
-                    const float e = fexp2(-d * d);
-                    c_ = fmaf(e, v.y, c_);
-                    s_ = fmaf(e, v.z, s_);
-                }
-                accc[b] = c_;
-                accs[b] = s_;
-            }
-        }
-    };
+    for (int b = 0; b < MAXLB; ++b) {
+        const int l = b * 64 + ll;
+        rsl[b] = (b * 64 < nRs3) ? sk3 * sRs3[l < nRs3 ? l : 0] : 0.0f;
+    }
     // fold the triple sub-slots and store the block of pair (p,q)
     auto store_block = [&](int sbase, const float (&accc)[MAXLB], const float (&accs)[MAXLB]) {
 #pragma unroll
@@ -487,78 +491,137 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
             }
         }
     };
-
     const int ntrip = nn * (nn - 1) / 2;
-    if (ntrip <= a.tcap) {
-        // All triples at once (three passes of 64 lanes at 20 neighbours instead of one or
-        // more per element pair): the table is ordered by element pair, pbase[p*ns+q] is
-        // the first entry of pair (p<=q), and a triple's slot follows from its position in
-        // the sorted list.
-        if (lane == 0) {
-            int acc = 0;
-            for (int p = 0; p < ns; ++p) {
-                const int np_ = s.goff[p + 1] - s.goff[p];
-                for (int q = p; q < ns; ++q) {
-                    pbase[p * ns + q] = acc;
-                    const int ntr = (p == q) ? np_ * (np_ - 1) / 2 : np_ * (s.goff[q + 1] - s.goff[q]);
-                    acc += idiv_small(ntr + TS - 1, TS) * TS;   // segments start on a multiple of TS
+
+    // The rest of the kernel, with the sub-slot count as a compile-time constant where it is one of
+    // the common ones (TSC = 0: any): the table reads of a round then sit at fixed offsets from
+    // one address per lane.
+    auto three_body = [&](auto tsc) {
+        constexpr int TSC = decltype(tsc)::value;
+        const int TSv = TSC ? TSC : TS;
+        // bin sums of `rounds` rounds of table entries starting at `first`, added to the
+        // accumulators.  A segment is padded with zero entries to whole rounds, so every sub-slot
+        // runs the same number of rounds and the loop is wavefront-uniform (scalar control, unrollable).
+        auto accumulate = [&](int first, int rounds, float (&accc)[MAXLB], float (&accs)[MAXLB]) {
+            const float4* src = reinterpret_cast<const float4*>(trip) + first + (tsub < TSv ? tsub : 0);
+#pragma unroll
+            for (int b = 0; b < MAXLB; ++b) {
+                if (b * 64 < nRs3) {
+                    const float rs = rsl[b];
+                    float c_ = accc[b], s_ = accs[b];
+#pragma unroll 4
+                    for (int it = 0; it < rounds; ++it) {
+                        const float3v v = *reinterpret_cast<const float3v*>(src + it * TSv);   // one 12-byte LDS read
+                        const float d = v.x - rs;
+                        const float e = fexp2(-d * d);
+                        c_ = fmaf(e, v.y, c_);
+                        s_ = fmaf(e, v.z, s_);
+                    }
+                    accc[b] = c_;
+                    accs[b] = s_;
                 }
             }
+        };
+        if (ntrip <= a.tcap) {
+            // All triples at once (three passes of 64 lanes at 20 neighbours instead of one or
+            // more per element pair): the table is ordered by element pair, pbase[p*ns+q] is
+            // the first entry of pair (p<=q), prounds[p*ns+q] its length in rounds, and a triple's
+            // slot follows from its position in the sorted list.
+            if (ns * ns <= QMLL_WAVE) {
+                // lane p*ns+q takes pair (p,q); an exclusive scan over the lanes gives the starts
+                const int p = idiv_small(lane, ns), q = lane - p * ns;
+                int rounds = 0;
+                if (lane < ns * ns && q >= p) {
+                    const int np_ = s.goff[p + 1] - s.goff[p], nq = s.goff[q + 1] - s.goff[q];
+                    const int ntr = (p == q) ? (__mul24(np_, np_ - 1) >> 1) : __mul24(np_, nq);
+                    rounds = idiv_small(ntr + TSv - 1, TSv);
+                }
+                const int size = rounds * TSv;               // segments start on a multiple of TS
+                int incl = size;
+                for (int o = 1; o < ns * ns; o <<= 1) {
+                    const int up = __shfl_up(incl, o, 64);
+                    if (lane >= o) incl += up;
+                }
+                if (lane < ns * ns) {
+                    pbase[lane] = incl - size;
+                    prounds[lane] = rounds;
+                }
+            } else if (lane == 0) {
+                int acc = 0;
+                for (int p = 0; p < ns; ++p) {
+                    const int np_ = s.goff[p + 1] - s.goff[p];
+                    for (int q = p; q < ns; ++q) {
+                        const int ntr = (p == q) ? np_ * (np_ - 1) / 2 : np_ * (s.goff[q + 1] - s.goff[q]);
+                        const int rounds = idiv_small(ntr + TSv - 1, TSv);
+                        pbase[p * ns + q] = acc;
+                        prounds[p * ns + q] = rounds;
+                        acc += rounds * TSv;
+                    }
+                }
+            }
+            __syncthreads();
+            for (int tt = lane; tt < ntrip; tt += QMLL_WAVE) {
+                int j, k;
+                unrank_pair_kmajor(tt, j, k);
+                const float4 Aj = rA[j], Ak = rA[k], Bj = rB[j], Bk = rB[k];
+                const int p = __float_as_int(Bj.z), q = __float_as_int(Bk.z);   // p <= q: the list is sorted by type
+                const int wj = __float_as_int(Bj.w), wk = __float_as_int(Bk.w);
+                const int jl = wj & 0xffff, kl = wk & 0xffff;
+                // any one-to-one numbering of a pair's triples does: k-major within one type, row by row else
+                const int local = (p == q ? (__mul24(kl, kl - 1) >> 1) : __mul24(kl, wj >> 16)) + jl;
+                reinterpret_cast<float4*>(trip)[pbase[__mul24(p, ns) + q] + local] = table_entry(Aj, Bj, Ak, Bk);
+            }
+            __syncthreads();
+            for (int p = 0; p < ns; ++p) {
+                for (int q = p; q < ns; ++q) {
+                    float accc[MAXLB], accs[MAXLB];
+#pragma unroll
+                    for (int b = 0; b < MAXLB; ++b) accc[b] = accs[b] = 0.0f;
+                    accumulate(pbase[p * ns + q], prounds[p * ns + q], accc, accs);
+                    store_block(pair_offset(p, q, ns, nRs2, nRs3), accc, accs);
+                }
+            }
+            return;
         }
-        __syncthreads();
-        for (int tt = lane; tt < ntrip; tt += QMLL_WAVE) {
-            int j, k;
-            unrank_pair_kmajor(tt, j, k);
-            const int p = s.el[j], q = s.el[k];           // p <= q: the list is sorted by type
-            const int jl = j - s.goff[p], kl = k - s.goff[q];
-            // any one-to-one numbering of a pair's triples does: k-major within one type, row by row else
-            const int local = (p == q) ? (kl * (kl - 1)) / 2 + jl : kl * (s.goff[p + 1] - s.goff[p]) + jl;
-            *reinterpret_cast<float4*>(trip + (pbase[p * ns + q] + local) * 4) = table_entry(j, k);
-        }
-        __syncthreads();
+        // more triples than the table holds: element pair by element pair, in chunks of the table
         for (int p = 0; p < ns; ++p) {
-            const int np_ = s.goff[p + 1] - s.goff[p];
+            const int op = s.goff[p], np_ = s.goff[p + 1] - op;
             for (int q = p; q < ns; ++q) {
-                const int nq = s.goff[q + 1] - s.goff[q];
+                const int oq = s.goff[q], nq = s.goff[q + 1] - oq;
                 const int ntr = (p == q) ? np_ * (np_ - 1) / 2 : np_ * nq;
                 float accc[MAXLB], accs[MAXLB];
 #pragma unroll
                 for (int b = 0; b < MAXLB; ++b) accc[b] = accs[b] = 0.0f;
-                accumulate(pbase[p * ns + q], ntr, accc, accs);
+                for (int t0 = 0; t0 < ntr; t0 += a.tcap) {
+                    const int nchunk = min(a.tcap, ntr - t0);
+                    const int rounds = idiv_small(nchunk + TSv - 1, TSv);
+                    __syncthreads();
+                    for (int tt = lane; tt < nchunk; tt += QMLL_WAVE) {
+                        int ja, kb;
+                        if (p == q) {
+                            unrank_pair(t0 + tt, np_, ja, kb);
+                        } else {
+                            ja = (t0 + tt) / nq;
+                            kb = (t0 + tt) - ja * nq;
+                        }
+                        reinterpret_cast<float4*>(trip)[tt] =
+                            table_entry(rA[op + ja], rB[op + ja], rA[oq + kb], rB[oq + kb]);
+                    }
+                    if (lane < rounds * TSv - nchunk)
+                        *reinterpret_cast<float4*>(trip + (nchunk + lane) * 4) = make_float4(0.f, 0.f, 0.f, 0.f);
+                    __syncthreads();
+                    accumulate(0, rounds, accc, accs);
+                }
                 store_block(pair_offset(p, q, ns, nRs2, nRs3), accc, accs);
             }
         }
-        return;
-    }
-    // more triples than the table holds: element pair by element pair, in chunks of the table
-    for (int p = 0; p < ns; ++p) {
-        const int op = s.goff[p], np_ = s.goff[p + 1] - op;
-        for (int q = p; q < ns; ++q) {
-            const int oq = s.goff[q], nq = s.goff[q + 1] - oq;
-            const int ntr = (p == q) ? np_ * (np_ - 1) / 2 : np_ * nq;
-            float accc[MAXLB], accs[MAXLB];
-#pragma unroll
-            for (int b = 0; b < MAXLB; ++b) accc[b] = accs[b] = 0.0f;
-            for (int t0 = 0; t0 < ntr; t0 += a.tcap) {
-                const int nchunk = min(a.tcap, ntr - t0);
-                __syncthreads();
-                for (int tt = lane; tt < nchunk; tt += QMLL_WAVE) {
-                    int ja, kb;
-                    if (p == q) {
-                        unrank_pair(t0 + tt, np_, ja, kb);
-                    } else {
-                        ja = (t0 + tt) / nq;
-                        kb = (t0 + tt) - ja * nq;
-                    }
-                    *reinterpret_cast<float4*>(trip + tt * 4) = table_entry(op + ja, oq + kb);
-                }
-                if (lane < idiv_small(nchunk + TS - 1, TS) * TS - nchunk)
-                    *reinterpret_cast<float4*>(trip + (nchunk + lane) * 4) = make_float4(0.f, 0.f, 0.f, 0.f);
-                __syncthreads();
-                accumulate(0, nchunk, accc, accs);
-            }
-            store_block(pair_offset(p, q, ns, nRs2, nRs3), accc, accs);
-        }
+    };
+    switch (TS) {
+        case 1: three_body(std::integral_constant<int, 1>{}); break;
+        case 2: three_body(std::integral_constant<int, 2>{}); break;
+        case 3: three_body(std::integral_constant<int, 3>{}); break;
+        case 4: three_body(std::integral_constant<int, 4>{}); break;
+        default: three_body(std::integral_constant<int, 0>{}); break;
     }
 }
 
@@ -1163,10 +1226,10 @@ extern "C" int qmll_fchl19_forward(const float* X, const int* types, const float
     // each of the ns (ns+1)/2 segments is padded to a multiple of the triple sub-slot count
     const int tsub_slots = prm->nRs3 < 64 ? 64 / prm->nRs3 : 1;
     a.tpad = prm->nspecies * (prm->nspecies + 1) / 2 * (tsub_slots - 1);
-    // triple table, neighbour arrays + type offsets, per-neighbour two-body factors [cap][4] (behind up
+    // triple table, neighbour arrays + type offsets, three per-neighbour records [cap][4] (behind up
     // to 3 floats of alignment), the radial grids, the table's segment starts
-    const size_t lds = sizeof(float) * ((size_t)(STAGE_ARRAYS + 4) * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 +
-                                        4 * (size_t)(a.tcap + a.tpad) + (size_t)prm->nspecies * prm->nspecies + 4);
+    const size_t lds = sizeof(float) * ((size_t)(STAGE_ARRAYS + 12) * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 +
+                                        4 * (size_t)(a.tcap + a.tpad) + 2 * (size_t)prm->nspecies * prm->nspecies + 4);
     QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
                  "qmll_fchl19_forward: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R, LDS_LIMIT);
     hipLaunchKernelGGL(fchl19_forward_kernel, dim3(A), dim3(64), lds, (hipStream_t)stream, a, rep);
