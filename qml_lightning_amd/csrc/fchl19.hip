@@ -108,12 +108,15 @@ __device__ __forceinline__ void min_image(float& dx, float& dy, float& dz, const
 }
 
 
-// Fill the LDS neighbour arrays of atom (m,i), sorted by element type; returns the
-// neighbour count.  Neighbours whose element type is negative (charge not in `species`)
-// are dropped.  Up to 64 candidates take a single pass; beyond, pass 0 counts per type (lane e
-// keeps the count of type e) and pass 1 scatters each neighbour to goff[type] + its rank among
-// the earlier neighbours of that type.
-__device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i, int lane) {
+// Visit the neighbours of atom (m,i) sorted by element type; returns the neighbour count.
+// goff[e]..goff[e+1] becomes the slice of type e, and emit(pos, rank, count, e, j, dx, dy, dz, r2)
+// is called once per neighbour by the lane that found it: pos its place in the sorted list, rank
+// its place among the `count` neighbours of its type e, j its atom index, d = R_i - R_j.
+// Neighbours whose element type is negative (charge not in `species`) are dropped.  Up to 64
+// candidates take a single pass; beyond, pass 0 counts per type (lane e keeps the count of type
+// e) and pass 1 places each neighbour at goff[type] + its rank among the earlier ones of that type.
+template <class Emit>
+__device__ __forceinline__ int visit_neighbours(const FchlArgs& a, int* goff, int m, int i, int lane, Emit emit) {
     const float* Xm = a.X + (size_t)m * a.n * 3;
     const int* tm = a.types + (size_t)m * a.n;
     const int ns = a.p.nspecies;
@@ -132,7 +135,6 @@ __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i,
     const float xo = Xm[own * 3 + 0], yo = Xm[own * 3 + 1], zo = Xm[own * 3 + 2];
     const int eo = tm[own];
     const float rc2 = a.p.rcut * a.p.rcut;
-    const float inv_rc = frcp(a.p.rcut);
     const bool have_list = a.nlist != nullptr;
     int total;
     const int* li = nullptr;
@@ -167,30 +169,22 @@ __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i,
         // a supplied list is authoritative (it may be stale on purpose, e.g. finite
         // differences with a frozen list); only the built-in search applies the cutoff
         const bool ok = jok && (have_list ? (r2 > 0.0f) : (r2 < rc2 && r2 > 0.0f)) && e >= 0 && e < ns;
-        int start = 0, pos = 0;
+        int start = 0, pos = 0, rank = 0, count = 0;
         const unsigned long long below = (1ull << lane) - 1ull;
         for (int ep = 0; ep < ns; ++ep) {
             const unsigned long long mask = __ballot(ok && e == ep);
-            if (lane == 0) s.goff[ep] = start;
-            if (e == ep) pos = start + __popcll(mask & below);
-            start += __popcll(mask);
+            if (lane == 0) goff[ep] = start;
+            const int cnt = __popcll(mask);
+            if (e == ep) {
+                rank = __popcll(mask & below);
+                pos = start + rank;
+                count = cnt;
+            }
+            start += cnt;
         }
         const int nn = start < a.cap ? start : a.cap;
-        if (lane == 0) s.goff[ns] = nn;
-        if (ok && pos < a.cap) {
-            const float r = fsqrt(r2);
-            s.dx[pos] = dx;
-            s.dy[pos] = dy;
-            s.dz[pos] = dz;
-            s.r[pos] = r;
-            // fc = (cos(pi r/rc) + 1)/2 and its r-derivative from one sine / cosine pair
-            float sn, cs;
-            sincos_hw(r * PI_F * inv_rc, &sn, &cs);
-            s.fc[pos] = 0.5f * (cs + 1.0f);
-            s.dfc[pos] = -0.5f * PI_F * inv_rc * sn;
-            s.el[pos] = e;
-            s.j[pos] = j;
-        }
+        if (lane == 0) goff[ns] = nn;
+        if (ok && pos < a.cap) emit(pos, rank, count, e, j, dx, dy, dz, r2);
         return nn;
     }
     int mycount = 0;   // lane e: neighbours of type e seen so far
@@ -203,10 +197,10 @@ __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i,
                 const int up = __shfl_up(incl, o, 64);
                 if (lane >= o) incl += up;
             }
-            if (lane < ns) s.goff[lane] = incl - mycount;
+            if (lane < ns) goff[lane] = incl - mycount;
             nn = __shfl(incl, ns - 1, 64);
             if (nn > a.cap) nn = a.cap;
-            if (lane == 0) s.goff[ns] = nn;
+            if (lane == 0) goff[ns] = nn;
             mycount = 0;
             __syncthreads();
         }
@@ -235,27 +229,40 @@ __device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i,
                 const unsigned long long mask = __ballot(ok && e == ep);
                 const int before = __builtin_amdgcn_readlane(mycount, ep);
                 if (pass == 1 && ok && e == ep) {
-                    const int pos = s.goff[ep] + before + __popcll(mask & ((1ull << lane) - 1ull));
-                    if (pos < a.cap) {
-                        const float r = fsqrt(r2);
-                        s.dx[pos] = dx;
-                        s.dy[pos] = dy;
-                        s.dz[pos] = dz;
-                        s.r[pos] = r;
-                        // fc = (cos(pi r/rc) + 1)/2 and its r-derivative from one sine / cosine pair
-                        float sn, cs;
-                        sincos_hw(r * PI_F * inv_rc, &sn, &cs);
-                        s.fc[pos] = 0.5f * (cs + 1.0f);
-                        s.dfc[pos] = -0.5f * PI_F * inv_rc * sn;
-                        s.el[pos] = e;
-                        s.j[pos] = j;
-                    }
+                    const int first = goff[ep];
+                    const int rank = before + __popcll(mask & ((1ull << lane) - 1ull));
+                    // goff of the last type's end may have been clipped to the capacity
+                    if (first + rank < a.cap) emit(first + rank, rank, goff[ep + 1] - first, e, j, dx, dy, dz, r2);
                 }
                 if (lane == ep) mycount += __popcll(mask);
             }
         }
     }
     return nn;
+}
+
+// the cosine cutoff fc = (cos(pi r / rc) + 1) / 2 and its r-derivative from one sine / cosine pair
+__device__ __forceinline__ void cutoff(float r, float inv_rc, float& fc, float& dfc) {
+    float sn, cs;
+    sincos_hw(r * PI_F * inv_rc, &sn, &cs);
+    fc = 0.5f * (cs + 1.0f);
+    dfc = -0.5f * PI_F * inv_rc * sn;
+}
+
+// the neighbour arrays of `Stage` filled by visit_neighbours
+__device__ int stage_neighbours(const FchlArgs& a, const Stage& s, int m, int i, int lane) {
+    const float inv_rc = frcp(a.p.rcut);
+    return visit_neighbours(a, s.goff, m, i, lane,
+                            [&](int pos, int, int, int e, int j, float dx, float dy, float dz, float r2) {
+                                const float r = fsqrt(r2);
+                                s.dx[pos] = dx;
+                                s.dy[pos] = dy;
+                                s.dz[pos] = dz;
+                                s.r[pos] = r;
+                                cutoff(r, inv_rc, s.fc[pos], s.dfc[pos]);
+                                s.el[pos] = e;
+                                s.j[pos] = j;
+                            });
 }
 
 // 2^x and log2(x) on the transcendental unit (1 ulp)
@@ -348,20 +355,19 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     const int ns = a.p.nspecies, nRs2 = a.p.nRs2, nRs3 = a.p.nRs3;
     const int R = ns * nRs2 + ns * (ns + 1) * nRs3;
 
-    float* trip = smem;             // [tcap][4]: sk3 rho, K cos, K sin, -   (first: 16-byte aligned)
-    Stage s = carve(smem + 4 * (a.tcap + a.tpad), a.cap, ns);
-    // [cap][4] per neighbour: mu_j, log2(e) / (2 sigma_j^2), r^-d2 fc / (sigma sqrt(2pi)), -
-    // (16-byte aligned: one LDS read per neighbour in the two-body loop)
-    float* s2b = s.next + ((4 - ((size_t)(s.next - smem) & 3)) & 3);
-    // [cap][4] per neighbour, read with one instruction each by the triples: (d_ij, 1 / r) and
-    // (sk3 r / 2, fc r^-d3, element type, index within the type | neighbours of the type << 16)
-    float* recA = s2b + 4 * a.cap;
-    float* recB = recA + 4 * a.cap;
-    float* slnRs2 = recB + 4 * a.cap;  // [nRs2]
-    float* sinvRs2 = slnRs2 + nRs2; // [nRs2]
-    float* sRs3 = sinvRs2 + nRs2;   // [nRs3]
-    int* pbase = (int*)(sRs3 + nRs3);   // [ns*ns] first table entry of each element pair
-    int* prounds = pbase + ns * ns;     // [ns*ns] rounds of each element pair's segment
+    // LDS: the triple table, three records per neighbour (read with one instruction each), the
+    // type offsets, the radial grids, the table's segments
+    float* trip = smem;                                  // [tcap + tpad][4]: sk3 rho, K cos, K sin, -
+    float* recA = trip + 4 * (a.tcap + a.tpad);          // [cap][4]: d_ij, 1 / r
+    float* recB = recA + 4 * a.cap;                      // [cap][4]: sk3 r / 2, fc r^-d3, element type,
+                                                         //           index within the type | neighbours of the type << 16
+    float* s2b = recB + 4 * a.cap;                       // [cap][4]: mu_j, log2(e) / (2 sigma_j^2), r^-d2 fc / (sigma sqrt(2pi)), -
+    int* goff = (int*)(s2b + 4 * a.cap);                 // [ns+1] slices of the sorted neighbour list by type
+    float* slnRs2 = (float*)(goff + ns + 1);             // [nRs2]
+    float* sinvRs2 = slnRs2 + nRs2;                      // [nRs2]
+    float* sRs3 = sinvRs2 + nRs2;                        // [nRs3]
+    int* pbase = (int*)(sRs3 + nRs3);                    // [ns*ns] first table entry of each element pair
+    int* prounds = pbase + ns * ns;                      // [ns*ns] rounds of each element pair's segment
 
     // Global loads that do not depend on the neighbourhood are issued first and consumed after
     // the staging, so their latency overlaps the staging's own loads.
@@ -371,7 +377,26 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     for (int t = lane; t < a.tcap + a.tpad; t += QMLL_WAVE)
         reinterpret_cast<float4*>(trip)[t] = make_float4(0.f, 0.f, 0.f, 0.f);
 
-    const int nn = stage_neighbours(a, s, m, i, lane);
+    const float zeta2 = 0.014383766711652736f;   // 2 exp(-pi^2 / 2)
+    const float k3 = a.p.eta3 * LOG2E;
+    const float sk3 = fsqrt(k3);                 // exp(-eta3 (rho - Rs)^2) = exp2(-(sk3 rho - sk3 Rs)^2)
+    const float inv_rc = frcp(a.p.rcut);
+    // every neighbour's factors of the two-body bins and of the triples, by the lane that found it
+    const int nn = visit_neighbours(
+        a, goff, m, i, lane, [&](int pos, int rank, int count, int e, int, float dx, float dy, float dz, float r2) {
+            const float ir = __builtin_amdgcn_rsqf(r2), r = r2 * ir;
+            float fc, dfc;
+            cutoff(r, inv_rc, fc, dfc);
+            const float l2r = flog2(r);
+            const float s2 = flog(fmaf(a.p.eta2 * ir, ir, 1.0f));
+            reinterpret_cast<float4*>(s2b)[pos] = make_float4(
+                fmaf(l2r, 0.6931471805599453f, -0.5f * s2),   // ln(r / sqrt(1 + eta2/r^2))
+                0.5f * LOG2E * frcp(s2),
+                rsqrtf(s2) * 0.3989422804014327f * fexp2(-a.p.two_body_decay * l2r) * fc, 0.0f);
+            reinterpret_cast<float4*>(recA)[pos] = make_float4(dx, dy, dz, ir);
+            reinterpret_cast<float4*>(recB)[pos] = make_float4(sk3 * 0.5f * r, fc * fexp2(-a.p.three_body_decay * l2r),
+                                                               __int_as_float(e), __int_as_float(rank | (count << 16)));
+        });
     if (lane < nRs2) {
         slnRs2[lane] = flog(rs2v);
         sinvRs2[lane] = frcp(rs2v);
@@ -383,26 +408,6 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
         sinvRs2[t] = frcp(v);
     }
     for (int t = lane + QMLL_WAVE; t < nRs3; t += QMLL_WAVE) sRs3[t] = a.Rs3[t];
-    __syncthreads();
-
-    const float zeta2 = 0.014383766711652736f;   // 2 exp(-pi^2 / 2)
-    const float k3 = a.p.eta3 * LOG2E;
-    const float sk3 = fsqrt(k3);                 // exp(-eta3 (rho - Rs)^2) = exp2(-(sk3 rho - sk3 Rs)^2)
-    // per-neighbour factors of the two-body bins and of the triples
-    for (int j = lane; j < nn; j += QMLL_WAVE) {
-        const float r = s.r[j], fc = s.fc[j];
-        const float ir = frcp(r), l2r = flog2(r);
-        const float s2 = flog(fmaf(a.p.eta2 * ir, ir, 1.0f));
-        reinterpret_cast<float4*>(s2b)[j] = make_float4(
-            fmaf(l2r, 0.6931471805599453f, -0.5f * s2),   // ln(r / sqrt(1 + eta2/r^2))
-            0.5f * LOG2E * frcp(s2),
-            rsqrtf(s2) * 0.3989422804014327f * fexp2(-a.p.two_body_decay * l2r) * fc, 0.0f);
-        const int e = s.el[j], g0 = s.goff[e];
-        reinterpret_cast<float4*>(recA)[j] = make_float4(s.dx[j], s.dy[j], s.dz[j], ir);
-        reinterpret_cast<float4*>(recB)[j] = make_float4(sk3 * 0.5f * r, fc * fexp2(-a.p.three_body_decay * l2r),
-                                                         __int_as_float(e),
-                                                         __int_as_float((j - g0) | ((s.goff[e + 1] - g0) << 16)));
-    }
     __syncthreads();
 
     float* out = rep + ((size_t)m * a.n + i) * R;
@@ -420,7 +425,7 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
             for (int e = 0; e < ns; ++e) {
                 // the same number of rounds for every lane (the loop stays scalar and unrolls);
                 // a sub-slot past the end of the type's neighbours reads a valid entry with weight 0
-                const int j0 = s.goff[e], j1 = s.goff[e + 1];
+                const int j0 = goff[e], j1 = goff[e + 1];
                 const int rounds = idiv_small(j1 - j0 + JS - 1, JS);
                 float acc = 0.0f;
 #pragma unroll 2
@@ -532,7 +537,7 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
                 const int p = idiv_small(lane, ns), q = lane - p * ns;
                 int rounds = 0;
                 if (lane < ns * ns && q >= p) {
-                    const int np_ = s.goff[p + 1] - s.goff[p], nq = s.goff[q + 1] - s.goff[q];
+                    const int np_ = goff[p + 1] - goff[p], nq = goff[q + 1] - goff[q];
                     const int ntr = (p == q) ? (__mul24(np_, np_ - 1) >> 1) : __mul24(np_, nq);
                     rounds = idiv_small(ntr + TSv - 1, TSv);
                 }
@@ -549,9 +554,9 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
             } else if (lane == 0) {
                 int acc = 0;
                 for (int p = 0; p < ns; ++p) {
-                    const int np_ = s.goff[p + 1] - s.goff[p];
+                    const int np_ = goff[p + 1] - goff[p];
                     for (int q = p; q < ns; ++q) {
-                        const int ntr = (p == q) ? np_ * (np_ - 1) / 2 : np_ * (s.goff[q + 1] - s.goff[q]);
+                        const int ntr = (p == q) ? np_ * (np_ - 1) / 2 : np_ * (goff[q + 1] - goff[q]);
                         const int rounds = idiv_small(ntr + TSv - 1, TSv);
                         pbase[p * ns + q] = acc;
                         prounds[p * ns + q] = rounds;
@@ -585,9 +590,9 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
         }
         // more triples than the table holds: element pair by element pair, in chunks of the table
         for (int p = 0; p < ns; ++p) {
-            const int op = s.goff[p], np_ = s.goff[p + 1] - op;
+            const int op = goff[p], np_ = goff[p + 1] - op;
             for (int q = p; q < ns; ++q) {
-                const int oq = s.goff[q], nq = s.goff[q + 1] - oq;
+                const int oq = goff[q], nq = goff[q + 1] - oq;
                 const int ntr = (p == q) ? np_ * (np_ - 1) / 2 : np_ * nq;
                 float accc[MAXLB], accs[MAXLB];
 #pragma unroll
@@ -706,8 +711,13 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
     const int ns = a.p.nspecies, nRs2 = a.p.nRs2, nRs3 = a.p.nRs3;
     const int R = ns * nRs2 + ns * (ns + 1) * nRs3;
 
-    Stage s = carve(smem, a.cap, ns);
-    float* sgx = s.next;             // [cap] gradient on neighbour j
+    // [cap][4] per neighbour, read with one instruction each: (d_ij, r) and
+    // (1 / r, fc, dfc / dr, element type); first in LDS, 16-byte aligned
+    float* recA = smem;
+    float* recB = recA + 4 * a.cap;
+    int* sj = (int*)(recB + 4 * a.cap);   // [cap] atom index of neighbour j
+    int* goff = sj + a.cap;              // [ns+1] slices of the sorted neighbour list by type
+    float* sgx = (float*)(goff + ns + 1);   // [cap] gradient on neighbour j
     float* sgy = sgx + a.cap;
     float* sgz = sgy + a.cap;
     float* slnRs2 = sgz + a.cap;     // [nRs2]
@@ -715,6 +725,8 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
     float* sRs3 = sinvRs2 + nRs2;    // [nRs3]
     float* gin = sRs3 + nRs3;        // [R]
     float* tab = gin + R;            // TABLE: [6][ntrip]
+    const float4* rA = reinterpret_cast<const float4*>(recA);
+    const float4* rB = reinterpret_cast<const float4*>(recB);
 
     // Global loads that do not depend on the neighbourhood (grid tables, the incoming gradient
     // row) are issued first and consumed after the staging, so their latency overlaps the
@@ -731,7 +743,16 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
         sgy[t] = 0.0f;
         sgz[t] = 0.0f;
     }
-    const int nn = stage_neighbours(a, s, m, i, lane);
+    const float inv_rc = frcp(a.p.rcut);
+    const int nn = visit_neighbours(a, goff, m, i, lane,
+                                    [&](int pos, int, int, int e, int j, float dx, float dy, float dz, float r2) {
+                                        const float ir = __builtin_amdgcn_rsqf(r2), r = r2 * ir;
+                                        float fc, dfc;
+                                        cutoff(r, inv_rc, fc, dfc);
+                                        reinterpret_cast<float4*>(recA)[pos] = make_float4(dx, dy, dz, r);
+                                        reinterpret_cast<float4*>(recB)[pos] = make_float4(ir, fc, dfc, __int_as_float(e));
+                                        sj[pos] = j;
+                                    });
 #pragma unroll
     for (int k = 0; k < GREG; ++k)
         if (lane + QMLL_WAVE * k < R) gin[lane + QMLL_WAVE * k] = gr[k];
@@ -752,7 +773,6 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
     for (int t = lane + QMLL_WAVE; t < nRs3; t += QMLL_WAVE) sRs3[t] = sk3 * a.Rs3[t];
     __syncthreads();
 
-
     float gix = 0.0f, giy = 0.0f, giz = 0.0f;
 
     // two-body: lanes = (bin group g, neighbour j); group g takes the bins z = g, g+G, ...
@@ -763,9 +783,12 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
             const int j = G > 1 ? lane - g * nn : base + lane;
             const bool active = g < G && j < nn;
             float gr = 0.0f;
+            float4 Aj = make_float4(0.f, 0.f, 0.f, 1.f), Bj = make_float4(1.f, 0.f, 0.f, 0.f);
             if (active) {
-                const TwoBody tb = two_body_setup(s.r[j], s.fc[j], s.dfc[j], a.p);
-                const float* gz = gin + s.el[j] * nRs2;
+                Aj = rA[j];
+                Bj = rB[j];
+                const TwoBody tb = two_body_setup(Aj.w, Bj.y, Bj.z, a.p);
+                const float* gz = gin + __float_as_int(Bj.w) * nRs2;
                 for (int z = g; z < nRs2; z += G) {
                     float val, dval;
                     two_body_bin(tb, slnRs2[z], sinvRs2[z], val, dval);
@@ -775,8 +798,7 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
             float tot = gr;
             for (int k = 1; k < G; ++k) tot += __shfl(gr, (lane + nn * k) & 63, 64);
             if (active && g == 0) {
-                const float ir = frcp(s.r[j]);
-                const float ux = s.dx[j] * ir, uy = s.dy[j] * ir, uz = s.dz[j] * ir;   // dr/dR_i
+                const float ux = Aj.x * Bj.x, uy = Aj.y * Bj.x, uz = Aj.z * Bj.x;   // dr/dR_i
                 gix += tot * ux;
                 giy += tot * uy;
                 giz += tot * uz;
@@ -788,18 +810,51 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
     }
     __syncthreads();
 
-    // three-body: lane per triple, serial over radial bins
+    // three-body: lane per triple, serial over radial bins.  With a = d_ij, b = d_ik, c = b - a
+    // (= R_j - R_k) and X = cos_i cos_j cos_k the partials of P = 1 + 3 X by the three distances
+    // follow from the law of cosines:
+    //   P_a / 3 = cos_j cos_k / |b| + cos_i cos_k / |c| - cos_i cos_j |a| / (|b| |c|) - 2 X / |a|
+    // and cyclically; K = w3 P (abc)^-d3 fc(a) fc(b) and its partials share the factor
+    // dec = w3 (abc)^-d3, applied once at the end together with 2 exp(-pi^2 / 2).
     const int ntrip = nn * (nn - 1) / 2;
     const float zeta2 = 0.014383766711652736f;   // 2 exp(-pi^2 / 2)
+    const float d3 = a.p.three_body_decay;
     for (int tt = lane; tt < ntrip; tt += QMLL_WAVE) {
         int j, k;
         unrank_pair_kmajor(tt, j, k);                     // tt = k (k - 1) / 2 + j
-        const Triple t = triple_geometry(s, j, k);
-        const TripleDeriv d = triple_derivatives(t, a.p, s.fc[j], s.dfc[j], s.fc[k], s.dfc[k]);
-        const float* g = gin + pair_offset(s.el[j], s.el[k], ns, nRs2, nRs3);
+        const float4 Aj = rA[j], Ak = rA[k], Bj = rB[j], Bk = rB[k];
+        const float ia = Bj.x, ib = Bk.x;
+        const float cx = Ak.x - Aj.x, cy = Ak.y - Aj.y, cz = Ak.z - Aj.z;
+        const float c2 = cx * cx + cy * cy + cz * cz;
+        const float ic = __builtin_amdgcn_rsqf(c2), c = c2 * ic;
+        const float vi = Aj.x * Ak.x + Aj.y * Ak.y + Aj.z * Ak.z;
+        const float dac = Aj.x * cx + Aj.y * cy + Aj.z * cz;
+        const float dcb = cx * Ak.x + cy * Ak.y + cz * Ak.z;
+        const float w = ia * ib, iaic = ia * ic, ibic = ib * ic;
+        const float ci = vi * w, cj = -dac * iaic, ck = dcb * ibic;
+        // a^2 b^2 - (d_ij.d_ik)^2 = |d_ij x d_ik|^2 (Lagrange): the cross product keeps full
+        // relative accuracy near collinear triples, where the difference of squares cancels
+        const float px = Aj.y * Ak.z - Aj.z * Ak.y, py = Aj.z * Ak.x - Aj.x * Ak.z, pz = Aj.x * Ak.y - Aj.y * Ak.x;
+        const float cross2 = px * px + py * py + pz * pz;
+        const float cosT = fminf(1.0f, fmaxf(-1.0f, ci));
+        const float sinT = fminf(1.0f, fsqrt(cross2) * w);
+        const float guard_inv = Aj.w * Ak.w * __builtin_amdgcn_rsqf(fmaxf(1e-10f, cross2));
+        const float q1 = cj * ck, q2 = ci * ck, q3 = ci * cj;
+        const float X = ci * q1, X2 = X + X;
+        const float P = fmaf(3.0f, X, 1.0f);
+        const float Pa3 = fmaf(q1, ib, fmaf(q2, ic, fmaf(-q3 * Aj.w, ibic, -X2 * ia)));
+        const float Pb3 = fmaf(q1, ia, fmaf(q3, ic, fmaf(-q2 * Ak.w, iaic, -X2 * ib)));
+        const float Pc3 = fmaf(q2, ia, fmaf(q3, ib, fmaf(-q1 * c, w, -X2 * ic)));
+        const float Z = zeta2 * a.p.three_body_weight * fexp2(-d3 * flog2(Aj.w * Ak.w * c));
+        const float fa = Bj.y, dfa = Bj.z, fb = Bk.y, dfb = Bk.z;
+        const float F = fa * fb, d3P = d3 * P, FP = F * P;
+        const float ka = fmaf(F, fmaf(3.0f, Pa3, -d3P * ia), P * dfa * fb);   // K_a / dec
+        const float kb = fmaf(F, fmaf(3.0f, Pb3, -d3P * ib), P * fa * dfb);
+        const float kc = F * fmaf(3.0f, Pc3, -d3P * ic);
+        const float* g = gin + pair_offset(__float_as_int(Bj.w), __float_as_int(Bk.w), ns, nRs2, nRs3);
         // exp(-eta3 (rho - Rs)^2) = exp2(-(sk3 rho - sk3 Rs)^2) with the grid stored pre-scaled;
         // d e / d rho = -2 eta3 (rho - Rs) e = hfac (sk3 rho - sk3 Rs) e, the factor applied after the sums
-        const float rho = sk3 * 0.5f * (t.a + t.b);
+        const float rho = sk3 * 0.5f * (Aj.w + Ak.w);
         float Gc = 0.f, Gs = 0.f, Hc = 0.f, Hs = 0.f;
 #pragma unroll 4
         for (int l = 0; l < nRs3; ++l) {
@@ -812,34 +867,32 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
             Hc = fmaf(gc, de, Hc);
             Hs = fmaf(gs, de, Hs);
         }
-        Hc *= hfac;
-        Hs *= hfac;
-        const float S0 = Gc * t.cosT + Gs * t.sinT;
-        const float S1 = 0.5f * (Hc * t.cosT + Hs * t.sinT);                      // d rho/da = d rho/db = 1/2
-        const float Sth = (Gc * t.sinT - Gs * t.cosT) * t.guard_inv;               // multiplies d cos_i
-        const float Ea = zeta2 * (d.Ka * S0 + d.K * (S1 + Sth * d.cia));
-        const float Eb = zeta2 * (d.Kb * S0 + d.K * (S1 + Sth * d.cib));
-        const float Ec = zeta2 * (d.Kc * S0 + d.K * (Sth * d.cic));
-        const float ia = frcp(t.a), ib = frcp(t.b);
-        const float uax = s.dx[j] * ia, uay = s.dy[j] * ia, uaz = s.dz[j] * ia;   // u_ij
-        const float ubx = s.dx[k] * ib, uby = s.dy[k] * ib, ubz = s.dz[k] * ib;   // u_ik
-        gix += Ea * uax + Eb * ubx;
-        giy += Ea * uay + Eb * uby;
-        giz += Ea * uaz + Eb * ubz;
+        const float S0 = Gc * cosT + Gs * sinT;
+        const float S1 = 0.5f * hfac * (Hc * cosT + Hs * sinT);                   // d rho/da = d rho/db = 1/2
+        const float Sth = (Gc * sinT - Gs * cosT) * guard_inv;                     // multiplies d cos_i
+        // d cos_i / d distance: 1/b - cos_i / a, 1/a - cos_i / b, -c / (a b)
+        const float ea = Z * ia * fmaf(ka, S0, FP * fmaf(Sth, fmaf(-ci, ia, ib), S1));   // (d L / d a) / a
+        const float eb = Z * ib * fmaf(kb, S0, FP * fmaf(Sth, fmaf(-ci, ib, ia), S1));
+        const float ec = Z * ic * fmaf(kc, S0, -FP * Sth * c * w);
+        gix = fmaf(ea, Aj.x, fmaf(eb, Ak.x, gix));
+        giy = fmaf(ea, Aj.y, fmaf(eb, Ak.y, giy));
+        giz = fmaf(ea, Aj.z, fmaf(eb, Ak.z, giz));
+        const float tjx = fmaf(ec, cx, -ea * Aj.x), tjy = fmaf(ec, cy, -ea * Aj.y), tjz = fmaf(ec, cz, -ea * Aj.z);
+        const float tkx = fmaf(-ec, cx, -eb * Ak.x), tky = fmaf(-ec, cy, -eb * Ak.y), tkz = fmaf(-ec, cz, -eb * Ak.z);
         if constexpr (TABLE) {
-            tab[0 * ntrip + tt] = -Ea * uax + Ec * t.ujk[0];
-            tab[1 * ntrip + tt] = -Ea * uay + Ec * t.ujk[1];
-            tab[2 * ntrip + tt] = -Ea * uaz + Ec * t.ujk[2];
-            tab[3 * ntrip + tt] = -Eb * ubx - Ec * t.ujk[0];
-            tab[4 * ntrip + tt] = -Eb * uby - Ec * t.ujk[1];
-            tab[5 * ntrip + tt] = -Eb * ubz - Ec * t.ujk[2];
+            tab[0 * ntrip + tt] = tjx;
+            tab[1 * ntrip + tt] = tjy;
+            tab[2 * ntrip + tt] = tjz;
+            tab[3 * ntrip + tt] = tkx;
+            tab[4 * ntrip + tt] = tky;
+            tab[5 * ntrip + tt] = tkz;
         } else {
-            atomicAdd(&sgx[j], -Ea * uax + Ec * t.ujk[0]);
-            atomicAdd(&sgy[j], -Ea * uay + Ec * t.ujk[1]);
-            atomicAdd(&sgz[j], -Ea * uaz + Ec * t.ujk[2]);
-            atomicAdd(&sgx[k], -Eb * ubx - Ec * t.ujk[0]);
-            atomicAdd(&sgy[k], -Eb * uby - Ec * t.ujk[1]);
-            atomicAdd(&sgz[k], -Eb * ubz - Ec * t.ujk[2]);
+            atomicAdd(&sgx[j], tjx);
+            atomicAdd(&sgy[j], tjy);
+            atomicAdd(&sgz[j], tjz);
+            atomicAdd(&sgx[k], tkx);
+            atomicAdd(&sgy[k], tky);
+            atomicAdd(&sgz[k], tkz);
         }
     }
     __syncthreads();
@@ -869,11 +922,11 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
                 sum += tj[idx];
                 idx += k;
             }
-            atomicAdd(&gm[s.j[x] * 3 + c], sum);
+            atomicAdd(&gm[sj[x] * 3 + c], sum);
         }
     } else {
         for (int j = lane; j < nn; j += QMLL_WAVE) {
-            const int jj = s.j[j];
+            const int jj = sj[j];
             atomicAdd(&gm[jj * 3 + 0], sgx[j]);
             atomicAdd(&gm[jj * 3 + 1], sgy[j]);
             atomicAdd(&gm[jj * 3 + 2], sgz[j]);
@@ -1220,15 +1273,17 @@ extern "C" int qmll_fchl19_forward(const float* X, const int* types, const float
     QMLL_REQUIRE(prm->nRs3 <= 256, QMLL_ERR_INVALID,
                  "qmll_fchl19_forward: nRs3=%d: at most 256 three-body radial bins are supported", prm->nRs3);
     const int R = prm->nspecies * prm->nRs2 + prm->nspecies * (prm->nspecies + 1) * prm->nRs3;
-    // table for every triple of a full neighbourhood when that stays small
-    const long long alltrip = (long long)a.cap * (a.cap - 1) / 2;
-    a.tcap = alltrip <= TCH ? TCH : (alltrip <= TCH_MAX ? (int)alltrip : TCH);
+    // table for every triple of a full neighbourhood when that stays small: an atom has at most cap
+    // neighbours from a given list and at most max_atoms - 1 otherwise
+    const long long maxnn = nlist ? a.cap : (a.cap > 1 ? a.cap - 1 : 1);
+    const long long alltrip = maxnn * (maxnn - 1) / 2;
+    a.tcap = alltrip <= TCH_MAX ? (int)(alltrip > 0 ? alltrip : 1) : TCH;
     // each of the ns (ns+1)/2 segments is padded to a multiple of the triple sub-slot count
     const int tsub_slots = prm->nRs3 < 64 ? 64 / prm->nRs3 : 1;
     a.tpad = prm->nspecies * (prm->nspecies + 1) / 2 * (tsub_slots - 1);
-    // triple table, neighbour arrays + type offsets, three per-neighbour records [cap][4] (behind up
-    // to 3 floats of alignment), the radial grids, the table's segment starts
-    const size_t lds = sizeof(float) * ((size_t)(STAGE_ARRAYS + 12) * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 +
+    // triple table, three per-neighbour records [cap][4], type offsets, the radial grids, the table's
+    // segment starts and lengths
+    const size_t lds = sizeof(float) * ((size_t)12 * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 +
                                         4 * (size_t)(a.tcap + a.tpad) + 2 * (size_t)prm->nspecies * prm->nspecies + 4);
     QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
                  "qmll_fchl19_forward: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R, LDS_LIMIT);
@@ -1249,11 +1304,14 @@ extern "C" int qmll_fchl19_vjp(const float* X, const int* types, const float* ce
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(grad_rep && grad_X, QMLL_ERR_INVALID, "qmll_fchl19_vjp: null gradient pointer");
     const int R = prm->nspecies * prm->nRs2 + prm->nspecies * (prm->nspecies + 1) * prm->nRs3;
-    size_t lds = sizeof(float) * ((size_t)(STAGE_ARRAYS + 3) * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 + R);
+    // two records [cap][4], atom indices, neighbour gradients [3][cap], type offsets, grids, the gradient row
+    size_t lds = sizeof(float) * ((size_t)12 * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 + R);
     QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
                  "qmll_fchl19_vjp: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R, LDS_LIMIT);
-    // per-triple force table [6][cap (cap-1) / 2] while it stays small; LDS atomics beyond
-    const size_t table = sizeof(float) * 6 * ((size_t)a.cap * (a.cap - 1) / 2);
+    // per-triple force table [6][maxnn (maxnn-1) / 2] while it stays small; LDS atomics beyond.  An atom has
+    // at most cap neighbours from a given list and at most max_atoms - 1 otherwise
+    const size_t maxnn = nlist ? (size_t)a.cap : (size_t)(a.cap > 1 ? a.cap - 1 : 1);
+    const size_t table = sizeof(float) * 6 * (maxnn * (maxnn - 1) / 2);
     if (table <= 16 * 1024 && lds + table <= LDS_LIMIT) {
         lds += table;
         hipLaunchKernelGGL(fchl19_vjp_kernel<true>, dim3(A), dim3(64), lds, (hipStream_t)stream, a, grad_rep, grad_X);
