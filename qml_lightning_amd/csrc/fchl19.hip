@@ -697,7 +697,7 @@ __device__ __forceinline__ TripleDeriv triple_derivatives(const Triple& t, const
 // ---------------------------------------------------------------------------------
 // VJP
 // ---------------------------------------------------------------------------------
-// TABLE: the per-triple forces on the two neighbours go to an LDS table [6][ntrip] and are
+// TABLE: the three force coefficients of a triple go to an LDS table [3][ntrip] and are
 // summed per neighbour afterwards (each triple index is computed, never searched), instead
 // of LDS atomics, which serialise badly here: the 64 triples of a pass share 3-4 values of j.
 template <bool TABLE>
@@ -724,7 +724,7 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
     float* sinvRs2 = slnRs2 + nRs2;  // [nRs2]
     float* sRs3 = sinvRs2 + nRs2;    // [nRs3]
     float* gin = sRs3 + nRs3;        // [R]
-    float* tab = gin + R;            // TABLE: [6][ntrip]
+    float* tab = gin + R;            // TABLE: [3][ntrip]
     const float4* rA = reinterpret_cast<const float4*>(recA);
     const float4* rB = reinterpret_cast<const float4*>(recB);
 
@@ -877,22 +877,19 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
         gix = fmaf(ea, Aj.x, fmaf(eb, Ak.x, gix));
         giy = fmaf(ea, Aj.y, fmaf(eb, Ak.y, giy));
         giz = fmaf(ea, Aj.z, fmaf(eb, Ak.z, giz));
-        const float tjx = fmaf(ec, cx, -ea * Aj.x), tjy = fmaf(ec, cy, -ea * Aj.y), tjz = fmaf(ec, cz, -ea * Aj.z);
-        const float tkx = fmaf(-ec, cx, -eb * Ak.x), tky = fmaf(-ec, cy, -eb * Ak.y), tkz = fmaf(-ec, cz, -eb * Ak.z);
         if constexpr (TABLE) {
-            tab[0 * ntrip + tt] = tjx;
-            tab[1 * ntrip + tt] = tjy;
-            tab[2 * ntrip + tt] = tjz;
-            tab[3 * ntrip + tt] = tkx;
-            tab[4 * ntrip + tt] = tky;
-            tab[5 * ntrip + tt] = tkz;
+            // force on j: ec d_ik - (ec + ea) d_ij, on k: ec d_ij - (eb + ec) d_ik; the three
+            // coefficients go to the table, the products are formed when a neighbour's triples are summed
+            tab[0 * ntrip + tt] = ec + ea;
+            tab[1 * ntrip + tt] = eb + ec;
+            tab[2 * ntrip + tt] = ec;
         } else {
-            atomicAdd(&sgx[j], tjx);
-            atomicAdd(&sgy[j], tjy);
-            atomicAdd(&sgz[j], tjz);
-            atomicAdd(&sgx[k], tkx);
-            atomicAdd(&sgy[k], tky);
-            atomicAdd(&sgz[k], tkz);
+            atomicAdd(&sgx[j], fmaf(ec, cx, -ea * Aj.x));
+            atomicAdd(&sgy[j], fmaf(ec, cy, -ea * Aj.y));
+            atomicAdd(&sgz[j], fmaf(ec, cz, -ea * Aj.z));
+            atomicAdd(&sgx[k], fmaf(-ec, cx, -eb * Ak.x));
+            atomicAdd(&sgy[k], fmaf(-ec, cy, -eb * Ak.y));
+            atomicAdd(&sgz[k], fmaf(-ec, cz, -eb * Ak.z));
         }
     }
     __syncthreads();
@@ -906,23 +903,32 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
         atomicAdd(&gm[i * 3 + 2], giz);
     }
     if constexpr (TABLE) {
-        // lane = (neighbour x, component c).  Triple (j,k) sits at k (k - 1) / 2 + j: the triples
-        // (j,x) with x second are the run of x entries starting at x (x - 1) / 2; the triples (x,k)
-        // with x first sit at k (k - 1) / 2 + x for k = x+1 .. nn-1, k entries further each step
+        // lane = (neighbour x, component c).  The force on x is sum_y ec(x,y) d_iy - d_ix s_x with s_x
+        // the sum of its own coefficients.  Triple (j,k) sits at k (k - 1) / 2 + j: the triples (j,x)
+        // with x second are the run of x entries starting at x (x - 1) / 2; the triples (x,k) with x
+        // first sit at k (k - 1) / 2 + x for k = x+1 .. nn-1, k entries further each step
         for (int it = lane; it < 3 * nn; it += QMLL_WAVE) {
             const int x = idiv_small(it, 3), c = it - 3 * x;
             float sum = c == 0 ? sgx[x] : (c == 1 ? sgy[x] : sgz[x]);
-            const float* tk = tab + (3 + c) * ntrip + (x * (x - 1)) / 2;
+            float own = 0.0f;
+            const float* dc = recA + c;                       // component c of d_iy at dc[4 y]
+            const float* e1 = tab + 1 * ntrip + (x * (x - 1)) / 2;
+            const float* e2 = e1 + ntrip;
 #pragma unroll 4
-            for (int q = 0; q < x; ++q) sum += tk[q];
-            const float* tj = tab + c * ntrip + x;
+            for (int q = 0; q < x; ++q) {
+                sum = fmaf(e2[q], dc[4 * q], sum);
+                own += e1[q];
+            }
+            const float* e0 = tab + x;
+            const float* e2b = e0 + 2 * ntrip;
             int idx = ((x + 1) * x) / 2;
 #pragma unroll 4
             for (int k = x + 1; k < nn; ++k) {
-                sum += tj[idx];
+                sum = fmaf(e2b[idx], dc[4 * k], sum);
+                own += e0[idx];
                 idx += k;
             }
-            atomicAdd(&gm[sj[x] * 3 + c], sum);
+            atomicAdd(&gm[sj[x] * 3 + c], fmaf(-dc[4 * x], own, sum));
         }
     } else {
         for (int j = lane; j < nn; j += QMLL_WAVE) {
@@ -1308,10 +1314,10 @@ extern "C" int qmll_fchl19_vjp(const float* X, const int* types, const float* ce
     size_t lds = sizeof(float) * ((size_t)12 * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 + R);
     QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
                  "qmll_fchl19_vjp: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R, LDS_LIMIT);
-    // per-triple force table [6][maxnn (maxnn-1) / 2] while it stays small; LDS atomics beyond.  An atom has
+    // per-triple coefficient table [3][maxnn (maxnn-1) / 2] while it stays small; LDS atomics beyond.  An atom has
     // at most cap neighbours from a given list and at most max_atoms - 1 otherwise
     const size_t maxnn = nlist ? (size_t)a.cap : (size_t)(a.cap > 1 ? a.cap - 1 : 1);
-    const size_t table = sizeof(float) * 6 * (maxnn * (maxnn - 1) / 2);
+    const size_t table = sizeof(float) * 3 * (maxnn * (maxnn - 1) / 2);
     if (table <= 16 * 1024 && lds + table <= LDS_LIMIT) {
         lds += table;
         hipLaunchKernelGGL(fchl19_vjp_kernel<true>, dim3(A), dim3(64), lds, (hipStream_t)stream, a, grad_rep, grad_X);
