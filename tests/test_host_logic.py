@@ -165,9 +165,9 @@ def test_model_species_for_the_element_sort():
 
 def test_closed_form_pair_unranking_is_exact():
     """The FCHL19 kernels number the pairs j < k of a neighbour list k-major, t = k (k - 1) / 2 + j,
-    and recover (j, k) from t in fp32: k = floor((1 + sqrt(8 t + 1)) / 2) from a 1-ulp square root,
-    corrected by one comparison either way (csrc/fchl19.hip, unrank_pair_kmajor).  Emulated here in
-    fp32 with the square root pushed one ulp either way, for every t below 2^20."""
+    and recover (j, k) from t in fp32 with no correction step: k = int(1/2 + sqrt(2 t + 1.25)),
+    j = t - k (k - 1) / 2 (csrc/fchl19.hip, unrank_pair_kmajor).  Emulated here in fp32 with the
+    square root pushed up to two ulps either way, for every t below 2^20."""
     t = np.arange(0, 1 << 20, dtype=np.int64)
     tf = t.astype(np.float32)
     kk = ((1 + np.sqrt(1 + 8 * t.astype(np.float64))) // 2).astype(np.int64)
@@ -176,14 +176,9 @@ def test_closed_form_pair_unranking_is_exact():
     jj = t - kk * (kk - 1) // 2
     assert (jj >= 0).all() and (jj < kk).all()
     f32 = np.float32
-    for push in (-1, 0, 1):
-        sq = np.sqrt((f32(8) * tf + f32(1)).astype(np.float32)).astype(np.float32)
-        if push:
+    for push in (-2, -1, 0, 1, 2):
+        sq = np.sqrt((f32(2) * tf + f32(1.25)).astype(np.float32)).astype(np.float32)
+        for _ in range(abs(push)):
             sq = np.nextafter(sq, f32(np.inf if push > 0 else -np.inf)).astype(np.float32)
-        kf = np.floor(f32(0.5) + f32(0.5) * sq).astype(np.float32)
-        tri = (f32(0.5) * (kf * kf - kf)).astype(np.float32)
-        kf = kf - (tri > tf)
-        tri = (f32(0.5) * (kf * kf - kf)).astype(np.float32)
-        up = (tri + kf <= tf).astype(np.float32)
-        tri, kf = tri + up * kf, kf + up
-        assert np.array_equal(kf.astype(np.int64), kk) and np.array_equal((tf - tri).astype(np.int64), jj), push
+        k = (f32(0.5) + sq).astype(np.float32).astype(np.int64)       # conversion truncates
+        assert np.array_equal(k, kk) and np.array_equal(t - k * (k - 1) // 2, jj), push
