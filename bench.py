@@ -195,6 +195,55 @@ def other_configs(torch, dev):
     del m5
     torch.cuda.empty_cache()
     out["config5_sorf_32768"] = predict_rate(sorf_model(SPECIES, 128, 256, 500), coords, charges, True)
+    # one C9H8O4 molecule with the config-2 model: the latency of the step's chain of dependent launches,
+    # eager, through forward + autograd.grad, and replayed from a captured HIP graph (each replay checked)
+    m2 = sorf_model(SPECIES, NPCAS, NSTACKS, 500)
+    one = predict_rate(m2, coords[:1], charges[:1], True, steps=200, warm=20)
+    data = m2.format_data([coords[0].astype(np.float32)], charges[:1])
+    X, Z = data['coordinates'], data['charges']
+    aid, mid, nat = data['atomIDs'], data['molIDs'], data['natom_counts']
+
+    def autograd_step():
+        Xg = X.detach().requires_grad_(True)
+        E = m2.forward(Xg, Z, aid, mid, nat)
+        return E, torch.autograd.grad(-E.sum(), Xg)[0]
+    for _ in range(20):
+        autograd_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(200):
+        autograd_step()
+    torch.cuda.synchronize()
+    one["autograd_ms_per_step"] = (time.perf_counter() - t0) / 200 * 1e3
+    Xs = X.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            m2.energies_and_forces(Xs, Z, aid, mid, nat, forces=True)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        Eg, Fg = m2.energies_and_forces(Xs, Z, aid, mid, nat, forces=True)
+    ok = True
+    for it in range(4):      # replays with changed inputs, eager work and synchronisations between them
+        Xp = X + 0.01 * it
+        Ee, Fe = m2.energies_and_forces(Xp, Z, aid, mid, nat, forces=True)
+        torch.cuda.synchronize()
+        Xs.copy_(Xp)
+        graph.replay()
+        torch.cuda.synchronize()
+        ok = ok and bool(torch.equal(Eg, Ee)) and bool((Fg - Fe).abs().max() <= 1e-5 * Fe.abs().max())
+    for _ in range(20):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(200):
+        graph.replay()
+    torch.cuda.synchronize()
+    one["graph_replay_ms_per_step"] = (time.perf_counter() - t0) / 200 * 1e3
+    one["graph_replays_match_eager"] = ok
+    out["one_molecule_c9h8o4"] = one
     return out
 
 
