@@ -316,6 +316,54 @@ def test_kernels_follow_the_current_stream():
     assert (f0 - f1).abs().max() <= 1e-6 * f0.abs().max()
 
 
+@pytest.mark.parametrize("kind", ["sorf", "rff"])
+def test_predict_step_replayed_from_a_captured_graph(kind):
+    """The predict step allocates only through torch and records no memset nodes, so it can be captured
+    in a HIP graph.  The graph is replayed five times with changed coordinates, with the program's own
+    eager work and synchronisations between the replays, and every replay is checked against the eager
+    result of the same coordinates (SORF energies bit-equal: they are summed in a fixed order; the RFF
+    kernel adds its feature shares with fp32 atomics; forces to the rounding of the atomic scatters)."""
+    species = [1, 6, 8]
+    coords, charges = helpers.fixed_composition_batch(helpers.ASPIRIN, 3, 1)
+    if kind == "sorf":
+        m, _ = build_sorf_model(species, 128, 8)
+    else:
+        from qml_lightning_amd.models.random_features import RandomFourrierFeaturesModel
+        from qml_lightning_amd.representations.FCHL import FCHLCuda
+        rep = FCHLCuda(species=np.array(species))
+        np.random.seed(3)
+        m = RandomFourrierFeaturesModel(rep=rep, elements=np.array(species), sigma=3.0, llambda=1e-5, npcas=64,
+                                        nstacks=4, nbatch_train=4, nbatch_test=5)
+        red, _, _, alpha = helpers.model_weights(len(species), rep.get_repsize(), 64, 4)
+        m.reductors = t32(red)
+        m.alpha = torch.tensor(alpha, device=dev())
+        m.is_trained = True
+    X, Z, aid, mid, nat = inputs(*make_batch(coords, charges))
+    Xs = X.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            m.energies_and_forces(Xs, Z, aid, mid, nat)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        eg, fg = m.energies_and_forces(Xs, Z, aid, mid, nat)
+    for it in range(5):
+        Xp = X + 0.02 * it
+        ee, fe = m.energies_and_forces(Xp, Z, aid, mid, nat)      # eager work between the replays
+        torch.cuda.synchronize()
+        Xs.copy_(Xp)
+        graph.replay()
+        torch.cuda.synchronize()
+        if kind == "sorf":
+            assert torch.equal(eg, ee), (kind, it)
+        else:
+            assert (eg - ee).abs().max() <= 1e-6 * ee.abs().max(), (kind, it)
+        assert (fg - fe).abs().max() <= 1e-5 * fe.abs().max(), (kind, it)
+    assert not torch.equal(fe, m.energies_and_forces(X, Z, aid, mid, nat)[1])   # the inputs did change the result
+
+
 def test_reductor_fit_matches_an_svd_of_the_samples():
     """get_reductors (kernel.py:447-540): per element the leading left singular vectors of the
     sampled representations; here via the Gram matrix and an eigensolve, checked against numpy's SVD."""
