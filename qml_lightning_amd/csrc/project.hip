@@ -376,6 +376,85 @@ __global__ __launch_bounds__(256) void zero_untyped_rows_kernel(const int* __res
     }
 }
 
+// Small batches (a molecule or a few): the tiled kernels above run one or two workgroups through
+// ten dependent load-and-multiply steps, 17-26 us for 21 atoms.  Here a workgroup takes ONE atom and
+// spreads the contraction over its threads, so all loads of an atom are in flight at once.
+constexpr int SMALL_ATOMS = 128;   // above, the reductor re-reads from L2 (R d floats per atom) outweigh the latency
+constexpr int SMALL_KS = 8;        // slices of the contraction in project_small_kernel
+
+__device__ __forceinline__ int type_of_position(const int* __restrict__ type_offsets, int ne, int p) {
+    int e = 0;
+    while (e + 1 < ne && p >= type_offsets[e + 1]) ++e;
+    return e;
+}
+
+// x[p, :] = rep[slot(p), :] . U_e: thread = (contraction slice, four columns), slices folded through LDS
+__global__ __launch_bounds__(256) void project_small_kernel(const float* __restrict__ rep,
+                                                            const int* __restrict__ sorted_slots,
+                                                            const int* __restrict__ type_offsets,
+                                                            const float* __restrict__ reductors, int ne, int R, int d,
+                                                            float* __restrict__ x) {
+    extern __shared__ float sm[];
+    float* srow = sm;                                  // [R]
+    float* spart = sm + ((R + 3) & ~3);                // [SMALL_KS][d]
+    const int p = blockIdx.x, tid = threadIdx.x;
+    if (p >= type_offsets[ne]) return;                 // past the sorted list (atoms of no known element)
+    const int e = type_of_position(type_offsets, ne, p);
+    const float* row = rep + (size_t)sorted_slots[p] * R;
+    for (int k = tid; k < R; k += 256) srow[k] = row[k];
+    __syncthreads();
+    const float* U = reductors + (size_t)e * R * d;
+    const int ks = tid >> 5, l32 = tid & 31;
+    for (int c4 = l32; c4 < d / 4; c4 += 32) {
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 8
+        for (int k = ks; k < R; k += SMALL_KS) {
+            const float4 u = *reinterpret_cast<const float4*>(U + (size_t)k * d + 4 * c4);
+            const float r = srow[k];
+            acc.x = fmaf(r, u.x, acc.x);
+            acc.y = fmaf(r, u.y, acc.y);
+            acc.z = fmaf(r, u.z, acc.z);
+            acc.w = fmaf(r, u.w, acc.w);
+        }
+        *reinterpret_cast<float4*>(spart + ks * d + 4 * c4) = acc;
+    }
+    __syncthreads();
+    for (int c = tid; c < d; c += 256) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int q = 0; q < SMALL_KS; ++q) sum += spart[q * d + c];
+        x[(size_t)p * d + c] = sum;
+    }
+}
+
+// g_rep[slot(p), :] = gx[p, :] . U_e^T: thread = output entry r, its reductor row is contiguous
+__global__ __launch_bounds__(256) void project_bt_small_kernel(const float* __restrict__ gx,
+                                                               const int* __restrict__ sorted_slots,
+                                                               const int* __restrict__ type_offsets,
+                                                               const float* __restrict__ reductors, int ne, int R, int d,
+                                                               float* __restrict__ g_rep) {
+    extern __shared__ float sm[];                      // [d]
+    const int p = blockIdx.x, tid = threadIdx.x;
+    if (p >= type_offsets[ne]) return;                 // past the sorted list (atoms of no known element)
+    const int e = type_of_position(type_offsets, ne, p);
+    for (int c = tid; c < d; c += 256) sm[c] = gx[(size_t)p * d + c];
+    __syncthreads();
+    const float* U = reductors + (size_t)e * R * d;
+    float* out = g_rep + (size_t)sorted_slots[p] * R;
+    const float4* g4 = reinterpret_cast<const float4*>(sm);
+    for (int r = tid; r < R; r += 256) {
+        const float4* u4 = reinterpret_cast<const float4*>(U + (size_t)r * d);
+        float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll 8
+        for (int c4 = 0; c4 < d / 4; ++c4) {
+            const float4 u = u4[c4], g = g4[c4];
+            a0 = fmaf(u.x, g.x, fmaf(u.y, g.y, a0));
+            a1 = fmaf(u.z, g.z, fmaf(u.w, g.w, a1));
+        }
+        out[r] = a0 + a1;
+    }
+}
+
 __global__ void zero_ints_kernel(int* __restrict__ p, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0;
@@ -474,6 +553,15 @@ extern "C" int qmll_project_typed(const float* rep, const int* sorted_slots, con
     QMLL_REQUIRE(rep && sorted_slots && type_offsets && reductors && x, QMLL_ERR_INVALID,
                  "qmll_project_typed: null pointer");
     const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(rep) && aligned16(reductors);
+    if (vec && A <= SMALL_ATOMS) {
+        const size_t lds = sizeof(float) * (((size_t)R + 3) / 4 * 4 + (size_t)SMALL_KS * d);
+        if (lds <= 64 * 1024) {
+            hipLaunchKernelGGL(project_small_kernel, dim3(A), dim3(256), lds, (hipStream_t)stream, rep, sorted_slots,
+                               type_offsets, reductors, ne, R, d, x);
+            QMLL_CHECK_LAUNCH("qmll_project_typed");
+            return QMLL_OK;
+        }
+    }
     const int tiles = (A + PM - 1) / PM + ne;
     // the wide tile when it wastes no columns and still leaves every CU a few workgroups
     const bool wide = vec && d % 128 == 0 && (long long)tiles * (d / 128) >= 2 * 256;
@@ -507,7 +595,10 @@ extern "C" int qmll_project_typed_backward(const float* gx, const int* sorted_sl
                  "qmll_project_typed_backward: null pointer");
     const dim3 grid((A + PM - 1) / PM + ne, (R + PN - 1) / PN);
     const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(gx) && aligned16(reductors);
-    if (vec && (d == 64 || d == 128)) {
+    if (vec && A <= SMALL_ATOMS && (size_t)d * sizeof(float) <= 64 * 1024) {
+        hipLaunchKernelGGL(project_bt_small_kernel, dim3(A), dim3(256), sizeof(float) * d, (hipStream_t)stream, gx,
+                           sorted_slots, type_offsets, reductors, ne, R, d, g_rep);
+    } else if (vec && (d == 64 || d == 128)) {
         // short contraction: the gradient rows stay in registers, every row is read once
         const dim3 g1((A + PM - 1) / PM + ne);
         if (d == 128)

@@ -562,8 +562,10 @@ constexpr int ROWS_NA = 4;   // atoms per workgroup = rows of 16 lanes per wavef
 
 // MULTI: more than one transform per stack (T > 1); the first sign diagonal stays in registers
 // as for T = 1, the later ones are fetched where they are used (forward and again in the adjoint).
-template <int LOG2D, bool WITH_GRAD, bool MULTI>
-__global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
+// NW: wavefronts per workgroup, which share out the stacks (16 for a few atoms: a molecule then takes
+// a quarter of the time, its stacks being the only parallelism there is).
+template <int LOG2D, bool WITH_GRAD, bool MULTI, int NW = SORF_WAVES>
+__global__ __launch_bounds__(64 * NW) void sorf_energy_rows_kernel(
     const float* __restrict__ x, const float* __restrict__ D, const float* __restrict__ bias,
     const float* __restrict__ alpha, const int* __restrict__ out_index, const int* __restrict__ type_offsets, int ne,
     int A, int S, int T_, float scale, float normf, float* __restrict__ e_atom, float* __restrict__ gx) {
@@ -572,8 +574,8 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
     constexpr int EPL = d / 16;                 // registers per lane
     constexpr int NA = ROWS_NA;
     static_assert(EPL >= 4 && EPL % 4 == 0, "groups of four butterfly chains per lane");
-    __shared__ float red[SORF_WAVES][NA][d];
-    __shared__ float ered[SORF_WAVES][NA];
+    __shared__ float red[NW][NA][d];
+    __shared__ float ered[NW][NA];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
@@ -689,20 +691,20 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
                 const size_t off = (size_t)s * d + e0;               // the same for the four rows
                 load_row<EPL>(bv, bias + off);
                 load_row<EPL>(av, alpha + off);
-                load_row<EPL>(d1, D + (size_t)(s + SORF_WAVES < S ? s + SORF_WAVES : s) * d + e0);
+                load_row<EPL>(d1, D + (size_t)(s + NW < S ? s + NW : s) * d + e0);
                 stack(d0, bv, av);
             }
-            s += SORF_WAVES;
+            s += NW;
             if (s >= S) break;
             {
                 float bv[EPL], av[EPL];
                 const size_t off = (size_t)s * d + e0;
                 load_row<EPL>(bv, bias + off);
                 load_row<EPL>(av, alpha + off);
-                load_row<EPL>(d0, D + (size_t)(s + SORF_WAVES < S ? s + SORF_WAVES : s) * d + e0);
+                load_row<EPL>(d0, D + (size_t)(s + NW < S ? s + NW : s) * d + e0);
                 stack(d1, bv, av);
             }
-            s += SORF_WAVES;
+            s += NW;
         }
         energy = row_sum(energy);
         if (i16 == 0) ered[wave][row] = energy;
@@ -717,12 +719,12 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
     float dv[EPL], bv[EPL], av[EPL];
     int s = wave;
     if (s < S) load_row<EPL>(dv, D + (size_t)s * d + e0);
-    for (; s < S; s += SORF_WAVES) {
+    for (; s < S; s += NW) {
         const size_t off = (size_t)s * d + e0;               // the same for the four rows
         load_row<EPL>(bv, bias + off);
         load_row<EPL>(av, alpha + off);
         float dn[EPL];
-        load_row<EPL>(dn, D + (size_t)(s + SORF_WAVES < S ? s + SORF_WAVES : s) * d + e0);
+        load_row<EPL>(dn, D + (size_t)(s + NW < S ? s + NW : s) * d + e0);
 
         float v[EPL];
 #pragma unroll
@@ -794,17 +796,17 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_rows_kernel(
     if (threadIdx.x < rows) {
         float t = 0.0f;
 #pragma unroll
-        for (int w = 0; w < SORF_WAVES; ++w) t += ered[w][threadIdx.x];
+        for (int w = 0; w < NW; ++w) t += ered[w][threadIdx.x];
         const int a = row0 + threadIdx.x;
         e_atom[out_index ? out_index[a] : a] = normf * t;
     }
     if constexpr (WITH_GRAD) {
         const float gscale = -scale * normf;
-        for (int e = threadIdx.x; e < rows * d; e += SORF_THREADS) {
+        for (int e = threadIdx.x; e < rows * d; e += 64 * NW) {
             const int j = e / d, c = e % d;
             float t = 0.0f;
 #pragma unroll
-            for (int w = 0; w < SORF_WAVES; ++w) t += red[w][j][c];
+            for (int w = 0; w < NW; ++w) t += red[w][j][c];
             gx[(size_t)(row0 + j) * d + c] = gscale * t;
         }
     }
@@ -1565,14 +1567,21 @@ static int launch_fused(const char* who, const float* x, const float* D, const f
         // 4 to 16 registers per lane, atoms groupable by element: the instruction-lean kernel
         // (four atoms per workgroup)
         const dim3 grid((A + ROWS_NA - 1) / ROWS_NA + (type_offsets ? ne : 0));
+        // a few atoms: sixteen wavefronts per workgroup share out the stacks
+        const bool few = A <= 256 && S >= 64 && d <= 128 && T == 1;
 #define LAUNCH_ROWS(L, G, M)                                                                                       \
-    hipLaunchKernelGGL((sorf_energy_rows_kernel<L, G, M>), grid, dim3(SORF_THREADS), 0, stream, x, D, bias, alpha, \
-                       out_index, type_offsets, ne, A, S, T, scale, normf, e_atom, gx)
-#define CALL_ROWS(L)                                  \
-    if (gx && T == 1) LAUNCH_ROWS(L, true, false);    \
-    else if (gx) LAUNCH_ROWS(L, true, true);          \
-    else if (T == 1) LAUNCH_ROWS(L, false, false);    \
-    else LAUNCH_ROWS(L, false, true)
+    if (few && !(M))                                                                                               \
+        hipLaunchKernelGGL((sorf_energy_rows_kernel<L, G, false, ((L) <= 7 ? 16 : SORF_WAVES)>), grid, dim3(1024), \
+                           0, stream, x, D, bias,                                                                  \
+                           alpha, out_index, type_offsets, ne, A, S, T, scale, normf, e_atom, gx);                 \
+    else                                                                                                           \
+        hipLaunchKernelGGL((sorf_energy_rows_kernel<L, G, M>), grid, dim3(SORF_THREADS), 0, stream, x, D, bias,    \
+                           alpha, out_index, type_offsets, ne, A, S, T, scale, normf, e_atom, gx)
+#define CALL_ROWS(L)                                    \
+    if (gx && T == 1) { LAUNCH_ROWS(L, true, false); }  \
+    else if (gx) { LAUNCH_ROWS(L, true, true); }        \
+    else if (T == 1) { LAUNCH_ROWS(L, false, false); }  \
+    else { LAUNCH_ROWS(L, false, true); }
         switch (qmll_log2(d)) {
             case 6: { CALL_ROWS(6); } break;
             case 7: { CALL_ROWS(7); } break;

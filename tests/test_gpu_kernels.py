@@ -448,10 +448,14 @@ def test_sort_by_type_is_a_stable_counting_sort(A, N, ne):
 
 
 @pytest.mark.parametrize("R,d,ne,N,A", [(312, 128, 3, 500, 500), (75, 64, 2, 90, 61), (720, 256, 5, 700, 523),
-                                        (10, 8, 1, 5, 3), (496, 256, 4, 130, 130)])
+                                        (10, 8, 1, 5, 3), (496, 256, 4, 130, 130),
+                                        # up to 128 listed atoms: one workgroup per atom instead of matrix tiles
+                                        (312, 128, 3, 100, 100), (312, 128, 3, 140, 128), (312, 128, 3, 140, 129),
+                                        (312, 64, 2, 40, 21), (720, 256, 5, 60, 33), (76, 20, 2, 30, 17)])
 def test_project_typed_forward_and_backward(R, d, ne, N, A):
-    """Element-sorted projection on the matrix cores against fp64 matmul, both directions:
-    gathered rows, tiles that end inside a type, R not a multiple of 4, unknown elements."""
+    """Element-sorted projection against fp64 matmul, both directions: gathered rows, tiles that end
+    inside a type, R not a multiple of 4, unknown elements; the matrix-core kernels and the
+    one-workgroup-per-atom kernels of small batches."""
     from qml_lightning_amd import ops
     rng = np.random.default_rng(R + d)
     rep = rng.normal(size=(N, R)).astype(np.float32)
@@ -478,13 +482,14 @@ def test_project_typed_forward_and_backward(R, d, ne, N, A):
     assert (g.cpu().numpy()[mask] == 0).all()
 
 
-@pytest.mark.parametrize("T", [1, 2])
-def test_sorted_fused_energy_matches_per_atom_oracle(T):
+@pytest.mark.parametrize("T,S,d", [(1, 6, 64), (2, 6, 64), (1, 64, 128), (1, 70, 64), (2, 64, 64)])
+def test_sorted_fused_energy_matches_per_atom_oracle(T, S, d):
     """Element-sorted rows through the fused kernel: energies land in the atoms' slots, the
-    gradient stays in sorted order, rows past the last known atom give zero."""
+    gradient stays in sorted order, rows past the last known atom give zero.  From 64 stacks on, a
+    batch this small runs with sixteen wavefronts per workgroup sharing out the stacks."""
     from qml_lightning_amd import ops
     rng = np.random.default_rng(19)
-    ne, d, S, N, A = 3, 64, 6, 50, 37
+    ne, N, A = 3, 50, 37
     F = S * d
     types = rng.integers(-1, ne, N).astype(np.int32)
     slots = np.sort(rng.choice(N, size=A, replace=False)).astype(np.int32)
