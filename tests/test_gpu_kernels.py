@@ -74,6 +74,10 @@ CASES = {
                            [1, 6, 8], {}),
     "short_cutoff": lambda: (helpers.fixed_composition_batch(helpers.ASPIRIN, 2, 5), [1, 6, 8],
                              {"rcut": 3.1, "nRs2": 7, "nRs3": 5}),
+    # more radial bins than a wavefront has lanes: several bin blocks per lane, one triple per round
+    "many_bins": lambda: (helpers.fixed_composition_batch(helpers.ASPIRIN, 2, 6), [1, 6, 8], {"nRs2": 80, "nRs3": 70}),
+    # 33 to 64 three-body bins: one triple per round, one bin block
+    "forty_bins": lambda: (helpers.fixed_composition_batch(helpers.ASPIRIN, 1, 7), [1, 6, 8], {"nRs2": 33, "nRs3": 40}),
 }
 
 
