@@ -327,6 +327,17 @@ int qmll_gram_f64(const double* Z, const double* y, int M, int F, double* ZTZ, d
 int qmll_gram_upper_f64(const double* Z, const double* y, int M, int F, double* ZTZ, double* ZTy,
                         qmll_stream_t stream);
 
+/* qmll_gram_upper_f64 with a device workspace of qmll_gram_workspace_bytes() bytes (same part of
+ * kernel.py:190-192).  The tiles run in rounds of one per workgroup slot; when the last round is
+ * less than half full (64 of 8256 tiles at F = 16 384) its tiles are cut into row ranges that fill
+ * the slots, the partial tiles go to the workspace and are added in a fixed order, so the result
+ * stays deterministic (it differs from qmll_gram_upper_f64 by the rounding of that regrouping).
+ * With workspace NULL, fewer bytes, fewer than 2048 rows or a well-filled last round it is
+ * qmll_gram_upper_f64. */
+size_t qmll_gram_workspace_bytes(void);
+int qmll_gram_upper_ws_f64(const double* Z, const double* y, int M, int F, double* ZTZ, double* ZTy,
+                           double* workspace, size_t workspace_bytes, qmll_stream_t stream);
+
 /* ZTZ[j,i] = ZTZ[i,j] for the tiles strictly above the diagonal: completes a matrix built with
  * qmll_gram_upper_f64 (both triangles bit-identical). */
 int qmll_gram_mirror_f64(double* ZTZ, int F, qmll_stream_t stream);

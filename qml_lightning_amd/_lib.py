@@ -63,6 +63,8 @@ PROTOTYPES = {
     "qmll_rff_energy_sorted": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, P, P, P],
     "qmll_gram_f64": [P, P, c_int, c_int, P, P, P],
     "qmll_gram_upper_f64": [P, P, c_int, c_int, P, P, P],
+    "qmll_gram_workspace_bytes": [],
+    "qmll_gram_upper_ws_f64": [P, P, c_int, c_int, P, P, P, c_size_t, P],
     "qmll_gram_mirror_f64": [P, c_int, P],
     "qmll_cholesky_workspace_bytes": [c_int],
     "qmll_cholesky_f64": [P, c_int, c_longlong, P, P, P],
@@ -76,7 +78,8 @@ PROTOTYPES = {
     "qmll_probe_mix": [c_int, c_int, c_int, P, P],
 }
 _RESTYPES = {"qmll_last_error": c_char_p, "qmll_sort_by_type_workspace": c_size_t,
-             "qmll_cholesky_workspace_bytes": c_size_t, "qmll_probe_out_bytes": c_size_t, "qmll_probe_rate": c_double,
+             "qmll_cholesky_workspace_bytes": c_size_t, "qmll_gram_workspace_bytes": c_size_t,
+             "qmll_probe_out_bytes": c_size_t, "qmll_probe_rate": c_double,
              "qmll_probe_mix": c_double}
 
 _lib = None

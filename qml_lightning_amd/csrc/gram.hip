@@ -5,8 +5,9 @@
 // C[i,j] += sum_m Z[m,i] Z[m,j].  Z is row-major [M,F], so for a fixed m both operand
 // fragments are contiguous in memory: the A fragment of v_mfma_f64_16x16x4_f64 (16 rows i
 // x 4 steps k) is Z[m0+k, i0+i] and the B fragment is Z[m0+k, j0+j]; no transpose is
-// ever materialised.  A workgroup (256 threads, 4 wavefronts) owns a 128x128 tile of C;
-// each wavefront keeps a 64x64 sub-tile (4x4 MFMA tiles, 128 accumulator registers) and
+// ever materialised.  A workgroup (512 threads, 8 wavefronts) owns a 128x128 tile of C;
+// each wavefront keeps a 64x32 sub-tile (4x2 MFMA tiles, 64 accumulator registers; four wavefronts
+// per SIMD hold the matrix pipe busier than two with 64x64 sub-tiles did) and
 // the two 128-wide column panels of Z are staged through LDS KB rows at a time with the
 // next panel's global loads in flight during the MFMAs.  In the symmetric mode only tiles
 // on or above the diagonal are computed; the mirror image is copied by a separate pass
@@ -22,7 +23,13 @@ typedef double double2_t __attribute__((ext_vector_type(2)));
 
 constexpr int TILE = 128;     // C tile edge per workgroup
 constexpr int KB = 16;        // rows of Z staged per step
-constexpr int GT = 256;       // threads
+constexpr int NWAVE = 8;      // wavefronts per workgroup: 2 along i x NWAVE/2 along j
+constexpr int GT = 64 * NWAVE;
+constexpr int WJ = NWAVE / 2;            // wavefronts along j
+constexpr int NQ = TILE / WJ / 16;       // 16-column MFMA tiles per wavefront along j (4 along i)
+constexpr int TPR = GT / KB;             // threads per staged row
+constexpr int CPT = TILE / TPR;          // doubles per thread and row
+constexpr int UN = CPT / 2;              // 16-byte units per thread
 // doubles per staged row: 128 + 16, i.e. consecutive rows start 32 banks apart, so the two
 // k-rows a half-wavefront reads in one ds_read_b64 never share a bank
 constexpr int LDS_STRIDE = TILE + 16;
@@ -42,10 +49,16 @@ constexpr int DIAG_TILES = SUPER * (SUPER + 1) / 2;
 struct TileMap {
     int off_per;    // strictly-upper super-tiles per XCD (symmetric) / all super-tiles per XCD
     int diag_per;   // diagonal super-tiles per XCD (symmetric mode only)
+    // split launch of the last tiles (symmetric mode with a workspace, see gram_launch): workgroup w
+    // takes rows [piece * piece_rows, ...) of tile id tail_first + w / pieces, piece = w % pieces, and
+    // writes its partial tile to the workspace; pieces = 0: the ordinary launch
+    int pieces;
+    int piece_rows;
+    unsigned tail_first;
 };
 
 template <bool SYM>
-__device__ __forceinline__ void tile_of_block(unsigned b, int nti, int ntj, TileMap tm, int& ti, int& tj) {
+__host__ __device__ __forceinline__ void tile_of_block(unsigned b, int nti, int ntj, TileMap tm, int& ti, int& tj) {
     const unsigned xcd = b % NXCD, k = b / NXCD;
     const int sr_n = (nti + SUPER - 1) / SUPER, sc_n = (ntj + SUPER - 1) / SUPER;
     ti = tj = -1;
@@ -63,7 +76,7 @@ __device__ __forceinline__ void tile_of_block(unsigned b, int nti, int ntj, Tile
         if (g >= (unsigned)(sc_n * n1 / 2)) return;
         const float bb = (float)(2 * n1 + 1);
         int r = (int)((bb - sqrtf(fmaxf(bb * bb - 8.0f * (float)g, 0.0f))) * 0.5f);
-        r = min(max(r, 0), n1 - 1);
+        r = r < 0 ? 0 : (r > n1 - 1 ? n1 - 1 : r);
         while (r > 0 && (unsigned)(r * n1 - (r * (r - 1)) / 2) > g) --r;
         while (r + 1 < n1 && (unsigned)((r + 1) * n1 - ((r + 1) * r) / 2) <= g) ++r;
         const int sc = r + 1 + (int)(g - (unsigned)(r * n1 - (r * (r - 1)) / 2));
@@ -92,18 +105,35 @@ __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ 
                                                       int nti, int ntj, TileMap tm, double* __restrict__ C,
                                                       long long ldz_, long long ldc_, double sign_,
                                                       const double* __restrict__ Za_, long long lda_, int overwrite_) {
+    unsigned bid = blockIdx.x;
+    const bool split = GEN && tm.pieces > 1;          // one of several row ranges of a tile, to the workspace
+    if (split) {
+        const unsigned piece = bid % (unsigned)tm.pieces;
+        bid = tm.tail_first + bid / (unsigned)tm.pieces;
+        const long long m0 = (long long)piece * tm.piece_rows;
+        const long long left = (long long)M - m0;
+        M = left < 0 ? 0 : (int)(left < tm.piece_rows ? left : tm.piece_rows);
+        if (M > 0) {
+            Z += (size_t)m0 * ldz_;
+            Za_ += (size_t)m0 * lda_;
+        }
+    }
     const long long ldz = GEN ? ldz_ : (long long)F, ldc = GEN ? ldc_ : (long long)F, lda = GEN ? lda_ : (long long)F;
     const double sign = GEN ? sign_ : 1.0;
     const double* __restrict__ Za = GEN ? Za_ : Z;
     const int overwrite = GEN ? overwrite_ : 0;
     // two copies of each staged panel: the next one is written while the current one is read,
-    // one barrier per step (2 x 2 x 18 KB per workgroup, two workgroups per CU)
+    // one barrier per step (2 x 2 x 18 KB per workgroup, two workgroups of eight wavefronts per CU)
     __shared__ __attribute__((aligned(16))) double sA[2][KB][LDS_STRIDE];
     __shared__ __attribute__((aligned(16))) double sB[2][KB][LDS_STRIDE];
 
     int ti, tj;
-    tile_of_block<SYM>(blockIdx.x, nti, ntj, tm, ti, tj);
+    tile_of_block<SYM>(bid, nti, ntj, tm, ti, tj);
     if (ti < 0 || (SYM && ti > tj)) return;
+    if (split && M <= 0) {           // a row range past the end: its partial tile is zero
+        for (int e = threadIdx.x; e < TILE * TILE; e += GT) C[(size_t)blockIdx.x * (TILE * TILE) + e] = 0.0;
+        return;
+    }
     const int i0 = f0 + ti * TILE;   // first feature of the A panel (rows of C)
     const int j0 = tj * TILE;        // first feature of the B panel (columns of C)
     const int ilim = SYM ? F : f1;
@@ -112,20 +142,20 @@ __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ 
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;   // wavefront's 64x64 sub-tile
+    const int wi = (wave / WJ) * 64, wj = (wave % WJ) * (16 * NQ);   // wavefront's 64 x 16 NQ sub-tile
     const int l16 = lane & 15, lk = lane >> 4;
 
-    double4_t acc[4][4];
+    double4_t acc[4][NQ];
 #pragma unroll
     for (int p = 0; p < 4; ++p)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) acc[p][q] = (double4_t){0.0, 0.0, 0.0, 0.0};
+        for (int q = 0; q < NQ; ++q) acc[p][q] = (double4_t){0.0, 0.0, 0.0, 0.0};
 
-    // global -> register staging: KB x 128 doubles per panel = 2048 = 256 threads x 8:
-    // thread t loads row t/16, columns (t%16)*8 .. +8
-    const int lr = tid >> 4;
-    const int lc = (tid & 15) * 8;
-    double2_t ra[4], rb[4];
+    // global -> register staging: KB x 128 doubles per panel = 2048 = 512 threads x 4:
+    // thread t loads row t/32, columns (t%32)*4 .. +4
+    const int lr = tid / TPR;
+    const int lc = (tid % TPR) * CPT;
+    double2_t ra[UN], rb[UN];
     bool loaded_rowok = true;
 
     auto load_panels = [&](int m0) {
@@ -140,16 +170,16 @@ __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ 
             // have been issued, so the zeroing of tail rows happens at the LDS store
             loaded_rowok = rowok;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) ra[q] = pa[q];
+            for (int q = 0; q < UN; ++q) ra[q] = pa[q];
             if (!same) {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) rb[q] = pb[q];
+                for (int q = 0; q < UN; ++q) rb[q] = pb[q];
             }
         } else {
             const double* zr = Z + (size_t)m * ldz;
             const double* zar = Za + (size_t)m * lda;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
+            for (int q = 0; q < UN; ++q) {
                 const int ca = i0 + lc + 2 * q;
                 ra[q].x = (rowok && ca < ilim) ? zar[ca] : 0.0;
                 ra[q].y = (rowok && ca + 1 < ilim) ? zar[ca + 1] : 0.0;
@@ -164,18 +194,18 @@ __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ 
         double2_t* db = reinterpret_cast<double2_t*>(&sB[buf][lr][lc]);
         if (__builtin_expect(loaded_rowok, 1)) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) da[q] = ra[q];
+            for (int q = 0; q < UN; ++q) da[q] = ra[q];
             if (!same) {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) db[q] = rb[q];
+                for (int q = 0; q < UN; ++q) db[q] = rb[q];
             }
         } else {   // a row past the end of Z (last step only) contributes zeros
             const double2_t zero = {0.0, 0.0};
 #pragma unroll
-            for (int q = 0; q < 4; ++q) da[q] = zero;
+            for (int q = 0; q < UN; ++q) da[q] = zero;
             if (!same) {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) db[q] = zero;
+                for (int q = 0; q < UN; ++q) db[q] = zero;
             }
         }
     };
@@ -191,15 +221,15 @@ __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ 
         if (step + 1 < nsteps) load_panels((step + 1) * KB);   // in flight during the MFMAs
 #pragma unroll
         for (int kk = 0; kk < KB; kk += 4) {
-            double fa[4], fb[4];
+            double fa[4], fb[NQ];
 #pragma unroll
             for (int p = 0; p < 4; ++p) fa[p] = pa[kk + lk][wi + p * 16 + l16];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) fb[q] = pb[kk + lk][wj + q * 16 + l16];
+            for (int q = 0; q < NQ; ++q) fb[q] = pb[kk + lk][wj + q * 16 + l16];
 #pragma unroll
             for (int p = 0; p < 4; ++p)
 #pragma unroll
-                for (int q = 0; q < 4; ++q)
+                for (int q = 0; q < NQ; ++q)
                     acc[p][q] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[p], fb[q], acc[p][q], 0, 0, 0);
         }
         // the other copy was last read in the previous step, which every wavefront left
@@ -213,14 +243,16 @@ __global__ __launch_bounds__(GT, 2) void gram_kernel(const double* __restrict__ 
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < NQ; ++q) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int gi = i0 + wi + p * 16 + lk + 4 * r;
                 const int gj = j0 + wj + q * 16 + l16;
                 if (gi < ilim && gj < F) {
                     const double v = sign * acc[p][q][r];
-                    if (SYM) {
+                    if (split) {
+                        C[(size_t)blockIdx.x * (TILE * TILE) + (size_t)(gi - i0) * TILE + (gj - j0)] = v;
+                    } else if (SYM) {
                         C[(size_t)gi * ldc + gj] += v;             // the mirror image is a separate pass
                     } else if (overwrite) {
                         C[(size_t)(gi - f0) * ldc + gj] = v;
@@ -251,6 +283,24 @@ __global__ __launch_bounds__(256) void gram_mirror_kernel(double* __restrict__ C
     for (int r = ty; r < MT; r += 256 / MT) {
         const int gj = bj * MT + r, gi = bi * MT + tx;
         if (gi < F && gj < F) C[(size_t)gj * F + gi] = t[tx][r];
+    }
+}
+
+// C tile += the partial tiles of its row ranges, added in the order of the ranges (split launch of the
+// last tiles of the symmetric mode); one workgroup per tile id from tail_first on
+__global__ __launch_bounds__(256) void gram_tail_reduce_kernel(const double* __restrict__ ws, int nt, TileMap tm, int F,
+                                                                double* __restrict__ C, long long ldc) {
+    int ti, tj;
+    tile_of_block<true>(tm.tail_first + blockIdx.x, nt, nt, tm, ti, tj);
+    if (ti < 0 || ti > tj) return;
+    const double* w = ws + (size_t)blockIdx.x * tm.pieces * (TILE * TILE);
+    for (int e = threadIdx.x; e < TILE * TILE; e += 256) {
+        const int gi = ti * TILE + e / TILE, gj = tj * TILE + e % TILE;
+        if (gi < F && gj < F) {
+            double sum = 0.0;
+            for (int p = 0; p < tm.pieces; ++p) sum += w[(size_t)p * (TILE * TILE) + e];
+            C[(size_t)gi * ldc + gj] += sum;
+        }
     }
 }
 
@@ -296,9 +346,15 @@ __global__ __launch_bounds__(MR* MR) void matmul_and_reduce_kernel(const float* 
 }  // namespace
 
 // Z: M rows of F used columns, row stride ldz; C: row stride ldc; C += sign * Z^T Z
+// bytes of workspace that let the symmetric launch split its last tiles (see below): at most one
+// workgroup slot's worth of partial tiles, ids without a tile included
+constexpr size_t GRAM_WS_TILES = 1024;
+constexpr size_t GRAM_WS_BYTES = GRAM_WS_TILES * TILE * TILE * sizeof(double);
+
 static int gram_launch(const double* Z, const double* y, int M, int F, int f0, int f1, bool sym, bool mirror, double* C,
                        double* ZTy, hipStream_t stream, const char* who, long long ldz = 0, long long ldc = 0,
-                       double sign = 1.0, const double* Za = nullptr, long long lda = 0, int overwrite = 0) {
+                       double sign = 1.0, const double* Za = nullptr, long long lda = 0, int overwrite = 0,
+                       double* ws = nullptr, size_t ws_bytes = 0) {
     if (ldz == 0) ldz = F;
     if (ldc == 0) ldc = F;
     if (!Za) {   // the Gram product: both operands are Z
@@ -327,8 +383,47 @@ static int gram_launch(const double* Z, const double* y, int M, int F, int f0, i
         tm.diag_per = 0;
         per_xcd = (long long)tm.off_per * SUPER * SUPER;
     }
-    const long long nblocks = per_xcd * NXCD;
+    tm.pieces = 0;
+    tm.piece_rows = 0;
+    tm.tail_first = 0;
+    long long nblocks = per_xcd * NXCD;
     QMLL_REQUIRE(nblocks < 2147483647LL, QMLL_ERR_INVALID, "%s: too many tiles", who);
+    // The tiles run in rounds of one per workgroup slot (two per CU); when the last round is less
+    // than half full its tiles are cut into row ranges that fill the slots, each range writing a
+    // partial tile to the workspace, and a small kernel adds the partial tiles in the order of the
+    // ranges: the sums stay deterministic.  At F = 16 384 that is 64 of 8256 tiles in 8 ranges each,
+    // 16.1 rounds instead of 17.
+    TileMap tail = tm;
+    long long ntail_ids = 0;
+    if (sym && ws && M >= 2048) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0) {
+            const long long slots = 2LL * cus;
+            const long long ntiles = (long long)ntj * (ntj + 1) / 2;
+            const long long left = ntiles % slots;
+            if (ntiles > slots && left > 0 && 2 * left <= slots) {
+                // the ids of the last `left` tiles (ids past the last tile or without one are skipped over)
+                long long b = nblocks, found = 0;
+                while (b > 0 && found < left) {
+                    int ti, tj;
+                    tile_of_block<true>((unsigned)(b - 1), nti, ntj, tm, ti, tj);
+                    if (ti >= 0 && ti <= tj) ++found;
+                    --b;
+                }
+                const long long ids = nblocks - b;
+                long long pieces = slots / left;
+                if (pieces > 8) pieces = 8;
+                if (found == left && pieces > 1 && (size_t)(ids * pieces) * TILE * TILE * sizeof(double) <= ws_bytes) {
+                    tail.pieces = (int)pieces;
+                    tail.piece_rows = (int)((((long long)M + pieces - 1) / pieces + KB - 1) / KB * KB);
+                    tail.tail_first = (unsigned)b;
+                    ntail_ids = ids;
+                    nblocks = b;      // the ordinary launch stops before the tail
+                }
+            }
+        }
+    }
     const bool guard = (F % TILE) != 0 || ((f1 - f0) % TILE) != 0 || (f0 % 2) != 0 || (ldz % 2) != 0 ||
                        (lda % 2) != 0 || (reinterpret_cast<uintptr_t>(Z) % 16) != 0 ||
                        (reinterpret_cast<uintptr_t>(Za) % 16) != 0;
@@ -350,6 +445,18 @@ static int gram_launch(const double* Z, const double* y, int M, int F, int f0, i
     }
 #undef QMLL_GRAM_LAUNCH
     QMLL_CHECK_LAUNCH(who);
+    if (ntail_ids > 0) {
+        const dim3 tgrid((unsigned)(ntail_ids * tail.pieces));
+        if (guard)
+            hipLaunchKernelGGL((gram_kernel<true, true, true>), tgrid, block, 0, stream, Z, M, F, 0, F, nti, ntj, tail, ws,
+                               ldz, ldc, sign, Za, lda, overwrite);
+        else
+            hipLaunchKernelGGL((gram_kernel<true, false, true>), tgrid, block, 0, stream, Z, M, F, 0, F, nti, ntj, tail, ws,
+                               ldz, ldc, sign, Za, lda, overwrite);
+        QMLL_CHECK_LAUNCH(who);
+        hipLaunchKernelGGL(gram_tail_reduce_kernel, dim3((unsigned)ntail_ids), dim3(256), 0, stream, ws, ntj, tail, F, C, ldc);
+        QMLL_CHECK_LAUNCH(who);
+    }
     if (sym && mirror && ldc == F) {
         const unsigned nb = (unsigned)((F + MT - 1) / MT);
         hipLaunchKernelGGL(gram_mirror_kernel, dim3(nb, nb), dim3(256), 0, stream, C, F);
@@ -371,6 +478,14 @@ extern "C" int qmll_gram_f64(const double* Z, const double* y, int M, int F, dou
 extern "C" int qmll_gram_upper_f64(const double* Z, const double* y, int M, int F, double* ZTZ, double* ZTy,
                                    qmll_stream_t stream) {
     return gram_launch(Z, y, M, F, 0, F > 0 ? F : 1, true, false, ZTZ, ZTy, (hipStream_t)stream, "qmll_gram_upper_f64");
+}
+
+extern "C" size_t qmll_gram_workspace_bytes(void) { return GRAM_WS_BYTES; }
+
+extern "C" int qmll_gram_upper_ws_f64(const double* Z, const double* y, int M, int F, double* ZTZ, double* ZTy,
+                                      double* workspace, size_t workspace_bytes, qmll_stream_t stream) {
+    return gram_launch(Z, y, M, F, 0, F > 0 ? F : 1, true, false, ZTZ, ZTy, (hipStream_t)stream, "qmll_gram_upper_ws_f64", 0, 0,
+                       1.0, nullptr, 0, 0, workspace, workspace_bytes);
 }
 
 extern "C" int qmll_gram_mirror_f64(double* ZTZ, int F, qmll_stream_t stream) {

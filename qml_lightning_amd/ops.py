@@ -563,8 +563,16 @@ def gram(Zrows, y, ZTZ, ZTy, f0=None, f1=None, mirror=True):
             raise RuntimeError("targets have %d rows, features have %d" % (yv.shape[0], M))
     zty = ZTy if ZTy is not None else None
     if f0 is None:
-        fn = _lib.lib().qmll_gram_f64 if mirror else _lib.lib().qmll_gram_upper_f64
-        check(fn(_ptr(Zrows), _ptr(yv), M, F, _ptr(ZTZ), _ptr(zty), _stream()), "qmll_gram_f64")
+        # with a workspace the last, sparsely filled round of tiles is split over the idle CUs (the
+        # buffer comes from torch's caching allocator, which keeps its reuse ordered per stream)
+        ws = None
+        if M >= 2048:
+            ws = torch.empty(int(_lib.lib().qmll_gram_workspace_bytes()) // 8, dtype=torch.float64, device=Zrows.device)
+        check(_lib.lib().qmll_gram_upper_ws_f64(_ptr(Zrows), _ptr(yv), M, F, _ptr(ZTZ), _ptr(zty), _ptr(ws),
+                                                ws.numel() * 8 if ws is not None else 0, _stream()),
+              "qmll_gram_upper_ws_f64")
+        if mirror:
+            check(_lib.lib().qmll_gram_mirror_f64(_ptr(ZTZ), F, _stream()), "qmll_gram_mirror_f64")
     else:
         check(_lib.lib().qmll_gram_tile_f64(_ptr(Zrows), _ptr(yv), M, F, int(f0), int(f1), _ptr(ZTZ), _ptr(zty),
                                             _stream()), "qmll_gram_tile_f64")

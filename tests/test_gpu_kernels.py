@@ -574,6 +574,53 @@ def test_gram_upper_batches_then_one_mirror(F):
     close(up, ref, 1e-13, "batched ZTZ")
 
 
+@pytest.mark.parametrize("F,M", [(4096, 2500), (4100, 2100)])
+def test_gram_with_workspace_splits_the_last_round_of_tiles(F, M):
+    """More tiles than workgroup slots and a sparsely filled last round (528 tiles at F = 4096, 561
+    at 4100 where every load is bounds-checked): with a workspace the last tiles are cut into row ranges
+    whose partial tiles are added in a fixed order.  Against fp64 matmul, against the entry without a
+    workspace (equal up to the regrouping of the sums), bit-equal from call to call, accumulating onto
+    what is already there, and untouched below the diagonal tiles."""
+    from qml_lightning_amd import _lib
+    from qml_lightning_amd.ops import _ptr, _stream
+    L = _lib.lib()
+    g = torch.Generator(device="cpu").manual_seed(F)
+    Z = torch.randn(M, F, dtype=torch.float64, generator=g).to(dev())
+    y = torch.randn(M, dtype=torch.float64, generator=g).to(dev())
+    ws = torch.empty(int(L.qmll_gram_workspace_bytes()) // 8, dtype=torch.float64, device=dev())
+    ws.fill_(float("nan"))                       # whatever the workspace holds must not matter
+
+    def run(with_ws, start):
+        C = torch.full((F, F), start, dtype=torch.float64, device=dev())
+        zy = torch.zeros(F, dtype=torch.float64, device=dev())
+        if with_ws:
+            rc = L.qmll_gram_upper_ws_f64(_ptr(Z), _ptr(y), M, F, _ptr(C), _ptr(zy), _ptr(ws), ws.numel() * 8, _stream())
+        else:
+            rc = L.qmll_gram_upper_f64(_ptr(Z), _ptr(y), M, F, _ptr(C), _ptr(zy), _stream())
+        assert rc == 0, _lib.last_error()
+        return C, zy
+    plain, zy0 = run(False, 0.0)
+    split, zy1 = run(True, 0.0)
+    again, _ = run(True, 0.0)
+    assert torch.equal(split, again)
+    zy_ref = torch.matmul(Z.T, y)                # Z^T y adds its row blocks with fp64 atomics: equal to rounding
+    assert (zy0 - zy_ref).abs().max() <= 1e-13 * zy_ref.abs().max() and (zy1 - zy_ref).abs().max() <= 1e-13 * zy_ref.abs().max()
+    ref = torch.matmul(Z.T, Z)
+    tiles = torch.arange(F, device=dev()) // 128
+    upper = tiles[:, None] <= tiles[None, :]
+    scale = ref.abs().max().item()
+    assert (split - ref)[upper].abs().max().item() <= 1e-13 * scale
+    assert (split - plain)[upper].abs().max().item() <= 1e-13 * scale
+    assert not torch.equal(split, plain)         # the split did run: the last tiles are summed in another grouping
+    assert (split[~upper] == 0).all()
+    onto, _ = run(True, 3.0)                     # accumulates: C += Z^T Z on the tiles it owns
+    assert (onto - 3.0 - ref)[upper].abs().max().item() <= 1e-13 * scale and (onto[~upper] == 3.0).all()
+    # too small a workspace, or none: the ordinary launch, bit-equal to the entry without one
+    C = torch.zeros(F, F, dtype=torch.float64, device=dev())
+    assert L.qmll_gram_upper_ws_f64(_ptr(Z), None, M, F, _ptr(C), None, _ptr(ws), 1024, _stream()) == 0
+    assert torch.equal(C, plain)
+
+
 @pytest.mark.parametrize("F", [6, 100, 128, 300, 1064, 2176])
 def test_cholesky_solve_matches_lapack(F):
     """(Z^T Z + lambda I) x = b by the library's blocked Cholesky against numpy's LU solve (the
