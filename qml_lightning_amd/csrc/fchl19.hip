@@ -29,6 +29,7 @@ namespace {
 // instructions each, several times per neighbour and per triple
 __device__ __forceinline__ float frcp(float x) { return __builtin_amdgcn_rcpf(x); }
 __device__ __forceinline__ float fsqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
+__device__ __forceinline__ float frsq(float x) { return __builtin_amdgcn_rsqf(x); }
 __device__ __forceinline__ float flog(float x) { return __builtin_amdgcn_logf(x) * 0.6931471805599453f; }
 // floor(x / d) for 0 <= x < 1e6, 0 < d: (x + 0.5) / d is at least 0.5 / d away from an integer,
 // far more than the rounding of the 1-ulp reciprocal, so the truncation is exact; five
@@ -373,10 +374,6 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
     // the staging, so their latency overlaps the staging's own loads.
     const float rs2v = lane < nRs2 ? a.Rs2[lane] : 1.0f;
     const float rs3v = lane < nRs3 ? a.Rs3[lane] : 0.0f;
-    // the table starts as zero entries: the padding between its segments contributes nothing
-    for (int t = lane; t < a.tcap + a.tpad; t += QMLL_WAVE)
-        reinterpret_cast<float4*>(trip)[t] = make_float4(0.f, 0.f, 0.f, 0.f);
-
     const float zeta2 = 0.014383766711652736f;   // 2 exp(-pi^2 / 2)
     const float k3 = a.p.eta3 * LOG2E;
     const float sk3 = fsqrt(k3);                 // exp(-eta3 (rho - Rs)^2) = exp2(-(sk3 rho - sk3 Rs)^2)
@@ -392,7 +389,7 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
             reinterpret_cast<float4*>(s2b)[pos] = make_float4(
                 fmaf(l2r, 0.6931471805599453f, -0.5f * s2),   // ln(r / sqrt(1 + eta2/r^2))
                 0.5f * LOG2E * frcp(s2),
-                rsqrtf(s2) * 0.3989422804014327f * fexp2(-a.p.two_body_decay * l2r) * fc, 0.0f);
+                frsq(s2) * 0.3989422804014327f * fexp2(-a.p.two_body_decay * l2r) * fc, 0.0f);
             reinterpret_cast<float4*>(recA)[pos] = make_float4(dx, dy, dz, ir);
             reinterpret_cast<float4*>(recB)[pos] = make_float4(sk3 * 0.5f * r, fc * fexp2(-a.p.three_body_decay * l2r),
                                                                __int_as_float(e), __int_as_float(rank | (count << 16)));
@@ -462,7 +459,7 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
         const float dac = Aj.x * cx + Aj.y * cy + Aj.z * cz;
         const float dcb = cx * Ak.x + cy * Ak.y + cz * Ak.z;
         const float w = Aj.w * Ak.w;
-        const float W = w * rsqrtf(c2);
+        const float W = w * frsq(c2);
         const float px = Aj.y * Ak.z - Aj.z * Ak.y, py = Aj.z * Ak.x - Aj.x * Ak.z, pz = Aj.x * Ak.y - Aj.y * Ak.x;
         const float f = zw3 * fmaf(-3.0f * vi * dac, dcb * W * W, 1.0f) * Bj.y * Bk.y * fexp2(hd3 * flog2(c2));
         const float cosT = fminf(1.0f, fmaxf(-1.0f, vi * w));
@@ -535,10 +532,10 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
             if (ns * ns <= QMLL_WAVE) {
                 // lane p*ns+q takes pair (p,q); an exclusive scan over the lanes gives the starts
                 const int p = idiv_small(lane, ns), q = lane - p * ns;
-                int rounds = 0;
+                int rounds = 0, ntr = 0;
                 if (lane < ns * ns && q >= p) {
                     const int np_ = goff[p + 1] - goff[p], nq = goff[q + 1] - goff[q];
-                    const int ntr = (p == q) ? (__mul24(np_, np_ - 1) >> 1) : __mul24(np_, nq);
+                    ntr = (p == q) ? (__mul24(np_, np_ - 1) >> 1) : __mul24(np_, nq);
                     rounds = idiv_small(ntr + TSv - 1, TSv);
                 }
                 const int size = rounds * TSv;               // segments start on a multiple of TS
@@ -550,6 +547,9 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
                 if (lane < ns * ns) {
                     pbase[lane] = incl - size;
                     prounds[lane] = rounds;
+                    // the padding of the segment is zero entries: they contribute nothing
+                    for (int t = incl - size + ntr; t < incl; ++t)
+                        reinterpret_cast<float4*>(trip)[t] = make_float4(0.f, 0.f, 0.f, 0.f);
                 }
             } else if (lane == 0) {
                 int acc = 0;
@@ -560,6 +560,8 @@ __global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* _
                         const int rounds = idiv_small(ntr + TSv - 1, TSv);
                         pbase[p * ns + q] = acc;
                         prounds[p * ns + q] = rounds;
+                        for (int t = acc + ntr; t < acc + rounds * TSv; ++t)
+                            reinterpret_cast<float4*>(trip)[t] = make_float4(0.f, 0.f, 0.f, 0.f);
                         acc += rounds * TSv;
                     }
                 }
@@ -644,7 +646,7 @@ __device__ __forceinline__ TwoBody two_body_setup(float r, float fc, float dfc, 
     t.mu = flog(r) - 0.5f * t.s2;
     t.s2p = -2.0f * p.eta2 * frcp(r * (r2 + p.eta2));      // d sigma^2 / dr
     t.mup = frcp(r) - 0.5f * t.s2p;                   // d mu / dr
-    t.pre = rsqrtf(t.s2) * 0.3989422804014327f * fexp2(-p.two_body_decay * flog2(r));
+    t.pre = frsq(t.s2) * 0.3989422804014327f * fexp2(-p.two_body_decay * flog2(r));
     t.fc = fc;
     t.dfc = dfc;
     t.d2_over_r = p.two_body_decay * frcp(r);
