@@ -3,11 +3,12 @@
 // :676-1005 and :1007-1323 (Jacobian) of the reference.
 //
 // Layout: one wavefront (64 lanes, one workgroup) per central atom.  The atom's
-// neighbour list is staged in LDS as displacement vectors d_ij = R_i - R_j (minimum-imaged
-// once when a cell is given), distances, element types and atom indices; it is either
-// read from a caller-supplied list or built in the kernel from the molecule's coordinates
-// with a ballot/popcount compaction (ascending j, same rule as the neighbour-list kernel),
-// so the forward/backward pair needs no host round trip for max(nneigh).
+// neighbour list is staged in LDS sorted by element, as displacement vectors d_ij = R_i - R_j
+// (minimum-imaged once when a cell is given) with whatever else of a neighbour the kernel reads
+// again (forward and VJP: 16-byte records written by the lane that finds the neighbour; Jacobian:
+// one array per quantity); it is either read from a caller-supplied list or built in the kernel
+// from the molecule's coordinates with a ballot/popcount compaction (ascending j, same rule as the
+// neighbour-list kernel), so the forward/backward pair needs no host round trip for max(nneigh).
 //
 // Arithmetic per atom (nn neighbours): nn*nRs2 + nn(nn-1)/2*nRs3 exponentials forward;
 // the kernels are VALU/transcendental bound, HBM traffic is 4R bytes out (forward) or in
