@@ -450,18 +450,46 @@ __global__ __launch_bounds__(SORF_THREADS) void sorf_energy_fused_kernel(
         : "+v"(w0), "+v"(w1), "+v"(w2), "+v"(w3)                                                 \
         : "v"(c))
 
+// eight registers behind one pair of wait states (the hazard is between the instruction that
+// wrote a register and the first DPP read of it; inside the block every read is at least
+// eight instructions behind its write in the block before)
+#define QMLL_DPP_STAGE8(CTRL, w, g, c)                                                           \
+    asm("s_nop 1\n\t"                                                                            \
+        "v_fmac_f32_dpp %0, %0, %8 " CTRL " row_mask:0xf bank_mask:0xf\n\t"                      \
+        "v_fmac_f32_dpp %1, %1, %8 " CTRL " row_mask:0xf bank_mask:0xf\n\t"                      \
+        "v_fmac_f32_dpp %2, %2, %8 " CTRL " row_mask:0xf bank_mask:0xf\n\t"                      \
+        "v_fmac_f32_dpp %3, %3, %8 " CTRL " row_mask:0xf bank_mask:0xf\n\t"                      \
+        "v_fmac_f32_dpp %4, %4, %8 " CTRL " row_mask:0xf bank_mask:0xf\n\t"                      \
+        "v_fmac_f32_dpp %5, %5, %8 " CTRL " row_mask:0xf bank_mask:0xf\n\t"                      \
+        "v_fmac_f32_dpp %6, %6, %8 " CTRL " row_mask:0xf bank_mask:0xf\n\t"                      \
+        "v_fmac_f32_dpp %7, %7, %8 " CTRL " row_mask:0xf bank_mask:0xf"                          \
+        : "+v"(w[g]), "+v"(w[g + 1]), "+v"(w[g + 2]), "+v"(w[g + 3]), "+v"(w[g + 4]), "+v"(w[g + 5]),     \
+          "+v"(w[g + 6]), "+v"(w[g + 7])                                                         \
+        : "v"(c))
+
 // the four in-row stages for NV registers (NV a multiple of 4); cs[k] = -1 in lanes whose
 // stage bit k is set, +1 elsewhere
 template <int NV>
 __device__ __forceinline__ void row_stages(float (&w)[NV], const float (&cs)[4]) {
+    if constexpr (NV % 8 == 0) {
 #pragma unroll
-    for (int g = 0; g < NV; g += 4) QMLL_DPP_STAGE4("quad_perm:[1,0,3,2]", w[g], w[g + 1], w[g + 2], w[g + 3], cs[0]);
+        for (int g = 0; g < NV; g += 8) QMLL_DPP_STAGE8("quad_perm:[1,0,3,2]", w, g, cs[0]);
 #pragma unroll
-    for (int g = 0; g < NV; g += 4) QMLL_DPP_STAGE4("quad_perm:[2,3,0,1]", w[g], w[g + 1], w[g + 2], w[g + 3], cs[1]);
+        for (int g = 0; g < NV; g += 8) QMLL_DPP_STAGE8("quad_perm:[2,3,0,1]", w, g, cs[1]);
 #pragma unroll
-    for (int g = 0; g < NV; g += 4) QMLL_DPP_STAGE4("row_half_mirror", w[g], w[g + 1], w[g + 2], w[g + 3], cs[2]);
+        for (int g = 0; g < NV; g += 8) QMLL_DPP_STAGE8("row_half_mirror", w, g, cs[2]);
 #pragma unroll
-    for (int g = 0; g < NV; g += 4) QMLL_DPP_STAGE4("row_ror:8", w[g], w[g + 1], w[g + 2], w[g + 3], cs[3]);
+        for (int g = 0; g < NV; g += 8) QMLL_DPP_STAGE8("row_ror:8", w, g, cs[3]);
+    } else {
+#pragma unroll
+        for (int g = 0; g < NV; g += 4) QMLL_DPP_STAGE4("quad_perm:[1,0,3,2]", w[g], w[g + 1], w[g + 2], w[g + 3], cs[0]);
+#pragma unroll
+        for (int g = 0; g < NV; g += 4) QMLL_DPP_STAGE4("quad_perm:[2,3,0,1]", w[g], w[g + 1], w[g + 2], w[g + 3], cs[1]);
+#pragma unroll
+        for (int g = 0; g < NV; g += 4) QMLL_DPP_STAGE4("row_half_mirror", w[g], w[g + 1], w[g + 2], w[g + 3], cs[2]);
+#pragma unroll
+        for (int g = 0; g < NV; g += 4) QMLL_DPP_STAGE4("row_ror:8", w[g], w[g + 1], w[g + 2], w[g + 3], cs[3]);
+    }
 }
 
 template <int EPL>
@@ -633,7 +661,9 @@ __global__ __launch_bounds__(64 * NW) void sorf_energy_rows_kernel(
         constexpr float INV2PI = 0.15915494309189535f;
         const float xs = scale * INV2PI;
         const float csig = sigma * INV2PI;
-        const float ncs[4] = {-cs[0], -cs[1], -cs[2], -cs[3]};
+        float ncs[4] = {-cs[0], -cs[1], -cs[2], -cs[3]};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) asm("" : "+v"(ncs[q]));   // kept in registers, not negated again in every stack
 #pragma unroll
         for (int p = 0; p < EPL; ++p) xv[p] *= xs;
         // v_sin_f32 / v_cos_f32 reduce the range themselves up to 256 revolutions.  The rounding of
