@@ -243,6 +243,16 @@ size_t qmll_sort_by_type_workspace(int A, int ne);
 int qmll_sort_by_type(const int* types, const int* slots, int A, int ne, void* workspace, size_t workspace_bytes,
                       int* sorted_slots, int* type_offsets, qmll_stream_t stream);
 
+/* qmll_sort_by_type for the listed atoms of a padded batch: slot of atom a = molIDs[a] * n +
+ * atomIDs[a] (the index the reference builds as torch.where(Z == e) over the [B, n] charges,
+ * models/hadamard_features.py:99-107).  atomIDs, molIDs i32 [A], types i32 [B * n].  Up to 1024
+ * atoms the whole sort is one launch and needs no workspace (qmll_sort_atoms_workspace returns 0);
+ * beyond, the slots are written to the workspace and qmll_sort_by_type runs on them. */
+size_t qmll_sort_atoms_workspace(int A, int ne);
+int qmll_sort_atoms_by_type(const int* types, const int* atomIDs, const int* molIDs, int n, int A, int ne,
+                            void* workspace, size_t workspace_bytes, int* sorted_slots, int* type_offsets,
+                            qmll_stream_t stream);
+
 /* qmll_sort_by_type for callers that cannot allocate device memory or carry a workspace: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
  * counterpart in the reference (whose wrappers allocate with torch::zeros on every call).

@@ -54,6 +54,8 @@ PROTOTYPES = {
     "qmll_sorf_energy_typed": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, P, P, P],
     "qmll_sort_by_type_workspace": [c_int, c_int],
     "qmll_sort_by_type": [P, P, c_int, c_int, P, c_size_t, P, P, P],
+    "qmll_sort_atoms_workspace": [c_int, c_int],
+    "qmll_sort_atoms_by_type": [P, P, P, c_int, c_int, c_int, P, c_size_t, P, P, P],
     "qmll_sort_by_type_noalloc": [P, P, c_int, c_int, P, P, P],
     "qmll_project_typed": [P, P, P, P, c_int, c_int, c_int, c_int, P, P],
     "qmll_project_typed_backward": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
@@ -77,7 +79,7 @@ PROTOTYPES = {
     "qmll_probe_rate": [c_int, c_int, c_int, P, P],
     "qmll_probe_mix": [c_int, c_int, c_int, P, P],
 }
-_RESTYPES = {"qmll_last_error": c_char_p, "qmll_sort_by_type_workspace": c_size_t,
+_RESTYPES = {"qmll_last_error": c_char_p, "qmll_sort_by_type_workspace": c_size_t, "qmll_sort_atoms_workspace": c_size_t,
              "qmll_cholesky_workspace_bytes": c_size_t, "qmll_gram_workspace_bytes": c_size_t,
              "qmll_probe_out_bytes": c_size_t, "qmll_probe_rate": c_double,
              "qmll_probe_mix": c_double}

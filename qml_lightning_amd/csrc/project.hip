@@ -101,6 +101,57 @@ __global__ __launch_bounds__(ST) void type_place_kernel(const int* __restrict__ 
     for (int i = start[ne] + a; i < A; i += nb * ST) sorted[i] = 0;
 }
 
+// slot of listed atom a in the padded [B, n] layout
+__global__ __launch_bounds__(256) void atom_slots_kernel(const int* __restrict__ atomIDs, const int* __restrict__ molIDs,
+                                                         int n, int A, int* __restrict__ slots) {
+    const int a = blockIdx.x * 256 + threadIdx.x;
+    if (a < A) slots[a] = molIDs[a] * n + atomIDs[a];
+}
+
+// The whole sort in one workgroup for up to 1024 listed atoms (a molecule, a few dozen molecules):
+// slot = molIDs * n + atomIDs, count, prefix and placement without a second launch or a workspace.
+constexpr int SORT_SMALL = 1024;
+__global__ __launch_bounds__(SORT_SMALL) void type_sort_small_kernel(const int* __restrict__ types,
+                                                                     const int* __restrict__ atomIDs,
+                                                                     const int* __restrict__ molIDs, int n, int A, int ne,
+                                                                     int* __restrict__ sorted, int* __restrict__ offsets) {
+    __shared__ int wcnt[SORT_SMALL / 64][MAXNE];   // atoms of type e in wavefront w, then: of earlier wavefronts
+    __shared__ int total[MAXNE], start[MAXNE + 1];
+    const int a = threadIdx.x, lane = a & 63, wave = a >> 6;
+    const int slot = a < A ? molIDs[a] * n + atomIDs[a] : 0;
+    const int t = a < A ? types[slot] : -1;
+    int rank = 0;
+    for (int e = 0; e < ne; ++e) {
+        const unsigned long long m = __ballot(t == e);
+        if (lane == 0) wcnt[wave][e] = __popcll(m);
+        if (t == e) rank = __popcll(m & ((1ull << lane) - 1ull));
+    }
+    __syncthreads();
+    if (a < ne) {          // thread e: exclusive prefix of its type over the wavefronts
+        int s = 0;
+        for (int w = 0; w < SORT_SMALL / 64; ++w) {
+            const int c = wcnt[w][a];
+            wcnt[w][a] = s;
+            s += c;
+        }
+        total[a] = s;
+    }
+    __syncthreads();
+    if (a == 0) {
+        int s = 0;
+        for (int e = 0; e < ne; ++e) {
+            start[e] = s;
+            s += total[e];
+        }
+        start[ne] = s;
+    }
+    __syncthreads();
+    if (a <= ne) offsets[a] = start[a];
+    if (t >= 0 && t < ne) sorted[start[t] + wcnt[wave][t] + rank] = slot;
+    // entries past the last typed atom name a valid slot, so gathers through them stay in bounds
+    for (int i = start[ne] + a; i < A; i += SORT_SMALL) sorted[i] = 0;
+}
+
 // ---- typed GEMM -------------------------------------------------------------------------
 constexpr int PT = 256;            // threads (4 wavefronts, each 32 rows x 64 columns)
 constexpr int PM = 128;            // rows per workgroup
@@ -362,9 +413,9 @@ __global__ __launch_bounds__(PT) void typed_gemm_bt_rows_kernel(const float* __r
 
 // rows of real atoms whose element the model does not know get a zero gradient
 // (lane = slot; the rare untyped slots of a wavefront are then zeroed row by row by all lanes)
-__global__ __launch_bounds__(256) void zero_untyped_rows_kernel(const int* __restrict__ types, int N, int ne, int R,
-                                                                float* __restrict__ out) {
-    const int slot = blockIdx.x * 256 + threadIdx.x;
+__device__ __forceinline__ void zero_untyped_rows(const int* __restrict__ types, int N, int ne, int R,
+                                                  float* __restrict__ out, int chunk) {
+    const int slot = chunk * 256 + threadIdx.x;
     const int lane = threadIdx.x & 63;
     const int t = slot < N ? types[slot] : 0;
     unsigned long long todo = __ballot(slot < N && (t < 0 || t >= ne));
@@ -374,6 +425,11 @@ __global__ __launch_bounds__(256) void zero_untyped_rows_kernel(const int* __res
         const size_t row = (size_t)(slot - lane + l) * R;
         for (int c = lane; c < R; c += 64) out[row + c] = 0.0f;
     }
+}
+
+__global__ __launch_bounds__(256) void zero_untyped_rows_kernel(const int* __restrict__ types, int N, int ne, int R,
+                                                                float* __restrict__ out) {
+    zero_untyped_rows(types, N, ne, R, out, blockIdx.x);
 }
 
 // Small batches (a molecule or a few): the tiled kernels above run one or two workgroups through
@@ -428,12 +484,18 @@ __global__ __launch_bounds__(256) void project_small_kernel(const float* __restr
 }
 
 // g_rep[slot(p), :] = gx[p, :] . U_e^T: thread = output entry r, its reductor row is contiguous
+// (workgroups past the A atoms zero the rows of slots whose type is outside [0, ne), 256 slots each)
 __global__ __launch_bounds__(256) void project_bt_small_kernel(const float* __restrict__ gx,
                                                                const int* __restrict__ sorted_slots,
                                                                const int* __restrict__ type_offsets,
                                                                const float* __restrict__ reductors, int ne, int R, int d,
-                                                               float* __restrict__ g_rep) {
+                                                               float* __restrict__ g_rep, int A,
+                                                               const int* __restrict__ types, int N) {
     extern __shared__ float sm[];                      // [d]
+    if ((int)blockIdx.x >= A) {
+        zero_untyped_rows(types, N, ne, R, g_rep, (int)blockIdx.x - A);
+        return;
+    }
     const int p = blockIdx.x, tid = threadIdx.x;
     if (p >= type_offsets[ne]) return;                 // past the sorted list (atoms of no known element)
     const int e = type_of_position(type_offsets, ne, p);
@@ -491,6 +553,41 @@ extern "C" int qmll_sort_by_type(const int* types, const int* slots, int A, int 
                        sorted_slots, type_offsets);
     QMLL_CHECK_LAUNCH("qmll_sort_by_type");
     return QMLL_OK;
+}
+
+extern "C" size_t qmll_sort_atoms_workspace(int A, int ne) {
+    if (A <= SORT_SMALL) return 0;
+    return qmll_sort_by_type_workspace(A, ne) + sizeof(int) * (size_t)(A > 0 ? A : 0);
+}
+
+extern "C" int qmll_sort_atoms_by_type(const int* types, const int* atomIDs, const int* molIDs, int n, int A, int ne,
+                                       void* workspace, size_t workspace_bytes, int* sorted_slots, int* type_offsets,
+                                       qmll_stream_t stream) {
+    QMLL_REQUIRE(A >= 0 && n > 0 && ne > 0 && ne <= MAXNE, QMLL_ERR_INVALID,
+                 "qmll_sort_atoms_by_type: bad size A=%d n=%d ne=%d (at most %d types)", A, n, ne, MAXNE);
+    QMLL_REQUIRE(type_offsets, QMLL_ERR_INVALID, "qmll_sort_atoms_by_type: null pointer");
+    if (A == 0) {
+        hipLaunchKernelGGL(zero_ints_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, type_offsets, ne + 1);
+        QMLL_CHECK_LAUNCH("qmll_sort_atoms_by_type");
+        return QMLL_OK;
+    }
+    QMLL_REQUIRE(types && atomIDs && molIDs && sorted_slots, QMLL_ERR_INVALID, "qmll_sort_atoms_by_type: null pointer");
+    if (A <= SORT_SMALL) {
+        hipLaunchKernelGGL(type_sort_small_kernel, dim3(1), dim3(SORT_SMALL), 0, (hipStream_t)stream, types, atomIDs,
+                           molIDs, n, A, ne, sorted_slots, type_offsets);
+        QMLL_CHECK_LAUNCH("qmll_sort_atoms_by_type");
+        return QMLL_OK;
+    }
+    const size_t need = qmll_sort_atoms_workspace(A, ne);
+    QMLL_REQUIRE(workspace && workspace_bytes >= need, QMLL_ERR_INVALID,
+                 "qmll_sort_atoms_by_type: workspace of %zu bytes, %zu needed", workspace_bytes, need);
+    // the slots go behind the counts of the general sort
+    const size_t counts_bytes = qmll_sort_by_type_workspace(A, ne);
+    int* slots = reinterpret_cast<int*>(static_cast<char*>(workspace) + counts_bytes);
+    hipLaunchKernelGGL(atom_slots_kernel, dim3((A + 255) / 256), dim3(256), 0, (hipStream_t)stream, atomIDs, molIDs, n, A,
+                       slots);
+    QMLL_CHECK_LAUNCH("qmll_sort_atoms_by_type");
+    return qmll_sort_by_type(types, slots, A, ne, workspace, counts_bytes, sorted_slots, type_offsets, stream);
 }
 
 // ---- the same sort for callers that cannot allocate -------------------------------------
@@ -584,7 +681,9 @@ extern "C" int qmll_project_typed_backward(const float* gx, const int* sorted_sl
                                            int d, float* g_rep, qmll_stream_t stream) {
     QMLL_REQUIRE(A >= 0 && N >= 0 && ne > 0 && R > 0 && d > 0, QMLL_ERR_INVALID,
                  "qmll_project_typed_backward: bad size A=%d N=%d ne=%d R=%d d=%d", A, N, ne, R, d);
-    if (types && N > 0) {
+    const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(gx) && aligned16(reductors);
+    const bool small = vec && A > 0 && A <= SMALL_ATOMS && (size_t)d * sizeof(float) <= 64 * 1024 && N <= 64 * 256;
+    if (types && N > 0 && !small) {
         QMLL_REQUIRE(g_rep, QMLL_ERR_INVALID, "qmll_project_typed_backward: null pointer");
         hipLaunchKernelGGL(zero_untyped_rows_kernel, dim3((N + 255) / 256), dim3(256), 0, (hipStream_t)stream, types, N, ne,
                            R, g_rep);
@@ -594,10 +693,11 @@ extern "C" int qmll_project_typed_backward(const float* gx, const int* sorted_sl
     QMLL_REQUIRE(gx && sorted_slots && type_offsets && reductors && g_rep, QMLL_ERR_INVALID,
                  "qmll_project_typed_backward: null pointer");
     const dim3 grid((A + PM - 1) / PM + ne, (R + PN - 1) / PN);
-    const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(gx) && aligned16(reductors);
-    if (vec && A <= SMALL_ATOMS && (size_t)d * sizeof(float) <= 64 * 1024) {
-        hipLaunchKernelGGL(project_bt_small_kernel, dim3(A), dim3(256), sizeof(float) * d, (hipStream_t)stream, gx,
-                           sorted_slots, type_offsets, reductors, ne, R, d, g_rep);
+    if (small) {
+        // one launch: a workgroup per atom, and one per 256 slots for the rows of unknown elements
+        const int zero_groups = (types && N > 0) ? (N + 255) / 256 : 0;
+        hipLaunchKernelGGL(project_bt_small_kernel, dim3(A + zero_groups), dim3(256), sizeof(float) * d, (hipStream_t)stream,
+                           gx, sorted_slots, type_offsets, reductors, ne, R, d, g_rep, A, types, N);
     } else if (vec && (d == 64 || d == 128)) {
         // short contraction: the gradient rows stay in registers, every row is read once
         const dim3 g1((A + PM - 1) / PM + ne);

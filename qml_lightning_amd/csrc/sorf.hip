@@ -622,7 +622,16 @@ __global__ __launch_bounds__(64 * NW) void sorf_energy_rows_kernel(
             }
             b -= nt;
         }
-        if (rows == 0) return;
+        if (rows == 0) {
+            // a workgroup past the last tile (the launch adds at least one): its share of the gradient
+            // rows past the last atom of a known element, which are zero
+            if constexpr (WITH_GRAD) {
+                const int spare = b, nspare = (int)gridDim.x - ((int)blockIdx.x - b);
+                for (int r = type_offsets[ne] + spare; r < A; r += nspare)
+                    for (int c = threadIdx.x; c < d; c += 64 * NW) gx[(size_t)r * d + c] = 0.0f;
+            }
+            return;
+        }
         D += (size_t)t * T * S * d;
         bias += (size_t)t * S * d;
     } else {
@@ -842,13 +851,6 @@ __global__ __launch_bounds__(64 * NW) void sorf_energy_rows_kernel(
     }
 }
 
-// gradient rows past the last atom of a known element are zero
-__global__ void zero_tail_rows_kernel(const int* __restrict__ type_offsets, int ne, int A, int d, float* __restrict__ gx) {
-    const int total = type_offsets[ne];
-    const size_t n = (size_t)(A - total) * d;
-    for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (size_t)gridDim.x * blockDim.x)
-        gx[(size_t)total * d + t] = 0.0f;
-}
 
 // ---- two-op contract in the 16-lane-row layout (64 <= d <= 256) ---------------------------
 // The four rows of a wavefront carry four consecutive stacks of ONE atom, so a workgroup has
@@ -1596,7 +1598,10 @@ static int launch_fused(const char* who, const float* x, const float* D, const f
     if (d >= 64 && d <= 256 && types == nullptr) {
         // 4 to 16 registers per lane, atoms groupable by element: the instruction-lean kernel
         // (four atoms per workgroup)
-        const dim3 grid((A + ROWS_NA - 1) / ROWS_NA + (type_offsets ? ne : 0));
+        // with type offsets: up to ne tiles more than A / 4 (every type rounds up), and 1 to 64 workgroups
+        // that zero the gradient rows past the last atom of a known element
+        const int zero_groups = A >= 65536 ? 64 : (A >> 10) + 1;
+        const dim3 grid((A + ROWS_NA - 1) / ROWS_NA + (type_offsets ? ne + zero_groups : 0));
         // a few atoms: sixteen wavefronts per workgroup share out the stacks
         const bool few = A <= 256 && S >= 64 && d <= 128 && T == 1;
 #define LAUNCH_ROWS(L, G, M)                                                                                       \
@@ -1621,10 +1626,6 @@ static int launch_fused(const char* who, const float* x, const float* D, const f
 #undef LAUNCH_ROWS
 #undef CALL_ROWS
         QMLL_CHECK_LAUNCH(who);
-        if (gx && type_offsets) {
-            hipLaunchKernelGGL(zero_tail_rows_kernel, dim3(64), dim3(256), 0, stream, type_offsets, ne, A, d, gx);
-            QMLL_CHECK_LAUNCH(who);
-        }
         return QMLL_OK;
     }
 #define CALL(L)                                                                                                  \

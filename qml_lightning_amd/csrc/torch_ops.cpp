@@ -401,6 +401,22 @@ std::tuple<Tensor, Tensor> sort_by_type(const Tensor& types, const Tensor& slots
     return {sorted, offsets};
 }
 
+// sort_by_type of the listed atoms of a padded batch (slot = molIDs * n + atomIDs), one launch for small batches
+std::tuple<Tensor, Tensor> sort_atoms_by_type(const Tensor& types, const Tensor& atomIDs, const Tensor& molIDs, int64_t n,
+                                              int64_t ne) {
+    need_cuda(types, "types");
+    Tensor ty = i32(types).reshape({-1}), ai = i32(atomIDs).reshape({-1}), mi = i32(molIDs).reshape({-1});
+    const int A = (int)ai.size(0);
+    TORCH_CHECK(mi.size(0) == A, "sort_atoms_by_type: ", A, " atom indices, ", mi.size(0), " molecule indices");
+    Tensor sorted = at::empty({A}, ty.options()), offsets = at::empty({ne + 1}, ty.options());
+    const size_t nbytes = qmll_sort_atoms_workspace(A, (int)ne);
+    Tensor work = nbytes ? at::empty({(int64_t)(nbytes / 4)}, ty.options()) : Tensor();
+    check(qmll_sort_atoms_by_type(ip(ty), ip(ai), ip(mi), (int)n, A, (int)ne, nbytes ? work.data_ptr<int>() : nullptr, nbytes,
+                                  A ? sorted.data_ptr<int>() : nullptr, offsets.data_ptr<int>(), stream()),
+          "qmll_sort_atoms_by_type");
+    return {sorted, offsets};
+}
+
 Tensor project_typed_impl(const Tensor& rep, const Tensor& sorted_slots, const Tensor& type_offsets,
                           const Tensor& reductors) {
     Tensor r = f32(rep), red = f32(reductors), ss = i32(sorted_slots), off = i32(type_offsets);
@@ -451,9 +467,11 @@ Tensor project_typed(const Tensor& rep, const Tensor& ss, const Tensor& off, con
     return ProjectFn::apply(rep, ss, off, red, types);
 }
 
+// e_zeroed: the caller's zero-filled f32 [nslots] for the energies (one fill then serves several outputs), or undefined
 std::tuple<Tensor, Tensor> sorf_energy_sorted_impl(const Tensor& x_, const Tensor& type_offsets, const Tensor& sorted_slots,
                                                    const Tensor& Dmat, const Tensor& bias, const Tensor& alpha,
-                                                   const Tensor& cn, const Tensor& nt, int64_t nslots, bool with_grad) {
+                                                   const Tensor& cn, const Tensor& nt, int64_t nslots, bool with_grad,
+                                                   const Tensor& e_zeroed = Tensor()) {
     Tensor x = f32(x_), DD = f32(Dmat), bb = f32(bias), al = f32(alpha), off = i32(type_offsets), ss = i32(sorted_slots);
     need_cuda(x, "x");
     const int ne = (int)DD.size(0), Tn = (int)DD.size(1), S = (int)DD.size(2), d = (int)DD.size(3);
@@ -464,7 +482,7 @@ std::tuple<Tensor, Tensor> sorf_energy_sorted_impl(const Tensor& x_, const Tenso
     TORCH_CHECK(bb.dim() == 2 && bb.size(0) == ne && bb.size(1) == (int64_t)S * d && al.numel() == (int64_t)S * d,
                 "sorf_energy_sorted: bias [", bb.sizes(), "] / alpha with ", al.numel(), " entries do not fit ", ne,
                 " elements and ", S * d, " features");
-    Tensor e = at::zeros({nslots}, x.options());
+    Tensor e = e_zeroed.defined() ? e_zeroed : at::zeros({nslots}, x.options());
     Tensor gx = with_grad ? at::empty({A, d}, x.options()) : empty_like_none(x);
     check(qmll_sorf_energy_sorted(fp(x), ip(off), ip(ss), fp(DD), fp(bb), fp(al), A, ne, d, S, T, scalar(cn),
                                   nslots ? e.data_ptr<float>() : nullptr, with_grad && A ? gx.data_ptr<float>() : nullptr,
@@ -510,14 +528,14 @@ std::tuple<Tensor, Tensor> sorf_energy_sorted(const Tensor& x, const Tensor& off
 
 std::tuple<Tensor, Tensor> rff_energy_sorted_impl(const Tensor& x_, const Tensor& type_offsets, const Tensor& sorted_slots,
                                                   const Tensor& W, const Tensor& b, const Tensor& alpha, int64_t nslots,
-                                                  bool with_grad) {
+                                                  bool with_grad, const Tensor& e_zeroed = Tensor()) {
     Tensor x = f32(x_), WW = f32(W), bb = f32(b), al = f32(alpha), off = i32(type_offsets), ss = i32(sorted_slots);
     need_cuda(x, "x");
     const int ne = (int)WW.size(0), d = (int)WW.size(1), F = (int)WW.size(2), A = (int)ss.size(0);
     TORCH_CHECK(x.size(0) == A && x.size(1) == d && off.size(0) == ne + 1 && bb.size(0) == ne && bb.size(1) == F,
                 "rff_energy_sorted: x, W and b do not fit together");
     TORCH_CHECK(al.numel() == F, "rff_energy_sorted: alpha has ", al.numel(), " entries for ", F, " features");
-    Tensor e = at::zeros({nslots}, x.options());
+    Tensor e = e_zeroed.defined() ? e_zeroed : at::zeros({nslots}, x.options());
     Tensor gx = with_grad ? at::empty({A, d}, x.options()) : empty_like_none(x);
     check(qmll_rff_energy_sorted(fp(x), ip(off), ip(ss), fp(WW), fp(bb), fp(al), A, ne, d, F,
                                  nslots ? e.data_ptr<float>() : nullptr, with_grad && A ? gx.data_ptr<float>() : nullptr,
@@ -581,17 +599,19 @@ Tensor fchl_sorf_energy_impl(FCHL_TENSORS, MODEL_TENSORS, bool with_grad, Tensor
     Tensor rep = at::empty({in.B, in.n, in.R}, in.X.options());
     check(qmll_fchl19_forward(FCHL_ABI(in), rep.data_ptr<float>(), stream()), "qmll_fchl19_forward");
     const int64_t nslots = (int64_t)in.B * in.n;
-    Tensor slots = at::add(in.atomIDs, in.molIDs, in.n);      // molIDs * n + atomIDs in one launch
-    auto sorted = sort_by_type(sort_types, slots, ne_model);
+    auto sorted = sort_atoms_by_type(sort_types, in.atomIDs, in.molIDs, in.n, ne_model);
     const Tensor& ss = std::get<0>(sorted);
     const Tensor& off = std::get<1>(sorted);
     Tensor x = project_typed_impl(rep.view({nslots, in.R}), ss, off, reductors);
-    auto eg = rff ? rff_energy_sorted_impl(x, off, ss, Dmat, bias, alpha, nslots, with_grad)
-                  : sorf_energy_sorted_impl(x, off, ss, Dmat, bias, alpha, cn, nt, nslots, with_grad);
+    // the per-slot energies and the coordinate gradient both start from zero: one fill for the two
+    Tensor zeroed = at::zeros({with_grad ? 4 * nslots : nslots}, in.X.options());
+    Tensor e0 = zeroed.narrow(0, 0, nslots);
+    auto eg = rff ? rff_energy_sorted_impl(x, off, ss, Dmat, bias, alpha, nslots, with_grad, e0)
+                  : sorf_energy_sorted_impl(x, off, ss, Dmat, bias, alpha, cn, nt, nslots, with_grad, e0);
     Tensor energies = std::get<0>(eg).view({in.B, in.n}).sum(1);
     if (with_grad) {
         Tensor g_rep = project_typed_backward(std::get<1>(eg), ss, off, reductors, sort_types, nslots);
-        Tensor gX = at::zeros({in.B, in.n, 3}, in.X.options());
+        Tensor gX = zeroed.narrow(0, nslots, 3 * nslots).view({in.B, in.n, 3});
         check(qmll_fchl19_vjp(FCHL_ABI(in), fp(g_rep), gX.data_ptr<float>(), stream()), "qmll_fchl19_vjp");
         *gX_out = gX;
     }

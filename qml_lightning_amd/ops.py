@@ -401,6 +401,22 @@ def sort_by_type(types, slots, ne):
     return sorted_slots, offsets
 
 
+def sort_atoms_by_type(types, atomIDs, molIDs, n, ne):
+    """`sort_by_type` of the listed atoms of a padded [B, n] batch, slot = molIDs * n + atomIDs; one
+    launch and no workspace up to 1024 atoms."""
+    types, atomIDs, molIDs = _i32(types).reshape(-1), _i32(atomIDs).reshape(-1), _i32(molIDs).reshape(-1)
+    A = int(atomIDs.shape[0])
+    if int(molIDs.shape[0]) != A:
+        raise RuntimeError("sort_atoms_by_type: %d atom indices, %d molecule indices" % (A, int(molIDs.shape[0])))
+    sorted_slots = torch.empty(A, dtype=torch.int32, device=types.device)
+    offsets = torch.empty(ne + 1, dtype=torch.int32, device=types.device)
+    nbytes = int(_lib.lib().qmll_sort_atoms_workspace(A, ne))
+    work = torch.empty(nbytes // 4, dtype=torch.int32, device=types.device) if nbytes else None
+    check(_lib.lib().qmll_sort_atoms_by_type(_ptr(types), _ptr(atomIDs), _ptr(molIDs), int(n), A, int(ne), _ptr(work), nbytes,
+                                             _ptr(sorted_slots), _ptr(offsets), _stream()), "qmll_sort_atoms_by_type")
+    return sorted_slots, offsets
+
+
 def project_typed(rep, sorted_slots, type_offsets, reductors):
     """x [A,d]: row a = rep[sorted_slots[a]] . reductors[type of a] (rep [N,R], reductors [ne,R,d])."""
     rep, reductors = _f32(rep), _f32(reductors)

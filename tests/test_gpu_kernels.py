@@ -451,6 +451,24 @@ def test_sort_by_type_is_a_stable_counting_sort(A, N, ne):
     assert (got[len(ref):] == 0).all()
 
 
+@pytest.mark.parametrize("B,n,ne", [(1, 21, 3), (0, 5, 2), (48, 21, 3), (49, 21, 3), (300, 29, 5), (4, 1, 1)])
+def test_sort_atoms_by_type_equals_the_sort_of_their_slots(B, n, ne):
+    """The sort that builds slot = molIDs * n + atomIDs itself (one launch up to 1024 atoms, the slots
+    through the workspace beyond) against `sort_by_type` of the explicit slots, on ragged batches with
+    elements the model does not know."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(B * 31 + n)
+    counts = rng.integers(1, n + 1, B)
+    aid = np.concatenate([np.arange(c) for c in counts]).astype(np.int32) if B else np.zeros(0, np.int32)
+    mid = np.repeat(np.arange(B), counts).astype(np.int32)
+    types = rng.integers(-1, ne + 1, B * n).astype(np.int32) if B else np.zeros(0, np.int32)
+    got_s, got_o = ops.sort_atoms_by_type(ti32(types), ti32(aid), ti32(mid), n, ne)
+    ref_s, ref_o = ops.sort_by_type(ti32(types), ti32(mid * n + aid), ne)
+    assert torch.equal(got_o, ref_o)
+    total = int(ref_o[-1].item())
+    assert torch.equal(got_s[:total], ref_s[:total]) and (got_s[total:] == 0).all()
+
+
 @pytest.mark.parametrize("R,d,ne,N,A", [(312, 128, 3, 500, 500), (75, 64, 2, 90, 61), (720, 256, 5, 700, 523),
                                         (10, 8, 1, 5, 3), (496, 256, 4, 130, 130),
                                         # up to 128 listed atoms: one workgroup per atom instead of matrix tiles
