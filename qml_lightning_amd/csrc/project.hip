@@ -432,10 +432,15 @@ __global__ __launch_bounds__(256) void zero_untyped_rows_kernel(const int* __res
     zero_untyped_rows(types, N, ne, R, out, blockIdx.x);
 }
 
-// Small batches (a molecule or a few): the tiled kernels above run one or two workgroups through
+// Small batches (a molecule to a few dozen): the tiled kernels above run a few workgroups through
 // ten dependent load-and-multiply steps, 17-26 us for 21 atoms.  Here a workgroup takes ONE atom and
 // spreads the contraction over its threads, so all loads of an atom are in flight at once.
-constexpr int SMALL_ATOMS = 128;   // above, the reductor re-reads from L2 (R d floats per atom) outweigh the latency
+// above these, the reductor re-reads from L2 (R d floats per atom) outweigh the latency: measured
+// cross-over near 1500 atoms at R d = 40 000 (0.077 against 0.100 ms per predict step at 1008 atoms,
+// 0.149 against 0.131 at 2688)
+constexpr int SMALL_ATOMS = 2048;
+constexpr size_t SMALL_READS = 48u << 20;   // floats of reductor read by all workgroups together
+__host__ inline bool small_batch(int A, int R, int d) { return A <= SMALL_ATOMS && (size_t)A * R * d <= SMALL_READS; }
 constexpr int SMALL_KS = 8;        // slices of the contraction in project_small_kernel
 
 __device__ __forceinline__ int type_of_position(const int* __restrict__ type_offsets, int ne, int p) {
@@ -650,7 +655,7 @@ extern "C" int qmll_project_typed(const float* rep, const int* sorted_slots, con
     QMLL_REQUIRE(rep && sorted_slots && type_offsets && reductors && x, QMLL_ERR_INVALID,
                  "qmll_project_typed: null pointer");
     const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(rep) && aligned16(reductors);
-    if (vec && A <= SMALL_ATOMS) {
+    if (vec && small_batch(A, R, d)) {
         const size_t lds = sizeof(float) * (((size_t)R + 3) / 4 * 4 + (size_t)SMALL_KS * d);
         if (lds <= 64 * 1024) {
             hipLaunchKernelGGL(project_small_kernel, dim3(A), dim3(256), lds, (hipStream_t)stream, rep, sorted_slots,
@@ -682,7 +687,7 @@ extern "C" int qmll_project_typed_backward(const float* gx, const int* sorted_sl
     QMLL_REQUIRE(A >= 0 && N >= 0 && ne > 0 && R > 0 && d > 0, QMLL_ERR_INVALID,
                  "qmll_project_typed_backward: bad size A=%d N=%d ne=%d R=%d d=%d", A, N, ne, R, d);
     const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(gx) && aligned16(reductors);
-    const bool small = vec && A > 0 && A <= SMALL_ATOMS && (size_t)d * sizeof(float) <= 64 * 1024 && N <= 64 * 256;
+    const bool small = vec && A > 0 && small_batch(A, R, d) && (size_t)d * sizeof(float) <= 64 * 1024 && N <= 256 * 256;
     if (types && N > 0 && !small) {
         QMLL_REQUIRE(g_rep, QMLL_ERR_INVALID, "qmll_project_typed_backward: null pointer");
         hipLaunchKernelGGL(zero_untyped_rows_kernel, dim3((N + 255) / 256), dim3(256), 0, (hipStream_t)stream, types, N, ne,

@@ -471,9 +471,12 @@ def test_sort_atoms_by_type_equals_the_sort_of_their_slots(B, n, ne):
 
 @pytest.mark.parametrize("R,d,ne,N,A", [(312, 128, 3, 500, 500), (75, 64, 2, 90, 61), (720, 256, 5, 700, 523),
                                         (10, 8, 1, 5, 3), (496, 256, 4, 130, 130),
-                                        # up to 128 listed atoms: one workgroup per atom instead of matrix tiles
-                                        (312, 128, 3, 100, 100), (312, 128, 3, 140, 128), (312, 128, 3, 140, 129),
-                                        (312, 64, 2, 40, 21), (720, 256, 5, 60, 33), (76, 20, 2, 30, 17)])
+                                        # small batches: one workgroup per atom instead of matrix tiles
+                                        (312, 128, 3, 100, 100), (312, 128, 3, 140, 128), (312, 128, 3, 1300, 1201),
+                                        (312, 64, 2, 40, 21), (720, 256, 5, 60, 33), (76, 20, 2, 30, 17),
+                                        # large enough for the matrix tiles at 128 and 64 components (rows in registers
+                                        # in the transpose), and the last size the small kernels take at 312 x 128
+                                        (312, 128, 3, 3000, 2900), (312, 64, 3, 2600, 2500), (312, 128, 3, 1300, 1260)])
 def test_project_typed_forward_and_backward(R, d, ne, N, A):
     """Element-sorted projection against fp64 matmul, both directions: gathered rows, tiles that end
     inside a type, R not a multiple of 4, unknown elements; the matrix-core kernels and the
