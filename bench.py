@@ -198,6 +198,7 @@ def other_configs(torch, dev):
     # one C9H8O4 molecule with the config-2 model: the latency of the step's chain of dependent launches,
     # eager, through forward + autograd.grad, and replayed from a captured HIP graph (each replay checked)
     m2 = sorf_model(SPECIES, NPCAS, NSTACKS, 500)
+    out["c9h8o4_48_molecules"] = predict_rate(m2, coords[:48], charges[:48], True, steps=200, warm=20)   # 1008 atoms
     one = predict_rate(m2, coords[:1], charges[:1], True, steps=200, warm=20)
     data = m2.format_data([coords[0].astype(np.float32)], charges[:1])
     X, Z = data['coordinates'], data['charges']
