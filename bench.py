@@ -631,6 +631,13 @@ def main():
         "two_op_route": two_op_route,
         "from_host_arrays": from_host,
         "kernels": kernels,
+        "step_kernels_sum_ms": 1e3 * sum(kernels[k]["seconds"] for k in ("fchl19_forward", "sort_by_type", "project_typed",
+                                                                        "sorf_energy_fused", "project_typed_backward",
+                                                                        "fchl19_vjp")),
+        "step_kernels_sum_note": "the step's kernels timed one at a time (several launches of one kernel in a row between two "
+                                 "HIP events); inside the step they overlap at their boundaries (a kernel's last workgroups "
+                                 "run beside the next kernel's first) and run at the clock of the whole step, so this sum "
+                                 "exceeds ms_per_step, which is the measured quantity",
     }
     out.update(train)
     if "gram_f64" in kernels:
