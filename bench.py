@@ -334,6 +334,14 @@ def main():
                                "mfma_f32_16x16x4": best["mfma_f32_16x16x4_x32"] / 32 * 1e9},
         "fused_kernel_stack_ns": best["fused_kernel_stack"] * 1e9,
         "fused_kernel_stack_mfma_trial_ns": best["fused_kernel_stack_mfma_trial"] * 1e9,
+        "half_precision_matrix_route": {
+            "mfma_f32_16x16x32_f16_ns": best["mfma_f16_16x16x32_x16"] / 16 * 1e9,
+            "plain_x128_ns": best["plain_fp32_x128"] * 1e9, "mfma_f16_x16_ns": best["mfma_f16_16x16x32_x16"] * 1e9,
+            "both_interleaved_ns": best["plain_fp32_x128_with_mfma_f16_x16"] * 1e9,
+            "split_instruction_ns": best["split_f16_x32"] / 64 * 1e9, "vop3_instruction_ns": best["vop3_fp32_x128"] / 128 * 1e9,
+            "note": "the matrix instructions do not run beside the vector instructions (both_interleaved = the sum, not the "
+                    "longer of the two), and the conversion / mixed-precision instructions of the split cost two plain ones each",
+        },
         "note": "one iteration of fused_kernel_stack = 92 plain + 64 DPP + 16 transcendental wavefront instructions = one "
                 "stack of four atoms at 128 components; the trial replaces the 64 DPP by 16 v_mfma_f32_16x16x4_f32 + 16 plain",
     }
@@ -539,6 +547,23 @@ def main():
         ZTZ, ZTy = model.build_Z_components(tc, tq, E=Et, F=Ft, print_info=False)
         torch.cuda.synchronize()
         t_build = time.perf_counter() - t0
+        # one 500-molecule batch of that build, phase by phase (each timed alone, so their sum exceeds the
+        # batch's share of the build, where the host runs ahead of the device)
+        bd = model.format_data(tc[:500], tq[:500], E=Et[:500], F=Ft[:500])
+        t_rep = timed(lambda: model.rep.get_representation_and_derivative(
+            bd['coordinates'], bd['charges'], bd['atomIDs'], bd['molIDs'], bd['natom_counts'], bd['cells'], bd['inv_cells']), iters=3)
+        t_proj = timed(lambda: model._batch_projected(bd, True), iters=3)
+        proj = model._batch_projected(bd, True)
+        t_rows = timed(lambda: model._rows_from_projected(proj, True), iters=3)
+        brow = model._rows_from_projected(proj, True)
+        btar = model._targets(bd, 500, True, True)
+        bz = torch.zeros(F, F, dtype=torch.float64, device=dev)
+        by = torch.zeros(F, 1, dtype=torch.float64, device=dev)
+        t_bgram = timed(lambda: ops.gram(brow, btar, bz, by, mirror=False), iters=2)
+        batch_phases = {"molecules": 500, "rows": int(brow.shape[0]), "format_data_ms": t_format / (NMOL_TRAIN / 500) * 1e3,
+                        "representation_and_jacobian_ms": t_rep * 1e3, "projection_of_all_rows_ms": (t_proj - t_rep) * 1e3,
+                        "feature_rows_ms": t_rows * 1e3, "gram_ms": t_bgram * 1e3}
+        del bd, proj, brow, btar, bz, by
         # the step after the build: (Z^T Z + lambda I) alpha = Z^T y by the library's blocked
         # Cholesky, with the torch (rocSOLVER) factorisation of the same matrix beside it
         solve = {}
@@ -558,7 +583,7 @@ def main():
         train = {"ztz_seconds": t_build, "ztz_molecules": NMOL_TRAIN, "ztz_rows": M, "ztz_features": F,
                  "ztz_includes": "host format_data + FCHL19 Jacobian + projection + SORF rows + Gram, 500 molecules per batch",
                  "ztz_seconds_excluding_format_data": t_build - t_format, "format_data_seconds": t_format,
-                 "gram_kernel_seconds": t_gram}
+                 "gram_kernel_seconds": t_gram, "one_batch_phases": batch_phases}
         train.update(solve)
         if solve:
             kernels["cholesky_solve_f64"] = {"seconds": solve["solve_seconds"], "bound": "mfma",

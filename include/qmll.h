@@ -272,6 +272,18 @@ int qmll_sort_by_type_noalloc(const int* types, const int* slots, int A, int ne,
 int qmll_project_typed(const float* rep, const int* sorted_slots, const int* type_offsets, const float* reductors,
                        int A, int ne, int R, int d, float* x, qmll_stream_t stream);
 
+/* The same product for `group` rows per atom: rows f32 [N*group, R] holds rows
+ * slot*group ... slot*group + group - 1 for every slot, x f32 [A*group, d] receives
+ * x[a*group + g, :] = rows[sorted_slots[a]*group + g, :] . reductors[type of a].  With
+ * group = 3n and rows = the FCHL19 Jacobian [N, n, 3, R] this is the projection of the
+ * derivative rows of every element in one launch, in place of the per-element
+ * index_select + torch.matmul of the reference (qml_lightning/models/kernel.py:143-160,
+ * representations/dimensionality_reduction.py:61-72); the rows of element t are
+ * x[type_offsets[t]*group : type_offsets[t+1]*group].  A*group must stay below 2^31 - 128. */
+int qmll_project_typed_rows(const float* rows, const int* sorted_slots, const int* type_offsets,
+                            const float* reductors, int A, int ne, int R, int d, int group, float* x,
+                            qmll_stream_t stream);
+
 /* Transpose of qmll_project_typed: g_rep[sorted_slots[a], :] = gx[a, :] . reductors[type]^T
  * (g_rep f32 [N,R]).  Rows of slots that are not in the sorted list are not written, except
  * that with types != NULL (i32 [N]) the rows of slots whose type is outside [0,ne) are set
@@ -401,7 +413,10 @@ double qmll_probe_rate(int which, int iters, int blocks_per_cu, void* out, qmll_
  * registers: mix = 0 128 plain fp32, 1 128 DPP fmac, 2 128 v_sin_f32, 3 32 v_mfma_f32_16x16x4_f32,
  * 4 the per-stack mix of the fused kernel at 128 components (92 plain + 64 DPP + 16
  * transcendental), 5 the same with the in-row stages as 16 matrix instructions and 16 more plain
- * ones instead of the 64 DPP.  Returns wavefront-iterations per SIMD (blocks_per_cu x iters), so
+ * ones instead of the 64 DPP, 6 16 v_mfma_f32_16x16x32_f16, 7 the 128 plain fp32 of mix 0 with the 16
+ * matrix instructions of mix 6 spread between them, 8 the split of 32 fp32 values into two fp16
+ * parts each (64 instructions), 9 128 v_mul_f32 in the 64-bit encoding (a source modifier).
+ * Returns wavefront-iterations per SIMD (blocks_per_cu x iters), so
  * duration x clock / that = SIMD clocks per iteration; negative on error. */
 double qmll_probe_mix(int mix, int iters, int blocks_per_cu, void* out, qmll_stream_t stream);
 

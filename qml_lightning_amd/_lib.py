@@ -58,6 +58,7 @@ PROTOTYPES = {
     "qmll_sort_atoms_by_type": [P, P, P, c_int, c_int, c_int, P, c_size_t, P, P, P],
     "qmll_sort_by_type_noalloc": [P, P, c_int, c_int, P, P, P],
     "qmll_project_typed": [P, P, P, P, c_int, c_int, c_int, c_int, P, P],
+    "qmll_project_typed_rows": [P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
     "qmll_project_typed_backward": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
     "qmll_sorf_energy_sorted": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_float, P, P, P],
     "qmll_rff_features": [P, P, P, P, c_int, c_int, c_int, c_int, P, P],

@@ -112,9 +112,19 @@ __global__ __launch_bounds__(PT) void probe_exp_kernel(int iters, float* __restr
 //   MIX_MFMA_TRIAL 108 plain fp32 + 16 transcendental + 16 v_mfma_f32_16x16x4_f32: the in-row stages
 //                  (a 16-point +-1 Hadamard block per 16 lanes, forward and adjoint, 2 x 2 tiles x K = 16)
 //                  on the matrix pipe, 16 plain instructions for the operand layout, no data movement
-enum { MIX_PLAIN = 0, MIX_DPP = 1, MIX_TRANS = 2, MIX_MFMA16 = 3, MIX_FUSED = 4, MIX_MFMA_TRIAL = 5, MIX_COUNT = 6 };
+// and the pieces of a half-precision form of those stages (a 16-point +-1 block is exact in fp16, the
+// fp32 operand being split into two fp16 parts):
+//   MIX_MFMA_F16      16 v_mfma_f32_16x16x32_f16
+//   MIX_PLAIN_MFMA_F16 the 128 plain instructions of MIX_PLAIN with those 16 matrix instructions spread
+//                  between them (independent registers): the time of the two together against their sum
+//   MIX_SPLIT_F16  the split of 32 fp32 values: per pair v_cvt_pkrtz_f16_f32, two v_fma_mix_f32
+//                  (value - first part), v_cvt_pkrtz_f16_f32 = 64 instructions
+//   MIX_VOP3       128 v_mul_f32 with a source modifier, i.e. in the 64-bit encoding
+enum { MIX_PLAIN = 0, MIX_DPP = 1, MIX_TRANS = 2, MIX_MFMA16 = 3, MIX_FUSED = 4, MIX_MFMA_TRIAL = 5, MIX_MFMA_F16 = 6,
+       MIX_PLAIN_MFMA_F16 = 7, MIX_SPLIT_F16 = 8, MIX_VOP3 = 9, MIX_COUNT = 10 };
 
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 
 template <int N>
 __device__ __forceinline__ void plain_ops(float (&v)[8], float c) {
@@ -138,6 +148,30 @@ __device__ __forceinline__ void mfma_ops(float4_t (&acc)[4], float a, float b) {
     for (int k = 0; k < N; ++k) acc[k & 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[k & 3], 0, 0, 0);
 }
 
+template <int N>
+__device__ __forceinline__ void mfma_f16_ops(float4_t (&acc)[4], half8_t a, half8_t b) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) acc[k & 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[k & 3], 0, 0, 0);
+}
+template <int N>
+__device__ __forceinline__ void vop3_ops(float (&v)[8], float c) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) asm volatile("v_mul_f32_e64 %0, %0, -%1" : "+v"(v[k & 7]) : "v"(c));
+}
+// two fp16 parts of each of 8 fp32 values; the parts are folded into `sink` so that they stay live
+__device__ __forceinline__ void split_f16_ops(float (&v)[8], unsigned& sink) {
+#pragma unroll
+    for (int k = 0; k < 8; k += 2) {
+        unsigned h1, h2;
+        float r0, r1;
+        asm volatile("v_cvt_pkrtz_f16_f32 %0, %1, %2" : "=v"(h1) : "v"(v[k]), "v"(v[k + 1]));
+        asm volatile("v_fma_mix_f32 %0, -%1, 1.0, %2 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(r0) : "v"(h1), "v"(v[k]));
+        asm volatile("v_fma_mix_f32 %0, -%1, 1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r1) : "v"(h1), "v"(v[k + 1]));
+        asm volatile("v_cvt_pkrtz_f16_f32 %0, %1, %2" : "=v"(h2) : "v"(r0), "v"(r1));
+        sink ^= h2;
+    }
+}
+
 template <int MIX>
 __global__ __launch_bounds__(PT) void probe_mix_kernel(int iters, float* __restrict__ out) {
     float v[8];
@@ -148,6 +182,13 @@ __global__ __launch_bounds__(PT) void probe_mix_kernel(int iters, float* __restr
 #pragma unroll
     for (int k = 0; k < 4; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
     const float a = 1e-3f * (float)(threadIdx.x & 7), b = (threadIdx.x & 2) ? 1.0f : -1.0f;
+    half8_t ah, bh;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        ah[k] = (_Float16)(((threadIdx.x + k) & 1) ? 1.0f : -1.0f);
+        bh[k] = (_Float16)(0.01f * (float)(threadIdx.x & 15));
+    }
+    unsigned sink = 0;
     for (int it = 0; it < iters; ++it) {
         if constexpr (MIX == MIX_PLAIN) plain_ops<128>(v, c);
         if constexpr (MIX == MIX_DPP) dpp_ops<128>(v, c);
@@ -173,8 +214,23 @@ __global__ __launch_bounds__(PT) void probe_mix_kernel(int iters, float* __restr
             mfma_ops<8>(acc, a, b);
             plain_ops<36>(v, c);
         }
+        if constexpr (MIX == MIX_MFMA_F16) mfma_f16_ops<16>(acc, ah, bh);
+        if constexpr (MIX == MIX_PLAIN_MFMA_F16) {
+#pragma unroll
+            for (int g = 0; g < 16; ++g) {
+                mfma_f16_ops<1>(acc, ah, bh);
+                plain_ops<8>(v, c);
+            }
+        }
+        if constexpr (MIX == MIX_SPLIT_F16) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                split_f16_ops(v, sink);
+            }
+        }
+        if constexpr (MIX == MIX_VOP3) vop3_ops<128>(v, c);
     }
-    float s = 0.0f;
+    float s = (float)(sink & 1u);
 #pragma unroll
     for (int k = 0; k < 8; ++k) s += v[k];
 #pragma unroll
@@ -260,7 +316,11 @@ extern "C" double qmll_probe_mix(int mix, int iters, int blocks_per_cu, void* ou
         case MIX_TRANS: hipLaunchKernelGGL(probe_mix_kernel<MIX_TRANS>, grid, block, 0, st, iters, o); break;
         case MIX_MFMA16: hipLaunchKernelGGL(probe_mix_kernel<MIX_MFMA16>, grid, block, 0, st, iters, o); break;
         case MIX_FUSED: hipLaunchKernelGGL(probe_mix_kernel<MIX_FUSED>, grid, block, 0, st, iters, o); break;
-        default: hipLaunchKernelGGL(probe_mix_kernel<MIX_MFMA_TRIAL>, grid, block, 0, st, iters, o); break;
+        case MIX_MFMA_TRIAL: hipLaunchKernelGGL(probe_mix_kernel<MIX_MFMA_TRIAL>, grid, block, 0, st, iters, o); break;
+        case MIX_MFMA_F16: hipLaunchKernelGGL(probe_mix_kernel<MIX_MFMA_F16>, grid, block, 0, st, iters, o); break;
+        case MIX_PLAIN_MFMA_F16: hipLaunchKernelGGL(probe_mix_kernel<MIX_PLAIN_MFMA_F16>, grid, block, 0, st, iters, o); break;
+        case MIX_SPLIT_F16: hipLaunchKernelGGL(probe_mix_kernel<MIX_SPLIT_F16>, grid, block, 0, st, iters, o); break;
+        default: hipLaunchKernelGGL(probe_mix_kernel<MIX_VOP3>, grid, block, 0, st, iters, o); break;
     }
     if (hipGetLastError() != hipSuccess) {
         qmll_set_error("qmll_probe_mix: launch failed");

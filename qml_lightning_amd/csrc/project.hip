@@ -160,11 +160,12 @@ constexpr int PK = 32;             // contraction chunk staged in LDS
 constexpr int PKS = PK + 4;        // LDS row stride of k-contiguous tiles: 16-byte reads of 16
                                    // consecutive rows fall into 16 distinct groups of 4 banks
 
-// which sorted rows a workgroup owns: tiles never straddle two types
+// which sorted rows a workgroup owns: tiles never straddle two types.  group: rows per sorted
+// entry (1 for one row per atom; the offsets count entries)
 __device__ __forceinline__ bool tile_of_block(const int* __restrict__ offsets, int ne, int b, int& type, int& row0,
-                                              int& rows) {
+                                              int& rows, int group = 1) {
     for (int t = 0; t < ne; ++t) {
-        const int o0 = offsets[t], o1 = offsets[t + 1];
+        const int o0 = offsets[t] * group, o1 = offsets[t + 1] * group;
         const int nt = (o1 - o0 + PM - 1) / PM;
         if (b < nt) {
             type = t;
@@ -188,12 +189,15 @@ __global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(PNT > 64 ? 3
                                                          const int* __restrict__ a_rows, const float* __restrict__ Bm,
                                                          size_t b_type_stride, int ldb, float* __restrict__ C, int ldc,
                                                          const int* __restrict__ c_rows,
-                                                         const int* __restrict__ offsets, int ne, int K, int N) {
+                                                         const int* __restrict__ offsets, int ne, int K, int N,
+                                                         int group = 1) {
+    // group > 1: every sorted entry stands for `group` consecutive rows, entry e of the list being rows
+    // a_rows[e] * group ... of A and rows e * group ... of C (the 3n derivative rows of an atom)
     __shared__ __attribute__((aligned(16))) float sA[PM * PKS];
     constexpr int NJ = PNT / 32;       // 32-column MFMA blocks per wavefront
     __shared__ __attribute__((aligned(16))) float sB[BT ? PNT * PKS : PK * PNT];   // BT: [PNT][PKS]; else [PK][PNT], rotated rows
     int type, row0, rows;
-    if (!tile_of_block(offsets, ne, blockIdx.x, type, row0, rows)) return;
+    if (!tile_of_block(offsets, ne, blockIdx.x, type, row0, rows, group)) return;
     const int col0 = blockIdx.y * PNT;
     const float* Bt = Bm + (size_t)type * b_type_stride;
 
@@ -208,8 +212,16 @@ __global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(PNT > 64 ? 3
     for (int v = 0; v < 4; ++v) {
         const int r = ar + 32 * v;
         arow_ok[v] = r < rows;
-        const int src = arow_ok[v] ? (a_rows ? a_rows[row0 + r] : row0 + r) : 0;
-        arow[v] = A + (size_t)src * lda;
+        size_t src = 0;
+        if (arow_ok[v]) {
+            if (group > 1) {
+                const int e = (row0 + r) / group;
+                src = (size_t)a_rows[e] * group + (size_t)(row0 + r - e * group);
+            } else {
+                src = (size_t)(a_rows ? a_rows[row0 + r] : row0 + r);
+            }
+        }
+        arow[v] = A + src * lda;
     }
     // B tile: !BT 32 k x PNT n = 8 PNT float4 -> k = tid/(PNT/4) + (1024/PNT) v, n4 = tid%(PNT/4)
     //          BT PNT n x 32 k = 8 PNT float4 -> n = tid/8 + 32v,  k4 = tid%8
@@ -678,6 +690,37 @@ extern "C" int qmll_project_typed(const float* rep, const int* sorted_slots, con
         hipLaunchKernelGGL((typed_gemm_kernel<false, false, PN>), grid, dim3(PT), 0, (hipStream_t)stream, rep, R,
                            sorted_slots, reductors, (size_t)R * d, d, x, d, (const int*)nullptr, type_offsets, ne, R, d);
     QMLL_CHECK_LAUNCH("qmll_project_typed");
+    return QMLL_OK;
+}
+
+extern "C" int qmll_project_typed_rows(const float* rows, const int* sorted_slots, const int* type_offsets,
+                                       const float* reductors, int A, int ne, int R, int d, int group, float* x,
+                                       qmll_stream_t stream) {
+    QMLL_REQUIRE(A >= 0 && ne > 0 && R > 0 && d > 0 && group > 0, QMLL_ERR_INVALID,
+                 "qmll_project_typed_rows: bad size A=%d ne=%d R=%d d=%d group=%d", A, ne, R, d, group);
+    if (A == 0) return QMLL_OK;
+    QMLL_REQUIRE(rows && sorted_slots && type_offsets && reductors && x, QMLL_ERR_INVALID,
+                 "qmll_project_typed_rows: null pointer");
+    QMLL_REQUIRE((long long)A * group < (1ll << 31) - PM, QMLL_ERR_INVALID,
+                 "qmll_project_typed_rows: %d atoms x %d rows exceed the 32-bit row count of one launch", A, group);
+    const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(rows) && aligned16(reductors);
+    const long long nrows = (long long)A * group;
+    const int tiles = (int)((nrows + PM - 1) / PM) + ne;
+    const bool wide = vec && d % 128 == 0 && (long long)tiles * (d / 128) >= 2 * 256;
+    const dim3 grid(tiles, wide ? d / 128 : (d + PN - 1) / PN);
+    if (wide)
+        hipLaunchKernelGGL((typed_gemm_kernel<false, true, 128>), grid, dim3(PT), 0, (hipStream_t)stream, rows, R,
+                           sorted_slots, reductors, (size_t)R * d, d, x, d, (const int*)nullptr, type_offsets, ne, R, d,
+                           group);
+    else if (vec)
+        hipLaunchKernelGGL((typed_gemm_kernel<false, true, PN>), grid, dim3(PT), 0, (hipStream_t)stream, rows, R,
+                           sorted_slots, reductors, (size_t)R * d, d, x, d, (const int*)nullptr, type_offsets, ne, R, d,
+                           group);
+    else
+        hipLaunchKernelGGL((typed_gemm_kernel<false, false, PN>), grid, dim3(PT), 0, (hipStream_t)stream, rows, R,
+                           sorted_slots, reductors, (size_t)R * d, d, x, d, (const int*)nullptr, type_offsets, ne, R, d,
+                           group);
+    QMLL_CHECK_LAUNCH("qmll_project_typed_rows");
     return QMLL_OK;
 }
 

@@ -16,7 +16,6 @@ import torch
 
 from .. import ops
 from ..cuda.utils_gpu import matmul_and_reduce
-from ..representations.dimensionality_reduction import project_derivative, project_representation
 
 
 def _default_device():
@@ -96,19 +95,32 @@ class BaseKernel():
                                                          inv_cells)
             rep_derivative = None
         flat_rep = representation.view(B * n, -1)
-        flat_jac = rep_derivative.view(B * n, n, 3, -1) if with_forces else None
-        items = []
+        # the atoms of every element, element after element in the order of the projection matrices:
+        # one typed product then serves all elements (for the derivative rows, 3n rows per atom), where
+        # the reference copies each element's rows out and multiplies them one element at a time
+        ne = self.reductors.shape[0]
+        lists = [None] * ne
         for e in self.elements:
-            idx = self._element_index(data, charges, int(e))
-            if idx.shape[0] == 0:
-                continue
-            element_idx = self.element2index[int(e)]
-            batch_indexes = torch.div(idx, n, rounding_mode='floor').to(torch.int32)
-            sub = project_representation(flat_rep.index_select(0, idx), self.reductors[element_idx])
-            sub_grad = None
+            lists[self.element2index[int(e)]] = (e, self._element_index(data, charges, int(e)))
+        counts = [0 if l is None else int(l[1].shape[0]) for l in lists]
+        offsets = np.concatenate(([0], np.cumsum(counts))).astype(np.int32)
+        items = []
+        if offsets[-1] > 0:
+            slots = torch.cat([l[1] for l in lists if l is not None and l[1].shape[0] > 0]).to(torch.int32)
+            type_offsets = torch.from_numpy(offsets).to(slots.device)
+            # the tiled product for both: a row's result then does not depend on how many rows the batch has
+            x_all = ops.project_typed_rows(flat_rep, slots, type_offsets, self.reductors, 1)
+            g_all = None
             if with_forces:
-                sub_grad = project_derivative(flat_jac.index_select(0, idx), self.reductors[element_idx])
-            items.append((e, batch_indexes, sub, sub_grad))
+                g_all = ops.project_typed_rows(rep_derivative.view(B * n * n * 3, -1), slots, type_offsets,
+                                               self.reductors, 3 * n)
+            mol_of_atom = torch.div(slots, n, rounding_mode='floor')
+            for t, l in enumerate(lists):
+                if counts[t] == 0:
+                    continue
+                o0, o1 = int(offsets[t]), int(offsets[t + 1])
+                sub_grad = g_all[o0 * 3 * n:o1 * 3 * n].view(o1 - o0, n, 3, -1) if with_forces else None
+                items.append((l[0], mol_of_atom[o0:o1], x_all[o0:o1], sub_grad))
         return {'B': B, 'n': n, 'device': coordinates.device, 'items': items}
 
     def _rows_from_projected(self, proj, with_forces, zero_energy_rows=False):

@@ -432,6 +432,23 @@ def project_typed(rep, sorted_slots, type_offsets, reductors):
     return x
 
 
+def project_typed_rows(rows, sorted_slots, type_offsets, reductors, group):
+    """x [A*group,d]: x[a*group+g] = rows[sorted_slots[a]*group+g] . reductors[type of a]
+    (rows [N*group,R], `group` consecutive rows per slot; reductors [ne,R,d])."""
+    rows, reductors = _f32(rows), _f32(reductors)
+    sorted_slots, type_offsets = _i32(sorted_slots), _i32(type_offsets)
+    ne, R, d = reductors.shape
+    group = int(group)
+    if rows.dim() != 2 or rows.shape[1] != R or type_offsets.shape[0] != ne + 1 or group < 1 or rows.shape[0] % group:
+        raise RuntimeError("project_typed_rows: rows %s, reductors %s, %d offsets, group %d do not fit together"
+                           % (tuple(rows.shape), tuple(reductors.shape), type_offsets.shape[0], group))
+    A = int(sorted_slots.shape[0])
+    x = torch.empty((A * group, d), dtype=torch.float32, device=rows.device)
+    check(_lib.lib().qmll_project_typed_rows(_ptr(rows), _ptr(sorted_slots), _ptr(type_offsets), _ptr(reductors), A, ne, R,
+                                             d, group, _ptr(x), _stream()), "qmll_project_typed_rows")
+    return x
+
+
 def project_typed_backward(gx, sorted_slots, type_offsets, reductors, types, nslots):
     """g_rep [nslots,R] with g_rep[sorted_slots[a]] = gx[a] . reductors[type]^T, zero elsewhere."""
     gx, reductors = _f32(gx), _f32(reductors)

@@ -60,7 +60,8 @@ def measure(nbytes=1 << 30, device="cuda:0"):
 
 
 MIXES = ("plain_fp32_x128", "dpp_fmac_x128", "transcendental_x128", "mfma_f32_16x16x4_x32", "fused_kernel_stack",
-         "fused_kernel_stack_mfma_trial")
+         "fused_kernel_stack_mfma_trial", "mfma_f16_16x16x32_x16", "plain_fp32_x128_with_mfma_f16_x16", "split_f16_x32",
+         "vop3_fp32_x128")
 
 
 def instruction_mixes(device="cuda:0", iters=2000):

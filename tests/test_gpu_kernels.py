@@ -507,6 +507,35 @@ def test_project_typed_forward_and_backward(R, d, ne, N, A):
     assert (g.cpu().numpy()[mask] == 0).all()
 
 
+@pytest.mark.parametrize("R,d,ne,N,A,group", [(312, 128, 3, 80, 61, 63), (53, 20, 2, 40, 40, 7), (312, 128, 3, 600, 600, 9),
+                                               (64, 256, 4, 30, 17, 36)])
+def test_project_typed_rows_projects_a_group_of_rows_per_atom(R, d, ne, N, A, group):
+    """`group` rows per slot (the 3n derivative rows of an atom) through the typed product, against
+    fp64 matmul of each atom's rows with its element's matrix: tiles that start and end inside an atom's
+    group and inside a type, an element without atoms, unknown elements, R not a multiple of 4."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(R + d + group)
+    rows = rng.normal(size=(N * group, R)).astype(np.float32)
+    red = rng.normal(size=(ne, R, d)).astype(np.float32)
+    types = rng.integers(0, ne, N).astype(np.int32)
+    if ne > 2:
+        types[types == 1] = 0                      # no atom of element 1
+    types[rng.choice(N, size=max(1, N // 20), replace=False)] = -1
+    slots = np.sort(rng.choice(N, size=A, replace=False)).astype(np.int32)
+    ss, off = ops.sort_by_type(ti32(types), ti32(slots), ne)
+    x = ops.project_typed_rows(t32(rows), ss, off, t32(red), group)
+    assert tuple(x.shape) == (A * group, d)
+    ssn, total = ss.cpu().numpy(), int(off[-1].item())
+    assert total > 0
+    r3 = rows.reshape(N, group, R).astype(np.float64)
+    x_ref = np.concatenate([r3[s_] @ red[types[s_]].astype(np.float64) for s_ in ssn[:total]])
+    close(x[:total * group], x_ref, REL_REP, "projection of grouped rows")
+    # group = 1 is the plain projection
+    x1 = ops.project_typed_rows(t32(rows[:N]), ss, off, t32(red), 1)
+    close(x1[:total], ops.project_typed(t32(rows[:N]), ss, off, t32(red))[:total].double().cpu().numpy(), REL_REP,
+          "one row per atom")
+
+
 @pytest.mark.parametrize("T,S,d", [(1, 6, 64), (2, 6, 64), (1, 64, 128), (1, 70, 64), (2, 64, 64)])
 def test_sorted_fused_energy_matches_per_atom_oracle(T, S, d):
     """Element-sorted rows through the fused kernel: energies land in the atoms' slots, the
