@@ -580,6 +580,14 @@ def main():
         gram_flops = float(M) * F * (F + 1) + 2.0 * M * F
         kernels["gram_f64"] = {"seconds": t_gram, "bound": "mfma", "TFLOPs": gram_flops / t_gram / 1e12,
                                "frac": gram_flops / t_gram / 1e12 / FP64_PEAK_TFLOPS}
+        # half the width: 64 x 64 tiles, whose 28 strictly-upper super-tiles do not divide by the 8 XCDs
+        rows_h = rows[:32000, :F // 2].contiguous()
+        ZTZ_h = torch.zeros(F // 2, F // 2, dtype=torch.float64, device=dev)
+        t_gram_h = timed(lambda: ops.gram(rows_h, None, ZTZ_h, None), iters=3)
+        fl_h = 32000.0 * (F // 2) * (F // 2 + 1)
+        kernels["gram_f64_half_width"] = {"seconds": t_gram_h, "bound": "mfma", "rows": 32000, "features": F // 2,
+                                          "TFLOPs": fl_h / t_gram_h / 1e12, "frac": fl_h / t_gram_h / 1e12 / FP64_PEAK_TFLOPS}
+        del rows_h, ZTZ_h
         train = {"ztz_seconds": t_build, "ztz_molecules": NMOL_TRAIN, "ztz_rows": M, "ztz_features": F,
                  "ztz_includes": "host format_data + FCHL19 Jacobian + projection + SORF rows + Gram, 500 molecules per batch",
                  "ztz_seconds_excluding_format_data": t_build - t_format, "format_data_seconds": t_format,

@@ -15,13 +15,13 @@
 // panel by the tiles of one row/column are served from L2: consecutive workgroup ids walk
 // along a tile row).
 #include "qmll_common.h"
+#include "gram_tiles.h"
 
 namespace {
 
 typedef double double4_t __attribute__((ext_vector_type(4)));
 typedef double double2_t __attribute__((ext_vector_type(2)));
 
-constexpr int TILE = 128;     // C tile edge per workgroup
 constexpr int KB = 16;        // rows of Z staged per step
 constexpr int NWAVE = 8;      // wavefronts per workgroup: 2 along i x NWAVE/2 along j
 constexpr int GT = 64 * NWAVE;
@@ -33,67 +33,6 @@ constexpr int UN = CPT / 2;              // 16-byte units per thread
 // doubles per staged row: 128 + 16, i.e. consecutive rows start 32 banks apart, so the two
 // k-rows a half-wavefront reads in one ds_read_b64 never share a bank
 constexpr int LDS_STRIDE = TILE + 16;
-constexpr int SUPER = 8;      // tiles per edge of a super-tile (L2 locality unit)
-constexpr int NXCD = 8;       // workgroup ids go round-robin over the 8 XCDs
-
-// Workgroup id -> C tile.  Hardware deals consecutive workgroup ids to the 8 XCDs in turn
-// and every XCD has its own L2.  The tiles are grouped in super-tiles of 8x8, dealt to the
-// XCDs round-robin; the k-th workgroup of an XCD works on tile k%64 of that XCD's (k/64)-th
-// super-tile, so the ~64 tiles an XCD runs at a time share 16 panels of Z.
-// Symmetric mode: every XCD must get the same number of REAL tiles per id range, because
-// ids are handed out in order and a full XCD holds back the ids of the others.  So the
-// super-tiles strictly above the diagonal (64 tiles each) are dealt first, then the diagonal
-// super-tiles, whose 36 tiles on or above the diagonal are numbered without gaps.
-constexpr int DIAG_TILES = SUPER * (SUPER + 1) / 2;
-
-struct TileMap {
-    int off_per;    // strictly-upper super-tiles per XCD (symmetric) / all super-tiles per XCD
-    int diag_per;   // diagonal super-tiles per XCD (symmetric mode only)
-    // split launch of the last tiles (symmetric mode with a workspace, see gram_launch): workgroup w
-    // takes rows [piece * piece_rows, ...) of tile id tail_first + w / pieces, piece = w % pieces, and
-    // writes its partial tile to the workspace; pieces = 0: the ordinary launch
-    int pieces;
-    int piece_rows;
-    unsigned tail_first;
-};
-
-template <bool SYM>
-__host__ __device__ __forceinline__ void tile_of_block(unsigned b, int nti, int ntj, TileMap tm, int& ti, int& tj) {
-    const unsigned xcd = b % NXCD, k = b / NXCD;
-    const int sr_n = (nti + SUPER - 1) / SUPER, sc_n = (ntj + SUPER - 1) / SUPER;
-    ti = tj = -1;
-    if (!SYM) {
-        const unsigned g = (k / (SUPER * SUPER)) * NXCD + xcd;
-        const unsigned in_super = k % (SUPER * SUPER);
-        const int sr = (int)(g / sc_n), sc = (int)(g % sc_n);
-        if (sr >= sr_n) return;
-        ti = sr * SUPER + (int)(in_super / SUPER);
-        tj = sc * SUPER + (int)(in_super % SUPER);
-    } else if (k < (unsigned)tm.off_per * (SUPER * SUPER)) {
-        const unsigned g = (k / (SUPER * SUPER)) * NXCD + xcd;
-        const unsigned in_super = k % (SUPER * SUPER);
-        const int n1 = sc_n - 1;                                // row r holds n1 - r super-tiles
-        if (g >= (unsigned)(sc_n * n1 / 2)) return;
-        const float bb = (float)(2 * n1 + 1);
-        int r = (int)((bb - sqrtf(fmaxf(bb * bb - 8.0f * (float)g, 0.0f))) * 0.5f);
-        r = r < 0 ? 0 : (r > n1 - 1 ? n1 - 1 : r);
-        while (r > 0 && (unsigned)(r * n1 - (r * (r - 1)) / 2) > g) --r;
-        while (r + 1 < n1 && (unsigned)((r + 1) * n1 - ((r + 1) * r) / 2) <= g) ++r;
-        const int sc = r + 1 + (int)(g - (unsigned)(r * n1 - (r * (r - 1)) / 2));
-        ti = r * SUPER + (int)(in_super / SUPER);
-        tj = sc * SUPER + (int)(in_super % SUPER);
-    } else {
-        const unsigned k2 = k - (unsigned)tm.off_per * (SUPER * SUPER);
-        const unsigned dg = (k2 / DIAG_TILES) * NXCD + xcd;
-        if (dg >= (unsigned)sc_n) return;
-        int t = (int)(k2 % DIAG_TILES), a = 0;
-        while (t >= SUPER - a) { t -= SUPER - a; ++a; }         // row a of the triangle holds 8 - a tiles
-        ti = (int)dg * SUPER + a;
-        tj = (int)dg * SUPER + a + t;
-    }
-    if (ti >= nti || tj >= ntj) ti = tj = -1;
-}
-
 // GUARD: some panel sticks out of the matrix (F or the row block not a multiple of 128, or
 // odd F): every element load is bounds-checked.  !GUARD: whole panels, 16-byte vector loads.
 // GEN: general operands for the Cholesky updates (separate A operand Za, row strides, sign,
@@ -371,21 +310,8 @@ static int gram_launch(const double* Z, const double* y, int M, int F, int f0, i
     const int ntj = (F + TILE - 1) / TILE;
     const int nti = sym ? ntj : (f1 - f0 + TILE - 1) / TILE;
     // super-tiles are dealt round-robin to the XCDs; ids of tiles outside the matrix exit at once
-    const long long sr = (nti + SUPER - 1) / SUPER, sc = (ntj + SUPER - 1) / SUPER;
-    TileMap tm;
     long long per_xcd;
-    if (sym) {
-        tm.off_per = (int)((sc * (sc - 1) / 2 + NXCD - 1) / NXCD);
-        tm.diag_per = (int)((sc + NXCD - 1) / NXCD);
-        per_xcd = (long long)tm.off_per * SUPER * SUPER + (long long)tm.diag_per * DIAG_TILES;
-    } else {
-        tm.off_per = (int)((sr * sc + NXCD - 1) / NXCD);
-        tm.diag_per = 0;
-        per_xcd = (long long)tm.off_per * SUPER * SUPER;
-    }
-    tm.pieces = 0;
-    tm.piece_rows = 0;
-    tm.tail_first = 0;
+    TileMap tm = gram_tile_map(nti, ntj, sym, per_xcd);
     long long nblocks = per_xcd * NXCD;
     QMLL_REQUIRE(nblocks < 2147483647LL, QMLL_ERR_INVALID, "%s: too many tiles", who);
     // The tiles run in rounds of one per workgroup slot (two per CU); when the last round is less

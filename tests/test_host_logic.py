@@ -1,6 +1,9 @@
 """Host-side logic that needs no GPU: batch formatting, targets layout, model attributes
 and TorchScript compilation of the forward methods."""
+import os
+
 import numpy as np
+import pytest
 import torch
 
 from oracle import model as omodel
@@ -182,3 +185,21 @@ def test_closed_form_pair_unranking_is_exact():
             sq = np.nextafter(sq, f32(np.inf if push > 0 else -np.inf)).astype(np.float32)
         k = (f32(0.5) + sq).astype(np.float32).astype(np.int64)       # conversion truncates
         assert np.array_equal(k, kk) and np.array_equal(t - k * (k - 1) // 2, jj), push
+
+
+def test_gram_tile_map_meets_every_tile_once_and_balances_the_xcds(tmp_path):
+    """tests/cpp/check_gram_tiles.cpp walks the Gram kernel's workgroup-id -> tile map (the header the
+    kernel and its launch use) for 1..140 tiles per edge: every tile on or above the diagonal exactly
+    once, nothing below it, XCD shares within one tile of each other for whole super-tiles; the full
+    mode every tile once."""
+    import shutil
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    if shutil.which("g++") is None:
+        pytest.skip("needs g++")
+    exe = str(tmp_path / "check_gram_tiles")
+    subprocess.run(["g++", "-O2", "-std=c++17", "-I", os.path.join(root, "qml_lightning_amd", "csrc"),
+                    os.path.join(root, "tests", "cpp", "check_gram_tiles.cpp"), "-o", exe], check=True)
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert out.stdout.startswith("ok")
