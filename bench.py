@@ -615,7 +615,7 @@ def main():
         if v["bound"] == "hbm" and "GBs" in v:
             v["frac_of_measured"] = v["GBs"] / max(peaks["hbm_fill_GBs"], peaks["hbm_copy_GBs"])
         elif v["bound"] == "mfma":
-            ref = peaks["mfma_f64_TFLOPs"] if k in ("gram_f64", "cholesky_solve_f64") else peaks["mfma_f32_TFLOPs"]
+            ref = peaks["mfma_f64_TFLOPs"] if k in ("gram_f64", "gram_f64_half_width", "cholesky_solve_f64") else peaks["mfma_f32_TFLOPs"]
             v["frac_of_measured"] = v["TFLOPs"] / ref
         elif "exp_per_s" in v:
             v["frac"] = v["exp_per_s"] / exp_nominal
