@@ -572,8 +572,11 @@ def test_sorted_fused_energy_matches_per_atom_oracle(T, S, d):
 
 
 # ---------------------------------------------------------------------------------------
-@pytest.mark.parametrize("M,F", [(37, 24), (300, 128), (1000, 384), (513, 200), (40, 2176), (33, 3000), (20, 4224)])
+@pytest.mark.parametrize("M,F", [(37, 24), (300, 128), (1000, 384), (513, 200), (40, 2176), (33, 3000), (20, 4224),
+                                 (18, 1100), (25, 8200)])
 def test_gram_matches_fp64_matmul(M, F):
+    """Widths from one tile to 65 tiles per edge: whole super-tiles per XCD, left-over super-tiles shared
+    row by row (4 of 36 at F = 8200), left-over diagonal super-tiles dealt tile by tile, partial tiles."""
     from qml_lightning_amd import ops
     rng = np.random.default_rng(M)
     Zr = rng.normal(size=(M, F))
