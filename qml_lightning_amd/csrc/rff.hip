@@ -384,6 +384,295 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
     }
 }
 
+// The same chain on the half-precision matrix cores.  v_mfma_f32_32x32x16_f16 runs 13 times as fast per
+// flop as the fp32 instruction above, so each fp32 operand is split into two fp16 parts (hi = the value
+// rounded to fp16, lo = the rounded rest: 22 bits together) and a product becomes three matrix
+// instructions, hi.hi + hi.lo + lo.hi, accumulated in fp32; lo.lo is below the rounding of the sum.
+// fp16 has five exponent bits, so every operand is scaled by a power of two first (exact): x by the
+// wavefront's 2^kx (largest |x| of its 32 atoms to [2^13, 2^14)), alpha by the workgroup's 2^kp (largest
+// |alpha| norm of its feature range), every chunk of W by its own 2^kw (largest |W| of the chunk); the
+// sine argument, the chunk's contribution to the gradient and the outputs take the inverse factors.
+// fp16 subnormals are kept by the matrix cores, so small entries beside large ones lose only bits
+// below 2^-38 of the largest.
+//
+// W is staged twice per chunk, split on the way: feature-major with k contiguous (A operand of the
+// first product, rows = features) and k-major with the chunk's 32 features contiguous (A operand of the
+// second, rows = k), the features in the order in which the first product's accumulator registers hold
+// them (register r of half h: feature 8(r/4) + 4h + r%4), so the split P goes straight from registers
+// into the B operand.
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void split_f16(float v, _Float16& hi, _Float16& lo) {
+    // v as it was rounded to fp32: when v is a product, the compiler may otherwise contract the
+    // multiply into one of the two conversions (v_fma_mix) and not the other, and the two parts then
+    // refer to different roundings of v near a tie (an error of one fp16 unit in the last place)
+    asm("" : "+v"(v));
+    hi = (_Float16)v;
+    lo = (_Float16)(v - (float)hi);
+}
+
+// 2^k with k clamped to what a float holds
+__device__ __forceinline__ float pow2i(int k) { return __int_as_float((min(max(k, -126), 127) + 127) << 23); }
+
+// k such that m 2^k lies in [2^13, 2^14) (m > 0 finite), 0 for m = 0
+__device__ __forceinline__ int scale_exponent(float m) {
+    if (!(m > 0.0f)) return 0;
+    const int e = (int)((__float_as_uint(m) >> 23) & 0xff) - 127;      // floor(log2 m) for normal m
+    return 13 - max(e, -126);
+}
+
+template <int D, bool WITH_GRAD>
+__global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void rff_energy_sorted_f16_kernel(
+    const float* __restrict__ x, const int* __restrict__ type_offsets, const int* __restrict__ sorted_slots,
+    const float* __restrict__ W, const float* __restrict__ b, const float* __restrict__ alpha, int ne, int F,
+    float norm, float* __restrict__ e_slots, float* __restrict__ gx) {
+    constexpr int LD1 = D + 8;                // halves per row of the feature-major copy
+    constexpr int LD2 = RE_FC + 8;            // halves per row of the k-major copy
+    constexpr int KS = D / 16;                // matrix instructions along k per product term
+    constexpr int NP = D / 64;                // pairs of adjacent k rows staged per thread per chunk
+    __shared__ __attribute__((aligned(16))) _Float16 sW1h[RE_FC * LD1], sW1l[RE_FC * LD1];
+    __shared__ __attribute__((aligned(16))) _Float16 sW2h[D * LD2], sW2l[D * LD2];
+    __shared__ __attribute__((aligned(16))) float sb[RE_FC], sa[RE_FC];
+    __shared__ float swmax[2][RE_T / 64];     // largest |W| of a chunk per wavefront, two chunks in flight
+
+    int type = -1, row0 = 0, rows = 0;
+    {
+        int bidx = blockIdx.x;
+        for (int t = 0; t < ne; ++t) {
+            const int o0 = type_offsets[t], o1 = type_offsets[t + 1];
+            const int nt = (o1 - o0 + RE_M - 1) / RE_M;
+            if (bidx < nt) {
+                type = t;
+                row0 = o0 + bidx * RE_M;
+                rows = min(RE_M, o1 - row0);
+                break;
+            }
+            bidx -= nt;
+        }
+    }
+    if (type < 0) return;
+    const float* Wt = W + (size_t)type * D * F;
+    const float* bt = b + (size_t)type * F;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i = lane & 31, h = lane >> 5;
+    const int arow = 32 * wave + i;
+    const bool aok = arow < rows;
+    const int fsplit = F / (int)gridDim.y;
+    const int fbeg = (int)blockIdx.y * fsplit, fend = fbeg + fsplit;
+
+    // x^T as the B operand of the first product: instruction j contracts k = 16 j + 8 h + (0..7)
+    half8_t xh[KS], xl[KS];
+    float inv_sx;
+    {
+        float xv[KS][8];
+        const float* xr = x + (size_t)(row0 + (aok ? arow : 0)) * D + 8 * h;
+        float m = 0.0f;
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+            const float4 v0 = aok ? *reinterpret_cast<const float4*>(xr + 16 * j) : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float4 v1 = aok ? *reinterpret_cast<const float4*>(xr + 16 * j + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+            xv[j][0] = v0.x; xv[j][1] = v0.y; xv[j][2] = v0.z; xv[j][3] = v0.w;
+            xv[j][4] = v1.x; xv[j][5] = v1.y; xv[j][6] = v1.z; xv[j][7] = v1.w;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) m = fmaxf(m, fabsf(xv[j][q]));
+        }
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        const int kx = scale_exponent(m);
+        const float sx = pow2i(kx);
+        inv_sx = pow2i(-kx);
+#pragma unroll
+        for (int j = 0; j < KS; ++j)
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                _Float16 a, c;
+                split_f16(xv[j][q] * sx, a, c);
+                xh[j][q] = a;
+                xl[j][q] = c;
+            }
+    }
+    // the workgroup's alpha scale (every wavefront finds the same value)
+    float sp, inv_sp;
+    {
+        float m = 0.0f;
+        for (int f = fbeg + lane; f < fend; f += 64) m = fmaxf(m, fabsf(alpha[f]));
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        const int kp = scale_exponent(m * norm);
+        sp = pow2i(kp);
+        inv_sp = pow2i(-kp);
+    }
+
+    float16_t gacc[D / 32];
+    if constexpr (WITH_GRAD) {
+#pragma unroll
+        for (int blk = 0; blk < D / 32; ++blk)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) gacc[blk][r] = 0.0f;
+    }
+    float energy = 0.0f;
+
+    // staging of a chunk: thread -> features sf .. sf+3 of the rows k0 = 2 (tid / 8) + 64 p and k0 + 1
+    const int sf = (tid & 7) * 4, skp = 2 * (tid >> 3);
+    // place of features sf .. sf+3 in a row of the k-major copy: f = 16 t + 8 c + 4 h' + e -> 16 t + 8 h' + 4 c + e
+    const int pos2 = (sf & 16) | ((sf & 4) << 1) | ((sf & 8) >> 1);
+    float4 stage[NP][2];
+    auto fetch = [&](int f0) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            stage[p][0] = *reinterpret_cast<const float4*>(Wt + (size_t)(skp + 64 * p) * F + f0 + sf);
+            stage[p][1] = *reinterpret_cast<const float4*>(Wt + (size_t)(skp + 64 * p + 1) * F + f0 + sf);
+        }
+    };
+    fetch(fbeg);
+    int par = 0;
+    for (int f0 = fbeg; f0 < fend; f0 += RE_FC, par ^= 1) {
+        // the chunk's own power of two for W (largest |W| of its D x 32 entries to 2^13): the part of a
+        // small W below fp16's smallest normal number would otherwise lose its low bits.  Every
+        // wavefront leaves the largest entry of what it staged, all read the four values after the
+        // barrier; the copy of the chunk before is no longer read by then.
+        {
+            float m = 0.0f;
+#pragma unroll
+            for (int p = 0; p < NP; ++p)
+#pragma unroll
+                for (int r = 0; r < 2; ++r)
+                    m = fmaxf(fmaxf(fmaxf(m, fabsf(stage[p][r].x)), fmaxf(fabsf(stage[p][r].y), fabsf(stage[p][r].z))),
+                              fabsf(stage[p][r].w));
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+            if (lane == 0) swmax[par][wave] = m;
+        }
+        __syncthreads();
+        const int kw = scale_exponent(fmaxf(fmaxf(swmax[par][0], swmax[par][1]), fmaxf(swmax[par][2], swmax[par][3])));
+        const float sw = pow2i(kw), inv_sw = pow2i(-kw);
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int k0 = skp + 64 * p;
+            const float w0[4] = {stage[p][0].x * sw, stage[p][0].y * sw, stage[p][0].z * sw, stage[p][0].w * sw};
+            const float w1[4] = {stage[p][1].x * sw, stage[p][1].y * sw, stage[p][1].z * sw, stage[p][1].w * sw};
+            half4_t r0h, r0l, r1h, r1l;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                _Float16 a, c;
+                split_f16(w0[e], a, c);
+                r0h[e] = a; r0l[e] = c;
+                split_f16(w1[e], a, c);
+                r1h[e] = a; r1l[e] = c;
+                *reinterpret_cast<half2_t*>(&sW1h[(sf + e) * LD1 + k0]) = (half2_t){r0h[e], r1h[e]};
+                *reinterpret_cast<half2_t*>(&sW1l[(sf + e) * LD1 + k0]) = (half2_t){r0l[e], r1l[e]};
+            }
+            *reinterpret_cast<half4_t*>(&sW2h[k0 * LD2 + pos2]) = r0h;
+            *reinterpret_cast<half4_t*>(&sW2l[k0 * LD2 + pos2]) = r0l;
+            *reinterpret_cast<half4_t*>(&sW2h[(k0 + 1) * LD2 + pos2]) = r1h;
+            *reinterpret_cast<half4_t*>(&sW2l[(k0 + 1) * LD2 + pos2]) = r1l;
+        }
+        if (tid < RE_FC) {
+            sb[tid] = bt[f0 + tid];
+            sa[tid] = alpha[f0 + tid] * norm * sp;
+        }
+        __syncthreads();
+        if (f0 + RE_FC < fend) fetch(f0 + RE_FC);
+
+        // first product: 2^(kx + kw) S^T (32 features x 32 atoms)
+        const float inv_sxw = inv_sx * inv_sw;
+        float16_t sacc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[r] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+            const half8_t ah = *reinterpret_cast<const half8_t*>(&sW1h[i * LD1 + 16 * j + 8 * h]);
+            const half8_t al = *reinterpret_cast<const half8_t*>(&sW1l[i * LD1 + 16 * j + 8 * h]);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, xh[j], sacc, 0, 0, 0);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, xl[j], sacc, 0, 0, 0);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, xh[j], sacc, 0, 0, 0);
+        }
+        // accumulator register r: feature 8(r/4) + 4h + r%4 of the chunk, atom = lane%32
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int fl = 8 * q + 4 * h;
+            const float4 bv = *reinterpret_cast<const float4*>(&sb[fl]);
+            const float4 av = *reinterpret_cast<const float4*>(&sa[fl]);
+            const float bq[4] = {bv.x, bv.y, bv.z, bv.w}, aq[4] = {av.x, av.y, av.z, av.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float sn, cs;
+                const float arg = fmaf(sacc[4 * q + e], inv_sxw, bq[e]);
+                sincos_hw(arg, &sn, &cs);
+                if (__builtin_expect(fabsf(arg) > 32000.0f, 0)) sincos_large(arg, &sn, &cs);
+                energy = fmaf(aq[e], cs, energy);
+                sacc[4 * q + e] = -aq[e] * sn;           // 2^kp P
+            }
+        }
+        if constexpr (WITH_GRAD) {
+            // second product: 2^kp GX^T[k, a] += 2^-kw sum_f 2^kw W[k, f] 2^kp P[f, a]; instruction t contracts the
+            // features of registers 8 t .. 8 t + 7.  The chunk's contribution is summed from zero and
+            // added to the running sums by the vector unit: the matrix instruction aligns its products
+            // to the accumulator it is given, and against a sum over a thousand chunks their low bits
+            // would be cut off
+            half8_t ph[2], pl[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    _Float16 a, c;
+                    split_f16(sacc[8 * t + q], a, c);
+                    ph[t][q] = a;
+                    pl[t][q] = c;
+                }
+#pragma unroll
+            for (int blk = 0; blk < D / 32; ++blk) {
+                float16_t part;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) part[r] = 0.0f;
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const half8_t ah = *reinterpret_cast<const half8_t*>(&sW2h[(32 * blk + i) * LD2 + 16 * t + 8 * h]);
+                    const half8_t al = *reinterpret_cast<const half8_t*>(&sW2l[(32 * blk + i) * LD2 + 16 * t + 8 * h]);
+                    part = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, ph[t], part, 0, 0, 0);
+                    part = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, pl[t], part, 0, 0, 0);
+                    part = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, ph[t], part, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) gacc[blk][r] = fmaf(part[r], inv_sw, gacc[blk][r]);
+            }
+        }
+    }
+
+    energy = (energy + __shfl_xor(energy, 32, 64)) * inv_sp;
+    if (gridDim.y == 1) {
+        if (h == 0 && aok) e_slots[sorted_slots[row0 + arow]] = energy;
+        if constexpr (WITH_GRAD) {
+            if (aok) {
+                float* gr = gx + (size_t)(row0 + arow) * D;
+#pragma unroll
+                for (int blk = 0; blk < D / 32; ++blk)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        *reinterpret_cast<float4*>(gr + 32 * blk + 8 * q + 4 * h) =
+                            make_float4(gacc[blk][4 * q] * inv_sp, gacc[blk][4 * q + 1] * inv_sp,
+                                        gacc[blk][4 * q + 2] * inv_sp, gacc[blk][4 * q + 3] * inv_sp);
+            }
+        }
+    } else {
+        // the feature parts add into zero-filled outputs
+        if (h == 0 && aok) atomicAdd(&e_slots[sorted_slots[row0 + arow]], energy);
+        if constexpr (WITH_GRAD) {
+            if (aok) {
+                float* gr = gx + (size_t)(row0 + arow) * D;
+#pragma unroll
+                for (int blk = 0; blk < D / 32; ++blk)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        atomicAdd(gr + 32 * blk + 8 * (r / 4) + 4 * h + (r % 4), gacc[blk][r] * inv_sp);
+            }
+        }
+    }
+}
+
 __global__ void zero_fill_kernel(float* __restrict__ p, size_t n) {
     for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (size_t)gridDim.x * blockDim.x) p[t] = 0.0f;
 }
@@ -483,12 +772,20 @@ extern "C" int qmll_rff_energy_sorted(const float* x, const int* type_offsets, c
         hipLaunchKernelGGL(zero_fill_kernel, dim3(1024), dim3(256), 0, st, gx, (size_t)A * d);
         QMLL_CHECK_LAUNCH("qmll_rff_energy_sorted");
     }
+    static const bool fp32_products = getenv("QMLL_RFF_FP32") != nullptr;
 #define CALL(DD)                                                                                                     \
-    if (gx)                                                                                                          \
-        hipLaunchKernelGGL((rff_energy_sorted_kernel<DD, true>), grid, dim3(RE_T), 0, st, x, type_offsets, sorted_slots, \
-                           W, b, alpha, ne, F, norm, e_slots, gx);                                                    \
+    if (fp32_products) {                                                                                             \
+        if (gx)                                                                                                      \
+            hipLaunchKernelGGL((rff_energy_sorted_kernel<DD, true>), grid, dim3(RE_T), 0, st, x, type_offsets,         \
+                               sorted_slots, W, b, alpha, ne, F, norm, e_slots, gx);                                  \
+        else                                                                                                         \
+            hipLaunchKernelGGL((rff_energy_sorted_kernel<DD, false>), grid, dim3(RE_T), 0, st, x, type_offsets,        \
+                               sorted_slots, W, b, alpha, ne, F, norm, e_slots, gx);                                  \
+    } else if (gx)                                                                                                   \
+        hipLaunchKernelGGL((rff_energy_sorted_f16_kernel<DD, true>), grid, dim3(RE_T), 0, st, x, type_offsets,         \
+                           sorted_slots, W, b, alpha, ne, F, norm, e_slots, gx);                                      \
     else                                                                                                             \
-        hipLaunchKernelGGL((rff_energy_sorted_kernel<DD, false>), grid, dim3(RE_T), 0, st, x, type_offsets,            \
+        hipLaunchKernelGGL((rff_energy_sorted_f16_kernel<DD, false>), grid, dim3(RE_T), 0, st, x, type_offsets,        \
                            sorted_slots, W, b, alpha, ne, F, norm, e_slots, gx)
     if (d == 64) {
         CALL(64);
