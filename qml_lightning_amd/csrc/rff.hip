@@ -205,8 +205,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D <= 128 ? 
 // forward (qml_lightning/models/random_features.py:88-100) and its autograd transpose
 // without ever writing the [atoms, F] feature matrix.
 //
-// Two chained fp32 matrix-core products per 32-feature chunk of W (staged in LDS, feature
-// major): S^T[f,a] = W^T x^T  ->  P[f,a] = -norm alpha_f sin(S + b_f)  ->  GX^T[k,a] += W P.
+// Two chained matrix-core products per 32-feature chunk of W (staged in LDS):
+// S^T[f,a] = W^T x^T  ->  P[f,a] = -norm alpha_f sin(S + b_f)  ->  GX^T[k,a] += W P.
 // Everything is kept transposed so that the accumulator registers of the first product (row
 // = feature, column = atom) are exactly the B operand the second one needs (contraction
 // index = feature): P never leaves the registers.  x^T (B operand of the first product)
@@ -215,177 +215,10 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 
 constexpr int RE_T = 256;        // threads: 4 wavefronts x 32 atoms
 constexpr int RE_M = 128;        // atoms per workgroup
-constexpr int RE_FC = 32;        // features per staged chunk (one MFMA block of 32)
+constexpr int RE_FC = 32;        // features per staged chunk (one block of 32 rows)
 
-template <int D, bool WITH_GRAD>
-__global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void rff_energy_sorted_kernel(const float* __restrict__ x,
-                                                                 const int* __restrict__ type_offsets,
-                                                                 const int* __restrict__ sorted_slots,
-                                                                 const float* __restrict__ W,
-                                                                 const float* __restrict__ b,
-                                                                 const float* __restrict__ alpha, int ne, int F,
-                                                                 float norm, float* __restrict__ e_slots,
-                                                                 float* __restrict__ gx) {
-    constexpr int LD = D + 4;                 // LDS row stride of the feature-major W chunk
-    constexpr int HK = D / 2;                 // contraction values per wavefront half
-    constexpr int NV = RE_FC * D / 4 / RE_T;  // float4 staged per thread per chunk
-    __shared__ __attribute__((aligned(16))) float sW[RE_FC * LD];
-    __shared__ __attribute__((aligned(16))) float sb[RE_FC], sa[RE_FC];
-
-    // tile of sorted atoms owned by this workgroup (never straddles two elements)
-    int type = -1, row0 = 0, rows = 0;
-    {
-        int bidx = blockIdx.x;
-        for (int t = 0; t < ne; ++t) {
-            const int o0 = type_offsets[t], o1 = type_offsets[t + 1];
-            const int nt = (o1 - o0 + RE_M - 1) / RE_M;
-            if (bidx < nt) {
-                type = t;
-                row0 = o0 + bidx * RE_M;
-                rows = min(RE_M, o1 - row0);
-                break;
-            }
-            bidx -= nt;
-        }
-    }
-    if (type < 0) return;
-    const float* Wt = W + (size_t)type * D * F;
-    const float* bt = b + (size_t)type * F;
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int i = lane & 31, h = lane >> 5;
-    const int arow = 32 * wave + i;           // this lane's atom within the tile
-    const bool aok = arow < rows;
-
-    // x^T as the B operand of the first product: MFMA step s contracts k = s (lanes 0-31)
-    // and k = D/2 + s (lanes 32-63)
-    float xb[HK];
-    {
-        const float* xr = x + (size_t)(row0 + (aok ? arow : 0)) * D + HK * h;
-#pragma unroll
-        for (int q = 0; q < HK / 4; ++q) {
-            const float4 v = aok ? *reinterpret_cast<const float4*>(xr + 4 * q) : make_float4(0.f, 0.f, 0.f, 0.f);
-            xb[4 * q] = v.x; xb[4 * q + 1] = v.y; xb[4 * q + 2] = v.z; xb[4 * q + 3] = v.w;
-        }
-    }
-    float16_t gacc[D / 32];
-    if constexpr (WITH_GRAD) {
-#pragma unroll
-        for (int blk = 0; blk < D / 32; ++blk)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) gacc[blk][r] = 0.0f;
-    }
-    float energy = 0.0f;
-
-    // staging of a chunk: rows k of W, RE_FC consecutive features each: thread -> k =
-    // tid/TPR + (256/TPR) v, features 4*(tid%TPR) .. +3; stored feature-major (transposed) in LDS
-    constexpr int TPR = RE_FC / 4, KSTEP = RE_T / TPR;
-    const int sk = tid / TPR, sf = (tid % TPR) * 4;
-    float4 stage[NV];
-    auto fetch = [&](int f0) {
-#pragma unroll
-        for (int v = 0; v < NV; ++v)
-            stage[v] = *reinterpret_cast<const float4*>(Wt + (size_t)(sk + KSTEP * v) * F + f0 + sf);
-    };
-    // feature range of this workgroup: gridDim.y splits of F (each a multiple of RE_FC)
-    const int fsplit = F / (int)gridDim.y;
-    const int fbeg = (int)blockIdx.y * fsplit, fend = fbeg + fsplit;
-    fetch(fbeg);
-    for (int f0 = fbeg; f0 < fend; f0 += RE_FC) {
-        __syncthreads();
-#pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const int k = sk + KSTEP * v;
-            sW[(sf + 0) * LD + k] = stage[v].x;
-            sW[(sf + 1) * LD + k] = stage[v].y;
-            sW[(sf + 2) * LD + k] = stage[v].z;
-            sW[(sf + 3) * LD + k] = stage[v].w;
-        }
-        if (tid < RE_FC) {
-            sb[tid] = bt[f0 + tid];
-            sa[tid] = alpha[f0 + tid] * norm;
-        }
-        __syncthreads();
-        if (f0 + RE_FC < fend) fetch(f0 + RE_FC);
-
-        // one block of 32 features at a time
-#pragma unroll
-        for (int fb = 0; fb < RE_FC / 32; ++fb) {
-            // first product: S^T block (32 features x 32 atoms)
-            float16_t sacc;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) sacc[r] = 0.0f;
-#pragma unroll
-            for (int q = 0; q < HK / 4; ++q) {
-                const float4 wa = *reinterpret_cast<const float4*>(&sW[(32 * fb + i) * LD + HK * h + 4 * q]);
-                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(wa.x, xb[4 * q], sacc, 0, 0, 0);
-                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(wa.y, xb[4 * q + 1], sacc, 0, 0, 0);
-                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(wa.z, xb[4 * q + 2], sacc, 0, 0, 0);
-                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(wa.w, xb[4 * q + 3], sacc, 0, 0, 0);
-            }
-            // accumulator register r: feature 8(r/4) + 4h + r%4 of the block, atom = lane%32
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int fl = 32 * fb + 8 * q + 4 * h;
-                const float4 bv = *reinterpret_cast<const float4*>(&sb[fl]);
-                const float4 av = *reinterpret_cast<const float4*>(&sa[fl]);
-                const float bq[4] = {bv.x, bv.y, bv.z, bv.w}, aq[4] = {av.x, av.y, av.z, av.w};
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float sn, cs;
-                    const float arg = sacc[4 * q + e] + bq[e];
-                    sincos_hw(arg, &sn, &cs);
-                    if (__builtin_expect(fabsf(arg) > 32000.0f, 0)) sincos_large(arg, &sn, &cs);
-                    energy = fmaf(aq[e], cs, energy);
-                    sacc[4 * q + e] = -aq[e] * sn;
-                }
-            }
-            if constexpr (WITH_GRAD) {
-                // second product: GX^T[k, a] += sum_f W[k, f] P[f, a]; step r contracts the two
-                // features the wavefront halves hold in register r
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int fl = 32 * fb + 8 * (r / 4) + 4 * h + (r % 4);
-#pragma unroll
-                    for (int blk = 0; blk < D / 32; ++blk)
-                        gacc[blk] = __builtin_amdgcn_mfma_f32_32x32x2f32(sW[fl * LD + 32 * blk + i], sacc[r], gacc[blk],
-                                                                         0, 0, 0);
-                }
-            }
-        }
-    }
-
-    energy += __shfl_xor(energy, 32, 64);
-    if (gridDim.y == 1) {
-        if (h == 0 && aok) e_slots[sorted_slots[row0 + arow]] = energy;
-        if constexpr (WITH_GRAD) {
-            if (aok) {
-                float* gr = gx + (size_t)(row0 + arow) * D;
-#pragma unroll
-                for (int blk = 0; blk < D / 32; ++blk)
-#pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        *reinterpret_cast<float4*>(gr + 32 * blk + 8 * q + 4 * h) =
-                            make_float4(gacc[blk][4 * q], gacc[blk][4 * q + 1], gacc[blk][4 * q + 2], gacc[blk][4 * q + 3]);
-            }
-        }
-    } else {
-        // the feature parts add into zero-filled outputs
-        if (h == 0 && aok) atomicAdd(&e_slots[sorted_slots[row0 + arow]], energy);
-        if constexpr (WITH_GRAD) {
-            if (aok) {
-                float* gr = gx + (size_t)(row0 + arow) * D;
-#pragma unroll
-                for (int blk = 0; blk < D / 32; ++blk)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) atomicAdd(gr + 32 * blk + 8 * (r / 4) + 4 * h + (r % 4), gacc[blk][r]);
-            }
-        }
-    }
-}
-
-// The same chain on the half-precision matrix cores.  v_mfma_f32_32x32x16_f16 runs 13 times as fast per
-// flop as the fp32 instruction above, so each fp32 operand is split into two fp16 parts (hi = the value
+// The products run on the half-precision matrix cores.  v_mfma_f32_32x32x16_f16 runs 13 times as fast per
+// flop as v_mfma_f32_32x32x2_f32 (40 against 64 clocks for eight times the flops), so each fp32 operand is split into two fp16 parts (hi = the value
 // rounded to fp16, lo = the rounded rest: 22 bits together) and a product becomes three matrix
 // instructions, hi.hi + hi.lo + lo.hi, accumulated in fp32; lo.lo is below the rounding of the sum.
 // fp16 has five exponent bits, so every operand is scaled by a power of two first (exact): x by the
@@ -755,8 +588,7 @@ extern "C" int qmll_rff_energy_sorted(const float* x, const int* type_offsets, c
                  "qmll_rff_energy_sorted: x, W and gx must be 16-byte aligned");
     const float norm = sqrtf(2.0f / (float)F);
     hipStream_t st = (hipStream_t)stream;
-    // Two workgroups fit a CU (two wavefronts per SIMD), and a workgroup's time is set by the
-    // matrix pipe, so the launch takes ceil(workgroups / 512) rounds of 1/fs of a tile's work
+    // Two workgroups fit a CU (two wavefronts per SIMD) and all run the same chunk loop, so the launch takes ceil(workgroups / 512) rounds of 1/fs of a tile's work
     // when the features are split over fs workgroups per tile.  fs is the power of two up to
     // 64 with the shortest estimate (a larger one has to win by 5 %): 672 tiles take 2 rounds
     // with fs = 1 and 21/16 with fs = 16; one molecule takes 1/64 instead of 1.  For fs > 1
@@ -772,16 +604,8 @@ extern "C" int qmll_rff_energy_sorted(const float* x, const int* type_offsets, c
         hipLaunchKernelGGL(zero_fill_kernel, dim3(1024), dim3(256), 0, st, gx, (size_t)A * d);
         QMLL_CHECK_LAUNCH("qmll_rff_energy_sorted");
     }
-    static const bool fp32_products = getenv("QMLL_RFF_FP32") != nullptr;
 #define CALL(DD)                                                                                                     \
-    if (fp32_products) {                                                                                             \
-        if (gx)                                                                                                      \
-            hipLaunchKernelGGL((rff_energy_sorted_kernel<DD, true>), grid, dim3(RE_T), 0, st, x, type_offsets,         \
-                               sorted_slots, W, b, alpha, ne, F, norm, e_slots, gx);                                  \
-        else                                                                                                         \
-            hipLaunchKernelGGL((rff_energy_sorted_kernel<DD, false>), grid, dim3(RE_T), 0, st, x, type_offsets,        \
-                               sorted_slots, W, b, alpha, ne, F, norm, e_slots, gx);                                  \
-    } else if (gx)                                                                                                   \
+    if (gx)                                                                                                          \
         hipLaunchKernelGGL((rff_energy_sorted_f16_kernel<DD, true>), grid, dim3(RE_T), 0, st, x, type_offsets,         \
                            sorted_slots, W, b, alpha, ne, F, norm, e_slots, gx);                                      \
     else                                                                                                             \

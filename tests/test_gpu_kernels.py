@@ -850,6 +850,35 @@ def test_rff_energy_sorted_kernel(d, F, ne, A):
     close(e2, e_ref, REL_EF, "fused rff energies only")
 
 
+@pytest.mark.parametrize("wscale,ascale,xscale", [(0.125, 1.0, 1.0), (1e-3, 1e4, 1.0), (1e-4, 1e20, 1.0), (0.125, 1e-6, 1.0),
+                                                  (125.0, 1e-20, 1e-3), (2e-6, 1.0, 6e4), (0.125, 1.0, 0.0)])
+def test_rff_energy_sorted_kernel_over_operand_scales(wscale, ascale, xscale):
+    """The fused kernel multiplies on the fp16 matrix cores with every fp32 operand split in two fp16
+    parts behind a power-of-two scale of its own (x per wavefront, alpha per workgroup, W per chunk of 32
+    features): W, alpha and x far outside fp16's range, one feature with a tie between two fp16 values,
+    and an all-zero x, against fp64 at fp32 accuracy (5e-6 of the largest entry; arguments up to ~15; an
+    operand part lost to fp16's range or a split that mixes two roundings costs 1e-5 to 1e-3)."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(7)
+    d, F, A, ne = 128, 1056, 150, 1
+    types = np.zeros(A, dtype=np.int32)
+    ss, off = ops.sort_by_type(ti32(types), ti32(np.arange(A, dtype=np.int32)), ne)
+    x = (rng.normal(size=(A, d)) * xscale).astype(np.float32)
+    W = (rng.normal(size=(ne, d, F)) * wscale).astype(np.float32)
+    W[0, :, 40:72] *= 1e-3                                    # a chunk of small entries beside the others
+    b = rng.uniform(0, 2 * np.pi, (ne, F)).astype(np.float32)
+    alpha = (rng.normal(size=F) * ascale).astype(np.float32)
+    alpha[5] = 0.0
+    e, gx = ops.rff_energy_sorted(t32(x), off, ss, t32(W), t32(b), t32(alpha), A)
+    arg = x.astype(np.float64) @ W[0].astype(np.float64) + b[0]
+    nf = np.sqrt(2.0 / F)
+    e_ref = nf * np.cos(arg) @ alpha.astype(np.float64)
+    g_ref = -nf * (np.sin(arg) * alpha.astype(np.float64)) @ W[0].astype(np.float64).T
+    assert np.abs(arg).max() < 40
+    close(e, e_ref, 5e-6, "fused rff energies")
+    close(gx, g_ref, 5e-6, "fused rff gradient")
+
+
 @pytest.mark.parametrize("d,F,n", [(64, 200, 6), (128, 704, 21), (128, 130, 29), (256, 64, 9), (16, 40, 6)])
 def test_rff_derivatives_molecule_major(d, F, n):
     """Matrix-core route (segments instead of a molecule index); accumulates onto G;
