@@ -333,6 +333,163 @@ __global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(PNT > 64 ? 3
     }
 }
 
+// The forward product on the half-precision matrix cores, 128 x 128 tiles (A [rows, K] gathered through
+// a_rows, B_type [K, N] row-major, K and N multiples of 4, 16-byte aligned bases).  Per chunk of 32 k the
+// tile of A and the tile of B are split into two fp16 parts each on their way into LDS (both k-contiguous:
+// B is transposed as it is staged), three v_mfma_f32_32x32x16_f16 per product term.  The chunk of A and
+// the chunk of B each take their own power of two (every wavefront leaves the largest entries of what it
+// is about to stage, all read the four pairs after the barrier the loop has anyway), so a chunk's product
+// is summed from zero and added to the running sums by the vector unit with the inverse factor (which
+// also keeps the low bits of a small chunk beside a large sum).
+__global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(2, 3))) void typed_gemm_f16_kernel(
+    const float* __restrict__ A, int lda, const int* __restrict__ a_rows, const float* __restrict__ Bm,
+    size_t b_type_stride, int ldb, float* __restrict__ C, int ldc, const int* __restrict__ offsets, int ne, int K, int N,
+    int group) {
+    constexpr int LDH = PK + 8;        // halves per staged row
+    __shared__ __attribute__((aligned(16))) _Float16 sAh[PM * LDH], sAl[PM * LDH], sBh[128 * LDH], sBl[128 * LDH];
+    __shared__ float smax[2][PT / 64][2];     // largest |A|, |B| of a chunk per wavefront, two chunks in flight
+    int type, row0, rows;
+    if (!tile_of_block(offsets, ne, blockIdx.x, type, row0, rows, group)) return;
+    const int col0 = blockIdx.y * 128;
+    const float* Bt = Bm + (size_t)type * b_type_stride;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i = lane & 31, h = lane >> 5;
+
+    // staging of A: rows tid/8 + 32 v, k = (tid%8)*4 .. +3 of the chunk
+    const int ar = tid >> 3, ak = (tid & 7) * 4;
+    const float* arow[4];
+    bool arow_ok[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const int r = ar + 32 * v;
+        arow_ok[v] = r < rows;
+        size_t src = 0;
+        if (arow_ok[v]) {
+            if (group > 1) {
+                const int e = (row0 + r) / group;
+                src = (size_t)a_rows[e] * group + (size_t)(row0 + r - e * group);
+            } else {
+                src = (size_t)(a_rows ? a_rows[row0 + r] : row0 + r);
+            }
+        }
+        arow[v] = A + src * lda;
+    }
+    // staging of B: columns (tid/8)*4 .. +3, rows k = 2 (tid%8) + 16 u and the next one
+    const int bn = (tid >> 3) * 4, bkp = 2 * (tid & 7);
+    float4 ra[4], rb[2][2];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+            ra[v] = (arow_ok[v] && k0 + ak < K) ? *reinterpret_cast<const float4*>(arow[v] + k0 + ak) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int k = k0 + bkp + 16 * u + e;
+                rb[u][e] = (k < K && col0 + bn < N) ? *reinterpret_cast<const float4*>(Bt + (size_t)k * ldb + col0 + bn)
+                                                   : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+    };
+    auto max4 = [](float m, float4 v) { return fmaxf(fmaxf(fmaxf(m, fabsf(v.x)), fmaxf(fabsf(v.y), fabsf(v.z))), fabsf(v.w)); };
+
+    float16_t acc[4];
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[jt][r] = 0.0f;
+
+    const int nchunks = (K + PK - 1) / PK;
+    fetch(0);
+    for (int c = 0; c < nchunks; ++c) {
+        const int par = c & 1;
+        {
+            float ma = 0.0f, mb = 0.0f;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) ma = max4(ma, ra[v]);
+#pragma unroll
+            for (int u = 0; u < 2; ++u) mb = max4(max4(mb, rb[u][0]), rb[u][1]);
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) {
+                ma = fmaxf(ma, __shfl_xor(ma, o, 64));
+                mb = fmaxf(mb, __shfl_xor(mb, o, 64));
+            }
+            if (lane == 0) {
+                smax[par][wave][0] = ma;
+                smax[par][wave][1] = mb;
+            }
+        }
+        __syncthreads();     // the chunk before has been read, and the largest entries of this one are known
+        const int ka = scale_exponent(fmaxf(fmaxf(smax[par][0][0], smax[par][1][0]), fmaxf(smax[par][2][0], smax[par][3][0])));
+        const int kb = scale_exponent(fmaxf(fmaxf(smax[par][0][1], smax[par][1][1]), fmaxf(smax[par][2][1], smax[par][3][1])));
+        const float sa = pow2i(ka), sb = pow2i(kb), inv = pow2i(-ka) * pow2i(-kb);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const float w[4] = {ra[v].x * sa, ra[v].y * sa, ra[v].z * sa, ra[v].w * sa};
+            half4_t wh, wl;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                _Float16 a, cc;
+                split_f16(w[e], a, cc);
+                wh[e] = a;
+                wl[e] = cc;
+            }
+            *reinterpret_cast<half4_t*>(&sAh[(ar + 32 * v) * LDH + ak]) = wh;
+            *reinterpret_cast<half4_t*>(&sAl[(ar + 32 * v) * LDH + ak]) = wl;
+        }
+        {
+            const float bv[2][2][4] = {{{rb[0][0].x, rb[0][0].y, rb[0][0].z, rb[0][0].w}, {rb[0][1].x, rb[0][1].y, rb[0][1].z, rb[0][1].w}},
+                                       {{rb[1][0].x, rb[1][0].y, rb[1][0].z, rb[1][0].w}, {rb[1][1].x, rb[1][1].y, rb[1][1].z, rb[1][1].w}}};
+#pragma unroll
+            for (int cc = 0; cc < 4; ++cc)
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    _Float16 h0, l0, h1, l1;
+                    split_f16(bv[u][0][cc] * sb, h0, l0);
+                    split_f16(bv[u][1][cc] * sb, h1, l1);
+                    *reinterpret_cast<half2_t*>(&sBh[(bn + cc) * LDH + bkp + 16 * u]) = (half2_t){h0, h1};
+                    *reinterpret_cast<half2_t*>(&sBl[(bn + cc) * LDH + bkp + 16 * u]) = (half2_t){l0, l1};
+                }
+        }
+        __syncthreads();
+        if (c + 1 < nchunks) fetch((c + 1) * PK);
+#pragma unroll
+        for (int j0 = 0; j0 < 4; j0 += 2) {
+            float16_t part[2];
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) part[jj][r] = 0.0f;
+#pragma unroll
+            for (int s2 = 0; s2 < PK / 16; ++s2) {
+                const half8_t ahv = *reinterpret_cast<const half8_t*>(&sAh[(32 * wave + i) * LDH + 16 * s2 + 8 * h]);
+                const half8_t alv = *reinterpret_cast<const half8_t*>(&sAl[(32 * wave + i) * LDH + 16 * s2 + 8 * h]);
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj) {
+                    const half8_t bhv = *reinterpret_cast<const half8_t*>(&sBh[(32 * (j0 + jj) + i) * LDH + 16 * s2 + 8 * h]);
+                    const half8_t blv = *reinterpret_cast<const half8_t*>(&sBl[(32 * (j0 + jj) + i) * LDH + 16 * s2 + 8 * h]);
+                    part[jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(alv, bhv, part[jj], 0, 0, 0);
+                    part[jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ahv, blv, part[jj], 0, 0, 0);
+                    part[jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ahv, bhv, part[jj], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[j0 + jj][r] = fmaf(part[jj][r], inv, acc[j0 + jj][r]);
+        }
+    }
+
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt) {
+        const int col = col0 + 32 * jt + i;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = 32 * wave + 8 * (r / 4) + 4 * h + (r % 4);
+            if (row < rows && col < N) C[(size_t)(row0 + row) * ldc + col] = acc[jt][r];
+        }
+    }
+}
+
 // Transpose product for a short contraction (K = projected dimension 64 or 128):
 //     C[c_rows[row], :] = A[row, :] . B_type^T,   A [rows, K] (the gradient rows), B_type [N, K] row-major.
 // A wavefront keeps its 32 rows of A in registers for the whole kernel (lane (i, h) holds
@@ -416,6 +573,133 @@ __global__ __launch_bounds__(PT) void typed_gemm_bt_rows_kernel(const float* __r
 #pragma unroll
             for (int q = 0; q < 16; ++q)
                 if (dst[q] >= 0) C[(size_t)dst[q] * ldc + col] = acc[q];
+        }
+        // the other copy was last read in the previous round, which every wavefront left through the barrier below
+        if (b + 1 < nblk) stash(cur ^ 1);
+        __syncthreads();
+    }
+}
+
+// The same transpose product on the half-precision matrix cores (v_mfma_f32_32x32x16_f16: eight times
+// the flops of the fp32 instruction in 40 clocks against 64): both operands as two fp16 parts each, three
+// matrix instructions per product term.  The rows of A take the wavefront's power of two, every row of B
+// (a column of the product) its own, found by the eight lanes that stage it; the product leaves the
+// accumulators through the two inverse factors.
+template <int K>
+__global__ __launch_bounds__(PT) void typed_gemm_bt_rows_f16_kernel(const float* __restrict__ A, const float* __restrict__ Bm,
+                                                                     size_t b_type_stride, float* __restrict__ C, int ldc,
+                                                                     const int* __restrict__ c_rows,
+                                                                     const int* __restrict__ offsets, int ne, int N) {
+    constexpr int KS = K / 16;         // matrix instructions along k per product term
+    constexpr int LDB = K + 8;         // halves per staged row of B
+    constexpr int NV = K / 32;         // float4 per thread and staged block
+    __shared__ __attribute__((aligned(16))) _Float16 sBh[2][32 * LDB], sBl[2][32 * LDB];
+    __shared__ float sinv[2][32];      // inverse scale of each staged row
+    int type, row0, rows;
+    if (!tile_of_block(offsets, ne, blockIdx.x, type, row0, rows)) return;
+    const float* Bt = Bm + (size_t)type * b_type_stride;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i = lane & 31, h = lane >> 5;
+
+    const int r = 32 * wave + i;
+    const bool rok = r < rows;
+    // instruction j contracts k = 16 j + 8 h + (0..7)
+    half8_t ah[KS], al[KS];
+    float inv_sa;
+    {
+        float av[KS][8];
+        const float* ap = A + (size_t)(row0 + (rok ? r : 0)) * K + 8 * h;
+        float m = 0.0f;
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+            const float4 v0 = rok ? *reinterpret_cast<const float4*>(ap + 16 * j) : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float4 v1 = rok ? *reinterpret_cast<const float4*>(ap + 16 * j + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+            av[j][0] = v0.x; av[j][1] = v0.y; av[j][2] = v0.z; av[j][3] = v0.w;
+            av[j][4] = v1.x; av[j][5] = v1.y; av[j][6] = v1.z; av[j][7] = v1.w;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) m = fmaxf(m, fabsf(av[j][q]));
+        }
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        const int ka = scale_exponent(m);
+        const float sa = pow2i(ka);
+        inv_sa = pow2i(-ka);
+#pragma unroll
+        for (int j = 0; j < KS; ++j)
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                _Float16 a, c;
+                split_f16(av[j][q] * sa, a, c);
+                ah[j][q] = a;
+                al[j][q] = c;
+            }
+    }
+    // staging of a block of B: thread -> row tid/8 of the block, floats (tid%8)*4 + 32 v
+    const int bn = tid >> 3, bk = (tid & 7) * 4;
+    float4 rb[NV];
+    auto fetch = [&](int b) {
+        const int n = 32 * b + bn;
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+            rb[v] = n < N ? *reinterpret_cast<const float4*>(Bt + (size_t)n * K + bk + 32 * v) : make_float4(0.f, 0.f, 0.f, 0.f);
+    };
+    auto stash = [&](int buf) {
+        float m = 0.0f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) m = fmaxf(fmaxf(fmaxf(m, fabsf(rb[v].x)), fmaxf(fabsf(rb[v].y), fabsf(rb[v].z))), fabsf(rb[v].w));
+        m = fmaxf(m, lane_xor<1>(m));            // the eight lanes of a row are neighbours
+        m = fmaxf(m, lane_xor<2>(m));
+        m = fmaxf(m, lane_xor<4>(m));
+        const int kb = scale_exponent(m);
+        const float sb = pow2i(kb);
+        if ((tid & 7) == 0) sinv[buf][bn] = pow2i(-kb);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const float w[4] = {rb[v].x * sb, rb[v].y * sb, rb[v].z * sb, rb[v].w * sb};
+            half4_t wh, wl;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                _Float16 a, c;
+                split_f16(w[e], a, c);
+                wh[e] = a;
+                wl[e] = c;
+            }
+            *reinterpret_cast<half4_t*>(&sBh[buf][bn * LDB + bk + 32 * v]) = wh;
+            *reinterpret_cast<half4_t*>(&sBl[buf][bn * LDB + bk + 32 * v]) = wl;
+        }
+    };
+    int dst[16];                        // destination rows of the 16 accumulator registers
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+        const int row = 32 * wave + 8 * (q / 4) + 4 * h + (q % 4);
+        dst[q] = row < rows ? (c_rows ? c_rows[row0 + row] : row0 + row) : -1;
+    }
+    const int nblk = (N + 31) / 32;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int b = 0; b < nblk; ++b) {
+        const int cur = b & 1;
+        if (b + 1 < nblk) fetch(b + 1);
+        float16_t acc;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc[q] = 0.0f;
+        const _Float16* bph = &sBh[cur][i * LDB + 8 * h];
+        const _Float16* bpl = &sBl[cur][i * LDB + 8 * h];
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+            const half8_t bh = *reinterpret_cast<const half8_t*>(bph + 16 * j);
+            const half8_t bl = *reinterpret_cast<const half8_t*>(bpl + 16 * j);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[j], bh, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[j], bl, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[j], bh, acc, 0, 0, 0);
+        }
+        const float f = inv_sa * sinv[cur][i];
+        const int col = 32 * b + i;
+        if (col < N) {
+#pragma unroll
+            for (int q = 0; q < 16; ++q)
+                if (dst[q] >= 0) C[(size_t)dst[q] * ldc + col] = acc[q] * f;
         }
         // the other copy was last read in the previous round, which every wavefront left through the barrier below
         if (b + 1 < nblk) stash(cur ^ 1);
@@ -681,8 +965,8 @@ extern "C" int qmll_project_typed(const float* rep, const int* sorted_slots, con
     const bool wide = vec && d % 128 == 0 && (long long)tiles * (d / 128) >= 2 * 256;
     const dim3 grid(tiles, wide ? d / 128 : (d + PN - 1) / PN);
     if (wide)
-        hipLaunchKernelGGL((typed_gemm_kernel<false, true, 128>), grid, dim3(PT), 0, (hipStream_t)stream, rep, R,
-                           sorted_slots, reductors, (size_t)R * d, d, x, d, (const int*)nullptr, type_offsets, ne, R, d);
+        hipLaunchKernelGGL(typed_gemm_f16_kernel, grid, dim3(PT), 0, (hipStream_t)stream, rep, R, sorted_slots, reductors,
+                           (size_t)R * d, d, x, d, type_offsets, ne, R, d, 1);
     else if (vec)
         hipLaunchKernelGGL((typed_gemm_kernel<false, true, PN>), grid, dim3(PT), 0, (hipStream_t)stream, rep, R, sorted_slots,
                            reductors, (size_t)R * d, d, x, d, (const int*)nullptr, type_offsets, ne, R, d);
@@ -708,6 +992,9 @@ extern "C" int qmll_project_typed_rows(const float* rows, const int* sorted_slot
     const int tiles = (int)((nrows + PM - 1) / PM) + ne;
     const bool wide = vec && d % 128 == 0 && (long long)tiles * (d / 128) >= 2 * 256;
     const dim3 grid(tiles, wide ? d / 128 : (d + PN - 1) / PN);
+    // the fp32 matrix instructions here: a row's result then does not depend on the rows that share its
+    // tile (the half-precision kernel scales a whole chunk of the tile by one power of two), so the rows
+    // of a training batch are the same however the training set is cut into batches
     if (wide)
         hipLaunchKernelGGL((typed_gemm_kernel<false, true, 128>), grid, dim3(PT), 0, (hipStream_t)stream, rows, R,
                            sorted_slots, reductors, (size_t)R * d, d, x, d, (const int*)nullptr, type_offsets, ne, R, d,
@@ -750,10 +1037,10 @@ extern "C" int qmll_project_typed_backward(const float* gx, const int* sorted_sl
         // short contraction: the gradient rows stay in registers, every row is read once
         const dim3 g1((A + PM - 1) / PM + ne);
         if (d == 128)
-            hipLaunchKernelGGL((typed_gemm_bt_rows_kernel<128>), g1, dim3(PT), 0, (hipStream_t)stream, gx, reductors,
+            hipLaunchKernelGGL((typed_gemm_bt_rows_f16_kernel<128>), g1, dim3(PT), 0, (hipStream_t)stream, gx, reductors,
                                (size_t)R * d, g_rep, R, sorted_slots, type_offsets, ne, R);
         else
-            hipLaunchKernelGGL((typed_gemm_bt_rows_kernel<64>), g1, dim3(PT), 0, (hipStream_t)stream, gx, reductors,
+            hipLaunchKernelGGL((typed_gemm_bt_rows_f16_kernel<64>), g1, dim3(PT), 0, (hipStream_t)stream, gx, reductors,
                                (size_t)R * d, g_rep, R, sorted_slots, type_offsets, ne, R);
     } else if (vec)
         hipLaunchKernelGGL((typed_gemm_kernel<true, true, PN>), grid, dim3(PT), 0, (hipStream_t)stream, gx, d,

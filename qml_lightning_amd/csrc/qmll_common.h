@@ -137,4 +137,33 @@ __device__ __forceinline__ float sin_hw(float x) {
     return s;
 }
 
+// ---- fp32 operands for the half-precision matrix cores --------------------------------------
+// An fp32 value as two fp16 parts, hi = the value rounded to fp16 and lo = the rounded rest (22 bits
+// together): a product of two such values is hi.hi + hi.lo + lo.hi on v_mfma_f32_32x32x16_f16,
+// accumulated in fp32.  fp16 has five exponent bits, so the caller first scales by a power of two
+// (exact) that takes the largest entry of the operand to [2^13, 2^14); the matrix cores keep fp16
+// subnormals, so smaller entries lose only bits below 2^-38 of the largest.
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void split_f16(float v, _Float16& hi, _Float16& lo) {
+    // v as it was rounded to fp32: when v is a product, the compiler may otherwise contract the
+    // multiply into one of the two conversions (v_fma_mix) and not the other, and the two parts then
+    // refer to different roundings of v near a tie (an error of one fp16 unit in the last place)
+    asm("" : "+v"(v));
+    hi = (_Float16)v;
+    lo = (_Float16)(v - (float)hi);
+}
+
+// 2^k with k clamped to what a float holds
+__device__ __forceinline__ float pow2i(int k) { return __int_as_float((min(max(k, -126), 127) + 127) << 23); }
+
+// k such that m 2^k lies in [2^13, 2^14) (m > 0 finite), 0 for m = 0
+__device__ __forceinline__ int scale_exponent(float m) {
+    if (!(m > 0.0f)) return 0;
+    const int e = (int)((__float_as_uint(m) >> 23) & 0xff) - 127;      // floor(log2 m) for normal m
+    return 13 - max(e, -126);
+}
+
 #endif  // __HIPCC__

@@ -233,29 +233,6 @@ constexpr int RE_FC = 32;        // features per staged chunk (one block of 32 r
 // second, rows = k), the features in the order in which the first product's accumulator registers hold
 // them (register r of half h: feature 8(r/4) + 4h + r%4), so the split P goes straight from registers
 // into the B operand.
-typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ void split_f16(float v, _Float16& hi, _Float16& lo) {
-    // v as it was rounded to fp32: when v is a product, the compiler may otherwise contract the
-    // multiply into one of the two conversions (v_fma_mix) and not the other, and the two parts then
-    // refer to different roundings of v near a tie (an error of one fp16 unit in the last place)
-    asm("" : "+v"(v));
-    hi = (_Float16)v;
-    lo = (_Float16)(v - (float)hi);
-}
-
-// 2^k with k clamped to what a float holds
-__device__ __forceinline__ float pow2i(int k) { return __int_as_float((min(max(k, -126), 127) + 127) << 23); }
-
-// k such that m 2^k lies in [2^13, 2^14) (m > 0 finite), 0 for m = 0
-__device__ __forceinline__ int scale_exponent(float m) {
-    if (!(m > 0.0f)) return 0;
-    const int e = (int)((__float_as_uint(m) >> 23) & 0xff) - 127;      // floor(log2 m) for normal m
-    return 13 - max(e, -126);
-}
-
 template <int D, bool WITH_GRAD>
 __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void rff_energy_sorted_f16_kernel(
     const float* __restrict__ x, const int* __restrict__ type_offsets, const int* __restrict__ sorted_slots,
