@@ -536,6 +536,40 @@ def test_project_typed_rows_projects_a_group_of_rows_per_atom(R, d, ne, N, A, gr
           "one row per atom")
 
 
+@pytest.mark.parametrize("rscale,uscale", [(1.0, 1.0), (1e-6, 1e3), (3e4, 1e-4), (1e10, 1e-12), (0.0, 1.0)])
+def test_projection_on_the_fp16_matrix_cores_over_operand_scales(rscale, uscale):
+    """The projection of a large batch and the transposed projection multiply on the fp16 matrix cores with
+    every fp32 operand split in two fp16 parts behind powers of two (per chunk of the tile, per wavefront,
+    per row of the matrix): operands far outside fp16's range, rows that are small beside their tile's
+    largest, a zero operand; against fp64 at fp32 accuracy (2e-6 of the largest entry)."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(11)
+    R, d, ne, N = 312, 128, 2, 66000          # 516 tiles of 128 rows: the large-batch kernel
+    rep = torch.randn(N, R, device=dev(), generator=torch.Generator(device=dev()).manual_seed(3)) * rscale
+    rep[::7] *= 1e-3                           # rows that are small beside the others of their tile
+    rep[5::11, 100:] = 0.0
+    red = (rng.normal(size=(ne, R, d)) * uscale).astype(np.float32)
+    red[1, :, 64:] *= 1e-2
+    types = torch.tensor(rng.integers(0, ne, N).astype(np.int32), device=dev())
+    ss, off = ops.sort_by_type(types, torch.arange(N, dtype=torch.int32, device=dev()), ne)
+    x = ops.project_typed(rep, ss, off, t32(red))
+    pick = torch.tensor(rng.choice(N, size=3000, replace=False), device=dev())
+    ssl = ss.long()[pick]
+    U = torch.tensor(red, device=dev()).double()[types.long()[ssl]]
+    x_ref = torch.einsum('ar,ard->ad', rep[ssl].double(), U)
+    scale = float(x_ref.abs().max())
+    assert float((x[pick].double() - x_ref).abs().max()) <= 2e-6 * max(scale, 1e-300)
+    # rows small beside their tile's largest keep their own accuracy down to 2^-17 of it
+    small = (ssl % 7 == 0)
+    if rscale > 0 and bool(small.any()):
+        ref_s = x_ref[small]
+        assert float((x[pick][small].double() - ref_s).abs().max()) <= 1e-5 * float(ref_s.abs().max())
+    gx = torch.randn(N, d, device=dev(), generator=torch.Generator(device=dev()).manual_seed(4)) * rscale
+    g = ops.project_typed_backward(gx, ss, off, t32(red), types, N)
+    g_ref = torch.einsum('ad,ard->ar', gx[pick].double(), U)
+    assert float((g[ssl].double() - g_ref).abs().max()) <= 2e-6 * max(float(g_ref.abs().max()), 1e-300)
+
+
 @pytest.mark.parametrize("T,S,d", [(1, 6, 64), (2, 6, 64), (1, 64, 128), (1, 70, 64), (2, 64, 64)])
 def test_sorted_fused_energy_matches_per_atom_oracle(T, S, d):
     """Element-sorted rows through the fused kernel: energies land in the atoms' slots, the
