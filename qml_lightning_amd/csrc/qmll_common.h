@@ -159,11 +159,12 @@ __device__ __forceinline__ void split_f16(float v, _Float16& hi, _Float16& lo) {
 // 2^k with k clamped to what a float holds
 __device__ __forceinline__ float pow2i(int k) { return __int_as_float((min(max(k, -126), 127) + 127) << 23); }
 
-// k such that m 2^k lies in [2^13, 2^14) (m > 0 finite), 0 for m = 0
+// k such that m 2^k lies in [2^13, 2^14) (m > 0 finite), 0 for m = 0; at most 126, so that 2^k and
+// 2^-k are both floats (operands below 2^-113 then sit lower in fp16's range)
 __device__ __forceinline__ int scale_exponent(float m) {
     if (!(m > 0.0f)) return 0;
     const int e = (int)((__float_as_uint(m) >> 23) & 0xff) - 127;      // floor(log2 m) for normal m
-    return 13 - max(e, -126);
+    return min(13 - max(e, -126), 126);
 }
 
 #endif  // __HIPCC__
