@@ -16,7 +16,7 @@ import torch
 from .. import ops
 from ..cuda.sorf_gpu import compute_hadamard_features, compute_partial_feature_derivatives
 from ..representations.dimensionality_reduction import project_representation
-from .kernel import BaseKernel, _default_device, alpha_f32
+from .kernel import BaseKernel, _default_device, alpha_f32, rep_from_attribute_tree
 
 _fused_registered = False
 
@@ -524,6 +524,30 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         if forces:
             return (predict_energies, predict_forces)
         return predict_energies
+
+    @classmethod
+    def from_reference_file(cls, file_name, fused=True, separate_ops=False):
+        """A HadamardFeaturesModel holding the weights of a model file written by
+        `save_jit_model` (hadamard_features.py:253-255 of the reference): by the reference
+        itself or by this class.  The archive is read as data (attribute tree walked opcode by
+        opcode, storages through numpy): nothing in it is unpickled or executed, no operator
+        library and no GPU are needed to open it.  The result predicts through the fused route
+        (or, with `fused=False`, the reference's operator sequence) and can be trained further
+        or saved again."""
+        from ..utils import model_files
+        tree = model_files.read_attribute_tree(file_name)
+        if not str(tree.get("__class__", "")).endswith("HadamardFeaturesModel"):
+            raise ValueError("%s holds a %r, not a HadamardFeaturesModel" % (file_name, tree.get("__class__")))
+        rep = rep_from_attribute_tree(tree["rep"])
+        model = cls(rep=rep, elements=np.asarray(tree["elements"], dtype=np.int64),
+                    ntransforms=int(tree["ntransforms"]), sigma=float(tree["sigma"]), llambda=float(tree["llambda"]),
+                    npcas=int(tree["npcas"]), nbatch_train=int(tree["nbatch_train"]),
+                    nbatch_test=int(tree["nbatch_test"]), nstacks=int(tree["nstacks"]), fused=fused,
+                    separate_ops=separate_ops)
+        model._fill_from_attribute_tree(tree, {"Dmat": torch.float32, "bias": torch.float32})
+        if not bool(((model.Dmat == 1) | (model.Dmat == -1)).all()):
+            raise ValueError("%s: the SORF diagonals are not all +-1" % file_name)
+        return model
 
     @torch.jit.unused
     def save_jit_model(self, file_name='model_sorf.pt'):

@@ -38,6 +38,33 @@ def alpha_f32(model):
     return hit[2]
 
 
+def rep_from_attribute_tree(tree):
+    """An FCHLCuda with exactly the tensors a saved model's `rep` sub-module holds (attribute
+    names and dtypes of qml_lightning/representations/FCHL.py:21-46): the radial grids, the
+    weight with sqrt(eta3/pi) already folded in and the fp32 scalars are taken as stored, not
+    recomputed from rounded hyper-parameters."""
+    from ..representations.FCHL import FCHLCuda
+    if not str(tree.get("__class__", "")).endswith("FCHLCuda"):
+        raise ValueError("model file: the representation is %r, only FCHLCuda is supported" % tree.get("__class__"))
+    species = np.asarray(tree["species"])
+    rep = FCHLCuda(species=species.astype(np.int64), rcut=float(tree["rcut"]), nRs2=int(tree["nRs2"]),
+                   nRs3=int(tree["nRs3"]), eta2=float(tree["eta2"]), eta3=float(tree["eta3"]),
+                   two_body_decay=float(tree["two_body_decay"]), three_body_weight=1.0,
+                   three_body_decay=float(tree["three_body_decay"]))
+    dev = rep.device
+    rep.species = torch.from_numpy(species.astype(np.float32)).to(dev)
+    for name in ("rcut", "eta2", "eta3", "two_body_decay", "three_body_weight", "three_body_decay"):
+        setattr(rep, name, torch.from_numpy(np.asarray(tree[name], dtype=np.float32).reshape(())).clone())
+    rep.nRs2 = torch.tensor(int(tree["nRs2"]))
+    rep.nRs3 = torch.tensor(int(tree["nRs3"]))
+    rep.Rs2 = torch.from_numpy(np.asarray(tree["Rs2"], dtype=np.float32)).to(dev)
+    rep.Rs3 = torch.from_numpy(np.asarray(tree["Rs3"], dtype=np.float32)).to(dev)
+    if int(tree["fp_size"]) != rep.fp_size:
+        raise ValueError("model file: fp_size %d does not follow from its species and grids (%d)"
+                         % (int(tree["fp_size"]), rep.fp_size))
+    return rep
+
+
 class BaseKernel():
 
     def __init__(self, rep, npcas, elements, sigma, llambda):
@@ -470,6 +497,35 @@ class BaseKernel():
         V = V * torch.where(lead < 0, -1.0, 1.0)
         k = min(rows.shape)                      # an SVD of [repsize, nsamples] has min(...) vectors
         return V[:, :k].to(mat.dtype), torch.sqrt(w[:k].clamp_min(0.0)).to(mat.dtype)
+
+    # -- model files ------------------------------------------------------------------------
+    def _fill_from_attribute_tree(self, tree, tensors):
+        """Copy what a saved model carries beside its feature tensors (kernel.py:24-41 of the
+        reference: reductors, element2index, self_energy, unit flags, alpha) and the feature
+        tensors named in `tensors` ({attribute: dtype}), checking every shape against the one
+        this model was constructed with."""
+        dev = self.device
+        for name, dtype in dict(tensors, reductors=torch.float32).items():
+            have = getattr(self, name)
+            new = torch.from_numpy(np.ascontiguousarray(tree[name])).to(dtype)
+            if tuple(new.shape) != tuple(have.shape):
+                raise ValueError("model file: %s has shape %s, the hyper-parameters give %s"
+                                 % (name, tuple(new.shape), tuple(have.shape)))
+            setattr(self, name, new.to(dev))
+        e2i = torch.from_numpy(np.asarray(tree["element2index"], dtype=np.int64))
+        if not torch.equal(e2i, self.element2index):
+            raise ValueError("model file: element2index does not follow from its element list")
+        alpha = torch.from_numpy(np.ascontiguousarray(tree["alpha"]))          # fp64 once trained
+        if alpha.shape != (self.nfeatures(),):
+            raise ValueError("model file: alpha has %d entries for %d features" % (alpha.numel(), self.nfeatures()))
+        self.alpha = alpha.to(dev)
+        self.is_trained = bool(tree.get("is_trained", True))
+        se = tree.get("self_energy")
+        self.self_energy = None if se is None else torch.from_numpy(np.asarray(se, dtype=np.float64))
+        self._convert_from_hartree_to_kcal = bool(tree.get("_convert_from_hartree_to_kcal", False))
+        self._subtract_self_energies = bool(tree.get("_subtract_self_energies", False))
+        self.hartree2kcalmol = float(tree.get("hartree2kcalmol", 627.5))
+        return self
 
     # -- unit conversion / self energies ----------------------------------------------------
     def set_subtract_self_energies(self, subtract):

@@ -9,7 +9,7 @@ from .. import ops
 from ..cuda.rff_gpu import get_rff
 from ..representations.dimensionality_reduction import project_representation
 from . import hadamard_features  # noqa: F401  (registers the fused operators)
-from .kernel import BaseKernel, _default_device, alpha_f32
+from .kernel import BaseKernel, _default_device, alpha_f32, rep_from_attribute_tree
 
 
 class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
@@ -187,6 +187,32 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
         if forces:
             return (predict_energies, predict_forces)
         return predict_energies
+
+    @classmethod
+    def from_reference_file(cls, file_name, fused=True, separate_ops=False):
+        """A RandomFourrierFeaturesModel holding the weights of a model file written by
+        `save_jit_model` (random_features.py:233-235 of the reference), read as data: see
+        HadamardFeaturesModel.from_reference_file.  `nstacks` is recovered from the number of
+        features the file's W has."""
+        from ..utils import model_files
+        tree = model_files.read_attribute_tree(file_name)
+        if not str(tree.get("__class__", "")).endswith("RandomFourrierFeaturesModel"):
+            raise ValueError("%s holds a %r, not a RandomFourrierFeaturesModel" % (file_name, tree.get("__class__")))
+        rep = rep_from_attribute_tree(tree["rep"])
+        npcas = int(tree["npcas"])
+        nfeatures = int(np.asarray(tree["W"]).shape[2])
+        if nfeatures % npcas != 0:
+            raise ValueError("%s: %d features are not a multiple of npcas = %d" % (file_name, nfeatures, npcas))
+        state = np.random.get_state()        # the constructor draws a W that is replaced at once
+        try:
+            model = cls(rep=rep, elements=np.asarray(tree["elements"], dtype=np.int64), sigma=float(tree["sigma"]),
+                        llambda=float(tree["llambda"]), nstacks=nfeatures // npcas, npcas=npcas,
+                        nbatch_train=int(tree["nbatch_train"]), nbatch_test=int(tree["nbatch_test"]), fused=fused,
+                        separate_ops=separate_ops)
+        finally:
+            np.random.set_state(state)
+        model._fill_from_attribute_tree(tree, {"W": torch.float32, "b": torch.float32})
+        return model
 
     @torch.jit.unused
     def save_jit_model(self, file_name='model_rff.pt'):

@@ -1,43 +1,30 @@
 """Write tests/golden/aspirin_sorf_kat.npz from the reference's own known-answer test.
 
 Data only: the tensors are the raw little-endian storages inside the reference's
-saved model (``unit_tests/models/saved_models/model_sorf.pt``, an uncompressed zip;
-storage number -> attribute name / dtype / shape is listed by ``pickletools.dis`` of
-its ``data.pkl``), read with ``numpy.frombuffer``; nothing from the file is unpickled,
-imported or executed.  Coordinates, charges and the expected energy / forces are the
+saved model (``unit_tests/models/saved_models/model_sorf.pt``, an uncompressed zip), found
+through the package's weights-only reader (``qml_lightning_amd/utils/model_files.py``: the
+attribute tree of ``data.pkl`` walked opcode by opcode, storages read with
+``numpy.frombuffer``); nothing from the file is unpickled, imported or executed.  Coordinates, charges and the expected energy / forces are the
 literals of ``unit_tests/models/unit_test_sorf.py:11-31,57,59-80``.
 
 Run once in the build container (the reference tree does not exist on the GPU box):
     python tests/golden/make_aspirin_fixture.py
 """
 import os
-import zipfile
+import sys
 
 import numpy as np
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))))
+from qml_lightning_amd.utils import model_files  # noqa: E402
 
 REF = "/root/reference/unit_tests/models/saved_models/model_sorf.pt"
 OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "aspirin_sorf_kat.npz")
 
-# storage key -> (name, dtype, shape)   (from pickletools.dis of model_sorf/data.pkl)
-STORAGES = {
-    0: ("self_energy", "<f8", (9,)),
-    1: ("elements", "<i8", (3,)),
-    2: ("reductors", "<f4", (3, 336, 128)),
-    3: ("element2index", "<i8", (9,)),
-    4: ("ntransforms", "<i8", ()),
-    5: ("species", "<f4", (3,)),
-    6: ("Dmat", "<f4", (3, 1, 128, 128)),
-    7: ("bias", "<f4", (3, 16384)),
-    8: ("alpha", "<f8", (16384,)),
-    10: ("rcut", "<f4", ()),
-    13: ("eta2", "<f4", ()),
-    14: ("eta3", "<f4", ()),
-    15: ("two_body_decay", "<f4", ()),
-    16: ("three_body_weight", "<f4", ()),
-    17: ("three_body_decay", "<f4", ()),
-    18: ("Rs2", "<f4", (24,)),
-    19: ("Rs3", "<f4", (22,)),
-}
+# attributes of the model and of its `rep` sub-module that the known-answer test needs
+MODEL_TENSORS = ("self_energy", "elements", "reductors", "element2index", "ntransforms", "Dmat", "bias", "alpha")
+REP_TENSORS = ("species", "rcut", "eta2", "eta3", "two_body_decay", "three_body_weight", "three_body_decay", "Rs2",
+               "Rs3")
 
 # unit_tests/models/unit_test_sorf.py:11-31
 coordinates = np.array([[2.25571364, -0.38562082, 0.25521779],
@@ -89,18 +76,15 @@ ref_forces = np.array([[7.1108e+00, -2.3761e+01, 4.6022e+00],
 
 
 def main():
-    z = zipfile.ZipFile(REF)
-    out = {}
-    for key, (name, dtype, shape) in STORAGES.items():
-        raw = z.read("model_sorf/data/%d" % key)
-        arr = np.frombuffer(raw, dtype=dtype).reshape(shape).copy()
-        out[name] = arr
+    tree = model_files.read_attribute_tree(REF)
+    out = {name: tree[name] for name in MODEL_TENSORS}
+    out.update({name: tree["rep"][name] for name in REP_TENSORS})
     # +-1 diagonals travel as int8
     assert set(np.unique(out["Dmat"])) <= {-1.0, 1.0}
     out["Dmat"] = out["Dmat"].astype(np.int8)
-    out["sigma"] = np.float64(2.0)        # data.pkl attribute 'sigma'
-    out["npcas"] = np.int64(128)          # data.pkl attribute 'npcas'
-    out["nstacks"] = np.int64(128)        # data.pkl attribute 'nstacks'
+    out["sigma"] = np.float64(tree["sigma"])
+    out["npcas"] = np.int64(tree["npcas"])
+    out["nstacks"] = np.int64(tree["nstacks"])
     out["coordinates"] = coordinates
     out["charges"] = charges
     out["ref_energy"] = np.float64(ref_energy)

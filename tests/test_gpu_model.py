@@ -200,6 +200,50 @@ def test_torchscript_roundtrip(tmp_path):
         assert ("get_SORF_coefficients" in code) == (not fused)
 
 
+def test_known_answer_through_a_model_file_read_as_data(kat, tmp_path):
+    """The aspirin model written in the reference's file layout (the reference's operator
+    sequence, its attribute names and dtypes: checked on the host in test_model_files.py), read
+    back by `from_reference_file` without unpickling, then run through the fused route, the
+    reference route and `torch.jit.load` of the same file: the three agree and reproduce the
+    reference's printed energy and forces (unit_test_sorf.py:59-80,93-101)."""
+    from qml_lightning_amd.models.hadamard_features import HadamardFeaturesModel
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    from qml_lightning_amd.utils import model_files
+    d = kat
+    rep = FCHLCuda(species=np.array([1, 6, 8]), rcut=6.0, nRs2=24, nRs3=22, eta2=0.28, eta3=3.2,
+                   two_body_decay=2.3, three_body_weight=18.8, three_body_decay=0.65)
+    rep.three_body_weight = torch.tensor(float(d["three_body_weight"]))
+    src = HadamardFeaturesModel(rep=rep, elements=np.array([1, 6, 8]), ntransforms=1, sigma=2.0, llambda=1e-5,
+                                npcas=128, nstacks=128, nbatch_test=256, fused=False)
+    src.reductors, src.Dmat, src.bias = t32(d["reductors"]), t32(d["Dmat"].astype(np.float32)), t32(d["bias"])
+    src.alpha = torch.tensor(d["alpha"], device=dev())
+    src.self_energy = torch.tensor(d["self_energy"])
+    src.set_subtract_self_energies(True)
+    src.is_trained = True
+    path = os.path.join(tmp_path, "model_sorf.pt")
+    src.save_jit_model(path)
+    model_files.check_reference_loadable(path)
+    n = d["coordinates"].shape[0]
+    Z = t32(d["charges"]).unsqueeze(0)
+    ids = (torch.arange(n, dtype=torch.int32, device=dev()), torch.zeros(n, dtype=torch.int32, device=dev()), ti32([n]))
+    results = []
+    for fused in (True, False, None):
+        m = torch.jit.load(path) if fused is None else HadamardFeaturesModel.from_reference_file(path, fused=fused)
+        X = t32(d["coordinates"]).unsqueeze(0).requires_grad_(True)
+        E = m.forward(X, Z, *ids)
+        F, = torch.autograd.grad(-E.sum(), X)
+        se = d["self_energy"] if fused is None else m.self_energy.numpy()
+        total = se[d["charges"]].sum() + E.item()
+        assert np.isclose(float(d["ref_energy"]), total) and abs(total - float(d["ref_energy"])) < 0.1
+        got = F.squeeze(0).cpu().numpy()
+        assert np.isclose(d["ref_forces"], got, rtol=1e-4, atol=1e-3).all()
+        results.append((E.item(), got))
+    # the reference route from the file read as data IS the scripted file's arithmetic
+    assert results[1][0] == results[2][0] and np.array_equal(results[1][1], results[2][1])
+    assert abs(results[0][0] - results[1][0]) < 1e-4 * abs(results[1][0])
+    assert np.abs(results[0][1] - results[1][1]).max() < 1e-4 * np.abs(results[1][1]).max()
+
+
 def test_predict_from_lists_and_predict_cuda():
     species = [1, 6, 7, 8, 9]
     coords, charges = helpers.ragged_batch(11, 4)
