@@ -402,20 +402,17 @@ int qmll_probe_fill(float* dst, size_t nfloats, float value, qmll_stream_t strea
 int qmll_probe_copy(const float* src, float* dst, size_t nfloats, qmll_stream_t stream);
 
 /* A loop of `iters` rounds of independent instructions on every SIMD of the chip: which = 0
- * v_mfma_f64_16x16x4_f64, 1 v_mfma_f32_32x32x2_f32, 2 v_exp_f32; blocks_per_cu (1..16) workgroups
- * of four wavefronts per compute unit, i.e. that many wavefronts per SIMD.  out: device scratch of
- * qmll_probe_out_bytes() bytes.  Returns the number of operations the launch performs (flop, or
- * exponentials for which = 2), to be divided by the measured duration; negative on error. */
+ * v_mfma_f64_16x16x4_f64, 1 v_mfma_f32_32x32x2_f32, 2 v_exp_f32, 3 v_mfma_f32_32x32x16_f16;
+ * blocks_per_cu (1..16) workgroups of four wavefronts per compute unit, i.e. that many wavefronts
+ * per SIMD.  out: device scratch of qmll_probe_out_bytes() bytes.  Returns the number of operations
+ * the launch performs (flop, or exponentials for which = 2), to be divided by the measured
+ * duration; negative on error. */
 size_t qmll_probe_out_bytes(void);
 double qmll_probe_rate(int which, int iters, int blocks_per_cu, void* out, qmll_stream_t stream);
 
 /* Straight-line loops of the instruction classes the fused SORF kernel issues, on independent
- * registers: mix = 0 128 plain fp32, 1 128 DPP fmac, 2 128 v_sin_f32, 3 32 v_mfma_f32_16x16x4_f32,
- * 4 the per-stack mix of the fused kernel at 128 components (92 plain + 64 DPP + 16
- * transcendental), 5 the same with the in-row stages as 16 matrix instructions and 16 more plain
- * ones instead of the 64 DPP, 6 16 v_mfma_f32_16x16x32_f16, 7 the 128 plain fp32 of mix 0 with the 16
- * matrix instructions of mix 6 spread between them, 8 the split of 32 fp32 values into two fp16
- * parts each (64 instructions), 9 128 v_mul_f32 in the 64-bit encoding (a source modifier).
+ * registers: mix = 0 128 plain fp32, 1 128 DPP fmac, 2 128 v_sin_f32, 3 the per-stack mix of the
+ * fused kernel at 128 components (92 plain + 64 DPP + 16 transcendental).
  * Returns wavefront-iterations per SIMD (blocks_per_cu x iters), so
  * duration x clock / that = SIMD clocks per iteration; negative on error. */
 double qmll_probe_mix(int mix, int iters, int blocks_per_cu, void* out, qmll_stream_t stream);

@@ -1,5 +1,5 @@
 // Measured ceilings of the device the library runs on: plain fill and copy kernels (HBM), a loop
-// of independent matrix-core instructions in fp64 and fp32, and a loop of independent
+// of independent matrix-core instructions in fp64, fp32 and fp16, and a loop of independent
 // transcendental instructions.  The benchmark divides each kernel's rate by these next to the
 // nominal peaks; the copy kernel is also the known-size reference for scaling the FETCH_SIZE /
 // WRITE_SIZE counters of a profiler run.  No counterpart in the reference.
@@ -9,6 +9,7 @@ namespace {
 
 typedef double double4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 
 constexpr int PT = 256;
 
@@ -88,6 +89,30 @@ __global__ __launch_bounds__(PT) void probe_mfma_f32_kernel(int iters, float* __
     out[(size_t)blockIdx.x * PT + threadIdx.x] = s;
 }
 
+// the instruction of the split-operand products (projection, random Fourier features): two
+// independent 32 x 32 accumulator tiles per wavefront, fp16 operands, fp32 accumulation
+__global__ __launch_bounds__(PT) void probe_mfma_f16_kernel(int iters, float* __restrict__ out) {
+    half8_t a, b;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        a[k] = (_Float16)(1e-3f * (float)((threadIdx.x + k) & 7));
+        b[k] = (_Float16)(1e-3f * (float)((threadIdx.x + 2 * k) & 3));
+    }
+    float16_t c0, c1;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) c0[r] = c1[r] = 0.0f;
+    for (int it = 0; it < iters; ++it) {
+        c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c1, 0, 0, 0);
+        c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(b, a, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(b, a, c1, 0, 0, 0);
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += c0[r] + c1[r];
+    out[(size_t)blockIdx.x * PT + threadIdx.x] = s;
+}
+
 // eight independent chains of v_exp_f32 per lane (arguments stay in [-1, 0])
 __global__ __launch_bounds__(PT) void probe_exp_kernel(int iters, float* __restrict__ out) {
     float v[8];
@@ -105,26 +130,11 @@ __global__ __launch_bounds__(PT) void probe_exp_kernel(int iters, float* __restr
 
 // ---- instruction mixes -------------------------------------------------------------------
 // Straight-line loops of the instruction classes the fused SORF kernel issues, alone and mixed,
-// on independent registers: what a wavefront instruction of each class costs a SIMD, and how far
-// the matrix pipe runs beside the vector pipe.  One iteration of a mix stands for one stack of
-// one wavefront of that kernel at 128 components (8 registers per lane, four atoms per wavefront):
-//   MIX_FUSED      92 plain fp32 + 64 DPP fmac + 16 transcendental (the kernel as it is, counted in its ISA)
-//   MIX_MFMA_TRIAL 108 plain fp32 + 16 transcendental + 16 v_mfma_f32_16x16x4_f32: the in-row stages
-//                  (a 16-point +-1 Hadamard block per 16 lanes, forward and adjoint, 2 x 2 tiles x K = 16)
-//                  on the matrix pipe, 16 plain instructions for the operand layout, no data movement
-// and the pieces of a half-precision form of those stages (a 16-point +-1 block is exact in fp16, the
-// fp32 operand being split into two fp16 parts):
-//   MIX_MFMA_F16      16 v_mfma_f32_16x16x32_f16
-//   MIX_PLAIN_MFMA_F16 the 128 plain instructions of MIX_PLAIN with those 16 matrix instructions spread
-//                  between them (independent registers): the time of the two together against their sum
-//   MIX_SPLIT_F16  the split of 32 fp32 values: per pair v_cvt_pkrtz_f16_f32, two v_fma_mix_f32
-//                  (value - first part), v_cvt_pkrtz_f16_f32 = 64 instructions
-//   MIX_VOP3       128 v_mul_f32 with a source modifier, i.e. in the 64-bit encoding
-enum { MIX_PLAIN = 0, MIX_DPP = 1, MIX_TRANS = 2, MIX_MFMA16 = 3, MIX_FUSED = 4, MIX_MFMA_TRIAL = 5, MIX_MFMA_F16 = 6,
-       MIX_PLAIN_MFMA_F16 = 7, MIX_SPLIT_F16 = 8, MIX_VOP3 = 9, MIX_COUNT = 10 };
-
-typedef float float4_t __attribute__((ext_vector_type(4)));
-typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+// on independent registers: what a wavefront instruction of each class costs a SIMD.  One
+// iteration of MIX_FUSED stands for one stack of one wavefront of that kernel at 128 components
+// (8 registers per lane, four atoms per wavefront): 92 plain fp32 + 64 DPP fmac + 16
+// transcendental instructions, counted in its ISA.
+enum { MIX_PLAIN = 0, MIX_DPP = 1, MIX_TRANS = 2, MIX_FUSED = 3, MIX_COUNT = 4 };
 
 template <int N>
 __device__ __forceinline__ void plain_ops(float (&v)[8], float c) {
@@ -142,35 +152,6 @@ __device__ __forceinline__ void trans_ops(float (&v)[8]) {
 #pragma unroll
     for (int k = 0; k < N; ++k) v[k & 7] = __builtin_amdgcn_sinf(v[k & 7]);
 }
-template <int N>
-__device__ __forceinline__ void mfma_ops(float4_t (&acc)[4], float a, float b) {
-#pragma unroll
-    for (int k = 0; k < N; ++k) acc[k & 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[k & 3], 0, 0, 0);
-}
-
-template <int N>
-__device__ __forceinline__ void mfma_f16_ops(float4_t (&acc)[4], half8_t a, half8_t b) {
-#pragma unroll
-    for (int k = 0; k < N; ++k) acc[k & 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[k & 3], 0, 0, 0);
-}
-template <int N>
-__device__ __forceinline__ void vop3_ops(float (&v)[8], float c) {
-#pragma unroll
-    for (int k = 0; k < N; ++k) asm volatile("v_mul_f32_e64 %0, %0, -%1" : "+v"(v[k & 7]) : "v"(c));
-}
-// two fp16 parts of each of 8 fp32 values; the parts are folded into `sink` so that they stay live
-__device__ __forceinline__ void split_f16_ops(float (&v)[8], unsigned& sink) {
-#pragma unroll
-    for (int k = 0; k < 8; k += 2) {
-        unsigned h1, h2;
-        float r0, r1;
-        asm volatile("v_cvt_pkrtz_f16_f32 %0, %1, %2" : "=v"(h1) : "v"(v[k]), "v"(v[k + 1]));
-        asm volatile("v_fma_mix_f32 %0, -%1, 1.0, %2 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(r0) : "v"(h1), "v"(v[k]));
-        asm volatile("v_fma_mix_f32 %0, -%1, 1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r1) : "v"(h1), "v"(v[k + 1]));
-        asm volatile("v_cvt_pkrtz_f16_f32 %0, %1, %2" : "=v"(h2) : "v"(r0), "v"(r1));
-        sink ^= h2;
-    }
-}
 
 template <int MIX>
 __global__ __launch_bounds__(PT) void probe_mix_kernel(int iters, float* __restrict__ out) {
@@ -178,22 +159,10 @@ __global__ __launch_bounds__(PT) void probe_mix_kernel(int iters, float* __restr
 #pragma unroll
     for (int k = 0; k < 8; ++k) v[k] = 0.001f * (float)((threadIdx.x & 31) + k);
     const float c = (threadIdx.x & 1) ? -0.5f : 0.5f;
-    float4_t acc[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) acc[k] = (float4_t){0.f, 0.f, 0.f, 0.f};
-    const float a = 1e-3f * (float)(threadIdx.x & 7), b = (threadIdx.x & 2) ? 1.0f : -1.0f;
-    half8_t ah, bh;
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-        ah[k] = (_Float16)(((threadIdx.x + k) & 1) ? 1.0f : -1.0f);
-        bh[k] = (_Float16)(0.01f * (float)(threadIdx.x & 15));
-    }
-    unsigned sink = 0;
     for (int it = 0; it < iters; ++it) {
         if constexpr (MIX == MIX_PLAIN) plain_ops<128>(v, c);
         if constexpr (MIX == MIX_DPP) dpp_ops<128>(v, c);
         if constexpr (MIX == MIX_TRANS) trans_ops<128>(v);
-        if constexpr (MIX == MIX_MFMA16) mfma_ops<32>(acc, a, b);
         if constexpr (MIX == MIX_FUSED) {
             // forward: sign multiply + register stages, in-row stages, argument, sincos, products;
             // adjoint: register stages, in-row stages, accumulate
@@ -205,36 +174,10 @@ __global__ __launch_bounds__(PT) void probe_mix_kernel(int iters, float* __restr
             dpp_ops<32>(v, c);
             plain_ops<28>(v, c);
         }
-        if constexpr (MIX == MIX_MFMA_TRIAL) {
-            plain_ops<36>(v, c);
-            mfma_ops<8>(acc, a, b);
-            plain_ops<18>(v, c);
-            trans_ops<16>(v);
-            plain_ops<18>(v, c);
-            mfma_ops<8>(acc, a, b);
-            plain_ops<36>(v, c);
-        }
-        if constexpr (MIX == MIX_MFMA_F16) mfma_f16_ops<16>(acc, ah, bh);
-        if constexpr (MIX == MIX_PLAIN_MFMA_F16) {
-#pragma unroll
-            for (int g = 0; g < 16; ++g) {
-                mfma_f16_ops<1>(acc, ah, bh);
-                plain_ops<8>(v, c);
-            }
-        }
-        if constexpr (MIX == MIX_SPLIT_F16) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                split_f16_ops(v, sink);
-            }
-        }
-        if constexpr (MIX == MIX_VOP3) vop3_ops<128>(v, c);
     }
-    float s = (float)(sink & 1u);
+    float s = 0.0f;
 #pragma unroll
     for (int k = 0; k < 8; ++k) s += v[k];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) s += acc[k][0] + acc[k][1] + acc[k][2] + acc[k][3];
     out[(size_t)blockIdx.x * PT + threadIdx.x] = s;
 }
 
@@ -288,8 +231,11 @@ extern "C" double qmll_probe_rate(int which, int iters, int blocks_per_cu, void*
     } else if (which == 2) {
         hipLaunchKernelGGL(probe_exp_kernel, dim3(PROBE_BLOCKS), dim3(PT), 0, (hipStream_t)stream, iters, (float*)out);
         ops = waves * 64.0 * iters * 8.0;
+    } else if (which == 3) {
+        hipLaunchKernelGGL(probe_mfma_f16_kernel, dim3(PROBE_BLOCKS), dim3(PT), 0, (hipStream_t)stream, iters, (float*)out);
+        ops = waves * iters * 4.0 * (2.0 * 32 * 32 * 16);
     } else {
-        qmll_set_error("qmll_probe_rate: which = %d (0: fp64 matrix loop, 1: fp32 matrix loop, 2: exp loop)", which);
+        qmll_set_error("qmll_probe_rate: which = %d (0: fp64 matrix loop, 1: fp32 matrix loop, 2: exp loop, 3: fp16 matrix loop)", which);
         return -1.0;
     }
     if (hipGetLastError() != hipSuccess) {
@@ -314,13 +260,7 @@ extern "C" double qmll_probe_mix(int mix, int iters, int blocks_per_cu, void* ou
         case MIX_PLAIN: hipLaunchKernelGGL(probe_mix_kernel<MIX_PLAIN>, grid, block, 0, st, iters, o); break;
         case MIX_DPP: hipLaunchKernelGGL(probe_mix_kernel<MIX_DPP>, grid, block, 0, st, iters, o); break;
         case MIX_TRANS: hipLaunchKernelGGL(probe_mix_kernel<MIX_TRANS>, grid, block, 0, st, iters, o); break;
-        case MIX_MFMA16: hipLaunchKernelGGL(probe_mix_kernel<MIX_MFMA16>, grid, block, 0, st, iters, o); break;
-        case MIX_FUSED: hipLaunchKernelGGL(probe_mix_kernel<MIX_FUSED>, grid, block, 0, st, iters, o); break;
-        case MIX_MFMA_TRIAL: hipLaunchKernelGGL(probe_mix_kernel<MIX_MFMA_TRIAL>, grid, block, 0, st, iters, o); break;
-        case MIX_MFMA_F16: hipLaunchKernelGGL(probe_mix_kernel<MIX_MFMA_F16>, grid, block, 0, st, iters, o); break;
-        case MIX_PLAIN_MFMA_F16: hipLaunchKernelGGL(probe_mix_kernel<MIX_PLAIN_MFMA_F16>, grid, block, 0, st, iters, o); break;
-        case MIX_SPLIT_F16: hipLaunchKernelGGL(probe_mix_kernel<MIX_SPLIT_F16>, grid, block, 0, st, iters, o); break;
-        default: hipLaunchKernelGGL(probe_mix_kernel<MIX_VOP3>, grid, block, 0, st, iters, o); break;
+        default: hipLaunchKernelGGL(probe_mix_kernel<MIX_FUSED>, grid, block, 0, st, iters, o); break;
     }
     if (hipGetLastError() != hipSuccess) {
         qmll_set_error("qmll_probe_mix: launch failed");

@@ -491,100 +491,15 @@ __global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(2, 3))) void
 }
 
 // Transpose product for a short contraction (K = projected dimension 64 or 128):
-//     C[c_rows[row], :] = A[row, :] . B_type^T,   A [rows, K] (the gradient rows), B_type [N, K] row-major.
-// A wavefront keeps its 32 rows of A in registers for the whole kernel (lane (i, h) holds
-// A[i][K/2 h .. K/2 h + K/2), the contraction order of v_mfma_f32_32x32x2f32 being free), so every
-// row of A is read exactly once; the workgroup walks the N columns in blocks of 32, each block of
-// B staged through LDS (k contiguous, two copies) while the previous block is multiplied, and
-// every 32 x 32 block of C leaves straight from the accumulators.  The tiled kernel above re-reads
-// its A tile once per 64 columns (five times at N = 312).
-template <int K>
-__global__ __launch_bounds__(PT) void typed_gemm_bt_rows_kernel(const float* __restrict__ A, const float* __restrict__ Bm,
-                                                                 size_t b_type_stride, float* __restrict__ C, int ldc,
-                                                                 const int* __restrict__ c_rows,
-                                                                 const int* __restrict__ offsets, int ne, int N) {
-    constexpr int KH = K / 2;          // contraction values per lane
-    constexpr int LDB = K + 4;         // LDS stride of a staged B row: 16-byte reads of 8 consecutive rows cover all banks
-    constexpr int NV = K / 32;         // float4 per thread and staged block
-    __shared__ __attribute__((aligned(16))) float sB[2][32 * LDB];
-    int type, row0, rows;
-    if (!tile_of_block(offsets, ne, blockIdx.x, type, row0, rows)) return;
-    const float* Bt = Bm + (size_t)type * b_type_stride;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int i = lane & 31, h = lane >> 5;
-
-    const int r = 32 * wave + i;
-    const bool rok = r < rows;
-    float a[KH];
-    {
-        const float* ap = A + (size_t)(row0 + (rok ? r : 0)) * K + KH * h;
-#pragma unroll
-        for (int q = 0; q < KH / 4; ++q) {
-            const float4 v = rok ? *reinterpret_cast<const float4*>(ap + 4 * q) : make_float4(0.f, 0.f, 0.f, 0.f);
-            a[4 * q + 0] = v.x;
-            a[4 * q + 1] = v.y;
-            a[4 * q + 2] = v.z;
-            a[4 * q + 3] = v.w;
-        }
-    }
-    // staging of a block of B: thread -> row tid/8 of the block, floats (tid%8)*4 + 32 v
-    const int bn = tid >> 3, bk = (tid & 7) * 4;
-    float4 rb[NV];
-    auto fetch = [&](int b) {
-        const int n = 32 * b + bn;
-#pragma unroll
-        for (int v = 0; v < NV; ++v)
-            rb[v] = n < N ? *reinterpret_cast<const float4*>(Bt + (size_t)n * K + bk + 32 * v) : make_float4(0.f, 0.f, 0.f, 0.f);
-    };
-    auto stash = [&](int buf) {
-#pragma unroll
-        for (int v = 0; v < NV; ++v) *reinterpret_cast<float4*>(&sB[buf][bn * LDB + bk + 32 * v]) = rb[v];
-    };
-    int dst[16];                        // destination rows of the 16 accumulator registers
-#pragma unroll
-    for (int q = 0; q < 16; ++q) {
-        const int row = 32 * wave + 8 * (q / 4) + 4 * h + (q % 4);
-        dst[q] = row < rows ? (c_rows ? c_rows[row0 + row] : row0 + row) : -1;
-    }
-    const int nblk = (N + 31) / 32;
-    fetch(0);
-    stash(0);
-    __syncthreads();
-    for (int b = 0; b < nblk; ++b) {
-        const int cur = b & 1;
-        if (b + 1 < nblk) fetch(b + 1);
-        // two accumulator chains, so that an instruction never waits for the result of the one before it
-        float16_t acc, acc1;
-#pragma unroll
-        for (int q = 0; q < 16; ++q) acc[q] = acc1[q] = 0.0f;
-        const float* bp = &sB[cur][i * LDB + KH * h];
-#pragma unroll
-        for (int q = 0; q < KH / 4; ++q) {
-            const float4 v = *reinterpret_cast<const float4*>(bp + 4 * q);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * q + 0], v.x, acc, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * q + 1], v.y, acc1, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * q + 2], v.z, acc, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * q + 3], v.w, acc1, 0, 0, 0);
-        }
-#pragma unroll
-        for (int q = 0; q < 16; ++q) acc[q] += acc1[q];
-        const int col = 32 * b + i;
-        if (col < N) {
-#pragma unroll
-            for (int q = 0; q < 16; ++q)
-                if (dst[q] >= 0) C[(size_t)dst[q] * ldc + col] = acc[q];
-        }
-        // the other copy was last read in the previous round, which every wavefront left through the barrier below
-        if (b + 1 < nblk) stash(cur ^ 1);
-        __syncthreads();
-    }
-}
-
-// The same transpose product on the half-precision matrix cores (v_mfma_f32_32x32x16_f16: eight times
-// the flops of the fp32 instruction in 40 clocks against 64): both operands as two fp16 parts each, three
-// matrix instructions per product term.  The rows of A take the wavefront's power of two, every row of B
-// (a column of the product) its own, found by the eight lanes that stage it; the product leaves the
-// accumulators through the two inverse factors.
+//     C[c_rows[row], :] = A[row, :] . B_type^T,   A [rows, K] (the gradient rows), B_type [N, K] row-major,
+// on the half-precision matrix cores (v_mfma_f32_32x32x16_f16: eight times the flops of the fp32
+// instruction in 40 clocks against 64): both operands as two fp16 parts each, three matrix
+// instructions per product term.  A wavefront keeps its 32 rows of A in registers for the whole
+// kernel, so every row of A is read exactly once; the workgroup walks the N columns in blocks of 32,
+// each block of B staged through LDS (k contiguous, two copies) while the previous block is
+// multiplied, and every 32 x 32 block of C leaves straight from the accumulators.  The rows of A
+// take the wavefront's power of two, every row of B (a column of the product) its own, found by the
+// eight lanes that stage it; the product leaves the accumulators through the two inverse factors.
 template <int K>
 __global__ __launch_bounds__(PT) void typed_gemm_bt_rows_f16_kernel(const float* __restrict__ A, const float* __restrict__ Bm,
                                                                      size_t b_type_stride, float* __restrict__ C, int ldc,

@@ -62,9 +62,15 @@ def fchl_backwards(coordinates, charges, species, element_types, cell, inv_cell,
 
 def _counts(coordinates, charges):
     """The reference's signatures carry no atom counts (its kernels only walk the neighbour list
-    they are given).  Here they are recovered from the zero-padded charges (a real atom has a
-    positive charge, models/kernel.py:631-648), so that a call without a list, where the kernel
-    finds the neighbours itself, does not take padded slots for atoms at the origin."""
+    they are given).  Here they are recovered from the zero-padded charges (padding has charge
+    0 and trails the real atoms, models/kernel.py:631-648): the count of a molecule is the index
+    of its last atom with a non-zero charge, plus one, so that a call without a list, where the
+    kernel finds the neighbours itself, does not take padded slots for atoms at the origin,
+    and a dummy atom of charge zero INSIDE a molecule does not cut the molecule short (it gets
+    element type -1 and the kernels skip it as a neighbour; the reference's kernels index out of
+    bounds with such a type, fchl_cuda_kernel.cu:1732-1739)."""
     if charges.dim() == 1:
         charges = charges.unsqueeze(0)
-    return (charges > 0).sum(dim=1, dtype=torch.int32)
+    n = charges.shape[1]
+    pos = torch.arange(1, n + 1, device=charges.device, dtype=torch.int32)
+    return (pos * (charges != 0)).amax(dim=1).to(torch.int32) if n > 0 else charges.new_zeros(charges.shape[0], dtype=torch.int32)

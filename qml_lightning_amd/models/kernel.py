@@ -374,26 +374,47 @@ class BaseKernel():
             print("Best error: ", best[2], "sigma = ", best[0], "lambda = ", best[1])
         return best[0], best[1]
 
-    #: bytes of projected rows (all training batches of one fold) the grid search keeps on the device
+    #: upper bound, in bytes, on the projected rows (all training batches of one fold) the grid search keeps
+    #: on the device; the budget actually used is the smaller of this and half of the device memory that
+    #: is free once one batch's transient arrays (dense Jacobian, fp64 row matrix) are set aside
     grid_search_cache_bytes = 64 << 30
 
+    def _grid_search_budget(self, nmax, with_forces):
+        budget = int(self.grid_search_cache_bytes)
+        if torch.cuda.is_available() and self.device.type == "cuda":
+            free, _ = torch.cuda.mem_get_info(self.device)
+            free += torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device)
+            nb = int(self.nbatch_train)
+            rows = nb * (1 + (3 * nmax if with_forces else 0))
+            transient = 8 * rows * self.nfeatures()                                     # fp64 row matrix of a batch
+            if with_forces:
+                transient += 4 * nb * nmax * nmax * 3 * self.rep.get_repsize()          # its dense Jacobian
+            budget = min(budget, max(0, (free - transient) // 2))
+        return budget
+
     def _projected_batches(self, X, Q, E, F, cells, inv_cells):
-        """[(projected rows, targets)] of every training batch, or None when they would take more
-        than `grid_search_cache_bytes` (per atom: npcas floats, times 1 + 3 n with forces)."""
+        """[(projected rows, targets)] of every training batch, or None (the caller then rebuilds
+        the rows per grid point) when they would take more than the budget (per atom: npcas
+        floats, times 1 + 3 n with forces) or the device runs out of memory while building them."""
         nmax = max((len(q) for q in Q), default=0)
         natoms = sum(len(q) for q in Q)
         need = 4 * self.npcas * natoms * (1 + (3 * nmax if F is not None else 0))
-        if need > self.grid_search_cache_bytes:
+        if need > self._grid_search_budget(nmax, F is not None):
             return None
         out = []
-        for i in range(0, len(X), self.nbatch_train):
-            sl = slice(i, i + self.nbatch_train)
-            data = self.format_data(X[sl], Q[sl], E=E[sl] if E is not None else None,
-                                    F=F[sl] if F is not None else None,
-                                    cells=cells[sl] if cells is not None else None,
-                                    inv_cells=inv_cells[sl] if cells is not None else None)
-            targets = self._targets(data, data['charges'].shape[0], E is not None, F is not None)
-            out.append((self._batch_projected(data, F is not None), targets))
+        try:
+            for i in range(0, len(X), self.nbatch_train):
+                sl = slice(i, i + self.nbatch_train)
+                data = self.format_data(X[sl], Q[sl], E=E[sl] if E is not None else None,
+                                        F=F[sl] if F is not None else None,
+                                        cells=cells[sl] if cells is not None else None,
+                                        inv_cells=inv_cells[sl] if cells is not None else None)
+                targets = self._targets(data, data['charges'].shape[0], E is not None, F is not None)
+                out.append((self._batch_projected(data, F is not None), targets))
+        except torch.cuda.OutOfMemoryError:
+            del out
+            torch.cuda.empty_cache()
+            return None
         return out
 
     #: atoms the fused predict route aims to put into one launch chain (see _fused_batch)

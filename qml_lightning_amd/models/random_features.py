@@ -13,21 +13,27 @@ from .kernel import BaseKernel, _default_device, alpha_f32, rep_from_attribute_t
 
 
 class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
-    """`fused=True` (default where the kernel applies: npcas 64 or 128, a multiple of 32
-    features) runs forward() through one matrix-core kernel that never writes the
-    [atoms, nfeatures] matrix; `fused=False` is the reference's own operator sequence."""
+    """`fused=True` runs forward() through one matrix-core kernel that never writes the
+    [atoms, nfeatures] matrix; it exists for npcas 64 or 128 and a multiple of 32 features and
+    raises for other shapes.  `fused=False` is the reference's own operator sequence (library
+    GEMM).  `fused=None` (default) takes the fused kernel where it exists."""
 
     fused: Final[bool]
     separate_ops: Final[bool]
 
     def __init__(self, rep=None, elements=np.array([1, 6, 7, 8]), sigma=2.0, llambda=1e-10,
-                 nstacks=8192, npcas=128, nbatch_train=64, nbatch_test=64, fused=True,
+                 nstacks=8192, npcas=128, nbatch_train=64, nbatch_test=64, fused=None,
                  separate_ops=False):
         torch.nn.Module.__init__(self)
         BaseKernel.__init__(self, rep, npcas, elements, sigma, llambda)
         self.device = _default_device()
         self.npcas = npcas
-        self.fused = bool(fused) and npcas in (64, 128) and (nstacks * npcas) % 32 == 0
+        has_kernel = npcas in (64, 128) and (nstacks * npcas) % 32 == 0
+        if fused and not has_kernel:
+            raise ValueError("RandomFourrierFeaturesModel(fused=True): the fused kernel exists for npcas 64 or 128 and a "
+                             "multiple of 32 features, not npcas = %d with %d features; pass fused=False for the "
+                             "operator sequence of the reference" % (npcas, nstacks * npcas))
+        self.fused = has_kernel if fused is None else bool(fused)
         self.separate_ops = separate_ops   # fused route as five operators (one node each) instead of one
         self.nbatch_train = nbatch_train
         self.nbatch_test = nbatch_test
@@ -189,7 +195,7 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
         return predict_energies
 
     @classmethod
-    def from_reference_file(cls, file_name, fused=True, separate_ops=False):
+    def from_reference_file(cls, file_name, fused=None, separate_ops=False):
         """A RandomFourrierFeaturesModel holding the weights of a model file written by
         `save_jit_model` (random_features.py:233-235 of the reference), read as data: see
         HadamardFeaturesModel.from_reference_file.  `nstacks` is recovered from the number of

@@ -1,5 +1,5 @@
 """Measured ceilings of the GPU the library runs on, next to the nominal ones: fill and copy
-bandwidth, fp64 / fp32 matrix-core rate, transcendental rate.  Each probe is a few milliseconds
+bandwidth, fp64 / fp32 / fp16 matrix-core rate, transcendental rate.  Each probe is a few milliseconds
 of the library's own probe kernels, timed with HIP events on the current stream."""
 import ctypes
 
@@ -8,7 +8,7 @@ import torch
 from .. import _lib
 from ..ops import _ptr, _stream
 
-NOMINAL = {"hbm_GBs": 8000.0, "mfma_f64_TFLOPs": 78.6, "mfma_f32_TFLOPs": 157.3}
+NOMINAL = {"hbm_GBs": 8000.0, "mfma_f64_TFLOPs": 78.6, "mfma_f32_TFLOPs": 157.3, "mfma_f16_TFLOPs": 2500.0}
 
 
 def _timed(fn, iters):
@@ -25,7 +25,7 @@ def _timed(fn, iters):
 
 def measure(nbytes=1 << 30, device="cuda:0"):
     """{'hbm_fill_GBs', 'hbm_copy_GBs' (bytes read + written), 'mfma_f64_TFLOPs',
-    'mfma_f32_TFLOPs', 'exp_per_s'} of the current device."""
+    'mfma_f32_TFLOPs', 'mfma_f16_TFLOPs', 'exp_per_s'} of the current device."""
     L = _lib.lib()
     n = nbytes // 4
     src = torch.empty(n, dtype=torch.float32, device=device)
@@ -43,7 +43,7 @@ def measure(nbytes=1 << 30, device="cuda:0"):
     # the best over 1, 2, 4 and 8 wavefronts per SIMD (the rate a loop of nothing but matrix or
     # transcendental instructions holds depends on how many wavefronts issue them)
     for key, which, iters, scale in (("mfma_f64_TFLOPs", 0, 1000, 1e12), ("mfma_f32_TFLOPs", 1, 4000, 1e12),
-                                     ("exp_per_s", 2, 4000, 1.0)):
+                                     ("mfma_f16_TFLOPs", 3, 4000, 1e12), ("exp_per_s", 2, 4000, 1.0)):
         best = 0.0
         for per_cu in (1, 2, 4, 8):
             ops = [0.0]
@@ -59,9 +59,7 @@ def measure(nbytes=1 << 30, device="cuda:0"):
     return out
 
 
-MIXES = ("plain_fp32_x128", "dpp_fmac_x128", "transcendental_x128", "mfma_f32_16x16x4_x32", "fused_kernel_stack",
-         "fused_kernel_stack_mfma_trial", "mfma_f16_16x16x32_x16", "plain_fp32_x128_with_mfma_f16_x16", "split_f16_x32",
-         "vop3_fp32_x128")
+MIXES = ("plain_fp32_x128", "dpp_fmac_x128", "transcendental_x128", "fused_kernel_stack")
 
 
 def instruction_mixes(device="cuda:0", iters=2000):

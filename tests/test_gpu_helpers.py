@@ -56,29 +56,6 @@ def test_autograd_wrappers_forward_and_gradient():
     close(xt.grad, sorf.sorf_adjoint(g_c.reshape(A, S, d), D, norm), 1e-4, "gradient")
 
 
-def test_free_functions_of_the_sorf_module():
-    from qml_lightning_amd.features import SORF
-    x, D, b, idx, u = case(3, T=1)
-    A, d = x.shape
-    S, nmol, norm = D.shape[1], 4, 2.25
-    Dt, bt, it = torch.tensor(D, device=dev()), torch.tensor(b, device=dev()), torch.tensor(idx, device=dev())
-    coeffs = SORF.get_SORF_coefficients(torch.tensor(x, device=dev()), Dt, norm)
-    c_ref = sorf.sorf_coefficients(x, D, norm).reshape(A, -1)
-    close(coeffs, c_ref, REL, "get_SORF_coefficients")
-    feats = SORF.get_features(coeffs, bt, it, nmol)
-    assert feats.dtype == torch.float64
-    close(feats, sorf.cos_features(c_ref, b, idx, nmol), REL, "get_features")
-    G = SORF.get_feature_derivatives(coeffs, bt, Dt, torch.tensor(u, device=dev()), it, nmol, norm)
-    ref = sorf.derivative_features(sorf.sin_coeffs(c_ref, b), norm, idx, u, D, nmol)
-    close(G, ref, REL, "get_feature_derivatives")
-    np.random.seed(5)
-    Dm = SORF.get_SORF_diagonals([1, 6], 2, 3, 8)
-    bm = SORF.get_bias([1, 6], 24)
-    assert set(Dm) == {1, 6} and Dm[6].shape == (2, 3, 8) and Dm[1].is_cuda
-    assert torch.all(Dm[1].abs() == 1.0) and not torch.equal(Dm[1], Dm[6])
-    assert bm[1].shape == (24,) and float(bm[1].min()) >= 0.0 and float(bm[6].max()) <= 2 * np.pi
-
-
 def test_per_element_reductor_fit():
     """Columns = leading left singular vectors of the element's rows: orthonormal, and they span
     the same subspace as numpy's SVD of the same rows (all rows are used while there are at most

@@ -203,3 +203,14 @@ def test_gram_tile_map_meets_every_tile_once_and_balances_the_xcds(tmp_path):
     out = subprocess.run([exe], capture_output=True, text=True)
     assert out.returncode == 0, out.stdout + out.stderr
     assert out.stdout.startswith("ok")
+
+
+def test_rff_fused_true_refuses_a_width_without_a_fused_kernel():
+    from qml_lightning_amd.models.random_features import RandomFourrierFeaturesModel
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    rep = FCHLCuda(species=np.array([1, 6]))
+    with pytest.raises(ValueError, match="fused kernel exists for npcas 64 or 128"):
+        RandomFourrierFeaturesModel(rep=rep, elements=np.array([1, 6]), nstacks=2, npcas=256, fused=True)
+    auto = RandomFourrierFeaturesModel(rep=rep, elements=np.array([1, 6]), nstacks=2, npcas=256)
+    assert auto.fused is False
+    assert RandomFourrierFeaturesModel(rep=rep, elements=np.array([1, 6]), nstacks=2, npcas=64).fused is True
