@@ -1,8 +1,10 @@
-"""The benchmark configurations at their full sizes, checked through properties that do not need
-the CPU oracle (which takes minutes at these sizes): the result of one large batch equals the
-results of its parts, energies are invariant and forces covariant under rigid motions, forces are
-the directional derivative of the energy, the Gram matrix satisfies its checksum identities and the
-solve its residual bound.  Small-size parity against the oracle is in test_gpu_kernels.py /
+"""The benchmark configurations at their full sizes.  Against the CPU oracle: a seeded sample of
+molecules drawn from the full batch's OWN output (the oracle needs minutes for a whole batch, the
+molecules are independent, so the large-batch kernels are checked on the rows they wrote).  Beyond
+the sample, through properties that do not need the oracle: the result of one large batch equals
+the results of its parts, energies are invariant and forces covariant under rigid motions, forces
+are the directional derivative of the energy, the Gram matrix satisfies its checksum identities and
+the solve its residual bound.  Small-size parity against the oracle is in test_gpu_kernels.py /
 test_gpu_model.py."""
 import numpy as np
 import pytest
@@ -38,6 +40,31 @@ def step(m, coords, charges, forces=True):
     return out, None
 
 
+def sample_against_oracle(m, species, coords, charges, E, F, nsample, seed, rff=False, tol=1e-4):
+    """Energies (and forces) of `nsample` molecules picked from the full batch's output against the
+    fp64 oracle run on just those molecules; tolerance of energies and forces, 1e-4 of the sample's
+    largest entry."""
+    from oracle import model as omodel
+    from tests.test_gpu_kernels import make_batch, oracle_prm
+    pick = np.sort(np.random.default_rng(seed).choice(len(coords), size=nsample, replace=False))
+    X, Z, aid, mid, nat = make_batch([coords[i] for i in pick], [charges[i] for i in pick])
+    prm = oracle_prm(species)
+    red = m.reductors.double().cpu().numpy()
+    alpha = m.alpha.float().double().cpu().numpy()              # the predict route contracts with fp32 alpha
+    if rff:
+        Eo, Fo, _ = omodel.rff_energy_forces(X, Z, aid, mid, nat, prm, species, red, m.W.double().cpu().numpy(),
+                                             m.b.double().cpu().numpy(), alpha, forces=F is not None)
+    else:
+        Eo, Fo, _ = omodel.sorf_energy_forces(X, Z, aid, mid, nat, prm, species, red, m.Dmat.double().cpu().numpy(),
+                                              m.bias.double().cpu().numpy(), alpha, float(m.sigma),
+                                              forces=F is not None)
+    idx = torch.tensor(pick, device=dev())
+    within(E[idx].double(), torch.tensor(Eo, device=dev()), tol, "sampled energies vs oracle")
+    if F is not None:
+        n = Fo.shape[1]
+        within(F[idx][:, :n].double(), torch.tensor(Fo, device=dev()), tol, "sampled forces vs oracle")
+
+
 def within(a, b, tol, what):
     """max |a - b| <= tol * max |b|, with a short message."""
     err, scale = float((a - b).abs().max()), float(b.abs().max())
@@ -62,6 +89,8 @@ def test_config2_batch_of_4096_equals_its_parts_and_respects_rigid_motions():
     assert E.shape == (4096,) and F.shape == (4096, 21, 3)
     assert torch.isfinite(E).all() and torch.isfinite(F).all()
     escale, fscale = float(E.abs().max()), float(F.abs().max())
+    # 32 molecules of this very output against the oracle
+    sample_against_oracle(m, species, coords, charges, E, F, 32, seed=21)
     # the same molecules in batches of 500 and in reversed order
     for lo in range(0, 4096, 500):
         e, f = step(m, coords[lo:lo + 500], charges[lo:lo + 500])
@@ -105,6 +134,7 @@ def test_config3_ragged_8192_energies_equal_their_parts():
     E, _ = step(m, coords, charges, forces=False)
     assert E.shape == (8192,) and torch.isfinite(E).all()
     scale = float(E.abs().max())
+    sample_against_oracle(m, [1, 6, 7, 8, 9], coords, charges, E, None, 32, seed=22)
     for lo in (0, 3000, 8000):
         e, _ = step(m, coords[lo:lo + 192], charges[lo:lo + 192], forces=False)
         within(e, E[lo:lo + 192], 1e-5, "e")
@@ -120,6 +150,7 @@ def test_config4_32768_features_batch_equals_its_parts():
     m = sorf_model([1, 6, 7, 8], 256, 128)
     E, F = step(m, coords, charges)
     assert torch.isfinite(E).all() and torch.isfinite(F).all()
+    sample_against_oracle(m, [1, 6, 7, 8], coords, charges, E, F, 8, seed=23)
     e, f = step(m, coords[1000:1300], charges[1000:1300])
     within(e, E[1000:1300], 1e-5, "e")
     within(f, F[1000:1300], 1e-5, "f")
@@ -157,6 +188,7 @@ def test_config5_rff_32768_features_batch_equals_its_parts():
     m.is_trained = True
     E, F = step(m, coords, charges)
     assert torch.isfinite(E).all() and torch.isfinite(F).all()
+    sample_against_oracle(m, species, coords, charges, E, F, 8, seed=24, rff=True)
     e, f = step(m, coords[700:900], charges[700:900])
     # 32768 fp32 terms per energy, summed in an order that depends on the batch size
     within(e, E[700:900], 5e-5, "rff energies, part vs whole")

@@ -238,8 +238,10 @@ def test_known_answer_through_a_model_file_read_as_data(kat, tmp_path):
         got = F.squeeze(0).cpu().numpy()
         assert np.isclose(d["ref_forces"], got, rtol=1e-4, atol=1e-3).all()
         results.append((E.item(), got))
-    # the reference route from the file read as data IS the scripted file's arithmetic
-    assert results[1][0] == results[2][0] and np.array_equal(results[1][1], results[2][1])
+    # the reference route from the file read as data IS the scripted file's arithmetic (the forces
+    # go through the FCHL19 backward kernel, whose cross-atom sums are fp32 atomics in any order)
+    assert results[1][0] == results[2][0]
+    assert np.abs(results[1][1] - results[2][1]).max() < 2e-6 * np.abs(results[2][1]).max()
     assert abs(results[0][0] - results[1][0]) < 1e-4 * abs(results[1][0])
     assert np.abs(results[0][1] - results[1][1]).max() < 1e-4 * np.abs(results[1][1]).max()
 
