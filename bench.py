@@ -543,6 +543,24 @@ def main():
         ZTZ, ZTy = model.build_Z_components(tc, tq, E=Et, F=Ft, print_info=False)
         torch.cuda.synchronize()
         t_build = time.perf_counter() - t0
+        # the same training set handed over as zero-padded arrays (X [N,n,3], Q [N,n], E [N], F [N,n,3]):
+        # the formatter then uploads the arrays as they are and everything else happens on the device
+        Xp = np.ascontiguousarray(np.stack(tc), dtype=np.float32)
+        Qp = np.ascontiguousarray(np.stack(tq), dtype=np.float32)
+        Fp = np.stack(Ft)
+        model.format_data(Xp[:64], Qp[:64], E=Et[:64], F=Fp[:64])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for b0 in range(0, NMOL_TRAIN, 500):
+            model.format_data(Xp[b0:b0 + 500], Qp[b0:b0 + 500], E=Et[b0:b0 + 500], F=Fp[b0:b0 + 500])
+        torch.cuda.synchronize()
+        t_format_padded = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        ZTZp, ZTyp = model.build_Z_components(Xp, Qp, E=Et, F=Fp, print_info=False)
+        torch.cuda.synchronize()
+        t_build_padded = time.perf_counter() - t0
+        padded_equal = bool(torch.equal(ZTZp, ZTZ))
+        del ZTZp, ZTyp
         # one 500-molecule batch of that build, phase by phase (each timed alone, so their sum exceeds the
         # batch's share of the build, where the host runs ahead of the device)
         bd = model.format_data(tc[:500], tq[:500], E=Et[:500], F=Ft[:500])
@@ -587,7 +605,9 @@ def main():
         train = {"ztz_seconds": t_build, "ztz_molecules": NMOL_TRAIN, "ztz_rows": M, "ztz_features": F,
                  "ztz_includes": "host format_data + FCHL19 Jacobian + projection + SORF rows + Gram, 500 molecules per batch",
                  "ztz_seconds_excluding_format_data": t_build - t_format, "format_data_seconds": t_format,
-                 "gram_kernel_seconds": t_gram, "one_batch_phases": batch_phases}
+                 "gram_kernel_seconds": t_gram, "one_batch_phases": batch_phases,
+                 "from_padded_arrays": {"ztz_seconds": t_build_padded, "format_data_seconds": t_format_padded,
+                                        "ztz_bit_equal_to_list_route": padded_equal}}
         train.update(solve)
         if solve:
             kernels["cholesky_solve_f64"] = {"seconds": solve["solve_seconds"], "bound": "mfma",

@@ -126,15 +126,33 @@ class BaseKernel():
         # one typed product then serves all elements (for the derivative rows, 3n rows per atom), where
         # the reference copies each element's rows out and multiplies them one element at a time
         ne = self.reductors.shape[0]
-        lists = [None] * ne
-        for e in self.elements:
-            lists[self.element2index[int(e)]] = (e, self._element_index(data, charges, int(e)))
-        counts = [0 if l is None else int(l[1].shape[0]) for l in lists]
-        offsets = np.concatenate(([0], np.cumsum(counts))).astype(np.int32)
         items = []
+        ecounts = data.get('element_counts')
+        if ecounts is not None:
+            # the element-sorted atom index is built on the device (one counting sort over the batch,
+            # stable: ascending slot within an element, the order of `rep[Z == e]`); only the per-element
+            # counts, which the formatter took from the host copy of the charges, are needed here
+            counts = [0] * ne
+            order = [None] * ne
+            for e in self.elements:
+                t = int(self.element2index[int(e)])
+                counts[t], order[t] = int(ecounts.get(int(e), 0)), e
+            offsets = np.concatenate(([0], np.cumsum(counts))).astype(np.int32)
+            if offsets[-1] > 0:
+                types = ops.element_types(coordinates, charges, natom_counts, self._sort_species_tensor())
+                slots, type_offsets = ops.sort_atoms_by_type(types, atomIDs, molIDs, n, ne)
+                slots = slots[:int(offsets[-1])]
+        else:
+            lists = [None] * ne
+            for e in self.elements:
+                lists[self.element2index[int(e)]] = (e, self._element_index(data, charges, int(e)))
+            counts = [0 if l is None else int(l[1].shape[0]) for l in lists]
+            order = [None if l is None else l[0] for l in lists]
+            offsets = np.concatenate(([0], np.cumsum(counts))).astype(np.int32)
+            if offsets[-1] > 0:
+                slots = torch.cat([l[1] for l in lists if l is not None and l[1].shape[0] > 0]).to(torch.int32)
+                type_offsets = torch.from_numpy(offsets).to(slots.device)
         if offsets[-1] > 0:
-            slots = torch.cat([l[1] for l in lists if l is not None and l[1].shape[0] > 0]).to(torch.int32)
-            type_offsets = torch.from_numpy(offsets).to(slots.device)
             # the tiled product for both: a row's result then does not depend on how many rows the batch has
             x_all = ops.project_typed_rows(flat_rep, slots, type_offsets, self.reductors, 1)
             g_all = None
@@ -142,12 +160,12 @@ class BaseKernel():
                 g_all = ops.project_typed_rows(rep_derivative.view(B * n * n * 3, -1), slots, type_offsets,
                                                self.reductors, 3 * n)
             mol_of_atom = torch.div(slots, n, rounding_mode='floor')
-            for t, l in enumerate(lists):
+            for t in range(ne):
                 if counts[t] == 0:
                     continue
                 o0, o1 = int(offsets[t]), int(offsets[t + 1])
                 sub_grad = g_all[o0 * 3 * n:o1 * 3 * n].view(o1 - o0, n, 3, -1) if with_forces else None
-                items.append((l[0], mol_of_atom[o0:o1], x_all[o0:o1], sub_grad))
+                items.append((order[t], mol_of_atom[o0:o1], x_all[o0:o1], sub_grad))
         return {'B': B, 'n': n, 'device': coordinates.device, 'items': items}
 
     def _rows_from_projected(self, proj, with_forces, zero_energy_rows=False):
@@ -177,16 +195,22 @@ class BaseKernel():
         """Rows of one formatted batch: representation (+ Jacobian), projection, features."""
         return self._rows_from_projected(self._batch_projected(data, with_forces), with_forces, zero_energy_rows)
 
+    def _sort_species_tensor(self):
+        """The model's elements as the float tensor `ops.element_types` compares charges with, in
+        the order of the projection matrices (element2index)."""
+        t = getattr(self, '_sort_species_cache', None)
+        if t is None or t.device != self.reductors.device:
+            vals = np.zeros(self.reductors.shape[0], dtype=np.float32)
+            for e in self.elements:
+                vals[int(self.element2index[int(e)])] = float(e)
+            t = torch.from_numpy(vals).to(self.reductors.device)
+            self._sort_species_cache = t
+        return t
+
     @staticmethod
     def _element_index(data, charges, e):
-        """Flat (molecule-major) indices of the atoms of element e.  `format_data` prepares
-        them on the host; tensors that did not come from it fall back to a device search."""
-        table = data.get('element_index')
-        if table is not None:
-            idx = table.get(e)
-            if idx is None:
-                return torch.zeros(0, dtype=torch.long, device=charges.device)
-            return idx
+        """Flat (molecule-major) indices of the atoms of element e by a device search (the reductor
+        fit, and batches that did not come from `format_data`)."""
         return torch.nonzero(charges.reshape(-1).int() == e).reshape(-1)
 
     # -- training -------------------------------------------------------------------------
@@ -579,22 +603,26 @@ class BaseKernel():
         print("Self Energies: ", self.self_energy)
 
     # -- batch formatting -------------------------------------------------------------------
-    def _format_padded_arrays(self, X, Q, cells=None, inv_cells=None):
+    def _format_padded_arrays(self, X, Q, E=None, F=None, cells=None, inv_cells=None):
         """format_data for a batch that already is one zero-padded array pair X [B,n,3], Q [B,n]
         (charge 0 = padding, real atoms first in every row: the layout format_data itself
-        produces, kernel.py:630-695).  Two uploads; counts, atom and molecule indices are built
-        on the device, with no Python loop over molecules."""
+        produces, kernel.py:630-695), with energies E [B] and forces F [B,n,3] (zero-padded) when
+        it is a training batch.  One upload per array; counts, atom and molecule indices, the
+        self-energy correction and the unit conversion are done on the device, with no Python loop
+        over molecules; the per-element atom index is left to a device sort (`_batch_projected`),
+        for which only the element counts are taken here, from the host copy of the charges."""
         dev = self.device
         B, n = Q.shape
         coords = torch.from_numpy(np.ascontiguousarray(X, dtype=np.float32)).to(dev)
         charges = torch.from_numpy(np.ascontiguousarray(Q, dtype=np.float32)).to(dev)
         mask = charges > 0
         counts = mask.sum(dim=1, dtype=torch.int32)
-        if bool(mask.all()):                               # fixed composition: no search needed
+        hostmask = np.asarray(Q) > 0
+        if hostmask.all():                                 # fixed composition: no search needed
             flat = torch.arange(B * n, device=dev)
         else:
             # padding must trail the real atoms of its row
-            if bool((mask[:, 1:] & ~mask[:, :-1]).any()):
+            if (hostmask[:, 1:] & ~hostmask[:, :-1]).any():
                 raise RuntimeError("format_data: padded rows must hold their real atoms first")
             flat = mask.reshape(-1).nonzero()[:, 0]
         data = {
@@ -607,11 +635,36 @@ class BaseKernel():
             'forces': None,
             'cells': torch.empty((0, 3, 3), device=dev),
             'inv_cells': torch.empty((0, 3, 3), device=dev),
-        }   # no 'element_index': the per-element lists are searched on the device when a caller needs them
+        }
+        if E is not None or F is not None:
+            data['element_counts'] = self._element_counts(np.asarray(Q).reshape(-1))
+        if E is not None:
+            energies = torch.from_numpy(np.ascontiguousarray(E, dtype=np.float64).reshape(B)).to(dev)
+            if self.convert_hartree2kcal():
+                energies = energies * self.hartree2kcalmol
+            if self.subtract_self_energies():
+                se = self.self_energy.to(dev)
+                energies = energies - se[charges.long()].sum(dim=1)        # se[0] = 0: padding adds nothing
+            data['energies'] = energies
+        if F is not None:
+            Fa = np.asarray(F, dtype=np.float64)
+            if Fa.shape != (B, n, 3):
+                raise RuntimeError("format_data: forces of a padded batch must be one [B, n, 3] array, got %s"
+                                   % (Fa.shape,))
+            forces = torch.from_numpy(np.ascontiguousarray(Fa)).to(dev)
+            if self.convert_hartree2kcal():
+                forces = forces * self.hartree2kcalmol
+            data['forces'] = forces * mask[:, :, None]                      # padded slots carry no target
         if cells is not None:
             data['cells'] = torch.from_numpy(np.asarray(cells, dtype=np.float32).reshape(B, 3, 3)).to(dev)
             data['inv_cells'] = torch.from_numpy(np.asarray(inv_cells, dtype=np.float32).reshape(B, 3, 3)).to(dev)
         return data
+
+    def _element_counts(self, flat_charges):
+        """{element: number of atoms} of a batch from the host copy of its charges (one bincount)."""
+        q = np.asarray(flat_charges).astype(np.int64, copy=False)
+        hist = np.bincount(q[q >= 0], minlength=int(self.element2index.shape[0]))
+        return {int(e): int(hist[int(e)]) for e in self.elements}
 
     @staticmethod
     def _concat_rows(items, width, dtype):
@@ -629,17 +682,17 @@ class BaseKernel():
     def format_data(self, X, Q, E=None, F=None, cells=None, inv_cells=None):
         """Lists of per-molecule arrays -> zero-padded device tensors with the keys
         coordinates / charges / natom_counts / atomIDs / molIDs / energies / forces /
-        cells / inv_cells (kernel.py:601-722), plus 'element_index': {element: int64 flat
-        indices of its atoms}, computed here on the host so later gathers need no device
-        search."""
+        cells / inv_cells (kernel.py:601-722), plus, for a training batch, 'element_counts':
+        {element: number of its atoms}, so that the element-sorted atom index can be built by a
+        device sort without a host round trip.  X [B,n,3] and Q [B,n] given as zero-padded
+        arrays (with E [B], F [B,n,3]) are uploaded as they are."""
         if self.subtract_self_energies() and self.self_energy is None:
             raise RuntimeError("ERROR: must call model.calculate_self_energy first - this computes atomic "
                                "contributes to the potential energy.")
         dev = self.device
         zbatch = len(X)
-        if (isinstance(X, np.ndarray) and X.ndim == 3 and isinstance(Q, np.ndarray) and Q.ndim == 2
-                and E is None and F is None and not self.subtract_self_energies()):
-            return self._format_padded_arrays(X, Q, cells, inv_cells)
+        if isinstance(X, np.ndarray) and X.ndim == 3 and isinstance(Q, np.ndarray) and Q.ndim == 2:
+            return self._format_padded_arrays(X, Q, E, F, cells, inv_cells)
         counts = np.fromiter(map(len, X), dtype=np.int32, count=zbatch)
         n = int(counts.max()) if zbatch else 0
         # one concatenation and one scatter instead of a Python loop over molecules
@@ -665,10 +718,9 @@ class BaseKernel():
         }
         flat_q = charges.reshape(-1).astype(np.int64)
         if E is not None or F is not None:
-            # training batches gather rows per element: the index lists are cheap to build here on
-            # the host; a predict batch never needs them (its atoms are sorted on the device)
-            data['element_index'] = {int(e): torch.from_numpy(np.nonzero(flat_q == int(e))[0]).to(dev)
-                                     for e in self.elements}
+            # training batches gather rows per element: the element-sorted atom index is built on the
+            # device (`_batch_projected`), which needs only the per-element counts from here
+            data['element_counts'] = self._element_counts(flat_q)
         if E is not None:
             energies = np.array(E, dtype=np.float64).reshape(zbatch).copy()
             if self.convert_hartree2kcal():

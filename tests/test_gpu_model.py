@@ -306,6 +306,55 @@ def test_training_rows_and_gram_vs_oracle(mode):
         assert m.alpha.shape == (m.nfeatures(),) and torch.isfinite(m.alpha).all()
 
 
+def test_training_rows_of_a_padded_array_batch_vs_oracle_and_list_route():
+    """A ragged training batch handed over as one zero-padded array pair with E [B] and F [B,n,3]
+    (device-side formatter, element index by a device sort) gives the rows of the fp64 oracle and,
+    bit for bit, the rows and Z^T Z of the per-molecule-list route (kernel.py:601-722,143-160)."""
+    species = [1, 6, 7, 8, 9]
+    coords, charges = helpers.ragged_batch(9, 4)
+    m, (red, D, bias, alpha) = build_sorf_model(species, 64, 2)
+    m.nbatch_train = 9
+    prm = oracle_prm(species)
+    rng = np.random.default_rng(3)
+    c32 = [np.asarray(c, dtype=np.float32) for c in coords]
+    B, n = len(c32), max(len(q) for q in charges)
+    E = rng.normal(size=B)
+    Fl = [rng.normal(size=(len(q), 3)) for q in charges]
+    Xp, Qp, Fp = np.zeros((B, n, 3), dtype=np.float32), np.zeros((B, n), dtype=np.float32), np.zeros((B, n, 3))
+    for i, (c, q, f) in enumerate(zip(c32, charges, Fl)):
+        Xp[i, :len(q)], Qp[i, :len(q)], Fp[i, :len(q)] = c, q, f
+    dl = m.format_data(c32, charges, E=E, F=Fl)
+    dp = m.format_data(Xp, Qp, E=E, F=Fp)
+    for key in ("coordinates", "charges", "natom_counts", "atomIDs", "molIDs", "energies", "forces"):
+        assert dl[key].dtype == dp[key].dtype and torch.equal(dl[key], dp[key]), key
+    rl, rp = m._batch_rows(dl, True), m._batch_rows(dp, True)
+    assert torch.equal(rl, rp)
+    X, Z, aid, mid, nat = make_batch(coords, charges)
+    Fo = np.zeros((B, n, 3))
+    for i, f in enumerate(Fl):
+        Fo[i, :len(f)] = f
+    r, y = omodel.sorf_training_rows(X, Z, aid, mid, nat, prm, species, red, D, bias, 2.0, E=E, F=Fo)
+    close(rp, r, REL_REP, "rows of the padded batch")
+    close(m._targets(dp, B, True, True), y, 1e-14, "targets of the padded batch")
+    # the element index of the device sort is the molecule-major search of the reference
+    types = m._sort_species_tensor()
+    assert [float(v) for v in types.cpu()] == [float(e) for e in species]
+    Zl, yl = m.build_Z_components(c32, charges, E=E, F=Fl, print_info=False)
+    Zp, yp = m.build_Z_components(Xp, Qp, E=E, F=Fp, print_info=False)
+    assert torch.equal(Zl, Zp) and torch.allclose(yl, yp, rtol=1e-12, atol=1e-12)   # Z^T y: fp64 atomics
+    # a model whose elements are a permuted subset of the batch's: atoms of other elements give no rows
+    from qml_lightning_amd.models.hadamard_features import HadamardFeaturesModel
+    sub = HadamardFeaturesModel(rep=m.rep, elements=np.array([8, 1, 6]), ntransforms=1, sigma=2.0, npcas=64, nstacks=2)
+    perm = [species.index(e) for e in (8, 1, 6)]
+    sub.reductors, sub.Dmat, sub.bias = m.reductors[perm].clone(), m.Dmat[perm].clone(), m.bias[perm].clone()
+    ds = sub.format_data(Xp, Qp, E=E, F=Fp)
+    rs = sub._batch_rows(ds, True)
+    # the oracle's element loop (hadamard_features.py:99) never selects the N and F atoms either
+    r_sub, _ = omodel.sorf_training_rows(X, Z, aid, mid, nat, prm, [8, 1, 6], red[perm], D[perm], bias[perm], 2.0,
+                                         E=E, F=Fo)
+    close(rs, r_sub, REL_REP, "rows of a model with fewer elements than the batch")
+
+
 @pytest.mark.parametrize("ragged", [False, True])
 def test_format_data_of_padded_arrays_equals_the_list_route(ragged):
     """One zero-padded array pair goes through the device-side formatter; lists of per-molecule
@@ -328,8 +377,6 @@ def test_format_data_of_padded_arrays_equals_the_list_route(ragged):
     b = m.format_data(Xp, Qp)
     for key in ("coordinates", "charges", "natom_counts", "atomIDs", "molIDs"):
         assert a[key].dtype == b[key].dtype and torch.equal(a[key], b[key]), key
-    for e in species:
-        assert torch.equal(m._element_index(a, a["charges"], e), m._element_index(b, b["charges"], e))
     ea, fa = m.predict(c32, charges, n, forces=True, print_info=False)
     eb, fb = m.predict(Xp, Qp, n, forces=True, print_info=False)
     assert torch.equal(ea, eb)

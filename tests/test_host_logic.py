@@ -44,8 +44,10 @@ def test_format_data_matches_oracle_layout():
     assert (d['forces'][0, 3:] == 0).all()
     assert d['cells'].shape == (0, 3, 3)
     flat = Z.reshape(-1).astype(int)
+    # a training batch carries the per-element atom counts (the index itself is a device sort)
+    assert d['element_counts'] == {e: int((flat == e).sum()) for e in (1, 6, 8)}
     for e in (1, 6, 8):
-        assert (d['element_index'][e].cpu().numpy() == np.nonzero(flat == e)[0]).all()
+        assert (m._element_index(d, d['charges'], e).cpu().numpy() == np.nonzero(flat == e)[0]).all()
     t = m._targets(d, 3, True, True)
     assert t.shape == (3 + 3 * 5 * 3, 1) and t[1, 0] == 2.0
     assert np.allclose(t[3:, 0].cpu().numpy(), d['forces'].cpu().numpy().reshape(-1))
@@ -55,9 +57,26 @@ def test_format_data_matches_oracle_layout():
     d2 = m.format_data([c.tolist() for c in coords], [q.tolist() for q in charges])
     for key in ("coordinates", "charges", "atomIDs", "molIDs", "natom_counts"):
         assert torch.equal(d2[key], d[key]), key
-    assert 'element_index' not in d2 and d2['energies'] is None and d2['forces'] is None
-    for e in (1, 6, 8):
-        assert torch.equal(m._element_index(d2, d2['charges'], e), d['element_index'][e])
+    assert 'element_counts' not in d2 and d2['energies'] is None and d2['forces'] is None
+    # the same batch as one zero-padded array pair with targets: identical tensors, self energies included
+    Xp, Qp, Fp = np.zeros((3, 5, 3)), np.zeros((3, 5)), np.zeros((3, 5, 3))
+    for k, (c, q, f) in enumerate(zip(coords, charges, F)):
+        Xp[k, :len(q)], Qp[k, :len(q)], Fp[k, :len(q)] = c, q, f
+    Fp[0, 4] = 7.0                                    # a target in a padded slot is dropped
+    d3 = m.format_data(Xp, Qp, E=np.array(E), F=Fp)
+    for key in ("coordinates", "charges", "atomIDs", "molIDs", "natom_counts", "energies", "forces"):
+        assert d3[key].dtype == d[key].dtype and torch.equal(d3[key], d[key]), key
+    assert d3['element_counts'] == d['element_counts']
+    m.self_energy = torch.tensor([0.0, -0.5, 0, 0, 0, 0, -38.0, 0, -75.0], dtype=torch.float64)
+    m.set_subtract_self_energies(True)
+    m.set_convert_hartree2kcal(True)
+    dl = m.format_data(coords, charges, E=E, F=F)
+    dp = m.format_data(Xp, Qp, E=np.array(E), F=Fp)
+    assert torch.allclose(dl['energies'], dp['energies'], rtol=1e-14, atol=0) and torch.equal(dl['forces'], dp['forces'])
+    m.set_subtract_self_energies(False)
+    m.set_convert_hartree2kcal(False)
+    with pytest.raises(RuntimeError, match="real atoms first"):
+        m.format_data(Xp[:, ::-1].copy(), Qp[:, ::-1].copy())
     # the fallback for rows that do not stack directly (a flattened force array)
     rows = m._concat_rows([np.arange(6.0), np.arange(9.0).reshape(3, 3)], 3, np.float64)
     assert rows.shape == (5, 3) and rows[1, 0] == 3.0 and rows[2, 1] == 1.0
