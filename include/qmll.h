@@ -321,16 +321,31 @@ int qmll_rff_derivative_features(const float* x, const float* grad, const double
                                  const int* mol_index, const int* seg_offsets, int A, int n, int d, int F,
                                  int nmol, double* G, qmll_stream_t stream);
 
+/* W f32 [ne,d,F] of a RandomFourrierFeaturesModel (qml_lightning/models/random_features.py:42-55) is
+ * a constant of the model: it is split ONCE into the form the fused predict kernel multiplies with
+ * (per element and 32-feature chunk: the chunk scaled by a power of two of its own, every entry as two
+ * fp16 parts, in the two layouts the kernel's matrix instructions read, laid out byte for byte as
+ * the kernel keeps it in LDS) so that no workgroup repeats the split.  d is 64 or 128, F a multiple
+ * of 32.  qmll_rff_presplit_bytes: size of that form in bytes (0 for unsupported sizes); the caller
+ * owns the buffer (16-byte aligned) and refreshes it when W changes. */
+size_t qmll_rff_presplit_bytes(int ne, int d, int F);
+int qmll_rff_presplit(const float* W, int ne, int d, int F, void* W_split, size_t W_split_bytes, qmll_stream_t stream);
+
 /* Fused RFF predict path on element-sorted rows (x f32 [A,d] from qmll_project_typed).
  * Replaces, for all elements at once, the loop body of the reference's TorchScript forward
  * (qml_lightning/models/random_features.py:88-102: matmul(sub, W[e]) + b, cos, index_add,
  * matmul(Ztest, alpha)) and its autograd transpose; the [atoms,F] feature matrix is never
- * written.  W f32 [ne,d,F], b f32 [ne,F], alpha f32 [F]; d is 64 or 128, F a multiple of 32.
+ * written.  W_split: W [ne,d,F] as prepared by qmll_rff_presplit, b f32 [ne,F], alpha f32 [F];
+ * d is 64 or 128, F a multiple of 32.
  *   -> e_slots[sorted_slots[a]] = sqrt(2/F) sum_f alpha_f cos(x_a . W_t[:,f] + b_t[f])
  *      (only atoms a < type_offsets[ne]; e_slots must arrive zero-filled: the launch may
- *      split the features in two halves that add into it)
- *   -> gx f32 [A,d] = d e / d x (rows beyond type_offsets[ne] zero; NULL = energies only) */
-int qmll_rff_energy_sorted(const float* x, const int* type_offsets, const int* sorted_slots, const float* W,
+ *      split the features in parts that add into it)
+ *   -> gx f32 [A,d] = d e / d x (rows beyond type_offsets[ne] zero; NULL = energies only)
+ * The products run on the fp16 matrix cores with every fp32 operand as two fp16 parts behind a
+ * power-of-two scale (x per 32 atoms, W per chunk, alpha per launch part) and fp32 accumulation:
+ * a row's rounding depends on the largest entry among the 32 rows that share its wavefront, and
+ * non-finite entries of x, W or alpha give non-finite (not necessarily equal) results. */
+int qmll_rff_energy_sorted(const float* x, const int* type_offsets, const int* sorted_slots, const void* W_split,
                            const float* b, const float* alpha, int A, int ne, int d, int F, float* e_slots,
                            float* gx, qmll_stream_t stream);
 

@@ -228,24 +228,98 @@ constexpr int RE_FC = 32;        // features per staged chunk (one block of 32 r
 // fp16 subnormals are kept by the matrix cores, so small entries beside large ones lose only bits
 // below 2^-38 of the largest.
 //
-// W is staged twice per chunk, split on the way: feature-major with k contiguous (A operand of the
-// first product, rows = features) and k-major with the chunk's 32 features contiguous (A operand of the
-// second, rows = k), the features in the order in which the first product's accumulator registers hold
-// them (register r of half h: feature 8(r/4) + 4h + r%4), so the split P goes straight from registers
-// into the B operand.
+// W is a constant of the model, so it is split ONCE (rff_presplit_kernel) into the very bytes the
+// predict kernel wants in LDS: per element and 32-feature chunk an image holding the chunk twice,
+// feature-major with k contiguous (A operand of the first product, rows = features) and k-major with
+// the chunk's 32 features contiguous (A operand of the second, rows = k), the features in the order in
+// which the first product's accumulator registers hold them (register r of half h: feature
+// 8(r/4) + 4h + r%4), so the split P goes straight from registers into the B operand; hi and lo parts
+// each, row padding included.  The predict kernel then moves an image into LDS with direct
+// global-to-LDS loads (no registers, no vector instructions), the next chunk's while this one is
+// multiplied.
+template <int D>
+struct RffImage {
+    static constexpr int LD1 = D + 8;                // halves per row of the feature-major copy
+    static constexpr int LD2 = RE_FC + 8;            // halves per row of the k-major copy
+    static constexpr int W1H = 0, W1L = RE_FC * LD1, W2H = 2 * RE_FC * LD1, W2L = W2H + D * LD2;
+    static constexpr int HALVES = W2L + D * LD2;
+    static constexpr int BYTES = HALVES * 2;         // 37888 (D = 128), 19456 (D = 64): whole KiB
+    static constexpr int BLOCKS = BYTES / 1024;      // 1 KiB = one wavefront's 64 x 16-byte load
+    static_assert(BYTES % 1024 == 0, "an image is moved in 1 KiB blocks");
+};
+
+// One workgroup per (chunk, element): the chunk's power of two, then the image through LDS.
+template <int D>
+__global__ __launch_bounds__(RE_T) void rff_presplit_kernel(const float* __restrict__ W, int F, _Float16* __restrict__ images,
+                                                            int* __restrict__ exponents) {
+    using Img = RffImage<D>;
+    constexpr int NP = D / 64;                // pairs of adjacent k rows staged per thread
+    __shared__ __attribute__((aligned(16))) _Float16 img[Img::HALVES];
+    __shared__ float swmax[RE_T / 64];
+    const int chunk = blockIdx.x, type = blockIdx.y, nchunks = gridDim.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float* Wt = W + (size_t)type * D * F;
+    const int f0 = chunk * RE_FC;
+    // thread -> features sf .. sf+3 of the rows k0 = 2 (tid / 8) + 64 p and k0 + 1
+    const int sf = (tid & 7) * 4, skp = 2 * (tid >> 3);
+    // place of features sf .. sf+3 in a row of the k-major copy: f = 16 t + 8 c + 4 h' + e -> 16 t + 8 h' + 4 c + e
+    const int pos2 = (sf & 16) | ((sf & 4) << 1) | ((sf & 8) >> 1);
+    float4 stage[NP][2];
+    float m = 0.0f;
+#pragma unroll
+    for (int p = 0; p < NP; ++p)
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            stage[p][r] = *reinterpret_cast<const float4*>(Wt + (size_t)(skp + 64 * p + r) * F + f0 + sf);
+            m = fmaxf(fmaxf(fmaxf(m, fabsf(stage[p][r].x)), fmaxf(fabsf(stage[p][r].y), fabsf(stage[p][r].z))),
+                      fabsf(stage[p][r].w));
+        }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    if (lane == 0) swmax[wave] = m;
+    for (int t = tid; t < Img::HALVES / 2; t += RE_T) reinterpret_cast<unsigned*>(img)[t] = 0u;    // row padding
+    __syncthreads();
+    const int kw = scale_exponent(fmaxf(fmaxf(swmax[0], swmax[1]), fmaxf(swmax[2], swmax[3])));
+    const float sw = pow2i(kw);
+    if (tid == 0) exponents[type * nchunks + chunk] = kw;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        const int k0 = skp + 64 * p;
+        const float w0[4] = {stage[p][0].x * sw, stage[p][0].y * sw, stage[p][0].z * sw, stage[p][0].w * sw};
+        const float w1[4] = {stage[p][1].x * sw, stage[p][1].y * sw, stage[p][1].z * sw, stage[p][1].w * sw};
+        half4_t r0h, r0l, r1h, r1l;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            _Float16 a, c;
+            split_f16(w0[e], a, c);
+            r0h[e] = a; r0l[e] = c;
+            split_f16(w1[e], a, c);
+            r1h[e] = a; r1l[e] = c;
+            *reinterpret_cast<half2_t*>(&img[Img::W1H + (sf + e) * Img::LD1 + k0]) = (half2_t){r0h[e], r1h[e]};
+            *reinterpret_cast<half2_t*>(&img[Img::W1L + (sf + e) * Img::LD1 + k0]) = (half2_t){r0l[e], r1l[e]};
+        }
+        *reinterpret_cast<half4_t*>(&img[Img::W2H + k0 * Img::LD2 + pos2]) = r0h;
+        *reinterpret_cast<half4_t*>(&img[Img::W2L + k0 * Img::LD2 + pos2]) = r0l;
+        *reinterpret_cast<half4_t*>(&img[Img::W2H + (k0 + 1) * Img::LD2 + pos2]) = r1h;
+        *reinterpret_cast<half4_t*>(&img[Img::W2L + (k0 + 1) * Img::LD2 + pos2]) = r1l;
+    }
+    __syncthreads();
+    float4* dst = reinterpret_cast<float4*>(images + (size_t)(type * nchunks + chunk) * Img::HALVES);
+    for (int t = tid; t < Img::BYTES / 16; t += RE_T) dst[t] = reinterpret_cast<const float4*>(img)[t];
+}
+
 template <int D, bool WITH_GRAD>
 __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void rff_energy_sorted_f16_kernel(
     const float* __restrict__ x, const int* __restrict__ type_offsets, const int* __restrict__ sorted_slots,
-    const float* __restrict__ W, const float* __restrict__ b, const float* __restrict__ alpha, int ne, int F,
-    float norm, float* __restrict__ e_slots, float* __restrict__ gx) {
-    constexpr int LD1 = D + 8;                // halves per row of the feature-major copy
-    constexpr int LD2 = RE_FC + 8;            // halves per row of the k-major copy
+    const _Float16* __restrict__ images, const int* __restrict__ exponents, const float* __restrict__ b,
+    const float* __restrict__ alpha, int ne, int F, float norm, float* __restrict__ e_slots, float* __restrict__ gx) {
+    using Img = RffImage<D>;
+    constexpr int LD1 = Img::LD1, LD2 = Img::LD2;
     constexpr int KS = D / 16;                // matrix instructions along k per product term
-    constexpr int NP = D / 64;                // pairs of adjacent k rows staged per thread per chunk
-    __shared__ __attribute__((aligned(16))) _Float16 sW1h[RE_FC * LD1], sW1l[RE_FC * LD1];
-    __shared__ __attribute__((aligned(16))) _Float16 sW2h[D * LD2], sW2l[D * LD2];
-    __shared__ __attribute__((aligned(16))) float sb[RE_FC], sa[RE_FC];
-    __shared__ float swmax[2][RE_T / 64];     // largest |W| of a chunk per wavefront, two chunks in flight
+    // two images, this chunk's and the next one's, as two arrays of their own: the compiler then knows
+    // that the loads into one do not touch what is read from the other and does not wait for them
+    __shared__ __attribute__((aligned(16))) _Float16 simg0[Img::HALVES], simg1[Img::HALVES];
+    __shared__ __attribute__((aligned(16))) float sba[2 * 2 * RE_FC];     // [2][2][RE_FC]: b / 2 pi, alpha norm 2^kp of the two chunks
 
     int type = -1, row0 = 0, rows = 0;
     {
@@ -263,7 +337,6 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
         }
     }
     if (type < 0) return;
-    const float* Wt = W + (size_t)type * D * F;
     const float* bt = b + (size_t)type * F;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -272,6 +345,26 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
     const bool aok = arow < rows;
     const int fsplit = F / (int)gridDim.y;
     const int fbeg = (int)blockIdx.y * fsplit, fend = fbeg + fsplit;
+    const int nchunks = F / RE_FC;
+    // a scalar base and one per-lane offset: the loads then need no per-lane 64-bit addresses
+    const unsigned char* img0 = reinterpret_cast<const unsigned char*>(images) + (size_t)type * nchunks * Img::BYTES;
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    const unsigned lane16 = (unsigned)lane * 16u;
+    const int* kws = exponents + type * nchunks;
+    // chunk `c` of this element into LDS copy `par`: every wavefront moves the 1 KiB blocks wave, wave + 4, ...
+    // (64 lanes x 16 bytes per instruction, written to LDS at block start + 16 lane)
+    auto dma = [&](int c, _Float16* to) {
+        const unsigned char* src = img0 + (size_t)c * Img::BYTES;
+        unsigned char* dst = reinterpret_cast<unsigned char*>(to);
+#pragma unroll
+        for (int u0 = 0; u0 < Img::BLOCKS; u0 += RE_T / 64) {
+            const int u = u0 + wave_s;
+            if (u < Img::BLOCKS)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + u * 1024 + lane16),
+                                                 (__attribute__((address_space(3))) void*)(dst + u * 1024), 16, 0, 0);
+        }
+    };
+    dma(fbeg / RE_FC, simg0);
 
     // x^T as the B operand of the first product: instruction j contracts k = 16 j + 8 h + (0..7)
     half8_t xh[KS], xl[KS];
@@ -315,6 +408,10 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
         sp = pow2i(kp);
         inv_sp = pow2i(-kp);
     }
+    if (tid < RE_FC) {
+        sba[tid] = bt[fbeg + tid] * 0.15915494309189535f;
+        sba[RE_FC + tid] = alpha[fbeg + tid] * norm * sp;
+    }
 
     float16_t gacc[D / 32];
     if constexpr (WITH_GRAD) {
@@ -325,67 +422,26 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
     }
     float energy = 0.0f;
 
-    // staging of a chunk: thread -> features sf .. sf+3 of the rows k0 = 2 (tid / 8) + 64 p and k0 + 1
-    const int sf = (tid & 7) * 4, skp = 2 * (tid >> 3);
-    // place of features sf .. sf+3 in a row of the k-major copy: f = 16 t + 8 c + 4 h' + e -> 16 t + 8 h' + 4 c + e
-    const int pos2 = (sf & 16) | ((sf & 4) << 1) | ((sf & 8) >> 1);
-    float4 stage[NP][2];
-    auto fetch = [&](int f0) {
-#pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            stage[p][0] = *reinterpret_cast<const float4*>(Wt + (size_t)(skp + 64 * p) * F + f0 + sf);
-            stage[p][1] = *reinterpret_cast<const float4*>(Wt + (size_t)(skp + 64 * p + 1) * F + f0 + sf);
-        }
-    };
-    fetch(fbeg);
-    int par = 0;
-    for (int f0 = fbeg; f0 < fend; f0 += RE_FC, par ^= 1) {
-        // the chunk's own power of two for W (largest |W| of its D x 32 entries to 2^13): the part of a
-        // small W below fp16's smallest normal number would otherwise lose its low bits.  Every
-        // wavefront leaves the largest entry of what it staged, all read the four values after the
-        // barrier; the copy of the chunk before is no longer read by then.
-        {
-            float m = 0.0f;
-#pragma unroll
-            for (int p = 0; p < NP; ++p)
-#pragma unroll
-                for (int r = 0; r < 2; ++r)
-                    m = fmaxf(fmaxf(fmaxf(m, fabsf(stage[p][r].x)), fmaxf(fabsf(stage[p][r].y), fabsf(stage[p][r].z))),
-                              fabsf(stage[p][r].w));
-#pragma unroll
-            for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
-            if (lane == 0) swmax[par][wave] = m;
-        }
+    // one chunk: `img` holds it, the next one is loaded into `other`
+    auto round = [&](int f0, int par, const _Float16* img, _Float16* other) {
+        const bool more = f0 + RE_FC < fend;
+        // this chunk's image has landed (every wavefront waits for its own loads, then for the others),
+        // and the other copy, read in the round before, is free
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        const int kw = scale_exponent(fmaxf(fmaxf(swmax[par][0], swmax[par][1]), fmaxf(swmax[par][2], swmax[par][3])));
-        const float sw = pow2i(kw), inv_sw = pow2i(-kw);
-#pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            const int k0 = skp + 64 * p;
-            const float w0[4] = {stage[p][0].x * sw, stage[p][0].y * sw, stage[p][0].z * sw, stage[p][0].w * sw};
-            const float w1[4] = {stage[p][1].x * sw, stage[p][1].y * sw, stage[p][1].z * sw, stage[p][1].w * sw};
-            half4_t r0h, r0l, r1h, r1l;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                _Float16 a, c;
-                split_f16(w0[e], a, c);
-                r0h[e] = a; r0l[e] = c;
-                split_f16(w1[e], a, c);
-                r1h[e] = a; r1l[e] = c;
-                *reinterpret_cast<half2_t*>(&sW1h[(sf + e) * LD1 + k0]) = (half2_t){r0h[e], r1h[e]};
-                *reinterpret_cast<half2_t*>(&sW1l[(sf + e) * LD1 + k0]) = (half2_t){r0l[e], r1l[e]};
-            }
-            *reinterpret_cast<half4_t*>(&sW2h[k0 * LD2 + pos2]) = r0h;
-            *reinterpret_cast<half4_t*>(&sW2l[k0 * LD2 + pos2]) = r0l;
-            *reinterpret_cast<half4_t*>(&sW2h[(k0 + 1) * LD2 + pos2]) = r1h;
-            *reinterpret_cast<half4_t*>(&sW2l[(k0 + 1) * LD2 + pos2]) = r1l;
+        // b and alpha of the next chunk are requested before its image so that waiting for them does
+        // not wait for the image; they go to LDS at the end of the round
+        float bnext = 0.0f, anext = 0.0f;
+        if (more && tid < RE_FC) {
+            bnext = bt[f0 + RE_FC + tid];
+            anext = alpha[f0 + RE_FC + tid];
         }
-        if (tid < RE_FC) {
-            sb[tid] = bt[f0 + tid];
-            sa[tid] = alpha[f0 + tid] * norm * sp;
-        }
-        __syncthreads();
-        if (f0 + RE_FC < fend) fetch(f0 + RE_FC);
+        if (more) dma(f0 / RE_FC + 1, other);
+        const _Float16 *sW1h = img + Img::W1H, *sW1l = img + Img::W1L, *sW2h = img + Img::W2H, *sW2l = img + Img::W2L;
+        const float* sb = sba + par * 2 * RE_FC;
+        const float* sa = sb + RE_FC;
+        const int kw = kws[f0 / RE_FC];
+        const float inv_sw = pow2i(-kw);
 
         // first product: 2^(kx + kw) S^T (32 features x 32 atoms)
         const float inv_sxw = inv_sx * inv_sw;
@@ -400,22 +456,38 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
             sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, xl[j], sacc, 0, 0, 0);
             sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, xh[j], sacc, 0, 0, 0);
         }
-        // accumulator register r: feature 8(r/4) + 4h + r%4 of the chunk, atom = lane%32
+        // accumulator register r: feature 8(r/4) + 4h + r%4 of the chunk, atom = lane%32.  The sine
+        // argument is formed in REVOLUTIONS (b arrives divided by 2 pi, the product takes 1 / 2 pi with its
+        // inverse scales): v_sin_f32 / v_cos_f32 reduce the range themselves up to 256 revolutions; the
+        // rounding of the argument, |arg| 6e-8 radians, is that of an fp32 argument in radians.  Beyond
+        // 1500 radians whole revolutions are taken off first (u - rint(u) is exact in fp32).
+        constexpr float UMAX = 1500.0f * 0.15915494309189535f;
+        const float crev = inv_sxw * 0.15915494309189535f;
+        float umax = 0.0f;
+        float aq[16];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int fl = 8 * q + 4 * h;
             const float4 bv = *reinterpret_cast<const float4*>(&sb[fl]);
             const float4 av = *reinterpret_cast<const float4*>(&sa[fl]);
-            const float bq[4] = {bv.x, bv.y, bv.z, bv.w}, aq[4] = {av.x, av.y, av.z, av.w};
+            const float bq[4] = {bv.x, bv.y, bv.z, bv.w};
+            aq[4 * q] = av.x; aq[4 * q + 1] = av.y; aq[4 * q + 2] = av.z; aq[4 * q + 3] = av.w;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                float sn, cs;
-                const float arg = fmaf(sacc[4 * q + e], inv_sxw, bq[e]);
-                sincos_hw(arg, &sn, &cs);
-                if (__builtin_expect(fabsf(arg) > 32000.0f, 0)) sincos_large(arg, &sn, &cs);
-                energy = fmaf(aq[e], cs, energy);
-                sacc[4 * q + e] = -aq[e] * sn;           // 2^kp P
+                sacc[4 * q + e] = fmaf(sacc[4 * q + e], crev, bq[e]);
+                umax = fmaxf(umax, fabsf(sacc[4 * q + e]));
             }
+        }
+        if (__builtin_expect(__any(umax > UMAX), 0)) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (fabsf(sacc[r]) > UMAX) sacc[r] -= rintf(sacc[r]);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float sn = __builtin_amdgcn_sinf(sacc[r]), cs = __builtin_amdgcn_cosf(sacc[r]);
+            energy = fmaf(aq[r], cs, energy);
+            sacc[r] = -aq[r] * sn;                       // 2^kp P
         }
         if constexpr (WITH_GRAD) {
             // second product: 2^kp GX^T[k, a] += 2^-kw sum_f 2^kw W[k, f] 2^kp P[f, a]; instruction t contracts the
@@ -450,6 +522,15 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
                 for (int r = 0; r < 16; ++r) gacc[blk][r] = fmaf(part[r], inv_sw, gacc[blk][r]);
             }
         }
+        if (more && tid < RE_FC) {
+            float* nb = sba + (par ^ 1) * 2 * RE_FC;
+            nb[tid] = bnext * 0.15915494309189535f;
+            nb[RE_FC + tid] = anext * norm * sp;
+        }
+    };
+    for (int f0 = fbeg; f0 < fend; f0 += 2 * RE_FC) {
+        round(f0, 0, simg0, simg1);
+        if (f0 + RE_FC < fend) round(f0 + RE_FC, 1, simg1, simg0);
     }
 
     energy = (energy + __shfl_xor(energy, 32, 64)) * inv_sp;
@@ -551,7 +632,38 @@ extern "C" int qmll_rff_derivative_features(const float* x, const float* grad, c
     return QMLL_OK;
 }
 
-extern "C" int qmll_rff_energy_sorted(const float* x, const int* type_offsets, const int* sorted_slots, const float* W,
+// bytes of the pre-split form of W [ne, d, F]: the images, then one exponent per image
+static size_t rff_image_bytes(int d) { return d == 64 ? (size_t)RffImage<64>::BYTES : (size_t)RffImage<128>::BYTES; }
+
+extern "C" size_t qmll_rff_presplit_bytes(int ne, int d, int F) {
+    if (ne <= 0 || F <= 0 || F % RE_FC != 0 || (d != 64 && d != 128)) return 0;
+    const size_t n = (size_t)ne * (F / RE_FC);
+    return n * rff_image_bytes(d) + n * sizeof(int);
+}
+
+extern "C" int qmll_rff_presplit(const float* W, int ne, int d, int F, void* out, size_t out_bytes, qmll_stream_t stream) {
+    QMLL_REQUIRE(ne > 0 && F > 0, QMLL_ERR_INVALID, "qmll_rff_presplit: bad size ne=%d F=%d", ne, F);
+    QMLL_REQUIRE(d == 64 || d == 128, QMLL_ERR_INVALID, "qmll_rff_presplit: d=%d is not 64 or 128", d);
+    QMLL_REQUIRE(F % RE_FC == 0, QMLL_ERR_INVALID, "qmll_rff_presplit: F=%d is not a multiple of %d", F, RE_FC);
+    QMLL_REQUIRE(W && out, QMLL_ERR_INVALID, "qmll_rff_presplit: null pointer");
+    QMLL_REQUIRE(out_bytes >= qmll_rff_presplit_bytes(ne, d, F), QMLL_ERR_INVALID,
+                 "qmll_rff_presplit: output of %zu bytes, %zu are needed", out_bytes, qmll_rff_presplit_bytes(ne, d, F));
+    QMLL_REQUIRE((((uintptr_t)W | (uintptr_t)out) & 15) == 0, QMLL_ERR_INVALID,
+                 "qmll_rff_presplit: W and the output must be 16-byte aligned");
+    const int nchunks = F / RE_FC;
+    QMLL_REQUIRE(ne <= 65535, QMLL_ERR_INVALID, "qmll_rff_presplit: ne=%d too large", ne);
+    _Float16* images = (_Float16*)out;
+    int* exponents = (int*)((char*)out + (size_t)ne * nchunks * rff_image_bytes(d));
+    const dim3 grid(nchunks, ne);
+    if (d == 64)
+        hipLaunchKernelGGL(rff_presplit_kernel<64>, grid, dim3(RE_T), 0, (hipStream_t)stream, W, F, images, exponents);
+    else
+        hipLaunchKernelGGL(rff_presplit_kernel<128>, grid, dim3(RE_T), 0, (hipStream_t)stream, W, F, images, exponents);
+    QMLL_CHECK_LAUNCH("qmll_rff_presplit");
+    return QMLL_OK;
+}
+
+extern "C" int qmll_rff_energy_sorted(const float* x, const int* type_offsets, const int* sorted_slots, const void* W_split,
                                       const float* b, const float* alpha, int A, int ne, int d, int F, float* e_slots,
                                       float* gx, qmll_stream_t stream) {
     QMLL_REQUIRE(A >= 0 && ne > 0 && d > 0 && F > 0, QMLL_ERR_INVALID, "qmll_rff_energy_sorted: bad size A=%d ne=%d d=%d F=%d",
@@ -559,10 +671,12 @@ extern "C" int qmll_rff_energy_sorted(const float* x, const int* type_offsets, c
     QMLL_REQUIRE(d == 64 || d == 128, QMLL_ERR_INVALID, "qmll_rff_energy_sorted: d=%d is not 64 or 128", d);
     QMLL_REQUIRE(F % RE_FC == 0, QMLL_ERR_INVALID, "qmll_rff_energy_sorted: F=%d is not a multiple of %d", F, RE_FC);
     if (A == 0) return QMLL_OK;
-    QMLL_REQUIRE(x && type_offsets && sorted_slots && W && b && alpha && e_slots, QMLL_ERR_INVALID,
+    QMLL_REQUIRE(x && type_offsets && sorted_slots && W_split && b && alpha && e_slots, QMLL_ERR_INVALID,
                  "qmll_rff_energy_sorted: null pointer");
-    QMLL_REQUIRE((((uintptr_t)x | (uintptr_t)W | (uintptr_t)gx) & 15) == 0, QMLL_ERR_INVALID,
-                 "qmll_rff_energy_sorted: x, W and gx must be 16-byte aligned");
+    QMLL_REQUIRE((((uintptr_t)x | (uintptr_t)W_split | (uintptr_t)gx) & 15) == 0, QMLL_ERR_INVALID,
+                 "qmll_rff_energy_sorted: x, W_split and gx must be 16-byte aligned");
+    const _Float16* images = (const _Float16*)W_split;
+    const int* exponents = (const int*)((const char*)W_split + (size_t)ne * (F / RE_FC) * rff_image_bytes(d));
     const float norm = sqrtf(2.0f / (float)F);
     hipStream_t st = (hipStream_t)stream;
     // Two workgroups fit a CU (two wavefronts per SIMD) and all run the same chunk loop, so the launch takes ceil(workgroups / 512) rounds of 1/fs of a tile's work
@@ -584,14 +698,14 @@ extern "C" int qmll_rff_energy_sorted(const float* x, const int* type_offsets, c
 #define CALL(DD)                                                                                                     \
     if (gx)                                                                                                          \
         hipLaunchKernelGGL((rff_energy_sorted_f16_kernel<DD, true>), grid, dim3(RE_T), 0, st, x, type_offsets,         \
-                           sorted_slots, W, b, alpha, ne, F, norm, e_slots, gx);                                      \
+                           sorted_slots, images, exponents, b, alpha, ne, F, norm, e_slots, gx);                      \
     else                                                                                                             \
         hipLaunchKernelGGL((rff_energy_sorted_f16_kernel<DD, false>), grid, dim3(RE_T), 0, st, x, type_offsets,        \
-                           sorted_slots, W, b, alpha, ne, F, norm, e_slots, gx)
+                           sorted_slots, images, exponents, b, alpha, ne, F, norm, e_slots, gx);
     if (d == 64) {
-        CALL(64);
+        CALL(64)
     } else {
-        CALL(128);
+        CALL(128)
     }
 #undef CALL
     QMLL_CHECK_LAUNCH("qmll_rff_energy_sorted");

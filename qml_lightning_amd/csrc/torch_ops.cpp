@@ -17,6 +17,9 @@
 #include <torch/autograd.h>
 #include <torch/library.h>
 
+#include <functional>
+#include <map>
+#include <mutex>
 #include <tuple>
 #include <vector>
 
@@ -48,6 +51,39 @@ const float* fp(const Tensor& t) { return t.defined() && t.numel() ? t.data_ptr<
 const int* ip(const Tensor& t) { return t.defined() && t.numel() ? t.data_ptr<int>() : nullptr; }
 
 float scalar(const Tensor& t) { return t.item<float>(); }
+
+// Model constants that a kernel wants in a prepared form (fp32 operands split into fp16 parts): prepared
+// once per tensor and kept until the tensor dies, is written to in place or changes its storage.
+struct Prepared {
+    c10::weak_intrusive_ptr<c10::TensorImpl> owner;
+    int64_t version;
+    const void* data;
+    Tensor buffer;
+};
+std::mutex prepared_mutex;
+std::map<std::pair<const c10::TensorImpl*, int>, Prepared> prepared;
+
+int64_t version_of(const Tensor& t) { return t.is_inference() ? -1 : (int64_t)t._version(); }
+
+Tensor prepared_form(const Tensor& t, int kind, const std::function<Tensor(const Tensor&)>& make) {
+    std::lock_guard<std::mutex> lock(prepared_mutex);
+    const auto key = std::make_pair((const c10::TensorImpl*)t.unsafeGetTensorImpl(), kind);
+    auto it = prepared.find(key);
+    if (it != prepared.end()) {
+        auto alive = it->second.owner.lock();
+        if (alive && alive.get() == t.unsafeGetTensorImpl() && it->second.version == version_of(t) &&
+            it->second.data == t.const_data_ptr())
+            return it->second.buffer;
+        prepared.erase(it);
+    }
+    if (prepared.size() >= 64) {      // forget tensors that are gone
+        for (auto e = prepared.begin(); e != prepared.end();) e = e->second.owner.expired() ? prepared.erase(e) : std::next(e);
+    }
+    Tensor buffer = make(t);
+    prepared.emplace(key, Prepared{c10::weak_intrusive_ptr<c10::TensorImpl>(t.getIntrusivePtr()), version_of(t),
+                                   t.const_data_ptr(), buffer});
+    return buffer;
+}
 
 // ---- FCHL19 -----------------------------------------------------------------------------
 struct FchlInputs {
@@ -535,9 +571,17 @@ std::tuple<Tensor, Tensor> rff_energy_sorted_impl(const Tensor& x_, const Tensor
     TORCH_CHECK(x.size(0) == A && x.size(1) == d && off.size(0) == ne + 1 && bb.size(0) == ne && bb.size(1) == F,
                 "rff_energy_sorted: x, W and b do not fit together");
     TORCH_CHECK(al.numel() == F, "rff_energy_sorted: alpha has ", al.numel(), " entries for ", F, " features");
+    Tensor Wsplit = prepared_form(WW, 0, [&](const Tensor& w) {
+        const size_t nbytes = qmll_rff_presplit_bytes(ne, d, F);
+        TORCH_CHECK(nbytes > 0, "rff_energy_sorted: the fused kernel exists for 64 or 128 components and a multiple of 32 "
+                    "features, not ", d, " and ", F);
+        Tensor out = at::empty({(int64_t)nbytes}, w.options().dtype(at::kByte));
+        check(qmll_rff_presplit(fp(w), ne, d, F, out.data_ptr(), nbytes, stream()), "qmll_rff_presplit");
+        return out;
+    });
     Tensor e = e_zeroed.defined() ? e_zeroed : at::zeros({nslots}, x.options());
     Tensor gx = with_grad ? at::empty({A, d}, x.options()) : empty_like_none(x);
-    check(qmll_rff_energy_sorted(fp(x), ip(off), ip(ss), fp(WW), fp(bb), fp(al), A, ne, d, F,
+    check(qmll_rff_energy_sorted(fp(x), ip(off), ip(ss), Wsplit.const_data_ptr(), fp(bb), fp(al), A, ne, d, F,
                                  nslots ? e.data_ptr<float>() : nullptr, with_grad && A ? gx.data_ptr<float>() : nullptr,
                                  stream()),
           "qmll_rff_energy_sorted");

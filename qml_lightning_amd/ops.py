@@ -14,6 +14,7 @@ there is no CPU implementation.
 import ctypes
 import math
 import os
+import weakref
 
 import torch
 
@@ -531,9 +532,46 @@ def rff_derivative_features(x, grad, W, b, mol_index, G, molecule_major=False):
     return G
 
 
+_PRESPLIT = {}    # (id(tensor), kind) -> (weak reference, version, address, prepared buffer)
+
+
+def _version(t):
+    try:
+        return t._version
+    except RuntimeError:      # inference tensors keep no version counter
+        return -1
+
+
+def presplit_cached(t, kind, make):
+    """The prepared (pre-split) form of a model constant `t`, made once by `make(t)` and reused until
+    the tensor object dies, is written to in place (its version counter moves) or changes its storage."""
+    key = (id(t), kind)
+    hit = _PRESPLIT.get(key)
+    if hit is not None and hit[0]() is t and hit[1] == _version(t) and hit[2] == t.data_ptr():
+        return hit[3]
+    buf = make(t)
+    _PRESPLIT[key] = (weakref.ref(t, lambda _r, k=key: _PRESPLIT.pop(k, None)), _version(t), t.data_ptr(), buf)
+    return buf
+
+
+def rff_presplit(W):
+    """W f32 [ne,d,F] in the form the fused RFF predict kernel multiplies with (qmll_rff_presplit):
+    an opaque uint8 device buffer."""
+    W = _f32(W)
+    ne, d, F = W.shape
+    nbytes = int(_lib.lib().qmll_rff_presplit_bytes(ne, d, F))
+    if nbytes == 0:
+        raise RuntimeError("rff_presplit: the fused kernel exists for d = 64 or 128 and a multiple of 32 features, "
+                           "not d = %d, F = %d" % (d, F))
+    out = torch.empty(nbytes, dtype=torch.uint8, device=W.device)
+    check(_lib.lib().qmll_rff_presplit(_ptr(W), ne, d, F, _ptr(out), nbytes, _stream()), "qmll_rff_presplit")
+    return out
+
+
 def rff_energy_sorted(x, type_offsets, sorted_slots, W, b, alpha, nslots, with_grad=True):
     """Fused RFF energy (and gradient) on element-sorted rows x [A,d]; W [ne,d,F], b [ne,F],
-    alpha [F] fp32 -> (e_slots [nslots], gx [A,d] or None)."""
+    alpha [F] fp32 -> (e_slots [nslots], gx [A,d] or None).  W is split for the kernel on its first
+    use and the split form kept until W changes."""
     x, W, b, alpha = _f32(x), _f32(W), _f32(b), _f32(alpha)
     type_offsets, sorted_slots = _i32(type_offsets), _i32(sorted_slots)
     ne, d, F = W.shape
@@ -543,9 +581,10 @@ def rff_energy_sorted(x, type_offsets, sorted_slots, W, b, alpha, nslots, with_g
                            % (tuple(x.shape), tuple(W.shape), tuple(b.shape)))
     if alpha.numel() != F:
         raise RuntimeError("rff_energy_sorted: alpha has %d entries for %d features" % (alpha.numel(), F))
+    Wsplit = presplit_cached(W, "rff", rff_presplit)
     e_slots = torch.zeros(int(nslots), dtype=torch.float32, device=x.device)
     gx = torch.empty((A, d), dtype=torch.float32, device=x.device) if with_grad else None
-    check(_lib.lib().qmll_rff_energy_sorted(_ptr(x), _ptr(type_offsets), _ptr(sorted_slots), _ptr(W), _ptr(b),
+    check(_lib.lib().qmll_rff_energy_sorted(_ptr(x), _ptr(type_offsets), _ptr(sorted_slots), _ptr(Wsplit), _ptr(b),
                                             _ptr(alpha), A, ne, d, F, _ptr(e_slots), _ptr(gx), _stream()),
           "qmll_rff_energy_sorted")
     return e_slots, gx
