@@ -267,10 +267,29 @@ int qmll_sort_atoms_by_type(const int* types, const int* atomIDs, const int* mol
 int qmll_sort_by_type_noalloc(const int* types, const int* slots, int A, int ne, int* sorted_slots,
                               int* type_offsets, qmll_stream_t stream);
 
+/* The projection matrices ("reductors", f32 [ne,R,d], qml_lightning/models/kernel.py:28) are constants
+ * of a model.  For large batches the two projections below multiply on the fp16 matrix cores with
+ * every fp32 operand as two fp16 parts behind power-of-two scales (fp32 accumulation): the
+ * reductors are prepared for that ONCE, here, in the layouts the kernels keep in LDS (forward: per
+ * element, 32-row chunk and 128-column block; transposed: per element and 32 rows of U), so that
+ * no workgroup repeats the split.  qmll_reductor_presplit_bytes: size of the prepared form (0 when
+ * no kernel would use one: R must be a multiple of 4, d 64 or a multiple of 128).  The caller owns
+ * the buffer (16-byte aligned) and refreshes it when the reductors change. */
+size_t qmll_reductor_presplit_bytes(int ne, int R, int d);
+int qmll_reductor_presplit(const float* reductors, int ne, int R, int d, void* reductors_split, size_t reductors_split_bytes,
+                           qmll_stream_t stream);
+
 /* x f32 [A,d]: row a = rep[sorted_slots[a], :] . reductors[type of a]  (rep f32 [N,R],
- * reductors f32 [ne,R,d]); rows at and beyond type_offsets[ne] are not written. */
+ * reductors f32 [ne,R,d]); rows at and beyond type_offsets[ne] are not written.
+ * reductors_split: the prepared form from qmll_reductor_presplit, or NULL.  With it, batches from
+ * about 65 000 atoms on (at d = 128) take the fp16 matrix-core kernel, whose results differ from the
+ * fp32 kernels' in the last bits (1.7e-7 of the row's largest entry against fp64; fp32 matrix
+ * instructions: 7.9e-7) and where a row's rounding depends on the largest entry among the 32 rows
+ * that share its wavefront: a molecule's projection can change in the last bit with the batch it
+ * is in.  Non-finite entries of rep give non-finite (not necessarily equal) results there.
+ * Without it every batch takes the fp32 kernels. */
 int qmll_project_typed(const float* rep, const int* sorted_slots, const int* type_offsets, const float* reductors,
-                       int A, int ne, int R, int d, float* x, qmll_stream_t stream);
+                       const void* reductors_split, int A, int ne, int R, int d, float* x, qmll_stream_t stream);
 
 /* The same product for `group` rows per atom: rows f32 [N*group, R] holds rows
  * slot*group ... slot*group + group - 1 for every slot, x f32 [A*group, d] receives
@@ -287,10 +306,12 @@ int qmll_project_typed_rows(const float* rows, const int* sorted_slots, const in
 /* Transpose of qmll_project_typed: g_rep[sorted_slots[a], :] = gx[a, :] . reductors[type]^T
  * (g_rep f32 [N,R]).  Rows of slots that are not in the sorted list are not written, except
  * that with types != NULL (i32 [N]) the rows of slots whose type is outside [0,ne) are set
- * to zero. */
+ * to zero.  reductors_split as for qmll_project_typed (NULL = fp32 kernels only); the fp16
+ * matrix-core kernel (d = 64 or 128, batches beyond the small-batch kernels) scales the 32 gradient
+ * rows of a wavefront by one power of two and every row of U by its own. */
 int qmll_project_typed_backward(const float* gx, const int* sorted_slots, const int* type_offsets,
-                                const float* reductors, const int* types, int A, int N, int ne, int R, int d,
-                                float* g_rep, qmll_stream_t stream);
+                                const float* reductors, const void* reductors_split, const int* types, int A, int N,
+                                int ne, int R, int d, float* g_rep, qmll_stream_t stream);
 
 /* qmll_sorf_energy_typed on compact element-sorted rows: x f32 [A,d] as written by
  * qmll_project_typed, D f32 [ne,T,S,d], bias f32 [ne,S*d], alpha f32 [S*d].

@@ -57,9 +57,11 @@ PROTOTYPES = {
     "qmll_sort_atoms_workspace": [c_int, c_int],
     "qmll_sort_atoms_by_type": [P, P, P, c_int, c_int, c_int, P, c_size_t, P, P, P],
     "qmll_sort_by_type_noalloc": [P, P, c_int, c_int, P, P, P],
-    "qmll_project_typed": [P, P, P, P, c_int, c_int, c_int, c_int, P, P],
+    "qmll_reductor_presplit_bytes": [c_int, c_int, c_int],
+    "qmll_reductor_presplit": [P, c_int, c_int, c_int, P, c_size_t, P],
+    "qmll_project_typed": [P, P, P, P, P, c_int, c_int, c_int, c_int, P, P],
     "qmll_project_typed_rows": [P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
-    "qmll_project_typed_backward": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
+    "qmll_project_typed_backward": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
     "qmll_sorf_energy_sorted": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_float, P, P, P],
     "qmll_rff_features": [P, P, P, P, c_int, c_int, c_int, c_int, P, P],
     "qmll_rff_derivative_features": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
@@ -82,7 +84,7 @@ PROTOTYPES = {
     "qmll_probe_rate": [c_int, c_int, c_int, P, P],
     "qmll_probe_mix": [c_int, c_int, c_int, P, P],
 }
-_RESTYPES = {"qmll_last_error": c_char_p, "qmll_rff_presplit_bytes": c_size_t, "qmll_sort_by_type_workspace": c_size_t, "qmll_sort_atoms_workspace": c_size_t,
+_RESTYPES = {"qmll_last_error": c_char_p, "qmll_rff_presplit_bytes": c_size_t, "qmll_reductor_presplit_bytes": c_size_t, "qmll_sort_by_type_workspace": c_size_t, "qmll_sort_atoms_workspace": c_size_t,
              "qmll_cholesky_workspace_bytes": c_size_t, "qmll_gram_workspace_bytes": c_size_t,
              "qmll_probe_out_bytes": c_size_t, "qmll_probe_rate": c_double,
              "qmll_probe_mix": c_double}

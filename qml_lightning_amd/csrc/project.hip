@@ -333,61 +333,205 @@ __global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(PNT > 64 ? 3
     }
 }
 
-// The forward product on the half-precision matrix cores, 128 x 128 tiles (A [rows, K] gathered through
-// a_rows, B_type [K, N] row-major, K and N multiples of 4, 16-byte aligned bases).  Per chunk of 32 k the
-// tile of A and the tile of B are split into two fp16 parts each on their way into LDS (both k-contiguous:
-// B is transposed as it is staged), three v_mfma_f32_32x32x16_f16 per product term.  The chunk of A and
-// the chunk of B each take their own power of two (every wavefront leaves the largest entries of what it
-// is about to stage, all read the four pairs after the barrier the loop has anyway), so a chunk's product
-// is summed from zero and added to the running sums by the vector unit with the inverse factor (which
-// also keeps the low bits of a small chunk beside a large sum).
-__global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(2, 3))) void typed_gemm_f16_kernel(
-    const float* __restrict__ A, int lda, const int* __restrict__ a_rows, const float* __restrict__ Bm,
-    size_t b_type_stride, int ldb, float* __restrict__ C, int ldc, const int* __restrict__ offsets, int ne, int K, int N,
+// ---- projections on the half-precision matrix cores -------------------------------------------
+// v_mfma_f32_32x32x16_f16 does eight times the flops of the fp32 instruction in 40 clocks against 64,
+// so both operands are taken as two fp16 parts (hi = the value rounded to fp16, lo = the rounded
+// rest: 22 bits together) behind exact power-of-two scales, and a product term is three matrix
+// instructions, hi.hi + hi.lo + lo.hi, accumulated in fp32.
+//
+// The reductors are constants of the model: they are split ONCE (reductor_presplit_*_kernel) into the
+// very bytes the two kernels keep in LDS, "images" that the kernels move with direct global-to-LDS
+// loads (no registers, no vector instructions), the next one while the current one is multiplied:
+//   forward  image (element, 32-k chunk c, 128-column block): columns x k, k contiguous, hi then lo
+//            parts, the chunk behind one power of two (its exponent in a table beside the images);
+//   backward image (element, block of 32 rows of U = 32 columns of the product): rows x k, hi then lo,
+//            every row behind its own power of two, the 32 inverse factors at the image's end.
+// The rows that change from call to call (representation rows forward, gradient rows backward) are
+// read from HBM straight into the register layout of the matrix instruction's A operand (lane (i, h)
+// holds row i, eight consecutive k), scaled by the power of two of the wavefront's 32 rows and split in
+// registers: they never pass through LDS, and no barrier waits on them.
+constexpr int FWD_LDH = PK + 8;                       // halves per column of a forward image
+constexpr int FWD_IMG_HALVES = 2 * 128 * FWD_LDH;     // hi and lo
+constexpr int FWD_IMG_BYTES = FWD_IMG_HALVES * 2;     // 20480
+static_assert(FWD_IMG_BYTES % 1024 == 0, "an image is moved in 1 KiB blocks");
+template <int K>
+struct BwdImage {
+    static constexpr int LDB = K + 8;                 // halves per row
+    static constexpr int HALVES = 2 * 32 * LDB;       // hi and lo
+    static constexpr int SINV = HALVES * 2;           // byte offset of the 32 inverse factors
+    static constexpr int BYTES = (SINV + 32 * 4 + 1023) / 1024 * 1024;    // 18432 (K = 128), 10240 (K = 64)
+};
+
+// one wavefront's share of a 1 KiB-blocked image: blocks wave, wave + 4, ... (64 lanes x 16 bytes each)
+template <int BYTES>
+__device__ __forceinline__ void image_to_lds(const unsigned char* __restrict__ src, void* dst, int wave_s, unsigned lane16) {
+#pragma unroll
+    for (int u0 = 0; u0 < BYTES / 1024; u0 += PT / 64) {
+        const int u = u0 + wave_s;
+        if (u < BYTES / 1024)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + u * 1024 + lane16),
+                                             (__attribute__((address_space(3))) void*)((unsigned char*)dst + u * 1024), 16, 0,
+                                             0);
+    }
+}
+
+// forward images: workgroup = (chunk, column block, element)
+__global__ __launch_bounds__(PT) void reductor_presplit_fwd_kernel(const float* __restrict__ U, int R, int d, int ncb,
+                                                                    _Float16* __restrict__ images, int* __restrict__ exponents) {
+    __shared__ __attribute__((aligned(16))) _Float16 img[FWD_IMG_HALVES];
+    __shared__ float smax[PT / 64];
+    const int c = blockIdx.x / ncb, cb = blockIdx.x % ncb, type = blockIdx.y, nchunks = gridDim.x / ncb;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float* Ut = U + (size_t)type * R * d;
+    // thread -> columns (tid/8)*4 .. +3, rows k = 2 (tid%8) + 16 u and the next one
+    const int bn = (tid >> 3) * 4, bkp = 2 * (tid & 7);
+    float4 rb[2][2];
+    float m = 0.0f;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int k = c * PK + bkp + 16 * u + e;
+            rb[u][e] = k < R ? *reinterpret_cast<const float4*>(Ut + (size_t)k * d + cb * 128 + bn) : make_float4(0.f, 0.f, 0.f, 0.f);
+            m = fmaxf(fmaxf(fmaxf(m, fabsf(rb[u][e].x)), fmaxf(fabsf(rb[u][e].y), fabsf(rb[u][e].z))), fabsf(rb[u][e].w));
+        }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    if (lane == 0) smax[wave] = m;
+    for (int t = tid; t < FWD_IMG_HALVES / 2; t += PT) reinterpret_cast<unsigned*>(img)[t] = 0u;     // column padding
+    __syncthreads();
+    const int kb = scale_exponent(fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3])));
+    const float sb = pow2i(kb);
+    const int index = (type * nchunks + c) * ncb + cb;
+    if (tid == 0) exponents[index] = kb;
+    const float bv[2][2][4] = {{{rb[0][0].x, rb[0][0].y, rb[0][0].z, rb[0][0].w}, {rb[0][1].x, rb[0][1].y, rb[0][1].z, rb[0][1].w}},
+                               {{rb[1][0].x, rb[1][0].y, rb[1][0].z, rb[1][0].w}, {rb[1][1].x, rb[1][1].y, rb[1][1].z, rb[1][1].w}}};
+#pragma unroll
+    for (int cc = 0; cc < 4; ++cc)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            _Float16 h0, l0, h1, l1;
+            split_f16(bv[u][0][cc] * sb, h0, l0);
+            split_f16(bv[u][1][cc] * sb, h1, l1);
+            *reinterpret_cast<half2_t*>(&img[(bn + cc) * FWD_LDH + bkp + 16 * u]) = (half2_t){h0, h1};
+            *reinterpret_cast<half2_t*>(&img[128 * FWD_LDH + (bn + cc) * FWD_LDH + bkp + 16 * u]) = (half2_t){l0, l1};
+        }
+    __syncthreads();
+    float4* dst = reinterpret_cast<float4*>(images + (size_t)index * FWD_IMG_HALVES);
+    for (int t = tid; t < FWD_IMG_BYTES / 16; t += PT) dst[t] = reinterpret_cast<const float4*>(img)[t];
+}
+
+// backward images: workgroup = (block of 32 rows of U, element)
+template <int K>
+__global__ __launch_bounds__(PT) void reductor_presplit_bwd_kernel(const float* __restrict__ U, int R,
+                                                                    unsigned char* __restrict__ images) {
+    using Img = BwdImage<K>;
+    constexpr int NV = K / 32;
+    __shared__ __attribute__((aligned(16))) unsigned char img[Img::BYTES];
+    const int b = blockIdx.x, type = blockIdx.y, nblk = gridDim.x;
+    const int tid = threadIdx.x;
+    const float* Ut = U + (size_t)type * R * K;
+    _Float16* ih = reinterpret_cast<_Float16*>(img);
+    _Float16* il = ih + 32 * Img::LDB;
+    float* sinv = reinterpret_cast<float*>(img + Img::SINV);
+    for (int t = tid; t < Img::BYTES / 4; t += PT) reinterpret_cast<unsigned*>(img)[t] = 0u;
+    __syncthreads();
+    // thread -> row tid/8 of the block, floats (tid%8)*4 + 32 v
+    const int bn = tid >> 3, bk = (tid & 7) * 4;
+    const int n = 32 * b + bn;
+    float4 rb[NV];
+    float m = 0.0f;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        rb[v] = n < R ? *reinterpret_cast<const float4*>(Ut + (size_t)n * K + bk + 32 * v) : make_float4(0.f, 0.f, 0.f, 0.f);
+        m = fmaxf(fmaxf(fmaxf(m, fabsf(rb[v].x)), fmaxf(fabsf(rb[v].y), fabsf(rb[v].z))), fabsf(rb[v].w));
+    }
+    m = fmaxf(m, lane_xor<1>(m));            // the eight lanes of a row are neighbours
+    m = fmaxf(m, lane_xor<2>(m));
+    m = fmaxf(m, lane_xor<4>(m));
+    const int kb = scale_exponent(m);
+    const float sb = pow2i(kb);
+    if ((tid & 7) == 0) sinv[bn] = pow2i(-kb);
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const float w[4] = {rb[v].x * sb, rb[v].y * sb, rb[v].z * sb, rb[v].w * sb};
+        half4_t wh, wl;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            _Float16 a, c;
+            split_f16(w[e], a, c);
+            wh[e] = a;
+            wl[e] = c;
+        }
+        *reinterpret_cast<half4_t*>(&ih[bn * Img::LDB + bk + 32 * v]) = wh;
+        *reinterpret_cast<half4_t*>(&il[bn * Img::LDB + bk + 32 * v]) = wl;
+    }
+    __syncthreads();
+    float4* dst = reinterpret_cast<float4*>(images + (size_t)(type * nblk + b) * Img::BYTES);
+    for (int t = tid; t < Img::BYTES / 16; t += PT) dst[t] = reinterpret_cast<const float4*>(img)[t];
+}
+
+// 2^-(ka + kb) applied to a chunk's product as it is added to the running sums: one factor when it is
+// a float, two multiplies at the ends of the exponent range (operands near the largest or smallest floats)
+__device__ __forceinline__ void add_scaled(float16_t& acc, const float16_t& part, int ka, int kb) {
+    const int ks = ka + kb;
+    if (ks >= -126 && ks <= 126) {
+        const float inv = pow2i(-ks);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = fmaf(part[r], inv, acc[r]);
+    } else {
+        const float ia = pow2i(-ka), ib = pow2i(-kb);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = fmaf(part[r] * ia, ib, acc[r]);
+    }
+}
+
+// Forward product x = rep . U_type, 128 x 128 tiles (A [rows, K] gathered through a_rows; K a multiple
+// of 4, N a multiple of 128, 16-byte aligned bases).  Per chunk of 32 k: the wavefront's 32 rows take
+// the power of two of their largest entry and are split in registers, the chunk of U arrives as its
+// image; a chunk's product is summed from zero and added to the running sums by the vector unit with
+// the inverse factor (which also keeps the low bits of a small chunk beside a large sum).
+__global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(3))) void typed_gemm_f16_kernel(
+    const float* __restrict__ A, int lda, const int* __restrict__ a_rows, const _Float16* __restrict__ images,
+    const int* __restrict__ exponents, float* __restrict__ C, int ldc, const int* __restrict__ offsets, int ne, int K, int N,
     int group) {
-    constexpr int LDH = PK + 8;        // halves per staged row
-    __shared__ __attribute__((aligned(16))) _Float16 sAh[PM * LDH], sAl[PM * LDH], sBh[128 * LDH], sBl[128 * LDH];
-    __shared__ float smax[2][PT / 64][2];     // largest |A|, |B| of a chunk per wavefront, two chunks in flight
+    // the two images as arrays of their own: the compiler then knows that the loads into one do not
+    // touch what is read from the other
+    __shared__ __attribute__((aligned(16))) _Float16 sB0[FWD_IMG_HALVES], sB1[FWD_IMG_HALVES];
     int type, row0, rows;
     if (!tile_of_block(offsets, ne, blockIdx.x, type, row0, rows, group)) return;
-    const int col0 = blockIdx.y * 128;
-    const float* Bt = Bm + (size_t)type * b_type_stride;
+    const int col0 = blockIdx.y * 128, ncb = gridDim.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int i = lane & 31, h = lane >> 5;
+    const int nchunks = (K + PK - 1) / PK;
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    const unsigned lane16 = (unsigned)lane * 16u;
+    const unsigned char* img0 = reinterpret_cast<const unsigned char*>(images) +
+                                ((size_t)type * nchunks * ncb + blockIdx.y) * FWD_IMG_BYTES;
+    const int* exps = exponents + (size_t)type * nchunks * ncb + blockIdx.y;
+    image_to_lds<FWD_IMG_BYTES>(img0, sB0, wave_s, lane16);
 
-    // staging of A: rows tid/8 + 32 v, k = (tid%8)*4 .. +3 of the chunk
-    const int ar = tid >> 3, ak = (tid & 7) * 4;
-    const float* arow[4];
-    bool arow_ok[4];
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        const int r = ar + 32 * v;
-        arow_ok[v] = r < rows;
-        size_t src = 0;
-        if (arow_ok[v]) {
-            if (group > 1) {
-                const int e = (row0 + r) / group;
-                src = (size_t)a_rows[e] * group + (size_t)(row0 + r - e * group);
-            } else {
-                src = (size_t)(a_rows ? a_rows[row0 + r] : row0 + r);
-            }
+    // this lane's row of A: row 32 wave + i, of each chunk the k = 16 s + 8 h + (0..7), s = 0, 1
+    const int r = 32 * wave + i;
+    const bool rok = r < rows;
+    size_t src = 0;
+    if (rok) {
+        if (group > 1) {
+            const int e = (row0 + r) / group;
+            src = (size_t)a_rows[e] * group + (size_t)(row0 + r - e * group);
+        } else {
+            src = (size_t)(a_rows ? a_rows[row0 + r] : row0 + r);
         }
-        arow[v] = A + src * lda;
     }
-    // staging of B: columns (tid/8)*4 .. +3, rows k = 2 (tid%8) + 16 u and the next one
-    const int bn = (tid >> 3) * 4, bkp = 2 * (tid & 7);
-    float4 ra[4], rb[2][2];
+    const float* arow = A + src * lda + 8 * h;
+    float4 ra[2][2];
     auto fetch = [&](int k0) {
 #pragma unroll
-        for (int v = 0; v < 4; ++v)
-            ra[v] = (arow_ok[v] && k0 + ak < K) ? *reinterpret_cast<const float4*>(arow[v] + k0 + ak) : make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
+        for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
-                const int k = k0 + bkp + 16 * u + e;
-                rb[u][e] = (k < K && col0 + bn < N) ? *reinterpret_cast<const float4*>(Bt + (size_t)k * ldb + col0 + bn)
-                                                   : make_float4(0.f, 0.f, 0.f, 0.f);
+                const int k = k0 + 16 * s2 + 8 * h + 4 * e;
+                ra[s2][e] = (rok && k < K) ? *reinterpret_cast<const float4*>(arow + k0 + 16 * s2 + 4 * e) : make_float4(0.f, 0.f, 0.f, 0.f);
             }
     };
     auto max4 = [](float m, float4 v) { return fmaxf(fmaxf(fmaxf(m, fabsf(v.x)), fmaxf(fabsf(v.y), fabsf(v.z))), fabsf(v.w)); };
@@ -396,125 +540,104 @@ __global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(2, 3))) void
 #pragma unroll
     for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[jt][r] = 0.0f;
+        for (int q = 0; q < 16; ++q) acc[jt][q] = 0.0f;
 
-    const int nchunks = (K + PK - 1) / PK;
     fetch(0);
-    for (int c = 0; c < nchunks; ++c) {
-        const int par = c & 1;
-        {
-            float ma = 0.0f, mb = 0.0f;
+    // one chunk: its image is in `cur`, the next one is loaded into `other`
+    auto round = [&](int c, const _Float16* cur, _Float16* other) {
+        // the rows of this chunk: the wavefront's power of two, two fp16 parts each
+        float ma = max4(max4(max4(max4(0.0f, ra[0][0]), ra[0][1]), ra[1][0]), ra[1][1]);
 #pragma unroll
-            for (int v = 0; v < 4; ++v) ma = max4(ma, ra[v]);
+        for (int o = 32; o >= 1; o >>= 1) ma = fmaxf(ma, __shfl_xor(ma, o, 64));
+        const int ka = scale_exponent(ma);
+        const float sa = pow2i(ka);
+        half8_t ahv[2], alv[2];
 #pragma unroll
-            for (int u = 0; u < 2; ++u) mb = max4(max4(mb, rb[u][0]), rb[u][1]);
+        for (int s2 = 0; s2 < 2; ++s2) {
+            const float w[8] = {ra[s2][0].x * sa, ra[s2][0].y * sa, ra[s2][0].z * sa, ra[s2][0].w * sa,
+                                ra[s2][1].x * sa, ra[s2][1].y * sa, ra[s2][1].z * sa, ra[s2][1].w * sa};
 #pragma unroll
-            for (int o = 32; o >= 1; o >>= 1) {
-                ma = fmaxf(ma, __shfl_xor(ma, o, 64));
-                mb = fmaxf(mb, __shfl_xor(mb, o, 64));
-            }
-            if (lane == 0) {
-                smax[par][wave][0] = ma;
-                smax[par][wave][1] = mb;
+            for (int q = 0; q < 8; ++q) {
+                _Float16 a_, c_;
+                split_f16(w[q], a_, c_);
+                ahv[s2][q] = a_;
+                alv[s2][q] = c_;
             }
         }
-        __syncthreads();     // the chunk before has been read, and the largest entries of this one are known
-        const int ka = scale_exponent(fmaxf(fmaxf(smax[par][0][0], smax[par][1][0]), fmaxf(smax[par][2][0], smax[par][3][0])));
-        const int kb = scale_exponent(fmaxf(fmaxf(smax[par][0][1], smax[par][1][1]), fmaxf(smax[par][2][1], smax[par][3][1])));
-        const float sa = pow2i(ka), sb = pow2i(kb), inv = pow2i(-ka) * pow2i(-kb);
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const float w[4] = {ra[v].x * sa, ra[v].y * sa, ra[v].z * sa, ra[v].w * sa};
-            half4_t wh, wl;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                _Float16 a, cc;
-                split_f16(w[e], a, cc);
-                wh[e] = a;
-                wl[e] = cc;
-            }
-            *reinterpret_cast<half4_t*>(&sAh[(ar + 32 * v) * LDH + ak]) = wh;
-            *reinterpret_cast<half4_t*>(&sAl[(ar + 32 * v) * LDH + ak]) = wl;
-        }
-        {
-            const float bv[2][2][4] = {{{rb[0][0].x, rb[0][0].y, rb[0][0].z, rb[0][0].w}, {rb[0][1].x, rb[0][1].y, rb[0][1].z, rb[0][1].w}},
-                                       {{rb[1][0].x, rb[1][0].y, rb[1][0].z, rb[1][0].w}, {rb[1][1].x, rb[1][1].y, rb[1][1].z, rb[1][1].w}}};
-#pragma unroll
-            for (int cc = 0; cc < 4; ++cc)
-#pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    _Float16 h0, l0, h1, l1;
-                    split_f16(bv[u][0][cc] * sb, h0, l0);
-                    split_f16(bv[u][1][cc] * sb, h1, l1);
-                    *reinterpret_cast<half2_t*>(&sBh[(bn + cc) * LDH + bkp + 16 * u]) = (half2_t){h0, h1};
-                    *reinterpret_cast<half2_t*>(&sBl[(bn + cc) * LDH + bkp + 16 * u]) = (half2_t){l0, l1};
-                }
-        }
+        // this chunk's image has landed (every wavefront waits for its own loads, then for the others),
+        // and the other copy, read in the round before, is free
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (c + 1 < nchunks) fetch((c + 1) * PK);
+        if (c + 1 < nchunks) {
+            image_to_lds<FWD_IMG_BYTES>(img0 + (size_t)(c + 1) * ncb * FWD_IMG_BYTES, other, wave_s, lane16);
+            fetch((c + 1) * PK);
+        }
+        const int kb = exps[(size_t)c * ncb];
+        const _Float16* sBh = cur;
+        const _Float16* sBl = cur + 128 * FWD_LDH;
 #pragma unroll
         for (int j0 = 0; j0 < 4; j0 += 2) {
             float16_t part[2];
 #pragma unroll
             for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) part[jj][r] = 0.0f;
+                for (int q = 0; q < 16; ++q) part[jj][q] = 0.0f;
 #pragma unroll
             for (int s2 = 0; s2 < PK / 16; ++s2) {
-                const half8_t ahv = *reinterpret_cast<const half8_t*>(&sAh[(32 * wave + i) * LDH + 16 * s2 + 8 * h]);
-                const half8_t alv = *reinterpret_cast<const half8_t*>(&sAl[(32 * wave + i) * LDH + 16 * s2 + 8 * h]);
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj) {
-                    const half8_t bhv = *reinterpret_cast<const half8_t*>(&sBh[(32 * (j0 + jj) + i) * LDH + 16 * s2 + 8 * h]);
-                    const half8_t blv = *reinterpret_cast<const half8_t*>(&sBl[(32 * (j0 + jj) + i) * LDH + 16 * s2 + 8 * h]);
-                    part[jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(alv, bhv, part[jj], 0, 0, 0);
-                    part[jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ahv, blv, part[jj], 0, 0, 0);
-                    part[jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ahv, bhv, part[jj], 0, 0, 0);
+                    const half8_t bhv = *reinterpret_cast<const half8_t*>(&sBh[(32 * (j0 + jj) + i) * FWD_LDH + 16 * s2 + 8 * h]);
+                    const half8_t blv = *reinterpret_cast<const half8_t*>(&sBl[(32 * (j0 + jj) + i) * FWD_LDH + 16 * s2 + 8 * h]);
+                    part[jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(alv[s2], bhv, part[jj], 0, 0, 0);
+                    part[jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ahv[s2], blv, part[jj], 0, 0, 0);
+                    part[jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ahv[s2], bhv, part[jj], 0, 0, 0);
                 }
             }
 #pragma unroll
-            for (int jj = 0; jj < 2; ++jj)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[j0 + jj][r] = fmaf(part[jj][r], inv, acc[j0 + jj][r]);
+            for (int jj = 0; jj < 2; ++jj) add_scaled(acc[j0 + jj], part[jj], ka, kb);
         }
+    };
+    for (int c = 0; c < nchunks; c += 2) {
+        round(c, sB0, sB1);
+        if (c + 1 < nchunks) round(c + 1, sB1, sB0);
     }
 
 #pragma unroll
     for (int jt = 0; jt < 4; ++jt) {
         const int col = col0 + 32 * jt + i;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int row = 32 * wave + 8 * (r / 4) + 4 * h + (r % 4);
-            if (row < rows && col < N) C[(size_t)(row0 + row) * ldc + col] = acc[jt][r];
+        for (int q = 0; q < 16; ++q) {
+            const int row = 32 * wave + 8 * (q / 4) + 4 * h + (q % 4);
+            if (row < rows && col < N) C[(size_t)(row0 + row) * ldc + col] = acc[jt][q];
         }
     }
 }
 
 // Transpose product for a short contraction (K = projected dimension 64 or 128):
-//     C[c_rows[row], :] = A[row, :] . B_type^T,   A [rows, K] (the gradient rows), B_type [N, K] row-major,
-// on the half-precision matrix cores (v_mfma_f32_32x32x16_f16: eight times the flops of the fp32
-// instruction in 40 clocks against 64): both operands as two fp16 parts each, three matrix
-// instructions per product term.  A wavefront keeps its 32 rows of A in registers for the whole
-// kernel, so every row of A is read exactly once; the workgroup walks the N columns in blocks of 32,
-// each block of B staged through LDS (k contiguous, two copies) while the previous block is
-// multiplied, and every 32 x 32 block of C leaves straight from the accumulators.  The rows of A
-// take the wavefront's power of two, every row of B (a column of the product) its own, found by the
-// eight lanes that stage it; the product leaves the accumulators through the two inverse factors.
+//     C[c_rows[row], :] = A[row, :] . U_type^T,   A [rows, K] (the gradient rows), U_type [N, K] row-major.
+// A wavefront keeps its 32 rows of A in registers for the whole kernel (two fp16 parts behind the
+// wavefront's power of two), so every row of A is read exactly once; the workgroup walks the N columns
+// in blocks of 32, each block's image arriving in LDS while the previous block is multiplied, and every
+// 32 x 32 block of C leaves straight from the accumulators through the two inverse factors.
 template <int K>
-__global__ __launch_bounds__(PT) void typed_gemm_bt_rows_f16_kernel(const float* __restrict__ A, const float* __restrict__ Bm,
-                                                                     size_t b_type_stride, float* __restrict__ C, int ldc,
+__global__ __launch_bounds__(PT) void typed_gemm_bt_rows_f16_kernel(const float* __restrict__ A,
+                                                                     const unsigned char* __restrict__ images,
+                                                                     float* __restrict__ C, int ldc,
                                                                      const int* __restrict__ c_rows,
                                                                      const int* __restrict__ offsets, int ne, int N) {
+    using Img = BwdImage<K>;
     constexpr int KS = K / 16;         // matrix instructions along k per product term
-    constexpr int LDB = K + 8;         // halves per staged row of B
-    constexpr int NV = K / 32;         // float4 per thread and staged block
-    __shared__ __attribute__((aligned(16))) _Float16 sBh[2][32 * LDB], sBl[2][32 * LDB];
-    __shared__ float sinv[2][32];      // inverse scale of each staged row
+    constexpr int LDB = Img::LDB;
+    __shared__ __attribute__((aligned(16))) unsigned char sI0[Img::BYTES], sI1[Img::BYTES];
     int type, row0, rows;
     if (!tile_of_block(offsets, ne, blockIdx.x, type, row0, rows)) return;
-    const float* Bt = Bm + (size_t)type * b_type_stride;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int i = lane & 31, h = lane >> 5;
+    const int nblk = (N + 31) / 32;
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    const unsigned lane16 = (unsigned)lane * 16u;
+    const unsigned char* img0 = images + (size_t)type * nblk * Img::BYTES;
+    image_to_lds<Img::BYTES>(img0, sI0, wave_s, lane16);
 
     const int r = 32 * wave + i;
     const bool rok = r < rows;
@@ -549,58 +672,22 @@ __global__ __launch_bounds__(PT) void typed_gemm_bt_rows_f16_kernel(const float*
                 al[j][q] = c;
             }
     }
-    // staging of a block of B: thread -> row tid/8 of the block, floats (tid%8)*4 + 32 v
-    const int bn = tid >> 3, bk = (tid & 7) * 4;
-    float4 rb[NV];
-    auto fetch = [&](int b) {
-        const int n = 32 * b + bn;
-#pragma unroll
-        for (int v = 0; v < NV; ++v)
-            rb[v] = n < N ? *reinterpret_cast<const float4*>(Bt + (size_t)n * K + bk + 32 * v) : make_float4(0.f, 0.f, 0.f, 0.f);
-    };
-    auto stash = [&](int buf) {
-        float m = 0.0f;
-#pragma unroll
-        for (int v = 0; v < NV; ++v) m = fmaxf(fmaxf(fmaxf(m, fabsf(rb[v].x)), fmaxf(fabsf(rb[v].y), fabsf(rb[v].z))), fabsf(rb[v].w));
-        m = fmaxf(m, lane_xor<1>(m));            // the eight lanes of a row are neighbours
-        m = fmaxf(m, lane_xor<2>(m));
-        m = fmaxf(m, lane_xor<4>(m));
-        const int kb = scale_exponent(m);
-        const float sb = pow2i(kb);
-        if ((tid & 7) == 0) sinv[buf][bn] = pow2i(-kb);
-#pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const float w[4] = {rb[v].x * sb, rb[v].y * sb, rb[v].z * sb, rb[v].w * sb};
-            half4_t wh, wl;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                _Float16 a, c;
-                split_f16(w[e], a, c);
-                wh[e] = a;
-                wl[e] = c;
-            }
-            *reinterpret_cast<half4_t*>(&sBh[buf][bn * LDB + bk + 32 * v]) = wh;
-            *reinterpret_cast<half4_t*>(&sBl[buf][bn * LDB + bk + 32 * v]) = wl;
-        }
-    };
     int dst[16];                        // destination rows of the 16 accumulator registers
 #pragma unroll
     for (int q = 0; q < 16; ++q) {
         const int row = 32 * wave + 8 * (q / 4) + 4 * h + (q % 4);
         dst[q] = row < rows ? (c_rows ? c_rows[row0 + row] : row0 + row) : -1;
     }
-    const int nblk = (N + 31) / 32;
-    fetch(0);
-    stash(0);
-    __syncthreads();
-    for (int b = 0; b < nblk; ++b) {
-        const int cur = b & 1;
-        if (b + 1 < nblk) fetch(b + 1);
+    // one block of 32 columns: its image is in `cur`, the next one is loaded into `other`
+    auto round = [&](int b, const unsigned char* cur, unsigned char* other) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (b + 1 < nblk) image_to_lds<Img::BYTES>(img0 + (size_t)(b + 1) * Img::BYTES, other, wave_s, lane16);
         float16_t acc;
 #pragma unroll
         for (int q = 0; q < 16; ++q) acc[q] = 0.0f;
-        const _Float16* bph = &sBh[cur][i * LDB + 8 * h];
-        const _Float16* bpl = &sBl[cur][i * LDB + 8 * h];
+        const _Float16* bph = reinterpret_cast<const _Float16*>(cur) + i * LDB + 8 * h;
+        const _Float16* bpl = bph + 32 * LDB;
 #pragma unroll
         for (int j = 0; j < KS; ++j) {
             const half8_t bh = *reinterpret_cast<const half8_t*>(bph + 16 * j);
@@ -609,16 +696,18 @@ __global__ __launch_bounds__(PT) void typed_gemm_bt_rows_f16_kernel(const float*
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[j], bl, acc, 0, 0, 0);
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[j], bh, acc, 0, 0, 0);
         }
-        const float f = inv_sa * sinv[cur][i];
+        const float sinv = reinterpret_cast<const float*>(cur + Img::SINV)[i];
         const int col = 32 * b + i;
         if (col < N) {
+            // the two inverse factors one after the other: their product need not be a float
 #pragma unroll
             for (int q = 0; q < 16; ++q)
-                if (dst[q] >= 0) C[(size_t)dst[q] * ldc + col] = acc[q] * f;
+                if (dst[q] >= 0) C[(size_t)dst[q] * ldc + col] = acc[q] * inv_sa * sinv;
         }
-        // the other copy was last read in the previous round, which every wavefront left through the barrier below
-        if (b + 1 < nblk) stash(cur ^ 1);
-        __syncthreads();
+    };
+    for (int b = 0; b < nblk; b += 2) {
+        round(b, sI0, sI1);
+        if (b + 1 < nblk) round(b + 1, sI1, sI0);
     }
 }
 
@@ -857,8 +946,62 @@ extern "C" int qmll_sort_by_type_noalloc(const int* types, const int* slots, int
                              stream);
 }
 
+// layout of the prepared reductors: forward images, backward images, forward exponents
+struct SplitLayout {
+    size_t fwd_bytes, bwd_bytes, exp_bytes;
+    int nchunks, ncb, nblk;
+    size_t bwd_image;
+    size_t total() const { return fwd_bytes + bwd_bytes + exp_bytes; }
+};
+static SplitLayout split_layout(int ne, int R, int d) {
+    SplitLayout L{};
+    if (ne <= 0 || R <= 0 || d <= 0 || R % 4 != 0) return L;
+    L.nchunks = (R + PK - 1) / PK;
+    L.nblk = (R + 31) / 32;
+    if (d % 128 == 0) {
+        L.ncb = d / 128;
+        L.fwd_bytes = (size_t)ne * L.nchunks * L.ncb * FWD_IMG_BYTES;
+        L.exp_bytes = ((size_t)ne * L.nchunks * L.ncb * sizeof(int) + 15) / 16 * 16;
+    }
+    if (d == 64 || d == 128) {
+        L.bwd_image = d == 64 ? (size_t)BwdImage<64>::BYTES : (size_t)BwdImage<128>::BYTES;
+        L.bwd_bytes = (size_t)ne * L.nblk * L.bwd_image;
+    }
+    return L;
+}
+
+extern "C" size_t qmll_reductor_presplit_bytes(int ne, int R, int d) { return split_layout(ne, R, d).total(); }
+
+extern "C" int qmll_reductor_presplit(const float* reductors, int ne, int R, int d, void* out, size_t out_bytes,
+                                      qmll_stream_t stream) {
+    QMLL_REQUIRE(ne > 0 && R > 0 && d > 0 && ne <= 65535, QMLL_ERR_INVALID, "qmll_reductor_presplit: bad size ne=%d R=%d d=%d", ne, R, d);
+    const SplitLayout L = split_layout(ne, R, d);
+    QMLL_REQUIRE(L.total() > 0, QMLL_ERR_INVALID,
+                 "qmll_reductor_presplit: no kernel takes prepared reductors of R=%d (a multiple of 4) x d=%d (64 or a multiple of 128)", R, d);
+    QMLL_REQUIRE(reductors && out && aligned16(reductors) && aligned16(out), QMLL_ERR_INVALID,
+                 "qmll_reductor_presplit: null or unaligned pointer");
+    QMLL_REQUIRE(out_bytes >= L.total(), QMLL_ERR_INVALID, "qmll_reductor_presplit: output of %zu bytes, %zu are needed",
+                 out_bytes, L.total());
+    unsigned char* base = (unsigned char*)out;
+    if (L.fwd_bytes) {
+        hipLaunchKernelGGL(reductor_presplit_fwd_kernel, dim3(L.nchunks * L.ncb, ne), dim3(PT), 0, (hipStream_t)stream,
+                           reductors, R, d, L.ncb, (_Float16*)base, (int*)(base + L.fwd_bytes + L.bwd_bytes));
+        QMLL_CHECK_LAUNCH("qmll_reductor_presplit");
+    }
+    if (L.bwd_bytes) {
+        if (d == 64)
+            hipLaunchKernelGGL(reductor_presplit_bwd_kernel<64>, dim3(L.nblk, ne), dim3(PT), 0, (hipStream_t)stream, reductors,
+                               R, base + L.fwd_bytes);
+        else
+            hipLaunchKernelGGL(reductor_presplit_bwd_kernel<128>, dim3(L.nblk, ne), dim3(PT), 0, (hipStream_t)stream, reductors,
+                               R, base + L.fwd_bytes);
+        QMLL_CHECK_LAUNCH("qmll_reductor_presplit");
+    }
+    return QMLL_OK;
+}
+
 extern "C" int qmll_project_typed(const float* rep, const int* sorted_slots, const int* type_offsets,
-                                  const float* reductors, int A, int ne, int R, int d, float* x,
+                                  const float* reductors, const void* reductors_split, int A, int ne, int R, int d, float* x,
                                   qmll_stream_t stream) {
     QMLL_REQUIRE(A >= 0 && ne > 0 && R > 0 && d > 0, QMLL_ERR_INVALID, "qmll_project_typed: bad size A=%d ne=%d R=%d d=%d", A,
                  ne, R, d);
@@ -879,9 +1022,15 @@ extern "C" int qmll_project_typed(const float* rep, const int* sorted_slots, con
     // the wide tile when it wastes no columns and still leaves every CU a few workgroups
     const bool wide = vec && d % 128 == 0 && (long long)tiles * (d / 128) >= 2 * 256;
     const dim3 grid(tiles, wide ? d / 128 : (d + PN - 1) / PN);
-    if (wide)
-        hipLaunchKernelGGL(typed_gemm_f16_kernel, grid, dim3(PT), 0, (hipStream_t)stream, rep, R, sorted_slots, reductors,
-                           (size_t)R * d, d, x, d, type_offsets, ne, R, d, 1);
+    if (wide && reductors_split) {
+        const SplitLayout L = split_layout(ne, R, d);
+        QMLL_REQUIRE(aligned16(reductors_split), QMLL_ERR_INVALID, "qmll_project_typed: reductors_split must be 16-byte aligned");
+        const unsigned char* base = (const unsigned char*)reductors_split;
+        hipLaunchKernelGGL(typed_gemm_f16_kernel, grid, dim3(PT), 0, (hipStream_t)stream, rep, R, sorted_slots,
+                           (const _Float16*)base, (const int*)(base + L.fwd_bytes + L.bwd_bytes), x, d, type_offsets, ne, R, d, 1);
+    } else if (wide)
+        hipLaunchKernelGGL((typed_gemm_kernel<false, true, 128>), grid, dim3(PT), 0, (hipStream_t)stream, rep, R, sorted_slots,
+                           reductors, (size_t)R * d, d, x, d, (const int*)nullptr, type_offsets, ne, R, d, 1);
     else if (vec)
         hipLaunchKernelGGL((typed_gemm_kernel<false, true, PN>), grid, dim3(PT), 0, (hipStream_t)stream, rep, R, sorted_slots,
                            reductors, (size_t)R * d, d, x, d, (const int*)nullptr, type_offsets, ne, R, d);
@@ -927,8 +1076,8 @@ extern "C" int qmll_project_typed_rows(const float* rows, const int* sorted_slot
 }
 
 extern "C" int qmll_project_typed_backward(const float* gx, const int* sorted_slots, const int* type_offsets,
-                                           const float* reductors, const int* types, int A, int N, int ne, int R,
-                                           int d, float* g_rep, qmll_stream_t stream) {
+                                           const float* reductors, const void* reductors_split, const int* types, int A,
+                                           int N, int ne, int R, int d, float* g_rep, qmll_stream_t stream) {
     QMLL_REQUIRE(A >= 0 && N >= 0 && ne > 0 && R > 0 && d > 0, QMLL_ERR_INVALID,
                  "qmll_project_typed_backward: bad size A=%d N=%d ne=%d R=%d d=%d", A, N, ne, R, d);
     const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(gx) && aligned16(reductors);
@@ -948,15 +1097,19 @@ extern "C" int qmll_project_typed_backward(const float* gx, const int* sorted_sl
         const int zero_groups = (types && N > 0) ? (N + 255) / 256 : 0;
         hipLaunchKernelGGL(project_bt_small_kernel, dim3(A + zero_groups), dim3(256), sizeof(float) * d, (hipStream_t)stream,
                            gx, sorted_slots, type_offsets, reductors, ne, R, d, g_rep, A, types, N);
-    } else if (vec && (d == 64 || d == 128)) {
+    } else if (vec && (d == 64 || d == 128) && reductors_split) {
         // short contraction: the gradient rows stay in registers, every row is read once
+        const SplitLayout L = split_layout(ne, R, d);
+        QMLL_REQUIRE(aligned16(reductors_split), QMLL_ERR_INVALID,
+                     "qmll_project_typed_backward: reductors_split must be 16-byte aligned");
+        const unsigned char* images = (const unsigned char*)reductors_split + L.fwd_bytes;
         const dim3 g1((A + PM - 1) / PM + ne);
         if (d == 128)
-            hipLaunchKernelGGL((typed_gemm_bt_rows_f16_kernel<128>), g1, dim3(PT), 0, (hipStream_t)stream, gx, reductors,
-                               (size_t)R * d, g_rep, R, sorted_slots, type_offsets, ne, R);
+            hipLaunchKernelGGL((typed_gemm_bt_rows_f16_kernel<128>), g1, dim3(PT), 0, (hipStream_t)stream, gx, images, g_rep,
+                               R, sorted_slots, type_offsets, ne, R);
         else
-            hipLaunchKernelGGL((typed_gemm_bt_rows_f16_kernel<64>), g1, dim3(PT), 0, (hipStream_t)stream, gx, reductors,
-                               (size_t)R * d, g_rep, R, sorted_slots, type_offsets, ne, R);
+            hipLaunchKernelGGL((typed_gemm_bt_rows_f16_kernel<64>), g1, dim3(PT), 0, (hipStream_t)stream, gx, images, g_rep,
+                               R, sorted_slots, type_offsets, ne, R);
     } else if (vec)
         hipLaunchKernelGGL((typed_gemm_kernel<true, true, PN>), grid, dim3(PT), 0, (hipStream_t)stream, gx, d,
                            (const int*)nullptr, reductors, (size_t)R * d, d, g_rep, R, sorted_slots, type_offsets, ne, d, R);

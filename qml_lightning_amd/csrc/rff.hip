@@ -464,14 +464,10 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
         constexpr float UMAX = 1500.0f * 0.15915494309189535f;
         const float crev = inv_sxw * 0.15915494309189535f;
         float umax = 0.0f;
-        float aq[16];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const int fl = 8 * q + 4 * h;
-            const float4 bv = *reinterpret_cast<const float4*>(&sb[fl]);
-            const float4 av = *reinterpret_cast<const float4*>(&sa[fl]);
+            const float4 bv = *reinterpret_cast<const float4*>(&sb[8 * q + 4 * h]);
             const float bq[4] = {bv.x, bv.y, bv.z, bv.w};
-            aq[4 * q] = av.x; aq[4 * q + 1] = av.y; aq[4 * q + 2] = av.z; aq[4 * q + 3] = av.w;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 sacc[4 * q + e] = fmaf(sacc[4 * q + e], crev, bq[e]);
@@ -484,10 +480,16 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
                 if (fabsf(sacc[r]) > UMAX) sacc[r] -= rintf(sacc[r]);
         }
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const float sn = __builtin_amdgcn_sinf(sacc[r]), cs = __builtin_amdgcn_cosf(sacc[r]);
-            energy = fmaf(aq[r], cs, energy);
-            sacc[r] = -aq[r] * sn;                       // 2^kp P
+        for (int q = 0; q < 4; ++q) {
+            const float4 av = *reinterpret_cast<const float4*>(&sa[8 * q + 4 * h]);
+            const float aq[4] = {av.x, av.y, av.z, av.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float u = sacc[4 * q + e];
+                const float sn = __builtin_amdgcn_sinf(u), cs = __builtin_amdgcn_cosf(u);
+                energy = fmaf(aq[e], cs, energy);
+                sacc[4 * q + e] = -aq[e] * sn;           // 2^kp P
+            }
         }
         if constexpr (WITH_GRAD) {
             // second product: 2^kp GX^T[k, a] += 2^-kw sum_f 2^kw W[k, f] 2^kp P[f, a]; instruction t contracts the

@@ -453,6 +453,21 @@ std::tuple<Tensor, Tensor> sort_atoms_by_type(const Tensor& types, const Tensor&
     return {sorted, offsets};
 }
 
+// the reductors prepared for the fp16 matrix-core projections (large batches only: the small-batch
+// kernels read the fp32 reductors), or an undefined tensor
+Tensor reductors_split(const Tensor& red, int A) {
+    if (A < 2049) return Tensor();
+    const int ne = (int)red.size(0), R = (int)red.size(1), d = (int)red.size(2);
+    const size_t nbytes = qmll_reductor_presplit_bytes(ne, R, d);
+    if (nbytes == 0) return Tensor();
+    return prepared_form(red, 1, [&](const Tensor& u) {
+        Tensor out = at::empty({(int64_t)nbytes}, u.options().dtype(at::kByte));
+        check(qmll_reductor_presplit(fp(u), ne, R, d, out.data_ptr(), nbytes, stream()), "qmll_reductor_presplit");
+        return out;
+    });
+}
+const void* vp(const Tensor& t) { return t.defined() && t.numel() ? t.const_data_ptr() : nullptr; }
+
 Tensor project_typed_impl(const Tensor& rep, const Tensor& sorted_slots, const Tensor& type_offsets,
                           const Tensor& reductors) {
     Tensor r = f32(rep), red = f32(reductors), ss = i32(sorted_slots), off = i32(type_offsets);
@@ -461,7 +476,9 @@ Tensor project_typed_impl(const Tensor& rep, const Tensor& sorted_slots, const T
     TORCH_CHECK(r.dim() == 2 && r.size(1) == R && off.size(0) == ne + 1,
                 "project_typed: rep, reductors and offsets do not fit together");
     Tensor x = at::empty({A, d}, r.options());
-    check(qmll_project_typed(fp(r), ip(ss), ip(off), fp(red), A, ne, R, d, A ? x.data_ptr<float>() : nullptr, stream()),
+    Tensor split = reductors_split(red, A);
+    check(qmll_project_typed(fp(r), ip(ss), ip(off), fp(red), vp(split), A, ne, R, d, A ? x.data_ptr<float>() : nullptr,
+                             stream()),
           "qmll_project_typed");
     return x;
 }
@@ -477,7 +494,8 @@ Tensor project_typed_backward(const Tensor& gx, const Tensor& sorted_slots, cons
     // every slot a real atom: the kernel writes every row of a known element and zeroes the rest
     const bool full = A == N;
     Tensor g_rep = full ? at::empty({N, R}, g.options()) : at::zeros({N, R}, g.options());
-    check(qmll_project_typed_backward(fp(g), ip(ss), ip(off), fp(red), full ? ip(ty) : nullptr, A, N, ne, R, d,
+    Tensor split = reductors_split(red, A);
+    check(qmll_project_typed_backward(fp(g), ip(ss), ip(off), fp(red), vp(split), full ? ip(ty) : nullptr, A, N, ne, R, d,
                                       N ? g_rep.data_ptr<float>() : nullptr, stream()),
           "qmll_project_typed_backward");
     return g_rep;

@@ -418,6 +418,29 @@ def sort_atoms_by_type(types, atomIDs, molIDs, n, ne):
     return sorted_slots, offsets
 
 
+def reductor_presplit(reductors):
+    """The reductors [ne,R,d] in the form the fp16 matrix-core projection kernels multiply with
+    (qmll_reductor_presplit): an opaque uint8 device buffer, or None when no kernel takes one."""
+    reductors = _f32(reductors)
+    ne, R, d = reductors.shape
+    nbytes = int(_lib.lib().qmll_reductor_presplit_bytes(ne, R, d))
+    if nbytes == 0:
+        return None
+    out = torch.empty(nbytes, dtype=torch.uint8, device=reductors.device)
+    check(_lib.lib().qmll_reductor_presplit(_ptr(reductors), ne, R, d, _ptr(out), nbytes, _stream()),
+          "qmll_reductor_presplit")
+    return out
+
+
+#: from this many atoms on the projections are handed the prepared reductors (below, the
+#: one-workgroup-per-atom kernels run, which read the fp32 reductors)
+SPLIT_FROM_ATOMS = 2049
+
+
+def _split_for(reductors, A):
+    return presplit_cached(reductors, "reductor", reductor_presplit) if A >= SPLIT_FROM_ATOMS else None
+
+
 def project_typed(rep, sorted_slots, type_offsets, reductors):
     """x [A,d]: row a = rep[sorted_slots[a]] . reductors[type of a] (rep [N,R], reductors [ne,R,d])."""
     rep, reductors = _f32(rep), _f32(reductors)
@@ -428,8 +451,9 @@ def project_typed(rep, sorted_slots, type_offsets, reductors):
                            % (tuple(rep.shape), tuple(reductors.shape), type_offsets.shape[0]))
     A = int(sorted_slots.shape[0])
     x = torch.empty((A, d), dtype=torch.float32, device=rep.device)
-    check(_lib.lib().qmll_project_typed(_ptr(rep), _ptr(sorted_slots), _ptr(type_offsets), _ptr(reductors), A, ne, R, d,
-                                        _ptr(x), _stream()), "qmll_project_typed")
+    check(_lib.lib().qmll_project_typed(_ptr(rep), _ptr(sorted_slots), _ptr(type_offsets), _ptr(reductors),
+                                        _ptr(_split_for(reductors, A)), A, ne, R, d, _ptr(x), _stream()),
+          "qmll_project_typed")
     return x
 
 
@@ -467,7 +491,8 @@ def project_typed_backward(gx, sorted_slots, type_offsets, reductors, types, nsl
         g_rep = torch.zeros((N, R), dtype=torch.float32, device=gx.device)
         tz = None
     check(_lib.lib().qmll_project_typed_backward(_ptr(gx), _ptr(sorted_slots), _ptr(type_offsets), _ptr(reductors),
-                                                 _ptr(tz), A, N, ne, R, d, _ptr(g_rep), _stream()),
+                                                 _ptr(_split_for(reductors, A)), _ptr(tz), A, N, ne, R, d, _ptr(g_rep),
+                                                 _stream()),
           "qmll_project_typed_backward")
     return g_rep
 
