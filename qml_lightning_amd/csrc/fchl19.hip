@@ -700,9 +700,11 @@ __device__ __forceinline__ TripleDeriv triple_derivatives(const Triple& t, const
 // ---------------------------------------------------------------------------------
 // VJP
 // ---------------------------------------------------------------------------------
-// TABLE: the three force coefficients of a triple go to an LDS table [3][ntrip] and are
-// summed per neighbour afterwards (each triple index is computed, never searched), instead
-// of LDS atomics, which serialise badly here: the 64 triples of a pass share 3-4 values of j.
+// TABLE: the force coefficients of a triple (j, k) go to a neighbour x neighbour matrix in LDS, entry
+// [x][y] = (ec, coefficient of d_ix) of the triple {x, y}, and every neighbour's row is summed
+// afterwards with a loop of the same length for every lane, instead of LDS atomics, which
+// serialise badly here: the 64 triples of a pass share 3-4 values of j.  a.tcap is the matrix's row
+// length (odd, so that rows start in different banks).
 template <bool TABLE>
 __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float* __restrict__ grad_rep,
                                                          float* __restrict__ grad_X) {
@@ -712,33 +714,41 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
     const int i = a.atomIDs[blockIdx.x];
     if (m < 0 || m >= a.B || i < 0 || i >= a.n) return;   // malformed index: write nothing
     const int ns = a.p.nspecies, nRs2 = a.p.nRs2, nRs3 = a.p.nRs3;
-    const int R = ns * nRs2 + ns * (ns + 1) * nRs3;
+    const int R2 = ns * nRs2;                        // two-body part of a representation row
+    const int NE3 = (ns * (ns + 1) / 2) * nRs3;      // (element pair, radial bin) entries of its three-body part
 
     // [cap][4] per neighbour, read with one instruction each: (d_ij, r) and
     // (1 / r, fc, dfc / dr, element type); first in LDS, 16-byte aligned
     float* recA = smem;
     float* recB = recA + 4 * a.cap;
-    int* sj = (int*)(recB + 4 * a.cap);   // [cap] atom index of neighbour j
+    float* eo = recB + 4 * a.cap;              // TABLE: [cap][tcap][2]
+    float* gin3 = eo + (TABLE ? 2 * a.cap * a.tcap : 0);   // [NE3][2] incoming gradient of the three-body bins (cos, sin), see below; 8-byte aligned
+    int* sj = (int*)(gin3 + 2 * NE3);          // [cap] atom index of neighbour j
     int* goff = sj + a.cap;              // [ns+1] slices of the sorted neighbour list by type
     float* sgx = (float*)(goff + ns + 1);   // [cap] gradient on neighbour j
     float* sgy = sgx + a.cap;
     float* sgz = sgy + a.cap;
     float* slnRs2 = sgz + a.cap;     // [nRs2]
-    float* sinvRs2 = slnRs2 + nRs2;  // [nRs2]
-    float* sRs3 = sinvRs2 + nRs2;    // [nRs3]
-    float* gin = sRs3 + nRs3;        // [R]
-    float* tab = gin + R;            // TABLE: [3][ntrip]
+    float* sRs3 = slnRs2 + nRs2;     // [nRs3] sk3 Rs3 (fast form: about the middle of the grid)
+    float* sfac = sRs3 + nRs3;       // [nRs3] 2^(-u^2) of every bin (fast form)
+    float* gin2 = sfac + nRs3;       // [R2] incoming gradient of the two-body bins, each divided by its Rs2
     const float4* rA = reinterpret_cast<const float4*>(recA);
     const float4* rB = reinterpret_cast<const float4*>(recB);
 
     // Global loads that do not depend on the neighbourhood (grid tables, the incoming gradient
     // row) are issued first and consumed after the staging, so their latency overlaps the
     // staging's own loads.
-    const float* gsrc = grad_rep + ((size_t)m * a.n + i) * R;
-    constexpr int GREG = 8;                      // gradient values per lane held in registers
-    float gr[GREG];
+    const float* gsrc = grad_rep + ((size_t)m * a.n + i) * (R2 + 2 * NE3);
+    constexpr int GREG2 = 2, GREG3 = 4;          // values / (cos, sin) pairs per lane held in registers
+    float gr2[GREG2], gr3c[GREG3], gr3s[GREG3];
 #pragma unroll
-    for (int k = 0; k < GREG; ++k) gr[k] = lane + QMLL_WAVE * k < R ? gsrc[lane + QMLL_WAVE * k] : 0.0f;
+    for (int k = 0; k < GREG2; ++k) gr2[k] = lane + QMLL_WAVE * k < R2 ? gsrc[lane + QMLL_WAVE * k] : 0.0f;
+#pragma unroll
+    for (int k = 0; k < GREG3; ++k) {
+        const int e = lane + QMLL_WAVE * k;
+        gr3c[k] = e < NE3 ? gsrc[R2 + 2 * e] : 0.0f;
+        gr3s[k] = e < NE3 ? gsrc[R2 + 2 * e + 1] : 0.0f;
+    }
     const float rs2v = lane < nRs2 ? a.Rs2[lane] : 1.0f;
     const float rs3v = lane < nRs3 ? a.Rs3[lane] : 0.0f;
     for (int t = lane; t < a.cap; t += QMLL_WAVE) {
@@ -756,29 +766,68 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
                                         reinterpret_cast<float4*>(recB)[pos] = make_float4(ir, fc, dfc, __int_as_float(e));
                                         sj[pos] = j;
                                     });
-#pragma unroll
-    for (int k = 0; k < GREG; ++k)
-        if (lane + QMLL_WAVE * k < R) gin[lane + QMLL_WAVE * k] = gr[k];
-    for (int t = lane + QMLL_WAVE * GREG; t < R; t += QMLL_WAVE) gin[t] = gsrc[t];
-    if (lane < nRs2) {
-        slnRs2[lane] = flog(rs2v);
-        sinvRs2[lane] = frcp(rs2v);
-    }
     const float k3 = a.p.eta3 * LOG2E;
     const float sk3 = fsqrt(k3);                       // the radial grid of the triples is kept as sk3 Rs3
     const float hfac = -2.0f * a.p.eta3 * frcp(sk3);
-    if (lane < nRs3) sRs3[lane] = sk3 * rs3v;
-    for (int t = lane + QMLL_WAVE; t < nRs2; t += QMLL_WAVE) {
-        const float v = a.Rs2[t];
-        slnRs2[t] = flog(v);
-        sinvRs2[t] = frcp(v);
+    // The radial factor of a triple, exp2(-(x - g_l)^2) with x = sk3 rho and g_l = sk3 Rs3_l, about the
+    // middle of the grid (y = x - mid, u_l = g_l - mid): exp2(2 y u_l - y^2) 2^(-u_l^2).  The second
+    // factor does not depend on the triple and goes into the staged gradient once per atom; the first
+    // is one fma and the exponential per (triple, bin).  It is at most 2^(u_l^2), so the form is taken
+    // only while u_l^2 <= 100 for every bin (eta3 rcut^2 up to about 270); beyond, the plain form runs.
+    const float mid = 0.5f * sk3 * a.p.rcut;
+    bool fast;
+    {
+        float um = fabsf(fmaf(sk3, rs3v, -mid));
+        if (lane >= nRs3) um = 0.0f;
+        for (int t = lane + QMLL_WAVE; t < nRs3; t += QMLL_WAVE) um = fmaxf(um, fabsf(fmaf(sk3, a.Rs3[t], -mid)));
+        um = fmaxf(um, lane_xor<1>(um));
+        um = fmaxf(um, lane_xor<2>(um));
+        um = fmaxf(um, lane_xor<4>(um));
+        um = fmaxf(um, lane_xor<8>(um));
+        um = fmaxf(um, lane_xor<16>(um));
+        um = fmaxf(um, lane_xor<32>(um));
+        fast = __builtin_amdgcn_readfirstlane(__float_as_int(um)) <= __float_as_int(10.0f);
     }
-    for (int t = lane + QMLL_WAVE; t < nRs3; t += QMLL_WAVE) sRs3[t] = sk3 * a.Rs3[t];
+    const float shift = fast ? mid : 0.0f;
+    // the gradient of the two-body bins, each divided by its grid point (the bin's 1 / Rs2 factor)
+#pragma unroll
+    for (int k = 0; k < GREG2; ++k) {
+        const int t = lane + QMLL_WAVE * k;
+        if (t < R2) gin2[t] = gr2[k] * frcp(a.Rs2[t - nRs2 * idiv_small(t, nRs2)]);
+    }
+    for (int t = lane + QMLL_WAVE * GREG2; t < R2; t += QMLL_WAVE)
+        gin2[t] = gsrc[t] * frcp(a.Rs2[t - nRs2 * idiv_small(t, nRs2)]);
+    if (lane < nRs2) slnRs2[lane] = flog(rs2v);
+    for (int t = lane + QMLL_WAVE; t < nRs2; t += QMLL_WAVE) slnRs2[t] = flog(a.Rs2[t]);
+    for (int t = lane; t < nRs3; t += QMLL_WAVE) {
+        const float u = fmaf(sk3, t == lane ? rs3v : a.Rs3[t], -shift);
+        sRs3[t] = u;
+        sfac[t] = fast ? fexp2(-u * u) : 1.0f;
+    }
+    __syncthreads();
+    // the gradient of the three-body bins per (element pair, radial bin), (cos, sin) parts, times the
+    // bin's constant factor s = 2^(-u^2): with e' = exp2(2 y u - y^2) the sums over the bins of g e and
+    // of g (x - g_l) e are sum (g s) e' and y sum (g s) e' - sum (g s) (u e')
+    auto stage3 = [&](int e, float gc, float gs) {
+        const float s_ = sfac[e - nRs3 * idiv_small(e, nRs3)];
+        reinterpret_cast<float2*>(gin3)[e] = make_float2(gc * s_, gs * s_);
+    };
+#pragma unroll
+    for (int k = 0; k < GREG3; ++k)
+        if (lane + QMLL_WAVE * k < NE3) stage3(lane + QMLL_WAVE * k, gr3c[k], gr3s[k]);
+    for (int e = lane + QMLL_WAVE * GREG3; e < NE3; e += QMLL_WAVE) stage3(e, gsrc[R2 + 2 * e], gsrc[R2 + 2 * e + 1]);
+    if constexpr (TABLE) {
+        // no triple writes the diagonal of the coefficient matrix
+        for (int t = lane; t < nn; t += QMLL_WAVE) reinterpret_cast<float2*>(eo)[t * a.tcap + t] = make_float2(0.0f, 0.0f);
+    }
     __syncthreads();
 
     float gix = 0.0f, giy = 0.0f, giz = 0.0f;
 
     // two-body: lanes = (bin group g, neighbour j); group g takes the bins z = g, g+G, ...
+    // With u = ln Rs - mu the r-derivative of a bin is B_z (fc Q + dfc), B_z = pre / Rs exp2(-c u^2) and
+    // Q a quadratic in u whose coefficients (and fc, dfc) depend on the neighbour only:
+    // per bin a subtraction, the exponential and two fma for the quadratic.
     {
         const int G = (nn > 0 && nn < 64) ? idiv_small(64, nn) : 1;
         for (int base = 0; base < nn; base += QMLL_WAVE) {
@@ -791,12 +840,19 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
                 Aj = rA[j];
                 Bj = rB[j];
                 const TwoBody tb = two_body_setup(Aj.w, Bj.y, Bj.z, a.p);
-                const float* gz = gin + __float_as_int(Bj.w) * nRs2;
+                const float inv_s2 = frcp(tb.s2);
+                const float nc = -0.5f * LOG2E * inv_s2;
+                const float hs = 0.5f * tb.s2p * inv_s2;
+                const float q0 = fmaf(tb.fc, -hs - tb.d2_over_r, tb.dfc);
+                const float q1 = tb.fc * inv_s2 * tb.mup;
+                const float q2 = tb.fc * hs * inv_s2;
+                const float* gz = gin2 + __float_as_int(Bj.w) * nRs2;
                 for (int z = g; z < nRs2; z += G) {
-                    float val, dval;
-                    two_body_bin(tb, slnRs2[z], sinvRs2[z], val, dval);
-                    gr = fmaf(gz[z], dval, gr);
+                    const float u = slnRs2[z] - tb.mu;
+                    const float e = fexp2(u * u * nc);
+                    gr = fmaf(gz[z] * e, fmaf(fmaf(q2, u, q1), u, q0), gr);
                 }
+                gr *= tb.pre;
             }
             float tot = gr;
             for (int k = 1; k < G; ++k) tot += __shfl(gr, (lane + nn * k) & 63, 64);
@@ -854,21 +910,40 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
         const float ka = fmaf(F, fmaf(3.0f, Pa3, -d3P * ia), P * dfa * fb);   // K_a / dec
         const float kb = fmaf(F, fmaf(3.0f, Pb3, -d3P * ib), P * fa * dfb);
         const float kc = F * fmaf(3.0f, Pc3, -d3P * ic);
-        const float* g = gin + pair_offset(__float_as_int(Bj.w), __float_as_int(Bk.w), ns, nRs2, nRs3);
-        // exp(-eta3 (rho - Rs)^2) = exp2(-(sk3 rho - sk3 Rs)^2) with the grid stored pre-scaled;
-        // d e / d rho = -2 eta3 (rho - Rs) e = hfac (sk3 rho - sk3 Rs) e, the factor applied after the sums
-        const float rho = sk3 * 0.5f * (Aj.w + Ak.w);
+        // the (element pair, radial bin) entries of this triple's pair: p <= q, the list is sorted by type
+        const int tp = __float_as_int(Bj.w), tq = __float_as_int(Bk.w);
+        const float2* g = reinterpret_cast<const float2*>(gin3) + __mul24(nRs3, __mul24(ns, tp) - (__mul24(tp, tp + 1) >> 1) + tq);
+        // exp(-eta3 (rho - Rs)^2) = exp2(-(x - g_l)^2), x = sk3 rho, the grid stored pre-scaled;
+        // d e / d rho = -2 eta3 (rho - Rs) e = hfac (x - g_l) e, the factor applied after the sums
+        const float y = fmaf(sk3 * 0.5f, Aj.w + Ak.w, -shift);
         float Gc = 0.f, Gs = 0.f, Hc = 0.f, Hs = 0.f;
+        if (fast) {
+            const float y2 = y + y, ny2 = -y * y;
 #pragma unroll 4
-        for (int l = 0; l < nRs3; ++l) {
-            const float dl = rho - sRs3[l];
-            const float e = fexp2(-(dl * dl));
-            const float de = dl * e;
-            const float gc = g[2 * l], gs = g[2 * l + 1];
-            Gc = fmaf(gc, e, Gc);
-            Gs = fmaf(gs, e, Gs);
-            Hc = fmaf(gc, de, Hc);
-            Hs = fmaf(gs, de, Hs);
+            for (int l = 0; l < nRs3; ++l) {
+                const float2 gv = g[l];
+                const float u = sRs3[l];
+                const float e = fexp2(fmaf(y2, u, ny2));
+                const float ue = u * e;
+                Gc = fmaf(gv.x, e, Gc);
+                Gs = fmaf(gv.y, e, Gs);
+                Hc = fmaf(gv.x, ue, Hc);
+                Hs = fmaf(gv.y, ue, Hs);
+            }
+            Hc = fmaf(y, Gc, -Hc);
+            Hs = fmaf(y, Gs, -Hs);
+        } else {
+#pragma unroll 4
+            for (int l = 0; l < nRs3; ++l) {
+                const float2 gv = g[l];
+                const float dl = y - sRs3[l];
+                const float e = fexp2(-(dl * dl));
+                const float de = dl * e;
+                Gc = fmaf(gv.x, e, Gc);
+                Gs = fmaf(gv.y, e, Gs);
+                Hc = fmaf(gv.x, de, Hc);
+                Hs = fmaf(gv.y, de, Hs);
+            }
         }
         const float S0 = Gc * cosT + Gs * sinT;
         const float S1 = 0.5f * hfac * (Hc * cosT + Hs * sinT);                   // d rho/da = d rho/db = 1/2
@@ -881,11 +956,9 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
         giy = fmaf(ea, Aj.y, fmaf(eb, Ak.y, giy));
         giz = fmaf(ea, Aj.z, fmaf(eb, Ak.z, giz));
         if constexpr (TABLE) {
-            // force on j: ec d_ik - (ec + ea) d_ij, on k: ec d_ij - (eb + ec) d_ik; the three
-            // coefficients go to the table, the products are formed when a neighbour's triples are summed
-            tab[0 * ntrip + tt] = ec + ea;
-            tab[1 * ntrip + tt] = eb + ec;
-            tab[2 * ntrip + tt] = ec;
+            // force on j: ec d_ik - (ec + ea) d_ij, on k: ec d_ij - (eb + ec) d_ik
+            reinterpret_cast<float2*>(eo)[j * a.tcap + k] = make_float2(ec, ec + ea);
+            reinterpret_cast<float2*>(eo)[k * a.tcap + j] = make_float2(ec, eb + ec);
         } else {
             atomicAdd(&sgx[j], fmaf(ec, cx, -ea * Aj.x));
             atomicAdd(&sgy[j], fmaf(ec, cy, -ea * Aj.y));
@@ -906,30 +979,19 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
         atomicAdd(&gm[i * 3 + 2], giz);
     }
     if constexpr (TABLE) {
-        // lane = (neighbour x, component c).  The force on x is sum_y ec(x,y) d_iy - d_ix s_x with s_x
-        // the sum of its own coefficients.  Triple (j,k) sits at k (k - 1) / 2 + j: the triples (j,x)
-        // with x second are the run of x entries starting at x (x - 1) / 2; the triples (x,k) with x
-        // first sit at k (k - 1) / 2 + x for k = x+1 .. nn-1, k entries further each step
+        // lane = (neighbour x, component c): the force on x is sum_y ec(x,y) d_iy - d_ix sum_y own(x,y)
+        // over row x of the matrix, plus what the two-body part left for x
         for (int it = lane; it < 3 * nn; it += QMLL_WAVE) {
             const int x = idiv_small(it, 3), c = it - 3 * x;
             float sum = c == 0 ? sgx[x] : (c == 1 ? sgy[x] : sgz[x]);
             float own = 0.0f;
             const float* dc = recA + c;                       // component c of d_iy at dc[4 y]
-            const float* e1 = tab + 1 * ntrip + (x * (x - 1)) / 2;
-            const float* e2 = e1 + ntrip;
+            const float2* row = reinterpret_cast<const float2*>(eo) + x * a.tcap;
 #pragma unroll 4
-            for (int q = 0; q < x; ++q) {
-                sum = fmaf(e2[q], dc[4 * q], sum);
-                own += e1[q];
-            }
-            const float* e0 = tab + x;
-            const float* e2b = e0 + 2 * ntrip;
-            int idx = ((x + 1) * x) / 2;
-#pragma unroll 4
-            for (int k = x + 1; k < nn; ++k) {
-                sum = fmaf(e2b[idx], dc[4 * k], sum);
-                own += e0[idx];
-                idx += k;
+            for (int yv = 0; yv < nn; ++yv) {
+                const float2 v = row[yv];
+                sum = fmaf(v.x, dc[4 * yv], sum);
+                own += v.y;
             }
             atomicAdd(&gm[sj[x] * 3 + c], fmaf(-dc[4 * x], own, sum));
         }
@@ -1313,15 +1375,16 @@ extern "C" int qmll_fchl19_vjp(const float* X, const int* types, const float* ce
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(grad_rep && grad_X, QMLL_ERR_INVALID, "qmll_fchl19_vjp: null gradient pointer");
     const int R = prm->nspecies * prm->nRs2 + prm->nspecies * (prm->nspecies + 1) * prm->nRs3;
-    // two records [cap][4], atom indices, neighbour gradients [3][cap], type offsets, grids, the gradient row
-    size_t lds = sizeof(float) * ((size_t)12 * a.cap + prm->nspecies + 1 + 2 * prm->nRs2 + prm->nRs3 + R);
+    // two records [cap][4], atom indices, neighbour gradients [3][cap], type offsets, grids, the bins' constant
+    // factors, the gradient row
+    size_t lds = sizeof(float) * ((size_t)12 * a.cap + prm->nspecies + 1 + prm->nRs2 + 2 * prm->nRs3 + R);
     QMLL_REQUIRE(lds <= LDS_LIMIT, QMLL_ERR_INVALID,
                  "qmll_fchl19_vjp: %zu B of LDS needed (max_atoms=%d, repsize=%d) exceeds %zu", lds, n, R, LDS_LIMIT);
-    // per-triple coefficient table [3][maxnn (maxnn-1) / 2] while it stays small; LDS atomics beyond.  An atom has
-    // at most cap neighbours from a given list and at most max_atoms - 1 otherwise
-    const size_t maxnn = nlist ? (size_t)a.cap : (size_t)(a.cap > 1 ? a.cap - 1 : 1);
-    const size_t table = sizeof(float) * 3 * (maxnn * (maxnn - 1) / 2);
-    if (table <= 16 * 1024 && lds + table <= LDS_LIMIT) {
+    // neighbour x neighbour coefficient matrix (two floats per entry, rows of odd length) while it stays small;
+    // LDS atomics beyond
+    a.tcap = a.cap | 1;
+    const size_t table = sizeof(float) * 2 * (size_t)a.cap * a.tcap;
+    if (table <= 24 * 1024 && lds + table <= LDS_LIMIT) {
         lds += table;
         hipLaunchKernelGGL(fchl19_vjp_kernel<true>, dim3(A), dim3(64), lds, (hipStream_t)stream, a, grad_rep, grad_X);
     } else {

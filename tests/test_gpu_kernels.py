@@ -932,3 +932,54 @@ def test_rff_derivatives_molecule_major(d, F, n):
     ops.rff_derivative_features(t32(x), t32(grad), torch.tensor(W, device=dev()), torch.tensor(b, device=dev()),
                                 ti32(idx), G, molecule_major=True)
     close(G, G0 + sorf.rff_derivative_features(x, grad, W, b, idx, nmol), 1e-12, "rff derivative features (segments)")
+
+
+def test_prepared_model_constants_follow_their_tensors():
+    """W of the RFF kernel and the reductors of the large-batch projections are split once and the
+    split form is kept per tensor: an in-place update (version counter), a new tensor and a tensor
+    that dies must each be noticed."""
+    import gc
+    from qml_lightning_amd import ops
+    g = torch.Generator(device=dev()).manual_seed(5)
+    A, d, F, R, ne = 2304, 128, 256, 312, 2
+    x = torch.randn(A, d, device=dev(), generator=g)
+    W = torch.randn(ne, d, F, device=dev(), generator=g) / 8
+    b = torch.rand(ne, F, device=dev(), generator=g) * 6.28
+    alpha = torch.randn(F, device=dev(), generator=g)
+    types = torch.arange(A, device=dev(), dtype=torch.int32) % ne
+    ss, off = ops.sort_by_type(types, torch.arange(A, device=dev(), dtype=torch.int32), ne)
+
+    def rff_ref(Wt):
+        t = types.long()[ss.long()]
+        arg = torch.einsum('ak,akf->af', x.double(), Wt.double()[t]) + b.double()[t]
+        return (2.0 / F) ** 0.5 * (torch.cos(arg) * alpha.double()).sum(dim=1)
+    e0, _ = ops.rff_energy_sorted(x, off, ss, W, b, alpha, A)
+    close(e0[ss.long()], rff_ref(W).cpu().numpy(), REL_EF, "first use")
+    nkeys = len(ops._PRESPLIT)
+    e0b, _ = ops.rff_energy_sorted(x, off, ss, W, b, alpha, A)
+    assert len(ops._PRESPLIT) == nkeys                # no second split
+    assert (e0 - e0b).abs().max() <= 1e-6 * e0.abs().max()     # the feature parts add with fp32 atomics
+    W.mul_(0.5)                                       # in place: same object, same address, new version
+    e1, _ = ops.rff_energy_sorted(x, off, ss, W, b, alpha, A)
+    close(e1[ss.long()], rff_ref(W).cpu().numpy(), REL_EF, "after an in-place update")
+    W2 = W * 3.0
+    e2, _ = ops.rff_energy_sorted(x, off, ss, W2, b, alpha, A)
+    close(e2[ss.long()], rff_ref(W2).cpu().numpy(), REL_EF, "another tensor")
+    del W2
+    gc.collect()
+    assert len(ops._PRESPLIT) == nkeys                # the dead tensor's entry is gone
+
+    rep = torch.randn(A, R, device=dev(), generator=g)
+    red = torch.randn(ne, R, d, device=dev(), generator=g)
+    gx = torch.randn(A, d, device=dev(), generator=g)
+
+    def bwd_ref(U):
+        return torch.einsum('ad,ard->ar', gx.double(), U.double()[types.long()[ss.long()]])
+    for scale in (1.0, -0.25):
+        if scale != 1.0:
+            red.mul_(scale)
+        gr = ops.project_typed_backward(gx, ss, off, red, types, A)      # beyond the small-batch kernels: prepared form
+        close(gr[ss.long()], bwd_ref(red).cpu().numpy(), REL_REP, "transposed projection, reductors x %g" % scale)
+        xs = ops.project_typed(rep, ss, off, red)
+        ref = torch.einsum('ar,ard->ad', rep[ss.long()].double(), red.double()[types.long()[ss.long()]])
+        close(xs, ref.cpu().numpy(), REL_REP, "projection, reductors x %g" % scale)
