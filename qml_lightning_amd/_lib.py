@@ -62,7 +62,7 @@ PROTOTYPES = {
     "qmll_project_typed": [P, P, P, P, P, c_int, c_int, c_int, c_int, P, P],
     "qmll_project_typed_rows": [P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
     "qmll_project_typed_backward": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
-    "qmll_sorf_energy_sorted": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_float, P, P, P],
+    "qmll_sorf_energy_sorted": [P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_float, P, P, P],
     "qmll_rff_features": [P, P, P, P, c_int, c_int, c_int, c_int, P, P],
     "qmll_rff_derivative_features": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
     "qmll_rff_presplit_bytes": [c_int, c_int, c_int],

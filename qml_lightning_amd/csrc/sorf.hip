@@ -14,6 +14,8 @@
 // Two-op contract (coefficients materialised, [A,S,d] fp32): both ops are HBM bound,
 // 4d + 4Sd bytes per atom forward.  The fused kernel keeps coefficients in registers and is
 // VALU bound (one sincos per feature).
+#include <type_traits>
+
 #include "qmll_common.h"
 
 namespace {
@@ -595,8 +597,9 @@ constexpr int ROWS_NA = 4;   // atoms per workgroup = rows of 16 lanes per wavef
 template <int LOG2D, bool WITH_GRAD, bool MULTI, int NW = SORF_WAVES>
 __global__ __launch_bounds__(64 * NW) void sorf_energy_rows_kernel(
     const float* __restrict__ x, const float* __restrict__ D, const float* __restrict__ bias,
-    const float* __restrict__ alpha, const int* __restrict__ out_index, const int* __restrict__ type_offsets, int ne,
-    int A, int S, int T_, float scale, float normf, float* __restrict__ e_atom, float* __restrict__ gx) {
+    const float* __restrict__ alpha, const float* __restrict__ bias_absmax, const int* __restrict__ out_index,
+    const int* __restrict__ type_offsets, int ne, int A, int S, int T_, float scale, float normf,
+    float* __restrict__ e_atom, float* __restrict__ gx) {
     const int T = MULTI ? T_ : 1;
     constexpr int d = 1 << LOG2D;
     constexpr int EPL = d / 16;                 // registers per lane
@@ -681,7 +684,20 @@ __global__ __launch_bounds__(64 * NW) void sorf_energy_rows_kernel(
         // Cody-Waite reduction in front (5e-7 at |arg| ~ 16, 2e-6 at ~100).  Beyond 1500 radians the
         // whole revolutions are taken off first: u - rint(u) is exact in fp32.
         constexpr float UMAX = 1500.0f * INV2PI;
-        auto stack = [&](const float (&dcur)[EPL], const float (&bv)[EPL], const float (&av)[EPL]) {
+        // Every coefficient of an atom is bounded by sum_q |x_q| (the butterflies only add and subtract)
+        // plus the largest |bias| (a constant of the model, handed in when the caller knows it): where
+        // that bound stays below UMAX for the four atoms of the wavefront, which is the rule, no stack
+        // needs to look at its arguments.  Without the bias bound every stack checks them.
+        bool track = true;
+        if (bias_absmax != nullptr) {
+            float bound = 0.0f;
+#pragma unroll
+            for (int p = 0; p < EPL; ++p) bound += fabsf(xv[p]);
+            bound = fmaf(*bias_absmax, INV2PI, row_sum(bound));
+            track = __any(!(bound <= UMAX));       // a NaN bound keeps the checks
+        }
+        auto stack = [&](auto tracked, const float (&dcur)[EPL], const float (&bv)[EPL], const float (&av)[EPL]) {
+            constexpr bool TRACK = decltype(tracked)::value;
             float v[EPL];
 #pragma unroll
             for (int p = 0; p < EPL; ++p) v[p] = xv[p] * dcur[p];
@@ -691,7 +707,7 @@ __global__ __launch_bounds__(64 * NW) void sorf_energy_rows_kernel(
 #pragma unroll
             for (int p = 0; p < EPL; ++p) {
                 u[p] = fmaf(bv[p], csig, v[p]);
-                umax = fmaxf(umax, fabsf(u[p]));
+                if constexpr (TRACK) umax = fmaxf(umax, fabsf(u[p]));
             }
 #pragma unroll
             for (int p = 0; p < EPL; ++p) {
@@ -699,15 +715,17 @@ __global__ __launch_bounds__(64 * NW) void sorf_energy_rows_kernel(
                 energy = fmaf(av[p], cs_, energy);
                 v[p] = av[p] * sn;                           // sigma * (-(d E / d coefficient) / normf)
             }
-            if (__builtin_expect(__any(umax > UMAX), 0)) {
+            if constexpr (TRACK) {
+                if (__builtin_expect(__any(umax > UMAX), 0)) {
 #pragma unroll
-                for (int p = 0; p < EPL; ++p) {
-                    if (fabsf(u[p]) > UMAX) {
-                        const float c0_ = __builtin_amdgcn_cosf(u[p]);
-                        const float ur = u[p] - rintf(u[p]);
-                        const float sn = __builtin_amdgcn_sinf(ur), cs_ = __builtin_amdgcn_cosf(ur);
-                        energy += av[p] * (cs_ - c0_);
-                        v[p] = av[p] * sn;
+                    for (int p = 0; p < EPL; ++p) {
+                        if (fabsf(u[p]) > UMAX) {
+                            const float c0_ = __builtin_amdgcn_cosf(u[p]);
+                            const float ur = u[p] - rintf(u[p]);
+                            const float sn = __builtin_amdgcn_sinf(ur), cs_ = __builtin_amdgcn_cosf(ur);
+                            energy += av[p] * (cs_ - c0_);
+                            v[p] = av[p] * sn;
+                        }
                     }
                 }
             }
@@ -721,30 +739,36 @@ __global__ __launch_bounds__(64 * NW) void sorf_energy_rows_kernel(
         // two stacks per round with the sign diagonals in two register sets that swap roles: the
         // diagonal of a stack is fetched one stack ahead (it is the first thing a stack needs),
         // bias and alpha at the start of their own stack (needed after the transform)
-        float d0[EPL], d1[EPL];
-        int s = wave;
-        if (s < S) load_row<EPL>(d0, D + (size_t)s * d + e0);
-        while (s < S) {
-            {
-                float bv[EPL], av[EPL];
-                const size_t off = (size_t)s * d + e0;               // the same for the four rows
-                load_row<EPL>(bv, bias + off);
-                load_row<EPL>(av, alpha + off);
-                load_row<EPL>(d1, D + (size_t)(s + NW < S ? s + NW : s) * d + e0);
-                stack(d0, bv, av);
+        auto stacks = [&](auto tracked) {
+            float d0[EPL], d1[EPL];
+            int s = wave;
+            if (s < S) load_row<EPL>(d0, D + (size_t)s * d + e0);
+            while (s < S) {
+                {
+                    float bv[EPL], av[EPL];
+                    const size_t off = (size_t)s * d + e0;               // the same for the four rows
+                    load_row<EPL>(bv, bias + off);
+                    load_row<EPL>(av, alpha + off);
+                    load_row<EPL>(d1, D + (size_t)(s + NW < S ? s + NW : s) * d + e0);
+                    stack(tracked, d0, bv, av);
+                }
+                s += NW;
+                if (s >= S) break;
+                {
+                    float bv[EPL], av[EPL];
+                    const size_t off = (size_t)s * d + e0;
+                    load_row<EPL>(bv, bias + off);
+                    load_row<EPL>(av, alpha + off);
+                    load_row<EPL>(d0, D + (size_t)(s + NW < S ? s + NW : s) * d + e0);
+                    stack(tracked, d1, bv, av);
+                }
+                s += NW;
             }
-            s += NW;
-            if (s >= S) break;
-            {
-                float bv[EPL], av[EPL];
-                const size_t off = (size_t)s * d + e0;
-                load_row<EPL>(bv, bias + off);
-                load_row<EPL>(av, alpha + off);
-                load_row<EPL>(d0, D + (size_t)(s + NW < S ? s + NW : s) * d + e0);
-                stack(d1, bv, av);
-            }
-            s += NW;
-        }
+        };
+        if (track)
+            stacks(std::true_type{});
+        else
+            stacks(std::false_type{});
         energy = row_sum(energy);
         if (i16 == 0) ered[wave][row] = energy;
         if constexpr (WITH_GRAD) {
@@ -1591,7 +1615,7 @@ extern "C" int qmll_sorf_adjoint(const float* g, const float* D, int A, int d, i
 }
 
 static int launch_fused(const char* who, const float* x, const float* D, const float* bias, const float* alpha,
-                        const int* out_index, const int* types, const int* type_offsets, int ne, int A, int d, int S,
+                        const float* bias_absmax, const int* out_index, const int* types, const int* type_offsets, int ne, int A, int d, int S,
                         int T, float normalisation, float* e_atom, float* gx, hipStream_t stream) {
     const float scale = normalisation * hnorm(d, T);
     const float normf = sqrtf(2.0f / ((float)S * (float)d));
@@ -1608,10 +1632,10 @@ static int launch_fused(const char* who, const float* x, const float* D, const f
     if (few && !(M))                                                                                               \
         hipLaunchKernelGGL((sorf_energy_rows_kernel<L, G, false, ((L) <= 7 ? 16 : SORF_WAVES)>), grid, dim3(1024), \
                            0, stream, x, D, bias,                                                                  \
-                           alpha, out_index, type_offsets, ne, A, S, T, scale, normf, e_atom, gx);                 \
+                           alpha, bias_absmax, out_index, type_offsets, ne, A, S, T, scale, normf, e_atom, gx);    \
     else                                                                                                           \
         hipLaunchKernelGGL((sorf_energy_rows_kernel<L, G, M>), grid, dim3(SORF_THREADS), 0, stream, x, D, bias,    \
-                           alpha, out_index, type_offsets, ne, A, S, T, scale, normf, e_atom, gx)
+                           alpha, bias_absmax, out_index, type_offsets, ne, A, S, T, scale, normf, e_atom, gx)
 #define CALL_ROWS(L)                                    \
     if (gx && T == 1) { LAUNCH_ROWS(L, true, false); }  \
     else if (gx) { LAUNCH_ROWS(L, true, true); }        \
@@ -1648,7 +1672,7 @@ extern "C" int qmll_sorf_energy_fused(const float* x, const float* D, const floa
     if (rc) return rc;
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(x && D && bias && alpha && e_atom, QMLL_ERR_INVALID, "qmll_sorf_energy_fused: null pointer");
-    return launch_fused("qmll_sorf_energy_fused", x, D, bias, alpha, out_index, nullptr, nullptr, 1, A, d, S, T, normalisation,
+    return launch_fused("qmll_sorf_energy_fused", x, D, bias, alpha, nullptr, out_index, nullptr, nullptr, 1, A, d, S, T, normalisation,
                         e_atom, gx, (hipStream_t)stream);
 }
 
@@ -1661,20 +1685,20 @@ extern "C" int qmll_sorf_energy_typed(const float* x_all, const int* types, cons
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(x_all && types && atom_slots && D && bias && alpha && e_slots, QMLL_ERR_INVALID,
                  "qmll_sorf_energy_typed: null pointer");
-    return launch_fused("qmll_sorf_energy_typed", x_all, D, bias, alpha, atom_slots, types, nullptr, ne, A, d, S, T,
+    return launch_fused("qmll_sorf_energy_typed", x_all, D, bias, alpha, nullptr, atom_slots, types, nullptr, ne, A, d, S, T,
                         normalisation, e_slots, gx_all, (hipStream_t)stream);
 }
 
 extern "C" int qmll_sorf_energy_sorted(const float* x, const int* type_offsets, const int* sorted_slots, const float* D,
-                                       const float* bias, const float* alpha, int A, int ne, int d, int S, int T,
-                                       float normalisation, float* e_slots, float* gx, qmll_stream_t stream) {
+                                       const float* bias, const float* alpha, const float* bias_absmax, int A, int ne, int d,
+                                       int S, int T, float normalisation, float* e_slots, float* gx, qmll_stream_t stream) {
     int rc = check_sorf("qmll_sorf_energy_sorted", A, d, S, T);
     if (rc) return rc;
     QMLL_REQUIRE(ne > 0, QMLL_ERR_INVALID, "qmll_sorf_energy_sorted: bad size ne=%d", ne);
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(x && type_offsets && sorted_slots && D && bias && alpha && e_slots, QMLL_ERR_INVALID,
                  "qmll_sorf_energy_sorted: null pointer");
-    return launch_fused("qmll_sorf_energy_sorted", x, D, bias, alpha, sorted_slots, nullptr, type_offsets, ne, A, d, S, T,
+    return launch_fused("qmll_sorf_energy_sorted", x, D, bias, alpha, bias_absmax, sorted_slots, nullptr, type_offsets, ne, A, d, S, T,
                         normalisation, e_slots, gx, (hipStream_t)stream);
 }
 

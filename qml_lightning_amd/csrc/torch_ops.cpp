@@ -538,7 +538,9 @@ std::tuple<Tensor, Tensor> sorf_energy_sorted_impl(const Tensor& x_, const Tenso
                 " elements and ", S * d, " features");
     Tensor e = e_zeroed.defined() ? e_zeroed : at::zeros({nslots}, x.options());
     Tensor gx = with_grad ? at::empty({A, d}, x.options()) : empty_like_none(x);
-    check(qmll_sorf_energy_sorted(fp(x), ip(off), ip(ss), fp(DD), fp(bb), fp(al), A, ne, d, S, T, scalar(cn),
+    // the largest |bias|, a constant of the model: computed once per tensor version, kept on the device
+    Tensor bmax = prepared_form(bb, 2, [](const Tensor& b) { return b.abs().max().reshape({1}); });
+    check(qmll_sorf_energy_sorted(fp(x), ip(off), ip(ss), fp(DD), fp(bb), fp(al), fp(bmax), A, ne, d, S, T, scalar(cn),
                                   nslots ? e.data_ptr<float>() : nullptr, with_grad && A ? gx.data_ptr<float>() : nullptr,
                                   stream()),
           "qmll_sorf_energy_sorted");

@@ -514,9 +514,11 @@ def sorf_energy_sorted(x, type_offsets, sorted_slots, Dmat, bias, alpha, normali
                            % (tuple(bias.shape), alpha.numel(), ne, S * d))
     e_slots = torch.zeros(int(nslots), dtype=torch.float32, device=x.device)
     gx = torch.empty((A, d), dtype=torch.float32, device=x.device) if with_grad else None
+    # the largest |bias|, a constant of the model, computed once per tensor version and left on the device
+    bmax = presplit_cached(bias, "absmax", lambda t: t.abs().max().reshape(1))
     check(_lib.lib().qmll_sorf_energy_sorted(_ptr(x), _ptr(type_offsets), _ptr(sorted_slots), _ptr(Dmat), _ptr(bias),
-                                             _ptr(alpha), A, ne, d, S, T, float(normalisation), _ptr(e_slots), _ptr(gx),
-                                             _stream()), "qmll_sorf_energy_sorted")
+                                             _ptr(alpha), _ptr(bmax), A, ne, d, S, T, float(normalisation), _ptr(e_slots),
+                                             _ptr(gx), _stream()), "qmll_sorf_energy_sorted")
     return e_slots, gx
 
 

@@ -403,6 +403,35 @@ def test_fused_energy_large_arguments(d):
         close(gx[a_], gx_ref[a_], REL_EF, "fused gradient, |arg| up to %.0f" % np.abs(arg[a_]).max())
 
 
+@pytest.mark.parametrize("bias_scale", [1.0, 500.0])
+def test_sorted_fused_energy_with_the_bias_bound_equals_the_checked_form(bias_scale):
+    """The element-sorted entry gets the largest |bias| and decides once per atom, from sum |x| and that
+    bound, whether any argument can leave the range the sine / cosine unit reduces itself; the
+    unsorted entry inspects every argument.  Atoms with small and with huge coefficients side by side
+    (the decision is per wavefront of four atoms), and a bias of thousands of radians: same results."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(11)
+    d, S, A = 128, 6, 37
+    F = S * d
+    x = rng.normal(size=(A, d)).astype(np.float32)
+    x[5] *= 400.0                      # arguments of thousands of radians in the middle of a tile
+    x[20:24] *= 3000.0                 # a whole wavefront beyond the range
+    x[30] = 0.0
+    D = np.where(rng.uniform(-1, 1, (1, 1, S, d)) > 0, 1.0, -1.0).astype(np.float32)
+    b = (rng.uniform(0, 2 * np.pi, (1, F)) * bias_scale).astype(np.float32)
+    alpha = rng.normal(size=F).astype(np.float32)
+    types = np.zeros(A, dtype=np.int32)
+    ss, off = ops.sort_by_type(ti32(types), ti32(np.arange(A, dtype=np.int32)), 1)
+    e_ref = torch.zeros(A, device=dev())
+    g_ref = ops.sorf_energy_fused(t32(x), t32(D[0]), t32(b[0]), t32(alpha), None, 2.5, 1, e_ref)
+    e, g = ops.sorf_energy_sorted(t32(x), off, ss, t32(D), t32(b), t32(alpha), 2.5, 1, A)
+    # the two entries run the same arithmetic per atom (the compiler may contract the two instances of
+    # the stack differently: last bits); only the decision differs
+    assert (e - e_ref).abs().max() <= 1e-6 * e_ref.abs().max()
+    for a_ in range(A):                # per atom: the gradient scales differ by orders of magnitude
+        assert (g[a_] - g_ref[a_]).abs().max() <= 2e-6 * g_ref[a_].abs().max() + 1e-30, a_
+
+
 def test_typed_fused_energy_matches_per_element_calls():
     """All elements in one launch == one fused call per element (slots, padded rows, unknown types)."""
     from qml_lightning_amd import ops
