@@ -191,6 +191,36 @@ def other_configs(torch, dev):
     m5.alpha = torch.tensor(alpha, device=dev)
     m5.is_trained = True
     r5 = predict_rate(m5, coords, charges, True)
+    # the fused RFF kernel of that step alone (HIP events on the launch stream), against the pipe it runs on
+    from qml_lightning_amd import ops
+    d5 = m5.format_data([c.astype(np.float32) for c in coords], charges)
+    prm5 = ops.make_params(len(SPECIES), rep.Rs2, rep.Rs3, rep.eta2, rep.eta3, rep.two_body_decay, rep.three_body_weight,
+                           rep.three_body_decay, rep.rcut)
+    t5 = ops.element_types(d5['coordinates'], d5['charges'], d5['natom_counts'], rep.species)
+    rep5 = ops.fchl_forward(d5['coordinates'], t5, None, None, d5['atomIDs'], d5['molIDs'], d5['natom_counts'], rep.Rs2,
+                            rep.Rs3, prm5)
+    B5, n5 = d5['charges'].shape
+    ss5, off5 = ops.sort_atoms_by_type(t5, d5['atomIDs'], d5['molIDs'], n5, len(SPECIES))
+    x5 = ops.project_typed(rep5.view(B5 * n5, -1), ss5, off5, m5.reductors)
+    a5 = m5.alpha.float()
+    for _ in range(2):
+        ops.rff_energy_sorted(x5, off5, ss5, m5.W, m5.b, a5, B5 * n5)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(5):
+        ops.rff_energy_sorted(x5, off5, ss5, m5.W, m5.b, a5, B5 * n5)
+    ev1.record()
+    torch.cuda.synchronize()
+    t_rff = ev0.elapsed_time(ev1) / 5 * 1e-3
+    fl5 = 4.0 * x5.shape[0] * x5.shape[1] * m5.nfeatures()          # x.W and its transpose product
+    r5["rff_energy_sorted_kernel"] = {
+        "seconds": t_rff, "bound": "mfma",
+        "pipe": "fp16 matrix cores (v_mfma_f32_32x32x16_f16), fp32 operands split in two fp16 parts (W once per model, x and "
+                "the sine factors in the kernel), fp32 accumulation",
+        "TFLOPs": fl5 / t_rff / 1e12, "executed_TFLOPs": 3.0 * fl5 / t_rff / 1e12, "peak_TFLOPs": FP16_PEAK_TFLOPS,
+        "frac": 3.0 * fl5 / t_rff / 1e12 / FP16_PEAK_TFLOPS}
+    del d5, rep5, x5
     r5.update(ztz_seconds(m5, [c.astype(np.float32) for c in coords[:NMOL_TRAIN]], charges[:NMOL_TRAIN], 21))
     out["config5_rff_32768"] = r5
     del m5
@@ -333,7 +363,7 @@ def main():
         "ns_per_instruction": {"plain_fp32": best["plain_fp32_x128"] / 128 * 1e9, "dpp_fmac": best["dpp_fmac_x128"] / 128 * 1e9,
                                "transcendental": best["transcendental_x128"] / 128 * 1e9},
         "fused_kernel_stack_ns": best["fused_kernel_stack"] * 1e9,
-        "note": "one iteration of fused_kernel_stack = 92 plain + 64 DPP + 16 transcendental wavefront instructions = one "
+        "note": "one iteration of fused_kernel_stack = 82 plain + 64 DPP + 16 transcendental wavefront instructions = one "
                 "stack of four atoms at 128 components",
     }
     torch.cuda.empty_cache()
@@ -508,11 +538,11 @@ def main():
     # fused kernel, algorithmic flops per atom: forward+adjoint butterflies 2*F*log2(d), D multiplies 2F,
     # scale+bias FMA 2F, one sin and one cos per feature 2F, energy FMA 2F, alpha*norm*sin 2F
     fused_flops = A * F * (2 * log2d + 10)
-    # 172 vector instructions per wavefront and stack in the kernel's main loop at d = 128 (8 coefficients
-    # per lane; counted in its ISA): 92 plain fp32, 64 DPP butterflies, 8 v_sin_f32 + 8 v_cos_f32
+    # 162 vector instructions per wavefront and stack in the kernel's main loop at d = 128 (8 coefficients
+    # per lane; counted in its ISA): 82 plain fp32, 64 DPP butterflies, 8 v_sin_f32 + 8 v_cos_f32
     kernels["sorf_energy_fused"] = {"seconds": t_fused, "bound": "valu", "TFLOPs": fused_flops / t_fused / 1e12,
                                     "sincos_per_s": A * F / t_fused,
-                                    "valu_wave_instr_per_s": 172.0 / 8.0 * A * F / 64 / t_fused}
+                                    "valu_wave_instr_per_s": 162.0 / 8.0 * A * F / 64 / t_fused}
     # the two-operator contract, kernel by kernel: `seconds` and the bytes are those of ONE launch, the
     # element with the most atoms (the launch the profiler's per-dispatch counters describe);
     # `seconds_all_elements` sums the launches of the three elements of one step
@@ -660,7 +690,7 @@ def main():
                             "flop per sin and per cos and per butterfly add, while a butterfly across lanes issues "
                             "at half rate and v_sin/v_cos at quarter rate, none of them an FMA, so the fraction of "
                             "the fp32 FMA peak understates it: frac_of_instruction_mix is the time a probe kernel needs for the "
-                            "bare instruction mix of one wavefront-stack (92 plain + 64 DPP + 16 transcendental, independent "
+                            "bare instruction mix of one wavefront-stack (82 plain + 64 DPP + 16 transcendental, independent "
                             "registers, no memory access) over the kernel's own time per wavefront-stack, both measured in this run; "
                             "traffic = bytes per launch from profiles/pmc_traffic.json"}
     else:

@@ -454,7 +454,7 @@ double qmll_probe_rate(int which, int iters, int blocks_per_cu, void* out, qmll_
 
 /* Straight-line loops of the instruction classes the fused SORF kernel issues, on independent
  * registers: mix = 0 128 plain fp32, 1 128 DPP fmac, 2 128 v_sin_f32, 3 the per-stack mix of the
- * fused kernel at 128 components (92 plain + 64 DPP + 16 transcendental).
+ * fused kernel at 128 components (82 plain + 64 DPP + 16 transcendental).
  * Returns wavefront-iterations per SIMD (blocks_per_cu x iters), so
  * duration x clock / that = SIMD clocks per iteration; negative on error. */
 double qmll_probe_mix(int mix, int iters, int blocks_per_cu, void* out, qmll_stream_t stream);

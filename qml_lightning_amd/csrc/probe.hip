@@ -132,7 +132,7 @@ __global__ __launch_bounds__(PT) void probe_exp_kernel(int iters, float* __restr
 // Straight-line loops of the instruction classes the fused SORF kernel issues, alone and mixed,
 // on independent registers: what a wavefront instruction of each class costs a SIMD.  One
 // iteration of MIX_FUSED stands for one stack of one wavefront of that kernel at 128 components
-// (8 registers per lane, four atoms per wavefront): 92 plain fp32 + 64 DPP fmac + 16
+// (8 registers per lane, four atoms per wavefront): 82 plain fp32 + 64 DPP fmac + 16
 // transcendental instructions, counted in its ISA.
 enum { MIX_PLAIN = 0, MIX_DPP = 1, MIX_TRANS = 2, MIX_FUSED = 3, MIX_COUNT = 4 };
 
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(PT) void probe_mix_kernel(int iters, float* __restr
             // adjoint: register stages, in-row stages, accumulate
             plain_ops<28>(v, c);
             dpp_ops<32>(v, c);
-            plain_ops<18>(v, c);
+            plain_ops<8>(v, c);
             trans_ops<16>(v);
             plain_ops<18>(v, c);
             dpp_ops<32>(v, c);
