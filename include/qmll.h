@@ -397,7 +397,10 @@ int qmll_gram_upper_f64(const double* Z, const double* y, int M, int F, double* 
  * the slots, the partial tiles go to the workspace and are added in a fixed order, so the result
  * stays deterministic (it differs from qmll_gram_upper_f64 by the rounding of that regrouping).
  * With workspace NULL, fewer bytes, fewer than 2048 rows or a well-filled last round it is
- * qmll_gram_upper_f64. */
+ * qmll_gram_upper_f64.  The number of slots, and with it whether and how the last tiles are cut, follows
+ * from the device's CU count (hipDeviceAttributeMultiprocessorCount): results are reproducible
+ * from run to run on one device model, and equal up to that regrouping's rounding (1e-16 relative)
+ * between device models or between calls with and without a workspace. */
 size_t qmll_gram_workspace_bytes(void);
 int qmll_gram_upper_ws_f64(const double* Z, const double* y, int M, int F, double* ZTZ, double* ZTy,
                            double* workspace, size_t workspace_bytes, qmll_stream_t stream);

@@ -549,6 +549,17 @@ __global__ __launch_bounds__(PT) __attribute__((amdgpu_waves_per_eu(3))) void ty
         float ma = max4(max4(max4(max4(0.0f, ra[0][0]), ra[0][1]), ra[1][0]), ra[1][1]);
 #pragma unroll
         for (int o = 32; o >= 1; o >>= 1) ma = fmaxf(ma, __shfl_xor(ma, o, 64));
+        if (__builtin_expect(not_finite(ma), 0)) {       // an infinity among the rows: the largest finite entry
+            ma = 0.0f;
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+                for (int e = 0; e < 2; ++e)
+                    ma = fmaxf(fmaxf(fmaxf(ma, finite_abs(ra[s2][e].x)), fmaxf(finite_abs(ra[s2][e].y), finite_abs(ra[s2][e].z))),
+                               finite_abs(ra[s2][e].w));
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) ma = fmaxf(ma, __shfl_xor(ma, o, 64));
+        }
         const int ka = scale_exponent(ma);
         const float sa = pow2i(ka);
         half8_t ahv[2], alv[2];
@@ -659,6 +670,15 @@ __global__ __launch_bounds__(PT) void typed_gemm_bt_rows_f16_kernel(const float*
         }
 #pragma unroll
         for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        if (__builtin_expect(not_finite(m), 0)) {        // an infinity among the rows: the largest finite entry
+            m = 0.0f;
+#pragma unroll
+            for (int j = 0; j < KS; ++j)
+#pragma unroll
+                for (int q = 0; q < 8; ++q) m = fmaxf(m, finite_abs(av[j][q]));
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        }
         const int ka = scale_exponent(m);
         const float sa = pow2i(ka);
         inv_sa = pow2i(-ka);

@@ -156,6 +156,15 @@ __device__ __forceinline__ void split_f16(float v, _Float16& hi, _Float16& lo) {
     lo = (_Float16)(v - (float)hi);
 }
 
+// |v| for finite v, 0 for an infinity or a NaN: the operand scales below are taken from the largest
+// FINITE entry, so that a non-finite entry spoils its own row only (its parts become Inf / NaN) and
+// not the rows that share its scale (which an infinite maximum would scale down to nothing)
+__device__ __forceinline__ float finite_abs(float v) {
+    const float a = fabsf(v);
+    return a <= 3.4028234663852886e38f ? a : 0.0f;
+}
+__device__ __forceinline__ bool not_finite(float m) { return !(m <= 3.4028234663852886e38f); }
+
 // 2^k with k clamped to what a float holds
 __device__ __forceinline__ float pow2i(int k) { return __int_as_float((min(max(k, -126), 127) + 127) << 23); }
 

@@ -384,6 +384,15 @@ __global__ __launch_bounds__(RE_T) __attribute__((amdgpu_waves_per_eu(2))) void 
         }
 #pragma unroll
         for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        if (__builtin_expect(not_finite(m), 0)) {        // an infinity among the rows: the largest finite entry
+            m = 0.0f;
+#pragma unroll
+            for (int j = 0; j < KS; ++j)
+#pragma unroll
+                for (int q = 0; q < 8; ++q) m = fmaxf(m, finite_abs(xv[j][q]));
+#pragma unroll
+            for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        }
         const int kx = scale_exponent(m);
         const float sx = pow2i(kx);
         inv_sx = pow2i(-kx);

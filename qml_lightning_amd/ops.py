@@ -648,6 +648,21 @@ def gram_mirror(ZTZ):
     return ZTZ
 
 
+_GRAM_WS = {}
+
+
+def _gram_workspace(device):
+    """The Gram kernel's workspace for the split last round of tiles: one buffer per device and
+    stream, kept between calls (calls on one stream are ordered; calls that may overlap on a device
+    must not share a workspace)."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), _stream().value)
+    ws = _GRAM_WS.get(key)
+    if ws is None:
+        ws = torch.empty(int(_lib.lib().qmll_gram_workspace_bytes()) // 8, dtype=torch.float64, device=device)
+        _GRAM_WS[key] = ws
+    return ws
+
+
 def gram(Zrows, y, ZTZ, ZTy, f0=None, f1=None, mirror=True):
     """ZTZ += Z^T Z (or the row block f0:f1 of it), ZTy += Z^T y, fp64, in place.
     mirror=False (full matrix only) accumulates just the tiles on or above the diagonal: a
@@ -662,11 +677,8 @@ def gram(Zrows, y, ZTZ, ZTy, f0=None, f1=None, mirror=True):
             raise RuntimeError("targets have %d rows, features have %d" % (yv.shape[0], M))
     zty = ZTy if ZTy is not None else None
     if f0 is None:
-        # with a workspace the last, sparsely filled round of tiles is split over the idle CUs (the
-        # buffer comes from torch's caching allocator, which keeps its reuse ordered per stream)
-        ws = None
-        if M >= 2048:
-            ws = torch.empty(int(_lib.lib().qmll_gram_workspace_bytes()) // 8, dtype=torch.float64, device=Zrows.device)
+        # with a workspace the last, sparsely filled round of tiles is split over the idle CUs
+        ws = _gram_workspace(Zrows.device) if M >= 2048 else None
         check(_lib.lib().qmll_gram_upper_ws_f64(_ptr(Zrows), _ptr(yv), M, F, _ptr(ZTZ), _ptr(zty), _ptr(ws),
                                                 ws.numel() * 8 if ws is not None else 0, _stream()),
               "qmll_gram_upper_ws_f64")

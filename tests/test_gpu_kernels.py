@@ -1012,3 +1012,41 @@ def test_prepared_model_constants_follow_their_tensors():
         xs = ops.project_typed(rep, ss, off, red)
         ref = torch.einsum('ar,ard->ad', rep[ss.long()].double(), red.double()[types.long()[ss.long()]])
         close(xs, ref.cpu().numpy(), REL_REP, "projection, reductors x %g" % scale)
+
+
+def test_a_non_finite_row_spoils_only_itself_in_the_fp16_matrix_core_kernels():
+    """The projection kernels on the fp16 matrix cores and the fused RFF kernel scale the 32 rows of a
+    wavefront by one power of two taken from their largest FINITE entry: a row holding an infinity (or
+    a NaN) comes out non-finite, the rows beside it are unchanged."""
+    from qml_lightning_amd import ops
+    g = torch.Generator(device=dev()).manual_seed(9)
+    A, R, d, ne, F = 2304, 312, 128, 2, 256
+    types = torch.arange(A, device=dev(), dtype=torch.int32) % ne
+    ss, off = ops.sort_by_type(types, torch.arange(A, device=dev(), dtype=torch.int32), ne)
+    red = torch.randn(ne, R, d, device=dev(), generator=g)
+    gx = torch.randn(A, d, device=dev(), generator=g)
+    clean = ops.project_typed_backward(gx, ss, off, red, types, A)
+    bad = gx.clone()
+    bad[7, 3] = float("inf")
+    bad[40, 100] = float("nan")
+    out = ops.project_typed_backward(bad, ss, off, red, types, A)
+    rows = ss.long()
+    hit = torch.zeros(A, dtype=torch.bool, device=dev())
+    hit[rows[7]] = hit[rows[40]] = True
+    assert not torch.isfinite(out[hit]).all(dim=1).any()
+    assert torch.equal(out[~hit], clean[~hit])
+    x = torch.randn(A, d, device=dev(), generator=g)
+    W = torch.randn(ne, d, F, device=dev(), generator=g) / 8
+    b = torch.rand(ne, F, device=dev(), generator=g) * 6.28
+    alpha = torch.randn(F, device=dev(), generator=g)
+    e0, g0 = ops.rff_energy_sorted(x, off, ss, W, b, alpha, A)
+    xb = x.clone()
+    xb[11, 5] = float("inf")
+    e1, g1 = ops.rff_energy_sorted(xb, off, ss, W, b, alpha, A)
+    keep = torch.ones(A, dtype=torch.bool, device=dev())
+    keep[11] = False
+    assert not torch.isfinite(g1[11]).all()
+    assert (g1[keep] - g0[keep]).abs().max() <= 1e-6 * g0.abs().max()      # feature parts add with fp32 atomics
+    slot_keep = torch.ones(A, dtype=torch.bool, device=dev())
+    slot_keep[rows[11]] = False
+    assert (e1[slot_keep] - e0[slot_keep]).abs().max() <= 1e-6 * e0.abs().max()
