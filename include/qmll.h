@@ -286,8 +286,9 @@ int qmll_reductor_presplit(const float* reductors, int ne, int R, int d, void* r
  * fp32 kernels' in the last bits (1.7e-7 of the row's largest entry against fp64; fp32 matrix
  * instructions: 7.9e-7) and where a row's rounding depends on the largest entry among the 32 rows
  * that share its wavefront: a molecule's projection can change in the last bit with the batch it
- * is in.  Non-finite entries of rep give non-finite (not necessarily equal) results there.
- * Without it every batch takes the fp32 kernels. */
+ * is in.  The shared scale comes from the largest FINITE entry: a row of rep holding an infinity or a
+ * NaN comes out non-finite (not necessarily the values the fp32 kernels give) and leaves the rows
+ * beside it as they are.  Without the prepared form every batch takes the fp32 kernels. */
 int qmll_project_typed(const float* rep, const int* sorted_slots, const int* type_offsets, const float* reductors,
                        const void* reductors_split, int A, int ne, int R, int d, float* x, qmll_stream_t stream);
 
@@ -308,7 +309,8 @@ int qmll_project_typed_rows(const float* rows, const int* sorted_slots, const in
  * that with types != NULL (i32 [N]) the rows of slots whose type is outside [0,ne) are set
  * to zero.  reductors_split as for qmll_project_typed (NULL = fp32 kernels only); the fp16
  * matrix-core kernel (d = 64 or 128, batches beyond the small-batch kernels) scales the 32 gradient
- * rows of a wavefront by one power of two and every row of U by its own. */
+ * rows of a wavefront by one power of two (of their largest finite entry: a non-finite gradient row
+ * spoils its own result only) and every row of U by its own. */
 int qmll_project_typed_backward(const float* gx, const int* sorted_slots, const int* type_offsets,
                                 const float* reductors, const void* reductors_split, const int* types, int A, int N,
                                 int ne, int R, int d, float* g_rep, qmll_stream_t stream);
@@ -370,8 +372,10 @@ int qmll_rff_presplit(const float* W, int ne, int d, int F, void* W_split, size_
  *   -> gx f32 [A,d] = d e / d x (rows beyond type_offsets[ne] zero; NULL = energies only)
  * The products run on the fp16 matrix cores with every fp32 operand as two fp16 parts behind a
  * power-of-two scale (x per 32 atoms, W per chunk, alpha per launch part) and fp32 accumulation:
- * a row's rounding depends on the largest entry among the 32 rows that share its wavefront, and
- * non-finite entries of x, W or alpha give non-finite (not necessarily equal) results. */
+ * a row's rounding depends on the largest finite entry among the 32 rows that share its wavefront;
+ * a row of x holding an infinity or a NaN gives a non-finite energy and gradient for its own atom
+ * only, non-finite entries of W or alpha make every result non-finite (not necessarily the values
+ * fp32 arithmetic gives). */
 int qmll_rff_energy_sorted(const float* x, const int* type_offsets, const int* sorted_slots, const void* W_split,
                            const float* b, const float* alpha, int A, int ne, int d, int F, float* e_slots,
                            float* gx, qmll_stream_t stream);
