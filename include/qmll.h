@@ -100,6 +100,16 @@ int qmll_fchl19_vjp(const float* X, const int* types, const float* cell, const f
                     const qmll_fchl_params* prm, const float* grad_rep, float* grad_X,
                     qmll_stream_t stream);
 
+/* The same with the result scaled: grad_X += scale * J^T grad_rep at no cost (the factor goes into
+ * the gradient row as it is staged).  scale = -1 turns dE/dX into forces in the kernel that forms
+ * them (the reference negates the gradient in a separate elementwise pass,
+ * qml_lightning/models/hadamard_features.py:156-162). */
+int qmll_fchl19_vjp_scaled(const float* X, const int* types, const float* cell, const float* inv_cell,
+                           const int* atomIDs, const int* molIDs, const int* natoms, const int* nlist,
+                           const int* nneigh, int nn_stride, int A, int B, int n, const float* Rs2, const float* Rs3,
+                           const qmll_fchl_params* prm, const float* grad_rep, float scale, float* grad_X,
+                           qmll_stream_t stream);
+
 /* Replaces fchl_gpu.get_fchl_and_derivative / FCHLRepresentationAndDerivativeCuda and
  * FCHLDerivativeCuda (fchl_cuda.cpp:97-167, launchers fchl_cuda_kernel.cu:1848-1883,
  * 1928-1964, kernels :676-1005, :1007-1323).  jac f32 [B,n,n,3,R] with
@@ -267,6 +277,22 @@ int qmll_sort_atoms_by_type(const int* types, const int* atomIDs, const int* mol
 int qmll_sort_by_type_noalloc(const int* types, const int* slots, int A, int ne, int* sorted_slots,
                               int* type_offsets, qmll_stream_t stream);
 
+/* Everything the fused predict chain needs before its first compute kernel, for a padded batch
+ * (Z f32 [B,n], natoms i32 [B], atomIDs / molIDs i32 [A]):
+ *   types i32 [B,n]      <- qmll_element_types(Z, natoms, species[nspecies])
+ *   sort_types i32 [B,n] <- the same by model_species[ne], the element list of the MODEL (its reductor /
+ *                           Dmat / bias rows; qml_lightning/models/hadamard_features.py:99-107 selects
+ *                           atoms over self.elements); model_species NULL: the model goes by `species`
+ *                           (ne = nspecies) and sort_types is not written
+ *   sorted_slots i32 [A], type_offsets i32 [ne+1] <- qmll_sort_atoms_by_type by that index
+ *   zero f32 [zero_count] <- 0 (the arrays the chain accumulates into)
+ * in ONE launch for up to 1024 listed atoms (16 384 slots, 65 536 floats to clear), else as the
+ * separate kernels.  workspace: as for qmll_sort_atoms_by_type (none up to 1024 atoms). */
+int qmll_prepare_batch(const float* Z, const int* natoms, const float* species, int nspecies, const float* model_species,
+                       int ne, const int* atomIDs, const int* molIDs, int B, int n, int A, void* workspace,
+                       size_t workspace_bytes, int* types, int* sort_types, int* sorted_slots, int* type_offsets,
+                       float* zero, size_t zero_count, qmll_stream_t stream);
+
 /* The projection matrices ("reductors", f32 [ne,R,d], qml_lightning/models/kernel.py:28) are constants
  * of a model.  For large batches the two projections below multiply on the fp16 matrix cores with
  * every fp32 operand as two fp16 parts behind power-of-two scales (fp32 accumulation): the
@@ -314,6 +340,18 @@ int qmll_project_typed_rows(const float* rows, const int* sorted_slots, const in
 int qmll_project_typed_backward(const float* gx, const int* sorted_slots, const int* type_offsets,
                                 const float* reductors, const void* reductors_split, const int* types, int A, int N,
                                 int ne, int R, int d, float* g_rep, qmll_stream_t stream);
+
+/* qmll_project_typed_backward and, with energies != NULL, the per-molecule energies of a padded batch
+ * as well: energies[m] = sum_i e_slots[m*n + i] (e_slots f32 [B*n] as written by
+ * qmll_sorf_energy_sorted / qmll_rff_energy_sorted into a zero-filled array; the index_add of
+ * qml_lightning/models/hadamard_features.py:119-121).  The two are independent; for small batches they
+ * share one launch (a single molecule's predict step is a chain of short dependent launches, and each
+ * one less counts), for large ones the sum is a launch of its own.  With A = 0 (and N = 0) only the
+ * sums are formed; they add a molecule's slots in ascending order, the same in both cases. */
+int qmll_project_typed_backward_sums(const float* gx, const int* sorted_slots, const int* type_offsets,
+                                     const float* reductors, const void* reductors_split, const int* types, int A, int N,
+                                     int ne, int R, int d, float* g_rep, const float* e_slots, int B, int n,
+                                     float* energies, qmll_stream_t stream);
 
 /* qmll_sorf_energy_typed on compact element-sorted rows: x f32 [A,d] as written by
  * qmll_project_typed, D f32 [ne,T,S,d], bias f32 [ne,S*d], alpha f32 [S*d].

@@ -40,6 +40,7 @@ PROTOTYPES = {
     "qmll_element_types": [P, P, P, c_int, c_int, c_int, P, P],
     "qmll_fchl19_forward": _FCHL_COMMON + [P, P],
     "qmll_fchl19_vjp": _FCHL_COMMON + [P, P, P],
+    "qmll_fchl19_vjp_scaled": _FCHL_COMMON + [P, c_float, P, P],
     "qmll_fchl19_jacobian": _FCHL_COMMON + [P, P, P],
     "qmll_sorf_forward": [P, P, c_int, c_int, c_int, c_int, c_float, P, P],
     "qmll_sorf_adjoint": [P, P, c_int, c_int, c_int, c_int, c_float, P, P],
@@ -62,6 +63,8 @@ PROTOTYPES = {
     "qmll_project_typed": [P, P, P, P, P, c_int, c_int, c_int, c_int, P, P],
     "qmll_project_typed_rows": [P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
     "qmll_project_typed_backward": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],
+    "qmll_project_typed_backward_sums": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P, c_int, c_int, P, P],
+    "qmll_prepare_batch": [P, P, P, c_int, P, c_int, P, P, c_int, c_int, c_int, P, c_size_t, P, P, P, P, P, c_size_t, P],
     "qmll_sorf_energy_sorted": [P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_float, P, P, P],
     "qmll_rff_features": [P, P, P, P, c_int, c_int, c_int, c_int, P, P],
     "qmll_rff_derivative_features": [P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P],

@@ -56,6 +56,7 @@ struct FchlArgs {
     const float* Rs2;
     const float* Rs3;
     qmll_fchl_params p;
+    float gscale;  // the backward kernel returns gscale * J^T g (folded into the staged gradient row)
 };
 
 constexpr int TCH = 256;      // smallest triple table
@@ -793,16 +794,16 @@ __global__ __launch_bounds__(64) void fchl19_vjp_kernel(FchlArgs a, const float*
 #pragma unroll
     for (int k = 0; k < GREG2; ++k) {
         const int t = lane + QMLL_WAVE * k;
-        if (t < R2) gin2[t] = gr2[k] * frcp(a.Rs2[t - nRs2 * idiv_small(t, nRs2)]);
+        if (t < R2) gin2[t] = gr2[k] * (a.gscale * frcp(a.Rs2[t - nRs2 * idiv_small(t, nRs2)]));
     }
     for (int t = lane + QMLL_WAVE * GREG2; t < R2; t += QMLL_WAVE)
-        gin2[t] = gsrc[t] * frcp(a.Rs2[t - nRs2 * idiv_small(t, nRs2)]);
+        gin2[t] = gsrc[t] * (a.gscale * frcp(a.Rs2[t - nRs2 * idiv_small(t, nRs2)]));
     if (lane < nRs2) slnRs2[lane] = flog(rs2v);
     for (int t = lane + QMLL_WAVE; t < nRs2; t += QMLL_WAVE) slnRs2[t] = flog(a.Rs2[t]);
     for (int t = lane; t < nRs3; t += QMLL_WAVE) {
         const float u = fmaf(sk3, t == lane ? rs3v : a.Rs3[t], -shift);
         sRs3[t] = u;
-        sfac[t] = fast ? fexp2(-u * u) : 1.0f;
+        sfac[t] = a.gscale * (fast ? fexp2(-u * u) : 1.0f);
     }
     __syncthreads();
     // the gradient of the three-body bins per (element pair, radial bin), (cos, sin) parts, times the
@@ -1324,6 +1325,7 @@ int fill_args(FchlArgs& a, const float* X, const int* types, const float* cell, 
     a.Rs2 = Rs2;
     a.Rs3 = Rs3;
     a.p = *prm;
+    a.gscale = 1.0f;
     return QMLL_OK;
 }
 
@@ -1368,10 +1370,20 @@ extern "C" int qmll_fchl19_vjp(const float* X, const int* types, const float* ce
                                const int* nneigh, int nn_stride, int A, int B, int n, const float* Rs2, const float* Rs3,
                                const qmll_fchl_params* prm, const float* grad_rep, float* grad_X,
                                qmll_stream_t stream) {
+    return qmll_fchl19_vjp_scaled(X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, nn_stride, A, B, n, Rs2,
+                                  Rs3, prm, grad_rep, 1.0f, grad_X, stream);
+}
+
+extern "C" int qmll_fchl19_vjp_scaled(const float* X, const int* types, const float* cell, const float* inv_cell,
+                                      const int* atomIDs, const int* molIDs, const int* natoms, const int* nlist,
+                                      const int* nneigh, int nn_stride, int A, int B, int n, const float* Rs2,
+                                      const float* Rs3, const qmll_fchl_params* prm, const float* grad_rep, float scale,
+                                      float* grad_X, qmll_stream_t stream) {
     FchlArgs a;
     int rc = fill_args(a, X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, nn_stride, A, B, n, Rs2, Rs3,
                        prm, "qmll_fchl19_vjp");
     if (rc) return rc;
+    a.gscale = scale;
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(grad_rep && grad_X, QMLL_ERR_INVALID, "qmll_fchl19_vjp: null gradient pointer");
     const int R = prm->nspecies * prm->nRs2 + prm->nspecies * (prm->nspecies + 1) * prm->nRs3;

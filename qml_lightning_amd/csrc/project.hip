@@ -152,6 +152,88 @@ __global__ __launch_bounds__(SORT_SMALL) void type_sort_small_kernel(const int* 
     for (int i = start[ne] + a; i < A; i += SORT_SMALL) sorted[i] = 0;
 }
 
+// index of charge z in a species list, -1 when it is not there (the rule of element_types_kernel)
+__device__ __forceinline__ int species_index(float z, const float* __restrict__ species, int ns) {
+    const int q = (int)z;
+    int t = -1;
+    for (int j = 0; j < ns; ++j)
+        if (q == (int)species[j]) t = j;
+    return t;
+}
+
+// Everything a small padded batch needs before its first compute kernel, in ONE workgroup: the element
+// index of every slot by the representation's species list (and, when the model keeps its own list, by
+// that one too), the listed atoms sorted by the index the model goes by (as type_sort_small_kernel),
+// and a float range set to zero.  Padded slots (beyond natoms of their molecule) get index 0.
+__global__ __launch_bounds__(SORT_SMALL) void prepare_small_kernel(
+    const float* __restrict__ Z, const int* __restrict__ natoms, const float* __restrict__ species, int ns,
+    const float* __restrict__ model_species, int ne, const int* __restrict__ atomIDs, const int* __restrict__ molIDs, int B,
+    int n, int A, int* __restrict__ types, int* __restrict__ sort_types, int* __restrict__ sorted, int* __restrict__ offsets,
+    float* __restrict__ zero, int zero_count) {
+    __shared__ int wcnt[SORT_SMALL / 64][MAXNE];
+    __shared__ int total[MAXNE], start[MAXNE + 1];
+    const int a = threadIdx.x, lane = a & 63, wave = a >> 6;
+    for (int idx = a; idx < B * n; idx += SORT_SMALL) {
+        const int m = idx / n;
+        const bool real = idx - m * n < natoms[m];
+        types[idx] = real ? species_index(Z[idx], species, ns) : 0;
+        if (model_species) sort_types[idx] = real ? species_index(Z[idx], model_species, ne) : 0;
+    }
+    for (int i = a; i < zero_count; i += SORT_SMALL) zero[i] = 0.0f;
+    int slot = 0, t = -1;
+    if (a < A) {
+        const int m = molIDs[a], i = atomIDs[a];
+        slot = m * n + i;
+        t = i < natoms[m] ? (model_species ? species_index(Z[slot], model_species, ne) : species_index(Z[slot], species, ns))
+                          : 0;
+    }
+    int rank = 0;
+    for (int e = 0; e < ne; ++e) {
+        const unsigned long long mk = __ballot(t == e);
+        if (lane == 0) wcnt[wave][e] = __popcll(mk);
+        if (t == e) rank = __popcll(mk & ((1ull << lane) - 1ull));
+    }
+    __syncthreads();
+    if (a < ne) {
+        int sum = 0;
+        for (int w = 0; w < SORT_SMALL / 64; ++w) {
+            const int c = wcnt[w][a];
+            wcnt[w][a] = sum;
+            sum += c;
+        }
+        total[a] = sum;
+    }
+    __syncthreads();
+    if (a == 0) {
+        int sum = 0;
+        for (int e = 0; e < ne; ++e) {
+            start[e] = sum;
+            sum += total[e];
+        }
+        start[ne] = sum;
+    }
+    __syncthreads();
+    if (a <= ne) offsets[a] = start[a];
+    if (t >= 0 && t < ne) sorted[start[t] + wcnt[wave][t] + rank] = slot;
+    for (int i = start[ne] + a; i < A; i += SORT_SMALL) sorted[i] = 0;
+}
+
+__global__ __launch_bounds__(256) void zero_floats_kernel(float* __restrict__ p, size_t count) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (size_t)gridDim.x * 256) p[i] = 0.0f;
+}
+
+// sums[m] = sum_i values[m*n + i]: thread = row (the per-molecule energy of a padded batch)
+__device__ __forceinline__ void row_sums(const float* __restrict__ values, int B, int n, float* __restrict__ sums, int chunk) {
+    const int m = chunk * 256 + threadIdx.x;
+    if (m >= B) return;
+    float acc = 0.0f;
+    for (int i = 0; i < n; ++i) acc += values[(size_t)m * n + i];
+    sums[m] = acc;
+}
+__global__ __launch_bounds__(256) void row_sums_kernel(const float* __restrict__ values, int B, int n, float* __restrict__ sums) {
+    row_sums(values, B, n, sums, blockIdx.x);
+}
+
 // ---- typed GEMM -------------------------------------------------------------------------
 constexpr int PT = 256;            // threads (4 wavefronts, each 32 rows x 64 columns)
 constexpr int PM = 128;            // rows per workgroup
@@ -809,14 +891,21 @@ __global__ __launch_bounds__(256) void project_small_kernel(const float* __restr
 }
 
 // g_rep[slot(p), :] = gx[p, :] . U_e^T: thread = output entry r, its reductor row is contiguous
-// (workgroups past the A atoms zero the rows of slots whose type is outside [0, ne), 256 slots each)
+// (workgroups past the A atoms zero the rows of slots whose type is outside [0, ne), 256 slots each, and
+// after those, when asked, sum the per-slot energies of 256 molecules each)
 __global__ __launch_bounds__(256) void project_bt_small_kernel(const float* __restrict__ gx,
                                                                const int* __restrict__ sorted_slots,
                                                                const int* __restrict__ type_offsets,
                                                                const float* __restrict__ reductors, int ne, int R, int d,
                                                                float* __restrict__ g_rep, int A,
-                                                               const int* __restrict__ types, int N) {
+                                                               const int* __restrict__ types, int N, int zero_groups,
+                                                               const float* __restrict__ e_slots, int B, int n,
+                                                               float* __restrict__ energies) {
     extern __shared__ float sm[];                      // [d]
+    if ((int)blockIdx.x >= A + zero_groups) {          // spare workgroups: the per-molecule energy sums
+        row_sums(e_slots, B, n, energies, (int)blockIdx.x - A - zero_groups);
+        return;
+    }
     if ((int)blockIdx.x >= A) {
         zero_untyped_rows(types, N, ne, R, g_rep, (int)blockIdx.x - A);
         return;
@@ -913,6 +1002,45 @@ extern "C" int qmll_sort_atoms_by_type(const int* types, const int* atomIDs, con
                        slots);
     QMLL_CHECK_LAUNCH("qmll_sort_atoms_by_type");
     return qmll_sort_by_type(types, slots, A, ne, workspace, counts_bytes, sorted_slots, type_offsets, stream);
+}
+
+extern "C" int qmll_prepare_batch(const float* Z, const int* natoms, const float* species, int nspecies,
+                                  const float* model_species, int ne, const int* atomIDs, const int* molIDs, int B, int n,
+                                  int A, void* workspace, size_t workspace_bytes, int* types, int* sort_types,
+                                  int* sorted_slots, int* type_offsets, float* zero, size_t zero_count, qmll_stream_t stream) {
+    QMLL_REQUIRE(B >= 0 && n >= 0 && A >= 0 && nspecies > 0 && ne > 0 && ne <= MAXNE, QMLL_ERR_INVALID,
+                 "qmll_prepare_batch: bad size B=%d n=%d A=%d nspecies=%d ne=%d (at most %d types)", B, n, A, nspecies, ne,
+                 MAXNE);
+    QMLL_REQUIRE(model_species || ne == nspecies, QMLL_ERR_INVALID,
+                 "qmll_prepare_batch: %d model elements for %d species and no model species given", ne, nspecies);
+    QMLL_REQUIRE(type_offsets && species && (zero || zero_count == 0), QMLL_ERR_INVALID, "qmll_prepare_batch: null pointer");
+    QMLL_REQUIRE(!model_species || sort_types || (size_t)B * n == 0, QMLL_ERR_INVALID,
+                 "qmll_prepare_batch: model species without a sort_types output");
+    const size_t slots = (size_t)B * n;
+    if (A > 0 && A <= SORT_SMALL && slots > 0 && slots <= 16384 && zero_count <= 65536) {
+        QMLL_REQUIRE(Z && natoms && atomIDs && molIDs && types && sorted_slots, QMLL_ERR_INVALID,
+                     "qmll_prepare_batch: null pointer");
+        hipLaunchKernelGGL(prepare_small_kernel, dim3(1), dim3(SORT_SMALL), 0, (hipStream_t)stream, Z, natoms, species, nspecies,
+                           model_species, ne, atomIDs, molIDs, B, n, A, types, sort_types, sorted_slots, type_offsets, zero,
+                           (int)zero_count);
+        QMLL_CHECK_LAUNCH("qmll_prepare_batch");
+        return QMLL_OK;
+    }
+    int rc = qmll_element_types(Z, natoms, species, B, n, nspecies, types, stream);
+    if (rc != QMLL_OK) return rc;
+    if (model_species) {
+        rc = qmll_element_types(Z, natoms, model_species, B, n, ne, sort_types, stream);
+        if (rc != QMLL_OK) return rc;
+    }
+    if (zero_count > 0) {
+        const size_t groups = (zero_count + 255) / 256;
+        hipLaunchKernelGGL(zero_floats_kernel, dim3((unsigned)(groups < 4096 ? groups : 4096)), dim3(256), 0,
+                           (hipStream_t)stream, zero, zero_count);
+        QMLL_CHECK_LAUNCH("qmll_prepare_batch");
+    }
+    if (n == 0) n = 1;                        // an empty batch: the sort below only writes the offsets
+    return qmll_sort_atoms_by_type(model_species ? sort_types : types, atomIDs, molIDs, n, A, ne, workspace, workspace_bytes,
+                                   sorted_slots, type_offsets, stream);
 }
 
 // ---- the same sort for callers that cannot allocate -------------------------------------
@@ -1098,8 +1226,18 @@ extern "C" int qmll_project_typed_rows(const float* rows, const int* sorted_slot
 extern "C" int qmll_project_typed_backward(const float* gx, const int* sorted_slots, const int* type_offsets,
                                            const float* reductors, const void* reductors_split, const int* types, int A,
                                            int N, int ne, int R, int d, float* g_rep, qmll_stream_t stream) {
+    return qmll_project_typed_backward_sums(gx, sorted_slots, type_offsets, reductors, reductors_split, types, A, N, ne, R, d,
+                                            g_rep, nullptr, 0, 0, nullptr, stream);
+}
+
+extern "C" int qmll_project_typed_backward_sums(const float* gx, const int* sorted_slots, const int* type_offsets,
+                                                const float* reductors, const void* reductors_split, const int* types,
+                                                int A, int N, int ne, int R, int d, float* g_rep, const float* e_slots,
+                                                int B, int n, float* energies, qmll_stream_t stream) {
     QMLL_REQUIRE(A >= 0 && N >= 0 && ne > 0 && R > 0 && d > 0, QMLL_ERR_INVALID,
                  "qmll_project_typed_backward: bad size A=%d N=%d ne=%d R=%d d=%d", A, N, ne, R, d);
+    const bool sums = energies != nullptr && B > 0;
+    QMLL_REQUIRE(!sums || (e_slots && n > 0), QMLL_ERR_INVALID, "qmll_project_typed_backward_sums: energies without e_slots");
     const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(gx) && aligned16(reductors);
     const bool small = vec && A > 0 && small_batch(A, R, d) && (size_t)d * sizeof(float) <= 64 * 1024 && N <= 256 * 256;
     if (types && N > 0 && !small) {
@@ -1108,15 +1246,22 @@ extern "C" int qmll_project_typed_backward(const float* gx, const int* sorted_sl
                            R, g_rep);
         QMLL_CHECK_LAUNCH("qmll_project_typed_backward");
     }
+    if (sums && !small) {
+        hipLaunchKernelGGL(row_sums_kernel, dim3((B + 255) / 256), dim3(256), 0, (hipStream_t)stream, e_slots, B, n, energies);
+        QMLL_CHECK_LAUNCH("qmll_project_typed_backward_sums");
+    }
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(gx && sorted_slots && type_offsets && reductors && g_rep, QMLL_ERR_INVALID,
                  "qmll_project_typed_backward: null pointer");
     const dim3 grid((A + PM - 1) / PM + ne, (R + PN - 1) / PN);
     if (small) {
-        // one launch: a workgroup per atom, and one per 256 slots for the rows of unknown elements
+        // one launch: a workgroup per atom, one per 256 slots for the rows of unknown elements, one per 256
+        // molecules for the energy sums
         const int zero_groups = (types && N > 0) ? (N + 255) / 256 : 0;
-        hipLaunchKernelGGL(project_bt_small_kernel, dim3(A + zero_groups), dim3(256), sizeof(float) * d, (hipStream_t)stream,
-                           gx, sorted_slots, type_offsets, reductors, ne, R, d, g_rep, A, types, N);
+        const int sum_groups = sums ? (B + 255) / 256 : 0;
+        hipLaunchKernelGGL(project_bt_small_kernel, dim3(A + zero_groups + sum_groups), dim3(256), sizeof(float) * d,
+                           (hipStream_t)stream, gx, sorted_slots, type_offsets, reductors, ne, R, d, g_rep, A, types, N,
+                           zero_groups, e_slots, B, n, energies);
     } else if (vec && (d == 64 || d == 128) && reductors_split) {
         // short contraction: the gradient rows stay in registers, every row is read once
         const SplitLayout L = split_layout(ne, R, d);

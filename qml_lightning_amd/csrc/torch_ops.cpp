@@ -108,7 +108,8 @@ Tensor element_types(const Tensor& X, const Tensor& Z, const Tensor& natoms, con
 FchlInputs prepare(const Tensor& X, const Tensor& Z, const Tensor& species, const Tensor& atomIDs, const Tensor& molIDs,
                    const Tensor& atom_counts, const Tensor& cell, const Tensor& inv_cell, const Tensor& Rs2,
                    const Tensor& Rs3, const Tensor& eta2, const Tensor& eta3, const Tensor& two_body_decay,
-                   const Tensor& three_body_weight, const Tensor& three_body_decay, const Tensor& rcut) {
+                   const Tensor& three_body_weight, const Tensor& three_body_decay, const Tensor& rcut,
+                   bool with_types = true) {
     need_cuda(X, "coordinates");   // torchscript/FCHL19.cpp:251-258
     need_cuda(Z, "charges");
     need_cuda(species, "species");
@@ -120,7 +121,7 @@ FchlInputs prepare(const Tensor& X, const Tensor& Z, const Tensor& species, cons
     FchlInputs in;
     in.X = f32(X.dim() == 2 ? X.unsqueeze(0) : X);   // fchl_cuda.cpp:72-76
     in.natoms = i32(atom_counts);
-    in.types = element_types(in.X, Z, in.natoms, species);
+    if (with_types) in.types = element_types(in.X, Z, in.natoms, species);
     if (cell.numel() > 0) {   // an empty [0,3,3] tensor means no periodic images
         in.cell = f32(cell);
         in.inv_cell = f32(inv_cell);
@@ -153,9 +154,10 @@ FchlInputs prepare(const Tensor& X, const Tensor& Z, const Tensor& species, cons
 #define FCHL_PASS                                                                                                \
     X, Z, species, atomIDs, molIDs, atom_counts, cell, inv_cell, Rs2, Rs3, eta2, eta3, two_body_decay,           \
         three_body_weight, three_body_decay, rcut
-#define FCHL_ABI(in)                                                                                             \
-    fp(in.X), ip(in.types), fp(in.cell), fp(in.inv_cell), ip(in.atomIDs), ip(in.molIDs), ip(in.natoms), nullptr, \
+#define FCHL_ABI_T(in, types)                                                                                \
+    fp(in.X), types, fp(in.cell), fp(in.inv_cell), ip(in.atomIDs), ip(in.molIDs), ip(in.natoms), nullptr,       \
         nullptr, 0, in.A, in.B, in.n, fp(in.Rs2), fp(in.Rs3), &in.prm
+#define FCHL_ABI(in) FCHL_ABI_T(in, ip(in.types))
 
 Tensor fchl_forwards_impl(FCHL_TENSORS) {
     FchlInputs in = prepare(FCHL_PASS);
@@ -521,29 +523,41 @@ Tensor project_typed(const Tensor& rep, const Tensor& ss, const Tensor& off, con
     return ProjectFn::apply(rep, ss, off, red, types);
 }
 
+// the fused SORF kernel on rows x f32 [A,d] of a model (ne elements): shape checks of the model's tensors and the launch;
+// e f32 [nslots] zero-filled, gx f32 [A,d] or nullptr
+void sorf_energy_sorted_raw(const float* x, const int* off, const int* ss, int A, int d_x, int ne_off, const Tensor& Dmat,
+                            const Tensor& bias, const Tensor& alpha, const Tensor& cn, const Tensor& nt, float* e, float* gx) {
+    Tensor DD = f32(Dmat), bb = f32(bias), al = f32(alpha);
+    need_cuda(DD, "Dmat");
+    TORCH_CHECK(DD.dim() == 4, "sorf_energy_sorted: Dmat is [", DD.sizes(), "], expected [elements, transforms, stacks, d]");
+    const int ne = (int)DD.size(0), Tn = (int)DD.size(1), S = (int)DD.size(2), d = (int)DD.size(3);
+    const int T = nt.item<int>();
+    TORCH_CHECK(d_x == d && ne_off == ne, "sorf_energy_sorted: x has ", d_x, " columns and the offsets ", ne_off,
+                " elements, expected ", d, " and ", ne);
+    TORCH_CHECK(T == Tn, "sorf_energy_sorted: ", Tn, " diagonals stored per stack, ", T, " transforms asked for");
+    TORCH_CHECK(bb.dim() == 2 && bb.size(0) == ne && bb.size(1) == (int64_t)S * d && al.numel() == (int64_t)S * d,
+                "sorf_energy_sorted: bias [", bb.sizes(), "] / alpha with ", al.numel(), " entries do not fit ", ne,
+                " elements and ", S * d, " features");
+    // the largest |bias|, a constant of the model: computed once per tensor version, kept on the device
+    Tensor bmax = prepared_form(bb, 2, [](const Tensor& b) { return b.abs().max().reshape({1}); });
+    check(qmll_sorf_energy_sorted(x, off, ss, fp(DD), fp(bb), fp(al), fp(bmax), A, ne, d, S, T, scalar(cn), e, A ? gx : nullptr,
+                                  stream()),
+          "qmll_sorf_energy_sorted");
+}
+
 // e_zeroed: the caller's zero-filled f32 [nslots] for the energies (one fill then serves several outputs), or undefined
 std::tuple<Tensor, Tensor> sorf_energy_sorted_impl(const Tensor& x_, const Tensor& type_offsets, const Tensor& sorted_slots,
                                                    const Tensor& Dmat, const Tensor& bias, const Tensor& alpha,
                                                    const Tensor& cn, const Tensor& nt, int64_t nslots, bool with_grad,
                                                    const Tensor& e_zeroed = Tensor()) {
-    Tensor x = f32(x_), DD = f32(Dmat), bb = f32(bias), al = f32(alpha), off = i32(type_offsets), ss = i32(sorted_slots);
+    Tensor x = f32(x_), off = i32(type_offsets), ss = i32(sorted_slots);
     need_cuda(x, "x");
-    const int ne = (int)DD.size(0), Tn = (int)DD.size(1), S = (int)DD.size(2), d = (int)DD.size(3);
-    const int A = (int)ss.size(0), T = nt.item<int>();
-    TORCH_CHECK(x.size(0) == A && x.size(1) == d && off.size(0) == ne + 1, "sorf_energy_sorted: x is [", x.size(0), ", ",
-                x.size(1), "], expected [", A, ", ", d, "]");
-    TORCH_CHECK(T == Tn, "sorf_energy_sorted: ", Tn, " diagonals stored per stack, ", T, " transforms asked for");
-    TORCH_CHECK(bb.dim() == 2 && bb.size(0) == ne && bb.size(1) == (int64_t)S * d && al.numel() == (int64_t)S * d,
-                "sorf_energy_sorted: bias [", bb.sizes(), "] / alpha with ", al.numel(), " entries do not fit ", ne,
-                " elements and ", S * d, " features");
+    const int A = (int)ss.size(0);
+    TORCH_CHECK(x.dim() == 2 && x.size(0) == A && off.dim() == 1, "sorf_energy_sorted: x is [", x.sizes(), "] for ", A, " atoms");
     Tensor e = e_zeroed.defined() ? e_zeroed : at::zeros({nslots}, x.options());
-    Tensor gx = with_grad ? at::empty({A, d}, x.options()) : empty_like_none(x);
-    // the largest |bias|, a constant of the model: computed once per tensor version, kept on the device
-    Tensor bmax = prepared_form(bb, 2, [](const Tensor& b) { return b.abs().max().reshape({1}); });
-    check(qmll_sorf_energy_sorted(fp(x), ip(off), ip(ss), fp(DD), fp(bb), fp(al), fp(bmax), A, ne, d, S, T, scalar(cn),
-                                  nslots ? e.data_ptr<float>() : nullptr, with_grad && A ? gx.data_ptr<float>() : nullptr,
-                                  stream()),
-          "qmll_sorf_energy_sorted");
+    Tensor gx = with_grad ? at::empty({A, x.size(1)}, x.options()) : empty_like_none(x);
+    sorf_energy_sorted_raw(fp(x), ip(off), ip(ss), A, (int)x.size(1), (int)off.size(0) - 1, Dmat, bias, alpha, cn, nt,
+                           nslots ? e.data_ptr<float>() : nullptr, with_grad ? gx.data_ptr<float>() : nullptr);
     return {e, gx};
 }
 
@@ -582,13 +596,14 @@ std::tuple<Tensor, Tensor> sorf_energy_sorted(const Tensor& x, const Tensor& off
     return {r[0], r[1]};
 }
 
-std::tuple<Tensor, Tensor> rff_energy_sorted_impl(const Tensor& x_, const Tensor& type_offsets, const Tensor& sorted_slots,
-                                                  const Tensor& W, const Tensor& b, const Tensor& alpha, int64_t nslots,
-                                                  bool with_grad, const Tensor& e_zeroed = Tensor()) {
-    Tensor x = f32(x_), WW = f32(W), bb = f32(b), al = f32(alpha), off = i32(type_offsets), ss = i32(sorted_slots);
-    need_cuda(x, "x");
-    const int ne = (int)WW.size(0), d = (int)WW.size(1), F = (int)WW.size(2), A = (int)ss.size(0);
-    TORCH_CHECK(x.size(0) == A && x.size(1) == d && off.size(0) == ne + 1 && bb.size(0) == ne && bb.size(1) == F,
+// the fused RFF kernel on rows x f32 [A,d]: shape checks of the model's tensors and the launch (e zero-filled)
+void rff_energy_sorted_raw(const float* x, const int* off, const int* ss, int A, int d_x, int ne_off, const Tensor& W,
+                           const Tensor& b, const Tensor& alpha, float* e, float* gx) {
+    Tensor WW = f32(W), bb = f32(b), al = f32(alpha);
+    need_cuda(WW, "W");
+    TORCH_CHECK(WW.dim() == 3 && bb.dim() == 2, "rff_energy_sorted: W is [", WW.sizes(), "], b is [", bb.sizes(), "]");
+    const int ne = (int)WW.size(0), d = (int)WW.size(1), F = (int)WW.size(2);
+    TORCH_CHECK(d_x == d && ne_off == ne && bb.size(0) == ne && bb.size(1) == F,
                 "rff_energy_sorted: x, W and b do not fit together");
     TORCH_CHECK(al.numel() == F, "rff_energy_sorted: alpha has ", al.numel(), " entries for ", F, " features");
     Tensor Wsplit = prepared_form(WW, 0, [&](const Tensor& w) {
@@ -599,14 +614,24 @@ std::tuple<Tensor, Tensor> rff_energy_sorted_impl(const Tensor& x_, const Tensor
         check(qmll_rff_presplit(fp(w), ne, d, F, out.data_ptr(), nbytes, stream()), "qmll_rff_presplit");
         return out;
     });
-    Tensor e = e_zeroed.defined() ? e_zeroed : at::zeros({nslots}, x.options());
-    Tensor gx = with_grad ? at::empty({A, d}, x.options()) : empty_like_none(x);
-    check(qmll_rff_energy_sorted(fp(x), ip(off), ip(ss), Wsplit.const_data_ptr(), fp(bb), fp(al), A, ne, d, F,
-                                 nslots ? e.data_ptr<float>() : nullptr, with_grad && A ? gx.data_ptr<float>() : nullptr,
-                                 stream()),
+    check(qmll_rff_energy_sorted(x, off, ss, Wsplit.const_data_ptr(), fp(bb), fp(al), A, ne, d, F, e, A ? gx : nullptr, stream()),
           "qmll_rff_energy_sorted");
+}
+
+std::tuple<Tensor, Tensor> rff_energy_sorted_impl(const Tensor& x_, const Tensor& type_offsets, const Tensor& sorted_slots,
+                                                  const Tensor& W, const Tensor& b, const Tensor& alpha, int64_t nslots,
+                                                  bool with_grad, const Tensor& e_zeroed = Tensor()) {
+    Tensor x = f32(x_), off = i32(type_offsets), ss = i32(sorted_slots);
+    need_cuda(x, "x");
+    const int A = (int)ss.size(0);
+    TORCH_CHECK(x.dim() == 2 && x.size(0) == A && off.dim() == 1, "rff_energy_sorted: x is [", x.sizes(), "] for ", A, " atoms");
+    Tensor e = e_zeroed.defined() ? e_zeroed : at::zeros({nslots}, x.options());
+    Tensor gx = with_grad ? at::empty({A, x.size(1)}, x.options()) : empty_like_none(x);
+    rff_energy_sorted_raw(fp(x), ip(off), ip(ss), A, (int)x.size(1), (int)off.size(0) - 1, W, b, alpha,
+                          nslots ? e.data_ptr<float>() : nullptr, with_grad ? gx.data_ptr<float>() : nullptr);
     return {e, gx};
 }
+
 
 struct RffEnergySortedFn : public Function<RffEnergySortedFn> {
     static variable_list forward(AutogradContext* ctx, const Tensor& x, const Tensor& off, const Tensor& ss,
@@ -644,41 +669,80 @@ std::tuple<Tensor, Tensor> rff_energy_sorted(const Tensor& x, const Tensor& off,
 // bias rows (the reference selects each element's atoms with Z == e over the MODEL's elements,
 // models/hadamard_features.py:99-107, while the representation indexes its bins by the
 // REPRESENTATION's species); an empty tensor says the two lists are the same.
-Tensor fchl_sorf_energy_impl(FCHL_TENSORS, MODEL_TENSORS, bool with_grad, Tensor* gX_out, bool rff = false) {
-    FchlInputs in = prepare(FCHL_PASS);
+// gscale: factor on the returned coordinate gradient (-1: forces)
+Tensor fchl_sorf_energy_impl(FCHL_TENSORS, MODEL_TENSORS, bool with_grad, Tensor* gX_out, bool rff = false,
+                             float gscale = 1.0f) {
+    FchlInputs in = prepare(FCHL_PASS, false);
+    need_cuda(reductors, "reductors");
     TORCH_CHECK(reductors.dim() == 3 && reductors.size(1) == in.R, "fchl_sorf_energy: reductors are [",
                 reductors.sizes(), "], the representation has ", in.R, " entries per atom");
-    const int64_t ne_model = reductors.size(0);
-    if (model_species.numel() == 0) {
-        TORCH_CHECK(ne_model == in.prm.nspecies, "fchl_sorf_energy: the model has ", ne_model,
-                    " elements, the representation ", in.prm.nspecies, " species, and no model species were given");
+    const int ne = (int)reductors.size(0), R = in.R, d = (int)reductors.size(2), A = in.A, B = in.B, n = in.n;
+    const bool own_list = model_species.numel() != 0;
+    if (!own_list) {
+        TORCH_CHECK(ne == in.prm.nspecies, "fchl_sorf_energy: the model has ", ne, " elements, the representation ",
+                    in.prm.nspecies, " species, and no model species were given");
     } else {
-        TORCH_CHECK(model_species.numel() == ne_model, "fchl_sorf_energy: ", model_species.numel(),
-                    " model species for ", ne_model, " reductors");
+        TORCH_CHECK(model_species.numel() == ne, "fchl_sorf_energy: ", model_species.numel(), " model species for ", ne,
+                    " reductors");
+        need_cuda(model_species, "model_species");
     }
-    // which reductor / Dmat / bias row an atom takes
-    const Tensor sort_types = model_species.numel() == 0 ? in.types : element_types(in.X, Z, in.natoms, model_species);
+    Tensor Zb = f32(Z.dim() == 1 ? Z.unsqueeze(0) : Z), sp = f32(species), msp = own_list ? f32(model_species) : Tensor();
+    Tensor red = f32(reductors);
+    TORCH_CHECK(Zb.dim() == 2 && Zb.size(0) == B && Zb.size(1) == n, "fchl_sorf_energy: charges are [", Zb.sizes(),
+                "], coordinates [", in.X.sizes(), "]");
+    const int64_t nslots = (int64_t)B * n;
+    // few allocations, cut up by hand: for one molecule the step is as long as its host side
+    //   ints:    element index by the representation's list | by the model's (only when it has its own) |
+    //            sorted slots | offsets | workspace of the sort
+    //   out:     per-slot energies | dE/dX   (what must start at zero)
+    //   scratch: representation | projected rows | their gradient | gradient of the representation
+    const size_t sort_bytes = qmll_sort_atoms_workspace(A, ne);
+    const int64_t types_ints = nslots * (own_list ? 2 : 1);
+    Tensor ints = at::empty({types_ints + A + ne + 1 + (int64_t)(sort_bytes / 4) + 1}, in.X.options().dtype(at::kInt));
+    int* types = ints.data_ptr<int>();
+    int* sort_types = own_list ? types + nslots : types;
+    int* ss = types + types_ints;
+    int* off = ss + A;
+    int* sort_work = off + ne + 1;
+    const int64_t nzero = (with_grad ? 4 : 1) * nslots;
+    Tensor out = at::empty({nzero}, in.X.options());
+    float* e_slots = nzero ? out.data_ptr<float>() : nullptr;
+    check(qmll_prepare_batch(fp(Zb), ip(in.natoms), fp(sp), in.prm.nspecies, fp(msp), ne, ip(in.atomIDs), ip(in.molIDs), B, n,
+                             A, sort_work, sort_bytes, types, own_list ? sort_types : nullptr, ss, off, e_slots,
+                             (size_t)nzero, stream()),
+          "qmll_prepare_batch");
+    auto pad = [](int64_t v) { return (v + 63) / 64 * 64; };          // every part 256-byte aligned
+    const int64_t rep_n = pad(nslots * R), x_n = pad((int64_t)A * d);
+    Tensor scratch = at::empty({rep_n + x_n + (with_grad ? x_n + rep_n : 0) + 64}, in.X.options());
+    float* rep = scratch.data_ptr<float>();
+    float* x = rep + rep_n;
+    float* gx = with_grad ? x + x_n : nullptr;
+    float* g_rep = with_grad ? gx + x_n : nullptr;
     // the forward kernel writes every bin of a listed atom's row, and only the rows of listed
-    // atoms are read below, so the padded rows need no clearing here
-    Tensor rep = at::empty({in.B, in.n, in.R}, in.X.options());
-    check(qmll_fchl19_forward(FCHL_ABI(in), rep.data_ptr<float>(), stream()), "qmll_fchl19_forward");
-    const int64_t nslots = (int64_t)in.B * in.n;
-    auto sorted = sort_atoms_by_type(sort_types, in.atomIDs, in.molIDs, in.n, ne_model);
-    const Tensor& ss = std::get<0>(sorted);
-    const Tensor& off = std::get<1>(sorted);
-    Tensor x = project_typed_impl(rep.view({nslots, in.R}), ss, off, reductors);
-    // the per-slot energies and the coordinate gradient both start from zero: one fill for the two
-    Tensor zeroed = at::zeros({with_grad ? 4 * nslots : nslots}, in.X.options());
-    Tensor e0 = zeroed.narrow(0, 0, nslots);
-    auto eg = rff ? rff_energy_sorted_impl(x, off, ss, Dmat, bias, alpha, nslots, with_grad, e0)
-                  : sorf_energy_sorted_impl(x, off, ss, Dmat, bias, alpha, cn, nt, nslots, with_grad, e0);
-    Tensor energies = std::get<0>(eg).view({in.B, in.n}).sum(1);
-    if (with_grad) {
-        Tensor g_rep = project_typed_backward(std::get<1>(eg), ss, off, reductors, sort_types, nslots);
-        Tensor gX = zeroed.narrow(0, nslots, 3 * nslots).view({in.B, in.n, 3});
-        check(qmll_fchl19_vjp(FCHL_ABI(in), fp(g_rep), gX.data_ptr<float>(), stream()), "qmll_fchl19_vjp");
-        *gX_out = gX;
+    // atoms are read below, so the padded rows need no clearing
+    check(qmll_fchl19_forward(FCHL_ABI_T(in, types), rep, stream()), "qmll_fchl19_forward");
+    Tensor split = reductors_split(red, A);
+    check(qmll_project_typed(rep, ss, off, fp(red), vp(split), A, ne, R, d, x, stream()), "qmll_project_typed");
+    if (rff)
+        rff_energy_sorted_raw(x, off, ss, A, d, ne, Dmat, bias, alpha, e_slots, gx);
+    else
+        sorf_energy_sorted_raw(x, off, ss, A, d, ne, Dmat, bias, alpha, cn, nt, e_slots, gx);
+    Tensor energies = at::empty({B}, in.X.options());
+    if (!with_grad) {        // the sums alone (A = 0), by the kernel that sums them beside the backward projection
+        check(qmll_project_typed_backward_sums(nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, ne, R, d, nullptr,
+                                               e_slots, B, n, B ? energies.data_ptr<float>() : nullptr, stream()),
+              "qmll_project_typed_backward_sums");
+        return energies;
     }
+    // rows of listed atoms whose element the model does not hold are zeroed (sort_types); the rows of
+    // padded slots are never read by the kernel below
+    check(qmll_project_typed_backward_sums(gx, ss, off, fp(red), vp(split), sort_types, A, (int)nslots, ne, R, d, g_rep,
+                                           e_slots, B, n, B ? energies.data_ptr<float>() : nullptr, stream()),
+          "qmll_project_typed_backward_sums");
+    Tensor gX = out.narrow(0, nslots, 3 * nslots).view({B, n, 3});
+    check(qmll_fchl19_vjp_scaled(FCHL_ABI_T(in, types), g_rep, gscale, nslots ? gX.data_ptr<float>() : nullptr, stream()),
+          "qmll_fchl19_vjp");
+    *gX_out = gX;
     return energies;
 }
 
@@ -708,6 +772,29 @@ struct FchlSorfEnergyFn : public Function<FchlSorfEnergyFn> {
 std::tuple<Tensor, Tensor> fchl_sorf_energy(FCHL_TENSORS, MODEL_TENSORS, bool with_grad) {
     auto r = FchlSorfEnergyFn::apply(FCHL_PASS, reductors, Dmat, bias, alpha, cn, nt, model_species, with_grad);
     return {r[0], r[1]};
+}
+
+// (energies [B], forces [B,n,3] = -dE/dX) outside autograd: what a predict call wants, the sign applied
+// inside the last kernel of the chain instead of by an elementwise pass afterwards
+void no_graph(const Tensor& X, const char* who) {
+    TORCH_CHECK(!(at::GradMode::is_enabled() && X.requires_grad()), who,
+                " builds no autograd graph: call it under no_grad, or use the _energy operator for a differentiable result");
+}
+std::tuple<Tensor, Tensor> fchl_sorf_forces(FCHL_TENSORS, MODEL_TENSORS) {
+    no_graph(X, "fchl_sorf_forces");
+    at::NoGradGuard guard;
+    Tensor F;
+    Tensor e = fchl_sorf_energy_impl(FCHL_PASS, reductors, Dmat, bias, alpha, cn, nt, model_species, true, &F, false, -1.0f);
+    return {e, X.dim() == 2 ? F.squeeze(0) : F};
+}
+std::tuple<Tensor, Tensor> fchl_rff_forces(FCHL_TENSORS, const Tensor& reductors, const Tensor& W, const Tensor& b,
+                                           const Tensor& alpha, const Tensor& model_species) {
+    no_graph(X, "fchl_rff_forces");
+    at::NoGradGuard guard;
+    Tensor F;
+    Tensor e = fchl_sorf_energy_impl(FCHL_PASS, reductors, W, b, alpha, Tensor(), Tensor(), model_species, true, &F, true,
+                                     -1.0f);
+    return {e, X.dim() == 2 ? F.squeeze(0) : F};
 }
 
 // the same chain with random Fourier features (models/random_features.py:82-102)
@@ -768,6 +855,8 @@ TORCH_LIBRARY(qml_lightning_sorf, m) {
     m.def("rff_energy_sorted", &rff_energy_sorted);
     m.def("fchl_sorf_energy", &fchl_sorf_energy);
     m.def("fchl_rff_energy", &fchl_rff_energy);
+    m.def("fchl_sorf_forces", &fchl_sorf_forces);
+    m.def("fchl_rff_forces", &fchl_rff_forces);
 }
 
 // names the loader can test for

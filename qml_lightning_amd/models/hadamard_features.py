@@ -159,10 +159,9 @@ def _register_fused_op():
                "Tensor coeff_normalisation, Tensor ntransforms, Tensor model_species, bool with_grad) "
                "-> (Tensor, Tensor)" % ops._FCHL_SIG)
 
-    def sort_types(Xb, Zb, atom_counts, types, species, model_species, reductors, R):
-        """Row of the model's reductors / diagonals / bias each atom takes: its index among the
-        MODEL's elements (hadamard_features.py:99-107 selects with Z == e over them), which
-        differs from the representation's species index when the two lists differ."""
+    def check_model(species, model_species, reductors, R):
+        """The model's element list (hadamard_features.py:99-107 selects atoms with Z == e over it) may
+        differ from the representation's species; its length must match the reductors."""
         if reductors.dim() != 3 or reductors.shape[1] != R:
             raise RuntimeError("fchl_sorf_energy: reductors are %s, the representation has %d entries per atom"
                                % (tuple(reductors.shape), R))
@@ -170,35 +169,34 @@ def _register_fused_op():
             if reductors.shape[0] != species.shape[0]:
                 raise RuntimeError("fchl_sorf_energy: the model has %d elements, the representation %d species, and "
                                    "no model species were given" % (reductors.shape[0], species.shape[0]))
-            return types
-        if model_species.numel() != reductors.shape[0]:
+        elif model_species.numel() != reductors.shape[0]:
             raise RuntimeError("fchl_sorf_energy: %d model species for %d reductors"
                                % (model_species.numel(), reductors.shape[0]))
-        return ops.element_types(Xb, Zb, atom_counts, model_species)
 
     def impl_chain(X, Z, species, atomIDs, molIDs, atom_counts, cell, inv_cell, Rs2, Rs3, eta2, eta3, two_body_decay,
                    three_body_weight, three_body_decay, rcut, reductors, Dmat, bias, alpha, cn, nt, model_species,
-                   with_grad):
+                   with_grad, gscale=1.0):
         Xb, Zb = ops._batched(X, Z)
         B, n = Zb.shape
         nslots = B * n
         prm = ops.make_params(species.shape[0], Rs2, Rs3, eta2, eta3, two_body_decay, three_body_weight,
                               three_body_decay, rcut)
-        types = ops.element_types(Xb, Zb, atom_counts, species)
+        check_model(species, model_species, reductors, ops.repsize(prm))
+        # element indices, the sort by the model's element and the zero fill of what the chain adds into
+        # (per-slot energies, then dE/dX): one launch for a small batch
+        types, stypes, ss, off, zeroed = ops.prepare_batch(Zb, atom_counts, species, atomIDs, molIDs, model_species,
+                                                           (4 if with_grad else 1) * nslots)
         cell_ = cell if cell.numel() > 0 else None
         inv_cell_ = inv_cell if inv_cell.numel() > 0 else None
         fargs = (Xb, types, cell_, inv_cell_, atomIDs, molIDs, atom_counts, Rs2, Rs3, prm)
-        rep = ops.fchl_forward(*fargs)
-        tflat = sort_types(Xb, Zb, atom_counts, types, species, model_species, reductors, ops.repsize(prm)).view(-1)
-        ss, off = ops.sort_by_type(tflat, molIDs * n + atomIDs, reductors.shape[0])
+        rep = ops.fchl_forward(*fargs, zero_fill=False)
         x = ops.project_typed(rep.view(nslots, -1), ss, off, reductors)
         e_slots, gx = ops.sorf_energy_sorted(x, off, ss, Dmat, bias, alpha, ops._scalar(cn), int(nt.item()), nslots,
-                                             with_grad=with_grad)
-        energies = e_slots.view(B, n).sum(dim=1)
+                                             with_grad=with_grad, e_zeroed=zeroed[:nslots])
         if not with_grad:
-            return energies, torch.empty(0, dtype=torch.float32, device=X.device)
-        g_rep = ops.project_typed_backward(gx, ss, off, reductors, tflat, nslots)
-        return energies, ops.fchl_vjp(g_rep.view(rep.shape), *fargs)
+            return ops.molecule_sums(e_slots, B, n), torch.empty(0, dtype=torch.float32, device=X.device)
+        g_rep, energies = ops.project_typed_backward_sums(gx, ss, off, reductors, stypes, nslots, e_slots, B, n)
+        return energies, ops.fchl_vjp(g_rep.view(rep.shape), *fargs, out=zeroed[nslots:].view(B, n, 3), scale=gscale)
 
     lib.impl("fchl_sorf_energy", impl_chain, "CompositeExplicitAutograd")
 
@@ -208,27 +206,52 @@ def _register_fused_op():
 
     def impl_chain_rff(X, Z, species, atomIDs, molIDs, atom_counts, cell, inv_cell, Rs2, Rs3, eta2, eta3,
                        two_body_decay, three_body_weight, three_body_decay, rcut, reductors, W, b, alpha,
-                       model_species, with_grad):
+                       model_species, with_grad, gscale=1.0):
         Xb, Zb = ops._batched(X, Z)
         B, n = Zb.shape
         nslots = B * n
         prm = ops.make_params(species.shape[0], Rs2, Rs3, eta2, eta3, two_body_decay, three_body_weight,
                               three_body_decay, rcut)
-        types = ops.element_types(Xb, Zb, atom_counts, species)
+        check_model(species, model_species, reductors, ops.repsize(prm))
+        types, stypes, ss, off, zeroed = ops.prepare_batch(Zb, atom_counts, species, atomIDs, molIDs, model_species,
+                                                           (4 if with_grad else 1) * nslots)
         fargs = (Xb, types, cell if cell.numel() > 0 else None, inv_cell if inv_cell.numel() > 0 else None, atomIDs,
                  molIDs, atom_counts, Rs2, Rs3, prm)
-        rep = ops.fchl_forward(*fargs)
-        tflat = sort_types(Xb, Zb, atom_counts, types, species, model_species, reductors, ops.repsize(prm)).view(-1)
-        ss, off = ops.sort_by_type(tflat, molIDs * n + atomIDs, reductors.shape[0])
+        rep = ops.fchl_forward(*fargs, zero_fill=False)
         x = ops.project_typed(rep.view(nslots, -1), ss, off, reductors)
-        e_slots, gx = ops.rff_energy_sorted(x, off, ss, W, b, alpha, nslots, with_grad=with_grad)
-        energies = e_slots.view(B, n).sum(dim=1)
+        e_slots, gx = ops.rff_energy_sorted(x, off, ss, W, b, alpha, nslots, with_grad=with_grad,
+                                            e_zeroed=zeroed[:nslots])
         if not with_grad:
-            return energies, torch.empty(0, dtype=torch.float32, device=X.device)
-        g_rep = ops.project_typed_backward(gx, ss, off, reductors, tflat, nslots)
-        return energies, ops.fchl_vjp(g_rep.view(rep.shape), *fargs)
+            return ops.molecule_sums(e_slots, B, n), torch.empty(0, dtype=torch.float32, device=X.device)
+        g_rep, energies = ops.project_typed_backward_sums(gx, ss, off, reductors, stypes, nslots, e_slots, B, n)
+        return energies, ops.fchl_vjp(g_rep.view(rep.shape), *fargs, out=zeroed[nslots:].view(B, n, 3), scale=gscale)
 
     lib.impl("fchl_rff_energy", impl_chain_rff, "CompositeExplicitAutograd")
+
+    # (energies, forces = -dE/dX) with no autograd graph: the sign is applied inside the last kernel of the chain
+    def no_graph(X, who):
+        if torch.is_grad_enabled() and X.requires_grad:
+            raise RuntimeError(who + " builds no autograd graph: call it under no_grad, or use the _energy operator "
+                               "for a differentiable result")
+
+    def impl_forces(*args):
+        no_graph(args[0], "fchl_sorf_forces")
+        with torch.no_grad():
+            e, F = impl_chain(*args, True, gscale=-1.0)
+        return e, (F.squeeze(0) if args[0].dim() == 2 else F)
+
+    def impl_forces_rff(*args):
+        no_graph(args[0], "fchl_rff_forces")
+        with torch.no_grad():
+            e, F = impl_chain_rff(*args, True, gscale=-1.0)
+        return e, (F.squeeze(0) if args[0].dim() == 2 else F)
+
+    lib.define("fchl_sorf_forces(%s, Tensor reductors, Tensor Dmat, Tensor bias, Tensor alpha, "
+               "Tensor coeff_normalisation, Tensor ntransforms, Tensor model_species) -> (Tensor, Tensor)" % ops._FCHL_SIG)
+    lib.impl("fchl_sorf_forces", impl_forces, "CompositeExplicitAutograd")
+    lib.define("fchl_rff_forces(%s, Tensor reductors, Tensor W, Tensor b, Tensor alpha, Tensor model_species) "
+               "-> (Tensor, Tensor)" % ops._FCHL_SIG)
+    lib.impl("fchl_rff_forces", impl_forces_rff, "CompositeExplicitAutograd")
 
     def setup_chain(ctx, inputs, output):
         ctx.save_for_backward(output[1])
@@ -271,6 +294,29 @@ def model_species_for_sort(species, rep):
     if rep is not None and tuple(rep.species.shape) == tuple(species.shape) and bool((rep.species.cpu() == species.cpu()).all()):
         return torch.empty(0, dtype=torch.float32, device=species.device)
     return species
+
+
+_NO_CELLS = {}
+_NORMALISATION = {}
+
+
+def _no_cells(device):
+    """The empty [0,3,3] tensor that says "no periodic images", one per device (a single molecule's
+    step is as long as its host side: nothing is built per call that can be kept)."""
+    t = _NO_CELLS.get(device)
+    if t is None:
+        t = _NO_CELLS[device] = torch.empty(0, 3, 3, device=device)
+    return t
+
+
+def _normalisation_tensor(npcas, sigma):
+    key = (int(npcas), float(sigma))
+    t = _NORMALISATION.get(key)
+    if t is None:
+        if len(_NORMALISATION) > 256:
+            _NORMALISATION.clear()
+        t = _NORMALISATION[key] = torch.tensor(float(np.sqrt(np.float32(npcas)) / np.float32(sigma)))
+    return t
 
 
 class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
@@ -434,20 +480,25 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         # one call of the operator that runs the whole chain (what `forward` dispatches to), outside
         # autograd: it returns the energies and dE/dX
         if cells is None or inv_cells is None:
-            cells = torch.empty(0, 3, 3, device=coordinates.device)
-            inv_cells = cells
+            cells = inv_cells = _no_cells(coordinates.device)
         if isinstance(self.sigma, float):       # sqrt(npcas) / sigma in fp32, as the tensor expression gives it
-            coeff_normalisation = torch.tensor(float(np.sqrt(np.float32(self.npcas)) / np.float32(self.sigma)))
+            coeff_normalisation = _normalisation_tensor(self.npcas, self.sigma)
         else:
             coeff_normalisation = torch.sqrt(torch.tensor(self.npcas)) / self.sigma
         rep = self.rep
         with torch.no_grad():
-            energies, gX = torch.ops.qml_lightning_sorf.fchl_sorf_energy(
+            if forces:      # energies and -dE/dX from one operator, the sign applied in its last kernel
+                return torch.ops.qml_lightning_sorf.fchl_sorf_forces(
+                    coordinates, charges, rep.species, atomIDs, molIDs, natom_counts, cells, inv_cells, rep.Rs2, rep.Rs3,
+                    rep.eta2, rep.eta3, rep.two_body_decay, rep.three_body_weight, rep.three_body_decay, rep.rcut,
+                    self.reductors, self.Dmat, self.bias, alpha_f32(self), coeff_normalisation, self.ntransforms,
+                    self.sort_species)
+            energies, _ = torch.ops.qml_lightning_sorf.fchl_sorf_energy(
                 coordinates, charges, rep.species, atomIDs, molIDs, natom_counts, cells, inv_cells, rep.Rs2, rep.Rs3,
                 rep.eta2, rep.eta3, rep.two_body_decay, rep.three_body_weight, rep.three_body_decay, rep.rcut,
                 self.reductors, self.Dmat, self.bias, alpha_f32(self), coeff_normalisation, self.ntransforms,
-                self.sort_species, forces)
-        return energies, (gX.neg_() if forces else None)
+                self.sort_species, False)
+        return energies, None
 
     @torch.jit.unused
     def predict_opt(self, coordinates, charges, atomIDs, molIDs, natom_counts, cells=None, inv_cells=None,

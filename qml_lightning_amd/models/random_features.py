@@ -9,6 +9,7 @@ from .. import ops
 from ..cuda.rff_gpu import get_rff
 from ..representations.dimensionality_reduction import project_representation
 from . import hadamard_features  # noqa: F401  (registers the fused operators)
+from .hadamard_features import _no_cells
 from .kernel import BaseKernel, _default_device, alpha_f32, rep_from_attribute_tree
 
 
@@ -127,15 +128,19 @@ class RandomFourrierFeaturesModel(BaseKernel, torch.nn.Module):
         asynchronously on the current stream; no autograd graph (the fused kernel returns
         dE/dx itself)."""
         if cells is None or inv_cells is None:
-            cells = torch.empty(0, 3, 3, device=coordinates.device)
-            inv_cells = cells
+            cells = inv_cells = _no_cells(coordinates.device)
         rep = self.rep
         with torch.no_grad():
-            energies, gX = torch.ops.qml_lightning_sorf.fchl_rff_energy(
+            if forces:      # energies and -dE/dX from one operator, the sign applied in its last kernel
+                return torch.ops.qml_lightning_sorf.fchl_rff_forces(
+                    coordinates, charges, rep.species, atomIDs, molIDs, natom_counts, cells, inv_cells, rep.Rs2, rep.Rs3,
+                    rep.eta2, rep.eta3, rep.two_body_decay, rep.three_body_weight, rep.three_body_decay, rep.rcut,
+                    self.reductors, self.W, self.b, alpha_f32(self), self.sort_species)
+            energies, _ = torch.ops.qml_lightning_sorf.fchl_rff_energy(
                 coordinates, charges, rep.species, atomIDs, molIDs, natom_counts, cells, inv_cells, rep.Rs2, rep.Rs3,
                 rep.eta2, rep.eta3, rep.two_body_decay, rep.three_body_weight, rep.three_body_decay, rep.rcut,
-                self.reductors, self.W, self.b, alpha_f32(self), self.sort_species, forces)
-        return energies, (gX.neg_() if forces else None)
+                self.reductors, self.W, self.b, alpha_f32(self), self.sort_species, False)
+        return energies, None
 
     @torch.jit.unused
     def predict_opt(self, coordinates, charges, atomIDs, molIDs, natom_counts, zcells=None, zinv_cells=None,

@@ -162,26 +162,36 @@ def repsize(prm):
     return prm.nspecies * prm.nRs2 + prm.nspecies * (prm.nspecies + 1) * prm.nRs3
 
 
-def fchl_forward(X, types, cell, inv_cell, atomIDs, molIDs, natoms, Rs2, Rs3, prm, nlist=None, nneigh=None):
-    """rep f32 [B,n,R]; zero rows for padded slots (fchl_cuda.cpp:83)."""
+def fchl_forward(X, types, cell, inv_cell, atomIDs, molIDs, natoms, Rs2, Rs3, prm, nlist=None, nneigh=None,
+                 zero_fill=True):
+    """rep f32 [B,n,R]; zero rows for padded slots (fchl_cuda.cpp:83).  zero_fill=False leaves the rows
+    of slots that are not listed unwritten (the kernel writes every bin of a listed atom's row): for
+    callers that read listed rows only."""
     X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3 = _fchl_prepare(
         X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3)
     B, n, _ = X.shape
-    rep = torch.zeros((B, n, repsize(prm)), dtype=torch.float32, device=X.device)
+    rep = (torch.zeros if zero_fill else torch.empty)((B, n, repsize(prm)), dtype=torch.float32, device=X.device)
     args = _fchl_args(X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3, prm)
     check(_lib.lib().qmll_fchl19_forward(*args, _ptr(rep), _stream()), "qmll_fchl19_forward")
     return rep
 
 
-def fchl_vjp(grad_rep, X, types, cell, inv_cell, atomIDs, molIDs, natoms, Rs2, Rs3, prm, nlist=None, nneigh=None):
-    """grad_X f32 [B,n,3] (fchl_cuda.cpp:196)."""
+def fchl_vjp(grad_rep, X, types, cell, inv_cell, atomIDs, molIDs, natoms, Rs2, Rs3, prm, nlist=None, nneigh=None,
+             out=None, scale=1.0):
+    """grad_X f32 [B,n,3] (fchl_cuda.cpp:196), times `scale` (-1: forces from an energy gradient).
+    out: a zero-filled contiguous f32 [B,n,3] to add into."""
     X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3 = _fchl_prepare(
         X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3)
     B, n, _ = X.shape
     grad_rep = _f32(grad_rep).reshape(B, n, repsize(prm))
-    gX = torch.zeros((B, n, 3), dtype=torch.float32, device=X.device)
+    if out is None:
+        gX = torch.zeros((B, n, 3), dtype=torch.float32, device=X.device)
+    else:
+        gX = out
+        if gX.dtype != torch.float32 or tuple(gX.shape) != (B, n, 3) or not gX.is_contiguous():
+            raise RuntimeError("fchl_vjp: out must be a contiguous float32 [%d, %d, 3] tensor" % (B, n))
     args = _fchl_args(X, types, cell, inv_cell, atomIDs, molIDs, natoms, nlist, nneigh, Rs2, Rs3, prm)
-    check(_lib.lib().qmll_fchl19_vjp(*args, _ptr(grad_rep), _ptr(gX), _stream()), "qmll_fchl19_vjp")
+    check(_lib.lib().qmll_fchl19_vjp_scaled(*args, _ptr(grad_rep), float(scale), _ptr(gX), _stream()), "qmll_fchl19_vjp")
     return gX
 
 
@@ -418,6 +428,34 @@ def sort_atoms_by_type(types, atomIDs, molIDs, n, ne):
     return sorted_slots, offsets
 
 
+def prepare_batch(Z, natoms, species, atomIDs, molIDs, model_species=None, zero_count=0):
+    """What the fused predict chain needs before its first compute kernel, in one launch for small
+    batches: (types [B,n] by `species`, sort_types [B,n] by `model_species` (types itself when that is
+    None), sorted_slots [A], type_offsets [ne+1], zeroed f32 [zero_count])."""
+    _need_cuda(Z, "charges")
+    Zb = _f32(Z if Z.dim() == 2 else Z.unsqueeze(0))
+    natoms, species = _i32(natoms), _f32(species)
+    atomIDs, molIDs = _i32(atomIDs).reshape(-1), _i32(molIDs).reshape(-1)
+    B, n = Zb.shape
+    A = int(atomIDs.shape[0])
+    own = model_species is not None and model_species.numel() > 0
+    msp = _f32(model_species) if own else None
+    ne = int(msp.shape[0]) if own else int(species.shape[0])
+    dev = Zb.device
+    types = torch.empty((B, n), dtype=torch.int32, device=dev)
+    sort_types = torch.empty((B, n), dtype=torch.int32, device=dev) if own else types
+    sorted_slots = torch.empty(A, dtype=torch.int32, device=dev)
+    offsets = torch.empty(ne + 1, dtype=torch.int32, device=dev)
+    zero = torch.empty(int(zero_count), dtype=torch.float32, device=dev)
+    nbytes = int(_lib.lib().qmll_sort_atoms_workspace(A, ne))
+    work = torch.empty(nbytes // 4, dtype=torch.int32, device=dev) if nbytes else None
+    check(_lib.lib().qmll_prepare_batch(_ptr(Zb), _ptr(natoms), _ptr(species), int(species.shape[0]), _ptr(msp), ne,
+                                        _ptr(atomIDs), _ptr(molIDs), B, n, A, _ptr(work), nbytes, _ptr(types),
+                                        _ptr(sort_types) if own else None, _ptr(sorted_slots), _ptr(offsets), _ptr(zero),
+                                        int(zero_count), _stream()), "qmll_prepare_batch")
+    return types, sort_types, sorted_slots, offsets, zero
+
+
 def reductor_presplit(reductors):
     """The reductors [ne,R,d] in the form the fp16 matrix-core projection kernels multiply with
     (qmll_reductor_presplit): an opaque uint8 device buffer, or None when no kernel takes one."""
@@ -497,9 +535,50 @@ def project_typed_backward(gx, sorted_slots, type_offsets, reductors, types, nsl
     return g_rep
 
 
+def project_typed_backward_sums(gx, sorted_slots, type_offsets, reductors, types, nslots, e_slots, B, n):
+    """(g_rep [nslots,R] as `project_typed_backward` but with the rows of padded slots left unwritten,
+    energies [B] = e_slots.view(B, n).sum(1)); one launch for small batches."""
+    gx, reductors, e_slots = _f32(gx), _f32(reductors), _f32(e_slots)
+    sorted_slots, type_offsets, types = _i32(sorted_slots), _i32(type_offsets), _i32(types).reshape(-1)
+    ne, R, d = reductors.shape
+    A, N = int(sorted_slots.shape[0]), int(nslots)
+    if gx.shape[0] != A or gx.shape[1] != d or types.shape[0] != N or e_slots.numel() != B * n:
+        raise RuntimeError("project_typed_backward_sums: gx %s for %d atoms, d=%d" % (tuple(gx.shape), A, d))
+    g_rep = torch.empty((N, R), dtype=torch.float32, device=gx.device)
+    energies = torch.empty(B, dtype=torch.float32, device=gx.device)
+    check(_lib.lib().qmll_project_typed_backward_sums(_ptr(gx), _ptr(sorted_slots), _ptr(type_offsets), _ptr(reductors),
+                                                      _ptr(_split_for(reductors, A)), _ptr(types), A, N, ne, R, d,
+                                                      _ptr(g_rep), _ptr(e_slots), int(B), int(n), _ptr(energies),
+                                                      _stream()),
+          "qmll_project_typed_backward_sums")
+    return g_rep, energies
+
+
+def molecule_sums(e_slots, B, n):
+    """energies [B] = sum over the n slots of each molecule of e_slots [B*n] (slots in ascending order:
+    the same sums `project_typed_backward_sums` forms)."""
+    e_slots = _f32(e_slots)
+    if e_slots.numel() != B * n:
+        raise RuntimeError("molecule_sums: %d slots for %d x %d" % (e_slots.numel(), B, n))
+    energies = torch.empty(B, dtype=torch.float32, device=e_slots.device)
+    check(_lib.lib().qmll_project_typed_backward_sums(None, None, None, None, None, None, 0, 0, 1, 1, 1, None,
+                                                      _ptr(e_slots), int(B), int(n), _ptr(energies), _stream()),
+          "qmll_project_typed_backward_sums")
+    return energies
+
+
+def _zeroed_slots(e_zeroed, nslots, device):
+    if e_zeroed is None:
+        return torch.zeros(int(nslots), dtype=torch.float32, device=device)
+    if e_zeroed.dtype != torch.float32 or e_zeroed.numel() != int(nslots) or not e_zeroed.is_contiguous():
+        raise RuntimeError("e_zeroed must be a contiguous float32 tensor of %d entries" % int(nslots))
+    return e_zeroed
+
+
 def sorf_energy_sorted(x, type_offsets, sorted_slots, Dmat, bias, alpha, normalisation, ntransforms, nslots,
-                       with_grad=True):
-    """Fused SORF + cos + energy on element-sorted rows x [A,d] -> (e_slots [nslots], gx [A,d] or None)."""
+                       with_grad=True, e_zeroed=None):
+    """Fused SORF + cos + energy on element-sorted rows x [A,d] -> (e_slots [nslots], gx [A,d] or None).
+    e_zeroed: the caller's zero-filled f32 [nslots] to take the energies (else one is made here)."""
     x, Dmat, bias, alpha = _f32(x), _f32(Dmat), _f32(bias), _f32(alpha)
     type_offsets, sorted_slots = _i32(type_offsets), _i32(sorted_slots)
     ne, Tn, S, d = Dmat.shape
@@ -512,7 +591,7 @@ def sorf_energy_sorted(x, type_offsets, sorted_slots, Dmat, bias, alpha, normali
     if tuple(bias.shape) != (ne, S * d) or alpha.numel() != S * d:
         raise RuntimeError("sorf_energy_sorted: bias %s / alpha with %d entries do not fit %d elements and %d features"
                            % (tuple(bias.shape), alpha.numel(), ne, S * d))
-    e_slots = torch.zeros(int(nslots), dtype=torch.float32, device=x.device)
+    e_slots = _zeroed_slots(e_zeroed, nslots, x.device)
     gx = torch.empty((A, d), dtype=torch.float32, device=x.device) if with_grad else None
     # the largest |bias|, a constant of the model, computed once per tensor version and left on the device
     bmax = presplit_cached(bias, "absmax", lambda t: t.abs().max().reshape(1))
@@ -595,10 +674,10 @@ def rff_presplit(W):
     return out
 
 
-def rff_energy_sorted(x, type_offsets, sorted_slots, W, b, alpha, nslots, with_grad=True):
+def rff_energy_sorted(x, type_offsets, sorted_slots, W, b, alpha, nslots, with_grad=True, e_zeroed=None):
     """Fused RFF energy (and gradient) on element-sorted rows x [A,d]; W [ne,d,F], b [ne,F],
     alpha [F] fp32 -> (e_slots [nslots], gx [A,d] or None).  W is split for the kernel on its first
-    use and the split form kept until W changes."""
+    use and the split form kept until W changes.  e_zeroed: as for sorf_energy_sorted."""
     x, W, b, alpha = _f32(x), _f32(W), _f32(b), _f32(alpha)
     type_offsets, sorted_slots = _i32(type_offsets), _i32(sorted_slots)
     ne, d, F = W.shape
@@ -609,7 +688,7 @@ def rff_energy_sorted(x, type_offsets, sorted_slots, W, b, alpha, nslots, with_g
     if alpha.numel() != F:
         raise RuntimeError("rff_energy_sorted: alpha has %d entries for %d features" % (alpha.numel(), F))
     Wsplit = presplit_cached(W, "rff", rff_presplit)
-    e_slots = torch.zeros(int(nslots), dtype=torch.float32, device=x.device)
+    e_slots = _zeroed_slots(e_zeroed, nslots, x.device)
     gx = torch.empty((A, d), dtype=torch.float32, device=x.device) if with_grad else None
     check(_lib.lib().qmll_rff_energy_sorted(_ptr(x), _ptr(type_offsets), _ptr(sorted_slots), _ptr(Wsplit), _ptr(b),
                                             _ptr(alpha), A, ne, d, F, _ptr(e_slots), _ptr(gx), _stream()),

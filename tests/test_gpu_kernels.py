@@ -1050,3 +1050,58 @@ def test_a_non_finite_row_spoils_only_itself_in_the_fp16_matrix_core_kernels():
     slot_keep = torch.ones(A, dtype=torch.bool, device=dev())
     slot_keep[rows[11]] = False
     assert (e1[slot_keep] - e0[slot_keep]).abs().max() <= 1e-6 * e0.abs().max()
+
+
+@pytest.mark.parametrize("nmol,model_list", [(1, None), (40, None), (40, [8.0, 1.0]), (300, [6.0, 9.0, 1.0]), (0, None)])
+def test_batch_preparation_in_one_call_equals_the_separate_kernels(nmol, model_list):
+    """qmll_prepare_batch (element indices by the representation's and by the model's species, the
+    sort of the listed atoms, the zero fill; one launch up to 1024 atoms) against qmll_element_types,
+    qmll_sort_atoms_by_type and a fill: bit-exact, ragged molecules with padding, a model list that is a
+    subset / permutation of the species and leaves some atoms without an element."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(nmol + 5)
+    n = 23
+    counts = rng.integers(1, n + 1, size=nmol).astype(np.int32)
+    Z = np.zeros((nmol, n), np.float32)
+    for m in range(nmol):
+        Z[m, :counts[m]] = rng.choice([1.0, 6.0, 8.0, 7.0], size=counts[m])          # 7: in no list
+    atomIDs = np.concatenate([np.arange(c) for c in counts]).astype(np.int32) if nmol else np.zeros(0, np.int32)
+    molIDs = np.repeat(np.arange(nmol), counts).astype(np.int32)
+    t = lambda a: torch.tensor(a, device=dev())
+    Zt, ct, ai, mi = t(Z), t(counts), t(atomIDs), t(molIDs)
+    species = t(np.array([1.0, 6.0, 8.0], np.float32))
+    msp = t(np.array(model_list, np.float32)) if model_list else None
+    nz = 4 * nmol * n
+    types, stypes, ss, off, zero = ops.prepare_batch(Zt, ct, species, ai, mi, msp, nz)
+    X0 = torch.zeros(nmol, n, 3, device=dev())
+    want_types = ops.element_types(X0, Zt, ct, species) if nmol else types
+    assert torch.equal(types, want_types.view(nmol, n))
+    want_st = ops.element_types(X0, Zt, ct, msp).view(nmol, n) if (msp is not None and nmol) else want_types.view(nmol, n)
+    assert torch.equal(stypes, want_st)
+    ne = len(model_list) if model_list else 3
+    want_ss, want_off = ops.sort_atoms_by_type(want_st, ai, mi, n, ne)
+    assert torch.equal(off, want_off)
+    last = int(off[-1])
+    assert torch.equal(ss[:last], want_ss[:last])
+    assert zero.shape[0] == nz and not zero.any()
+
+
+def test_transposed_projection_with_the_energy_sums_in_the_same_call():
+    """qmll_project_typed_backward_sums against qmll_project_typed_backward and a row sum, on both sides
+    of the small-batch switch; rows of atoms whose element the model does not hold come out zero."""
+    from qml_lightning_amd import ops
+    g = torch.Generator(device=dev()).manual_seed(3)
+    for B, n in ((1, 21), (48, 21), (400, 21)):
+        N = B * n
+        types = torch.randint(-1, 3, (N,), device=dev(), generator=g, dtype=torch.int32)
+        slots = torch.arange(N, device=dev(), dtype=torch.int32)
+        ss, off = ops.sort_by_type(types, slots, 3)
+        red = torch.randn(3, 312, 128, device=dev(), generator=g)
+        gx = torch.randn(N, 128, device=dev(), generator=g)
+        e_slots = torch.randn(N, device=dev(), generator=g)
+        want = ops.project_typed_backward(gx, ss, off, red, types, N)
+        got, energies = ops.project_typed_backward_sums(gx, ss, off, red, types, N, e_slots, B, n)
+        assert torch.equal(got, want)
+        assert not got[types < 0].any()
+        ref = e_slots.view(B, n).double().sum(1)
+        assert (energies.double() - ref).abs().max() <= 1e-6 * ref.abs().max()

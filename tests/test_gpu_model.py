@@ -30,6 +30,20 @@ def build_sorf_model(species, npcas, nstacks, ntransforms=1, sigma=2.0, fused=Tr
     return m, (red, D.astype(np.float64), bias, alpha.astype(np.float32).astype(np.float64))
 
 
+def build_rff_model(species, npcas, nstacks, seed=3):
+    from qml_lightning_amd.models.random_features import RandomFourrierFeaturesModel
+    from qml_lightning_amd.representations.FCHL import FCHLCuda
+    rep = FCHLCuda(species=np.array(species))
+    np.random.seed(seed)
+    m = RandomFourrierFeaturesModel(rep=rep, elements=np.array(species), sigma=3.0, llambda=1e-5, npcas=npcas,
+                                    nstacks=nstacks, nbatch_train=4, nbatch_test=5)
+    red, _, _, alpha = helpers.model_weights(len(species), rep.get_repsize(), npcas, nstacks)
+    m.reductors = t32(red)
+    m.alpha = torch.tensor(alpha, device=dev())
+    m.is_trained = True
+    return m, red
+
+
 def inputs(X, Z, aid, mid, nat):
     return t32(X), t32(Z), ti32(aid), ti32(mid), ti32(nat)
 
@@ -768,3 +782,41 @@ def test_training_at_the_default_regularisation_vs_fp64_oracle_rows(nmol, npcas,
     e, f = m.predict(c32[te], charges[te], 12, forces=True, print_info=False)
     close(e, E_g, 5e-4, "library predict with its own alpha, energies")     # fp32 contraction with an alpha of large entries
     close(f, F_g, 5e-4, "library predict with its own alpha, forces")
+
+
+@pytest.mark.parametrize("kind", ["sorf", "rff"])
+def test_forces_operator_equals_minus_the_gradient_of_the_energy_operator(kind):
+    """energies_and_forces takes energies and forces from ONE operator that builds no autograd graph and
+    applies the sign inside its last kernel (qmll_fchl19_vjp_scaled): same energies as `forward`, forces
+    equal to minus autograd's gradient, for a padded ragged batch and for a single unbatched molecule; with
+    a coordinate tensor that requires a gradient it refuses instead of returning something detached."""
+    species = [1, 6, 7, 8, 9]
+    coords, charges = helpers.ragged_batch(7, 11)
+    m = (build_sorf_model(species, 32, 4)[0] if kind == "sorf" else build_rff_model(species, 64, 4)[0])
+    X, Z, aid, mid, nat = make_batch(coords, charges)
+    gX, gZ, gaid, gmid, gnat = inputs(X, Z, aid, mid, nat)
+    e, f = m.energies_and_forces(gX, gZ, gaid, gmid, gnat)
+    Xg = gX.clone().requires_grad_(True)
+    e2 = m.forward(Xg, gZ, gaid, gmid, gnat)
+    g, = torch.autograd.grad(e2.sum(), Xg)
+    etol = 2e-6 * float(e.abs().max())          # the RFF kernel adds its feature shares with fp32 atomics
+    assert (e - e2.detach()).abs().max() <= (0.0 if kind == "sorf" else etol)
+    assert (f + g).abs().max() <= 2e-6 * g.abs().max()            # the cross-atom sums use atomics
+    e_only, none = m.energies_and_forces(gX, gZ, gaid, gmid, gnat, forces=False)
+    assert none is None and (e_only - e).abs().max() <= (0.0 if kind == "sorf" else etol)
+    op = torch.ops.qml_lightning_sorf.fchl_sorf_forces if kind == "sorf" else torch.ops.qml_lightning_sorf.fchl_rff_forces
+    rep = m.rep
+    head = (gZ, rep.species, gaid, gmid, gnat, torch.empty(0, 3, 3, device=dev()), torch.empty(0, 3, 3, device=dev()), rep.Rs2,
+            rep.Rs3, rep.eta2, rep.eta3, rep.two_body_decay, rep.three_body_weight, rep.three_body_decay, rep.rcut)
+    if kind == "sorf":
+        tail = (m.reductors, m.Dmat, m.bias, m.alpha.float(), torch.tensor(float(np.sqrt(np.float32(m.npcas)) / m.sigma)),
+                m.ntransforms, m.sort_species)
+    else:
+        tail = (m.reductors, m.W, m.b, m.alpha.float(), m.sort_species)
+    with pytest.raises(RuntimeError, match="no autograd graph"):
+        op(Xg, *head, *tail)
+    # one unbatched molecule: [n,3] coordinates and [n] charges in, [n,3] forces out
+    n0 = int(gnat[0])
+    one = op(gX[0], gZ[0], rep.species, gaid[:n0], gmid[:n0], gnat[:1], *head[5:], *tail)
+    assert one[1].shape == gX[0].shape
+    assert (one[1] - f[0]).abs().max() <= 2e-6 * f.abs().max() and abs(float(one[0][0] - e[0])) <= 1e-5 * float(e.abs().max())
