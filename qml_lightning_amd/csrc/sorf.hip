@@ -1626,8 +1626,9 @@ static int launch_fused(const char* who, const float* x, const float* D, const f
         // that zero the gradient rows past the last atom of a known element
         const int zero_groups = A >= 65536 ? 64 : (A >> 10) + 1;
         const dim3 grid((A + ROWS_NA - 1) / ROWS_NA + (type_offsets ? ne + zero_groups : 0));
-        // a few atoms: sixteen wavefronts per workgroup share out the stacks
-        const bool few = A <= 256 && S >= 64 && d <= 128 && T == 1;
+        // up to some 1500 atoms the chip has idle SIMDs: sixteen wavefronts per workgroup share out the stacks
+        // (measured at d = 128, 128 stacks: 17.4 -> 13.8 us at 1008 atoms, equal at 2016, slower from 2688 on)
+        const bool few = A <= 1536 && S >= 64 && d <= 128 && T == 1;
 #define LAUNCH_ROWS(L, G, M)                                                                                       \
     if (few && !(M))                                                                                               \
         hipLaunchKernelGGL((sorf_energy_rows_kernel<L, G, false, ((L) <= 7 ? 16 : SORF_WAVES)>), grid, dim3(1024), \

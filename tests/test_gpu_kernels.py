@@ -1105,3 +1105,40 @@ def test_transposed_projection_with_the_energy_sums_in_the_same_call():
         assert not got[types < 0].any()
         ref = e_slots.view(B, n).double().sum(1)
         assert (energies.double() - ref).abs().max() <= 1e-6 * ref.abs().max()
+
+
+def test_fused_energy_agrees_across_the_stack_sharing_switch():
+    """Up to 1536 atoms a workgroup of the fused kernel runs sixteen wavefronts that share out the stacks,
+    beyond that four: the same atoms evaluated in a batch on either side of the switch give the same
+    energies and gradient rows (the stacks are summed in another order: last bits), and a sample of them
+    matches the oracle."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(23)
+    ne, d, S = 3, 128, 64
+    F = S * d
+    A_big = 1800
+    x = rng.normal(size=(A_big, d)).astype(np.float32)
+    types = (np.arange(A_big) % ne).astype(np.int32)
+    D = np.where(rng.uniform(-1, 1, (ne, 1, S, d)) > 0, 1.0, -1.0).astype(np.float32)
+    b = rng.uniform(0, 2 * np.pi, (ne, F)).astype(np.float32)
+    alpha = rng.normal(size=F).astype(np.float32)
+    out = {}
+    for A in (1536, A_big):
+        ss, off = ops.sort_by_type(ti32(types[:A]), ti32(np.arange(A, dtype=np.int32)), ne)
+        xs = t32(x[:A])[ss.long()]                      # rows in sorted order
+        e, gx = ops.sorf_energy_sorted(xs, off, ss, t32(D), t32(b), t32(alpha), 3.0, 1, A)
+        g = torch.empty_like(gx)
+        g[ss.long()] = gx                               # back to atom order
+        out[A] = (e, g)
+    e0, g0 = out[1536]
+    e1, g1 = out[A_big]
+    assert (e0 - e1[:1536]).abs().max() <= 2e-6 * e1.abs().max()
+    assert (g0 - g1[:1536]).abs().max() <= 2e-6 * g1.abs().max()
+    for a_ in (0, 700, 1535):
+        t_ = types[a_]
+        c = sorf.sorf_coefficients(x[a_][None, :], D[t_], 3.0).reshape(1, F)
+        e_ref = (np.sqrt(2.0 / F) * np.cos(c + b[t_]) * alpha).sum()
+        gc = -np.sqrt(2.0 / F) * np.sin(c + b[t_]) * alpha
+        g_ref = sorf.sorf_adjoint(gc.reshape(1, S, d), D[t_], 3.0)[0]
+        assert abs(float(e0[a_]) - e_ref) <= REL_EF * float(e1.abs().max())
+        assert np.abs(g0[a_].cpu().numpy() - g_ref).max() <= REL_EF * float(g1.abs().max())
