@@ -890,44 +890,69 @@ __global__ __launch_bounds__(256) void project_small_kernel(const float* __restr
     }
 }
 
-// g_rep[slot(p), :] = gx[p, :] . U_e^T: thread = output entry r, its reductor row is contiguous
-// (workgroups past the A atoms zero the rows of slots whose type is outside [0, ne), 256 slots each, and
-// after those, when asked, sum the per-slot energies of 256 molecules each)
+// g_rep[slot(p), :] = gx[p, :] . U_e^T: thread = output entry r, its reductor row is contiguous.  A
+// workgroup takes NA consecutive sorted atoms of one element (tiles never straddle two elements), so a
+// reductor row read serves NA atoms: with one atom per workgroup 1008 atoms read 160 MB of reductors from
+// L2 (20 us), with eight 20 MB.  Workgroups past the tiles zero the rows of slots whose type is outside
+// [0, ne), 256 slots each, and after those, when asked, sum the per-slot energies of 256 molecules each.
+template <int NA>
 __global__ __launch_bounds__(256) void project_bt_small_kernel(const float* __restrict__ gx,
                                                                const int* __restrict__ sorted_slots,
                                                                const int* __restrict__ type_offsets,
                                                                const float* __restrict__ reductors, int ne, int R, int d,
-                                                               float* __restrict__ g_rep, int A,
+                                                               float* __restrict__ g_rep, int tiles,
                                                                const int* __restrict__ types, int N, int zero_groups,
                                                                const float* __restrict__ e_slots, int B, int n,
                                                                float* __restrict__ energies) {
-    extern __shared__ float sm[];                      // [d]
-    if ((int)blockIdx.x >= A + zero_groups) {          // spare workgroups: the per-molecule energy sums
-        row_sums(e_slots, B, n, energies, (int)blockIdx.x - A - zero_groups);
+    extern __shared__ float sm[];                      // [NA][d]
+    if ((int)blockIdx.x >= tiles + zero_groups) {      // spare workgroups: the per-molecule energy sums
+        row_sums(e_slots, B, n, energies, (int)blockIdx.x - tiles - zero_groups);
         return;
     }
-    if ((int)blockIdx.x >= A) {
-        zero_untyped_rows(types, N, ne, R, g_rep, (int)blockIdx.x - A);
+    if ((int)blockIdx.x >= tiles) {
+        zero_untyped_rows(types, N, ne, R, g_rep, (int)blockIdx.x - tiles);
         return;
     }
-    const int p = blockIdx.x, tid = threadIdx.x;
-    if (p >= type_offsets[ne]) return;                 // past the sorted list (atoms of no known element)
-    const int e = type_of_position(type_offsets, ne, p);
-    for (int c = tid; c < d; c += 256) sm[c] = gx[(size_t)p * d + c];
+    const int tid = threadIdx.x;
+    int e = -1, row0 = 0, rows = 0;
+    {
+        int b = blockIdx.x;
+        for (int t = 0; t < ne; ++t) {
+            const int o0 = type_offsets[t], o1 = type_offsets[t + 1];
+            const int nt = (o1 - o0 + NA - 1) / NA;
+            if (b < nt) {
+                e = t;
+                row0 = o0 + b * NA;
+                rows = min(NA, o1 - row0);
+                break;
+            }
+            b -= nt;
+        }
+    }
+    if (e < 0) return;                                 // a tile beyond the sorted list
+    for (int i = tid; i < NA * d; i += 256) sm[i] = i < rows * d ? gx[(size_t)row0 * d + i] : 0.0f;
     __syncthreads();
     const float* U = reductors + (size_t)e * R * d;
-    float* out = g_rep + (size_t)sorted_slots[p] * R;
     const float4* g4 = reinterpret_cast<const float4*>(sm);
+    const int d4 = d / 4;
     for (int r = tid; r < R; r += 256) {
         const float4* u4 = reinterpret_cast<const float4*>(U + (size_t)r * d);
-        float a0 = 0.0f, a1 = 0.0f;
-#pragma unroll 8
-        for (int c4 = 0; c4 < d / 4; ++c4) {
-            const float4 u = u4[c4], g = g4[c4];
-            a0 = fmaf(u.x, g.x, fmaf(u.y, g.y, a0));
-            a1 = fmaf(u.z, g.z, fmaf(u.w, g.w, a1));
+        float a0[NA], a1[NA];
+#pragma unroll
+        for (int a = 0; a < NA; ++a) a0[a] = a1[a] = 0.0f;
+#pragma unroll 4
+        for (int c4 = 0; c4 < d4; ++c4) {
+            const float4 u = u4[c4];
+#pragma unroll
+            for (int a = 0; a < NA; ++a) {
+                const float4 g = g4[a * d4 + c4];
+                a0[a] = fmaf(u.x, g.x, fmaf(u.y, g.y, a0[a]));
+                a1[a] = fmaf(u.z, g.z, fmaf(u.w, g.w, a1[a]));
+            }
         }
-        out[r] = a0 + a1;
+#pragma unroll
+        for (int a = 0; a < NA; ++a)
+            if (a < rows) g_rep[(size_t)sorted_slots[row0 + a] * R + r] = a0[a] + a1[a];
     }
 }
 
@@ -1239,7 +1264,7 @@ extern "C" int qmll_project_typed_backward_sums(const float* gx, const int* sort
     const bool sums = energies != nullptr && B > 0;
     QMLL_REQUIRE(!sums || (e_slots && n > 0), QMLL_ERR_INVALID, "qmll_project_typed_backward_sums: energies without e_slots");
     const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(gx) && aligned16(reductors);
-    const bool small = vec && A > 0 && small_batch(A, R, d) && (size_t)d * sizeof(float) <= 64 * 1024 && N <= 256 * 256;
+    const bool small = vec && A > 0 && small_batch(A, R, d) && (size_t)8 * d * sizeof(float) <= 64 * 1024 && N <= 256 * 256;
     if (types && N > 0 && !small) {
         QMLL_REQUIRE(g_rep, QMLL_ERR_INVALID, "qmll_project_typed_backward: null pointer");
         hipLaunchKernelGGL(zero_untyped_rows_kernel, dim3((N + 255) / 256), dim3(256), 0, (hipStream_t)stream, types, N, ne,
@@ -1259,9 +1284,17 @@ extern "C" int qmll_project_typed_backward_sums(const float* gx, const int* sort
         // molecules for the energy sums
         const int zero_groups = (types && N > 0) ? (N + 255) / 256 : 0;
         const int sum_groups = sums ? (B + 255) / 256 : 0;
-        hipLaunchKernelGGL(project_bt_small_kernel, dim3(A + zero_groups + sum_groups), dim3(256), sizeof(float) * d,
-                           (hipStream_t)stream, gx, sorted_slots, type_offsets, reductors, ne, R, d, g_rep, A, types, N,
-                           zero_groups, e_slots, B, n, energies);
+        // atoms per workgroup: one while the atoms are the only parallelism there is, more as the reductor
+        // reads of all workgroups together begin to count
+#define LAUNCH_BT_SMALL(NA)                                                                                         \
+    {                                                                                                               \
+        const int tiles = (A + (NA) - 1) / (NA) + ((NA) > 1 ? ne : 0);                                              \
+        hipLaunchKernelGGL(project_bt_small_kernel<NA>, dim3(tiles + zero_groups + sum_groups), dim3(256),          \
+                           sizeof(float) * (NA) * d, (hipStream_t)stream, gx, sorted_slots, type_offsets, reductors, \
+                           ne, R, d, g_rep, tiles, types, N, zero_groups, e_slots, B, n, energies);                 \
+    }
+        if (A < 64) LAUNCH_BT_SMALL(1) else if (A < 512) LAUNCH_BT_SMALL(4) else LAUNCH_BT_SMALL(8)
+#undef LAUNCH_BT_SMALL
     } else if (vec && (d == 64 || d == 128) && reductors_split) {
         // short contraction: the gradient rows stay in registers, every row is read once
         const SplitLayout L = split_layout(ne, R, d);
