@@ -286,8 +286,9 @@ int qmll_sort_by_type_noalloc(const int* types, const int* slots, int A, int ne,
  *                           (ne = nspecies) and sort_types is not written
  *   sorted_slots i32 [A], type_offsets i32 [ne+1] <- qmll_sort_atoms_by_type by that index
  *   zero f32 [zero_count] <- 0 (the arrays the chain accumulates into)
- * in ONE launch for up to 1024 listed atoms (16 384 slots, 65 536 floats to clear), else as the
- * separate kernels.  workspace: as for qmll_sort_atoms_by_type (none up to 1024 atoms). */
+ * in ONE launch for up to 4096 listed atoms (65 536 slots, 262 144 floats to clear), else as the
+ * separate kernels.  workspace: as for qmll_sort_atoms_by_type (none up to 1024 atoms; not used up to
+ * 4096). */
 int qmll_prepare_batch(const float* Z, const int* natoms, const float* species, int nspecies, const float* model_species,
                        int ne, const int* atomIDs, const int* molIDs, int B, int n, int A, void* workspace,
                        size_t workspace_bytes, int* types, int* sort_types, int* sorted_slots, int* type_offsets,

@@ -163,48 +163,61 @@ __device__ __forceinline__ int species_index(float z, const float* __restrict__ 
 
 // Everything a small padded batch needs before its first compute kernel, in ONE workgroup: the element
 // index of every slot by the representation's species list (and, when the model keeps its own list, by
-// that one too), the listed atoms sorted by the index the model goes by (as type_sort_small_kernel),
-// and a float range set to zero.  Padded slots (beyond natoms of their molecule) get index 0.
+// that one too), the listed atoms sorted by the index the model goes by (stable, as
+// type_sort_small_kernel; up to PREP_CHUNKS rounds of 1024 atoms), and a float range set to zero.
+// Padded slots (beyond natoms of their molecule) get index 0.
+constexpr int PREP_CHUNKS = 4;
 __global__ __launch_bounds__(SORT_SMALL) void prepare_small_kernel(
     const float* __restrict__ Z, const int* __restrict__ natoms, const float* __restrict__ species, int ns,
     const float* __restrict__ model_species, int ne, const int* __restrict__ atomIDs, const int* __restrict__ molIDs, int B,
     int n, int A, int* __restrict__ types, int* __restrict__ sort_types, int* __restrict__ sorted, int* __restrict__ offsets,
     float* __restrict__ zero, int zero_count) {
-    __shared__ int wcnt[SORT_SMALL / 64][MAXNE];
+    __shared__ int wcnt[PREP_CHUNKS][SORT_SMALL / 64][MAXNE];   // atoms of type e in (chunk, wavefront), then: before it
     __shared__ int total[MAXNE], start[MAXNE + 1];
-    const int a = threadIdx.x, lane = a & 63, wave = a >> 6;
-    for (int idx = a; idx < B * n; idx += SORT_SMALL) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int chunks = (A + SORT_SMALL - 1) / SORT_SMALL;
+    for (int idx = tid; idx < B * n; idx += SORT_SMALL) {
         const int m = idx / n;
         const bool real = idx - m * n < natoms[m];
         types[idx] = real ? species_index(Z[idx], species, ns) : 0;
         if (model_species) sort_types[idx] = real ? species_index(Z[idx], model_species, ne) : 0;
     }
-    for (int i = a; i < zero_count; i += SORT_SMALL) zero[i] = 0.0f;
-    int slot = 0, t = -1;
-    if (a < A) {
-        const int m = molIDs[a], i = atomIDs[a];
-        slot = m * n + i;
-        t = i < natoms[m] ? (model_species ? species_index(Z[slot], model_species, ne) : species_index(Z[slot], species, ns))
-                          : 0;
-    }
-    int rank = 0;
-    for (int e = 0; e < ne; ++e) {
-        const unsigned long long mk = __ballot(t == e);
-        if (lane == 0) wcnt[wave][e] = __popcll(mk);
-        if (t == e) rank = __popcll(mk & ((1ull << lane) - 1ull));
-    }
-    __syncthreads();
-    if (a < ne) {
-        int sum = 0;
-        for (int w = 0; w < SORT_SMALL / 64; ++w) {
-            const int c = wcnt[w][a];
-            wcnt[w][a] = sum;
-            sum += c;
+    for (int i = tid; i < zero_count; i += SORT_SMALL) zero[i] = 0.0f;
+    int slot[PREP_CHUNKS], t[PREP_CHUNKS], rank[PREP_CHUNKS];
+#pragma unroll
+    for (int k = 0; k < PREP_CHUNKS; ++k) {
+        slot[k] = 0;
+        t[k] = -1;
+        rank[k] = 0;
+        if (k < chunks) {
+            const int a = k * SORT_SMALL + tid;
+            if (a < A) {
+                const int m = molIDs[a], i = atomIDs[a];
+                slot[k] = m * n + i;
+                t[k] = i < natoms[m] ? (model_species ? species_index(Z[slot[k]], model_species, ne)
+                                                      : species_index(Z[slot[k]], species, ns))
+                                     : 0;
+            }
+            for (int e = 0; e < ne; ++e) {
+                const unsigned long long mk = __ballot(t[k] == e);
+                if (lane == 0) wcnt[k][wave][e] = __popcll(mk);
+                if (t[k] == e) rank[k] = __popcll(mk & ((1ull << lane) - 1ull));
+            }
         }
-        total[a] = sum;
     }
     __syncthreads();
-    if (a == 0) {
+    if (tid < ne) {          // thread e: exclusive prefix of its type over the chunks and wavefronts
+        int sum = 0;
+        for (int k = 0; k < chunks; ++k)
+            for (int w = 0; w < SORT_SMALL / 64; ++w) {
+                const int c = wcnt[k][w][tid];
+                wcnt[k][w][tid] = sum;
+                sum += c;
+            }
+        total[tid] = sum;
+    }
+    __syncthreads();
+    if (tid == 0) {
         int sum = 0;
         for (int e = 0; e < ne; ++e) {
             start[e] = sum;
@@ -213,9 +226,12 @@ __global__ __launch_bounds__(SORT_SMALL) void prepare_small_kernel(
         start[ne] = sum;
     }
     __syncthreads();
-    if (a <= ne) offsets[a] = start[a];
-    if (t >= 0 && t < ne) sorted[start[t] + wcnt[wave][t] + rank] = slot;
-    for (int i = start[ne] + a; i < A; i += SORT_SMALL) sorted[i] = 0;
+    if (tid <= ne) offsets[tid] = start[tid];
+#pragma unroll
+    for (int k = 0; k < PREP_CHUNKS; ++k)
+        if (k < chunks && t[k] >= 0 && t[k] < ne) sorted[start[t[k]] + wcnt[k][wave][t[k]] + rank[k]] = slot[k];
+    // entries past the last typed atom name a valid slot, so gathers through them stay in bounds
+    for (int i = start[ne] + tid; i < A; i += SORT_SMALL) sorted[i] = 0;
 }
 
 __global__ __launch_bounds__(256) void zero_floats_kernel(float* __restrict__ p, size_t count) {
@@ -1042,7 +1058,7 @@ extern "C" int qmll_prepare_batch(const float* Z, const int* natoms, const float
     QMLL_REQUIRE(!model_species || sort_types || (size_t)B * n == 0, QMLL_ERR_INVALID,
                  "qmll_prepare_batch: model species without a sort_types output");
     const size_t slots = (size_t)B * n;
-    if (A > 0 && A <= SORT_SMALL && slots > 0 && slots <= 16384 && zero_count <= 65536) {
+    if (A > 0 && A <= PREP_CHUNKS * SORT_SMALL && slots > 0 && slots <= 65536 && zero_count <= 262144) {
         QMLL_REQUIRE(Z && natoms && atomIDs && molIDs && types && sorted_slots, QMLL_ERR_INVALID,
                      "qmll_prepare_batch: null pointer");
         hipLaunchKernelGGL(prepare_small_kernel, dim3(1), dim3(SORT_SMALL), 0, (hipStream_t)stream, Z, natoms, species, nspecies,
