@@ -234,21 +234,30 @@ __global__ __launch_bounds__(SORT_SMALL) void prepare_small_kernel(
     for (int i = start[ne] + tid; i < A; i += SORT_SMALL) sorted[i] = 0;
 }
 
+// The same bookkeeping for a large batch, short of the sort itself: element indices of every slot, the
+// slot of every listed atom, the zero fill; one grid-stride launch instead of three or four
+__global__ __launch_bounds__(256) void prepare_large_kernel(const float* __restrict__ Z, const int* __restrict__ natoms,
+                                                            const float* __restrict__ species, int ns,
+                                                            const float* __restrict__ model_species, int ne,
+                                                            const int* __restrict__ atomIDs, const int* __restrict__ molIDs,
+                                                            size_t nslots, int n, int A, int* __restrict__ types,
+                                                            int* __restrict__ sort_types, int* __restrict__ slots,
+                                                            float* __restrict__ zero, size_t zero_count) {
+    const size_t first = (size_t)blockIdx.x * 256 + threadIdx.x, step = (size_t)gridDim.x * 256;
+    for (size_t idx = first; idx < nslots; idx += step) {
+        const size_t m = idx / n;
+        const bool real = (int)(idx - m * n) < natoms[m];
+        types[idx] = real ? species_index(Z[idx], species, ns) : 0;
+        if (model_species) sort_types[idx] = real ? species_index(Z[idx], model_species, ne) : 0;
+    }
+    for (size_t a = first; a < (size_t)A; a += step) slots[a] = molIDs[a] * n + atomIDs[a];
+    for (size_t i = first; i < zero_count; i += step) zero[i] = 0.0f;
+}
+
 __global__ __launch_bounds__(256) void zero_floats_kernel(float* __restrict__ p, size_t count) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (size_t)gridDim.x * 256) p[i] = 0.0f;
 }
 
-// sums[m] = sum_i values[m*n + i]: thread = row (the per-molecule energy of a padded batch)
-__device__ __forceinline__ void row_sums(const float* __restrict__ values, int B, int n, float* __restrict__ sums, int chunk) {
-    const int m = chunk * 256 + threadIdx.x;
-    if (m >= B) return;
-    float acc = 0.0f;
-    for (int i = 0; i < n; ++i) acc += values[(size_t)m * n + i];
-    sums[m] = acc;
-}
-__global__ __launch_bounds__(256) void row_sums_kernel(const float* __restrict__ values, int B, int n, float* __restrict__ sums) {
-    row_sums(values, B, n, sums, blockIdx.x);
-}
 
 // ---- typed GEMM -------------------------------------------------------------------------
 constexpr int PT = 256;            // threads (4 wavefronts, each 32 rows x 64 columns)
@@ -829,6 +838,14 @@ __global__ __launch_bounds__(PT) void typed_gemm_bt_rows_f16_kernel(const float*
     }
 }
 
+// sums[m] = sum_i values[m*n + i]: thread = row (the per-molecule energy of a padded batch)
+__device__ __forceinline__ void row_sums(const float* __restrict__ values, int B, int n, float* __restrict__ sums, int chunk) {
+    const int m = chunk * 256 + threadIdx.x;
+    if (m >= B) return;
+    float acc = 0.0f;
+    for (int i = 0; i < n; ++i) acc += values[(size_t)m * n + i];
+    sums[m] = acc;
+}
 // rows of real atoms whose element the model does not know get a zero gradient
 // (lane = slot; the rare untyped slots of a wavefront are then zeroed row by row by all lanes)
 __device__ __forceinline__ void zero_untyped_rows(const int* __restrict__ types, int N, int ne, int R,
@@ -846,8 +863,13 @@ __device__ __forceinline__ void zero_untyped_rows(const int* __restrict__ types,
 }
 
 __global__ __launch_bounds__(256) void zero_untyped_rows_kernel(const int* __restrict__ types, int N, int ne, int R,
-                                                                float* __restrict__ out) {
-    zero_untyped_rows(types, N, ne, R, out, blockIdx.x);
+                                                                float* __restrict__ out, int zero_groups,
+                                                                const float* __restrict__ e_slots, int B, int n,
+                                                                float* __restrict__ energies) {
+    if ((int)blockIdx.x < zero_groups)
+        zero_untyped_rows(types, N, ne, R, out, blockIdx.x);
+    else                                               // workgroups past the slots: the per-molecule energy sums
+        row_sums(e_slots, B, n, energies, (int)blockIdx.x - zero_groups);
 }
 
 // Small batches (a molecule to a few dozen): the tiled kernels above run a few workgroups through
@@ -1067,21 +1089,39 @@ extern "C" int qmll_prepare_batch(const float* Z, const int* natoms, const float
         QMLL_CHECK_LAUNCH("qmll_prepare_batch");
         return QMLL_OK;
     }
-    int rc = qmll_element_types(Z, natoms, species, B, n, nspecies, types, stream);
-    if (rc != QMLL_OK) return rc;
-    if (model_species) {
-        rc = qmll_element_types(Z, natoms, model_species, B, n, ne, sort_types, stream);
+    if (A == 0 || slots == 0) {               // nothing listed: clear what was asked and write the offsets
+        int rc = qmll_element_types(Z, natoms, species, B, n, nspecies, types, stream);
         if (rc != QMLL_OK) return rc;
+        if (model_species) {
+            rc = qmll_element_types(Z, natoms, model_species, B, n, ne, sort_types, stream);
+            if (rc != QMLL_OK) return rc;
+        }
+        if (zero_count > 0) {
+            const size_t groups = (zero_count + 255) / 256;
+            hipLaunchKernelGGL(zero_floats_kernel, dim3((unsigned)(groups < 4096 ? groups : 4096)), dim3(256), 0,
+                               (hipStream_t)stream, zero, zero_count);
+            QMLL_CHECK_LAUNCH("qmll_prepare_batch");
+        }
+        return qmll_sort_atoms_by_type(model_species ? sort_types : types, atomIDs, molIDs, n > 0 ? n : 1, 0, ne, workspace,
+                                       workspace_bytes, sorted_slots, type_offsets, stream);
     }
-    if (zero_count > 0) {
-        const size_t groups = (zero_count + 255) / 256;
-        hipLaunchKernelGGL(zero_floats_kernel, dim3((unsigned)(groups < 4096 ? groups : 4096)), dim3(256), 0,
-                           (hipStream_t)stream, zero, zero_count);
-        QMLL_CHECK_LAUNCH("qmll_prepare_batch");
-    }
-    if (n == 0) n = 1;                        // an empty batch: the sort below only writes the offsets
-    return qmll_sort_atoms_by_type(model_species ? sort_types : types, atomIDs, molIDs, n, A, ne, workspace, workspace_bytes,
-                                   sorted_slots, type_offsets, stream);
+    QMLL_REQUIRE(Z && natoms && atomIDs && molIDs && types && sorted_slots, QMLL_ERR_INVALID,
+                 "qmll_prepare_batch: null pointer");
+    const size_t need = qmll_sort_atoms_workspace(A, ne);
+    QMLL_REQUIRE(workspace && workspace_bytes >= need, QMLL_ERR_INVALID,
+                 "qmll_prepare_batch: workspace of %zu bytes, %zu needed", workspace_bytes, need);
+    // the slots of the listed atoms go behind the counts of the general sort, as in qmll_sort_atoms_by_type
+    const size_t counts_bytes = qmll_sort_by_type_workspace(A, ne);
+    int* atom_slots = reinterpret_cast<int*>(static_cast<char*>(workspace) + counts_bytes);
+    size_t work = slots > zero_count ? slots : zero_count;
+    if ((size_t)A > work) work = (size_t)A;
+    const size_t groups = (work + 255) / 256;
+    hipLaunchKernelGGL(prepare_large_kernel, dim3((unsigned)(groups < 8192 ? groups : 8192)), dim3(256), 0, (hipStream_t)stream,
+                       Z, natoms, species, nspecies, model_species, ne, atomIDs, molIDs, slots, n, A, types, sort_types,
+                       atom_slots, zero, zero_count);
+    QMLL_CHECK_LAUNCH("qmll_prepare_batch");
+    return qmll_sort_by_type(model_species ? sort_types : types, atom_slots, A, ne, workspace, counts_bytes, sorted_slots,
+                             type_offsets, stream);
 }
 
 // ---- the same sort for callers that cannot allocate -------------------------------------
@@ -1281,15 +1321,14 @@ extern "C" int qmll_project_typed_backward_sums(const float* gx, const int* sort
     QMLL_REQUIRE(!sums || (e_slots && n > 0), QMLL_ERR_INVALID, "qmll_project_typed_backward_sums: energies without e_slots");
     const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(gx) && aligned16(reductors);
     const bool small = vec && A > 0 && small_batch(A, R, d) && (size_t)8 * d * sizeof(float) <= 64 * 1024 && N <= 256 * 256;
-    if (types && N > 0 && !small) {
-        QMLL_REQUIRE(g_rep, QMLL_ERR_INVALID, "qmll_project_typed_backward: null pointer");
-        hipLaunchKernelGGL(zero_untyped_rows_kernel, dim3((N + 255) / 256), dim3(256), 0, (hipStream_t)stream, types, N, ne,
-                           R, g_rep);
+    if (!small && ((types && N > 0) || sums)) {
+        // the rows of unknown elements and the energy sums: one launch for the two
+        const int zero_groups = (types && N > 0) ? (N + 255) / 256 : 0;
+        const int sum_groups = sums ? (B + 255) / 256 : 0;
+        QMLL_REQUIRE(g_rep || zero_groups == 0, QMLL_ERR_INVALID, "qmll_project_typed_backward: null pointer");
+        hipLaunchKernelGGL(zero_untyped_rows_kernel, dim3(zero_groups + sum_groups), dim3(256), 0, (hipStream_t)stream, types,
+                           N, ne, R, g_rep, zero_groups, e_slots, B, n, energies);
         QMLL_CHECK_LAUNCH("qmll_project_typed_backward");
-    }
-    if (sums && !small) {
-        hipLaunchKernelGGL(row_sums_kernel, dim3((B + 255) / 256), dim3(256), 0, (hipStream_t)stream, e_slots, B, n, energies);
-        QMLL_CHECK_LAUNCH("qmll_project_typed_backward_sums");
     }
     if (A == 0) return QMLL_OK;
     QMLL_REQUIRE(gx && sorted_slots && type_offsets && reductors && g_rep, QMLL_ERR_INVALID,
