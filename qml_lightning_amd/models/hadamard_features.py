@@ -319,6 +319,19 @@ def _normalisation_tensor(npcas, sigma):
     return t
 
 
+@torch.jit.ignore
+def _eager_constants(model, device: torch.device, cell: Optional[torch.Tensor], inv_cell: Optional[torch.Tensor]):
+    if cell is None:
+        cell = _no_cells(device)
+    if inv_cell is None:
+        inv_cell = _no_cells(device)
+    if isinstance(model.sigma, float):
+        cn = _normalisation_tensor(model.npcas, model.sigma)
+    else:
+        cn = torch.sqrt(torch.tensor(model.npcas)) / model.sigma
+    return cell, inv_cell, cn, alpha_f32(model)
+
+
 class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
 
     fused: Final[bool]
@@ -402,10 +415,17 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
     def forward(self, X, Z, atomIDs, molIDs, atom_counts, cell: Optional[torch.Tensor] = None,
                 inv_cell: Optional[torch.Tensor] = None):
         """Total energies [B] (fp32), differentiable in X (hadamard_features.py:82-123)."""
-        if cell is None:
-            cell = torch.empty(0, 3, 3, device=X.device)
-        if inv_cell is None:
-            inv_cell = torch.empty(0, 3, 3, device=X.device)
+        if torch.jit.is_scripting():
+            if cell is None:
+                cell = torch.empty(0, 3, 3, device=X.device)
+            if inv_cell is None:
+                inv_cell = torch.empty(0, 3, 3, device=X.device)
+            coeff_normalisation = torch.sqrt(torch.tensor(self.npcas)) / self.sigma
+            alpha = self.alpha.float()
+        else:
+            # the same values without building them per call (a single molecule's step is as long as its
+            # host side): the empty cell tensor and the normalisation are kept, alpha converted once per value
+            cell, inv_cell, coeff_normalisation, alpha = _eager_constants(self, X.device, cell, inv_cell)
         assert X.is_cuda, "X tensor must reside on GPU"
         assert Z.is_cuda, "Z tensor must reside on GPU"
         assert atomIDs.is_cuda, "atomIDs tensor must reside on GPU"
@@ -413,9 +433,6 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
         assert atom_counts.is_cuda, "atom_counts tensor must reside on GPU"
         assert cell.is_cuda, "cell tensor must reside on GPU"
         assert inv_cell.is_cuda, "inv_cell tensor must reside on GPU"
-
-        coeff_normalisation = torch.sqrt(torch.tensor(self.npcas)) / self.sigma
-        alpha = self.alpha.float()
 
         if self.fused and not self.separate_ops:
             # the whole chain below (representation, sort by element, projection, SORF + cos +
