@@ -78,6 +78,9 @@ CASES = {
     "many_bins": lambda: (helpers.fixed_composition_batch(helpers.ASPIRIN, 2, 6), [1, 6, 8], {"nRs2": 80, "nRs3": 70}),
     # 33 to 64 three-body bins: one triple per round, one bin block
     "forty_bins": lambda: (helpers.fixed_composition_batch(helpers.ASPIRIN, 1, 7), [1, 6, 8], {"nRs2": 33, "nRs3": 40}),
+    # narrow three-body Gaussians: sqrt(eta3 log2 e) rcut / 2 = 12.5 is beyond what the backward kernel's
+    # form about the middle of the grid takes (10), so its plain radial loop runs
+    "sharp_radial": lambda: (helpers.fixed_composition_batch(helpers.ASPIRIN, 2, 8), [1, 6, 8], {"eta3": 12.0}),
 }
 
 
