@@ -1094,7 +1094,7 @@ def test_transposed_projection_with_the_energy_sums_in_the_same_call():
     of the small-batch switch; rows of atoms whose element the model does not hold come out zero."""
     from qml_lightning_amd import ops
     g = torch.Generator(device=dev()).manual_seed(3)
-    for B, n in ((1, 21), (48, 21), (400, 21)):
+    for B, n in ((1, 21), (10, 21), (48, 21), (400, 21)):      # one, four, eight atoms per workgroup; the tiled kernel
         N = B * n
         types = torch.randint(-1, 3, (N,), device=dev(), generator=g, dtype=torch.int32)
         slots = torch.arange(N, device=dev(), dtype=torch.int32)
