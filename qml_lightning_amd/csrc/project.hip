@@ -250,7 +250,8 @@ __global__ __launch_bounds__(256) void prepare_large_kernel(const float* __restr
         types[idx] = real ? species_index(Z[idx], species, ns) : 0;
         if (model_species) sort_types[idx] = real ? species_index(Z[idx], model_species, ne) : 0;
     }
-    for (size_t a = first; a < (size_t)A; a += step) slots[a] = molIDs[a] * n + atomIDs[a];
+    if (slots)
+        for (size_t a = first; a < (size_t)A; a += step) slots[a] = molIDs[a] * n + atomIDs[a];
     for (size_t i = first; i < zero_count; i += step) zero[i] = 0.0f;
 }
 
@@ -1107,12 +1108,14 @@ extern "C" int qmll_prepare_batch(const float* Z, const int* natoms, const float
     }
     QMLL_REQUIRE(Z && natoms && atomIDs && molIDs && types && sorted_slots, QMLL_ERR_INVALID,
                  "qmll_prepare_batch: null pointer");
+    // few listed atoms in a batch with many slots (heavy padding): the one-workgroup sort needs no workspace and
+    // builds the slots itself; else they go behind the counts of the general sort, as in qmll_sort_atoms_by_type
+    const bool one_workgroup_sort = A <= SORT_SMALL;
     const size_t need = qmll_sort_atoms_workspace(A, ne);
-    QMLL_REQUIRE(workspace && workspace_bytes >= need, QMLL_ERR_INVALID,
+    QMLL_REQUIRE(one_workgroup_sort || (workspace && workspace_bytes >= need), QMLL_ERR_INVALID,
                  "qmll_prepare_batch: workspace of %zu bytes, %zu needed", workspace_bytes, need);
-    // the slots of the listed atoms go behind the counts of the general sort, as in qmll_sort_atoms_by_type
     const size_t counts_bytes = qmll_sort_by_type_workspace(A, ne);
-    int* atom_slots = reinterpret_cast<int*>(static_cast<char*>(workspace) + counts_bytes);
+    int* atom_slots = one_workgroup_sort ? nullptr : reinterpret_cast<int*>(static_cast<char*>(workspace) + counts_bytes);
     size_t work = slots > zero_count ? slots : zero_count;
     if ((size_t)A > work) work = (size_t)A;
     const size_t groups = (work + 255) / 256;
@@ -1120,6 +1123,9 @@ extern "C" int qmll_prepare_batch(const float* Z, const int* natoms, const float
                        Z, natoms, species, nspecies, model_species, ne, atomIDs, molIDs, slots, n, A, types, sort_types,
                        atom_slots, zero, zero_count);
     QMLL_CHECK_LAUNCH("qmll_prepare_batch");
+    if (one_workgroup_sort)
+        return qmll_sort_atoms_by_type(model_species ? sort_types : types, atomIDs, molIDs, n, A, ne, nullptr, 0, sorted_slots,
+                                       type_offsets, stream);
     return qmll_sort_by_type(model_species ? sort_types : types, atom_slots, A, ne, workspace, counts_bytes, sorted_slots,
                              type_offsets, stream);
 }

@@ -1055,6 +1055,26 @@ def test_a_non_finite_row_spoils_only_itself_in_the_fp16_matrix_core_kernels():
     assert (e1[slot_keep] - e0[slot_keep]).abs().max() <= 1e-6 * e0.abs().max()
 
 
+def test_batch_preparation_of_few_atoms_among_many_padded_slots():
+    """700 listed atoms (no sort workspace is asked for up to 1024) in 70 000 slots (more than the
+    one-workgroup form takes): the general form without a workspace."""
+    from qml_lightning_amd import ops
+    B, n = 700, 100
+    rng = np.random.default_rng(2)
+    Z = np.zeros((B, n), np.float32)
+    Z[:, 0] = rng.choice([1.0, 6.0, 8.0], size=B)
+    t = lambda a: torch.tensor(a, device=dev())
+    counts = t(np.ones(B, np.int32))
+    ai, mi = t(np.zeros(B, np.int32)), t(np.arange(B, dtype=np.int32))
+    species = t(np.array([1.0, 6.0, 8.0], np.float32))
+    types, stypes, ss, off, zero = ops.prepare_batch(t(Z), counts, species, ai, mi, None, 4 * B * n)
+    want = ops.element_types(torch.zeros(B, n, 3, device=dev()), t(Z), counts, species)
+    assert torch.equal(types, want) and stypes is types
+    want_ss, want_off = ops.sort_atoms_by_type(want, ai, mi, n, 3)
+    assert torch.equal(off, want_off) and torch.equal(ss, want_ss)
+    assert zero.shape[0] == 4 * B * n and not zero.any()
+
+
 @pytest.mark.parametrize("nmol,model_list", [(1, None), (40, None), (40, [8.0, 1.0]), (300, [6.0, 9.0, 1.0]), (0, None)])
 def test_batch_preparation_in_one_call_equals_the_separate_kernels(nmol, model_list):
     """qmll_prepare_batch (element indices by the representation's and by the model's species, the
