@@ -873,14 +873,16 @@ __global__ __launch_bounds__(256) void zero_untyped_rows_kernel(const int* __res
         row_sums(e_slots, B, n, energies, (int)blockIdx.x - zero_groups);
 }
 
-// Small batches (a molecule to a few dozen): the tiled kernels above run a few workgroups through
-// ten dependent load-and-multiply steps, 17-26 us for 21 atoms.  Here a workgroup takes ONE atom and
-// spreads the contraction over its threads, so all loads of an atom are in flight at once.
-// above these, the reductor re-reads from L2 (R d floats per atom) outweigh the latency: measured
-// cross-over near 1500 atoms at R d = 40 000 (0.077 against 0.100 ms per predict step at 1008 atoms,
-// 0.149 against 0.131 at 2688)
-constexpr int SMALL_ATOMS = 2048;
-constexpr size_t SMALL_READS = 48u << 20;   // floats of reductor read by all workgroups together
+// Small batches (a molecule to a few thousand atoms): the tiled kernels above run a few workgroups
+// through ten dependent load-and-multiply steps, 17-26 us for 21 atoms and 20 / 14-18 us (forward /
+// transposed) up to 8000.  Here a workgroup takes one to eight atoms of one element and spreads the
+// contraction over its threads, so all loads of an atom are in flight at once and a reductor read serves
+// the workgroup's atoms.  Beyond these limits the reductor re-reads from L2 (R d floats per workgroup)
+// outweigh the latency: measured at R d = 40 000, forward 13 against 20 us up to 4000 atoms, 15 against 21
+// at 5400, 25 against 21 at 8000; transposed 12 against 14 at 2000, 16 against 18 at 4000, 20 against 18
+// at 5400
+constexpr int SMALL_ATOMS = 4096;
+constexpr size_t SMALL_READS = 192u << 20;   // floats of reductor per atom times atoms
 __host__ inline bool small_batch(int A, int R, int d) { return A <= SMALL_ATOMS && (size_t)A * R * d <= SMALL_READS; }
 constexpr int SMALL_KS = 8;        // slices of the contraction in project_small_kernel
 
@@ -890,42 +892,71 @@ __device__ __forceinline__ int type_of_position(const int* __restrict__ type_off
     return e;
 }
 
-// x[p, :] = rep[slot(p), :] . U_e: thread = (contraction slice, four columns), slices folded through LDS
+// NA consecutive sorted atoms of one element for workgroup b (tiles never straddle two elements)
+template <int NA>
+__device__ __forceinline__ bool small_tile(const int* __restrict__ type_offsets, int ne, int b, int& e, int& row0, int& rows) {
+    for (int t = 0; t < ne; ++t) {
+        const int o0 = type_offsets[t], o1 = type_offsets[t + 1];
+        const int nt = (o1 - o0 + NA - 1) / NA;
+        if (b < nt) {
+            e = t;
+            row0 = o0 + b * NA;
+            rows = min(NA, o1 - row0);
+            return true;
+        }
+        b -= nt;
+    }
+    return false;                                      // a tile beyond the sorted list
+}
+
+// x[p, :] = rep[slot(p), :] . U_e: thread = (contraction slice, four columns), slices folded through LDS;
+// a workgroup takes NA atoms of one element, so a reductor read serves them all
+template <int NA>
 __global__ __launch_bounds__(256) void project_small_kernel(const float* __restrict__ rep,
                                                             const int* __restrict__ sorted_slots,
                                                             const int* __restrict__ type_offsets,
                                                             const float* __restrict__ reductors, int ne, int R, int d,
                                                             float* __restrict__ x) {
     extern __shared__ float sm[];
-    float* srow = sm;                                  // [R]
-    float* spart = sm + ((R + 3) & ~3);                // [SMALL_KS][d]
-    const int p = blockIdx.x, tid = threadIdx.x;
-    if (p >= type_offsets[ne]) return;                 // past the sorted list (atoms of no known element)
-    const int e = type_of_position(type_offsets, ne, p);
-    const float* row = rep + (size_t)sorted_slots[p] * R;
-    for (int k = tid; k < R; k += 256) srow[k] = row[k];
+    const int R4 = (R + 3) & ~3;
+    float* srow = sm;                                  // [NA][R4]
+    float* spart = sm + NA * R4;                       // [SMALL_KS][NA][d]
+    const int tid = threadIdx.x;
+    int e, row0, rows;
+    if (!small_tile<NA>(type_offsets, ne, blockIdx.x, e, row0, rows)) return;
+    for (int a = 0; a < NA; ++a) {
+        const float* row = rep + (size_t)sorted_slots[row0 + (a < rows ? a : 0)] * R;
+        for (int k = tid; k < R; k += 256) srow[a * R4 + k] = a < rows ? row[k] : 0.0f;
+    }
     __syncthreads();
     const float* U = reductors + (size_t)e * R * d;
     const int ks = tid >> 5, l32 = tid & 31;
     for (int c4 = l32; c4 < d / 4; c4 += 32) {
-        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll 8
+        float4 acc[NA];
+#pragma unroll
+        for (int a = 0; a < NA; ++a) acc[a] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 4
         for (int k = ks; k < R; k += SMALL_KS) {
             const float4 u = *reinterpret_cast<const float4*>(U + (size_t)k * d + 4 * c4);
-            const float r = srow[k];
-            acc.x = fmaf(r, u.x, acc.x);
-            acc.y = fmaf(r, u.y, acc.y);
-            acc.z = fmaf(r, u.z, acc.z);
-            acc.w = fmaf(r, u.w, acc.w);
+#pragma unroll
+            for (int a = 0; a < NA; ++a) {
+                const float r = srow[a * R4 + k];
+                acc[a].x = fmaf(r, u.x, acc[a].x);
+                acc[a].y = fmaf(r, u.y, acc[a].y);
+                acc[a].z = fmaf(r, u.z, acc[a].z);
+                acc[a].w = fmaf(r, u.w, acc[a].w);
+            }
         }
-        *reinterpret_cast<float4*>(spart + ks * d + 4 * c4) = acc;
+#pragma unroll
+        for (int a = 0; a < NA; ++a) *reinterpret_cast<float4*>(spart + ((size_t)ks * NA + a) * d + 4 * c4) = acc[a];
     }
     __syncthreads();
-    for (int c = tid; c < d; c += 256) {
+    for (int i = tid; i < rows * d; i += 256) {
+        const int a = i / d, c = i - a * d;
         float sum = 0.0f;
 #pragma unroll
-        for (int q = 0; q < SMALL_KS; ++q) sum += spart[q * d + c];
-        x[(size_t)p * d + c] = sum;
+        for (int q = 0; q < SMALL_KS; ++q) sum += spart[((size_t)q * NA + a) * d + c];
+        x[(size_t)(row0 + a) * d + c] = sum;
     }
 }
 
@@ -953,22 +984,8 @@ __global__ __launch_bounds__(256) void project_bt_small_kernel(const float* __re
         return;
     }
     const int tid = threadIdx.x;
-    int e = -1, row0 = 0, rows = 0;
-    {
-        int b = blockIdx.x;
-        for (int t = 0; t < ne; ++t) {
-            const int o0 = type_offsets[t], o1 = type_offsets[t + 1];
-            const int nt = (o1 - o0 + NA - 1) / NA;
-            if (b < nt) {
-                e = t;
-                row0 = o0 + b * NA;
-                rows = min(NA, o1 - row0);
-                break;
-            }
-            b -= nt;
-        }
-    }
-    if (e < 0) return;                                 // a tile beyond the sorted list
+    int e, row0, rows;
+    if (!small_tile<NA>(type_offsets, ne, blockIdx.x, e, row0, rows)) return;
     for (int i = tid; i < NA * d; i += 256) sm[i] = i < rows * d ? gx[(size_t)row0 * d + i] : 0.0f;
     __syncthreads();
     const float* U = reductors + (size_t)e * R * d;
@@ -1245,10 +1262,25 @@ extern "C" int qmll_project_typed(const float* rep, const int* sorted_slots, con
                  "qmll_project_typed: null pointer");
     const bool vec = R % 4 == 0 && d % 4 == 0 && aligned16(rep) && aligned16(reductors);
     if (vec && small_batch(A, R, d)) {
-        const size_t lds = sizeof(float) * (((size_t)R + 3) / 4 * 4 + (size_t)SMALL_KS * d);
-        if (lds <= 64 * 1024) {
-            hipLaunchKernelGGL(project_small_kernel, dim3(A), dim3(256), lds, (hipStream_t)stream, rep, sorted_slots,
-                               type_offsets, reductors, ne, R, d, x);
+        // several atoms of one element per workgroup from some hundreds of atoms on, while their rows and partial
+        // sums fit in LDS
+        const size_t per_atom = sizeof(float) * (((size_t)R + 3) / 4 * 4 + (size_t)SMALL_KS * d);
+        // (measured at 312 x 128: one atom 8.4 us at 1008 atoms and 12.8 at 2016, two 8.1 / 8.7, four 10.2 / 10.7 and
+        // 11.8 at 4032, where two take 13.8; eight are never the fastest: the loads here are coalesced, the
+        // multiplications of a workgroup are what grows)
+        int na = A <= 768 ? 1 : (A <= 2304 ? 2 : 4);
+        while (na > 1 && na * per_atom > 64 * 1024) na >>= 1;
+        if (per_atom <= 64 * 1024) {
+            const dim3 grid((A + na - 1) / na + (na > 1 ? ne : 0));
+            if (na == 1)
+                hipLaunchKernelGGL(project_small_kernel<1>, grid, dim3(256), per_atom, (hipStream_t)stream, rep, sorted_slots,
+                                   type_offsets, reductors, ne, R, d, x);
+            else if (na == 2)
+                hipLaunchKernelGGL(project_small_kernel<2>, grid, dim3(256), 2 * per_atom, (hipStream_t)stream, rep,
+                                   sorted_slots, type_offsets, reductors, ne, R, d, x);
+            else
+                hipLaunchKernelGGL(project_small_kernel<4>, grid, dim3(256), 4 * per_atom, (hipStream_t)stream, rep,
+                                   sorted_slots, type_offsets, reductors, ne, R, d, x);
             QMLL_CHECK_LAUNCH("qmll_project_typed");
             return QMLL_OK;
         }

@@ -506,9 +506,12 @@ def test_sort_atoms_by_type_equals_the_sort_of_their_slots(B, n, ne):
                                         # small batches: one workgroup per atom instead of matrix tiles
                                         (312, 128, 3, 100, 100), (312, 128, 3, 140, 128), (312, 128, 3, 1300, 1201),
                                         (312, 64, 2, 40, 21), (720, 256, 5, 60, 33), (76, 20, 2, 30, 17),
-                                        # large enough for the matrix tiles at 128 and 64 components (rows in registers
-                                        # in the transpose), and the last size the small kernels take at 312 x 128
-                                        (312, 128, 3, 3000, 2900), (312, 64, 3, 2600, 2500), (312, 128, 3, 1300, 1260)])
+                                        (312, 128, 3, 3000, 2900), (312, 64, 3, 2600, 2500), (312, 128, 3, 1300, 1260),
+                                        # the last size the small kernels take (eight atoms per workgroup), and
+                                        # large enough for the matrix tiles at 128 and 64 components (rows in
+                                        # registers in the transpose); 720 x 256: four atoms per workgroup fit in LDS
+                                        (312, 128, 3, 4200, 4096), (312, 128, 3, 5000, 4900), (312, 64, 3, 4600, 4500),
+                                        (720, 256, 5, 1100, 1000), (720, 256, 5, 1300, 1200)])
 def test_project_typed_forward_and_backward(R, d, ne, N, A):
     """Element-sorted projection against fp64 matmul, both directions: gathered rows, tiles that end
     inside a type, R not a multiple of 4, unknown elements; the matrix-core kernels and the
