@@ -878,9 +878,9 @@ __global__ __launch_bounds__(256) void zero_untyped_rows_kernel(const int* __res
 // transposed) up to 8000.  Here a workgroup takes one to eight atoms of one element and spreads the
 // contraction over its threads, so all loads of an atom are in flight at once and a reductor read serves
 // the workgroup's atoms.  Beyond these limits the reductor re-reads from L2 (R d floats per workgroup)
-// outweigh the latency: measured at R d = 40 000, forward 13 against 20 us up to 4000 atoms, 15 against 21
-// at 5400, 25 against 21 at 8000; transposed 12 against 14 at 2000, 16 against 18 at 4000, 20 against 18
-// at 5400
+// outweigh the latency: measured at R d = 40 000, forward 9 against 20 us at 2000 atoms, 12 against 20 at
+// 4000, 15 against 21 at 5400 (eight atoms per workgroup; four were not tried there), 25 against 21 at
+// 8000; transposed 12 against 14 at 2000, 16 against 18 at 4000, 20 against 18 at 5400
 constexpr int SMALL_ATOMS = 4096;
 constexpr size_t SMALL_READS = 192u << 20;   // floats of reductor per atom times atoms
 __host__ inline bool small_batch(int A, int R, int d) { return A <= SMALL_ATOMS && (size_t)A * R * d <= SMALL_READS; }
