@@ -81,6 +81,38 @@ def test_reader_reproduces_the_fixture_from_the_reference_held_file(kat):
         "qml_lightning_sorf::get_cos_features": 1}
 
 
+REF_FILE_2 = "/root/reference/examples/MD17/model_sorf.pt"
+
+
+@pytest.mark.skipif(not os.path.exists(REF_FILE_2), reason="the reference checkout is not here")
+def test_reader_on_the_references_second_model_file():
+    """examples/MD17/model_sorf.pt: other weights, no expected outputs with it; the reader finds the same
+    layout, operators and hyper-parameters, orthonormal reductor columns and +-1 diagonals, and
+    from_reference_file builds a trained model from it."""
+    tree = model_files.read_attribute_tree(REF_FILE_2)
+    assert tree["__class__"] == "__torch__.qml_lightning.models.hadamard_features.HadamardFeaturesModel"
+    assert _layout(tree, REFERENCE_LAYOUT) == REFERENCE_LAYOUT
+    assert _layout(tree["rep"], REFERENCE_REP_LAYOUT) == REFERENCE_REP_LAYOUT
+    for k, t in REFERENCE_SCALARS.items():
+        assert type(tree[k]) is t, k
+    assert set(model_files.check_reference_loadable(REF_FILE_2)) == {
+        "qml_lightning_fchl::fchl_forwards", "qml_lightning_sorf::get_SORF_coefficients",
+        "qml_lightning_sorf::get_cos_features"}
+    ne, R, d = tree["reductors"].shape
+    assert (ne, d) == (len(tree["elements"]), tree["npcas"]) and R == tree["rep"]["fp_size"]
+    U = tree["reductors"].astype(np.float64)
+    for e in range(ne):
+        assert np.abs(U[e].T @ U[e] - np.eye(d)).max() < 5e-3
+    assert set(np.unique(tree["Dmat"])) <= {-1.0, 1.0}
+    assert tree["Dmat"].shape == (ne, int(tree["ntransforms"]), tree["nstacks"], d)
+    assert tree["bias"].shape == (ne, tree["nstacks"] * d) and 0.0 <= tree["bias"].min() and tree["bias"].max() <= 2 * np.pi
+    assert tree["alpha"].shape == (tree["nstacks"] * d,) and tree["alpha"].dtype == np.float64
+    from qml_lightning_amd.models.hadamard_features import HadamardFeaturesModel
+    m = HadamardFeaturesModel.from_reference_file(REF_FILE_2)
+    assert m.is_trained and m.nfeatures() == tree["nstacks"] * d
+    assert np.array_equal(m.alpha.cpu().numpy(), tree["alpha"])
+
+
 @needs_reference
 def test_from_reference_file_builds_the_model_of_the_known_answer_test(kat):
     from qml_lightning_amd.models.hadamard_features import HadamardFeaturesModel
