@@ -85,6 +85,13 @@ Tensor prepared_form(const Tensor& t, int kind, const std::function<Tensor(const
     return buffer;
 }
 
+// alpha as the kernels contract with it (fp32): a model stores it in fp64 (qml_lightning/models/kernel.py:226-234),
+// and the conversion, a launch per call otherwise, is kept per tensor version like the other prepared constants
+Tensor alpha32(const Tensor& alpha) {
+    if (alpha.scalar_type() == at::kFloat) return alpha.contiguous();
+    return prepared_form(alpha, 3, [](const Tensor& a) { return a.to(at::kFloat).contiguous(); });
+}
+
 // ---- FCHL19 -----------------------------------------------------------------------------
 struct FchlInputs {
     Tensor X, types, cell, inv_cell, atomIDs, molIDs, natoms, Rs2, Rs3;
@@ -340,7 +347,7 @@ Tensor empty_like_none(const Tensor& like) { return at::empty({0}, like.options(
 
 std::tuple<Tensor, Tensor> sorf_energy_impl(const Tensor& sub, const Tensor& D, const Tensor& bias, const Tensor& alpha,
                                             const Tensor& cn, const Tensor& nt) {
-    Tensor x = f32(sub), DD = f32(D), bb = f32(bias), al = f32(alpha);
+    Tensor x = f32(sub), DD = f32(D), bb = f32(bias), al = alpha32(alpha);
     need_cuda(x, "sub");
     const int A = (int)x.size(0), d = (int)x.size(1), S = (int)DD.size(1), T = nt.item<int>();
     TORCH_CHECK(DD.dim() == 3 && DD.size(2) == d && T <= DD.size(0) && bb.numel() == (int64_t)S * d &&
@@ -379,7 +386,7 @@ std::tuple<Tensor, Tensor> sorf_energy(const Tensor& sub, const Tensor& D, const
 std::tuple<Tensor, Tensor> sorf_energy_typed_impl(const Tensor& x_all, const Tensor& types, const Tensor& atom_slots,
                                                   const Tensor& Dmat, const Tensor& bias, const Tensor& alpha,
                                                   const Tensor& cn, const Tensor& nt, bool with_grad) {
-    Tensor x = f32(x_all), DD = f32(Dmat), bb = f32(bias), al = f32(alpha);
+    Tensor x = f32(x_all), DD = f32(Dmat), bb = f32(bias), al = alpha32(alpha);
     need_cuda(x, "x_all");
     Tensor ty = i32(types).reshape({-1}), sl = i32(atom_slots);
     const int ne = (int)DD.size(0), Tn = (int)DD.size(1), S = (int)DD.size(2), d = (int)DD.size(3);
@@ -527,7 +534,7 @@ Tensor project_typed(const Tensor& rep, const Tensor& ss, const Tensor& off, con
 // e f32 [nslots] zero-filled, gx f32 [A,d] or nullptr
 void sorf_energy_sorted_raw(const float* x, const int* off, const int* ss, int A, int d_x, int ne_off, const Tensor& Dmat,
                             const Tensor& bias, const Tensor& alpha, const Tensor& cn, const Tensor& nt, float* e, float* gx) {
-    Tensor DD = f32(Dmat), bb = f32(bias), al = f32(alpha);
+    Tensor DD = f32(Dmat), bb = f32(bias), al = alpha32(alpha);
     need_cuda(DD, "Dmat");
     TORCH_CHECK(DD.dim() == 4, "sorf_energy_sorted: Dmat is [", DD.sizes(), "], expected [elements, transforms, stacks, d]");
     const int ne = (int)DD.size(0), Tn = (int)DD.size(1), S = (int)DD.size(2), d = (int)DD.size(3);
@@ -599,7 +606,7 @@ std::tuple<Tensor, Tensor> sorf_energy_sorted(const Tensor& x, const Tensor& off
 // the fused RFF kernel on rows x f32 [A,d]: shape checks of the model's tensors and the launch (e zero-filled)
 void rff_energy_sorted_raw(const float* x, const int* off, const int* ss, int A, int d_x, int ne_off, const Tensor& W,
                            const Tensor& b, const Tensor& alpha, float* e, float* gx) {
-    Tensor WW = f32(W), bb = f32(b), al = f32(alpha);
+    Tensor WW = f32(W), bb = f32(b), al = alpha32(alpha);
     need_cuda(WW, "W");
     TORCH_CHECK(WW.dim() == 3 && bb.dim() == 2, "rff_energy_sorted: W is [", WW.sizes(), "], b is [", bb.sizes(), "]");
     const int ne = (int)WW.size(0), d = (int)WW.size(1), F = (int)WW.size(2);

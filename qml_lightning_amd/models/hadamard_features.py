@@ -421,7 +421,9 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
             if inv_cell is None:
                 inv_cell = torch.empty(0, 3, 3, device=X.device)
             coeff_normalisation = torch.sqrt(torch.tensor(self.npcas)) / self.sigma
-            alpha = self.alpha.float()
+            # the fused operators take alpha as it is stored (fp64) and keep its fp32 form per tensor
+            # version; the reference's route below converts it where it contracts with it
+            alpha = self.alpha
         else:
             # the same values without building them per call (a single molecule's step is as long as its
             # host side): the empty cell tensor and the normalisation are kept, alpha converted once per value
@@ -486,7 +488,7 @@ class HadamardFeaturesModel(BaseKernel, torch.nn.Module):
             features = torch.ops.qml_lightning_sorf.get_cos_features(coeffs, self.bias[element_idx],
                                                                      torch.tensor(nmol), batch_indexes)
             Ztest = Ztest + features
-        return torch.matmul(Ztest, alpha)
+        return torch.matmul(Ztest, alpha.float())
 
     @torch.jit.unused
     def energies_and_forces(self, coordinates, charges, atomIDs, molIDs, natom_counts, cells=None, inv_cells=None,

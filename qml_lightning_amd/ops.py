@@ -567,6 +567,13 @@ def molecule_sums(e_slots, B, n):
     return energies
 
 
+def _alpha32(alpha):
+    """alpha in fp32; a model's fp64 alpha is converted once per tensor version, not per call."""
+    if alpha.dtype == torch.float32:
+        return alpha.contiguous()
+    return presplit_cached(alpha, "f32", lambda t: t.float().contiguous())
+
+
 def _zeroed_slots(e_zeroed, nslots, device):
     if e_zeroed is None:
         return torch.zeros(int(nslots), dtype=torch.float32, device=device)
@@ -579,7 +586,7 @@ def sorf_energy_sorted(x, type_offsets, sorted_slots, Dmat, bias, alpha, normali
                        with_grad=True, e_zeroed=None):
     """Fused SORF + cos + energy on element-sorted rows x [A,d] -> (e_slots [nslots], gx [A,d] or None).
     e_zeroed: the caller's zero-filled f32 [nslots] to take the energies (else one is made here)."""
-    x, Dmat, bias, alpha = _f32(x), _f32(Dmat), _f32(bias), _f32(alpha)
+    x, Dmat, bias, alpha = _f32(x), _f32(Dmat), _f32(bias), _alpha32(alpha)
     type_offsets, sorted_slots = _i32(type_offsets), _i32(sorted_slots)
     ne, Tn, S, d = Dmat.shape
     A = int(sorted_slots.shape[0])
@@ -678,7 +685,7 @@ def rff_energy_sorted(x, type_offsets, sorted_slots, W, b, alpha, nslots, with_g
     """Fused RFF energy (and gradient) on element-sorted rows x [A,d]; W [ne,d,F], b [ne,F],
     alpha [F] fp32 -> (e_slots [nslots], gx [A,d] or None).  W is split for the kernel on its first
     use and the split form kept until W changes.  e_zeroed: as for sorf_energy_sorted."""
-    x, W, b, alpha = _f32(x), _f32(W), _f32(b), _f32(alpha)
+    x, W, b, alpha = _f32(x), _f32(W), _f32(b), _alpha32(alpha)
     type_offsets, sorted_slots = _i32(type_offsets), _i32(sorted_slots)
     ne, d, F = W.shape
     A = int(sorted_slots.shape[0])
