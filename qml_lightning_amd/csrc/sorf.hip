@@ -595,7 +595,7 @@ constexpr int ROWS_NA = 4;   // atoms per workgroup = rows of 16 lanes per wavef
 // NW: wavefronts per workgroup, which share out the stacks (16 for a few atoms: a molecule then takes
 // a quarter of the time, its stacks being the only parallelism there is).
 template <int LOG2D, bool WITH_GRAD, bool MULTI, int NW = SORF_WAVES>
-__global__ __launch_bounds__(64 * NW) void sorf_energy_rows_kernel(
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(LOG2D >= 8 ? 4 : 1, 8))) void sorf_energy_rows_kernel(
     const float* __restrict__ x, const float* __restrict__ D, const float* __restrict__ bias,
     const float* __restrict__ alpha, const float* __restrict__ bias_absmax, const int* __restrict__ out_index,
     const int* __restrict__ type_offsets, int ne, int A, int S, int T_, float scale, float normf,
@@ -696,8 +696,17 @@ __global__ __launch_bounds__(64 * NW) void sorf_energy_rows_kernel(
             bound = fmaf(*bias_absmax, INV2PI, row_sum(bound));
             track = __any(!(bound <= UMAX));       // a NaN bound keeps the checks
         }
-        auto stack = [&](auto tracked, const float (&dcur)[EPL], const float (&bv)[EPL], const float (&av)[EPL]) {
+        // dnext / next: the sign diagonal of the stack after this one and where it sits.  It is fetched one
+        // stack ahead (it is the first thing a stack needs): at the start of this stack, or, with sixteen
+        // registers per lane (d = 256), in its middle, when bias and alpha are done with and their registers
+        // free (a fourth wavefront per SIMD instead of three)
+        constexpr bool LATE_DIAGONAL = EPL >= 16;
+        auto stack = [&](auto tracked, const float (&dcur)[EPL], float (&dnext)[EPL], const float* next, size_t off) {
             constexpr bool TRACK = decltype(tracked)::value;
+            float bv[EPL], av[EPL];
+            load_row<EPL>(bv, bias + off);                   // the same for the four rows
+            load_row<EPL>(av, alpha + off);
+            if constexpr (!LATE_DIAGONAL) load_row<EPL>(dnext, next);
             float v[EPL];
 #pragma unroll
             for (int p = 0; p < EPL; ++p) v[p] = xv[p] * dcur[p];
@@ -729,6 +738,7 @@ __global__ __launch_bounds__(64 * NW) void sorf_energy_rows_kernel(
                     }
                 }
             }
+            if constexpr (LATE_DIAGONAL) load_row<EPL>(dnext, next);
             if constexpr (WITH_GRAD) {
                 register_stages<EPL>(v);
                 row_stages<EPL>(v, ncs);
@@ -744,24 +754,10 @@ __global__ __launch_bounds__(64 * NW) void sorf_energy_rows_kernel(
             int s = wave;
             if (s < S) load_row<EPL>(d0, D + (size_t)s * d + e0);
             while (s < S) {
-                {
-                    float bv[EPL], av[EPL];
-                    const size_t off = (size_t)s * d + e0;               // the same for the four rows
-                    load_row<EPL>(bv, bias + off);
-                    load_row<EPL>(av, alpha + off);
-                    load_row<EPL>(d1, D + (size_t)(s + NW < S ? s + NW : s) * d + e0);
-                    stack(tracked, d0, bv, av);
-                }
+                stack(tracked, d0, d1, D + (size_t)(s + NW < S ? s + NW : s) * d + e0, (size_t)s * d + e0);
                 s += NW;
                 if (s >= S) break;
-                {
-                    float bv[EPL], av[EPL];
-                    const size_t off = (size_t)s * d + e0;
-                    load_row<EPL>(bv, bias + off);
-                    load_row<EPL>(av, alpha + off);
-                    load_row<EPL>(d0, D + (size_t)(s + NW < S ? s + NW : s) * d + e0);
-                    stack(tracked, d1, bv, av);
-                }
+                stack(tracked, d1, d0, D + (size_t)(s + NW < S ? s + NW : s) * d + e0, (size_t)s * d + e0);
                 s += NW;
             }
         };
