@@ -14,6 +14,8 @@
 // depth of 128 the read-modify-write of the trailing matrix dominates.
 // Only elements on or above the diagonal are read; below the diagonal only the lower halves of
 // the 128x128 diagonal tiles are overwritten.  Flops: F^3/3.
+#include <type_traits>
+
 #include "qmll_common.h"
 
 // gram.hip: tiles on/above the diagonal of C[n,n] (row stride ldc) += sign * Z^T Z, Z = M rows
@@ -42,65 +44,106 @@ constexpr int G = 16;         // potrf thread grid edge: thread (ti,tj) owns row
 __global__ __launch_bounds__(256) void potrf_block_kernel(double* __restrict__ A, long long ld, int k0, int nb,
                                                           double* __restrict__ inv, double* __restrict__ invT,
                                                           int* __restrict__ info) {
-    __shared__ double rowS[2][NB], rowT[2][NB], dsq[NB];
+    __shared__ double rowS[2][2][NB], rowT[2][2][NB], dsq[NB];
     if (*info != 0) return;
     const int tid = threadIdx.x;
     const int ti = tid / G, tj = tid % G;
     double* blk = A + (size_t)k0 * ld + k0;
-    double s[8][8], t[8][8];
+    // one array for both: S(a,b), b >= a, the upper 16 x 16-element groups of the symmetric copy; T(a,b), b <= a,
+    // the lower groups of L^-1 (two [8][8] arrays, half empty, end up in scratch memory beside the step's temporaries)
+    double st[8][9];
+#define S_(a, b) st[a][(b) + 1]
+#define T_(a, b) st[a][b]
 #pragma unroll
     for (int a = 0; a < 8; ++a) {
 #pragma unroll
         for (int b = a; b < 8; ++b) {
             const int r = a * G + ti, c = b * G + tj;
             const int lo = r < c ? r : c, hi = r < c ? c : r;
-            s[a][b] = hi < nb ? blk[(size_t)lo * ld + hi] : (r == c ? 1.0 : 0.0);
+            S_(a, b) = hi < nb ? blk[(size_t)lo * ld + hi] : (r == c ? 1.0 : 0.0);
         }
 #pragma unroll
-        for (int b = 0; b <= a; ++b) t[a][b] = (a == b && ti == tj) ? 1.0 : 0.0;
+        for (int b = 0; b <= a; ++b) T_(a, b) = (a == b && ti == tj) ? 1.0 : 0.0;
     }
+    // reciprocal by the hardware estimate and two Newton steps (full fp64 accuracy up to a couple of
+    // ulps) instead of the much longer IEEE division sequence: it sits on the serial path of every step
+    auto reciprocal = [](double v) {
+        double ip = __builtin_amdgcn_rcp(v);
+        ip = fma(fma(-v, ip, 1.0), ip, ip);
+        return fma(fma(-v, ip, 1.0), ip, ip);
+    };
+    // Two pivots per barrier.  The kernel is bound by its chain of dependent steps (barrier, pivot row
+    // through LDS, reciprocal: 44 of 59 us remain when the elimination's multiply-adds are taken out), not by
+    // arithmetic.  Rows j and j+1 are published as they stand before step j; every thread forms what step j
+    // would have made of row j+1 (row1 - l row0, l = S[j,j+1] / S[j,j]) and applies both eliminations: the
+    // same operations in the same order as one pivot at a time, hence the same bits.  Halving the barriers
+    // buys less than their share (59 -> 53 us per block, 45.0 -> 44.2 ms per factorisation at 16 384): the LDS
+    // reads and the two reciprocals, the second of which waits for the first, are what a step is made of.
+    // (the register block index is a template constant, not a loop variable the unroller may or may not fix:
+    // with it dynamic the register arrays go to scratch memory)
+    auto eliminate = [&](auto ja_) -> bool {
+        constexpr int ja = decltype(ja_)::value;
+        for (int jj = 0; jj < G; jj += 2) {
+            const int j = ja * G + jj, buf = (jj >> 1) & 1;
+            if (ti == jj || ti == jj + 1) {
+                const int which = ti - jj;
 #pragma unroll
-    for (int ja = 0; ja < 8; ++ja) {
-        for (int jj = 0; jj < G; ++jj) {
-            const int j = ja * G + jj, buf = jj & 1;
-            if (ti == jj) {
+                for (int b = ja; b < 8; ++b) rowS[buf][which][b * G + tj] = S_(ja, b);
 #pragma unroll
-                for (int b = ja; b < 8; ++b) rowS[buf][b * G + tj] = s[ja][b];
-#pragma unroll
-                for (int b = 0; b <= ja; ++b) rowT[buf][b * G + tj] = t[ja][b];
+                for (int b = 0; b <= ja; ++b) rowT[buf][which][b * G + tj] = T_(ja, b);
             }
-            __syncthreads();   // the other copy was last read in step j-1, which ended at this barrier
-            const double piv = rowS[buf][j];
-            if (!(piv > 0.0)) {                       // the same value in every thread: uniform exit
+            __syncthreads();   // the other copy was last read in the step before, which ended at this barrier
+            const double piv0 = rowS[buf][0][j];
+            if (!(piv0 > 0.0)) {                      // the same value in every thread: uniform exit
                 if (tid == 0) *info = k0 + j + 1;
-                return;
+                return false;
             }
-            // reciprocal by the hardware estimate and two Newton steps (full fp64 accuracy up to a
-            // couple of ulps) instead of the much longer IEEE division sequence: this sits on the
-            // serial path of every step
-            double ip = __builtin_amdgcn_rcp(piv);
-            ip = fma(fma(-piv, ip, 1.0), ip, ip);
-            ip = fma(fma(-piv, ip, 1.0), ip, ip);
-            double rv[8], tv[8], f[8];
+            const double ip0 = reciprocal(piv0);
+            const double a01 = rowS[buf][0][j + 1];
+            const double l = a01 * ip0;
+            const double piv1 = fma(-l, a01, rowS[buf][1][j + 1]);
+            if (!(piv1 > 0.0)) {
+                if (tid == 0) *info = k0 + j + 2;
+                return false;
+            }
+            const double ip1 = reciprocal(piv1);
+            double rv0[8], rv1[8], tv0[8], tv1[8], f0[8], f1[8];
 #pragma unroll
-            for (int b = ja; b < 8; ++b) rv[b] = rowS[buf][b * G + tj];
+            for (int b = ja; b < 8; ++b) {
+                rv0[b] = rowS[buf][0][b * G + tj];
+                rv1[b] = fma(-l, rv0[b], rowS[buf][1][b * G + tj]);
+            }
 #pragma unroll
-            for (int b = 0; b <= ja; ++b) tv[b] = rowT[buf][b * G + tj];
+            for (int b = 0; b <= ja; ++b) {
+                tv0[b] = rowT[buf][0][b * G + tj];
+                tv1[b] = fma(-l, tv0[b], rowT[buf][1][b * G + tj]);
+            }
 #pragma unroll
-            for (int a = ja; a < 8; ++a) f[a] = (a * G + ti > j) ? rowS[buf][a * G + ti] * ip : 0.0;
+            for (int a = ja; a < 8; ++a) {
+                const int r = a * G + ti;
+                const double c0 = rowS[buf][0][r];
+                f0[a] = r > j ? c0 * ip0 : 0.0;
+                f1[a] = r > j + 1 ? fma(-l, c0, rowS[buf][1][r]) * ip1 : 0.0;
+            }
 #pragma unroll
             for (int a = ja; a < 8; ++a) {
 #pragma unroll
-                for (int b = a; b < 8; ++b) s[a][b] = fma(-f[a], rv[b], s[a][b]);
+                for (int b = a; b < 8; ++b) S_(a, b) = fma(-f1[a], rv1[b], fma(-f0[a], rv0[b], S_(a, b)));
 #pragma unroll
-                for (int b = 0; b <= ja; ++b) t[a][b] = fma(-f[a], tv[b], t[a][b]);
+                for (int b = 0; b <= ja; ++b) T_(a, b) = fma(-f1[a], tv1[b], fma(-f0[a], tv0[b], T_(a, b)));
             }
         }
-    }
+        return true;
+    };
+    if (!eliminate(std::integral_constant<int, 0>{}) || !eliminate(std::integral_constant<int, 1>{}) ||
+        !eliminate(std::integral_constant<int, 2>{}) || !eliminate(std::integral_constant<int, 3>{}) ||
+        !eliminate(std::integral_constant<int, 4>{}) || !eliminate(std::integral_constant<int, 5>{}) ||
+        !eliminate(std::integral_constant<int, 6>{}) || !eliminate(std::integral_constant<int, 7>{}))
+        return;
     // 1/sqrt(D_r) of every row, from the threads on the diagonal
     if (ti == tj) {
 #pragma unroll
-        for (int a = 0; a < 8; ++a) dsq[a * G + ti] = 1.0 / sqrt(s[a][a]);
+        for (int a = 0; a < 8; ++a) dsq[a * G + ti] = 1.0 / sqrt(S_(a, a));
     }
     __syncthreads();
 #pragma unroll
@@ -110,13 +153,15 @@ __global__ __launch_bounds__(256) void potrf_block_kernel(double* __restrict__ A
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
             const int c = b * G + tj;
-            if (b >= a && c >= r && c < nb) blk[(size_t)r * ld + c] = s[a][b] * dr;
-            const double v = b <= a ? t[a][b] * dr : 0.0;     // U^-1[c,r]
+            if (b >= a && c >= r && c < nb) blk[(size_t)r * ld + c] = S_(a, b) * dr;
+            const double v = b <= a ? T_(a, b) * dr : 0.0;     // U^-1[c,r]
             invT[r * NB + c] = v;
             inv[c * NB + r] = v;
         }
     }
 }
+#undef S_
+#undef T_
 
 // ---- triangular solves with one right-hand side -----------------------------------------
 
