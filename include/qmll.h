@@ -462,9 +462,13 @@ size_t qmll_cholesky_workspace_bytes(int F);
  * doubles, ld even).  Reads only elements on or above the diagonal; on exit they hold U.  Below
  * the diagonal, the lower halves of the 128 x 128 diagonal tiles are overwritten with junk, the
  * rest is untouched.  workspace (qmll_cholesky_workspace_bytes(F), 16-byte aligned) receives the
- * reciprocal diagonal of U and must be passed unchanged to qmll_cholesky_solve_f64.
+ * inverses of the 128 x 128 diagonal blocks of U and must be passed unchanged to
+ * qmll_cholesky_solve_f64.
  * info (device int, zeroed by the caller): 0 on success, else 1 + the index of the first pivot
- * that is not positive; U is then unusable. */
+ * that is not positive; U is then unusable.  When F is a multiple of 128 (and A 16-byte aligned) a
+ * panel of 512 rows and the trailing update of the panel before it are one launch whose workgroups
+ * wait for one another through flags in the workspace; every such wait is bounded, and one that
+ * runs out (never seen) leaves info = -1, which callers treat like a failed pivot. */
 int qmll_cholesky_f64(double* A, int F, long long ld, void* workspace, int* info, qmll_stream_t stream);
 
 /* b <- (U^T U)^-1 b for one right-hand side b[F], U and workspace from qmll_cholesky_f64. */

@@ -744,7 +744,8 @@ def test_gram_with_workspace_splits_the_last_round_of_tiles(F, M):
     assert torch.equal(C, plain)
 
 
-@pytest.mark.parametrize("F", [6, 100, 128, 300, 1064, 2176])
+# multiples of 128 take the one-launch-per-panel route (one, two and several panels), the others a launch per step
+@pytest.mark.parametrize("F", [6, 100, 128, 300, 384, 640, 1064, 1536, 2176])
 def test_cholesky_solve_matches_lapack(F):
     """(Z^T Z + lambda I) x = b by the library's blocked Cholesky against numpy's LU solve (the
     reference's route, kernel.py:231) and numpy's factor; conditioning as in training (few rows
@@ -841,15 +842,17 @@ def test_cholesky_in_place_on_a_strided_view():
     assert (outside == 5.0).all()
 
 
-def test_cholesky_reports_a_matrix_that_is_not_positive_definite():
+@pytest.mark.parametrize("F,bad", [(200, 150), (256, 150), (1152, 3), (1152, 300), (1152, 700), (1152, 1151)])
+def test_cholesky_reports_a_matrix_that_is_not_positive_definite(F, bad):
+    """On both routes (a launch per step; one launch per panel, where the other workgroups of the panel
+    and every later launch must leave without waiting for the block that failed)."""
     from qml_lightning_amd import ops
     rng = np.random.default_rng(5)
-    F = 200
     Zr = rng.normal(size=(F + 20, F))
     A = Zr.T @ Zr
-    A[150, 150] = -1.0                                             # pivot 150 cannot be positive
+    A[bad, bad] = -1.0                                             # this pivot cannot be positive
     x, info = ops.cholesky_solve_spd(torch.tensor(A, device=dev()), torch.zeros(F, 1, dtype=torch.float64, device=dev()))
-    assert int(info.item()) == 151
+    assert int(info.item()) == bad + 1
 
 
 def test_matmul_and_reduce_is_the_reference_kahan_sum():
