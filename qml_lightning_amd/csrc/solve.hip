@@ -17,6 +17,7 @@
 // Only elements on or above the diagonal are read; below the diagonal only the lower halves of
 // the 128x128 diagonal tiles are overwritten.  Flops: F^3/3.
 #include <type_traits>
+#include <utility>
 
 #include "qmll_common.h"
 #include "gram_tiles.h"
@@ -33,124 +34,281 @@ namespace {
 
 constexpr int NB = 128;       // block edge
 constexpr int OB = 512;       // panel depth of the trailing update
-constexpr int GR = 32, GC = 16;   // potrf thread grid: thread (ti,tj) owns rows ti + 32 a, columns tj + 16 b
-constexpr int PT = GR * GC;       // threads of a factorisation workgroup (and of the tile product's eight wavefronts)
+constexpr int PT = 512;           // threads of a factorisation workgroup (and of the tile product's eight wavefronts)
+constexpr int SB = 16;            // sub-block edge of the diagonal-block factorisation (one fp64 MFMA tile)
+constexpr int NSB = NB / SB;      // sub-blocks per edge
+constexpr int NSUB = NSB * (NSB + 1) / 2;     // sub-blocks on or above (or on or below) the diagonal
+constexpr int MWAVES = PT / 64 - 1;           // wavefronts that hold sub-blocks; wavefront 0 factors the diagonal ones
+constexpr int NSLOT = (2 * NSUB + MWAVES - 1) / MWAVES;
+constexpr int SSTRIDE = NB + 16;  // doubles per row of a 16-row strip in LDS (rows 32 banks apart, see gram.hip)
+constexpr int DSTRIDE = SB + 1;
 
-// Factor the nb x nb block at (k0,k0) (nb <= 128; the rest is padded with the identity).
-// Elimination without square roots on a symmetric copy held in registers, A = L D L^T: in step j
-// row r > j takes S[r,:] -= (S[j,r]/S[j,j]) S[j,:]; the same row operations applied to the
-// identity give T = L^-1.  At the end U[j,c] = S[j,c]/sqrt(D_j) and U^-1[m,i] = T[i,m]/sqrt(D_i).
-// Rows are dealt cyclically (32 x 16 threads, 4 x 8 elements each), so the shrinking active window
-// stays balanced; the pivot row travels through LDS, one barrier per step.  Only the 32 x 16-element
-// groups that hold live data are kept: for row group a the column groups b >= 2a of S and b <= 2a + 1 of T,
-// forty values per thread, which with a step's temporaries stays inside the 128 registers of a kernel that
-// runs two workgroups of 512 per CU.
-// The kernel is bound by its chain of 128 dependent steps (barrier, pivot row through LDS, reciprocal), not
-// by arithmetic: without the elimination's multiply-adds it still takes three quarters of its time.
-// Output: upper triangle of the block <- U11; inv[m*128+i] = U11^-1[m,i]; invT[i*128+m] the same.
-// info: 0, or 1 + the index of the first pivot that is not positive (later launches then exit).
+typedef double double4_t __attribute__((ext_vector_type(4)));
+
+// LDS of the diagonal-block factorisation, 41 KB
 struct PotrfShared {
-    double rowS[2][NB], rowT[2][NB], dsq[NB];
+    double ustrip[SB][SSTRIDE];   // block row K of U
+    double wstrip[SB][SSTRIDE];   // block row K of W = L^-1
+    double dblk[SB][DSTRIDE];     // the diagonal sub-block about to be factored
+    double vblk[SB][DSTRIDE];     // the inverse of its factor
+    int failed;
 };
+
+__device__ __forceinline__ double value_of_lane(double v, int lane) {
+    const unsigned long long b = (unsigned long long)__double_as_longlong(v);
+    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)b, lane);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(b >> 32), lane);
+    return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+}
+
+// Sub-block t of the list the wavefronts 1..7 are dealt their register slots from (wavefront w holds
+// t = 7 s + w - 1 in slot s): first the 36 sub-blocks of S on or above the diagonal, row by row, then the
+// 36 of W on or below it.  kind 0: S, 1: W.
+struct SubId {
+    int kind, i, j;
+};
+constexpr SubId sub_id(int t) {
+    SubId b{t >= NSUB ? 1 : 0, 0, 0};
+    int u = b.kind ? t - NSUB : t;
+    if (!b.kind) {
+        while (u >= NSB - b.i) { u -= NSB - b.i; ++b.i; }
+        b.j = b.i + u;
+    } else {
+        while (u >= b.i + 1) { u -= b.i + 1; ++b.i; }
+        b.j = u;
+    }
+    return b;
+}
+
+// f(integral_constant<int, 0>), ..., f(integral_constant<int, N - 1>); the second form stops at the first false
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_impl(F& f, std::integer_sequence<int, Is...>) {
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+template <class F, int... Is>
+__device__ __forceinline__ bool static_all_impl(F& f, std::integer_sequence<int, Is...>) {
+    return (f(std::integral_constant<int, Is>{}) && ...);
+}
+template <int N, class F>
+__device__ __forceinline__ bool static_all(F&& f) {
+    return static_all_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// Factor the nb x nb block at (k0,k0) (nb <= 128; the rest is padded with the identity) and invert the factor.
+// Blocked right-looking Cholesky on 16 x 16 sub-blocks, S = U^T U, with the same block operations applied to
+// the identity: W = L^-1 = U^-T.  The sub-blocks live in registers in the accumulator layout of
+// v_mfma_f64_16x16x4_f64 (register r of a lane: row lane/16 + 4r, column lane%16), which is also the layout
+// of both operands (row = the summed index), so a sub-block feeds the matrix pipe as it stands.  Wavefronts
+// 1..7 hold the 72 sub-blocks, up to eleven each; which ones is fixed at compile time (one instance of the code
+// per wavefront), so a finished sub-block's registers are free again and no index is computed at run time.
+// Wavefront 0 holds none and does the serial part.  Step K of eight:
+//   1. the owner of S(K,K) puts it into LDS; wavefront 0 factors it, a lane per column: sixteen pivots, each
+//      a reciprocal square root and the pivot row handed round with v_readlane, no barrier and no LDS inside;
+//      the same row operations on the identity give V = U_KK^-1;
+//   2. block row K: U(K,J) = V^T S(K,J), W(K,J) = V^T W(K,J), four MFMAs each, to LDS and to memory;
+//   3. S(I,J) -= U(K,I)^T U(K,J) and W(I,J) -= U(K,I)^T W(K,J) for the rows I > K.
+// 24 barriers instead of the 128 of an elimination pivot by pivot, and the multiply-adds on the matrix pipe.
+// Output: upper triangle of the block <- U11; inv[m*128+i] = U11^-1[m,i] = W[i,m]; invT[i*128+m] the same.
+// info: 0, or 1 + the index of the first pivot that is not positive (later launches then exit).
+
+// inv[m, 16 K + i] = W[16 K + i, m] for the columns m of block row K, from the strip in LDS: thread = (m, half a
+// row of sixteen), 64 contiguous bytes each
+__device__ __forceinline__ void store_inverse_columns(int K, double* inv, const PotrfShared& ps) {
+    const int m = (int)threadIdx.x >> 1, half = (int)threadIdx.x & 1;
+    if (m < (K + 1) * SB) {
+#pragma unroll
+        for (int q = 0; q < SB / 2; ++q) inv[m * NB + K * SB + half * (SB / 2) + q] = ps.wstrip[half * (SB / 2) + q][m];
+    }
+}
+
+// wavefront 0: the diagonal sub-blocks, one after the other
+__device__ __forceinline__ bool potrf_factor_wave(double* blk, long long ld, int k0, int nb, double* inv, int* info,
+                                                  PotrfShared& ps) {
+    const int lane = (int)threadIdx.x & 63, l16 = lane & 15;
+    for (int K = 0; K < NSB; ++K) {
+        __syncthreads();                                               // S(K,K) is in LDS
+        // column l16 of the sub-block in d, row l16 of V in w (the four groups of sixteen lanes hold copies)
+        double d[SB], w[SB];
+#pragma unroll
+        for (int i = 0; i < SB; ++i) {
+            d[i] = ps.dblk[i][l16];
+            w[i] = i == l16 ? 1.0 : 0.0;
+        }
+        int bad = -1;                                                  // the first pivot that is not positive
+#pragma unroll
+        for (int j = 0; j < SB; ++j) {
+            double piv = value_of_lane(d[j], j);                       // the same value in every lane
+            if (!(piv > 0.0)) {
+                bad = bad < 0 ? j : bad;
+                piv = 1.0;
+            }
+            // 1/sqrt by the hardware estimate and two Newton steps
+            double y = __builtin_amdgcn_rsq(piv);
+            const double h = 0.5 * piv;
+            y = fma(y, fma(-h * y, y, 0.5), y);
+            y = fma(y, fma(-h * y, y, 0.5), y);
+            const double u = d[j] * y;                                 // U[j, l16]
+            const double wj = w[j] * y;                                // W[j, l16]
+            d[j] = u;
+            w[j] = wj;
+#pragma unroll
+            for (int i = j + 1; i < SB; ++i) {
+                const double ui = value_of_lane(u, i);                 // U[j, i] = L[i, j]
+                d[i] = fma(-ui, u, d[i]);
+                w[i] = fma(-ui, wj, w[i]);
+                // pins the update to this step (no instruction is emitted): nothing needs w before the end, so
+                // left alone the compiler computes all of it there and carries every multiplier of every step
+                // in scalar registers it does not have
+                asm volatile("" : "+v"(w[i]));
+            }
+        }
+        if (bad >= 0 && lane == 0) {
+            *info = k0 + K * SB + bad + 1;
+            ps.failed = 1;
+        }
+        // (every lane stores: the four copies write the same values)
+#pragma unroll
+        for (int i = 0; i < SB; ++i) {
+            ps.vblk[l16][i] = w[i];                                    // V[c, i] = W[i, c]
+            const int row = K * SB + i, col = K * SB + l16;
+            if (lane < SB && i <= l16 && col < nb) blk[(size_t)row * ld + col] = d[i];
+        }
+        __syncthreads();                                               // V is in LDS
+        if (ps.failed) return false;
+        __syncthreads();                                               // block row K is in LDS
+        store_inverse_columns(K, inv, ps);
+    }
+    return true;
+}
+
+// wavefront WV = 1..7: its share of the sub-blocks
+template <int WV>
+__device__ __forceinline__ bool potrf_mfma_wave(double* blk, long long ld, int nb, double* inv, double* invT,
+                                                PotrfShared& ps) {
+    const int lane = (int)threadIdx.x & 63, l16 = lane & 15, lk = lane >> 4;
+    const int ldi = (int)ld;
+    // per-lane parts of every address; what is added per sub-block is a constant
+    double* const blk_lane = blk + (size_t)lk * ld + l16;
+    double* const invT_lane = invT + lk * NB + l16;
+    double* const us_lane = &ps.ustrip[lk][l16];
+    double* const ws_lane = &ps.wstrip[lk][l16];
+    double4_t sub[NSLOT];
+    static_for<NSLOT>([&](auto s_) {
+        constexpr int s = decltype(s_)::value, t = s * MWAVES + WV - 1;
+        if constexpr (t < 2 * NSUB) {
+            constexpr SubId b = sub_id(t);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = b.i * SB + lk + 4 * r, col = b.j * SB + l16;
+                if constexpr (b.kind == 0) {
+                    const int lo = row < col ? row : col, hi = row < col ? col : row;
+                    // (32-bit offsets: 128 rows of at most 2^23 doubles)
+                    sub[s][r] = hi < nb ? blk[(unsigned)(lo * ldi + hi)] : (row == col ? 1.0 : 0.0);
+                } else {
+                    sub[s][r] = row == col ? 1.0 : 0.0;
+                }
+            }
+        }
+    });
+    return static_all<NSB>([&](auto K_) -> bool {
+        constexpr int K = decltype(K_)::value;
+        static_for<NSLOT>([&](auto s_) {
+            constexpr int s = decltype(s_)::value, t = s * MWAVES + WV - 1;
+            if constexpr (t < 2 * NSUB) {
+                constexpr SubId b = sub_id(t);
+                if constexpr (b.kind == 0 && b.i == K && b.j == K) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) ps.dblk[lk + 4 * r][l16] = sub[s][r];
+                }
+            }
+        });
+        __syncthreads();                                               // S(K,K) is in LDS
+        __syncthreads();                                               // wavefront 0 has factored it: V is in LDS
+        if (ps.failed) return false;
+        double va[4];
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) va[kk] = ps.vblk[4 * kk + lk][l16];
+        static_for<NSLOT>([&](auto s_) {
+            constexpr int s = decltype(s_)::value, t = s * MWAVES + WV - 1;
+            if constexpr (t < 2 * NSUB) {
+                constexpr SubId b = sub_id(t);
+                if constexpr (b.i == K && (b.kind == 1 || b.j > K)) {
+                    double4_t res = {0.0, 0.0, 0.0, 0.0};
+#pragma unroll
+                    for (int kk = 0; kk < 4; ++kk)
+                        res = __builtin_amdgcn_mfma_f64_16x16x4f64(va[kk], sub[s][kk], res, 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if constexpr (b.kind == 0) {
+                            us_lane[4 * r * SSTRIDE + b.j * SB] = res[r];
+                            if (b.j * SB + l16 < nb && K * SB + lk + 4 * r < nb)
+                                blk_lane[(size_t)(K * SB + 4 * r) * ld + b.j * SB] = res[r];
+                        } else {
+                            ws_lane[4 * r * SSTRIDE + b.j * SB] = res[r];
+                            invT_lane[(K * SB + 4 * r) * NB + b.j * SB] = res[r];
+                        }
+                    }
+                }
+            }
+        });
+        __syncthreads();                                               // block row K is in LDS
+        store_inverse_columns(K, inv, ps);
+        static_for<NSLOT>([&](auto s_) {
+            constexpr int s = decltype(s_)::value, t = s * MWAVES + WV - 1;
+            if constexpr (t < 2 * NSUB) {
+                constexpr SubId b = sub_id(t);
+                if constexpr (b.i > K && (b.kind == 0 || b.j <= K)) {
+                    const double* right = b.kind == 0 ? us_lane : ws_lane;
+#pragma unroll
+                    for (int kk = 0; kk < 4; ++kk) {
+                        const double fa = -us_lane[4 * kk * SSTRIDE + b.i * SB];
+                        const double fb = right[4 * kk * SSTRIDE + b.j * SB];
+                        sub[s] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa, fb, sub[s], 0, 0, 0);
+                    }
+                }
+            }
+        });
+        return true;
+    });
+}
 
 // Called by all PT threads of the workgroup.  False when a pivot is not positive (info is then set).
 __device__ __forceinline__ bool potrf_block(double* A, long long ld, int k0, int nb, double* inv, double* invT,
                                             int* info, PotrfShared& ps) {
-    auto& rowS = ps.rowS;
-    auto& rowT = ps.rowT;
-    auto& dsq = ps.dsq;
     const int tid = threadIdx.x;
-    const int ti = tid / GC, tj = tid % GC;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     double* blk = A + (size_t)k0 * ld + k0;
-    double st[4][10];
-#define S_(a, b) st[a][(b) + 2]
-#define T_(a, b) st[a][b]
-#pragma unroll
-    for (int a = 0; a < 4; ++a) {
-        const int r = a * GR + ti;
-#pragma unroll
-        for (int b = 2 * a; b < 8; ++b) {
-            const int c = b * GC + tj;
-            const int lo = r < c ? r : c, hi = r < c ? c : r;
-            S_(a, b) = hi < nb ? blk[(size_t)lo * ld + hi] : (r == c ? 1.0 : 0.0);
-        }
-#pragma unroll
-        for (int b = 0; b <= 2 * a + 1; ++b) T_(a, b) = (r == b * GC + tj) ? 1.0 : 0.0;
+    // the sub-blocks of inv / invT that stay zero (the others are written when their block row is final)
+    for (int e = tid; e < (NSUB - NSB) * SB * SB; e += PT) {
+        int b = e / (SB * SB), I = 0;
+        const int r = (e / SB) % SB, c = e % SB;
+        while (b >= NSB - 1 - I) { b -= NSB - 1 - I; ++I; }
+        const int J = I + 1 + b;                                  // I < J
+        invT[(I * SB + r) * NB + J * SB + c] = 0.0;
+        inv[(J * SB + r) * NB + I * SB + c] = 0.0;
     }
-    // reciprocal by the hardware estimate and two Newton steps (full fp64 accuracy up to a couple of
-    // ulps) instead of the much longer IEEE division sequence: it sits on the serial path of every step
-    auto reciprocal = [](double v) {
-        double ip = __builtin_amdgcn_rcp(v);
-        ip = fma(fma(-v, ip, 1.0), ip, ip);
-        return fma(fma(-v, ip, 1.0), ip, ip);
-    };
-    // (the row group of the pivot is a template constant, not a loop variable the unroller may or may not
-    // fix: with it dynamic the register array goes to scratch memory)
-    auto eliminate = [&](auto ja_) -> bool {
-        constexpr int ja = decltype(ja_)::value;
-        for (int jj = 0; jj < GR; ++jj) {
-            const int j = ja * GR + jj, buf = jj & 1;
-            if (ti == jj) {
-#pragma unroll
-                for (int b = 2 * ja; b < 8; ++b) rowS[buf][b * GC + tj] = S_(ja, b);
-#pragma unroll
-                for (int b = 0; b <= 2 * ja + 1; ++b) rowT[buf][b * GC + tj] = T_(ja, b);
-            }
-            __syncthreads();   // the other copy was last read in the step before, which ended at this barrier
-            const double piv = rowS[buf][j];
-            if (!(piv > 0.0)) {                       // the same value in every thread: uniform exit
-                if (tid == 0) *info = k0 + j + 1;
-                return false;
-            }
-            const double ip = reciprocal(piv);
-            double rv[8], tv[8], f[4];
-#pragma unroll
-            for (int b = 2 * ja; b < 8; ++b) rv[b] = rowS[buf][b * GC + tj];
-#pragma unroll
-            for (int b = 0; b <= 2 * ja + 1; ++b) tv[b] = rowT[buf][b * GC + tj];
-#pragma unroll
-            for (int a = ja; a < 4; ++a) {
-                const int r = a * GR + ti;
-                f[a] = r > j ? rowS[buf][r] * ip : 0.0;
-            }
-#pragma unroll
-            for (int a = ja; a < 4; ++a) {
-#pragma unroll
-                for (int b = 2 * a; b < 8; ++b) S_(a, b) = fma(-f[a], rv[b], S_(a, b));
-#pragma unroll
-                for (int b = 0; b <= 2 * ja + 1; ++b) T_(a, b) = fma(-f[a], tv[b], T_(a, b));
-            }
-        }
-        return true;
-    };
-    if (!eliminate(std::integral_constant<int, 0>{}) || !eliminate(std::integral_constant<int, 1>{}) ||
-        !eliminate(std::integral_constant<int, 2>{}) || !eliminate(std::integral_constant<int, 3>{}))
-        return false;
-    // 1/sqrt(D_r) of every row, from the threads that hold the diagonal
-    if (tj == ti % GC) {
-#pragma unroll
-        for (int a = 0; a < 4; ++a) dsq[a * GR + ti] = 1.0 / sqrt(ti < GC ? S_(a, 2 * a) : S_(a, 2 * a + 1));
+    if (tid == 0) ps.failed = 0;
+    bool ok;
+    switch (wave) {
+        case 0: ok = potrf_factor_wave(blk, ld, k0, nb, inv, info, ps); break;
+        case 1: ok = potrf_mfma_wave<1>(blk, ld, nb, inv, invT, ps); break;
+        case 2: ok = potrf_mfma_wave<2>(blk, ld, nb, inv, invT, ps); break;
+        case 3: ok = potrf_mfma_wave<3>(blk, ld, nb, inv, invT, ps); break;
+        case 4: ok = potrf_mfma_wave<4>(blk, ld, nb, inv, invT, ps); break;
+        case 5: ok = potrf_mfma_wave<5>(blk, ld, nb, inv, invT, ps); break;
+        case 6: ok = potrf_mfma_wave<6>(blk, ld, nb, inv, invT, ps); break;
+        default: ok = potrf_mfma_wave<7>(blk, ld, nb, inv, invT, ps); break;
     }
+    if (!ok) return false;                                        // every wavefront saw the same flag
     __syncthreads();
-#pragma unroll
-    for (int a = 0; a < 4; ++a) {
-        const int r = a * GR + ti;
-        const double dr = dsq[r];
-#pragma unroll
-        for (int b = 0; b < 8; ++b) {
-            const int c = b * GC + tj;
-            if (b >= 2 * a && c >= r && c < nb) blk[(size_t)r * ld + c] = S_(a, b) * dr;
-            const double v = b <= 2 * a + 1 ? T_(a, b) * dr : 0.0;     // U^-1[c,r]
-            invT[r * NB + c] = v;
-            inv[c * NB + r] = v;
-        }
-    }
     return true;
 }
-#undef S_
-#undef T_
 
-__global__ __launch_bounds__(PT) void potrf_block_kernel(double* A, long long ld, int k0, int nb, double* inv,
+__global__ __launch_bounds__(PT, 4) void potrf_block_kernel(double* A, long long ld, int k0, int nb, double* inv,
                                                          double* invT, int* info) {
     __shared__ PotrfShared ps;
     if (*info != 0) return;
@@ -187,13 +345,13 @@ constexpr int PSTRIDE = NB + 16;        // doubles per staged row (see gram.hip)
 constexpr int P_TPR = PT / PKB;         // threads per staged row
 constexpr int P_CPT = NB / P_TPR;       // doubles per thread and row
 constexpr int P_UN = P_CPT / 2;         // 16-byte units per thread
-constexpr unsigned FLAG_DONE = 1u, FLAG_FAILED = 2u;
+constexpr unsigned FLAG_DONE = 1u, FLAG_FAILED = 0x80000000u;   // (a counter never gets near the second)
 constexpr int PBLK = OB / NB;                        // blocks per panel
 constexpr int FLAGS_PER_PANEL = PBLK + PBLK * PBLK;  // "block l factored": [l]; "strip (l, b) done": [PBLK + l PBLK + b]
+constexpr int SPLIT_HEADS_BELOW = 48;       // trailing tiles per edge
 constexpr unsigned SPIN_LIMIT = 1u << 21;   // polls of about a microsecond each before a wait gives up
 
 typedef double double2_t __attribute__((ext_vector_type(2)));
-typedef double double4_t __attribute__((ext_vector_type(4)));
 
 struct TileShared {
     double a[2][PKB][PSTRIDE], b[2][PKB][PSTRIDE];
@@ -268,22 +426,29 @@ __device__ __forceinline__ void tile_product(const double* Za, long long lda, co
     __syncthreads();
 }
 
-// every store of the workgroup so far becomes visible to the device, then the flag is set
+// every store of the workgroup so far becomes visible to the device, then the flag is set / counted up
 __device__ __forceinline__ void publish(unsigned* flag, unsigned value) {
     __threadfence();
     __syncthreads();
     if (threadIdx.x == 0) __hip_atomic_store(flag, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ void publish_one_more(unsigned* counter) {
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
 
-// true once the flag says done; false when its owner failed or the wait ran out (info <- -1)
-__device__ __forceinline__ bool await(unsigned* flag, unsigned spin_limit, int* info, unsigned& seen) {
+// Waits until the word is at least `target` and returns it; a wait that runs out sets info to -1 and
+// returns FLAG_FAILED.
+__device__ __forceinline__ unsigned await(unsigned* flag, unsigned target, unsigned spin_limit, int* info,
+                                          unsigned& seen) {
     if (threadIdx.x == 0) {
         unsigned v = __hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
-        for (unsigned n = 0; v == 0u && n < spin_limit; ++n) {
+        for (unsigned n = 0; v < target && n < spin_limit; ++n) {
             __builtin_amdgcn_s_sleep(32);
             v = __hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
         }
-        if (v == 0u) {
+        if (v < target) {
             atomicCAS(info, 0, -1);
             v = FLAG_FAILED;
         }
@@ -291,22 +456,50 @@ __device__ __forceinline__ bool await(unsigned* flag, unsigned spin_limit, int* 
     }
     __syncthreads();
     const unsigned v = seen;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");    // every wavefront reads what the owner published
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");    // every wavefront reads what was published
     __syncthreads();                                       // `seen` may be written again
-    return v == FLAG_DONE;
+    return v;
 }
 
 // Panel rows [P0, P0 + 128 nblk); [R0, P0) are the rows of the panel before it, whose update the trailing
-// matrix has not had yet (R0 = P0: nothing outstanding).  nown_pad: ids reserved for the column owners;
-// nt: tiles per edge of the trailing matrix below this panel (0: none).  flags: FLAGS_PER_PANEL words, zero.
+// matrix has not had yet (R0 = P0: nothing outstanding).  Workgroup ids: [0, nhead_pad) the tiles of this
+// panel's rows that take that update ("head": column w has min(w, nblk - 1) + 1 of them, columns in order),
+// then nown_pad ids for the column owners, then the tiles of the trailing matrix below this panel, nt per edge
+// (0: none).  flags: FLAGS_PER_PANEL words, then one counter per column (head tiles done), all zero.
 __global__ __launch_bounds__(PT, 4) void panel_kernel(double* A, long long ld, int F, int R0, int P0, int nblk,
-                                                      int nown_pad, int nt, TileMap tm, double* invs, int* info,
-                                                      unsigned* flags, unsigned spin_limit) {
-    __shared__ __attribute__((aligned(16))) TileShared sm;
-    __shared__ PotrfShared ps;
+                                                      int nhead_pad, int nown, int nown_pad, int nt, TileMap tm,
+                                                      double* invs, int* info, unsigned* flags, unsigned spin_limit) {
+    // the tile product and the factorisation never run at the same time: one piece of LDS for both, which
+    // is what lets two workgroups share a CU (2 x 74 KB)
+    __shared__ __attribute__((aligned(16))) union {
+        TileShared tile;
+        PotrfShared potrf;
+    } lds;
+    TileShared& sm = lds.tile;
+    PotrfShared& ps = lds.potrf;
     __shared__ unsigned seen;
     if (*info != 0) return;
-    const int bid = (int)blockIdx.x;
+    unsigned* heads_done = flags + FLAGS_PER_PANEL;
+    int bid = (int)blockIdx.x;
+    if (bid < nhead_pad) {                                   // a head tile: waits for nobody
+        int w, b;
+        const int tri = nblk * (nblk + 1) / 2;               // the columns of the panel itself form a triangle
+        if (bid < tri) {
+            w = 0;
+            while (bid >= (w + 1) * (w + 2) / 2) ++w;
+            b = bid - w * (w + 1) / 2;
+        } else {
+            w = nblk + (bid - tri) / nblk;
+            b = (bid - tri) % nblk;
+        }
+        const int k0 = P0 + b * NB, j0 = P0 + w * NB;
+        if (j0 >= F) return;
+        tile_product(A + (size_t)R0 * ld + k0, ld, A + (size_t)R0 * ld + j0, ld, P0 - R0, A + (size_t)k0 * ld + j0, ld,
+                     -1.0, false, sm);
+        publish_one_more(heads_done + w);
+        return;
+    }
+    bid -= nhead_pad;
     if (bid >= nown_pad) {                                   // a tile of the trailing matrix
         int ti, tj;
         tile_of_block<true>((unsigned)(bid - nown_pad), nt, nt, tm, ti, tj);
@@ -317,34 +510,47 @@ __global__ __launch_bounds__(PT, 4) void panel_kernel(double* A, long long ld, i
                      -1.0, false, sm);
         return;
     }
-    const int j0 = P0 + bid * NB;                            // first column of the owned tiles
-    if (j0 >= F) return;
+    // a column owner: owner o < nblk has column o of the panel, the one with its diagonal tile in it; the others
+    // have every (nown - nblk)-th column right of the panel
+    if (bid >= nown) return;
+    const int ncol = (F - P0) / NB;
+    const int stride = bid < nblk ? ncol : nown - nblk;
     const int mine = bid < nblk ? bid : nblk - 1;            // last block row with a tile on or above the diagonal
-    if (P0 > R0) {
-        for (int b = 0; b <= mine; ++b) {
-            const int k0 = P0 + b * NB;
-            tile_product(A + (size_t)R0 * ld + k0, ld, A + (size_t)R0 * ld + j0, ld, P0 - R0, A + (size_t)k0 * ld + j0, ld,
-                         -1.0, false, sm);
-        }
+    if (P0 > R0 && nhead_pad > 0) {
+        for (int w = bid; w < ncol; w += stride)
+            if (await(heads_done + w, (unsigned)(mine + 1), spin_limit, info, seen) == FLAG_FAILED) return;
+    } else if (P0 > R0) {                                    // no workgroups for the head tiles: the owner's own work
+        for (int w = bid; w < ncol; w += stride)
+            for (int b = 0; b <= mine; ++b)
+                tile_product(A + (size_t)R0 * ld + P0 + b * NB, ld, A + (size_t)R0 * ld + P0 + w * NB, ld, P0 - R0,
+                             A + (size_t)(P0 + b * NB) * ld + P0 + w * NB, ld, -1.0, false, sm);
     }
+    unsigned strips_seen = 0u;                               // "strip (l, b) done" flags this workgroup has seen set
     for (int l = 0; l < nblk; ++l) {
         const int k0 = P0 + l * NB;
-        double* tile = A + (size_t)k0 * ld + j0;
         double* inv = invs + (size_t)(k0 / NB) * 2 * NB * NB;
-        if (k0 == j0) {                                      // the own diagonal tile: every update is in
+        if (l == bid) {                                      // the own diagonal tile: every update is in
             const bool ok = potrf_block(A, ld, k0, NB, inv, inv + NB * NB, info, ps);
             // on failure every workgroup right of this column leaves at this flag, before it could wait for
             // anything that is now never set
             publish(flags + l, ok ? FLAG_DONE : FLAG_FAILED);
             return;
         }
-        if (!await(flags + l, spin_limit, info, seen)) return;
-        tile_product(inv, NB, tile, ld, NB, tile, ld, 1.0, true, sm);
-        if (bid < nblk) publish(flags + PBLK + l * PBLK + bid, FLAG_DONE);
-        for (int b = l + 1; b <= mine; ++b) {
-            if (b != bid && !await(flags + PBLK + l * PBLK + b, spin_limit, info, seen)) return;
-            tile_product(A + (size_t)k0 * ld + P0 + b * NB, ld, tile, ld, NB, A + (size_t)(P0 + b * NB) * ld + j0, ld, -1.0,
-                         false, sm);
+        if (await(flags + l, FLAG_DONE, spin_limit, info, seen) != FLAG_DONE) return;
+        for (int w = bid; w < ncol; w += stride) {
+            const int j0 = P0 + w * NB;                      // first column of the owned tiles
+            double* tile = A + (size_t)k0 * ld + j0;
+            tile_product(inv, NB, tile, ld, NB, tile, ld, 1.0, true, sm);
+            if (bid < nblk) publish(flags + PBLK + l * PBLK + bid, FLAG_DONE);
+            for (int b = l + 1; b <= mine; ++b) {
+                const unsigned bit = 1u << (l * PBLK + b);
+                if (b != bid && !(strips_seen & bit)) {
+                    if (await(flags + PBLK + l * PBLK + b, FLAG_DONE, spin_limit, info, seen) != FLAG_DONE) return;
+                    strips_seen |= bit;
+                }
+                tile_product(A + (size_t)k0 * ld + P0 + b * NB, ld, tile, ld, NB, A + (size_t)(P0 + b * NB) * ld + j0, ld,
+                             -1.0, false, sm);
+            }
         }
     }
 }
@@ -436,7 +642,7 @@ extern "C" size_t qmll_cholesky_workspace_bytes(int F) {
     if (F <= 0) return 0;
     const size_t nblk = ((size_t)F + NB - 1) / NB;
     const size_t npanel = ((size_t)F + OB - 1) / OB;
-    return (nblk * 2 * NB * NB + (size_t)F) * sizeof(double) + npanel * FLAGS_PER_PANEL * sizeof(unsigned) + 256;
+    return (nblk * 2 * NB * NB + (size_t)F) * sizeof(double) + npanel * (FLAGS_PER_PANEL + nblk) * sizeof(unsigned) + 256;
 }
 
 namespace {
@@ -467,6 +673,7 @@ int factor_block(double* A, int F, long long ld, int P0, int k0, double* invs, i
 extern "C" int qmll_cholesky_f64(double* A, int F, long long ld, void* workspace, int* info, qmll_stream_t stream_) {
     hipStream_t stream = (hipStream_t)stream_;
     QMLL_REQUIRE(F > 0 && ld >= F, QMLL_ERR_INVALID, "qmll_cholesky_f64: bad size F=%d ld=%lld", F, ld);
+    QMLL_REQUIRE(ld < (1LL << 23), QMLL_ERR_INVALID, "qmll_cholesky_f64: row stride %lld too large", ld);
     QMLL_REQUIRE(A && workspace && info, QMLL_ERR_INVALID, "qmll_cholesky_f64: null pointer");
     QMLL_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, QMLL_ERR_INVALID,
                  "qmll_cholesky_f64: the workspace must be 16-byte aligned");
@@ -477,21 +684,32 @@ extern "C" int qmll_cholesky_f64(double* A, int F, long long ld, void* workspace
     if (whole_tiles) {
         const size_t nblk_all = (size_t)F / NB;
         unsigned* flags = reinterpret_cast<unsigned*>(invs + nblk_all * 2 * NB * NB + (size_t)F);
-        const int nflags = (F + OB - 1) / OB * FLAGS_PER_PANEL;
+        const int per_panel = FLAGS_PER_PANEL + F / NB;
+        const int nflags = (F + OB - 1) / OB * per_panel;
         hipLaunchKernelGGL(zero_words_kernel, dim3((nflags + 255) / 256), dim3(256), 0, stream, flags, nflags);
         QMLL_CHECK_LAUNCH("qmll_cholesky_f64");
         for (int P0 = 0; P0 < F; P0 += OB) {
             const int pend = P0 + OB < F ? P0 + OB : F;       // this panel: rows [P0, pend)
             const int R0 = P0 >= OB ? P0 - OB : 0;            // the panel before it
-            const int nown = (F - P0) / NB;
-            const int nown_pad = (nown + NXCD - 1) / NXCD * NXCD;
+            const int nblk = (pend - P0) / NB;
+            const int ncol = (F - P0) / NB;                   // columns of tiles from the panel's first to the last
             const int nt = P0 > R0 ? (F - pend) / NB : 0;
+            const int nown = ncol;
+            // The head tiles (this panel's rows of the update of the panel before) go to workgroups of their own
+            // once the trailing matrix is small, where a launch lasts as long as its slowest owner: four head tiles
+            // and ten strip / update products in a row, 540 us, against a chain of four factorisations of 390.
+            // While the trailing tiles keep the chip busy for longer than that, the owners take their head tiles
+            // themselves and no slot waits for another.
+            const bool split_heads = P0 > R0 && nt <= SPLIT_HEADS_BELOW;
+            const int nown_pad = (nown + NXCD - 1) / NXCD * NXCD;
+            const int nhead = split_heads ? nblk * (nblk + 1) / 2 + (ncol - nblk) * nblk : 0;
+            const int nhead_pad = (nhead + NXCD - 1) / NXCD * NXCD;
             long long per_xcd = 0;
             TileMap tm = gram_tile_map(nt > 0 ? nt : 1, nt > 0 ? nt : 1, true, per_xcd);
-            const long long grid = nown_pad + (nt > 0 ? per_xcd * NXCD : 0);
+            const long long grid = (long long)nhead_pad + nown_pad + (nt > 0 ? per_xcd * NXCD : 0);
             QMLL_REQUIRE(grid < 2147483647LL, QMLL_ERR_INVALID, "qmll_cholesky_f64: too many tiles");
-            hipLaunchKernelGGL(panel_kernel, dim3((unsigned)grid), dim3(PT), 0, stream, A, ld, F, R0, P0, (pend - P0) / NB,
-                               nown_pad, nt, tm, invs, info, flags + (size_t)(P0 / OB) * FLAGS_PER_PANEL, SPIN_LIMIT);
+            hipLaunchKernelGGL(panel_kernel, dim3((unsigned)grid), dim3(PT), 0, stream, A, ld, F, R0, P0, nblk, nhead_pad,
+                               nown, nown_pad, nt, tm, invs, info, flags + (size_t)(P0 / OB) * per_panel, SPIN_LIMIT);
             QMLL_CHECK_LAUNCH("qmll_cholesky_f64");
         }
         return QMLL_OK;
