@@ -561,88 +561,172 @@ __global__ __launch_bounds__(256) void zero_words_kernel(unsigned* p, int n) {
 }
 
 // ---- triangular solves with one right-hand side -----------------------------------------
+//
+// One launch per direction, one workgroup per 128-row block.  Forward, U^T z = b: workgroup k keeps
+// acc = b_k - sum_{i<k} U(i,k)^T z_i, taking the tiles U(i,k) in the order of i, then z_k = U11_k^-T acc through
+// the stored inverse.  Backward, U x = z: the same from the last block to the first with the tiles U(k,j),
+// j > k.  The values handed from workgroup to workgroup are their own flags: z (and the exchange copy of x)
+// start out as a NaN with a payload no computation produces, a producer stores its 128 results with
+// device-scope atomic stores, and a consumer polls the very values it needs with device-scope atomic loads
+// (the tile they multiply is final and already on its way from memory): no fence, no separate flag, one trip
+// through memory per step of the chain.  Every workgroup waits only for workgroups with lower ids (the backward
+// launch numbers the blocks from the end), so whoever is waited for is running or done; the waits are bounded
+// all the same, and one that runs out hands on a NaN, which ends up in the solution instead of a wrong number.
+constexpr int ST = 512;            // threads of a solve workgroup
+constexpr int SQ = ST / NB;        // row quarters: thread (c = tid % 128, q = tid / 128) has rows 32 q .. 32 q + 31
+constexpr int SR = NB / SQ;
+constexpr unsigned long long NOT_YET = 0x7FF8C0DEC0DE0001ULL;
 
-// Block k of U^T z = b: z_k = U11^-T b_k (product with the stored inverse, recomputed by every
-// workgroup), then b[j] -= sum_r U[k0+r, j] z_k[r] for the columns j right of the block
-// (thread = column).  Workgroup 0 stores z_k into z.
-__global__ __launch_bounds__(256) void fwd_step_kernel(const double* __restrict__ U, long long ld, int k0, int nb,
-                                                       int F, const double* __restrict__ inv, double* __restrict__ b,
-                                                       double* __restrict__ z) {
-    __shared__ double rs[NB], xs[NB];
-    const int tid = threadIdx.x;
-    if (tid < NB) rs[tid] = tid < nb ? b[k0 + tid] : 0.0;
-    __syncthreads();
-    if (tid < NB) {
-        double s0 = 0.0, s1 = 0.0;
-        for (int m = 0; m < NB; m += 2) {
-            s0 = fma(inv[m * NB + tid], rs[m], s0);
-            s1 = fma(inv[(m + 1) * NB + tid], rs[m + 1], s1);
-        }
-        xs[tid] = s0 + s1;
-        if (blockIdx.x == 0 && tid < nb) z[k0 + tid] = s0 + s1;
-    }
-    __syncthreads();
-    const int j = k0 + NB + blockIdx.x * 256 + tid;
-    if (j >= F) return;
-    const double* col = U + (size_t)k0 * ld + j;
-    double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
-#pragma unroll 8
-    for (int r = 0; r < NB; r += 4) {
-        s0 = fma(col[(size_t)r * ld], xs[r], s0);
-        s1 = fma(col[(size_t)(r + 1) * ld], xs[r + 1], s1);
-        s2 = fma(col[(size_t)(r + 2) * ld], xs[r + 2], s2);
-        s3 = fma(col[(size_t)(r + 3) * ld], xs[r + 3], s3);
-    }
-    b[j] -= (s0 + s1) + (s2 + s3);
+__device__ __forceinline__ unsigned long long peek(const double* p) {
+    return __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void hand_on(double* p, double v) {
+    unsigned long long bits = (unsigned long long)__double_as_longlong(v);
+    if (bits == NOT_YET) bits ^= 2ULL;                                // (never: keeps a consumer from waiting for ever)
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Block k of U x = z: x_k = U11^-1 z_k (z_k already holds every later block's contribution), then
-// z[i] -= sum_c U[i, k0+c] x_k[c] for the rows i above the block: 16 lanes per row, 8 columns per
-// lane, 64 rows per workgroup.  Workgroup 0 stores x_k into x.
-constexpr int BWD_ROWS = 64;
-__global__ __launch_bounds__(256) void bwd_step_kernel(const double* __restrict__ U, long long ld, int k0, int nb,
-                                                       const double* __restrict__ invT, double* __restrict__ z,
-                                                       double* __restrict__ x) {
-    __shared__ double zs[NB], xs[NB];
-    const int tid = threadIdx.x;
-    if (tid < NB) zs[tid] = tid < nb ? z[k0 + tid] : 0.0;
+// out[c] = sum_m M[m,c] vec[m] with the thread's 32 rows of M in registers; the four partial sums through LDS
+__device__ __forceinline__ double block_product(const double (&iv)[SR], const double* vec, double (*part)[NB], int c,
+                                                int q) {
+    double s = 0.0;
+#pragma unroll
+    for (int m = 0; m < SR; ++m) s = fma(iv[m], vec[SR * q + m], s);
+    part[q][c] = s;
     __syncthreads();
+    return (part[0][c] + part[1][c]) + (part[2][c] + part[3][c]);
+}
+
+__global__ __launch_bounds__(ST) void fwd_solve_kernel(const double* U, long long ld, int F, const double* invs,
+                                                       const double* b, double* z, unsigned spin_limit) {
+    __shared__ double part[SQ][NB], vec[NB];
+    const int k = (int)blockIdx.x, k0 = k * NB;
+    const int tid = threadIdx.x, lane = tid & 63, c = tid & (NB - 1), q = tid / NB;
+    const double* inv = invs + (size_t)k * 2 * NB * NB;
+    double iv[SR];
+#pragma unroll
+    for (int m = 0; m < SR; ++m) iv[m] = inv[(SR * q + m) * NB + c];
+    const bool colok = k0 + c < F;
+    double acc = (q == 0 && colok) ? b[k0 + c] : 0.0;
+    for (int i = 0; i < k; ++i) {
+        const double* tile = U + (size_t)(i * NB + SR * q) * ld + k0 + c;
+        double u[SR];
+#pragma unroll
+        for (int r = 0; r < SR; ++r) u[r] = colok ? tile[(size_t)r * ld] : 0.0;
+        // lane r: row r of this wavefront's quarter of z_i
+        const double* mine = z + i * NB + SR * q + (lane & (SR - 1));
+        unsigned long long bits = peek(mine);
+        for (unsigned n = 0; __builtin_amdgcn_ballot_w64(bits == NOT_YET) != 0ULL && n < spin_limit; ++n) {
+            __builtin_amdgcn_s_sleep(4);
+            bits = peek(mine);
+        }
+        const double zr = bits == NOT_YET ? __builtin_nan("") : __longlong_as_double((long long)bits);
+#pragma unroll
+        for (int r = 0; r < SR; ++r) acc = fma(-u[r], value_of_lane(zr, r), acc);
+    }
+    part[q][c] = acc;
+    __syncthreads();
+    if (tid < NB) vec[tid] = (part[0][tid] + part[1][tid]) + (part[2][tid] + part[3][tid]);
+    __syncthreads();
+    const double zk = block_product(iv, vec, part, c, q);
+    if (tid < NB) hand_on(z + k0 + tid, zk);
+}
+
+__global__ __launch_bounds__(ST) void bwd_solve_kernel(const double* U, long long ld, int F, int nblk,
+                                                       const double* invs, const double* z, double* xs, double* x,
+                                                       unsigned spin_limit) {
+    __shared__ double part[SQ][NB], vec[NB];
+    const int k = nblk - 1 - (int)blockIdx.x, k0 = k * NB;
+    const int tid = threadIdx.x, c = tid & (NB - 1), q = tid / NB;
+    const int csub = tid & 15, rowgrp = tid >> 4;          // sixteen lanes of eight columns along a row; rows rowgrp + 32 a
+    const double* invT = invs + (size_t)k * 2 * NB * NB + NB * NB;
+    double iv[SR];
+#pragma unroll
+    for (int m = 0; m < SR; ++m) iv[m] = invT[(SR * q + m) * NB + c];
+    double acc[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) acc[a] = csub == 0 ? z[k0 + rowgrp + 32 * a] : 0.0;
+    for (int j = nblk - 1; j > k; --j) {
+        const int col0 = j * NB + 8 * csub;
+        double u[4][8];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const double* row = U + (size_t)(k0 + rowgrp + 32 * a) * ld + col0;     // k < nblk - 1: a whole block of rows
+#pragma unroll
+            for (int e = 0; e < 8; ++e) u[a][e] = col0 + e < F ? row[e] : 0.0;
+        }
+        unsigned long long bits[8];
+        bool pending = false;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            bits[e] = peek(xs + col0 + e);
+            pending |= bits[e] == NOT_YET;
+        }
+        for (unsigned n = 0; __builtin_amdgcn_ballot_w64(pending) != 0ULL && n < spin_limit; ++n) {
+            __builtin_amdgcn_s_sleep(4);
+            pending = false;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                bits[e] = peek(xs + col0 + e);
+                pending |= bits[e] == NOT_YET;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const double xv = bits[e] == NOT_YET ? __builtin_nan("") : __longlong_as_double((long long)bits[e]);
+#pragma unroll
+            for (int a = 0; a < 4; ++a) acc[a] = fma(-u[a][e], xv, acc[a]);
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+#pragma unroll
+        for (int m = 8; m >= 1; m >>= 1) acc[a] += __shfl_xor(acc[a], m, 16);
+        if (csub == 0) vec[rowgrp + 32 * a] = acc[a];
+    }
+    __syncthreads();
+    const double xk = block_product(iv, vec, part, c, q);
     if (tid < NB) {
-        double s0 = 0.0, s1 = 0.0;
-        for (int i = 0; i < NB; i += 2) {
-            s0 = fma(invT[i * NB + tid], zs[i], s0);
-            s1 = fma(invT[(i + 1) * NB + tid], zs[i + 1], s1);
-        }
-        xs[tid] = tid < nb ? s0 + s1 : 0.0;
-        if (blockIdx.x == 0 && tid < nb) x[k0 + tid] = s0 + s1;
+        hand_on(xs + k0 + tid, xk);                         // whole blocks: the columns past F are zero
+        if (k0 + tid < F) x[k0 + tid] = xk;
     }
-    __syncthreads();
-    const int sub = tid & 15;
-    double xv[8];
-#pragma unroll
-    for (int q = 0; q < 8; ++q) xv[q] = xs[sub * 8 + q];
-    for (int rr = tid >> 4; rr < BWD_ROWS; rr += 16) {
-        const int i = blockIdx.x * BWD_ROWS + rr;     // uniform over the 16 lanes of a row
-        double sacc = 0.0;
-        if (i < k0) {
-            const double* row = U + (size_t)i * ld + k0 + sub * 8;
-#pragma unroll
-            for (int q = 0; q < 8; ++q)
-                if (sub * 8 + q < nb) sacc = fma(row[q], xv[q], sacc);
-        }
-#pragma unroll
-        for (int m = 8; m >= 1; m >>= 1) sacc += __shfl_xor(sacc, m, 16);
-        if (i < k0 && sub == 0) z[i] -= sacc;
-    }
+}
+
+__global__ __launch_bounds__(256) void fill_words64_kernel(unsigned long long* p, int n, unsigned long long v) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = v;
 }
 
 }  // namespace
 
+// device workspace: the inverses of the diagonal blocks (both orientations), z of the forward solve and the
+// exchange copy of x of the backward solve (whole blocks each), and the flags of the panel launches (per panel:
+// FLAGS_PER_PANEL + one counter per block column)
+namespace {
+struct Workspace {
+    double* invs;
+    double* z;
+    double* xs;
+    unsigned* panel_flags;
+    size_t nblk, npanel, bytes;
+};
+Workspace workspace_layout(void* base, int F) {
+    Workspace w;
+    w.nblk = ((size_t)F + NB - 1) / NB;
+    w.npanel = ((size_t)F + OB - 1) / OB;
+    w.invs = reinterpret_cast<double*>(base);
+    w.z = w.invs + w.nblk * 2 * NB * NB;
+    w.xs = w.z + w.nblk * NB;
+    w.panel_flags = reinterpret_cast<unsigned*>(w.xs + w.nblk * NB);
+    w.bytes = (w.nblk * 2 * NB * NB + 2 * w.nblk * NB) * sizeof(double) +
+              w.npanel * (FLAGS_PER_PANEL + w.nblk) * sizeof(unsigned) + 256;
+    return w;
+}
+}  // namespace
+
 extern "C" size_t qmll_cholesky_workspace_bytes(int F) {
     if (F <= 0) return 0;
-    const size_t nblk = ((size_t)F + NB - 1) / NB;
-    const size_t npanel = ((size_t)F + OB - 1) / OB;
-    return (nblk * 2 * NB * NB + (size_t)F) * sizeof(double) + npanel * (FLAGS_PER_PANEL + nblk) * sizeof(unsigned) + 256;
+    return workspace_layout(nullptr, F).bytes;
 }
 
 namespace {
@@ -677,14 +761,14 @@ extern "C" int qmll_cholesky_f64(double* A, int F, long long ld, void* workspace
     QMLL_REQUIRE(A && workspace && info, QMLL_ERR_INVALID, "qmll_cholesky_f64: null pointer");
     QMLL_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, QMLL_ERR_INVALID,
                  "qmll_cholesky_f64: the workspace must be 16-byte aligned");
-    double* invs = reinterpret_cast<double*>(workspace);
+    const Workspace ws = workspace_layout(workspace, F);
+    double* invs = ws.invs;
     // whole tiles and 16-byte loads: one launch per panel, which also carries the trailing update of the panel
     // before it; otherwise a launch per step
     const bool whole_tiles = F % NB == 0 && ld % 2 == 0 && reinterpret_cast<uintptr_t>(A) % 16 == 0;
     if (whole_tiles) {
-        const size_t nblk_all = (size_t)F / NB;
-        unsigned* flags = reinterpret_cast<unsigned*>(invs + nblk_all * 2 * NB * NB + (size_t)F);
-        const int per_panel = FLAGS_PER_PANEL + F / NB;
+        unsigned* flags = ws.panel_flags;
+        const int per_panel = FLAGS_PER_PANEL + (int)ws.nblk;
         const int nflags = (F + OB - 1) / OB * per_panel;
         hipLaunchKernelGGL(zero_words_kernel, dim3((nflags + 255) / 256), dim3(256), 0, stream, flags, nflags);
         QMLL_CHECK_LAUNCH("qmll_cholesky_f64");
@@ -733,26 +817,17 @@ extern "C" int qmll_cholesky_solve_f64(const double* U, int F, long long ld, voi
     hipStream_t stream = (hipStream_t)stream_;
     QMLL_REQUIRE(F > 0 && ld >= F, QMLL_ERR_INVALID, "qmll_cholesky_solve_f64: bad size F=%d ld=%lld", F, ld);
     QMLL_REQUIRE(U && workspace && b, QMLL_ERR_INVALID, "qmll_cholesky_solve_f64: null pointer");
-    double* invs = reinterpret_cast<double*>(workspace);
-    const size_t nblk = ((size_t)F + NB - 1) / NB;
-    double* z = invs + nblk * 2 * NB * NB;
-    // U^T z = b, blocks in ascending order (b is used up)
-    for (int k0 = 0; k0 < F; k0 += NB) {
-        const int nb = F - k0 < NB ? F - k0 : NB;
-        const int n = F - k0 - nb;
-        const double* inv = invs + (size_t)(k0 / NB) * 2 * NB * NB;
-        const int grid = n > 0 ? (n + 255) / 256 : 1;
-        hipLaunchKernelGGL(fwd_step_kernel, dim3(grid), dim3(256), 0, stream, U, ld, k0, nb, F, inv, b, z);
-        QMLL_CHECK_LAUNCH("qmll_cholesky_solve_f64");
-    }
-    // U x = z, blocks in descending order, x into b
-    const int last = (F - 1) / NB * NB;
-    for (int k0 = last; k0 >= 0; k0 -= NB) {
-        const int nb = F - k0 < NB ? F - k0 : NB;
-        const double* invT = invs + (size_t)(k0 / NB) * 2 * NB * NB + NB * NB;
-        const int grid = k0 > 0 ? (k0 + BWD_ROWS - 1) / BWD_ROWS : 1;
-        hipLaunchKernelGGL(bwd_step_kernel, dim3(grid), dim3(256), 0, stream, U, ld, k0, nb, invT, z, b);
-        QMLL_CHECK_LAUNCH("qmll_cholesky_solve_f64");
-    }
+    const Workspace ws = workspace_layout(workspace, F);
+    const int nblk = (int)ws.nblk;
+    // z and the exchange copy of x are contiguous: "not yet" everywhere
+    hipLaunchKernelGGL(fill_words64_kernel, dim3((2 * nblk * NB + 255) / 256), dim3(256), 0, stream,
+                       reinterpret_cast<unsigned long long*>(ws.z), 2 * nblk * NB, NOT_YET);
+    QMLL_CHECK_LAUNCH("qmll_cholesky_solve_f64");
+    // U^T z = b, then U x = z with x into b
+    hipLaunchKernelGGL(fwd_solve_kernel, dim3(nblk), dim3(ST), 0, stream, U, ld, F, ws.invs, b, ws.z, SPIN_LIMIT);
+    QMLL_CHECK_LAUNCH("qmll_cholesky_solve_f64");
+    hipLaunchKernelGGL(bwd_solve_kernel, dim3(nblk), dim3(ST), 0, stream, U, ld, F, nblk, ws.invs, ws.z, ws.xs, b,
+                       SPIN_LIMIT);
+    QMLL_CHECK_LAUNCH("qmll_cholesky_solve_f64");
     return QMLL_OK;
 }
