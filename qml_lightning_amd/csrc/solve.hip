@@ -421,7 +421,10 @@ __device__ __forceinline__ void tile_product(const double* Za, long long lda, co
             for (int r = 0; r < 4; ++r) {
                 double* c = C + (size_t)(wi + p * 16 + lk + 4 * r) * ldc + wj + q * 16 + l16;
                 const double v = sign * acc[p][q][r];
-                *c = overwrite ? v : *c + v;
+                // (the sum is left to the memory side: no wait for the old value; every element of C takes
+                // exactly one addition per launch, so the result does not depend on any order)
+                if (overwrite) *c = v;
+                else unsafeAtomicAdd(c, v);
             }
     __syncthreads();
 }
