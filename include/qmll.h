@@ -471,7 +471,10 @@ size_t qmll_cholesky_workspace_bytes(int F);
  * runs out (never seen) leaves info = -1, which callers treat like a failed pivot. */
 int qmll_cholesky_f64(double* A, int F, long long ld, void* workspace, int* info, qmll_stream_t stream);
 
-/* b <- (U^T U)^-1 b for one right-hand side b[F], U and workspace from qmll_cholesky_f64. */
+/* b <- (U^T U)^-1 b for one right-hand side b[F], U and workspace from qmll_cholesky_f64.  One launch per
+ * direction, a workgroup per 128-row block; the blocks wait for one another's results with bounded waits,
+ * and one that runs out (never seen) leaves NaN in b rather than a wrong number.  Calls that share a
+ * workspace must not overlap. */
 int qmll_cholesky_solve_f64(const double* U, int F, long long ld, void* workspace, double* b, qmll_stream_t stream);
 
 /* Feature-tiled variant (kernel.py:172-181, ntiles > 1): ZTZ_tile f64 [f1-f0, F] +=
