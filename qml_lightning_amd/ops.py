@@ -707,7 +707,8 @@ def cholesky_solve_spd(A, b, overwrite_a=False):
     """x = A^-1 b for a symmetric positive definite fp64 A [F,F] and b [F] or [F,1], by the
     in-place upper Cholesky factorisation of the library.  Only the upper triangle of A is read.
     Returns (x, info): info is a device int32 tensor, 0 on success, else 1 + the index of the first
-    non-positive pivot (x is then meaningless).  A is destroyed when overwrite_a is True."""
+    non-positive pivot, or -1 if a bounded wait inside the library ran out (never seen); x is then
+    meaningless.  A is destroyed when overwrite_a is True."""
     if A.dtype != torch.float64 or A.dim() != 2 or A.shape[0] != A.shape[1] or A.stride(1) != 1:
         raise RuntimeError("cholesky_solve_spd needs a square float64 matrix with contiguous rows")
     F = int(A.shape[0])
