@@ -335,6 +335,11 @@ __global__ __launch_bounds__(PT, 4) void potrf_block_kernel(double* A, long long
 // whatever the number of workgroups resident at a time.  Every wait is bounded all the same: a wait that
 // runs out sets info to -1 and the workgroup leaves.
 //
+// Head tiles.  Once the trailing matrix is small a launch lasts as long as its slowest owner, and four of an
+// owner's fourteen tile products are that first update.  The host then puts workgroups for those tiles in
+// front of the owners (one per tile, waiting for nobody); each counts itself into its column's counter
+// when done, and an owner starts by waiting for its column's count.
+//
 // Trailing tiles.  The workgroups after the owners (their count rounded up to a multiple of eight, so
 // that the XCD of a tile is what gram_tiles.h deals) take the previous panel's update of the tiles
 // on or above the diagonal below this panel, 512 deep, and wait for nobody.  While the panel's chain of
