@@ -821,6 +821,27 @@ def test_solve_falls_back_to_lu_when_a_pivot_is_not_positive():
     assert np.abs(A @ x - b).max() <= 1e-9 * np.abs(x).max()
 
 
+def test_triangular_solves_hand_a_nan_on_instead_of_waiting_for_it():
+    """The blocks of the two solve launches hand their results on as the values themselves, with one NaN bit
+    pattern meaning "not yet".  A right-hand side that holds NaNs, that very pattern among them, must come back
+    as NaNs, not hang a consumer."""
+    from qml_lightning_amd import ops
+    rng = np.random.default_rng(12)
+    F = 640
+    Zr = rng.normal(size=(F + 20, F))
+    A = torch.tensor(Zr.T @ Zr + 1e-6 * np.eye(F), device=dev())
+    b = rng.normal(size=(F, 1))
+    b[7, 0] = np.nan
+    b[300, 0] = np.frombuffer(np.uint64(0x7FF8C0DEC0DE0001).tobytes(), dtype=np.float64)[0]
+    x, info = ops.cholesky_solve_spd(A, torch.tensor(b, device=dev()))
+    assert int(info.item()) == 0
+    assert torch.isnan(x).all()                      # block 0 is poisoned, and every later block takes it in
+    # and the same matrix with a clean right-hand side right after
+    b2 = rng.normal(size=(F, 1))
+    x2, _ = ops.cholesky_solve_spd(A, torch.tensor(b2, device=dev()))
+    assert np.abs(A.cpu().numpy() @ x2.cpu().numpy() - b2).max() <= 1e-7 * np.abs(b2).max()
+
+
 def test_cholesky_in_place_on_a_strided_view():
     """overwrite_a=True factors inside a wider buffer (row stride 700 for a 300 x 300 matrix) and
     touches nothing outside the matrix."""
