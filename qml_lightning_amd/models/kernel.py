@@ -308,7 +308,7 @@ class BaseKernel():
         if cpu_solve:
             self.alpha = torch.linalg.solve(ZTZ, ZtrainY.cpu())[:, 0].to(self.device)
         else:
-            self.alpha = self._solve_spd(ZTZ, ZtrainY)[:, 0]
+            self.alpha = self._solve_spd(ZTZ, ZtrainY, overwrite_a=True)[:, 0]     # Z^T Z is not needed again
         end.record()
         torch.cuda.synchronize()
         if print_info:
@@ -316,15 +316,36 @@ class BaseKernel():
         self.is_trained = True
 
     @staticmethod
-    def _solve_spd(A, b):
+    def _solve_spd(A, b, overwrite_a=False):
         """x = A^-1 b for the regularised normal matrix.  The reference calls
         torch.linalg.solve (LU, kernel.py:231); Z^T Z + lambda I is symmetric positive definite,
         so the library's blocked Cholesky factorisation gives the same solution for half the
-        flops; LU remains the fallback when rounding has left the matrix numerically indefinite."""
+        flops; LU remains the fallback when rounding has left the matrix numerically indefinite.
+
+        overwrite_a: A (symmetric, both triangles stored) may be used up.  The factorisation then
+        works in A itself instead of in a copy of it (2 GB at 16 384 features); it touches the
+        upper triangle and the 128 x 128 tiles on the diagonal only, so those tiles are kept aside
+        (16 MB) and, should a pivot fail, A is put together again from them and its lower
+        triangle before LU takes it."""
         if A.is_cuda and b.dim() == 2 and b.shape[1] == 1 and A.stride(1) == 1 and A.stride(0) % 2 == 0:
-            x, info = ops.cholesky_solve_spd(A, b)
+            if not overwrite_a:
+                x, info = ops.cholesky_solve_spd(A, b)
+                if int(info.item()) == 0:
+                    return x
+                return torch.linalg.solve(A, b)
+            n, ld, t = int(A.shape[0]), int(A.stride(0)), 128
+            whole = n // t
+            tiles = A.as_strided((whole, t, t), (t * (ld + 1), ld, 1))
+            kept = tiles.clone()
+            last = A[whole * t:, whole * t:].clone()
+            x, info = ops.cholesky_solve_spd(A, b, overwrite_a=True)
             if int(info.item()) == 0:
                 return x
+            low = torch.tril(A, -1)
+            A.copy_(low + low.T)
+            del low
+            tiles.copy_(kept)
+            A[whole * t:, whole * t:] = last
             return torch.linalg.solve(A, b)
         L, info = torch.linalg.cholesky_ex(A)
         if int(info.item()) == 0:

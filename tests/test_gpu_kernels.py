@@ -842,6 +842,31 @@ def test_triangular_solves_hand_a_nan_on_instead_of_waiting_for_it():
     assert np.abs(A.cpu().numpy() @ x2.cpu().numpy() - b2).max() <= 1e-7 * np.abs(b2).max()
 
 
+@pytest.mark.parametrize("F", [300, 640])
+def test_solve_in_the_matrix_itself_and_its_restoration_for_lu(F):
+    """train() lets _solve_spd use up Z^T Z: the same solution as from a copy when the matrix is positive
+    definite; when a pivot fails, the matrix is put together again (diagonal tiles kept aside, the rest from
+    the lower triangle) and LU solves the original system."""
+    from qml_lightning_amd.models.kernel import BaseKernel
+    rng = np.random.default_rng(F)
+    Zr = rng.normal(size=(F + 20, F))
+    A = Zr.T @ Zr + 1e-6 * np.eye(F)
+    b = rng.normal(size=(F, 1))
+    bt = torch.tensor(b, device=dev())
+    x_copy = BaseKernel._solve_spd(torch.tensor(A, device=dev()), bt)
+    x_used = BaseKernel._solve_spd(torch.tensor(A, device=dev()), bt, overwrite_a=True)
+    assert torch.equal(x_copy, x_used)
+    Q, _ = np.linalg.qr(rng.normal(size=(F, F)))
+    w = np.linspace(1.0, 2.0, F)
+    w[F // 2] = -1e-3                                       # one slightly negative eigenvalue
+    Ai = (Q * w) @ Q.T
+    Ai = 0.5 * (Ai + Ai.T)
+    At = torch.tensor(Ai, device=dev())
+    x = BaseKernel._solve_spd(At, bt, overwrite_a=True).cpu().numpy()
+    assert np.abs(Ai @ x - b).max() <= 1e-9 * np.abs(x).max()
+    assert torch.equal(At, torch.tensor(Ai, device=dev()))  # restored exactly
+
+
 def test_cholesky_in_place_on_a_strided_view():
     """overwrite_a=True factors inside a wider buffer (row stride 700 for a 300 x 300 matrix) and
     touches nothing outside the matrix."""
