@@ -468,7 +468,9 @@ size_t qmll_cholesky_workspace_bytes(int F);
  * that is not positive; U is then unusable.  When F is a multiple of 128 (and A 16-byte aligned) a
  * panel of 512 rows and the trailing update of the panel before it are one launch whose workgroups
  * wait for one another through flags in the workspace; every such wait is bounded, and one that
- * runs out (never seen) leaves info = -1, which callers treat like a failed pivot. */
+ * runs out (never seen) leaves info = -1, which callers treat like a failed pivot.  The tile products
+ * add into the trailing matrix with hardware fp64 atomic adds, which need A in ordinary device memory
+ * (hipMalloc; what torch allocates), not in host-mapped or managed memory. */
 int qmll_cholesky_f64(double* A, int F, long long ld, void* workspace, int* info, qmll_stream_t stream);
 
 /* b <- (U^T U)^-1 b for one right-hand side b[F], U and workspace from qmll_cholesky_f64.  One launch per
