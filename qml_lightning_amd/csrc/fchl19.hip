@@ -349,7 +349,11 @@ __device__ __forceinline__ Triple triple_geometry(const Stage& s, int j, int k) 
 // sub-slot, radial bin l) run over the table with the bin sums in registers.  Rows go
 // straight from registers to global memory.
 // ---------------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void fchl19_forward_kernel(FchlArgs a, float* __restrict__ rep) {
+// (96 scalar registers: the eighth wavefront per SIMD; a SIMD has 800 of them, handed out in sixteens, and left
+// alone the kernel takes 106.  The thirty-odd values that no longer fit are parked in the lanes of a vector
+// register.  The backward kernel's LDS request allows no eighth wavefront, and there the cap only costs.)
+__global__ __launch_bounds__(64) __attribute__((amdgpu_num_sgpr(96))) void fchl19_forward_kernel(FchlArgs a,
+                                                                                                 float* __restrict__ rep) {
     extern __shared__ float smem[];
     const int lane = threadIdx.x;
     const int m = a.molIDs[blockIdx.x];
