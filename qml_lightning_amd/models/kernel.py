@@ -716,6 +716,18 @@ class BaseKernel():
             return self._format_padded_arrays(X, Q, E, F, cells, inv_cells)
         counts = np.fromiter(map(len, X), dtype=np.int32, count=zbatch)
         n = int(counts.max()) if zbatch else 0
+        if zbatch and n > 0 and int(counts.min()) == n:
+            # molecules of one size (a trajectory, a fixed composition): the lists stacked are the padded
+            # array pair already, with nothing to pad and no index to build on the host
+            try:
+                Xa = self._concat_rows(X, 3, np.float32).reshape(zbatch, n, 3)
+                Qa = self._concat_rows(Q, 1, np.float32).reshape(zbatch, n)
+                Fa = None if F is None else self._concat_rows(F, 3, np.float64).reshape(zbatch, n, 3)
+                Ea = None if E is None else np.asarray(E, dtype=np.float64).reshape(zbatch)
+                if (Qa > 0).all():
+                    return self._format_padded_arrays(Xa, Qa, Ea, Fa, cells, inv_cells)
+            except ValueError:
+                pass                                        # odd shapes: the general route sorts them out or raises
         # one concatenation and one scatter instead of a Python loop over molecules
         molIDs = np.repeat(np.arange(zbatch, dtype=np.int32), counts)
         starts = np.cumsum(counts) - counts

@@ -391,6 +391,14 @@ def test_format_data_of_padded_arrays_equals_the_list_route(ragged):
     b = m.format_data(Xp, Qp)
     for key in ("coordinates", "charges", "natom_counts", "atomIDs", "molIDs"):
         assert a[key].dtype == b[key].dtype and torch.equal(a[key], b[key]), key
+    if not ragged:
+        # lists of equal-size molecules are stacked and take the device formatter too; the same molecules
+        # followed by a smaller one take the host formatter: the same tensors for the molecules they share
+        g = m.format_data(c32 + [c32[0][:4]], list(charges) + [charges[0][:4]])
+        natoms = sum(len(q) for q in charges)
+        assert torch.equal(g["coordinates"][:len(c32)], a["coordinates"]) and torch.equal(g["charges"][:len(c32)], a["charges"])
+        assert torch.equal(g["natom_counts"][:len(c32)], a["natom_counts"])
+        assert torch.equal(g["atomIDs"][:natoms], a["atomIDs"]) and torch.equal(g["molIDs"][:natoms], a["molIDs"])
     ea, fa = m.predict(c32, charges, n, forces=True, print_info=False)
     eb, fb = m.predict(Xp, Qp, n, forces=True, print_info=False)
     assert torch.equal(ea, eb)
